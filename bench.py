@@ -1,0 +1,153 @@
+#!/usr/bin/env python3
+"""Headline benchmark: the fused soft-staircase pass on one MI355X.
+
+Workload (BASELINE.json configs[1]): a flat fp32 tensor of 2^26 weights, uniform in [-1,1] with
+10 % of the elements placed within +-0.02 of a ternary level, an N(0,1) upstream gradient, and a
+sweep over five hardness values of the default schedule. One "step" is one fused pass
+(y = S(w), dw = g*S'(w) + gl*Q'(w), loss sum, clamp(w)) over the whole tensor at the next hardness
+value of the sweep. Inputs are resident in HBM before the timed region starts.
+
+Prints ONE JSON line: metric soft-step fwd+bwd GB/s on the algorithmic 20 B/element, with a
+`roofline` object for the dominant kernel (HIP-event timed per launch) and a `cpu_baseline`
+object (the op-for-op torch CPU restatement of the reference path, timed on this host's cores
+on a bounded sample).
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload softstep|gemv|gemm|...]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HARDNESS = [0.1, 1.1684210526315788, 3.0004, 4.72, 6.0]   # default schedule, epochs 0/21/79/88/149 of 150
+SHARPNESS, STRENGTH = 5.0, 5e-4
+HBM_PEAK_GBS = 8000.0
+BYTES_PER_ELEM = 20                                        # load w, g; store y, dw, clamp(w)
+
+
+def make_inputs(n, torch):
+    """Seeded CPU generation (identical bits for the CPU baseline and the GPU)."""
+    gen = lambda s: torch.Generator(device="cpu").manual_seed(s)
+    w = 2 * torch.rand(n, generator=gen(1)) - 1
+    mask = torch.rand(n, generator=gen(2)) < 0.10
+    level = torch.randint(-1, 2, (n,), generator=gen(3)).float()
+    offset = 0.04 * torch.rand(n, generator=gen(4)) - 0.02
+    w[mask] = (level + offset)[mask]
+    g = torch.randn(n, generator=gen(5))
+    return w, g
+
+
+def cpu_baseline(torch, sample_n, budget_s=15.0):
+    """The reference's CPU op chain (oracle/torch_path.py) on the first sample_n elements of the
+    same workload, all host cores torch uses; GB/s on the same 20 B/element."""
+    from oracle import torch_path as tp
+    w, g = make_inputs(sample_n, torch)
+    gl = 1.0 / sample_n
+    threads = torch.get_num_threads()
+    times = []
+    t_start = time.perf_counter()
+    reps = 0
+    while True:
+        d = HARDNESS[reps % len(HARDNESS)]
+        t0 = time.perf_counter()
+        tp.fused_step(w, g, d, SHARPNESS, STRENGTH, gl, -1.0, 1.0)
+        dt = time.perf_counter() - t0
+        if reps >= 1:                      # first repetition is the warm-up
+            times.append(dt)
+        reps += 1
+        if (len(times) >= 5 and time.perf_counter() - t_start > budget_s) or len(times) >= 25:
+            break
+    times.sort()
+    med = times[len(times) // 2]
+    return {"value": round(sample_n * BYTES_PER_ELEM / med / 1e9, 3), "unit": "GB/s", "cores": threads,
+            "kind": "port",
+            "sample": f"first {sample_n} elements of the workload, {len(times)} timed fused steps over the hardness "
+                      f"sweep, median; torch {torch.__version__} CPU ops in the reference's op order"}
+
+
+def bench_softstep(args, torch):
+    from tmq_amd import ops, _capi
+    dev = torch.device("cuda:0")
+    n = args.elements
+    w, g = make_inputs(n, torch)
+    tw, tg = w.to(dev), g.to(dev)
+    del w, g
+    gl = float(torch.tensor(1.0, dtype=torch.float32) / torch.tensor(float(n), dtype=torch.float32))
+    lib = _capi.load()
+    y, dw, wc = torch.empty_like(tw), torch.empty_like(tw), torch.empty_like(tw)
+    loss = torch.empty(1, dtype=torch.float64, device=dev)
+    ws = torch.empty(lib.tmq_softstep_fused_workspace_bytes(n), dtype=torch.uint8, device=dev)
+    out = (y, dw, wc, loss, ws)
+
+    def step(i):
+        ops.softstep_fused(tw, tg, HARDNESS[i % len(HARDNESS)], SHARPNESS, STRENGTH, gl, -1.0, 1.0, out=out)
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        ev[i][0].record()
+        step(i)
+        ev[i][1].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    per_launch_ms = [a.elapsed_time(b) for a, b in ev]
+    avg_ms = sum(per_launch_ms) / len(per_launch_ms)
+    bytes_per_launch = n * BYTES_PER_ELEM
+    value = bytes_per_launch * args.steps / wall / 1e9
+    achieved = bytes_per_launch / (avg_ms * 1e-3) / 1e9
+    res = {
+        "metric": "soft-step fwd+bwd GB/s", "value": round(value, 2), "unit": "GB/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(wall / args.steps * 1e3, 5),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "configs[1]: fused soft-step fwd+bwd+qloss+clamp, flat fp32 tensor, hardness sweep "
+                               "over 5 schedule values", "elements": n, "bytes_per_element": BYTES_PER_ELEM,
+                   "hardness": HARDNESS, "sharpness": SHARPNESS, "strength": STRENGTH},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "stream_kernel<FusedOp<15>> (+ 1-block loss finalisation in the same call)",
+                     "avg_launch_us": round(avg_ms * 1e3, 3),
+                     "per_hardness_us": {str(HARDNESS[k]): round(
+                         1e3 * sum(per_launch_ms[k::len(HARDNESS)]) / max(1, len(per_launch_ms[k::len(HARDNESS)])), 3)
+                         for k in range(min(len(HARDNESS), args.steps))}},
+    }
+    if not args.no_cpu:
+        res["cpu_baseline"] = cpu_baseline(torch, args.cpu_sample)
+    return res
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="softstep")
+    ap.add_argument("--elements", type=int, default=1 << 26)
+    ap.add_argument("--cpu-sample", type=int, default=1 << 22)
+    ap.add_argument("--no-cpu", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build targets one GPU; --gpus N with N > 1 is not supported (the path has no "
+              "cross-GPU work).", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    if args.workload == "softstep":
+        res = bench_softstep(args, torch)
+    else:
+        from tmq_amd import bench_extra
+        res = bench_extra.run(args, torch)
+    print(json.dumps(res))
+
+
+if __name__ == "__main__":
+    main()

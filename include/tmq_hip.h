@@ -1,0 +1,209 @@
+/*
+ * libtmq_hip -- C ABI of the MI355X (gfx950) implementation of TMQ's GPU hot path.
+ *
+ * Conventions
+ *   - Every entry point returns TMQ_OK (0) or a negative tmq_status; nothing throws.
+ *   - Pointers are raw device pointers unless a parameter is documented as host memory.
+ *     Tensors are dense and contiguous; `n` counts elements.
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream). Work is enqueued
+ *     asynchronously; no entry point synchronises, allocates or frees device memory. Workspaces
+ *     are passed in by the caller and sized with the *_workspace_bytes helpers.
+ *   - Hardness / strength scalars cross the boundary as C doubles, exactly as the Python
+ *     caller holds them; the library rounds them to fp32 once, the way torch does when a Python
+ *     scalar meets an fp32 tensor, so results are bit-identical to the reference's CPU chain
+ *     of separately rounded fp32 operations.
+ *   - Thread safe; no hidden mutable global state.
+ *
+ * Each declaration cites the reference interface it replaces (paths relative to the reference
+ * repository root).
+ */
+#ifndef TMQ_HIP_H
+#define TMQ_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum tmq_status {
+    TMQ_OK = 0,
+    TMQ_ERR_INVALID_ARG = -1, /* null pointer, negative size, misaligned or inconsistent shape */
+    TMQ_ERR_UNSUPPORTED = -2, /* dtype / shape combination this build does not implement */
+    TMQ_ERR_LAUNCH = -3,      /* HIP reported an error; see tmq_last_hip_error() */
+    TMQ_ERR_TOO_LARGE = -4,   /* size exceeds what the launch geometry can index */
+    TMQ_ERR_BAD_DATA = -5     /* host codec: malformed stream or illegal symbol */
+} tmq_status;
+
+/* Library version (major*10000 + minor*100 + patch) and a static description of a status. */
+int tmq_version(void);
+const char *tmq_status_string(int status);
+/* hipError_t of the last failing HIP call made by this library on the calling thread. */
+int tmq_last_hip_error(void);
+
+/* Element dtypes understood by the packer. */
+enum { TMQ_F32 = 0, TMQ_I32 = 1, TMQ_I8 = 2, TMQ_F16 = 3 };
+
+/* ------------------------------------------------------------------------------------------
+ * Soft-staircase transfer function (fp32).
+ * ---------------------------------------------------------------------------------------- */
+
+/* y = S(w; digamma).
+ * Replaces fwd_softstep / forwardSoftStepCUDA (tmq/tmq_cuda.cu:740-764, kernel 80-92) with the
+ * arithmetic of SoftStep.forward's CPU branch (tmq/tmq.py:417-419).                          */
+int tmq_softstep_fwd(const float *w, float *y, size_t n, double digamma, void *stream);
+
+/* dw = (scale*g) * S'(w; digamma).
+ * Replaces bwd_softstep / backwardSoftStepCUDA (tmq/tmq_cuda.cu:768-794, kernel 95-110);
+ * arithmetic of tmq/tmq.py:434-438.                                                          */
+int tmq_softstep_bwd(const float *w, const float *g, float *dw, size_t n, double digamma,
+                     double scale, void *stream);
+
+/* q = strength*digamma*dsig(arg)/(2 sig(digamma/2)) -- the quantization-loss integrand.
+ * Replaces fwd_softstep_derivative (tmq/tmq_cuda.cu:690-709, kernel 45-59); arithmetic of
+ * tmq/tmq.py:469-473.                                                                        */
+int tmq_softstep_deriv_fwd(const float *w, float *q, size_t n, double digamma, double strength,
+                           void *stream);
+
+/* dw = g * strength*digamma^2*d2sig(arg)/(2 sig(digamma/2)).
+ * Replaces bwd_softstep_derivative (tmq/tmq_cuda.cu:713-735, kernel 62-77); arithmetic of
+ * tmq/tmq.py:488-493.                                                                        */
+int tmq_softstep_deriv_bwd(const float *w, const float *g, float *dw, size_t n, double digamma,
+                           double strength, void *stream);
+
+/* w <- clamp(w, lo, hi) in place (NaN stays NaN).
+ * Replaces the torch.clamp pass of Linear.clamp / Conv2d.clamp (tmq/tmq.py:691-696, 874-879)
+ * driven by QuantizationControl.clamp (tmq/tmq.py:263-272).                                  */
+int tmq_clamp_inplace(float *w, size_t n, double lo, double hi, void *stream);
+
+/* w <- round_half_even(map(w; digamma)) in place, map with the association of
+ * SoftStep.map (tmq/tmq.py:335-338). Replaces the body of QuantizationControl.quantize
+ * (tmq/tmq.py:284-295). With digamma <= 0 it is plain round_half_even(w), i.e.
+ * Linear.quantize / Conv2d.quantize / quantize_weights (tmq/tmq.py:603, 886, 1109).          */
+int tmq_ternarize_inplace(float *w, size_t n, double digamma, void *stream);
+
+/* One fused pass over a flat tensor: everything the reference does to a weight tensor in a
+ * QAT step -- y = S(w; digamma); loss integrand q(w; sharpness, strength) reduced to a sum;
+ * dw = g*S'(w; digamma) + gl*Q'(w; sharpness, strength); wc = clamp(w, lo, hi).
+ * Fuses tmq/tmq.py:417-419, 434-438, 469-473 (+ the mean of 699), 488-493 and 696 -- seven
+ * separate passes in the reference (tmq/tmq_cuda.cu:45-110 + torch mean/add/clamp).
+ * Any of y, dw, wc may be NULL (that output is skipped; g may be NULL iff dw is NULL); wc may
+ * alias w. loss_sum (device, 1 double) receives sum_i q_i; it may be NULL. workspace must hold
+ * tmq_softstep_fused_workspace_bytes(n) bytes when loss_sum is non-NULL.                      */
+size_t tmq_softstep_fused_workspace_bytes(size_t n);
+int tmq_softstep_fused(const float *w, const float *g, float *y, float *dw, float *wc,
+                       double *loss_sum, void *workspace, size_t n, double digamma,
+                       double sharpness, double strength, float gl, double lo, double hi,
+                       void *stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Multi-tensor (one launch for every registered layer) forms of the per-layer Python loops of
+ * QuantizationControl.quantization_loss / clamp (tmq/tmq.py:298-310, 263-272).
+ *
+ * A segment table describes the tensors. The caller fills ptr/aux/n (+ scalar where stated),
+ * calls tmq_multi_plan() on the host copy to assign block ranges, and uploads the table.
+ * ---------------------------------------------------------------------------------------- */
+typedef struct tmq_segment {
+    void *ptr;            /* weight tensor (fp32) */
+    void *aux;            /* second tensor of the same size where the op needs one, else NULL */
+    uint64_t n;           /* elements */
+    uint32_t block_begin; /* filled by tmq_multi_plan */
+    float scalar;         /* per-tensor scalar where the op needs one */
+} tmq_segment;
+
+/* Host helper: fills block_begin for nseg segments, returns the launch's block count in
+ * *total_blocks. Empty tensors are legal.                                                    */
+int tmq_multi_plan(tmq_segment *segs_host, int nseg, uint32_t *total_blocks);
+
+/* Workspace (bytes) for tmq_qloss_multi with that plan. */
+size_t tmq_qloss_multi_workspace_bytes(uint32_t total_blocks);
+
+/* per_tensor[l] = mean_i q(w_l[i]; sharpness, strength); *total = fp32 sum over l in table
+ * order (the reference's Python loop of scalar adds, tmq/tmq.py:305-310). Either output may be
+ * NULL. Two launches: block partial sums, then an ordered fp64 finalisation (deterministic). */
+int tmq_qloss_multi(const tmq_segment *segs_dev, int nseg, uint32_t total_blocks, double sharpness,
+                    double strength, float *per_tensor, float *total, void *workspace,
+                    void *stream);
+
+/* aux_l[i] (= or +=) scalar_l * Q'(w_l[i]; sharpness, strength): the gradient of the loss above
+ * w.r.t. every weight, scalar_l = upstream_grad / n_l as autograd's mean backward produces it.
+ * accumulate != 0 adds into aux (fused grad accumulation), else overwrites.                  */
+int tmq_qloss_bwd_multi(const tmq_segment *segs_dev, int nseg, uint32_t total_blocks,
+                        double sharpness, double strength, int accumulate, void *stream);
+
+/* w_l <- clamp(w_l, lo, hi) for every segment, one launch. */
+int tmq_clamp_multi(const tmq_segment *segs_dev, int nseg, uint32_t total_blocks, double lo,
+                    double hi, void *stream);
+
+/* ------------------------------------------------------------------------------------------
+ * 2-bit ternary packing (16 codes per 32-bit word, first element in bits 31:30; 0->00, +1->01,
+ * -1->10; ragged tails zero-filled).
+ * ---------------------------------------------------------------------------------------- */
+
+/* W[N][K] (row-major, dtype TMQ_F32 / TMQ_I32 / TMQ_I8) -> words[K][ceil(N/16)]; word (k,q)
+ * holds W[16q+j][k], j = 0..15. fp32 values are rounded half away from zero, integers cast,
+ * then clamped to [-1,1].
+ * Replaces compactify_ternary (tmq/tmq_native.cpp:418-425): a Linear weight [out][in] is the
+ * case N=out, K=in (matrixTo2BitTernary 152-171 after the transpose at 311-314); a Conv2d
+ * weight [out][in][ky][kx] is N=out, K=in*ky*kx (kernelTo2BitTernary 185-208).                */
+int tmq_pack_ternary(const void *w, int dtype, int64_t N, int64_t K, uint32_t *words, void *stream);
+
+/* words[K][ceil(N/16)] -> fp32 W[N][K] in {-1,0,+1} (code 11 -> 0, as tmq/tmq_cuda.cu:464-466).
+ * Replaces expand_ternary (tmq/tmq_native.cpp:516-544; compactKernelTo32BitFloat 249-266).
+ * This is the true inverse of tmq_pack_ternary also for 2-D tensors.                         */
+int tmq_unpack_ternary(const uint32_t *words, int64_t N, int64_t K, float *w, void *stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Ternary inference: y[m][n] = scale[n] * sum_k x[m][k] * T[k][n] + bias[n]
+ * with T packed as words[K][ceil(N/16)], fp32 accumulation, fp32 output [M][N].
+ * scale / bias are optional fp32 [N] (NULL = 1 / 0). x_dtype is TMQ_F16 or TMQ_F32 (fp32
+ * activations are split into two fp16 terms so the product keeps fp32 accuracy).
+ * Replaces ternary_mvm_cuda (tmq/tmq_cuda.cu:563-603, kernel 242-286) for M == 1 and
+ * ternary_mmm_cuda (tmq/tmq_cuda.cu:478-549, kernel 289-427) for M > 1, plus the post-scale /
+ * bias passes of Linear.compact_forward (tmq/tmq.py:684-687).                                */
+int tmq_ternary_linear(const void *x, int x_dtype, int64_t M, int64_t K, const uint32_t *words,
+                       int64_t N, const float *scale, const float *bias, float *y, void *stream);
+
+/* Geometry of a 2-D convolution. */
+typedef struct tmq_conv_shape {
+    int32_t B, C, H, W;   /* input NCHW extents */
+    int32_t N;            /* output channels */
+    int32_t ky, kx, sy, sx, py, px, dy, dx;
+} tmq_conv_shape;
+
+/* Output extents (PyTorch's formula). */
+int tmq_conv2d_out_hw(const tmq_conv_shape *s, int32_t *ho, int32_t *wo);
+
+/* Ternary implicit-GEMM convolution, no materialised im2col. x is fp16, either NCHW
+ * (channels_last == 0) or NHWC (channels_last != 0); y is written in the same memory format,
+ * dtype y_dtype (TMQ_F32 or TMQ_F16). words is [C*ky*kx][ceil(N/16)] with row (c*ky+i)*kx+j.
+ * Optional fused epilogue: y = relu?( scale[n]*acc + bias[n] + residual ), residual in y's
+ * format and dtype. Replaces the unfold + ternary_mmm_cuda + fold path of
+ * Conv2d.compact_forward (tmq/tmq.py:856-871).                                               */
+int tmq_ternary_conv2d(const void *x, int channels_last, const tmq_conv_shape *shape,
+                       const uint32_t *words, const float *scale, const float *bias,
+                       const void *residual, int relu, void *y, int y_dtype, void *stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Host entropy codec for packed tensors (host memory in, host memory out; no GPU involved).
+ * ---------------------------------------------------------------------------------------- */
+
+/* Upper bound of the container size for rows*columns symbols. */
+size_t tmq_compress_bound(int64_t rows, int64_t columns);
+
+/* Range-code words[rows][ceil(columns/16)] into out (capacity out_cap); *out_size receives the
+ * container size. Byte-compatible with compress_ternary (tmq/tmq_native.cpp:439-477 ->
+ * entropyEncodeTernary 50-97 -> RangeEncoder tmq/rangecoder.h:41-112).                       */
+int tmq_compress_ternary(const uint32_t *words_host, int64_t rows, int64_t columns, uint8_t *out,
+                         size_t out_cap, size_t *out_size);
+
+/* Inverse. Replaces decompress_ternary (tmq/tmq_native.cpp:489-503 -> entropyDecodeTernary
+ * 111-140 -> RangeDecoder tmq/rangecoder.h:124-193).                                         */
+int tmq_decompress_ternary(const uint8_t *in, size_t in_size, uint32_t *words_host, int64_t rows,
+                           int64_t columns);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TMQ_HIP_H */

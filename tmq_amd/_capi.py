@@ -1,0 +1,116 @@
+"""ctypes view of libtmq_hip.so -- the C ABI declared in include/tmq_hip.h.
+
+torch is used only to own device memory and to name the current stream; every computation goes
+through the shared library. There is no CPU or PyTorch fallback: if the library is missing or a
+call fails, an exception is raised.
+"""
+import ctypes
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libtmq_hip.so")
+
+F32, I32, I8, F16 = 0, 1, 2, 3
+_DTYPE_CODE = {torch.float32: F32, torch.int32: I32, torch.int8: I8, torch.float16: F16}
+
+
+class TmqError(RuntimeError):
+    """A libtmq_hip entry point returned a non-zero status."""
+
+
+class Segment(ctypes.Structure):
+    """tmq_segment of include/tmq_hip.h (32 bytes)."""
+    _fields_ = [("ptr", ctypes.c_void_p), ("aux", ctypes.c_void_p), ("n", ctypes.c_uint64),
+                ("block_begin", ctypes.c_uint32), ("scalar", ctypes.c_float)]
+
+
+class ConvShape(ctypes.Structure):
+    """tmq_conv_shape of include/tmq_hip.h."""
+    _fields_ = [(k, ctypes.c_int32) for k in
+                ("B", "C", "H", "W", "N", "ky", "kx", "sy", "sx", "py", "px", "dy", "dx")]
+
+
+_vp, _sz, _dbl, _i64, _int, _flt, _u32 = (ctypes.c_void_p, ctypes.c_size_t, ctypes.c_double, ctypes.c_int64,
+                                           ctypes.c_int, ctypes.c_float, ctypes.c_uint32)
+
+# name -> (restype, argtypes); every symbol include/tmq_hip.h declares.
+SIGNATURES = {
+    "tmq_version": (_int, []),
+    "tmq_status_string": (ctypes.c_char_p, [_int]),
+    "tmq_last_hip_error": (_int, []),
+    "tmq_softstep_fwd": (_int, [_vp, _vp, _sz, _dbl, _vp]),
+    "tmq_softstep_bwd": (_int, [_vp, _vp, _vp, _sz, _dbl, _dbl, _vp]),
+    "tmq_softstep_deriv_fwd": (_int, [_vp, _vp, _sz, _dbl, _dbl, _vp]),
+    "tmq_softstep_deriv_bwd": (_int, [_vp, _vp, _vp, _sz, _dbl, _dbl, _vp]),
+    "tmq_clamp_inplace": (_int, [_vp, _sz, _dbl, _dbl, _vp]),
+    "tmq_ternarize_inplace": (_int, [_vp, _sz, _dbl, _vp]),
+    "tmq_softstep_fused_workspace_bytes": (_sz, [_sz]),
+    "tmq_softstep_fused": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _dbl, _dbl, _dbl, _flt, _dbl, _dbl, _vp]),
+    "tmq_multi_plan": (_int, [ctypes.POINTER(Segment), _int, ctypes.POINTER(_u32)]),
+    "tmq_qloss_multi_workspace_bytes": (_sz, [_u32]),
+    "tmq_qloss_multi": (_int, [_vp, _int, _u32, _dbl, _dbl, _vp, _vp, _vp, _vp]),
+    "tmq_qloss_bwd_multi": (_int, [_vp, _int, _u32, _dbl, _dbl, _int, _vp]),
+    "tmq_clamp_multi": (_int, [_vp, _int, _u32, _dbl, _dbl, _vp]),
+    "tmq_pack_ternary": (_int, [_vp, _int, _i64, _i64, _vp, _vp]),
+    "tmq_unpack_ternary": (_int, [_vp, _i64, _i64, _vp, _vp]),
+    "tmq_ternary_linear": (_int, [_vp, _int, _i64, _i64, _vp, _i64, _vp, _vp, _vp, _vp]),
+    "tmq_conv2d_out_hw": (_int, [ctypes.POINTER(ConvShape), ctypes.POINTER(ctypes.c_int32),
+                                 ctypes.POINTER(ctypes.c_int32)]),
+    "tmq_ternary_conv2d": (_int, [_vp, _int, ctypes.POINTER(ConvShape), _vp, _vp, _vp, _vp, _int, _vp, _int, _vp]),
+    "tmq_compress_bound": (_sz, [_i64, _i64]),
+    "tmq_compress_ternary": (_int, [_vp, _i64, _i64, _vp, _sz, ctypes.POINTER(_sz)]),
+    "tmq_decompress_ternary": (_int, [_vp, _sz, _vp, _i64, _i64]),
+}
+
+_lib = None
+
+
+def load():
+    """Load libtmq_hip.so once and attach the prototypes. Raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(
+                f"{LIB_PATH} is missing: build it with `make -C tmq_amd/csrc` (or __graft_entry__.build()). "
+                "tmq_amd has no CPU or PyTorch fallback for its kernels.")
+        lib = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = lib
+    return _lib
+
+
+def check(status, what):
+    if status != 0:
+        lib = load()
+        msg = lib.tmq_status_string(status).decode()
+        extra = f" (hipError {lib.tmq_last_hip_error()})" if status == -3 else ""
+        raise TmqError(f"{what}: {msg}{extra}")
+
+
+def ptr(t):
+    """Device (or host) address of a tensor, None for a missing optional tensor."""
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def stream_of(t):
+    """The current HIP stream of the tensor's device, as the void* the ABI expects."""
+    return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+def dtype_code(t):
+    try:
+        return _DTYPE_CODE[t.dtype]
+    except KeyError:
+        raise ValueError("Cannot handle the supplied data-type") from None
+
+
+def require_gpu(t, name="tensor"):
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must live on the GPU")
+    if not t.is_contiguous():
+        raise RuntimeError(f"{name} must be contiguous")

@@ -1,0 +1,55 @@
+// Shared host/device helpers of libtmq_hip (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "tmq_hip.h"
+
+namespace tmq {
+
+// Records the failing hipError_t for tmq_last_hip_error() and maps it to TMQ_ERR_LAUNCH.
+int note_hip_error(hipError_t e);
+
+inline int check_launch() {
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? TMQ_OK : note_hip_error(e);
+}
+
+inline hipStream_t as_stream(void *s) { return reinterpret_cast<hipStream_t>(s); }
+
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+constexpr int kWave = 64;
+
+#if defined(__HIPCC__)
+// Sum over the 64 lanes of a wavefront with DPP row operations (no LDS traffic): butterfly
+// inside each row of 16 lanes, then the four row sums are fetched with v_readlane.
+__device__ __forceinline__ float wave_sum(float v) {
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, false));   // quad_perm [1,0,3,2]
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, false));   // quad_perm [2,3,0,1]
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, false));  // row_half_mirror
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xF, 0xF, false));  // row_mirror
+    const int iv = __builtin_bit_cast(int, v);
+    float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(iv, 0));
+    float r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(iv, 16));
+    float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(iv, 32));
+    float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(iv, 48));
+    return (r0 + r1) + (r2 + r3);
+}
+
+// Block-wide sum (blockDim.x a multiple of 64, at most 1024): wave_sum, then one LDS slot per
+// wave, then the first wave adds the slots. The result is valid in thread 0.
+__device__ __forceinline__ float block_sum(float v, float *lds /* >= 16 floats */) {
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
+    v = wave_sum(v);
+    if (lane == 0) lds[wv] = v;
+    __syncthreads();
+    float t = 0.f;
+    if (threadIdx.x == 0)
+        for (int i = 0; i < nw; i++) t += lds[i];
+    return t;
+}
+#endif
+
+}  // namespace tmq

@@ -1,0 +1,134 @@
+// 2-bit ternary pack / unpack on the GPU (gfx950).
+//
+// Format (tmq/tmq_native.cpp:152-208): a weight matrix W[N][K] (N output channels, K = fan-in,
+// for a convolution K = C*ky*kx in that order) becomes words[K][ceil(N/16)]; word (k,q) holds
+// the codes of W[16q+j][k], j = 0..15, first element in bits 31:30; 0 -> 00, +1 -> 01, -1 -> 10.
+//
+// The layout is a transpose, so the kernels tile it: a workgroup owns 64 k x 256 n. Lane = k,
+// which makes every global fp32 access a coalesced 256-byte row segment of W; each lane builds
+// (or splits) whole words in registers; words cross between the "lane = k" and the "16 words
+// per row" arrangements through a 4 KiB LDS tile so that the packed side moves 64-byte segments.
+// Both directions are bound by the fp32 side: 4 B/weight + 1/8 B/weight.
+#include "common.h"
+
+namespace tmq {
+namespace {
+
+constexpr int kTileK = 64;   // lanes of one wave
+constexpr int kTileQ = 16;   // words per tile row (256 output channels); 4 per wave
+constexpr int kThreads = 256;
+
+// float -> code with the reference's semantics: roundf (half away from zero), then the x86
+// float->int conversion (NaN and |v| >= 2^31 become INT_MIN), then clamp to [-1, 1].
+__device__ __forceinline__ uint32_t code_of(float v) {
+    if (v >= 0.5f) return v < 2147483648.0f ? 1u : 2u;
+    if (v <= -0.5f) return 2u;
+    return (v != v) ? 2u : 0u;
+}
+__device__ __forceinline__ uint32_t code_of(int32_t v) { return v > 0 ? 1u : (v < 0 ? 2u : 0u); }
+__device__ __forceinline__ uint32_t code_of(int8_t v) { return v > 0 ? 1u : (v < 0 ? 2u : 0u); }
+
+template <typename T>
+__global__ __launch_bounds__(kThreads) void pack_kernel(const T *__restrict__ w, uint32_t *__restrict__ out, int64_t N,
+                                                        int64_t K, int64_t Q) {
+    __shared__ uint32_t tile[kTileK][kTileQ + 1];
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const int64_t k0 = (int64_t)blockIdx.x * kTileK, q0 = (int64_t)blockIdx.y * kTileQ;
+    const int64_t k = k0 + lane;
+#pragma unroll
+    for (int qi = 0; qi < 4; qi++) {
+        const int ql = wv * 4 + qi;
+        const int64_t nbase = (q0 + ql) * 16;
+        uint32_t word = 0;
+        if (k < K && nbase < N) {
+            T v[16];
+#pragma unroll
+            for (int j = 0; j < 16; j++) v[j] = (nbase + j < N) ? w[(nbase + j) * K + k] : T(0);
+#pragma unroll
+            for (int j = 0; j < 16; j++) word = (word << 2) | code_of(v[j]);
+        }
+        tile[lane][ql] = word;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int row = i * 16 + (threadIdx.x >> 4), col = threadIdx.x & 15;
+        if (k0 + row < K && q0 + col < Q) out[(k0 + row) * Q + q0 + col] = tile[row][col];
+    }
+}
+
+__global__ __launch_bounds__(kThreads) void unpack_kernel(const uint32_t *__restrict__ in, float *__restrict__ w,
+                                                          int64_t N, int64_t K, int64_t Q) {
+    __shared__ uint32_t tile[kTileK][kTileQ + 1];
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const int64_t k0 = (int64_t)blockIdx.x * kTileK, q0 = (int64_t)blockIdx.y * kTileQ;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int row = i * 16 + (threadIdx.x >> 4), col = threadIdx.x & 15;
+        tile[row][col] = (k0 + row < K && q0 + col < Q) ? in[(k0 + row) * Q + q0 + col] : 0u;
+    }
+    __syncthreads();
+    const int64_t k = k0 + lane;
+    if (k >= K) return;
+#pragma unroll
+    for (int qi = 0; qi < 4; qi++) {
+        const int ql = wv * 4 + qi;
+        const int64_t nbase = (q0 + ql) * 16;
+        if (nbase >= N) break;
+        const uint32_t word = tile[lane][ql];
+#pragma unroll
+        for (int j = 0; j < 16; j++) {
+            const uint32_t c = (word >> (30 - 2 * j)) & 3u;
+            const float v = c == 1u ? 1.0f : (c == 2u ? -1.0f : 0.0f);   // 11 decodes to 0
+            if (nbase + j < N) w[(nbase + j) * K + k] = v;
+        }
+    }
+}
+
+}  // namespace
+}  // namespace tmq
+
+using namespace tmq;
+
+extern "C" {
+
+int tmq_pack_ternary(const void *w, int dtype, int64_t N, int64_t K, uint32_t *words, void *stream) {
+    if (N < 0 || K < 0) return TMQ_ERR_INVALID_ARG;
+    if (N == 0 || K == 0) return TMQ_OK;
+    if (!w || !words) return TMQ_ERR_INVALID_ARG;
+    const int64_t Q = (N + 15) / 16;
+    const int64_t gx = (K + kTileK - 1) / kTileK, gy = (Q + kTileQ - 1) / kTileQ;
+    if (gx > 0x7FFFFFFF || gy > 65535) return TMQ_ERR_TOO_LARGE;
+    dim3 grid((uint32_t)gx, (uint32_t)gy), block(kThreads);
+    switch (dtype) {
+        case TMQ_F32:
+            hipLaunchKernelGGL(pack_kernel<float>, grid, block, 0, as_stream(stream), static_cast<const float *>(w),
+                               words, N, K, Q);
+            break;
+        case TMQ_I32:
+            hipLaunchKernelGGL(pack_kernel<int32_t>, grid, block, 0, as_stream(stream),
+                               static_cast<const int32_t *>(w), words, N, K, Q);
+            break;
+        case TMQ_I8:
+            hipLaunchKernelGGL(pack_kernel<int8_t>, grid, block, 0, as_stream(stream), static_cast<const int8_t *>(w),
+                               words, N, K, Q);
+            break;
+        default:
+            return TMQ_ERR_UNSUPPORTED;
+    }
+    return check_launch();
+}
+
+int tmq_unpack_ternary(const uint32_t *words, int64_t N, int64_t K, float *w, void *stream) {
+    if (N < 0 || K < 0) return TMQ_ERR_INVALID_ARG;
+    if (N == 0 || K == 0) return TMQ_OK;
+    if (!w || !words) return TMQ_ERR_INVALID_ARG;
+    const int64_t Q = (N + 15) / 16;
+    const int64_t gx = (K + kTileK - 1) / kTileK, gy = (Q + kTileQ - 1) / kTileQ;
+    if (gx > 0x7FFFFFFF || gy > 65535) return TMQ_ERR_TOO_LARGE;
+    hipLaunchKernelGGL(unpack_kernel, dim3((uint32_t)gx, (uint32_t)gy), dim3(kThreads), 0, as_stream(stream), words, w,
+                       N, K, Q);
+    return check_launch();
+}
+
+}  // extern "C"

@@ -1,0 +1,522 @@
+// Soft-staircase transfer function family for gfx950: forward, backward, quantization-loss
+// integrand and its gradient, clamp, ternarisation, the fused single pass and the multi-tensor
+// forms. All of them are streaming fp32 kernels bounded by HBM bandwidth: every thread moves
+// dwordx4 packets (kUnroll of them per tensor, issued before the arithmetic starts) and the
+// piecewise-rational evaluation stays in VALU registers.
+//
+// Arithmetic contract: the reference's CPU path is a chain of separate torch ops, each rounding
+// to fp32 (tmq/tmq.py:353-381, 404-438, 456-493). This file is compiled with -ffp-contract=off
+// and spells every operation in that association, with IEEE-correct division, so results are
+// bit-identical to that chain. Scalars arrive as doubles and are rounded to fp32 once on the
+// host (StepK), as torch does with Python scalars.
+#include "common.h"
+
+#include <math.h>
+
+namespace tmq {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kUnroll = 4;                            // dwordx4 packets per thread per tensor
+constexpr uint32_t kChunk = kThreads * 4 * kUnroll;   // elements per block
+
+// Host-rounded scalars of one staircase evaluation.
+struct StepK {
+    float d;   // float(digamma)
+    float h;   // float(digamma / 2)
+    float c;   // float(2 * sig(digamma / 2))
+    float k1;  // float(strength * digamma)
+    float k2;  // float(strength * digamma * digamma)
+};
+
+double scalar_sigmoid(double in) {  // tmq/tmq.py:384-391, evaluated in double like Python
+    double x = fmin(3.0, fmax(-3.0, in));
+    double x2 = x * x;
+    return x * (x2 + 27.0) / (27.0 + x2 * 9.0);
+}
+
+StepK make_step(double digamma, double strength) {
+    StepK k;
+    k.d = (float)digamma;
+    k.h = (float)(digamma / 2.0);
+    k.c = (float)(2.0 * scalar_sigmoid(digamma / 2.0));
+    k.k1 = (float)(strength * digamma);
+    k.k2 = (float)(strength * digamma * digamma);
+    return k;
+}
+
+// ---- per-element arithmetic ---------------------------------------------------------------
+
+// frac = w - floor(w); `bad` marks NaN/Inf weights, for which every torch op downstream yields
+// NaN (torch.clamp propagates NaN, v_med3_f32 does not).
+struct Frac {
+    float fw, frac;
+    bool bad;
+};
+__device__ __forceinline__ Frac split(float w) {
+    Frac f;
+    f.fw = floorf(w);
+    f.frac = w - f.fw;
+    f.bad = f.frac != f.frac;
+    return f;
+}
+
+// x = clamp(d*frac - h, -3, 3) with NaN kept (tmq/tmq.py:358, 418).
+__device__ __forceinline__ float clamped_arg(const Frac &f, float d, float h) {
+    float t = d * f.frac;
+    float arg = t - h;
+    float x = __builtin_amdgcn_fmed3f(arg, -3.0f, 3.0f);
+    return f.bad ? arg : x;
+}
+
+__device__ __forceinline__ float sig_of(float x) {  // tmq/tmq.py:359-360
+    float x2 = x * x;
+    float num = x * (x2 + 27.0f);
+    float den = 27.0f + x2 * 9.0f;
+    return num / den;
+}
+__device__ __forceinline__ float dsig_of(float x) {  // tmq/tmq.py:369-370
+    float x2 = x * x;
+    float a = x2 - 9.0f;
+    float b = 3.0f + x2;
+    float num = a * a;
+    float den = (9.0f * b) * b;
+    return num / den;
+}
+__device__ __forceinline__ float d2sig_of(float x) {  // tmq/tmq.py:379-381
+    float x2 = x * x;
+    float a = x2 + 3.0f;
+    float num = (16.0f * x) * (x2 - 9.0f);
+    float den = ((3.0f * a) * a) * a;
+    return num / den;
+}
+
+__device__ __forceinline__ float clamp_keep_nan(float w, float lo, float hi) {
+    float x = __builtin_amdgcn_fmed3f(w, lo, hi);
+    return (w != w) ? w : x;
+}
+
+// ---- element operators ----------------------------------------------------------------------
+// Each Op declares which streams it touches; `apply` sees one element.
+//   in0  : weight            (always loaded)
+//   in1  : second input      (kIn1)
+//   out0..out2 : outputs     (kOut0..2); out0 may alias in0 for the in-place ops
+//   acc  : per-thread loss accumulator (kLoss)
+
+struct FwdOp {  // tmq/tmq.py:417-419
+    static constexpr bool kIn1 = false, kOut0 = true, kOut1 = false, kOut2 = false, kLoss = false, kReadOut1 = false;
+    StepK s;
+    __device__ __forceinline__ void apply(float w, float, float, float &o0, float &, float &, float &) const {
+        Frac f = split(w);
+        float x = clamped_arg(f, s.d, s.h);
+        float v = sig_of(x) / s.c;
+        o0 = (v + 0.5f) + f.fw;
+    }
+};
+
+struct BwdOp {  // tmq/tmq.py:434-438
+    static constexpr bool kIn1 = true, kOut0 = true, kOut1 = false, kOut2 = false, kLoss = false, kReadOut1 = false;
+    StepK s;
+    float scale;
+    __device__ __forceinline__ void apply(float w, float g, float, float &o0, float &, float &, float &) const {
+        Frac f = split(w);
+        float x = clamped_arg(f, s.d, s.h);
+        float grad = (s.d * dsig_of(x)) / s.c;
+        o0 = (scale * g) * grad;
+    }
+};
+
+struct DerivFwdOp {  // tmq/tmq.py:469-473
+    static constexpr bool kIn1 = false, kOut0 = true, kOut1 = false, kOut2 = false, kLoss = false, kReadOut1 = false;
+    StepK s;
+    __device__ __forceinline__ void apply(float w, float, float, float &o0, float &, float &, float &) const {
+        Frac f = split(w);
+        float x = clamped_arg(f, s.d, s.h);
+        o0 = (s.k1 * dsig_of(x)) / s.c;
+    }
+};
+
+struct DerivBwdOp {  // tmq/tmq.py:488-493
+    static constexpr bool kIn1 = true, kOut0 = true, kOut1 = false, kOut2 = false, kLoss = false, kReadOut1 = false;
+    StepK s;
+    __device__ __forceinline__ void apply(float w, float g, float, float &o0, float &, float &, float &) const {
+        Frac f = split(w);
+        float x = clamped_arg(f, s.d, s.h);
+        float grad = (s.k2 * d2sig_of(x)) / s.c;
+        o0 = g * grad;
+    }
+};
+
+struct ClampOp {  // tmq/tmq.py:696, 879 (in place: out0 aliases in0)
+    static constexpr bool kIn1 = false, kOut0 = true, kOut1 = false, kOut2 = false, kLoss = false, kReadOut1 = false;
+    float lo, hi;
+    __device__ __forceinline__ void apply(float w, float, float, float &o0, float &, float &, float &) const {
+        o0 = clamp_keep_nan(w, lo, hi);
+    }
+};
+
+struct TernarizeOp {  // tmq/tmq.py:293-295 with SoftStep.map 335-338 (in place)
+    static constexpr bool kIn1 = false, kOut0 = true, kOut1 = false, kOut2 = false, kLoss = false, kReadOut1 = false;
+    StepK s;
+    bool use_map;
+    __device__ __forceinline__ void apply(float w, float, float, float &o0, float &, float &, float &) const {
+        float v = w;
+        if (use_map) {
+            float fw = floorf(w);
+            float arg = (s.d * w - s.d * fw) - s.h;  // association of SoftStep.map
+            float x = __builtin_amdgcn_fmed3f(arg, -3.0f, 3.0f);
+            x = (arg != arg) ? arg : x;
+            float t = sig_of(x) / s.c;
+            v = (t + 0.5f) + fw;
+        }
+        o0 = rintf(v);  // torch.round: half to even
+    }
+};
+
+// Loss only: acc += q(w). Used by the multi-tensor quantization loss.
+struct QLossOp {
+    static constexpr bool kIn1 = false, kOut0 = false, kOut1 = false, kOut2 = false, kLoss = true, kReadOut1 = false;
+    StepK q;  // sharpness constants
+    __device__ __forceinline__ void apply(float w, float, float, float &, float &, float &, float &acc) const {
+        Frac f = split(w);
+        float x = clamped_arg(f, q.d, q.h);
+        acc += (q.k1 * dsig_of(x)) / q.c;
+    }
+};
+
+// aux (=|+=) scalar * Q'(w): gradient of the mean quantization loss (out1 is the aux tensor).
+template <bool ACC>
+struct QLossBwdOp {
+    static constexpr bool kIn1 = false, kOut0 = false, kOut1 = true, kOut2 = false, kLoss = false, kReadOut1 = ACC;
+    StepK q;
+    __device__ __forceinline__ void apply(float w, float, float sc, float &, float &o1, float &, float &) const {
+        Frac f = split(w);
+        float x = clamped_arg(f, q.d, q.h);
+        float grad = (q.k2 * d2sig_of(x)) / q.c;
+        float t = sc * grad;
+        o1 = ACC ? (o1 + t) : t;
+    }
+};
+
+// The fused pass. MASK bits: 1 = y, 2 = dw, 4 = clamp(w), 8 = loss sum.
+template <int MASK>
+struct FusedOp {
+    static constexpr bool kIn1 = (MASK & 2) != 0, kOut0 = (MASK & 1) != 0, kOut1 = (MASK & 2) != 0,
+                          kOut2 = (MASK & 4) != 0, kLoss = (MASK & 8) != 0, kReadOut1 = false;
+    StepK s;  // hardness constants (forward / backward)
+    StepK q;  // sharpness constants (quantization loss)
+    float gl, lo, hi;
+    __device__ __forceinline__ void apply(float w, float g, float, float &o0, float &o1, float &o2, float &acc) const {
+        Frac f = split(w);
+        if constexpr ((MASK & 3) != 0) {
+            float x = clamped_arg(f, s.d, s.h);
+            if constexpr ((MASK & 1) != 0) {
+                float v = sig_of(x) / s.c;
+                o0 = (v + 0.5f) + f.fw;
+            }
+            if constexpr ((MASK & 2) != 0) {
+                float grad = (s.d * dsig_of(x)) / s.c;
+                float t1 = g * grad;  // scale is 1.0 at every reference call site (tmq/tmq.py:650, 812)
+                float x5 = clamped_arg(f, q.d, q.h);
+                float gq = (q.k2 * d2sig_of(x5)) / q.c;
+                float t2 = gl * gq;
+                o1 = t1 + t2;
+            }
+        }
+        if constexpr ((MASK & 8) != 0) {
+            float x5 = clamped_arg(f, q.d, q.h);
+            acc += (q.k1 * dsig_of(x5)) / q.c;
+        }
+        if constexpr ((MASK & 4) != 0) o2 = clamp_keep_nan(w, lo, hi);
+    }
+};
+
+// ---- tensor locators ------------------------------------------------------------------------
+struct View {
+    const float *in0;
+    const float *in1;
+    float *out0, *out1, *out2;
+    uint64_t n;
+    uint32_t block;  // block index inside this tensor
+    float scalar;
+    bool vec;        // all pointers 16-byte aligned
+};
+
+struct Single {
+    const float *in0;
+    const float *in1;
+    float *out0, *out1, *out2;
+    uint64_t n;
+    bool vec;
+    __device__ __forceinline__ View locate(uint32_t b) const {
+        return View{in0, in1, out0, out1, out2, n, b, 0.f, vec};
+    }
+};
+
+// Multi-tensor: binary search of the block range table (wave-uniform, scalar loads).
+struct Multi {
+    const tmq_segment *segs;
+    int nseg;
+    int inplace;  // out0 = ptr (in-place ops); out1 = aux
+    __device__ __forceinline__ View locate(uint32_t b) const {
+        int lo = 0, hi = nseg - 1;
+        while (lo < hi) {
+            int mid = (lo + hi + 1) >> 1;
+            if (segs[mid].block_begin <= b) lo = mid;
+            else hi = mid - 1;
+        }
+        const tmq_segment s = segs[lo];
+        float *p = static_cast<float *>(s.ptr);
+        float *a = static_cast<float *>(s.aux);
+        bool vec = ((reinterpret_cast<uintptr_t>(p) | reinterpret_cast<uintptr_t>(a)) & 15u) == 0;
+        return View{p, nullptr, inplace ? p : nullptr, a, nullptr, s.n, b - s.block_begin, s.scalar, vec};
+    }
+};
+
+// ---- the streaming kernel ---------------------------------------------------------------------
+template <class Op, class Loc>
+__global__ __launch_bounds__(kThreads) void stream_kernel(Loc loc, Op op, float *partials) {
+    __shared__ float lds[16];
+    const View v = loc.locate(blockIdx.x);
+    const uint64_t base = (uint64_t)v.block * kChunk;
+    const int tid = threadIdx.x;
+    float acc = 0.f;
+
+    if (base + kChunk <= v.n && v.vec) {
+        // Full chunk: issue every load first, then compute, then store.
+        float4 a[kUnroll], b[kUnroll], r1[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; u++) {
+            const uint64_t i = base + (uint64_t)(u * kThreads + tid) * 4;
+            a[u] = *reinterpret_cast<const float4 *>(v.in0 + i);
+            if constexpr (Op::kIn1) b[u] = *reinterpret_cast<const float4 *>(v.in1 + i);
+            if constexpr (Op::kReadOut1) r1[u] = *reinterpret_cast<const float4 *>(v.out1 + i);
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; u++) {
+            const uint64_t i = base + (uint64_t)(u * kThreads + tid) * 4;
+            float4 o0, o1, o2;
+            if constexpr (Op::kReadOut1) o1 = r1[u];
+            float gx = 0.f, gy = 0.f, gz = 0.f, gw = 0.f;
+            if constexpr (Op::kIn1) { gx = b[u].x; gy = b[u].y; gz = b[u].z; gw = b[u].w; }
+            op.apply(a[u].x, gx, v.scalar, o0.x, o1.x, o2.x, acc);
+            op.apply(a[u].y, gy, v.scalar, o0.y, o1.y, o2.y, acc);
+            op.apply(a[u].z, gz, v.scalar, o0.z, o1.z, o2.z, acc);
+            op.apply(a[u].w, gw, v.scalar, o0.w, o1.w, o2.w, acc);
+            if constexpr (Op::kOut0) *reinterpret_cast<float4 *>(v.out0 + i) = o0;
+            if constexpr (Op::kOut1) *reinterpret_cast<float4 *>(v.out1 + i) = o1;
+            if constexpr (Op::kOut2) *reinterpret_cast<float4 *>(v.out2 + i) = o2;
+        }
+    } else {
+        // Ragged tail or unaligned tensor: element-wise, coalesced dword accesses.
+        for (int u = 0; u < kUnroll * 4; u++) {
+            const uint64_t i = base + (uint64_t)(u * kThreads + tid);
+            if (i < v.n) {
+                float o0, o1 = 0.f, o2;
+                float g = 0.f;
+                if constexpr (Op::kIn1) g = v.in1[i];
+                if constexpr (Op::kReadOut1) o1 = v.out1[i];
+                op.apply(v.in0[i], g, v.scalar, o0, o1, o2, acc);
+                if constexpr (Op::kOut0) v.out0[i] = o0;
+                if constexpr (Op::kOut1) v.out1[i] = o1;
+                if constexpr (Op::kOut2) v.out2[i] = o2;
+            }
+        }
+    }
+    if constexpr (Op::kLoss) {
+        float s = block_sum(acc, lds);
+        if (tid == 0) partials[blockIdx.x] = s;
+    }
+}
+
+// Ordered fp64 finalisation of block partial sums. One block; segment l owns the partials
+// [begin_l, begin_{l+1}). mean_l = float(sum_l / n_l); total = fp32 running sum in table order
+// (the reference adds per-layer means one by one, tmq/tmq.py:309).
+__global__ __launch_bounds__(kThreads) void finalize_kernel(const tmq_segment *segs, int nseg, uint32_t total_blocks,
+                                                           const float *partials, float *per_tensor, float *total,
+                                                           double *sum_out) {
+    __shared__ double red[kThreads];
+    float running = 0.f;
+    for (int l = 0; l < nseg; l++) {
+        const uint32_t b0 = segs ? segs[l].block_begin : 0u;
+        const uint32_t b1 = segs ? (l + 1 < nseg ? segs[l + 1].block_begin : total_blocks) : total_blocks;
+        double s = 0.0;
+        for (uint32_t i = b0 + threadIdx.x; i < b1; i += kThreads) s += (double)partials[i];
+        red[threadIdx.x] = s;
+        __syncthreads();
+        for (int off = kThreads / 2; off > 0; off >>= 1) {
+            if ((int)threadIdx.x < off) red[threadIdx.x] += red[threadIdx.x + off];
+            __syncthreads();
+        }
+        if (threadIdx.x == 0) {
+            if (sum_out) sum_out[l] = red[0];
+            if (segs) {
+                const uint64_t n = segs[l].n;
+                float mean = (float)(red[0] / (double)n);  // n == 0 gives NaN like torch.mean of an empty tensor
+                if (per_tensor) per_tensor[l] = mean;
+                running = (l == 0) ? mean : running + mean;
+            }
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0 && total) *total = running;
+}
+
+inline uint32_t blocks_for(uint64_t n) { return (uint32_t)((n + kChunk - 1) / kChunk); }
+constexpr uint64_t kMaxElems = (uint64_t)0x7FFFFFFFu * kChunk / 2;  // keeps block counts in 31 bits
+
+template <class Op>
+int launch_single(const Op &op, const float *in0, const float *in1, float *o0, float *o1, float *o2, size_t n,
+                  float *partials, void *stream) {
+    if (n == 0) return TMQ_OK;
+    if (n > kMaxElems) return TMQ_ERR_TOO_LARGE;
+    Single loc{in0, in1, o0, o1, o2, (uint64_t)n,
+               aligned16(in0) && aligned16(in1) && aligned16(o0) && aligned16(o1) && aligned16(o2)};
+    hipLaunchKernelGGL((stream_kernel<Op, Single>), dim3(blocks_for(n)), dim3(kThreads), 0, as_stream(stream), loc, op,
+                       partials);
+    return check_launch();
+}
+
+template <class Op>
+int launch_multi(const Op &op, const tmq_segment *segs, int nseg, uint32_t total_blocks, int inplace, float *partials,
+                 void *stream) {
+    if (nseg < 0 || (nseg > 0 && !segs)) return TMQ_ERR_INVALID_ARG;
+    if (nseg == 0 || total_blocks == 0) return TMQ_OK;
+    Multi loc{segs, nseg, inplace};
+    hipLaunchKernelGGL((stream_kernel<Op, Multi>), dim3(total_blocks), dim3(kThreads), 0, as_stream(stream), loc, op,
+                       partials);
+    return check_launch();
+}
+
+bool bad_hardness(double d) { return !(d > 0.0) || !(d <= 1.0e6); }
+
+}  // namespace
+}  // namespace tmq
+
+using namespace tmq;
+
+extern "C" {
+
+int tmq_softstep_fwd(const float *w, float *y, size_t n, double digamma, void *stream) {
+    if (n && (!w || !y)) return TMQ_ERR_INVALID_ARG;
+    if (bad_hardness(digamma)) return TMQ_ERR_INVALID_ARG;
+    FwdOp op{make_step(digamma, 0.0)};
+    return launch_single(op, w, nullptr, y, nullptr, nullptr, n, nullptr, stream);
+}
+
+int tmq_softstep_bwd(const float *w, const float *g, float *dw, size_t n, double digamma, double scale,
+                     void *stream) {
+    if (n && (!w || !g || !dw)) return TMQ_ERR_INVALID_ARG;
+    if (bad_hardness(digamma)) return TMQ_ERR_INVALID_ARG;
+    BwdOp op{make_step(digamma, 0.0), (float)scale};
+    return launch_single(op, w, g, dw, nullptr, nullptr, n, nullptr, stream);
+}
+
+int tmq_softstep_deriv_fwd(const float *w, float *q, size_t n, double digamma, double strength, void *stream) {
+    if (n && (!w || !q)) return TMQ_ERR_INVALID_ARG;
+    if (bad_hardness(digamma)) return TMQ_ERR_INVALID_ARG;
+    DerivFwdOp op{make_step(digamma, strength)};
+    return launch_single(op, w, nullptr, q, nullptr, nullptr, n, nullptr, stream);
+}
+
+int tmq_softstep_deriv_bwd(const float *w, const float *g, float *dw, size_t n, double digamma, double strength,
+                           void *stream) {
+    if (n && (!w || !g || !dw)) return TMQ_ERR_INVALID_ARG;
+    if (bad_hardness(digamma)) return TMQ_ERR_INVALID_ARG;
+    DerivBwdOp op{make_step(digamma, strength)};
+    return launch_single(op, w, g, dw, nullptr, nullptr, n, nullptr, stream);
+}
+
+int tmq_clamp_inplace(float *w, size_t n, double lo, double hi, void *stream) {
+    if (n && !w) return TMQ_ERR_INVALID_ARG;
+    if (!(lo <= hi)) return TMQ_ERR_INVALID_ARG;
+    ClampOp op{(float)lo, (float)hi};
+    return launch_single(op, w, nullptr, w, nullptr, nullptr, n, nullptr, stream);
+}
+
+int tmq_ternarize_inplace(float *w, size_t n, double digamma, void *stream) {
+    if (n && !w) return TMQ_ERR_INVALID_ARG;
+    const bool use_map = digamma > 0.0;
+    if (use_map && bad_hardness(digamma)) return TMQ_ERR_INVALID_ARG;
+    TernarizeOp op{make_step(use_map ? digamma : 1.0, 0.0), use_map};
+    return launch_single(op, w, nullptr, w, nullptr, nullptr, n, nullptr, stream);
+}
+
+size_t tmq_softstep_fused_workspace_bytes(size_t n) { return (size_t)blocks_for(n) * sizeof(float) + 16; }
+
+int tmq_softstep_fused(const float *w, const float *g, float *y, float *dw, float *wc, double *loss_sum,
+                       void *workspace, size_t n, double digamma, double sharpness, double strength, float gl,
+                       double lo, double hi, void *stream) {
+    if (n && !w) return TMQ_ERR_INVALID_ARG;
+    if (dw && !g) return TMQ_ERR_INVALID_ARG;
+    if (loss_sum && !workspace) return TMQ_ERR_INVALID_ARG;
+    if (bad_hardness(digamma) || bad_hardness(sharpness) || !(lo <= hi)) return TMQ_ERR_INVALID_ARG;
+    if (n > kMaxElems) return TMQ_ERR_TOO_LARGE;
+    const int mask = (y ? 1 : 0) | (dw ? 2 : 0) | (wc ? 4 : 0) | (loss_sum ? 8 : 0);
+    if (mask == 0) return TMQ_OK;
+    float *partials = static_cast<float *>(workspace);
+    const StepK s = make_step(digamma, 0.0), q = make_step(sharpness, strength);
+    int rc = TMQ_OK;
+    if (n) {
+        switch (mask) {
+#define TMQ_CASE(M)                                                                               \
+    case M: {                                                                                     \
+        FusedOp<M> op{s, q, gl, (float)lo, (float)hi};                                            \
+        rc = launch_single(op, w, g, y, dw, wc, n, partials, stream);                             \
+    } break;
+            TMQ_CASE(1) TMQ_CASE(2) TMQ_CASE(3) TMQ_CASE(4) TMQ_CASE(5) TMQ_CASE(6) TMQ_CASE(7) TMQ_CASE(8)
+            TMQ_CASE(9) TMQ_CASE(10) TMQ_CASE(11) TMQ_CASE(12) TMQ_CASE(13) TMQ_CASE(14) TMQ_CASE(15)
+#undef TMQ_CASE
+        }
+        if (rc != TMQ_OK) return rc;
+    }
+    if (loss_sum) {
+        hipLaunchKernelGGL(finalize_kernel, dim3(1), dim3(kThreads), 0, as_stream(stream), nullptr, 1, blocks_for(n),
+                           partials, nullptr, nullptr, loss_sum);
+        rc = check_launch();
+    }
+    return rc;
+}
+
+int tmq_multi_plan(tmq_segment *segs, int nseg, uint32_t *total_blocks) {
+    if (nseg < 0 || (nseg > 0 && !segs) || !total_blocks) return TMQ_ERR_INVALID_ARG;
+    uint64_t b = 0;
+    for (int i = 0; i < nseg; i++) {
+        if (segs[i].n > kMaxElems) return TMQ_ERR_TOO_LARGE;
+        segs[i].block_begin = (uint32_t)b;
+        b += blocks_for(segs[i].n);
+        if (b > 0x7FFFFFFFull) return TMQ_ERR_TOO_LARGE;
+    }
+    *total_blocks = (uint32_t)b;
+    return TMQ_OK;
+}
+
+size_t tmq_qloss_multi_workspace_bytes(uint32_t total_blocks) { return (size_t)total_blocks * sizeof(float) + 16; }
+
+int tmq_qloss_multi(const tmq_segment *segs, int nseg, uint32_t total_blocks, double sharpness, double strength,
+                    float *per_tensor, float *total, void *workspace, void *stream) {
+    if (nseg <= 0 || !segs || !workspace) return TMQ_ERR_INVALID_ARG;
+    if (bad_hardness(sharpness)) return TMQ_ERR_INVALID_ARG;
+    float *partials = static_cast<float *>(workspace);
+    QLossOp op{make_step(sharpness, strength)};
+    int rc = launch_multi(op, segs, nseg, total_blocks, 0, partials, stream);
+    if (rc != TMQ_OK) return rc;
+    hipLaunchKernelGGL(finalize_kernel, dim3(1), dim3(kThreads), 0, as_stream(stream), segs, nseg, total_blocks,
+                       partials, per_tensor, total, nullptr);
+    return check_launch();
+}
+
+int tmq_qloss_bwd_multi(const tmq_segment *segs, int nseg, uint32_t total_blocks, double sharpness, double strength,
+                        int accumulate, void *stream) {
+    if (bad_hardness(sharpness)) return TMQ_ERR_INVALID_ARG;
+    const StepK q = make_step(sharpness, strength);
+    if (accumulate) return launch_multi(QLossBwdOp<true>{q}, segs, nseg, total_blocks, 0, nullptr, stream);
+    return launch_multi(QLossBwdOp<false>{q}, segs, nseg, total_blocks, 0, nullptr, stream);
+}
+
+int tmq_clamp_multi(const tmq_segment *segs, int nseg, uint32_t total_blocks, double lo, double hi, void *stream) {
+    if (!(lo <= hi)) return TMQ_ERR_INVALID_ARG;
+    return launch_multi(ClampOp{(float)lo, (float)hi}, segs, nseg, total_blocks, 1, nullptr, stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,300 @@
+"""Operator layer: the native-binding names of the reference (tmq_cuda / tmq_native), same
+argument order and error behaviour, implemented on libtmq_hip through its C ABI.
+
+Reference bindings: tmq/tmq_cuda.cu:800-809 and tmq/tmq_native.cpp:550-555. Every function
+returns a newly allocated tensor owned by the caller and never mutates its inputs, like the
+reference. Additive entry points (fused pass, multi-tensor forms, in-place clamp/ternarise, GPU
+pack/unpack) follow below the drop-in ones.
+"""
+import ctypes
+
+import torch
+
+from . import _capi
+from ._capi import check, ptr, stream_of
+
+
+def _lib():
+    return _capi.load()
+
+
+def _f32_cuda(t, name):
+    # tmq/tmq_cuda.cu:691-707: device check first, then the dtype ladder.
+    if not t.is_cuda:
+        raise RuntimeError(f"{name}: expected a tensor on the GPU")
+    if t.dtype == torch.float16:
+        raise ValueError("Not implemented yet")
+    if t.dtype != torch.float32:
+        raise ValueError("Expected either a float16 or a float32 tensor as input/output")
+    return t if t.is_contiguous() else t.contiguous()
+
+
+# ---- drop-in: soft-step family -------------------------------------------------------------
+def fwd_softstep(weights: torch.Tensor, digamma: float) -> torch.Tensor:
+    """Forward mapping for the soft-step function (tmq/tmq_cuda.cu:740-764)."""
+    w = _f32_cuda(weights, "fwd_softstep")
+    out = torch.empty_like(w)
+    with torch.cuda.device(w.device):
+        check(_lib().tmq_softstep_fwd(ptr(w), ptr(out), w.numel(), float(digamma), stream_of(w)), "fwd_softstep")
+    return out.view(weights.shape)
+
+
+def bwd_softstep(weights: torch.Tensor, digamma: float, scale: float, grad: torch.Tensor) -> torch.Tensor:
+    """Backward mapping incl. gradient multiplication (tmq/tmq_cuda.cu:768-794)."""
+    w = _f32_cuda(weights, "bwd_softstep")
+    if not grad.is_cuda:
+        raise RuntimeError("bwd_softstep: expected a gradient on the GPU")
+    if grad.dtype != w.dtype or grad.numel() != w.numel():
+        raise RuntimeError("bwd_softstep: gradient must match the weights in dtype and size")
+    g = grad if grad.is_contiguous() else grad.contiguous()
+    out = torch.empty_like(w)
+    with torch.cuda.device(w.device):
+        check(_lib().tmq_softstep_bwd(ptr(w), ptr(g), ptr(out), w.numel(), float(digamma), float(scale),
+                                      stream_of(w)), "bwd_softstep")
+    return out.view(weights.shape)
+
+
+def fwd_softstep_derivative(weights: torch.Tensor, digamma: float, strength: float) -> torch.Tensor:
+    """Forward mapping for the derivative of the soft-step function (tmq/tmq_cuda.cu:690-709)."""
+    w = _f32_cuda(weights, "fwd_softstep_derivative")
+    out = torch.empty_like(w)
+    with torch.cuda.device(w.device):
+        check(_lib().tmq_softstep_deriv_fwd(ptr(w), ptr(out), w.numel(), float(digamma), float(strength),
+                                            stream_of(w)), "fwd_softstep_derivative")
+    return out.view(weights.shape)
+
+
+def bwd_softstep_derivative(weights: torch.Tensor, digamma: float, scale: float, grad: torch.Tensor) -> torch.Tensor:
+    """Backward mapping for the derivative (tmq/tmq_cuda.cu:713-735); `scale` is the strength."""
+    w = _f32_cuda(weights, "bwd_softstep_derivative")
+    if not grad.is_cuda:
+        raise RuntimeError("bwd_softstep_derivative: expected a gradient on the GPU")
+    if grad.dtype != w.dtype or grad.numel() != w.numel():
+        raise RuntimeError("bwd_softstep_derivative: gradient must match the weights in dtype and size")
+    g = grad if grad.is_contiguous() else grad.contiguous()
+    out = torch.empty_like(w)
+    with torch.cuda.device(w.device):
+        check(_lib().tmq_softstep_deriv_bwd(ptr(w), ptr(g), ptr(out), w.numel(), float(digamma), float(scale),
+                                            stream_of(w)), "bwd_softstep_derivative")
+    return out.view(weights.shape)
+
+
+# ---- additive: in-place clamp / ternarise, fused pass -----------------------------------------
+def clamp_(weights: torch.Tensor, lo: float, hi: float) -> torch.Tensor:
+    """In-place clamp of an fp32 GPU tensor (value-equivalent to tmq/tmq.py:696, 879)."""
+    _capi.require_gpu(weights, "weights")
+    if weights.dtype != torch.float32:
+        raise ValueError("clamp_: fp32 only")
+    with torch.cuda.device(weights.device):
+        check(_lib().tmq_clamp_inplace(ptr(weights), weights.numel(), float(lo), float(hi), stream_of(weights)),
+              "clamp_")
+    return weights
+
+
+def ternarize_(weights: torch.Tensor, digamma: float = 0.0) -> torch.Tensor:
+    """In place: round_half_even(SoftStep.map(w; digamma)) (tmq/tmq.py:293-295); digamma <= 0
+    gives plain round_half_even (tmq/tmq.py:603, 886, 1109)."""
+    _capi.require_gpu(weights, "weights")
+    if weights.dtype != torch.float32:
+        raise ValueError("ternarize_: fp32 only")
+    with torch.cuda.device(weights.device):
+        check(_lib().tmq_ternarize_inplace(ptr(weights), weights.numel(), float(digamma), stream_of(weights)),
+              "ternarize_")
+    return weights
+
+
+def softstep_fused(weights, grad, digamma, sharpness, strength, gl, lo, hi, *, want_y=True, want_dw=True,
+                   want_clamp=True, want_loss=True, clamp_inplace=False, out=None):
+    """One pass: y = S(w), dw = g*S'(w) + gl*Q'(w), wc = clamp(w), loss_sum = sum q(w).
+
+    Returns (y, dw, wc, loss_sum) with None for outputs not requested; loss_sum is a 1-element
+    fp64 tensor. `out` may carry preallocated (y, dw, wc, loss_sum, workspace) to keep
+    allocations out of a timed loop."""
+    _capi.require_gpu(weights, "weights")
+    w = weights
+    n = w.numel()
+    lib = _lib()
+    if out is not None:
+        y, dw, wc, loss, ws = out
+    else:
+        y = torch.empty_like(w) if want_y else None
+        dw = torch.empty_like(w) if want_dw else None
+        wc = (w if clamp_inplace else torch.empty_like(w)) if want_clamp else None
+        loss = torch.empty(1, dtype=torch.float64, device=w.device) if want_loss else None
+        ws = torch.empty(lib.tmq_softstep_fused_workspace_bytes(n), dtype=torch.uint8, device=w.device) \
+            if want_loss else None
+    if dw is not None:
+        _capi.require_gpu(grad, "grad")
+        if grad.numel() != n or grad.dtype != torch.float32:
+            raise RuntimeError("softstep_fused: gradient must match the weights")
+    with torch.cuda.device(w.device):
+        check(lib.tmq_softstep_fused(ptr(w), ptr(grad) if dw is not None else None, ptr(y), ptr(dw), ptr(wc),
+                                     ptr(loss), ptr(ws), n, float(digamma), float(sharpness), float(strength),
+                                     ctypes.c_float(gl), float(lo), float(hi), stream_of(w)), "softstep_fused")
+    return y, dw, wc, loss
+
+
+# ---- additive: multi-tensor forms ----------------------------------------------------------------
+class SegmentTable:
+    """Device-resident table of (weight, aux, n, scalar) for the multi-tensor launches. Build it
+    once per set of tensors; rebuild when a tensor is reallocated."""
+
+    def __init__(self, tensors, aux=None, scalars=None):
+        lib = _lib()
+        self.nseg = len(tensors)
+        if self.nseg == 0:
+            raise ValueError("SegmentTable: no tensors")
+        dev = tensors[0].device
+        arr = (_capi.Segment * self.nseg)()
+        for i, t in enumerate(tensors):
+            _capi.require_gpu(t, "segment tensor")
+            if t.dtype != torch.float32 or t.device != dev:
+                raise ValueError("SegmentTable: fp32 tensors on one device only")
+            a = aux[i] if aux is not None else None
+            if a is not None:
+                _capi.require_gpu(a, "segment aux tensor")
+                if a.numel() != t.numel() or a.dtype != torch.float32:
+                    raise ValueError("SegmentTable: aux must match its tensor")
+            arr[i].ptr = t.data_ptr()
+            arr[i].aux = a.data_ptr() if a is not None else None
+            arr[i].n = t.numel()
+            arr[i].scalar = float(scalars[i]) if scalars is not None else 0.0
+        total = ctypes.c_uint32(0)
+        check(lib.tmq_multi_plan(arr, self.nseg, ctypes.byref(total)), "tmq_multi_plan")
+        self.total_blocks = total.value
+        self.key = tuple((t.data_ptr(), t.numel()) for t in tensors) + \
+            tuple(a.data_ptr() if a is not None else 0 for a in (aux or []))
+        host = torch.frombuffer(bytearray(bytes(arr)), dtype=torch.uint8)
+        self.device = dev
+        self.table = host.to(dev)
+        self.workspace = torch.empty(lib.tmq_qloss_multi_workspace_bytes(self.total_blocks), dtype=torch.uint8,
+                                     device=dev)
+        self._keep = (list(tensors), list(aux) if aux is not None else None)
+
+
+def qloss_multi(table: SegmentTable, sharpness: float, strength: float):
+    """(per_tensor_means [nseg] fp32, total [1] fp32) in one launch + an ordered finalisation."""
+    per = torch.empty(table.nseg, dtype=torch.float32, device=table.device)
+    tot = torch.empty(1, dtype=torch.float32, device=table.device)
+    with torch.cuda.device(table.device):
+        check(_lib().tmq_qloss_multi(ptr(table.table), table.nseg, table.total_blocks, float(sharpness),
+                                     float(strength), ptr(per), ptr(tot), ptr(table.workspace),
+                                     stream_of(table.table)), "qloss_multi")
+    return per, tot
+
+
+def qloss_bwd_multi(table: SegmentTable, sharpness: float, strength: float, accumulate: bool):
+    """aux_l (=|+=) scalar_l * Q'(w_l) for every segment, one launch."""
+    with torch.cuda.device(table.device):
+        check(_lib().tmq_qloss_bwd_multi(ptr(table.table), table.nseg, table.total_blocks, float(sharpness),
+                                         float(strength), int(bool(accumulate)), stream_of(table.table)),
+              "qloss_bwd_multi")
+
+
+def clamp_multi_(table: SegmentTable, lo: float, hi: float):
+    """In-place clamp of every segment's weight tensor, one launch."""
+    with torch.cuda.device(table.device):
+        check(_lib().tmq_clamp_multi(ptr(table.table), table.nseg, table.total_blocks, float(lo), float(hi),
+                                     stream_of(table.table)), "clamp_multi_")
+
+
+# ---- drop-in: 2-bit packing (tmq_native) ---------------------------------------------------------
+def _gpu_device():
+    if not torch.cuda.is_available():
+        raise RuntimeError("tmq_amd needs a GPU: its pack/unpack kernels have no CPU fallback")
+    return torch.device("cuda", torch.cuda.current_device())
+
+
+def compactify_ternary(input: torch.Tensor) -> torch.Tensor:
+    """Encode a ternary weight tensor into 16 elements per 32-bit word (tmq/tmq_native.cpp:418-425).
+
+    [out, in] -> int32 [in, ceil(out/16)]; [out, in, ky, kx] -> int32 [in, ky, kx, ceil(out/16)].
+    fp32 / int32 / int8 input. The reference accepts CPU tensors only; here a CPU tensor is staged
+    through the GPU and the result returned on the CPU, a GPU tensor is packed in place on its
+    device."""
+    if input.dim() > 2 and input.dim() != 4:
+        raise RuntimeError("compactify_ternary: expected a tensor with at most 2 or exactly 4 dimensions")
+    if input.dim() < 2:
+        raise RuntimeError("compactify_ternary: expected at least 2 dimensions")
+    if input.dtype not in (torch.float32, torch.int32, torch.int8):
+        raise ValueError("Cannot handle the supplied data-type")
+    on_cpu = not input.is_cuda
+    src = input.to(_gpu_device()) if on_cpu else input
+    src = src.contiguous()
+    N = src.shape[0]
+    K = src.numel() // N if N else 0
+    Q = (N + 15) // 16
+    shape = (src.shape[1], Q) if src.dim() == 2 else (src.shape[1], src.shape[2], src.shape[3], Q)
+    out = torch.empty(shape, dtype=torch.int32, device=src.device)
+    with torch.cuda.device(src.device):
+        check(_lib().tmq_pack_ternary(ptr(src), _capi.dtype_code(src), N, K, ptr(out), stream_of(src)),
+              "compactify_ternary")
+    return out.cpu() if on_cpu else out
+
+
+def expand_ternary(input: torch.Tensor, orig_shape, entropy_decode: bool = False) -> torch.Tensor:
+    """Decode compact (or, with entropy_decode, range-coded) ternary weights to fp32 in the original
+    shape (tmq/tmq_native.cpp:516-544). For 2-D tensors this is the true inverse of
+    compactify_ternary (the reference decodes them with rows and columns swapped)."""
+    orig_shape = [int(s) for s in orig_shape]
+    if entropy_decode:
+        input = decompress_ternary(input, orig_shape)
+    if input.dtype != torch.int32:
+        raise RuntimeError("expand_ternary: expected an int32 tensor")
+    if len(orig_shape) not in (2, 4):
+        raise ValueError("Shape needs to be of dim 2 or 4")
+    on_cpu = not input.is_cuda
+    src = (input.to(_gpu_device()) if on_cpu else input).contiguous()
+    N = orig_shape[0]
+    K = 1
+    for s in orig_shape[1:]:
+        K *= s
+    if src.numel() != K * ((N + 15) // 16):
+        raise RuntimeError("expand_ternary: packed tensor does not match the original shape")
+    out = torch.empty(orig_shape, dtype=torch.float32, device=src.device)
+    with torch.cuda.device(src.device):
+        check(_lib().tmq_unpack_ternary(ptr(src), N, K, ptr(out), stream_of(src)), "expand_ternary")
+    return out.cpu() if on_cpu else out
+
+
+def compress_ternary(input: torch.Tensor, orig_shape, from_compact: bool) -> torch.Tensor:
+    """Range-code a ternary weight tensor (tmq/tmq_native.cpp:439-477). Returns a 1-D int8 CPU tensor.
+    from_compact=True takes the int32 compact tensor, else fp32 weights (packed first)."""
+    orig_shape = [int(s) for s in orig_shape]
+    if from_compact:
+        if input.dtype != torch.int32 or input.dim() not in (2, 4):
+            raise RuntimeError("compress_ternary: expected a 2-D or 4-D int32 compact tensor")
+        words = input
+    else:
+        if input.dtype != torch.float32:
+            raise RuntimeError("compress_ternary: expected fp32 weights")
+        words = compactify_ternary(input)
+    words = words.detach().cpu().contiguous()
+    columns = orig_shape[0]
+    rows = words.numel() // ((columns + 15) // 16)
+    lib = _lib()
+    cap = lib.tmq_compress_bound(rows, columns)
+    buf = torch.empty(cap, dtype=torch.int8)
+    size = ctypes.c_size_t(0)
+    check(lib.tmq_compress_ternary(ptr(words), rows, columns, ptr(buf), cap, ctypes.byref(size)), "compress_ternary")
+    return buf[:size.value].clone()
+
+
+def decompress_ternary(input: torch.Tensor, orig_shape) -> torch.Tensor:
+    """Decode a range-coded stream into the int32 compact tensor (tmq/tmq_native.cpp:489-503)."""
+    orig_shape = [int(s) for s in orig_shape]
+    if input.is_cuda:
+        raise RuntimeError("decompress_ternary: expected a CPU tensor")
+    if input.dim() != 1 or input.dtype != torch.int8 or input.numel() < 26:
+        raise RuntimeError("decompress_ternary: expected a 1-D int8 stream of at least 26 bytes")
+    cols = orig_shape[0]
+    qcols = (cols + 15) // 16
+    if len(orig_shape) == 4:
+        rows = orig_shape[1] * orig_shape[2] * orig_shape[3]
+        out = torch.empty((orig_shape[1], orig_shape[2], orig_shape[3], qcols), dtype=torch.int32)
+    else:
+        rows = orig_shape[1]
+        out = torch.empty((rows, qcols), dtype=torch.int32)
+    src = input.contiguous()
+    check(_lib().tmq_decompress_ternary(ptr(src), src.numel(), ptr(out), rows, cols), "decompress_ternary")
+    return out
