@@ -97,6 +97,14 @@ int tmq_softstep_fused(const float *w, const float *g, float *y, float *dw, floa
                        double sharpness, double strength, float gl, double lo, double hi,
                        void *stream);
 
+/* Diagnostic with no counterpart in the reference: the kernels above replace IEEE division by
+ * cheaper FMA sequences; this proves on the device that they are bit-identical to IEEE
+ * division. counts (device, 5 x uint64) receives: [0..2] mismatches of the three rational
+ * pieces over every fp32 argument in [-3,3] (and NaN), [3] mismatches of x / c(digamma) over
+ * every mantissa, both signs, three binades, [4] the number of arguments swept (a sanity
+ * figure, 2*0x40400000 + 1 + NaNs). All mismatch counts must be 0.                           */
+int tmq_selfcheck_division(double digamma, uint64_t *counts, void *stream);
+
 /* ------------------------------------------------------------------------------------------
  * Multi-tensor (one launch for every registered layer) forms of the per-layer Python loops of
  * QuantizationControl.quantization_loss / clamp (tmq/tmq.py:298-310, 263-272).

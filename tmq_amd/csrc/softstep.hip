@@ -10,6 +10,7 @@
 // bit-identical to that chain. Scalars arrive as doubles and are rounded to fp32 once on the
 // host (StepK), as torch does with Python scalars.
 #include "common.h"
+#include "softstep_math.h"
 
 #include <math.h>
 
@@ -19,82 +20,7 @@ namespace {
 constexpr int kThreads = 256;
 constexpr int kUnroll = 4;                            // dwordx4 packets per thread per tensor
 constexpr uint32_t kChunk = kThreads * 4 * kUnroll;   // elements per block
-
-// Host-rounded scalars of one staircase evaluation.
-struct StepK {
-    float d;   // float(digamma)
-    float h;   // float(digamma / 2)
-    float c;   // float(2 * sig(digamma / 2))
-    float k1;  // float(strength * digamma)
-    float k2;  // float(strength * digamma * digamma)
-};
-
-double scalar_sigmoid(double in) {  // tmq/tmq.py:384-391, evaluated in double like Python
-    double x = fmin(3.0, fmax(-3.0, in));
-    double x2 = x * x;
-    return x * (x2 + 27.0) / (27.0 + x2 * 9.0);
-}
-
-StepK make_step(double digamma, double strength) {
-    StepK k;
-    k.d = (float)digamma;
-    k.h = (float)(digamma / 2.0);
-    k.c = (float)(2.0 * scalar_sigmoid(digamma / 2.0));
-    k.k1 = (float)(strength * digamma);
-    k.k2 = (float)(strength * digamma * digamma);
-    return k;
-}
-
-// ---- per-element arithmetic ---------------------------------------------------------------
-
-// frac = w - floor(w); `bad` marks NaN/Inf weights, for which every torch op downstream yields
-// NaN (torch.clamp propagates NaN, v_med3_f32 does not).
-struct Frac {
-    float fw, frac;
-    bool bad;
-};
-__device__ __forceinline__ Frac split(float w) {
-    Frac f;
-    f.fw = floorf(w);
-    f.frac = w - f.fw;
-    f.bad = f.frac != f.frac;
-    return f;
-}
-
-// x = clamp(d*frac - h, -3, 3) with NaN kept (tmq/tmq.py:358, 418).
-__device__ __forceinline__ float clamped_arg(const Frac &f, float d, float h) {
-    float t = d * f.frac;
-    float arg = t - h;
-    float x = __builtin_amdgcn_fmed3f(arg, -3.0f, 3.0f);
-    return f.bad ? arg : x;
-}
-
-__device__ __forceinline__ float sig_of(float x) {  // tmq/tmq.py:359-360
-    float x2 = x * x;
-    float num = x * (x2 + 27.0f);
-    float den = 27.0f + x2 * 9.0f;
-    return num / den;
-}
-__device__ __forceinline__ float dsig_of(float x) {  // tmq/tmq.py:369-370
-    float x2 = x * x;
-    float a = x2 - 9.0f;
-    float b = 3.0f + x2;
-    float num = a * a;
-    float den = (9.0f * b) * b;
-    return num / den;
-}
-__device__ __forceinline__ float d2sig_of(float x) {  // tmq/tmq.py:379-381
-    float x2 = x * x;
-    float a = x2 + 3.0f;
-    float num = (16.0f * x) * (x2 - 9.0f);
-    float den = ((3.0f * a) * a) * a;
-    return num / den;
-}
-
-__device__ __forceinline__ float clamp_keep_nan(float w, float lo, float hi) {
-    float x = __builtin_amdgcn_fmed3f(w, lo, hi);
-    return (w != w) ? w : x;
-}
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 // ---- element operators ----------------------------------------------------------------------
 // Each Op declares which streams it touches; `apply` sees one element.
@@ -108,8 +34,8 @@ struct FwdOp {  // tmq/tmq.py:417-419
     StepK s;
     __device__ __forceinline__ void apply(float w, float, float, float &o0, float &, float &, float &) const {
         Frac f = split(w);
-        float x = clamped_arg(f, s.d, s.h);
-        float v = sig_of(x) / s.c;
+        Rational r(clamped_arg(f, s.d, s.h));
+        float v = cdiv(r.sig(), s.c, s.rc);
         o0 = (v + 0.5f) + f.fw;
     }
 };
@@ -120,8 +46,8 @@ struct BwdOp {  // tmq/tmq.py:434-438
     float scale;
     __device__ __forceinline__ void apply(float w, float g, float, float &o0, float &, float &, float &) const {
         Frac f = split(w);
-        float x = clamped_arg(f, s.d, s.h);
-        float grad = (s.d * dsig_of(x)) / s.c;
+        Rational r(clamped_arg(f, s.d, s.h));
+        float grad = cdiv(s.d * r.dsig(), s.c, s.rc);
         o0 = (scale * g) * grad;
     }
 };
@@ -131,8 +57,8 @@ struct DerivFwdOp {  // tmq/tmq.py:469-473
     StepK s;
     __device__ __forceinline__ void apply(float w, float, float, float &o0, float &, float &, float &) const {
         Frac f = split(w);
-        float x = clamped_arg(f, s.d, s.h);
-        o0 = (s.k1 * dsig_of(x)) / s.c;
+        Rational r(clamped_arg(f, s.d, s.h));
+        o0 = cdiv(s.k1 * r.dsig(), s.c, s.rc);
     }
 };
 
@@ -141,8 +67,8 @@ struct DerivBwdOp {  // tmq/tmq.py:488-493
     StepK s;
     __device__ __forceinline__ void apply(float w, float g, float, float &o0, float &, float &, float &) const {
         Frac f = split(w);
-        float x = clamped_arg(f, s.d, s.h);
-        float grad = (s.k2 * d2sig_of(x)) / s.c;
+        Rational r(clamped_arg(f, s.d, s.h));
+        float grad = cdiv(s.k2 * r.d2sig(), s.c, s.rc);
         o0 = g * grad;
     }
 };
@@ -166,7 +92,8 @@ struct TernarizeOp {  // tmq/tmq.py:293-295 with SoftStep.map 335-338 (in place)
             float arg = (s.d * w - s.d * fw) - s.h;  // association of SoftStep.map
             float x = __builtin_amdgcn_fmed3f(arg, -3.0f, 3.0f);
             x = (arg != arg) ? arg : x;
-            float t = sig_of(x) / s.c;
+            Rational r(x);
+            float t = cdiv(r.sig(), s.c, s.rc);
             v = (t + 0.5f) + fw;
         }
         o0 = rintf(v);  // torch.round: half to even
@@ -179,8 +106,8 @@ struct QLossOp {
     StepK q;  // sharpness constants
     __device__ __forceinline__ void apply(float w, float, float, float &, float &, float &, float &acc) const {
         Frac f = split(w);
-        float x = clamped_arg(f, q.d, q.h);
-        acc += (q.k1 * dsig_of(x)) / q.c;
+        Rational r(clamped_arg(f, q.d, q.h));
+        acc += cdiv(q.k1 * r.dsig(), q.c, q.rc);
     }
 };
 
@@ -191,8 +118,8 @@ struct QLossBwdOp {
     StepK q;
     __device__ __forceinline__ void apply(float w, float, float sc, float &, float &o1, float &, float &) const {
         Frac f = split(w);
-        float x = clamped_arg(f, q.d, q.h);
-        float grad = (q.k2 * d2sig_of(x)) / q.c;
+        Rational r(clamped_arg(f, q.d, q.h));
+        float grad = cdiv(q.k2 * r.d2sig(), q.c, q.rc);
         float t = sc * grad;
         o1 = ACC ? (o1 + t) : t;
     }
@@ -209,23 +136,24 @@ struct FusedOp {
     __device__ __forceinline__ void apply(float w, float g, float, float &o0, float &o1, float &o2, float &acc) const {
         Frac f = split(w);
         if constexpr ((MASK & 3) != 0) {
-            float x = clamped_arg(f, s.d, s.h);
+            Rational r(clamped_arg(f, s.d, s.h));
             if constexpr ((MASK & 1) != 0) {
-                float v = sig_of(x) / s.c;
+                float v = cdiv(r.sig(), s.c, s.rc);
                 o0 = (v + 0.5f) + f.fw;
             }
             if constexpr ((MASK & 2) != 0) {
-                float grad = (s.d * dsig_of(x)) / s.c;
+                float grad = cdiv(s.d * r.dsig(), s.c, s.rc);
                 float t1 = g * grad;  // scale is 1.0 at every reference call site (tmq/tmq.py:650, 812)
-                float x5 = clamped_arg(f, q.d, q.h);
-                float gq = (q.k2 * d2sig_of(x5)) / q.c;
+                Rational r5(clamped_arg(f, q.d, q.h));
+                float gq = cdiv(q.k2 * r5.d2sig(), q.c, q.rc);
                 float t2 = gl * gq;
                 o1 = t1 + t2;
+                if constexpr ((MASK & 8) != 0) acc += cdiv(q.k1 * r5.dsig(), q.c, q.rc);
             }
         }
-        if constexpr ((MASK & 8) != 0) {
-            float x5 = clamped_arg(f, q.d, q.h);
-            acc += (q.k1 * dsig_of(x5)) / q.c;
+        if constexpr ((MASK & 8) != 0 && (MASK & 2) == 0) {
+            Rational r5(clamped_arg(f, q.d, q.h));
+            acc += cdiv(q.k1 * r5.dsig(), q.c, q.rc);
         }
         if constexpr ((MASK & 4) != 0) o2 = clamp_keep_nan(w, lo, hi);
     }
@@ -283,29 +211,32 @@ __global__ __launch_bounds__(kThreads) void stream_kernel(Loc loc, Op op, float 
     float acc = 0.f;
 
     if (base + kChunk <= v.n && v.vec) {
-        // Full chunk: issue every load first, then compute, then store.
-        float4 a[kUnroll], b[kUnroll], r1[kUnroll];
+        // Full chunk: issue every load first, then compute, then store. Each tensor is touched
+        // exactly once per pass, so accesses are marked non-temporal (streaming).
+        f32x4 a[kUnroll], b[kUnroll], r1[kUnroll];
 #pragma unroll
         for (int u = 0; u < kUnroll; u++) {
             const uint64_t i = base + (uint64_t)(u * kThreads + tid) * 4;
-            a[u] = *reinterpret_cast<const float4 *>(v.in0 + i);
-            if constexpr (Op::kIn1) b[u] = *reinterpret_cast<const float4 *>(v.in1 + i);
-            if constexpr (Op::kReadOut1) r1[u] = *reinterpret_cast<const float4 *>(v.out1 + i);
+            a[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(v.in0 + i));
+            if constexpr (Op::kIn1) b[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(v.in1 + i));
+            if constexpr (Op::kReadOut1) r1[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(v.out1 + i));
         }
 #pragma unroll
         for (int u = 0; u < kUnroll; u++) {
             const uint64_t i = base + (uint64_t)(u * kThreads + tid) * 4;
-            float4 o0, o1, o2;
+            f32x4 o0, o1, o2;
             if constexpr (Op::kReadOut1) o1 = r1[u];
-            float gx = 0.f, gy = 0.f, gz = 0.f, gw = 0.f;
-            if constexpr (Op::kIn1) { gx = b[u].x; gy = b[u].y; gz = b[u].z; gw = b[u].w; }
-            op.apply(a[u].x, gx, v.scalar, o0.x, o1.x, o2.x, acc);
-            op.apply(a[u].y, gy, v.scalar, o0.y, o1.y, o2.y, acc);
-            op.apply(a[u].z, gz, v.scalar, o0.z, o1.z, o2.z, acc);
-            op.apply(a[u].w, gw, v.scalar, o0.w, o1.w, o2.w, acc);
-            if constexpr (Op::kOut0) *reinterpret_cast<float4 *>(v.out0 + i) = o0;
-            if constexpr (Op::kOut1) *reinterpret_cast<float4 *>(v.out1 + i) = o1;
-            if constexpr (Op::kOut2) *reinterpret_cast<float4 *>(v.out2 + i) = o2;
+            f32x4 gv = {0.f, 0.f, 0.f, 0.f};
+            if constexpr (Op::kIn1) gv = b[u];
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                float t0, t1 = o1[e], t2;
+                op.apply(a[u][e], gv[e], v.scalar, t0, t1, t2, acc);
+                o0[e] = t0; o1[e] = t1; o2[e] = t2;
+            }
+            if constexpr (Op::kOut0) __builtin_nontemporal_store(o0, reinterpret_cast<f32x4 *>(v.out0 + i));
+            if constexpr (Op::kOut1) __builtin_nontemporal_store(o1, reinterpret_cast<f32x4 *>(v.out1 + i));
+            if constexpr (Op::kOut2) __builtin_nontemporal_store(o2, reinterpret_cast<f32x4 *>(v.out2 + i));
         }
     } else {
         // Ragged tail or unaligned tensor: element-wise, coalesced dword accesses.
@@ -360,6 +291,43 @@ __global__ __launch_bounds__(kThreads) void finalize_kernel(const tmq_segment *s
         __syncthreads();
     }
     if (threadIdx.x == 0 && total) *total = running;
+}
+
+// Exhaustive comparison of the FAST division forms with IEEE division.
+//   counts[0..2]: sig / dsig / d2sig mismatches over every fp32 x with |x| <= 3 (and NaN)
+//   counts[3]   : x / c mismatches over every mantissa, both signs, three binades
+//   counts[4]   : arguments visited by the first sweep
+__device__ __forceinline__ bool same_bits(float a, float b) {
+    return (__builtin_bit_cast(uint32_t, a) == __builtin_bit_cast(uint32_t, b)) || (a != a && b != b);
+}
+__global__ __launch_bounds__(kThreads) void selfcheck_kernel(float c, float rc, unsigned long long *counts) {
+    unsigned long long bad0 = 0, bad1 = 0, bad2 = 0, bad3 = 0, seen = 0;
+    const uint64_t stride = (uint64_t)gridDim.x * kThreads;
+    for (uint64_t i = (uint64_t)blockIdx.x * kThreads + threadIdx.x; i < (1ull << 32); i += stride) {
+        const float x = __builtin_bit_cast(float, (uint32_t)i);
+        if (!(fabsf(x) <= 3.0f) && x == x) continue;
+        seen++;
+        RationalT<true> f(x);
+        RationalT<false> r(x);
+        bad0 += !same_bits(f.sig(), r.sig());
+        bad1 += !same_bits(f.dsig(), r.dsig());
+        bad2 += !same_bits(f.d2sig(), r.d2sig());
+    }
+    for (uint64_t i = (uint64_t)blockIdx.x * kThreads + threadIdx.x; i < (6ull << 23); i += stride) {
+        const uint32_t m = (uint32_t)(i & 0x7FFFFFu), sel = (uint32_t)(i >> 23);
+        const uint32_t expo = (sel % 3 == 0) ? 107u : ((sel % 3 == 1) ? 127u : 137u);
+        const float x = __builtin_bit_cast(float, ((sel >= 3) ? 0x80000000u : 0u) | (expo << 23) | m);
+        bad3 += !same_bits(cdiv_t<true>(x, c, rc), cdiv_t<false>(x, c, rc));
+    }
+    if (blockIdx.x == 0 && threadIdx.x == 0) {   // signed zeros and NaN through the constant division
+        const float z[3] = {0.0f, -0.0f, __builtin_nanf("")};
+        for (float x : z) bad3 += !same_bits(cdiv_t<true>(x, c, rc), cdiv_t<false>(x, c, rc));
+    }
+    if (bad0) atomicAdd(&counts[0], bad0);
+    if (bad1) atomicAdd(&counts[1], bad1);
+    if (bad2) atomicAdd(&counts[2], bad2);
+    if (bad3) atomicAdd(&counts[3], bad3);
+    atomicAdd(&counts[4], seen);
 }
 
 inline uint32_t blocks_for(uint64_t n) { return (uint32_t)((n + kChunk - 1) / kChunk); }
@@ -476,6 +444,16 @@ int tmq_softstep_fused(const float *w, const float *g, float *y, float *dw, floa
         rc = check_launch();
     }
     return rc;
+}
+
+int tmq_selfcheck_division(double digamma, uint64_t *counts, void *stream) {
+    if (!counts || bad_hardness(digamma)) return TMQ_ERR_INVALID_ARG;
+    const StepK s = make_step(digamma, 0.0);
+    hipError_t e = hipMemsetAsync(counts, 0, 5 * sizeof(uint64_t), as_stream(stream));
+    if (e != hipSuccess) return note_hip_error(e);
+    hipLaunchKernelGGL(selfcheck_kernel, dim3(8192), dim3(kThreads), 0, as_stream(stream), s.c, s.rc,
+                       reinterpret_cast<unsigned long long *>(counts));
+    return check_launch();
 }
 
 int tmq_multi_plan(tmq_segment *segs, int nseg, uint32_t *total_blocks) {
