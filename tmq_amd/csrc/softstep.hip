@@ -13,112 +13,133 @@
 #include "softstep_math.h"
 
 #include <math.h>
+#include <type_traits>
 
 namespace tmq {
 namespace {
 
-constexpr int kThreads = 256;
-constexpr int kUnroll = 4;                            // dwordx4 packets per thread per tensor
+#ifndef TMQ_SS_THREADS
+#define TMQ_SS_THREADS 512
+#endif
+#ifndef TMQ_SS_UNROLL
+#define TMQ_SS_UNROLL 1
+#endif
+constexpr int kThreads = TMQ_SS_THREADS;
+constexpr int kUnroll = TMQ_SS_UNROLL;                // dwordx4 packets per thread per tensor
 constexpr uint32_t kChunk = kThreads * 4 * kUnroll;   // elements per block
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 // ---- element operators ----------------------------------------------------------------------
-// Each Op declares which streams it touches; `apply` sees one element.
+// Each Op declares which streams it touches; `apply<CAREFUL>` sees one element.
 //   in0  : weight            (always loaded)
 //   in1  : second input      (kIn1)
 //   out0..out2 : outputs     (kOut0..2); out0 may alias in0 for the in-place ops
-//   acc  : per-thread loss accumulator (kLoss)
+//   acc  : per-thread loss accumulator (kLoss). It sums dsig(arg) to ~1 ulp; the constant factor
+//          strength*sharpness/c is applied once, in fp64, by the finalisation kernel.
+#define TMQ_OP_FLAGS(in1, o0, o1, o2, loss, rd1)                                                   \
+    static constexpr bool kIn1 = in1, kOut0 = o0, kOut1 = o1, kOut2 = o2, kLoss = loss, kReadOut1 = rd1
 
 struct FwdOp {  // tmq/tmq.py:417-419
-    static constexpr bool kIn1 = false, kOut0 = true, kOut1 = false, kOut2 = false, kLoss = false, kReadOut1 = false;
+    TMQ_OP_FLAGS(false, true, false, false, false, false);
     StepK s;
+    template <bool CAREFUL>
     __device__ __forceinline__ void apply(float w, float, float, float &o0, float &, float &, float &) const {
         Frac f = split(w);
-        Rational r(clamped_arg(f, s.d, s.h));
+        Rational r(clamped_arg<CAREFUL>(f, s.d, s.h));
         float v = cdiv(r.sig(), s.c, s.rc);
         o0 = (v + 0.5f) + f.fw;
+        // fw is +-Inf for an infinite weight where the reference has NaN (Inf - Inf in frac)
+        if constexpr (CAREFUL) o0 = (f.frac != f.frac) ? f.frac : o0;
     }
 };
 
 struct BwdOp {  // tmq/tmq.py:434-438
-    static constexpr bool kIn1 = true, kOut0 = true, kOut1 = false, kOut2 = false, kLoss = false, kReadOut1 = false;
+    TMQ_OP_FLAGS(true, true, false, false, false, false);
     StepK s;
     float scale;
+    template <bool CAREFUL>
     __device__ __forceinline__ void apply(float w, float g, float, float &o0, float &, float &, float &) const {
         Frac f = split(w);
-        Rational r(clamped_arg(f, s.d, s.h));
+        Rational r(clamped_arg<CAREFUL>(f, s.d, s.h));
         float grad = cdiv(s.d * r.dsig(), s.c, s.rc);
         o0 = (scale * g) * grad;
     }
 };
 
 struct DerivFwdOp {  // tmq/tmq.py:469-473
-    static constexpr bool kIn1 = false, kOut0 = true, kOut1 = false, kOut2 = false, kLoss = false, kReadOut1 = false;
+    TMQ_OP_FLAGS(false, true, false, false, false, false);
     StepK s;
+    template <bool CAREFUL>
     __device__ __forceinline__ void apply(float w, float, float, float &o0, float &, float &, float &) const {
         Frac f = split(w);
-        Rational r(clamped_arg(f, s.d, s.h));
+        Rational r(clamped_arg<CAREFUL>(f, s.d, s.h));
         o0 = cdiv(s.k1 * r.dsig(), s.c, s.rc);
     }
 };
 
 struct DerivBwdOp {  // tmq/tmq.py:488-493
-    static constexpr bool kIn1 = true, kOut0 = true, kOut1 = false, kOut2 = false, kLoss = false, kReadOut1 = false;
+    TMQ_OP_FLAGS(true, true, false, false, false, false);
     StepK s;
+    template <bool CAREFUL>
     __device__ __forceinline__ void apply(float w, float g, float, float &o0, float &, float &, float &) const {
         Frac f = split(w);
-        Rational r(clamped_arg(f, s.d, s.h));
+        Rational r(clamped_arg<CAREFUL>(f, s.d, s.h));
         float grad = cdiv(s.k2 * r.d2sig(), s.c, s.rc);
         o0 = g * grad;
     }
 };
 
 struct ClampOp {  // tmq/tmq.py:696, 879 (in place: out0 aliases in0)
-    static constexpr bool kIn1 = false, kOut0 = true, kOut1 = false, kOut2 = false, kLoss = false, kReadOut1 = false;
+    TMQ_OP_FLAGS(false, true, false, false, false, false);
     float lo, hi;
+    template <bool CAREFUL>
     __device__ __forceinline__ void apply(float w, float, float, float &o0, float &, float &, float &) const {
-        o0 = clamp_keep_nan(w, lo, hi);
+        o0 = clamp_to<CAREFUL>(w, lo, hi);
     }
 };
 
 struct TernarizeOp {  // tmq/tmq.py:293-295 with SoftStep.map 335-338 (in place)
-    static constexpr bool kIn1 = false, kOut0 = true, kOut1 = false, kOut2 = false, kLoss = false, kReadOut1 = false;
+    TMQ_OP_FLAGS(false, true, false, false, false, false);
     StepK s;
     bool use_map;
+    template <bool CAREFUL>
     __device__ __forceinline__ void apply(float w, float, float, float &o0, float &, float &, float &) const {
         float v = w;
         if (use_map) {
             float fw = floorf(w);
             float arg = (s.d * w - s.d * fw) - s.h;  // association of SoftStep.map
             float x = __builtin_amdgcn_fmed3f(arg, -3.0f, 3.0f);
-            x = (arg != arg) ? arg : x;
+            if constexpr (CAREFUL) x = (arg != arg) ? arg : x;
             Rational r(x);
             float t = cdiv(r.sig(), s.c, s.rc);
             v = (t + 0.5f) + fw;
+            if constexpr (CAREFUL) v = (arg != arg) ? arg : v;
         }
         o0 = rintf(v);  // torch.round: half to even
     }
 };
 
-// Loss only: acc += q(w). Used by the multi-tensor quantization loss.
+// Loss only: acc += dsig(arg). Used by the multi-tensor quantization loss.
 struct QLossOp {
-    static constexpr bool kIn1 = false, kOut0 = false, kOut1 = false, kOut2 = false, kLoss = true, kReadOut1 = false;
+    TMQ_OP_FLAGS(false, false, false, false, true, false);
     StepK q;  // sharpness constants
+    template <bool CAREFUL>
     __device__ __forceinline__ void apply(float w, float, float, float &, float &, float &, float &acc) const {
         Frac f = split(w);
-        Rational r(clamped_arg(f, q.d, q.h));
-        acc += cdiv(q.k1 * r.dsig(), q.c, q.rc);
+        Rational r(clamped_arg<CAREFUL>(f, q.d, q.h));
+        acc += r.dsig_approx();
     }
 };
 
 // aux (=|+=) scalar * Q'(w): gradient of the mean quantization loss (out1 is the aux tensor).
 template <bool ACC>
 struct QLossBwdOp {
-    static constexpr bool kIn1 = false, kOut0 = false, kOut1 = true, kOut2 = false, kLoss = false, kReadOut1 = ACC;
+    TMQ_OP_FLAGS(false, false, true, false, false, ACC);
     StepK q;
+    template <bool CAREFUL>
     __device__ __forceinline__ void apply(float w, float, float sc, float &, float &o1, float &, float &) const {
         Frac f = split(w);
-        Rational r(clamped_arg(f, q.d, q.h));
+        Rational r(clamped_arg<CAREFUL>(f, q.d, q.h));
         float grad = cdiv(q.k2 * r.d2sig(), q.c, q.rc);
         float t = sc * grad;
         o1 = ACC ? (o1 + t) : t;
@@ -128,34 +149,35 @@ struct QLossBwdOp {
 // The fused pass. MASK bits: 1 = y, 2 = dw, 4 = clamp(w), 8 = loss sum.
 template <int MASK>
 struct FusedOp {
-    static constexpr bool kIn1 = (MASK & 2) != 0, kOut0 = (MASK & 1) != 0, kOut1 = (MASK & 2) != 0,
-                          kOut2 = (MASK & 4) != 0, kLoss = (MASK & 8) != 0, kReadOut1 = false;
+    TMQ_OP_FLAGS((MASK & 2) != 0, (MASK & 1) != 0, (MASK & 2) != 0, (MASK & 4) != 0, (MASK & 8) != 0, false);
     StepK s;  // hardness constants (forward / backward)
     StepK q;  // sharpness constants (quantization loss)
     float gl, lo, hi;
+    template <bool CAREFUL>
     __device__ __forceinline__ void apply(float w, float g, float, float &o0, float &o1, float &o2, float &acc) const {
         Frac f = split(w);
         if constexpr ((MASK & 3) != 0) {
-            Rational r(clamped_arg(f, s.d, s.h));
+            Rational r(clamped_arg<CAREFUL>(f, s.d, s.h));
             if constexpr ((MASK & 1) != 0) {
                 float v = cdiv(r.sig(), s.c, s.rc);
                 o0 = (v + 0.5f) + f.fw;
+                if constexpr (CAREFUL) o0 = (f.frac != f.frac) ? f.frac : o0;
             }
             if constexpr ((MASK & 2) != 0) {
                 float grad = cdiv(s.d * r.dsig(), s.c, s.rc);
                 float t1 = g * grad;  // scale is 1.0 at every reference call site (tmq/tmq.py:650, 812)
-                Rational r5(clamped_arg(f, q.d, q.h));
+                Rational r5(clamped_arg<CAREFUL>(f, q.d, q.h));
                 float gq = cdiv(q.k2 * r5.d2sig(), q.c, q.rc);
                 float t2 = gl * gq;
                 o1 = t1 + t2;
-                if constexpr ((MASK & 8) != 0) acc += cdiv(q.k1 * r5.dsig(), q.c, q.rc);
+                if constexpr ((MASK & 8) != 0) acc += r5.dsig_approx();
             }
         }
         if constexpr ((MASK & 8) != 0 && (MASK & 2) == 0) {
-            Rational r5(clamped_arg(f, q.d, q.h));
-            acc += cdiv(q.k1 * r5.dsig(), q.c, q.rc);
+            Rational r5(clamped_arg<CAREFUL>(f, q.d, q.h));
+            acc += r5.dsig_approx();
         }
-        if constexpr ((MASK & 4) != 0) o2 = clamp_keep_nan(w, lo, hi);
+        if constexpr ((MASK & 4) != 0) o2 = clamp_to<CAREFUL>(w, lo, hi);
     }
 };
 
@@ -219,25 +241,35 @@ __global__ __launch_bounds__(kThreads) void stream_kernel(Loc loc, Op op, float 
             const uint64_t i = base + (uint64_t)(u * kThreads + tid) * 4;
             a[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(v.in0 + i));
             if constexpr (Op::kIn1) b[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(v.in1 + i));
+            else b[u] = f32x4{0.f, 0.f, 0.f, 0.f};
             if constexpr (Op::kReadOut1) r1[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(v.out1 + i));
         }
+        auto run = [&](auto careful) {
+            constexpr bool CAREFUL = decltype(careful)::value;
 #pragma unroll
-        for (int u = 0; u < kUnroll; u++) {
-            const uint64_t i = base + (uint64_t)(u * kThreads + tid) * 4;
-            f32x4 o0, o1, o2;
-            if constexpr (Op::kReadOut1) o1 = r1[u];
-            f32x4 gv = {0.f, 0.f, 0.f, 0.f};
-            if constexpr (Op::kIn1) gv = b[u];
+            for (int u = 0; u < kUnroll; u++) {
+                const uint64_t i = base + (uint64_t)(u * kThreads + tid) * 4;
+                f32x4 o0, o1, o2;
 #pragma unroll
-            for (int e = 0; e < 4; e++) {
-                float t0, t1 = o1[e], t2;
-                op.apply(a[u][e], gv[e], v.scalar, t0, t1, t2, acc);
-                o0[e] = t0; o1[e] = t1; o2[e] = t2;
+                for (int e = 0; e < 4; e++) {
+                    float t0, t1 = 0.f, t2;
+                    if constexpr (Op::kReadOut1) t1 = r1[u][e];
+                    op.template apply<CAREFUL>(a[u][e], b[u][e], v.scalar, t0, t1, t2, acc);
+                    o0[e] = t0; o1[e] = t1; o2[e] = t2;
+                }
+                if constexpr (Op::kOut0) __builtin_nontemporal_store(o0, reinterpret_cast<f32x4 *>(v.out0 + i));
+                if constexpr (Op::kOut1) __builtin_nontemporal_store(o1, reinterpret_cast<f32x4 *>(v.out1 + i));
+                if constexpr (Op::kOut2) __builtin_nontemporal_store(o2, reinterpret_cast<f32x4 *>(v.out2 + i));
             }
-            if constexpr (Op::kOut0) __builtin_nontemporal_store(o0, reinterpret_cast<f32x4 *>(v.out0 + i));
-            if constexpr (Op::kOut1) __builtin_nontemporal_store(o1, reinterpret_cast<f32x4 *>(v.out1 + i));
-            if constexpr (Op::kOut2) __builtin_nontemporal_store(o2, reinterpret_cast<f32x4 *>(v.out2 + i));
-        }
+        };
+        // Vote once per wavefront: NaN / Inf weights take the variant with NaN-preserving clamps.
+        bool odd = false;
+#pragma unroll
+        for (int u = 0; u < kUnroll; u++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) odd |= not_finite(a[u][e]);
+        if (__builtin_amdgcn_ballot_w64(odd) == 0) run(std::false_type{});
+        else run(std::true_type{});
     } else {
         // Ragged tail or unaligned tensor: element-wise, coalesced dword accesses.
         for (int u = 0; u < kUnroll * 4; u++) {
@@ -247,7 +279,7 @@ __global__ __launch_bounds__(kThreads) void stream_kernel(Loc loc, Op op, float 
                 float g = 0.f;
                 if constexpr (Op::kIn1) g = v.in1[i];
                 if constexpr (Op::kReadOut1) o1 = v.out1[i];
-                op.apply(v.in0[i], g, v.scalar, o0, o1, o2, acc);
+                op.template apply<true>(v.in0[i], g, v.scalar, o0, o1, o2, acc);
                 if constexpr (Op::kOut0) v.out0[i] = o0;
                 if constexpr (Op::kOut1) v.out1[i] = o1;
                 if constexpr (Op::kOut2) v.out2[i] = o2;
@@ -264,8 +296,8 @@ __global__ __launch_bounds__(kThreads) void stream_kernel(Loc loc, Op op, float 
 // [begin_l, begin_{l+1}). mean_l = float(sum_l / n_l); total = fp32 running sum in table order
 // (the reference adds per-layer means one by one, tmq/tmq.py:309).
 __global__ __launch_bounds__(kThreads) void finalize_kernel(const tmq_segment *segs, int nseg, uint32_t total_blocks,
-                                                           const float *partials, float *per_tensor, float *total,
-                                                           double *sum_out) {
+                                                           const float *partials, double factor, float *per_tensor,
+                                                           float *total, double *sum_out) {
     __shared__ double red[kThreads];
     float running = 0.f;
     for (int l = 0; l < nseg; l++) {
@@ -280,10 +312,11 @@ __global__ __launch_bounds__(kThreads) void finalize_kernel(const tmq_segment *s
             __syncthreads();
         }
         if (threadIdx.x == 0) {
-            if (sum_out) sum_out[l] = red[0];
+            const double sum = red[0] * factor;   // partials hold sum dsig; factor = strength*sharpness/c
+            if (sum_out) sum_out[l] = sum;
             if (segs) {
                 const uint64_t n = segs[l].n;
-                float mean = (float)(red[0] / (double)n);  // n == 0 gives NaN like torch.mean of an empty tensor
+                float mean = (float)(sum / (double)n);  // n == 0 gives NaN like torch.mean of an empty tensor
                 if (per_tensor) per_tensor[l] = mean;
                 running = (l == 0) ? mean : running + mean;
             }
@@ -440,7 +473,7 @@ int tmq_softstep_fused(const float *w, const float *g, float *y, float *dw, floa
     }
     if (loss_sum) {
         hipLaunchKernelGGL(finalize_kernel, dim3(1), dim3(kThreads), 0, as_stream(stream), nullptr, 1, blocks_for(n),
-                           partials, nullptr, nullptr, loss_sum);
+                           partials, (double)q.k1 / (double)q.c, nullptr, nullptr, loss_sum);
         rc = check_launch();
     }
     return rc;
@@ -480,7 +513,7 @@ int tmq_qloss_multi(const tmq_segment *segs, int nseg, uint32_t total_blocks, do
     int rc = launch_multi(op, segs, nseg, total_blocks, 0, partials, stream);
     if (rc != TMQ_OK) return rc;
     hipLaunchKernelGGL(finalize_kernel, dim3(1), dim3(kThreads), 0, as_stream(stream), segs, nseg, total_blocks,
-                       partials, per_tensor, total, nullptr);
+                       partials, (double)op.q.k1 / (double)op.q.c, per_tensor, total, nullptr);
     return check_launch();
 }
 

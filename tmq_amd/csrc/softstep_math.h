@@ -128,6 +128,17 @@ struct RationalT {
         if constexpr (FAST) return vdiv(num, den, (rb * 0.11111111f) * rb);
         else return num / den;
     }
+    // dsig to ~1 ulp (no residual corrections): used only inside the loss reduction, whose
+    // result is a sum compared with a relative tolerance, never element by element.
+    __device__ __forceinline__ float dsig_approx() const {
+        float a = x2 - 9.0f;
+        float num = a * a;
+        float den = (9.0f * b) * b;
+        float y0 = ((FAST ? rb : rcp_(b)) * 0.11111111f) * (FAST ? rb : rcp_(b));
+        float e = fma_(-den, y0, 1.0f);
+        float y1 = fma_(e, y0, y0);
+        return num * y1;
+    }
     // tmq/tmq.py:379-381: ((16*x)*(x2-9)) / (((3*a)*a)*a), a = x2+3
     __device__ __forceinline__ float d2sig() const {
         float num = (16.0f * x) * (x2 - 9.0f);
@@ -138,31 +149,39 @@ struct RationalT {
 };
 using Rational = RationalT<TMQ_FAST_DIV != 0>;
 
-// frac = w - floor(w); `bad` marks NaN/Inf weights, for which every torch op downstream yields
-// NaN (torch.clamp propagates NaN, v_med3_f32 does not).
+// NaN / Inf weights: torch.clamp propagates NaN where v_med3_f32 returns a bound, so such
+// elements need two extra selects per chain. The streaming kernel evaluates a chunk with
+// CAREFUL = false (v_med3 only), votes across the wavefront whether any weight was not finite,
+// and only then re-evaluates the chunk with CAREFUL = true. Finite weights give identical bits
+// in both modes.
+__device__ __forceinline__ bool not_finite(float w) { return !(__builtin_fabsf(w) < INFINITY); }
+
+// frac = w - floor(w)
 struct Frac {
     float fw, frac;
-    bool bad;
 };
 __device__ __forceinline__ Frac split(float w) {
     Frac f;
     f.fw = floorf(w);
     f.frac = w - f.fw;
-    f.bad = f.frac != f.frac;
     return f;
 }
 
-// x = clamp(d*frac - h, -3, 3) with NaN kept (tmq/tmq.py:358, 418).
+// x = clamp(d*frac - h, -3, 3) (tmq/tmq.py:358, 418); CAREFUL keeps a NaN argument NaN.
+template <bool CAREFUL>
 __device__ __forceinline__ float clamped_arg(const Frac &f, float d, float h) {
     float t = d * f.frac;
     float arg = t - h;
     float x = __builtin_amdgcn_fmed3f(arg, -3.0f, 3.0f);
-    return f.bad ? arg : x;
+    if constexpr (CAREFUL) return (arg != arg) ? arg : x;
+    else return x;
 }
 
-__device__ __forceinline__ float clamp_keep_nan(float w, float lo, float hi) {
+template <bool CAREFUL>
+__device__ __forceinline__ float clamp_to(float w, float lo, float hi) {
     float x = __builtin_amdgcn_fmed3f(w, lo, hi);
-    return (w != w) ? w : x;
+    if constexpr (CAREFUL) return (w != w) ? w : x;
+    else return x;
 }
 
 #endif  // __HIPCC__
