@@ -29,6 +29,21 @@ HBM_PEAK_GBS = 8000.0
 BYTES_PER_ELEM = 20                                        # load w, g; store y, dw, clamp(w)
 
 
+def measured_traffic(path, n, default_n=1 << 26):
+    """HBM bytes per launch of the dominant kernel as measured with rocprofv3 --pmc FETCH_SIZE /
+    WRITE_SIZE (scaled by a copy of known size); the figure lives in the committed profile summary.
+    Only valid for the workload size it was measured at."""
+    try:
+        if n != default_n:
+            return None
+        for line in open(os.path.join(ROOT, "profiles", path)):
+            if line.startswith("traffic_bytes:"):
+                return int(line.split(":")[1])
+    except OSError:
+        pass
+    return None
+
+
 def make_inputs(n, torch):
     """Seeded CPU generation (identical bits for the CPU baseline and the GPU)."""
     gen = lambda s: torch.Generator(device="cpu").manual_seed(s)
@@ -121,7 +136,9 @@ def bench_softstep(args, torch):
                                "over 5 schedule values", "elements": n, "bytes_per_element": BYTES_PER_ELEM,
                    "hardness": HARDNESS, "sharpness": SHARPNESS, "strength": STRENGTH},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": measured_traffic("softstep_fused_2p26.md", n),
+                     "algorithmic_bytes": bytes_per_launch,
                      "kernel": "stream_kernel<FusedOp<15>> (+ 1-block loss finalisation in the same call)",
                      "avg_launch_us": round(avg_ms * 1e3, 3)},
     }

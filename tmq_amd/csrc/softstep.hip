@@ -292,38 +292,66 @@ __global__ __launch_bounds__(kThreads) void stream_kernel(Loc loc, Op op, float 
     }
 }
 
-// Ordered fp64 finalisation of block partial sums. One block; segment l owns the partials
-// [begin_l, begin_{l+1}). mean_l = float(sum_l / n_l); total = fp32 running sum in table order
-// (the reference adds per-layer means one by one, tmq/tmq.py:309).
-__global__ __launch_bounds__(kThreads) void finalize_kernel(const tmq_segment *segs, int nseg, uint32_t total_blocks,
-                                                           const float *partials, double factor, float *per_tensor,
-                                                           float *total, double *sum_out) {
-    __shared__ double red[kThreads];
-    float running = 0.f;
+// Ordered fp64 finalisation of block partial sums: one workgroup of 16 wavefronts. Segment l owns
+// the partials [begin_l, begin_{l+1}); its range is cut into tasks of kTaskLen partials, tasks are
+// dealt round-robin to the wavefronts (every load of a task is in flight at once, DPP reduction in
+// fp64), and one thread then adds the task sums in order. mean_l = float(sum_l / n_l); total = fp32
+// running sum in table order (the reference adds per-layer means one by one, tmq/tmq.py:309).
+// Deterministic: no atomics, fixed association.
+constexpr int kFinThreads = 1024, kFinWaves = kFinThreads / 64, kTaskLen = 2048, kMaxTasks = 2048;
+
+__device__ __forceinline__ double wave_sum_f64(double v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+
+__global__ __launch_bounds__(kFinThreads) void finalize_kernel(const tmq_segment *segs, int nseg,
+                                                              uint32_t total_blocks, const float *partials,
+                                                              double factor, float *per_tensor, float *total,
+                                                              double *sum_out) {
+    __shared__ double task_sum[kMaxTasks];
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    uint32_t task = 0;
     for (int l = 0; l < nseg; l++) {
         const uint32_t b0 = segs ? segs[l].block_begin : 0u;
         const uint32_t b1 = segs ? (l + 1 < nseg ? segs[l + 1].block_begin : total_blocks) : total_blocks;
-        double s = 0.0;
-        for (uint32_t i = b0 + threadIdx.x; i < b1; i += kThreads) s += (double)partials[i];
-        red[threadIdx.x] = s;
-        __syncthreads();
-        for (int off = kThreads / 2; off > 0; off >>= 1) {
-            if ((int)threadIdx.x < off) red[threadIdx.x] += red[threadIdx.x + off];
-            __syncthreads();
+        const uint32_t ntask = (b1 - b0 + kTaskLen - 1) / kTaskLen;
+        for (uint32_t t = 0; t < ntask; t++, task++) {
+            if ((int)(task % kFinWaves) != wv) continue;
+            const uint32_t t0 = b0 + t * kTaskLen, t1 = min(t0 + (uint32_t)kTaskLen, b1);
+            double s = 0.0;
+#pragma unroll 8
+            for (uint32_t i = t0 + lane; i < t1; i += 64) s += (double)partials[i];
+            s = wave_sum_f64(s);
+            if (lane == 0) task_sum[task] = s;
         }
-        if (threadIdx.x == 0) {
-            const double sum = red[0] * factor;   // partials hold sum dsig; factor = strength*sharpness/c
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float running = 0.f;
+        uint32_t tk = 0;
+        for (int l = 0; l < nseg; l++) {
+            const uint32_t b0 = segs ? segs[l].block_begin : 0u;
+            const uint32_t b1 = segs ? (l + 1 < nseg ? segs[l + 1].block_begin : total_blocks) : total_blocks;
+            const uint32_t ntask = (b1 - b0 + kTaskLen - 1) / kTaskLen;
+            double sum = 0.0;
+            for (uint32_t t = 0; t < ntask; t++) sum += task_sum[tk++];
+            sum *= factor;   // partials hold sum dsig; factor = strength*sharpness/c
             if (sum_out) sum_out[l] = sum;
             if (segs) {
                 const uint64_t n = segs[l].n;
-                float mean = (float)(sum / (double)n);  // n == 0 gives NaN like torch.mean of an empty tensor
+                float mean = (float)(sum / (double)n);   // n == 0 gives NaN like torch.mean of an empty tensor
                 if (per_tensor) per_tensor[l] = mean;
                 running = (l == 0) ? mean : running + mean;
             }
         }
-        __syncthreads();
+        if (total) *total = running;
     }
-    if (threadIdx.x == 0 && total) *total = running;
+}
+
+inline bool finalize_fits(int nseg, uint32_t total_blocks) {
+    return (uint64_t)nseg + total_blocks / kTaskLen <= (uint64_t)kMaxTasks;
 }
 
 // Exhaustive comparison of the FAST division forms with IEEE division.
@@ -452,7 +480,7 @@ int tmq_softstep_fused(const float *w, const float *g, float *y, float *dw, floa
     if (dw && !g) return TMQ_ERR_INVALID_ARG;
     if (loss_sum && !workspace) return TMQ_ERR_INVALID_ARG;
     if (bad_hardness(digamma) || bad_hardness(sharpness) || !(lo <= hi)) return TMQ_ERR_INVALID_ARG;
-    if (n > kMaxElems) return TMQ_ERR_TOO_LARGE;
+    if (n > kMaxElems || (loss_sum && !finalize_fits(1, blocks_for(n)))) return TMQ_ERR_TOO_LARGE;
     const int mask = (y ? 1 : 0) | (dw ? 2 : 0) | (wc ? 4 : 0) | (loss_sum ? 8 : 0);
     if (mask == 0) return TMQ_OK;
     float *partials = static_cast<float *>(workspace);
@@ -472,8 +500,8 @@ int tmq_softstep_fused(const float *w, const float *g, float *y, float *dw, floa
         if (rc != TMQ_OK) return rc;
     }
     if (loss_sum) {
-        hipLaunchKernelGGL(finalize_kernel, dim3(1), dim3(kThreads), 0, as_stream(stream), nullptr, 1, blocks_for(n),
-                           partials, (double)q.k1 / (double)q.c, nullptr, nullptr, loss_sum);
+        hipLaunchKernelGGL(finalize_kernel, dim3(1), dim3(kFinThreads), 0, as_stream(stream), nullptr, 1,
+                           blocks_for(n), partials, (double)q.k1 / (double)q.c, nullptr, nullptr, loss_sum);
         rc = check_launch();
     }
     return rc;
@@ -508,11 +536,12 @@ int tmq_qloss_multi(const tmq_segment *segs, int nseg, uint32_t total_blocks, do
                     float *per_tensor, float *total, void *workspace, void *stream) {
     if (nseg <= 0 || !segs || !workspace) return TMQ_ERR_INVALID_ARG;
     if (bad_hardness(sharpness)) return TMQ_ERR_INVALID_ARG;
+    if (!finalize_fits(nseg, total_blocks)) return TMQ_ERR_TOO_LARGE;
     float *partials = static_cast<float *>(workspace);
     QLossOp op{make_step(sharpness, strength)};
     int rc = launch_multi(op, segs, nseg, total_blocks, 0, partials, stream);
     if (rc != TMQ_OK) return rc;
-    hipLaunchKernelGGL(finalize_kernel, dim3(1), dim3(kThreads), 0, as_stream(stream), segs, nseg, total_blocks,
+    hipLaunchKernelGGL(finalize_kernel, dim3(1), dim3(kFinThreads), 0, as_stream(stream), segs, nseg, total_blocks,
                        partials, (double)op.q.k1 / (double)op.q.c, per_tensor, total, nullptr);
     return check_launch();
 }
