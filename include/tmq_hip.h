@@ -163,14 +163,31 @@ int tmq_pack_ternary(const void *w, int dtype, int64_t N, int64_t K, uint32_t *w
 int tmq_unpack_ternary(const uint32_t *words, int64_t N, int64_t K, float *w, void *stream);
 
 /* ------------------------------------------------------------------------------------------
- * Ternary inference: y[m][n] = scale[n] * sum_k x[m][k] * T[k][n] + bias[n]
- * with T packed as words[K][ceil(N/16)], fp32 accumulation, fp32 output [M][N].
- * scale / bias are optional fp32 [N] (NULL = 1 / 0). x_dtype is TMQ_F16 or TMQ_F32 (fp32
- * activations are split into two fp16 terms so the product keeps fp32 accuracy).
+ * Ternary inference: y[m][n] = scale[n] * sum_k x[m][k] * T[k][n] + bias[n], fp32 accumulation.
+ *
+ * The kernels read a kernel-native re-tiling of the packed weights (still 2 bits per weight:
+ * blocks of 16 channels x 256 reduction indices laid out in MFMA operand order). It is produced
+ * once per layer from the reference-format words by tmq_prepack_weights and cached by the
+ * caller; the reference-format tensor itself is never modified.
+ * ---------------------------------------------------------------------------------------- */
+
+/* Bytes of the native buffer for N output channels and reduction length K. */
+size_t tmq_native_weight_bytes(int64_t N, int64_t K);
+
+/* words[K][ceil(N/16)], K = C*ky*kx with row (c*ky + i)*kx + j (the format written by
+ * tmq_pack_ternary / compactify_ternary, tmq/tmq_native.cpp:152-208) -> native (16-byte aligned).
+ * Linear layers pass C = K, ky = kx = 1. For ky*kx > 1 the reduction index is reordered to
+ * (i, j, c) so that im2col rows are contiguous in NHWC activations. Code 11 becomes 0, as in the
+ * reference's device LUT (tmq/tmq_cuda.cu:464-466).                                           */
+int tmq_prepack_weights(const uint32_t *words, int64_t N, int64_t C, int64_t ky, int64_t kx,
+                        void *native, void *stream);
+
+/* x [M][K] row-major, x_dtype TMQ_F16 or TMQ_F32 (fp32 activations are split into two fp16 terms
+ * so the product keeps ~fp32 accuracy); y fp32 [M][N]; scale / bias optional fp32 [N] (NULL = 1 / 0).
  * Replaces ternary_mvm_cuda (tmq/tmq_cuda.cu:563-603, kernel 242-286) for M == 1 and
  * ternary_mmm_cuda (tmq/tmq_cuda.cu:478-549, kernel 289-427) for M > 1, plus the post-scale /
- * bias passes of Linear.compact_forward (tmq/tmq.py:684-687).                                */
-int tmq_ternary_linear(const void *x, int x_dtype, int64_t M, int64_t K, const uint32_t *words,
+ * bias passes of Linear.compact_forward (tmq/tmq.py:684-687). Any M, K, N (ragged tails masked). */
+int tmq_ternary_linear(const void *x, int x_dtype, int64_t M, int64_t K, const void *native,
                        int64_t N, const float *scale, const float *bias, float *y, void *stream);
 
 /* Geometry of a 2-D convolution. */

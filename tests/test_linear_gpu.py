@@ -1,0 +1,122 @@
+"""GPU parity of the ternary linear kernels (through the C ABI) vs the CPU oracle.
+
+Bar: relative error <= 1e-3 against an fp64-accumulated product on the exactly expanded weights
+(the stated tolerance for this path); in practice the fp32-accumulated MFMA result is ~1e-6.
+"""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+RTOL = 1e-3
+
+
+def _ternary(rng, N, K, p0=0.5):
+    u = rng.random((N, K))
+    return np.where(u < (1 - p0) / 2, 1.0, np.where(u < 1 - p0, -1.0, 0.0)).astype(np.float32)
+
+
+def _rel_err(got, want):
+    want = np.asarray(want, np.float64)
+    got = np.asarray(got, np.float64)
+    return np.max(np.abs(got - want)) / max(1e-30, np.max(np.abs(want)))
+
+
+SHAPES = [  # (M, K, N)
+    (1, 32, 16), (1, 256, 16), (1, 4096, 64), (1, 147, 64), (1, 512, 102), (3, 40, 17), (16, 512, 256),
+    (17, 300, 50), (33, 1000, 130), (64, 576, 64), (64, 512, 102), (48, 2304, 128), (1, 7, 5),
+    (100, 256, 48), (130, 147, 64), (256, 512, 96),
+]
+
+
+@pytest.mark.parametrize("M,K,N", SHAPES)
+def test_linear_fp16_matches_oracle(cuda, oracle, M, K, N):
+    from tmq_amd import ops
+    rng = np.random.default_rng(M * 7 + K * 3 + N)
+    W = _ternary(rng, N, K)
+    words = oracle.pack(W)
+    x = rng.standard_normal((M, K)).astype(np.float16)
+    scale = (0.5 + rng.random(N)).astype(np.float32)
+    bias = rng.standard_normal(N).astype(np.float32)
+    tw = torch.from_numpy(words.view(np.int32)).to(cuda)
+    nw = ops.NativeWeights(tw, N)
+    tx = torch.from_numpy(x).to(cuda)
+    y = ops.ternary_linear(tx, nw, torch.from_numpy(scale).to(cuda), torch.from_numpy(bias).to(cuda))
+    want = oracle.gemm(x.astype(np.float32), words, N, scale, bias)
+    assert y.shape == (M, N) and y.dtype == torch.float32
+    assert _rel_err(y.cpu().numpy(), want) <= RTOL
+    assert _rel_err(y.cpu().numpy(), want) <= 2e-6          # what fp32 accumulation actually delivers
+    y0 = ops.ternary_linear(tx, nw)                          # no scale / bias
+    assert _rel_err(y0.cpu().numpy(), oracle.gemm(x.astype(np.float32), words, N)) <= 2e-6
+    # the textbook routine on expanded weights
+    ref = x.astype(np.float64) @ W.astype(np.float64).T
+    assert _rel_err(y0.cpu().numpy(), ref) <= 2e-6
+
+
+@pytest.mark.parametrize("M,K,N", [(1, 4096, 4096), (16, 4096, 4096), (5, 300, 70), (64, 1024, 256), (200, 512, 64)])
+def test_linear_fp32_activations(cuda, oracle, M, K, N):
+    """fp32 activations (the reference's calling convention) keep fp32-level accuracy."""
+    from tmq_amd import ops
+    rng = np.random.default_rng(K + N + M)
+    W = _ternary(rng, N, K)
+    words = oracle.pack(W)
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    tw = torch.from_numpy(words.view(np.int32)).to(cuda)
+    y = ops.ternary_mmm_cuda(torch.from_numpy(x).to(cuda), tw, N)
+    ref = x.astype(np.float64) @ W.astype(np.float64).T
+    assert _rel_err(y.cpu().numpy(), ref) <= 5e-6
+    if M == 1:
+        for shape in ((K,), (1, K), (1, 1, K), (1, 1, 1, K)):
+            v = ops.ternary_mvm_cuda(torch.from_numpy(x.reshape(shape)).to(cuda), tw, N)
+            assert tuple(v.shape) == shape[:-1] + (N,)
+            assert _rel_err(v.cpu().numpy().reshape(1, N), ref) <= 5e-6
+
+
+def test_exactness_on_integers(cuda, oracle):
+    """With small-integer activations every product and partial sum is exact in fp32, so the
+    result must equal the integer matrix product bit for bit, whatever the summation order."""
+    from tmq_amd import ops
+    rng = np.random.default_rng(3)
+    for (M, K, N) in [(1, 4096, 256), (16, 1024, 48), (64, 147, 64), (300, 512, 32)]:
+        W = _ternary(rng, N, K)
+        x = rng.integers(-8, 9, (M, K)).astype(np.float16)
+        words = oracle.pack(W)
+        nw = ops.NativeWeights(torch.from_numpy(words.view(np.int32)).to(cuda), N)
+        y = ops.ternary_linear(torch.from_numpy(x).to(cuda), nw).cpu().numpy()
+        ref = (x.astype(np.int64) @ W.astype(np.int64).T).astype(np.float32)
+        assert np.array_equal(y, ref)
+
+
+def test_code_11_decodes_to_zero_and_linearity(cuda, oracle):
+    from tmq_amd import ops
+    rng = np.random.default_rng(5)
+    K, N, M = 512, 64, 8
+    W = _ternary(rng, N, K)
+    words = oracle.pack(W)
+    bad = words.copy()
+    bad[::7, ::2] |= (((bad[::7, ::2] >> 1) | bad[::7, ::2]) & 0x55555555 ^ 0x55555555) * 3   # turn 00 codes into 11
+    x = rng.standard_normal((M, K)).astype(np.float16)
+    tx = torch.from_numpy(x).to(cuda)
+    y = ops.ternary_linear(tx, ops.NativeWeights(torch.from_numpy(words.view(np.int32)).to(cuda), N))
+    yb = ops.ternary_linear(tx, ops.NativeWeights(torch.from_numpy(bad.view(np.int32)).to(cuda), N))
+    assert torch.equal(y, yb)
+    # linearity in x (exactly, for power-of-two factors)
+    y2 = ops.ternary_linear(tx * 2, ops.NativeWeights(torch.from_numpy(words.view(np.int32)).to(cuda), N))
+    assert torch.equal(y2, y * 2)
+
+
+def test_reference_binding_checks(cuda):
+    from tmq_amd import ops
+    w = torch.zeros(32, 4, dtype=torch.int32, device=cuda)
+    with pytest.raises(RuntimeError):
+        ops.ternary_mmm_cuda(torch.zeros(2, 32), w, 64)                       # CPU lhs
+    with pytest.raises(RuntimeError):
+        ops.ternary_mmm_cuda(torch.zeros(2, 32, device=cuda), w, 65)          # width check (tmq_cuda.cu:489)
+    with pytest.raises(RuntimeError):
+        ops.ternary_mmm_cuda(torch.zeros(2, 32, device=cuda), w, 48)          # width check (tmq_cuda.cu:490)
+    with pytest.raises(RuntimeError):
+        ops.ternary_mvm_cuda(torch.zeros(2, 32, device=cuda), w, 64)          # batch > 1 (tmq_cuda.cu:584)
+    with pytest.raises(RuntimeError):
+        ops.ternary_mmm_cuda(torch.zeros(2, 31, device=cuda), w, 64)          # K mismatch
+    assert tuple(ops.ternary_mmm_cuda(torch.zeros(32, device=cuda), w, 64).shape) == (1, 64)
+    assert tuple(ops.ternary_mmm_cuda(torch.zeros(1, 3, 5, 32, device=cuda), w, 64).shape) == (1, 3, 5, 64)

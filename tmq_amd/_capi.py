@@ -56,6 +56,8 @@ SIGNATURES = {
     "tmq_clamp_multi": (_int, [_vp, _int, _u32, _dbl, _dbl, _vp]),
     "tmq_pack_ternary": (_int, [_vp, _int, _i64, _i64, _vp, _vp]),
     "tmq_unpack_ternary": (_int, [_vp, _i64, _i64, _vp, _vp]),
+    "tmq_native_weight_bytes": (_sz, [_i64, _i64]),
+    "tmq_prepack_weights": (_int, [_vp, _i64, _i64, _i64, _i64, _vp, _vp]),
     "tmq_ternary_linear": (_int, [_vp, _int, _i64, _i64, _vp, _i64, _vp, _vp, _vp, _vp]),
     "tmq_conv2d_out_hw": (_int, [ctypes.POINTER(ConvShape), ctypes.POINTER(ctypes.c_int32),
                                  ctypes.POINTER(ctypes.c_int32)]),

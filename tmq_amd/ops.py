@@ -298,3 +298,111 @@ def decompress_ternary(input: torch.Tensor, orig_shape) -> torch.Tensor:
     src = input.contiguous()
     check(_lib().tmq_decompress_ternary(ptr(src), src.numel(), ptr(out), rows, cols), "decompress_ternary")
     return out
+
+
+# ---- ternary inference ---------------------------------------------------------------------------------
+class NativeWeights:
+    """Kernel-native re-tiling of a compact weight tensor (still 2 bits per weight), built once
+    per layer from the reference-format words; the compact tensor itself is left untouched."""
+
+    def __init__(self, words: torch.Tensor, columns: int, conv_kernel=None):
+        if words.dtype != torch.int32:
+            raise RuntimeError("expected int32 compact weights")
+        if not words.is_cuda:
+            raise RuntimeError("expected compact weights on the GPU")
+        w2 = words.reshape(-1, words.shape[-1]).contiguous()
+        self.N = int(columns)
+        self.K = int(w2.shape[0])
+        q = w2.shape[1]
+        if not (q * 16 >= self.N and q * 16 < self.N + 16):       # tmq/tmq_cuda.cu:489-490
+            raise RuntimeError("compact weight width does not match the number of output columns")
+        if conv_kernel is None:
+            C, ky, kx = self.K, 1, 1
+        else:
+            ky, kx = conv_kernel
+            if self.K % (ky * kx):
+                raise RuntimeError("compact weight rows do not match the kernel size")
+            C = self.K // (ky * kx)
+        self.C, self.ky, self.kx = C, ky, kx
+        lib = _lib()
+        self.buf = torch.empty(lib.tmq_native_weight_bytes(self.N, self.K), dtype=torch.uint8, device=words.device)
+        with torch.cuda.device(words.device):
+            check(lib.tmq_prepack_weights(ptr(w2), self.N, C, ky, kx, ptr(self.buf), stream_of(w2)), "prepack_weights")
+        self.key = (words.data_ptr(), tuple(words.shape), words._version)
+
+
+_native_cache = {}   # key -> (NativeWeights, compact tensor); insertion-ordered, least recently used first
+_NATIVE_CACHE_SIZE = 64
+
+
+def native_weights(words: torch.Tensor, columns: int, conv_kernel=None) -> NativeWeights:
+    """NativeWeights for a compact tensor, cached across calls of the raw binding functions.
+
+    The key is the storage address, shape and version counter of the compact tensor. The cache
+    keeps a reference to that tensor, so its address cannot be handed to another tensor while the
+    entry lives; entries are evicted least-recently-used."""
+    key = (words.data_ptr(), tuple(words.shape), tuple(words.stride()), words._version, int(columns), conv_kernel,
+           words.device.index)
+    hit = _native_cache.pop(key, None)
+    if hit is None:
+        hit = (NativeWeights(words, columns, conv_kernel), words)
+        while len(_native_cache) >= _NATIVE_CACHE_SIZE:
+            _native_cache.pop(next(iter(_native_cache)))
+    _native_cache[key] = hit
+    return hit[0]
+
+
+def ternary_linear(x: torch.Tensor, nw: NativeWeights, scale=None, bias=None) -> torch.Tensor:
+    """y[..., n] = scale[n] * sum_k x[..., k] T[k][n] + bias[n]; x fp16 or fp32, y fp32."""
+    _capi.require_gpu(x, "activations")
+    if x.dtype not in (torch.float16, torch.float32):
+        raise RuntimeError("ternary_linear: activations must be fp16 or fp32")
+    if x.shape[-1] != nw.K:
+        raise RuntimeError(f"ternary_linear: activations have {x.shape[-1]} features, weights expect {nw.K}")
+    for t, name in ((scale, "scale"), (bias, "bias")):
+        if t is not None:
+            _capi.require_gpu(t, name)
+            if t.dtype != torch.float32 or t.numel() != nw.N:
+                raise RuntimeError(f"ternary_linear: {name} must be fp32 with one entry per output channel")
+    M = x.numel() // nw.K if nw.K else 0
+    y = torch.empty(x.shape[:-1] + (nw.N,), dtype=torch.float32, device=x.device)
+    with torch.cuda.device(x.device):
+        check(_lib().tmq_ternary_linear(ptr(x), _capi.dtype_code(x), M, nw.K, ptr(nw.buf), nw.N, ptr(scale), ptr(bias),
+                                        ptr(y), stream_of(x)), "ternary_linear")
+    return y
+
+
+def _check_mm_args(lhs, weights, columns, name):
+    # tmq/tmq_cuda.cu:480-490, 566-575
+    if not lhs.is_cuda or not weights.is_cuda:
+        raise RuntimeError(f"{name}: expected tensors on the GPU")
+    if lhs.dtype not in (torch.float32, torch.float16):
+        raise RuntimeError(f"{name}: expected fp32 (or fp16) activations")
+    if weights.dim() != 2 or weights.dtype != torch.int32:
+        raise RuntimeError(f"{name}: expected 2-D int32 compact weights")
+    if not (weights.shape[1] * 16 >= columns and weights.shape[1] * 16 < columns + 16):
+        raise RuntimeError(f"{name}: compact weight width does not match the number of columns")
+
+
+def ternary_mmm_cuda(lhs: torch.Tensor, weights: torch.Tensor, columns: int) -> torch.Tensor:
+    """Ternary weights matrix/matrix multiplication (tmq/tmq_cuda.cu:478-549): lhs of rank 1..4
+    (rank 4 needs a leading 1), weights int32 [K][ceil(columns/16)]; returns lhs.dtype-agnostic fp32
+    of shape lhs.shape[:-1] + (columns,) (rank 1 gives [1, columns], like the reference)."""
+    _check_mm_args(lhs, weights, columns, "ternary_mmm_cuda")
+    if lhs.dim() < 1 or lhs.dim() > 4:
+        raise RuntimeError("ternary_mmm_cuda: expected an lhs of rank 1..4")
+    if lhs.dim() == 4 and lhs.shape[0] != 1:
+        raise RuntimeError("ternary_mmm_cuda: a rank-4 lhs needs a leading dimension of 1")
+    x = lhs.contiguous()
+    if x.dim() == 1:
+        x = x.view(1, -1)
+    return ternary_linear(x, native_weights(weights, columns))
+
+
+def ternary_mvm_cuda(vector: torch.Tensor, weights: torch.Tensor, columns: int) -> torch.Tensor:
+    """Ternary weights matrix/vector multiplication (tmq/tmq_cuda.cu:563-603); every leading
+    dimension of `vector` must be 1, the result keeps the rank."""
+    _check_mm_args(vector, weights, columns, "ternary_mvm_cuda")
+    if vector.dim() < 1 or vector.dim() > 4 or any(s != 1 for s in vector.shape[:-1]):
+        raise RuntimeError("ternary_mvm_cuda: expected a single vector (leading dimensions of 1)")
+    return ternary_linear(vector.contiguous(), native_weights(weights, columns))
