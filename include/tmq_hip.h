@@ -182,33 +182,45 @@ size_t tmq_native_weight_bytes(int64_t N, int64_t K);
 int tmq_prepack_weights(const uint32_t *words, int64_t N, int64_t C, int64_t ky, int64_t kx,
                         void *native, void *stream);
 
+/* Fused epilogue of the inference kernels: y = relu?( scale[n]*acc + bias[n] + residual ).
+ * scale / bias: optional fp32 [N] (NULL = 1 / 0) -- the per-channel generalisation of the
+ * reference's scalar post_scale and bias (tmq/tmq.py:684-687, 865-871), which is also where an
+ * eval-mode BatchNorm folds. residual: optional tensor of y's shape and dtype. y_dtype: TMQ_F32 or
+ * TMQ_F16. A NULL epilogue pointer means plain fp32 output.                                   */
+typedef struct tmq_epilogue {
+    const float *scale;
+    const float *bias;
+    const void *residual;
+    int32_t relu;
+    int32_t y_dtype;
+} tmq_epilogue;
+
 /* x [M][K] row-major, x_dtype TMQ_F16 or TMQ_F32 (fp32 activations are split into two fp16 terms
- * so the product keeps ~fp32 accuracy); y fp32 [M][N]; scale / bias optional fp32 [N] (NULL = 1 / 0).
+ * so the product keeps ~fp32 accuracy); y [M][N].
  * Replaces ternary_mvm_cuda (tmq/tmq_cuda.cu:563-603, kernel 242-286) for M == 1 and
  * ternary_mmm_cuda (tmq/tmq_cuda.cu:478-549, kernel 289-427) for M > 1, plus the post-scale /
  * bias passes of Linear.compact_forward (tmq/tmq.py:684-687). Any M, K, N (ragged tails masked). */
 int tmq_ternary_linear(const void *x, int x_dtype, int64_t M, int64_t K, const void *native,
-                       int64_t N, const float *scale, const float *bias, float *y, void *stream);
+                       int64_t N, const tmq_epilogue *epilogue, void *y, void *stream);
 
 /* Geometry of a 2-D convolution. */
 typedef struct tmq_conv_shape {
-    int32_t B, C, H, W;   /* input NCHW extents */
+    int32_t B, C, H, W;   /* input extents (batch, channels, height, width) */
     int32_t N;            /* output channels */
     int32_t ky, kx, sy, sx, py, px, dy, dx;
 } tmq_conv_shape;
 
-/* Output extents (PyTorch's formula). */
+/* Output extents (PyTorch's formula floor((h + 2p - d(k-1) - 1)/s) + 1; the reference's own
+ * expression at tmq/tmq.py:842-845 agrees with it on every ResNet shape).                     */
 int tmq_conv2d_out_hw(const tmq_conv_shape *s, int32_t *ho, int32_t *wo);
 
-/* Ternary implicit-GEMM convolution, no materialised im2col. x is fp16, either NCHW
- * (channels_last == 0) or NHWC (channels_last != 0); y is written in the same memory format,
- * dtype y_dtype (TMQ_F32 or TMQ_F16). words is [C*ky*kx][ceil(N/16)] with row (c*ky+i)*kx+j.
- * Optional fused epilogue: y = relu?( scale[n]*acc + bias[n] + residual ), residual in y's
- * format and dtype. Replaces the unfold + ternary_mmm_cuda + fold path of
- * Conv2d.compact_forward (tmq/tmq.py:856-871).                                               */
-int tmq_ternary_conv2d(const void *x, int channels_last, const tmq_conv_shape *shape,
-                       const uint32_t *words, const float *scale, const float *bias,
-                       const void *residual, int relu, void *y, int y_dtype, void *stream);
+/* Ternary implicit-GEMM convolution, no materialised im2col. x: fp16 NHWC [B][H][W][C]
+ * (channels_last memory); native: tmq_prepack_weights(words, N, C, ky, kx); y: NHWC
+ * [B][Ho][Wo][N] in epilogue->y_dtype. Replaces the unfold + ternary_mmm_cuda + fold path of
+ * Conv2d.compact_forward (tmq/tmq.py:856-871) and its per-batch kernel launches
+ * (tmq/tmq_cuda.cu:531-536).                                                                 */
+int tmq_ternary_conv2d(const void *x, const tmq_conv_shape *shape, const void *native,
+                       const tmq_epilogue *epilogue, void *y, void *stream);
 
 /* ------------------------------------------------------------------------------------------
  * Host entropy codec for packed tensors (host memory in, host memory out; no GPU involved).

@@ -1,0 +1,122 @@
+"""GPU parity of the MFMA tile kernel (large-M linear and implicit-GEMM convolution) vs the oracle."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _ternary(rng, shape, p0=0.5):
+    u = rng.random(shape)
+    return np.where(u < (1 - p0) / 2, 1.0, np.where(u < 1 - p0, -1.0, 0.0)).astype(np.float32)
+
+
+def _rel_err(got, want):
+    want = np.asarray(want, np.float64)
+    got = np.asarray(got, np.float64)
+    return np.max(np.abs(got - want)) / max(1e-30, np.max(np.abs(want)))
+
+
+GEMM_SHAPES = [(65, 64, 16), (128, 512, 64), (256, 4096, 256), (300, 147, 64), (1000, 576, 128), (513, 1000, 130),
+               (4096, 512, 512), (777, 2304, 256), (3136, 256, 102), (2048, 64, 64)]
+
+
+@pytest.mark.parametrize("M,K,N", GEMM_SHAPES)
+def test_large_m_linear(cuda, oracle, M, K, N):
+    from tmq_amd import ops
+    rng = np.random.default_rng(M + 3 * K + 5 * N)
+    W = _ternary(rng, (N, K))
+    words = oracle.pack(W)
+    x = rng.standard_normal((M, K)).astype(np.float16)
+    scale = (0.5 + rng.random(N)).astype(np.float32)
+    bias = rng.standard_normal(N).astype(np.float32)
+    nw = ops.NativeWeights(torch.from_numpy(words.view(np.int32)).to(cuda), N)
+    tx = torch.from_numpy(x).to(cuda)
+    ts, tb = torch.from_numpy(scale).to(cuda), torch.from_numpy(bias).to(cuda)
+    y = ops.ternary_linear(tx, nw, ts, tb)
+    ref = (x.astype(np.float64) @ W.astype(np.float64).T) * scale + bias
+    assert _rel_err(y.cpu().numpy(), ref) <= 1e-3
+    assert _rel_err(y.cpu().numpy(), ref) <= 3e-6
+    # exact on small integers, whatever the summation order
+    xi = rng.integers(-4, 5, (M, K)).astype(np.float16)
+    yi = ops.ternary_linear(torch.from_numpy(xi).to(cuda), nw).cpu().numpy()
+    assert np.array_equal(yi, (xi.astype(np.int64) @ W.astype(np.int64).T).astype(np.float32))
+    # fused epilogue: residual + relu, fp32 and fp16 outputs
+    res = torch.from_numpy(rng.standard_normal((M, N)).astype(np.float32)).to(cuda)
+    y2 = ops.ternary_linear(tx, nw, ts, tb, residual=res, relu=True)
+    assert _rel_err(y2.cpu().numpy(), np.maximum(ref + res.cpu().numpy(), 0)) <= 3e-6
+    y3 = ops.ternary_linear(tx, nw, ts, tb, residual=res.half(), relu=True, out_dtype=torch.float16)
+    want3 = np.maximum(ref + res.half().cpu().numpy().astype(np.float64), 0)
+    assert _rel_err(y3.float().cpu().numpy(), want3) <= 1e-3
+
+
+def test_skinny_and_tile_kernels_agree(cuda, oracle):
+    """M = 64 (skinny kernel) and M = 65 (tile kernel) must give the same rows for integer data."""
+    from tmq_amd import ops
+    rng = np.random.default_rng(0)
+    K, N = 1024, 192
+    W = _ternary(rng, (N, K))
+    nw = ops.NativeWeights(torch.from_numpy(oracle.pack(W).view(np.int32)).to(cuda), N)
+    x = torch.from_numpy(rng.integers(-6, 7, (65, K)).astype(np.float16)).to(cuda)
+    assert torch.equal(ops.ternary_linear(x[:64], nw), ops.ternary_linear(x, nw)[:64])
+
+
+CONV_CASES = [  # B, C, H, W, N, k, stride, pad, dil
+    (2, 8, 9, 9, 16, 3, 1, 1, 1), (1, 16, 14, 14, 32, 3, 2, 1, 1), (2, 64, 8, 8, 64, 3, 1, 1, 1),
+    (3, 3, 20, 20, 64, 7, 2, 3, 1), (2, 64, 7, 7, 128, 1, 2, 0, 1), (1, 24, 10, 11, 20, (3, 2), (2, 1), (1, 0), 1),
+    (1, 8, 12, 12, 17, 3, 1, 2, 2), (2, 5, 9, 9, 10, 3, 1, 1, 1), (1, 128, 14, 14, 256, 3, 1, 1, 1),
+    (4, 64, 16, 16, 64, 3, 1, 1, 1), (1, 8, 7, 7, 8, 3, 2, 0, 1),
+]
+
+
+@pytest.mark.parametrize("B,C,H,W,N,k,stride,pad,dil", CONV_CASES)
+def test_conv2d_matches_oracle(cuda, oracle, B, C, H, W, N, k, stride, pad, dil):
+    from tmq_amd import ops
+    pair = lambda v: tuple(v) if isinstance(v, tuple) else (v, v)
+    k, stride, pad, dil = pair(k), pair(stride), pair(pad), pair(dil)
+    rng = np.random.default_rng(B + C + H + N)
+    Wt = _ternary(rng, (N, C, k[0], k[1]))
+    words = oracle.pack(Wt.reshape(N, -1))
+    x = rng.standard_normal((B, C, H, W)).astype(np.float16)
+    scale = (0.5 + rng.random(N)).astype(np.float32)
+    bias = rng.standard_normal(N).astype(np.float32)
+    packed = ops.compactify_ternary(torch.from_numpy(Wt).to(cuda))
+    assert np.array_equal(packed.cpu().numpy().view(np.uint32).reshape(words.shape), words)
+    nw = ops.NativeWeights(packed, N, conv_kernel=k)
+    tx = torch.from_numpy(x).to(cuda)
+    ts, tb = torch.from_numpy(scale).to(cuda), torch.from_numpy(bias).to(cuda)
+    y = ops.ternary_conv2d(tx, nw, stride, pad, dil, ts, tb)
+    want = oracle.conv2d(x.astype(np.float32), words, N, k, stride, pad, dil, scale, bias)
+    assert tuple(y.shape) == want.shape
+    assert y.is_contiguous(memory_format=torch.channels_last)
+    assert _rel_err(y.cpu().numpy(), want) <= 1e-3
+    assert _rel_err(y.cpu().numpy(), want) <= 3e-6
+    # the library routine on expanded weights
+    ref = torch.nn.functional.conv2d(torch.from_numpy(x).double(), torch.from_numpy(Wt).double(), None, stride, pad, dil)
+    ref = ref * torch.from_numpy(scale).double().view(1, -1, 1, 1) + torch.from_numpy(bias).double().view(1, -1, 1, 1)
+    assert _rel_err(y.cpu().numpy(), ref.numpy()) <= 3e-6
+    # fp16 output with fused residual + relu
+    res = torch.from_numpy(rng.standard_normal(want.shape).astype(np.float16)).to(cuda).contiguous(
+        memory_format=torch.channels_last)
+    y16 = ops.ternary_conv2d(tx, nw, stride, pad, dil, ts, tb, residual=res, relu=True, out_dtype=torch.float16)
+    want16 = np.maximum(want + res.float().cpu().numpy(), 0)
+    assert _rel_err(y16.float().cpu().numpy(), want16) <= 1e-3
+
+
+def test_resnet_layer_shapes_against_torch(cuda):
+    """Full-size ResNet-18 layer shapes (batch 8): checked against torch's fp32 convolution on the
+    expanded weights, which the small cases above tie to the oracle."""
+    from tmq_amd import ops
+    g = torch.Generator().manual_seed(20)
+    shapes = [(3, 224, 64, 7, 2, 3), (64, 56, 64, 3, 1, 1), (64, 56, 128, 3, 2, 1), (64, 56, 128, 1, 2, 0),
+              (128, 28, 128, 3, 1, 1), (128, 28, 256, 3, 2, 1), (256, 14, 256, 3, 1, 1), (256, 14, 512, 3, 2, 1),
+              (512, 7, 512, 3, 1, 1)]
+    for C, HW, N, k, s, p in shapes:
+        u = torch.rand(N, C, k, k, generator=g)
+        Wt = torch.where(u < .25, 1.0, torch.where(u < .5, -1.0, 0.0))
+        x = torch.randn(8, C, HW, HW, generator=g).half()
+        nw = ops.NativeWeights(ops.compactify_ternary(Wt.to(cuda)), N, conv_kernel=(k, k))
+        y = ops.ternary_conv2d(x.to(cuda), nw, s, p)
+        ref = torch.nn.functional.conv2d(x.to(cuda).float(), Wt.to(cuda), None, s, p)
+        err = (y - ref).abs().max().item() / ref.abs().max().item()
+        assert err <= 1e-5, (C, HW, N, k, err)

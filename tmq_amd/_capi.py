@@ -32,6 +32,12 @@ class ConvShape(ctypes.Structure):
                 ("B", "C", "H", "W", "N", "ky", "kx", "sy", "sx", "py", "px", "dy", "dx")]
 
 
+class Epilogue(ctypes.Structure):
+    """tmq_epilogue of include/tmq_hip.h."""
+    _fields_ = [("scale", ctypes.c_void_p), ("bias", ctypes.c_void_p), ("residual", ctypes.c_void_p),
+                ("relu", ctypes.c_int32), ("y_dtype", ctypes.c_int32)]
+
+
 _vp, _sz, _dbl, _i64, _int, _flt, _u32 = (ctypes.c_void_p, ctypes.c_size_t, ctypes.c_double, ctypes.c_int64,
                                            ctypes.c_int, ctypes.c_float, ctypes.c_uint32)
 
@@ -58,10 +64,10 @@ SIGNATURES = {
     "tmq_unpack_ternary": (_int, [_vp, _i64, _i64, _vp, _vp]),
     "tmq_native_weight_bytes": (_sz, [_i64, _i64]),
     "tmq_prepack_weights": (_int, [_vp, _i64, _i64, _i64, _i64, _vp, _vp]),
-    "tmq_ternary_linear": (_int, [_vp, _int, _i64, _i64, _vp, _i64, _vp, _vp, _vp, _vp]),
+    "tmq_ternary_linear": (_int, [_vp, _int, _i64, _i64, _vp, _i64, _vp, _vp, _vp]),
     "tmq_conv2d_out_hw": (_int, [ctypes.POINTER(ConvShape), ctypes.POINTER(ctypes.c_int32),
                                  ctypes.POINTER(ctypes.c_int32)]),
-    "tmq_ternary_conv2d": (_int, [_vp, _int, ctypes.POINTER(ConvShape), _vp, _vp, _vp, _vp, _int, _vp, _int, _vp]),
+    "tmq_ternary_conv2d": (_int, [_vp, ctypes.POINTER(ConvShape), _vp, _vp, _vp, _vp]),
     "tmq_compress_bound": (_sz, [_i64, _i64]),
     "tmq_compress_ternary": (_int, [_vp, _i64, _i64, _vp, _sz, ctypes.POINTER(_sz)]),
     "tmq_decompress_ternary": (_int, [_vp, _sz, _vp, _i64, _i64]),

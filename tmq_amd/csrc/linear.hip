@@ -99,7 +99,8 @@ template <int MT, bool X32, bool VEC>
 __global__ __launch_bounds__(1024) void skinny_kernel(const void *__restrict__ x, int64_t M, int64_t K,
                                                       const u32x4 *__restrict__ native, int64_t Kb, int64_t N,
                                                       const float *__restrict__ scale, const float *__restrict__ bias,
-                                                      float *__restrict__ y) {
+                                                      const void *__restrict__ residual, int relu, void *__restrict__ y,
+                                                      int y_f16) {
     extern __shared__ float red[];   // [waves][MT][64][4]
     const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6, waves = blockDim.x >> 6;
     const int j = lane & 15, g = lane >> 4;
@@ -148,15 +149,27 @@ __global__ __launch_bounds__(1024) void skinny_kernel(const void *__restrict__ x
                 const float sc = (scale ? scale[n] : 1.0f) * (1.0f / kWeightUnit);
                 float v = s[r] * sc;
                 if (bias) v += bias[n];
-                y[m * N + n] = v;
+                const int64_t o = m * N + n;
+                if (y_f16) {
+                    if (residual) v += (float)static_cast<const _Float16 *>(residual)[o];
+                    if (relu) v = v > 0.f ? v : 0.f;
+                    static_cast<_Float16 *>(y)[o] = (_Float16)v;
+                } else {
+                    if (residual) v += static_cast<const float *>(residual)[o];
+                    if (relu) v = v > 0.f ? v : 0.f;
+                    static_cast<float *>(y)[o] = v;
+                }
             }
         }
     }
 }
 
 template <int MT, bool X32>
-int launch_skinny(const void *x, int64_t M, int64_t K, const void *native, int64_t N, const float *scale,
-                  const float *bias, float *y, void *stream) {
+int launch_skinny(const void *x, int64_t M, int64_t K, const void *native, int64_t N, const tmq_epilogue &ep,
+                  void *y, void *stream) {
+    const float *scale = ep.scale, *bias = ep.bias;
+    const void *residual = ep.residual;
+    const int relu = ep.relu, y_f16 = ep.y_dtype == TMQ_F16;
     const int64_t Nb = native_blocks_n(N), Kb = native_blocks_k(K);
     int waves = 16;
     while (waves > 1 && (waves > Kb || waves * MT > 32)) waves >>= 1;
@@ -167,35 +180,29 @@ int launch_skinny(const void *x, int64_t M, int64_t K, const void *native, int64
     const u32x4 *nat = static_cast<const u32x4 *>(native);
     if (vec)
         hipLaunchKernelGGL((skinny_kernel<MT, X32, true>), grid, block, lds, as_stream(stream), x, M, K, nat, Kb, N, scale,
-                           bias, y);
+                           bias, residual, relu, y, y_f16);
     else
         hipLaunchKernelGGL((skinny_kernel<MT, X32, false>), grid, block, lds, as_stream(stream), x, M, K, nat, Kb, N,
-                           scale, bias, y);
+                           scale, bias, residual, relu, y, y_f16);
     return check_launch();
+}
+
+template <bool X32>
+int skinny_rows(const void *x, int64_t M, int64_t K, const void *native, int64_t N, const tmq_epilogue &ep, void *y,
+                void *stream) {
+    switch ((int)((M + 15) / 16)) {
+        case 1: return launch_skinny<1, X32>(x, M, K, native, N, ep, y, stream);
+        case 2: return launch_skinny<2, X32>(x, M, K, native, N, ep, y, stream);
+        case 3: return launch_skinny<3, X32>(x, M, K, native, N, ep, y, stream);
+        default: return launch_skinny<4, X32>(x, M, K, native, N, ep, y, stream);
+    }
 }
 
 }  // namespace
 
-// Large M (temporary until the MFMA-bound tile kernel lands): 64-row slabs through the skinny kernel.
-int launch_gemm_dense(const void *x, int x_dtype, int64_t M, int64_t K, const void *native, int64_t N,
-                      const float *scale, const float *bias, float *y, void *stream) {
-    const bool x32 = x_dtype == TMQ_F32;
-    const size_t esz = x32 ? 4 : 2;
-    for (int64_t m0 = 0; m0 < M; m0 += 64) {
-        const int64_t mm = M - m0 < 64 ? M - m0 : 64;
-        const void *xs = static_cast<const char *>(x) + (size_t)m0 * K * esz;
-        const int mt = (int)((mm + 15) / 16);
-        int rc;
-        switch (mt) {
-            case 1: rc = x32 ? launch_skinny<1, true>(xs, mm, K, native, N, scale, bias, y + m0 * N, stream) : launch_skinny<1, false>(xs, mm, K, native, N, scale, bias, y + m0 * N, stream); break;
-            case 2: rc = x32 ? launch_skinny<2, true>(xs, mm, K, native, N, scale, bias, y + m0 * N, stream) : launch_skinny<2, false>(xs, mm, K, native, N, scale, bias, y + m0 * N, stream); break;
-            case 3: rc = x32 ? launch_skinny<3, true>(xs, mm, K, native, N, scale, bias, y + m0 * N, stream) : launch_skinny<3, false>(xs, mm, K, native, N, scale, bias, y + m0 * N, stream); break;
-            default: rc = x32 ? launch_skinny<4, true>(xs, mm, K, native, N, scale, bias, y + m0 * N, stream) : launch_skinny<4, false>(xs, mm, K, native, N, scale, bias, y + m0 * N, stream); break;
-        }
-        if (rc != TMQ_OK) return rc;
-    }
-    return TMQ_OK;
-}
+// gemm.hip: the MFMA-bound tile kernel for large M (fp16 activations).
+int launch_gemm_dense(const void *x, int64_t M, int64_t K, const void *native, int64_t N, const float *scale,
+                      const float *bias, const void *residual, int relu, void *y, int y_f16, void *stream);
 
 }  // namespace tmq
 
@@ -222,24 +229,32 @@ int tmq_prepack_weights(const uint32_t *words, int64_t N, int64_t C, int64_t ky,
 }
 
 int tmq_ternary_linear(const void *x, int x_dtype, int64_t M, int64_t K, const void *native, int64_t N,
-                       const float *scale, const float *bias, float *y, void *stream) {
+                       const tmq_epilogue *epilogue, void *y, void *stream) {
     if (M < 0 || K <= 0 || N <= 0) return TMQ_ERR_INVALID_ARG;
     if (M == 0) return TMQ_OK;
     if (!x || !native || !y || !aligned16(native)) return TMQ_ERR_INVALID_ARG;
     if (x_dtype != TMQ_F16 && x_dtype != TMQ_F32) return TMQ_ERR_UNSUPPORTED;
+    tmq_epilogue ep = {nullptr, nullptr, nullptr, 0, TMQ_F32};
+    if (epilogue) ep = *epilogue;
+    if (ep.y_dtype != TMQ_F16 && ep.y_dtype != TMQ_F32) return TMQ_ERR_UNSUPPORTED;
     const bool x32 = x_dtype == TMQ_F32;
-    if (M <= 64) {
-        const int mt = (int)((M + 15) / 16);
-#define TMQ_SK(MT)                                                                                      \
-    case MT:                                                                                            \
-        return x32 ? launch_skinny<MT, true>(x, M, K, native, N, scale, bias, y, stream)                \
-                   : launch_skinny<MT, false>(x, M, K, native, N, scale, bias, y, stream);
-        switch (mt) {
-            TMQ_SK(1) TMQ_SK(2) TMQ_SK(3) TMQ_SK(4)
-        }
-#undef TMQ_SK
+    if (M <= 64) return x32 ? skinny_rows<true>(x, M, K, native, N, ep, y, stream)
+                            : skinny_rows<false>(x, M, K, native, N, ep, y, stream);
+    if (!x32)
+        return launch_gemm_dense(x, M, K, native, N, ep.scale, ep.bias, ep.residual, ep.relu, y,
+                                 ep.y_dtype == TMQ_F16, stream);
+    // fp32 activations with M > 64: 64-row slabs through the two-term skinny kernel (keeps fp32
+    // accuracy; the fp16 tile kernel is the fast path).
+    const size_t ysz = ep.y_dtype == TMQ_F16 ? 2 : 4;
+    for (int64_t m0 = 0; m0 < M; m0 += 64) {
+        const int64_t mm = M - m0 < 64 ? M - m0 : 64;
+        tmq_epilogue e2 = ep;
+        if (ep.residual) e2.residual = static_cast<const char *>(ep.residual) + (size_t)m0 * N * ysz;
+        int rc = skinny_rows<true>(static_cast<const char *>(x) + (size_t)m0 * K * 4, mm, K, native, N, e2,
+                                   static_cast<char *>(y) + (size_t)m0 * N * ysz, stream);
+        if (rc != TMQ_OK) return rc;
     }
-    return launch_gemm_dense(x, x_dtype, M, K, native, N, scale, bias, y, stream);
+    return TMQ_OK;
 }
 
 }  // extern "C"

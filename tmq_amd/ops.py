@@ -352,23 +352,69 @@ def native_weights(words: torch.Tensor, columns: int, conv_kernel=None) -> Nativ
     return hit[0]
 
 
-def ternary_linear(x: torch.Tensor, nw: NativeWeights, scale=None, bias=None) -> torch.Tensor:
-    """y[..., n] = scale[n] * sum_k x[..., k] T[k][n] + bias[n]; x fp16 or fp32, y fp32."""
+def _epilogue(nw, scale, bias, residual, relu, out_dtype, y):
+    for t, name in ((scale, "scale"), (bias, "bias")):
+        if t is not None:
+            _capi.require_gpu(t, name)
+            if t.dtype != torch.float32 or t.numel() != nw.N:
+                raise RuntimeError(f"{name} must be fp32 with one entry per output channel")
+    if out_dtype not in (torch.float32, torch.float16):
+        raise RuntimeError("output dtype must be fp32 or fp16")
+    if residual is not None:
+        if residual.dtype != out_dtype or residual.shape != y.shape or residual.stride() != y.stride():
+            raise RuntimeError("residual must match the output in shape, dtype and memory format")
+    ep = _capi.Epilogue()
+    ep.scale = scale.data_ptr() if scale is not None else None
+    ep.bias = bias.data_ptr() if bias is not None else None
+    ep.residual = residual.data_ptr() if residual is not None else None
+    ep.relu = int(bool(relu))
+    ep.y_dtype = _capi.F16 if out_dtype == torch.float16 else _capi.F32
+    return ep
+
+
+def ternary_linear(x: torch.Tensor, nw: NativeWeights, scale=None, bias=None, residual=None, relu=False,
+                   out_dtype=torch.float32) -> torch.Tensor:
+    """y[..., n] = relu?(scale[n] * sum_k x[..., k] T[k][n] + bias[n] + residual); x fp16 or fp32."""
     _capi.require_gpu(x, "activations")
     if x.dtype not in (torch.float16, torch.float32):
         raise RuntimeError("ternary_linear: activations must be fp16 or fp32")
     if x.shape[-1] != nw.K:
         raise RuntimeError(f"ternary_linear: activations have {x.shape[-1]} features, weights expect {nw.K}")
-    for t, name in ((scale, "scale"), (bias, "bias")):
-        if t is not None:
-            _capi.require_gpu(t, name)
-            if t.dtype != torch.float32 or t.numel() != nw.N:
-                raise RuntimeError(f"ternary_linear: {name} must be fp32 with one entry per output channel")
     M = x.numel() // nw.K if nw.K else 0
-    y = torch.empty(x.shape[:-1] + (nw.N,), dtype=torch.float32, device=x.device)
+    y = torch.empty(x.shape[:-1] + (nw.N,), dtype=out_dtype, device=x.device)
+    ep = _epilogue(nw, scale, bias, residual, relu, out_dtype, y)
     with torch.cuda.device(x.device):
-        check(_lib().tmq_ternary_linear(ptr(x), _capi.dtype_code(x), M, nw.K, ptr(nw.buf), nw.N, ptr(scale), ptr(bias),
+        check(_lib().tmq_ternary_linear(ptr(x), _capi.dtype_code(x), M, nw.K, ptr(nw.buf), nw.N, ctypes.byref(ep),
                                         ptr(y), stream_of(x)), "ternary_linear")
+    return y
+
+
+def ternary_conv2d(x: torch.Tensor, nw: NativeWeights, stride=1, padding=0, dilation=1, scale=None, bias=None,
+                   residual=None, relu=False, out_dtype=torch.float32) -> torch.Tensor:
+    """Implicit-GEMM ternary convolution. x: fp16 [B, C, H, W] in channels_last memory (any other
+    layout / fp32 is converted first); nw: NativeWeights built with conv_kernel=(ky, kx). Returns
+    [B, N, Ho, Wo] in channels_last memory."""
+    pair = lambda v: tuple(v) if isinstance(v, (tuple, list)) else (v, v)
+    (sy, sx), (py, px), (dy, dx) = pair(stride), pair(padding), pair(dilation)
+    if not x.is_cuda or x.dim() != 4:
+        raise RuntimeError("ternary_conv2d: expected a 4-D GPU tensor")
+    if x.shape[1] != nw.C:
+        raise RuntimeError(f"ternary_conv2d: input has {x.shape[1]} channels, weights expect {nw.C}")
+    if x.dtype != torch.float16 or not x.is_contiguous(memory_format=torch.channels_last):
+        x = x.to(dtype=torch.float16, memory_format=torch.channels_last)
+    B, C, H, W = x.shape
+    shp = _capi.ConvShape(B, C, H, W, nw.N, nw.ky, nw.kx, sy, sx, py, px, dy, dx)
+    ho, wo = ctypes.c_int32(0), ctypes.c_int32(0)
+    lib = _lib()
+    check(lib.tmq_conv2d_out_hw(ctypes.byref(shp), ctypes.byref(ho), ctypes.byref(wo)), "conv2d_out_hw")
+    if ho.value <= 0 or wo.value <= 0:
+        raise RuntimeError("ternary_conv2d: empty output")
+    y = torch.empty((B, nw.N, ho.value, wo.value), dtype=out_dtype, device=x.device,
+                    memory_format=torch.channels_last)
+    ep = _epilogue(nw, scale, bias, residual, relu, out_dtype, y)
+    with torch.cuda.device(x.device):
+        check(lib.tmq_ternary_conv2d(ptr(x), ctypes.byref(shp), ptr(nw.buf), ctypes.byref(ep), ptr(y), stream_of(x)),
+              "ternary_conv2d")
     return y
 
 
