@@ -147,6 +147,49 @@ def bench_softstep(args, torch):
     return res
 
 
+def bench_linear(args, torch):
+    """BASELINE configs[2]: y = x W^T, K = N = 4096, 2-bit packed ternary W (P(0) = .5), fp16 x, one
+    fp32 scale per output channel, fp32 accumulation; M in {1, 16, 256, 4096}. M = 1 rotates over
+    distinct weight buffers (> 256 MB in total) so that the packed weights come from HBM, not
+    from L2 / Infinity Cache."""
+    from tmq_amd import ops
+    dev = torch.device("cuda:0")
+    K = N = 4096
+    gen = lambda s: torch.Generator(device="cpu").manual_seed(s)
+    u = torch.rand(N, K, generator=gen(10))
+    W = torch.where(u < .25, 1.0, torch.where(u < .5, -1.0, 0.0))
+    packed = ops.compactify_ternary(W.to(dev))
+    scale = (0.5 + torch.rand(N, generator=gen(11))).to(dev)
+    nrot = 72 if args.rotate else 1
+    natives = [ops.NativeWeights(packed.clone(), N) for _ in range(nrot)]
+    out = {}
+    for M in [int(m) for m in args.m_list.split(",")]:
+        x = torch.randn(M, K, generator=gen(12)).half().to(dev)
+        reps = args.steps if M < 4096 else max(10, args.steps // 4)
+        for i in range(max(args.warmup, 3)):
+            ops.ternary_linear(x, natives[i % nrot], scale)
+        t_settle = time.perf_counter()
+        while time.perf_counter() - t_settle < args.settle_ms * 1e-3:
+            ops.ternary_linear(x, natives[0], scale)
+            torch.cuda.synchronize()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for i in range(reps):
+            ops.ternary_linear(x, natives[i % nrot], scale)
+        e1.record()
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) / reps * 1e3
+        flops = 2.0 * M * N * K
+        byts = K * N / 4 + 2 * M * K + 4 * M * N + 4 * N
+        out[str(M)] = {"us": round(us, 3), "tflops": round(flops / us / 1e6, 3), "gbs": round(byts / us / 1e3, 2),
+                       "frac_hbm": round(byts / us / 1e3 / HBM_PEAK_GBS, 4),
+                       "frac_mfma_fp16": round(flops / us / 1e6 / 2500.0, 4)}
+    return {"metric": "ternary-GEMM eff. TFLOP/s (K=N=4096)", "unit": "TFLOP/s", "n_gpus": 1, "dtype": "f16",
+            "data": "synthetic", "config": {"workload": "configs[2]: ternary linear K=N=4096", "rotate_buffers": nrot},
+            "value": out.get("4096", {}).get("tflops"), "by_M": out}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -158,6 +201,8 @@ def main():
     ap.add_argument("--elements", type=int, default=1 << 26)
     ap.add_argument("--cpu-sample", type=int, default=1 << 22)
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--m-list", default="1,16,256,4096")
+    ap.add_argument("--rotate", type=int, default=1)
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build targets one GPU; --gpus N with N > 1 is not supported (the path has no "
@@ -169,9 +214,11 @@ def main():
         sys.exit(1)
     if args.workload == "softstep":
         res = bench_softstep(args, torch)
+    elif args.workload == "linear":
+        res = bench_linear(args, torch)
     else:
-        from tmq_amd import bench_extra
-        res = bench_extra.run(args, torch)
+        print(f"bench.py: unknown workload {args.workload}", file=sys.stderr)
+        sys.exit(2)
     print(json.dumps(res))
 
 

@@ -23,10 +23,6 @@
 #include <stdlib.h>
 #include <string.h>
 
-#if defined(__FP_FAST_FMAF) && 0
-#error "unexpected"
-#endif
-
 /* ------------------------------------------------------------------------------------------
  * Host scalars. The reference evaluates them as Python doubles and hands them to torch, which
  * rounds a Python scalar to fp32 once when it meets an fp32 tensor.
@@ -305,10 +301,13 @@ void tmq_oracle_unpack(const uint32_t *in, int64_t N, int64_t K, float *out, int
 
 /* The reference's 2-D expander as written (tmq/tmq_native.cpp:220-234, called at 520-523 with
  * rows = origShape[0], columns = origShape[1]): it reads the words as [rows][ceil(columns/16)],
- * which is NOT the layout the packer wrote unless rows == columns. Kept for documentation of
- * the defect; the product implements tmq_oracle_unpack.                                      */
-void tmq_oracle_unpack_ref2d_as_written(const uint32_t *in, int64_t rows, int64_t cols, float *out) {
+ * which is NOT the layout the packer wrote unless rows == columns, and it reads past the end of
+ * the packed buffer whenever rows*ceil(columns/16) exceeds the number of words. Kept only to
+ * document the defect; `nwords` bounds the reads (returns -1 if the reference would read out of
+ * bounds). The product implements tmq_oracle_unpack.                                          */
+int tmq_oracle_unpack_ref2d_as_written(const uint32_t *in, int64_t nwords, int64_t rows, int64_t cols, float *out) {
     int64_t Q = (cols + 15) / 16;
+    if (rows * Q > nwords) return -1;
     for (int64_t r = 0; r < rows; r++)
         for (int64_t c = 0; c < Q; c++) {
             uint32_t word = in[r * Q + c];
@@ -316,6 +315,7 @@ void tmq_oracle_unpack_ref2d_as_written(const uint32_t *in, int64_t rows, int64_
                 if (c * 16 + j < cols)
                     out[r * cols + c * 16 + j] = value_from_code((int)((word >> (2 * (15 - j))) & 3u), 1);
         }
+    return 0;
 }
 
 /* ------------------------------------------------------------------------------------------

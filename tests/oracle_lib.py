@@ -39,7 +39,8 @@ def lib():
         L.tmq_oracle_sum64.restype = _dbl
         L.tmq_oracle_pack.argtypes = [ctypes.c_void_p, _int, _i64, _i64, _u32p]
         L.tmq_oracle_unpack.argtypes = [_u32p, _i64, _i64, _f32p, _int]
-        L.tmq_oracle_unpack_ref2d_as_written.argtypes = [_u32p, _i64, _i64, _f32p]
+        L.tmq_oracle_unpack_ref2d_as_written.argtypes = [_u32p, _i64, _i64, _i64, _f32p]
+        L.tmq_oracle_unpack_ref2d_as_written.restype = _int
         L.tmq_oracle_gemm.argtypes = [_f32p, _i64, _i64, _u32p, _i64, ctypes.c_void_p, ctypes.c_void_p, _f64p]
         L.tmq_oracle_conv2d.argtypes = [_f32p] + [_i64] * 4 + [_u32p] + [_i64] * 9 + [ctypes.c_void_p,
                                                                                      ctypes.c_void_p, _f64p]
@@ -132,8 +133,8 @@ def unpack(words, N, K, host_rule=0):
 def unpack_ref2d_as_written(words, rows, cols):
     words = np.ascontiguousarray(words, dtype=np.uint32)
     out = np.zeros((rows, cols), dtype=np.float32)
-    lib().tmq_oracle_unpack_ref2d_as_written(words.reshape(-1), rows, cols, out.reshape(-1))
-    return out
+    rc = lib().tmq_oracle_unpack_ref2d_as_written(words.reshape(-1), words.size, rows, cols, out.reshape(-1))
+    return out if rc == 0 else None
 
 
 def _opt(a):
