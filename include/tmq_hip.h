@@ -72,6 +72,15 @@ int tmq_softstep_deriv_fwd(const float *w, float *q, size_t n, double digamma, d
 int tmq_softstep_deriv_bwd(const float *w, const float *g, float *dw, size_t n, double digamma,
                            double strength, void *stream);
 
+/* y = SoftStep.map(w) (derivative == 0) or SoftStep.dmap(w) (derivative != 0): the staircase /
+ * its slope with the argument association of tmq/tmq.py:335-338 / 348-350 (used for logging and
+ * for the final ternarisation).                                                              */
+int tmq_softstep_map(const float *w, float *y, size_t n, double digamma, int derivative, void *stream);
+
+/* y = sigmoid / dsigmoid / d2sigmoid (order 0 / 1 / 2) of an arbitrary fp32 tensor: the rational
+ * pieces SoftStep.sigmoid, dsigmoid, d2sigmoid (tmq/tmq.py:353-381).                          */
+int tmq_sigmoid_piece(const float *x, float *y, size_t n, int order, void *stream);
+
 /* w <- clamp(w, lo, hi) in place (NaN stays NaN).
  * Replaces the torch.clamp pass of Linear.clamp / Conv2d.clamp (tmq/tmq.py:691-696, 874-879)
  * driven by QuantizationControl.clamp (tmq/tmq.py:263-272).                                  */
@@ -134,11 +143,14 @@ int tmq_qloss_multi(const tmq_segment *segs_dev, int nseg, uint32_t total_blocks
                     double strength, float *per_tensor, float *total, void *workspace,
                     void *stream);
 
-/* aux_l[i] (= or +=) scalar_l * Q'(w_l[i]; sharpness, strength): the gradient of the loss above
- * w.r.t. every weight, scalar_l = upstream_grad / n_l as autograd's mean backward produces it.
- * accumulate != 0 adds into aux (fused grad accumulation), else overwrites.                  */
+/* aux_l[i] (= or +=) s_l * Q'(w_l[i]; sharpness, strength): the gradient of the loss above w.r.t.
+ * every weight. With upstream (device, 1 float: the gradient arriving at the total loss)
+ * s_l = upstream / float(n_l), the value autograd's mean backward produces; with upstream NULL
+ * s_l is the table's scalar_l. accumulate != 0 adds into aux (fused grad accumulation), else
+ * overwrites. Arithmetic of tmq/tmq.py:488-493.                                              */
 int tmq_qloss_bwd_multi(const tmq_segment *segs_dev, int nseg, uint32_t total_blocks,
-                        double sharpness, double strength, int accumulate, void *stream);
+                        double sharpness, double strength, const float *upstream, int accumulate,
+                        void *stream);
 
 /* w_l <- clamp(w_l, lo, hi) for every segment, one launch. */
 int tmq_clamp_multi(const tmq_segment *segs_dev, int nseg, uint32_t total_blocks, double lo,

@@ -1,2 +1,9 @@
-"""tmq_amd -- MI355X-native implementation of TMQ's GPU hot path behind TMQ's Python API."""
-from . import _capi  # noqa: F401
+"""tmq_amd -- MI355X-native implementation of TMQ's GPU hot path behind TMQ's Python API.
+
+    from tmq_amd import quantize_model, QuantizationControl, ...     # same names as the reference's `tmq`
+"""
+from .tmq import *  # noqa: F401,F403
+from .tmq import (QuantMode, TensorType, QuantizationScheduleBuilder, QuantizationControl, SoftStep,  # noqa: F401
+                  SoftStepDerivative, TMQLayer, Linear, Conv2d, ConvTranspose2d, quantize_weights, quantize_model,
+                  compressed_state_dict, prepare_compressed_load, load_compressed_state_dict, expand_compact_layers,
+                  CUDA_EXT_AVAILABLE, NATIVE_EXT_AVAILABLE)

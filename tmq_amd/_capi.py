@@ -50,6 +50,8 @@ SIGNATURES = {
     "tmq_softstep_bwd": (_int, [_vp, _vp, _vp, _sz, _dbl, _dbl, _vp]),
     "tmq_softstep_deriv_fwd": (_int, [_vp, _vp, _sz, _dbl, _dbl, _vp]),
     "tmq_softstep_deriv_bwd": (_int, [_vp, _vp, _vp, _sz, _dbl, _dbl, _vp]),
+    "tmq_softstep_map": (_int, [_vp, _vp, _sz, _dbl, _int, _vp]),
+    "tmq_sigmoid_piece": (_int, [_vp, _vp, _sz, _int, _vp]),
     "tmq_clamp_inplace": (_int, [_vp, _sz, _dbl, _dbl, _vp]),
     "tmq_ternarize_inplace": (_int, [_vp, _sz, _dbl, _vp]),
     "tmq_softstep_fused_workspace_bytes": (_sz, [_sz]),
@@ -58,7 +60,7 @@ SIGNATURES = {
     "tmq_multi_plan": (_int, [ctypes.POINTER(Segment), _int, ctypes.POINTER(_u32)]),
     "tmq_qloss_multi_workspace_bytes": (_sz, [_u32]),
     "tmq_qloss_multi": (_int, [_vp, _int, _u32, _dbl, _dbl, _vp, _vp, _vp, _vp]),
-    "tmq_qloss_bwd_multi": (_int, [_vp, _int, _u32, _dbl, _dbl, _int, _vp]),
+    "tmq_qloss_bwd_multi": (_int, [_vp, _int, _u32, _dbl, _dbl, _vp, _int, _vp]),
     "tmq_clamp_multi": (_int, [_vp, _int, _u32, _dbl, _dbl, _vp]),
     "tmq_pack_ternary": (_int, [_vp, _int, _i64, _i64, _vp, _vp]),
     "tmq_unpack_ternary": (_int, [_vp, _i64, _i64, _vp, _vp]),

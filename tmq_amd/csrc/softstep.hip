@@ -119,6 +119,42 @@ struct TernarizeOp {  // tmq/tmq.py:293-295 with SoftStep.map 335-338 (in place)
     }
 };
 
+// SoftStep.map / SoftStep.dmap (tmq/tmq.py:328-350): the same staircase and slope with the
+// argument association d*w - d*floor(w) - d/2 (map) and w*d - d*floor(w) - d/2 (dmap).
+template <bool DERIV>
+struct MapOp {
+    TMQ_OP_FLAGS(false, true, false, false, false, false);
+    StepK s;
+    template <bool CAREFUL>
+    __device__ __forceinline__ void apply(float w, float, float, float &o0, float &, float &, float &) const {
+        float fw = floorf(w);
+        float arg = (DERIV ? (w * s.d - s.d * fw) : (s.d * w - s.d * fw)) - s.h;
+        float x = __builtin_amdgcn_fmed3f(arg, -3.0f, 3.0f);
+        if constexpr (CAREFUL) x = (arg != arg) ? arg : x;
+        Rational r(x);
+        if constexpr (DERIV) {
+            o0 = cdiv(s.d * r.dsig(), s.c, s.rc);
+        } else {
+            float t = cdiv(r.sig(), s.c, s.rc);
+            o0 = (t + 0.5f) + fw;
+            if constexpr (CAREFUL) o0 = (arg != arg) ? arg : o0;
+        }
+    }
+};
+
+// SoftStep.sigmoid / dsigmoid / d2sigmoid on an arbitrary tensor (tmq/tmq.py:353-381).
+template <int WHICH>
+struct RationalOp {
+    TMQ_OP_FLAGS(false, true, false, false, false, false);
+    template <bool CAREFUL>
+    __device__ __forceinline__ void apply(float v, float, float, float &o0, float &, float &, float &) const {
+        float x = __builtin_amdgcn_fmed3f(v, -3.0f, 3.0f);
+        x = (v != v) ? v : x;
+        Rational r(x);
+        o0 = WHICH == 0 ? r.sig() : (WHICH == 1 ? r.dsig() : r.d2sig());
+    }
+};
+
 // Loss only: acc += dsig(arg). Used by the multi-tensor quantization loss.
 struct QLossOp {
     TMQ_OP_FLAGS(false, false, false, false, true, false);
@@ -208,6 +244,7 @@ struct Multi {
     const tmq_segment *segs;
     int nseg;
     int inplace;  // out0 = ptr (in-place ops); out1 = aux
+    const float *upstream;  // device scalar g: per-tensor scalar becomes g / float(n) (mean backward), or null
     __device__ __forceinline__ View locate(uint32_t b) const {
         int lo = 0, hi = nseg - 1;
         while (lo < hi) {
@@ -219,7 +256,8 @@ struct Multi {
         float *p = static_cast<float *>(s.ptr);
         float *a = static_cast<float *>(s.aux);
         bool vec = ((reinterpret_cast<uintptr_t>(p) | reinterpret_cast<uintptr_t>(a)) & 15u) == 0;
-        return View{p, nullptr, inplace ? p : nullptr, a, nullptr, s.n, b - s.block_begin, s.scalar, vec};
+        const float sc = upstream ? upstream[0] / (float)s.n : s.scalar;
+        return View{p, nullptr, inplace ? p : nullptr, a, nullptr, s.n, b - s.block_begin, sc, vec};
     }
 };
 
@@ -408,10 +446,10 @@ int launch_single(const Op &op, const float *in0, const float *in1, float *o0, f
 
 template <class Op>
 int launch_multi(const Op &op, const tmq_segment *segs, int nseg, uint32_t total_blocks, int inplace, float *partials,
-                 void *stream) {
+                 void *stream, const float *upstream = nullptr) {
     if (nseg < 0 || (nseg > 0 && !segs)) return TMQ_ERR_INVALID_ARG;
     if (nseg == 0 || total_blocks == 0) return TMQ_OK;
-    Multi loc{segs, nseg, inplace};
+    Multi loc{segs, nseg, inplace, upstream};
     hipLaunchKernelGGL((stream_kernel<Op, Multi>), dim3(total_blocks), dim3(kThreads), 0, as_stream(stream), loc, op,
                        partials);
     return check_launch();
@@ -454,6 +492,24 @@ int tmq_softstep_deriv_bwd(const float *w, const float *g, float *dw, size_t n, 
     if (bad_hardness(digamma)) return TMQ_ERR_INVALID_ARG;
     DerivBwdOp op{make_step(digamma, strength)};
     return launch_single(op, w, g, dw, nullptr, nullptr, n, nullptr, stream);
+}
+
+int tmq_softstep_map(const float *w, float *y, size_t n, double digamma, int derivative, void *stream) {
+    if (n && (!w || !y)) return TMQ_ERR_INVALID_ARG;
+    if (bad_hardness(digamma)) return TMQ_ERR_INVALID_ARG;
+    const StepK s = make_step(digamma, 0.0);
+    if (derivative) return launch_single(MapOp<true>{s}, w, nullptr, y, nullptr, nullptr, n, nullptr, stream);
+    return launch_single(MapOp<false>{s}, w, nullptr, y, nullptr, nullptr, n, nullptr, stream);
+}
+
+int tmq_sigmoid_piece(const float *x, float *y, size_t n, int order, void *stream) {
+    if (n && (!x || !y)) return TMQ_ERR_INVALID_ARG;
+    switch (order) {
+        case 0: return launch_single(RationalOp<0>{}, x, nullptr, y, nullptr, nullptr, n, nullptr, stream);
+        case 1: return launch_single(RationalOp<1>{}, x, nullptr, y, nullptr, nullptr, n, nullptr, stream);
+        case 2: return launch_single(RationalOp<2>{}, x, nullptr, y, nullptr, nullptr, n, nullptr, stream);
+        default: return TMQ_ERR_INVALID_ARG;
+    }
 }
 
 int tmq_clamp_inplace(float *w, size_t n, double lo, double hi, void *stream) {
@@ -547,11 +603,11 @@ int tmq_qloss_multi(const tmq_segment *segs, int nseg, uint32_t total_blocks, do
 }
 
 int tmq_qloss_bwd_multi(const tmq_segment *segs, int nseg, uint32_t total_blocks, double sharpness, double strength,
-                        int accumulate, void *stream) {
+                        const float *upstream, int accumulate, void *stream) {
     if (bad_hardness(sharpness)) return TMQ_ERR_INVALID_ARG;
     const StepK q = make_step(sharpness, strength);
-    if (accumulate) return launch_multi(QLossBwdOp<true>{q}, segs, nseg, total_blocks, 0, nullptr, stream);
-    return launch_multi(QLossBwdOp<false>{q}, segs, nseg, total_blocks, 0, nullptr, stream);
+    if (accumulate) return launch_multi(QLossBwdOp<true>{q}, segs, nseg, total_blocks, 0, nullptr, stream, upstream);
+    return launch_multi(QLossBwdOp<false>{q}, segs, nseg, total_blocks, 0, nullptr, stream, upstream);
 }
 
 int tmq_clamp_multi(const tmq_segment *segs, int nseg, uint32_t total_blocks, double lo, double hi, void *stream) {

@@ -183,12 +183,36 @@ def qloss_multi(table: SegmentTable, sharpness: float, strength: float):
     return per, tot
 
 
-def qloss_bwd_multi(table: SegmentTable, sharpness: float, strength: float, accumulate: bool):
-    """aux_l (=|+=) scalar_l * Q'(w_l) for every segment, one launch."""
+def qloss_bwd_multi(table: SegmentTable, sharpness: float, strength: float, accumulate: bool, upstream=None):
+    """aux_l (=|+=) s_l * Q'(w_l) for every segment, one launch; s_l = upstream / n_l when a device
+    scalar `upstream` (fp32, 1 element) is given, else the table's per-tensor scalar."""
+    if upstream is not None:
+        _capi.require_gpu(upstream, "upstream")
+        if upstream.dtype != torch.float32 or upstream.numel() != 1:
+            raise RuntimeError("qloss_bwd_multi: upstream must be one fp32 value")
     with torch.cuda.device(table.device):
         check(_lib().tmq_qloss_bwd_multi(ptr(table.table), table.nseg, table.total_blocks, float(sharpness),
-                                         float(strength), int(bool(accumulate)), stream_of(table.table)),
-              "qloss_bwd_multi")
+                                         float(strength), ptr(upstream), int(bool(accumulate)),
+                                         stream_of(table.table)), "qloss_bwd_multi")
+
+
+def softstep_map(weights: torch.Tensor, digamma: float, derivative: bool = False) -> torch.Tensor:
+    """SoftStep.map / SoftStep.dmap (tmq/tmq.py:328-350) on an fp32 GPU tensor."""
+    w = _f32_cuda(weights, "softstep_map")
+    out = torch.empty_like(w)
+    with torch.cuda.device(w.device):
+        check(_lib().tmq_softstep_map(ptr(w), ptr(out), w.numel(), float(digamma), int(bool(derivative)),
+                                      stream_of(w)), "softstep_map")
+    return out.view(weights.shape)
+
+
+def sigmoid_piece(x: torch.Tensor, order: int) -> torch.Tensor:
+    """SoftStep.sigmoid (order 0), dsigmoid (1), d2sigmoid (2) of an fp32 GPU tensor (tmq/tmq.py:353-381)."""
+    v = _f32_cuda(x, "sigmoid_piece")
+    out = torch.empty_like(v)
+    with torch.cuda.device(v.device):
+        check(_lib().tmq_sigmoid_piece(ptr(v), ptr(out), v.numel(), int(order), stream_of(v)), "sigmoid_piece")
+    return out.view(x.shape)
 
 
 def clamp_multi_(table: SegmentTable, lo: float, hi: float):

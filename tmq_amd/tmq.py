@@ -1,0 +1,822 @@
+"""TMQ's Python API on the MI355X-native kernels.
+
+Same public surface as the reference's tmq/tmq.py -- QuantMode, TensorType,
+QuantizationScheduleBuilder, QuantizationControl, SoftStep, SoftStepDerivative, TMQLayer, Linear,
+Conv2d, ConvTranspose2d, quantize_weights, quantize_model, compressed_state_dict,
+prepare_compressed_load, load_compressed_state_dict, expand_compact_layers -- with the same
+argument meaning and error behaviour, so user code switches by changing the import.
+
+What differs underneath:
+  * every tensor-valued computation of the hot path (soft staircase forward / backward,
+    quantization loss and its gradient, clamp, ternarisation, 2-bit packing, compact inference)
+    runs in libtmq_hip on the GPU; there is no CPU implementation of that math here, and weights
+    must live on the GPU (a clear error is raised otherwise);
+  * QuantizationControl.quantization_loss() and .clamp() are single multi-tensor launches over
+    all registered layers instead of per-layer Python loops, and clamp works in place;
+  * compact inference takes any batch shape and runs convolutions as implicit GEMM.
+Host-only logic (the hardness / penalty schedule, model surgery, state-dict metadata) is plain
+Python as in the reference.
+"""
+import fnmatch
+from enum import Enum
+
+import torch
+from torch import nn
+from torch.autograd.function import Function
+
+from . import ops
+from ._capi import load as _load_native
+
+# The reference exposes these two flags (tmq/tmq.py:28-46). Here the single native library is
+# mandatory: importing this module without it raises instead of degrading.
+_load_native()
+CUDA_EXT_AVAILABLE = True
+NATIVE_EXT_AVAILABLE = True
+
+
+class QuantMode(Enum):
+    """Quantization modes (tmq/tmq.py:49-63); only TERNARY is implemented, as in the reference."""
+    NONE = 0
+    TERNARY = 1
+    TWO_BIT = 2
+    THREE_BIT = 3
+    FOUR_BIT = 4
+    FIVE_BIT = 5
+    SIX_BIT = 6
+    EIGHT_BIT = 8
+
+
+class TensorType(Enum):
+    """Storage type of a TMQ layer's weight tensor (tmq/tmq.py:65-72)."""
+    FLOAT_32BIT = 0
+    FLOAT_16BIT = 1
+    COMPACT_TERNARY_32BIT = 2
+    COMPRESSED_TERNARY_32BIT = 3
+
+
+class QuantizationScheduleBuilder:
+    """tmq/tmq.py:75-82"""
+
+    @staticmethod
+    def default_schedule(max_epochs: int):
+        assert max_epochs >= 50, "Need at least 50 epochs for a default schedule"
+        return tuple(int(max_epochs * f) for f in (0.3, 0.8, 0.875, 0.93)) + (max_epochs,)
+
+
+def _require_gpu_weight(t, what):
+    if not t.is_cuda:
+        raise RuntimeError(f"tmq_amd: {what} needs its weights on the GPU (no CPU implementation is provided); "
+                           "move the model with .to('cuda') first")
+
+
+class QuantizationControl:
+    """Controller for quantization-aware training (tmq/tmq.py:85-310): owns the registry of TMQ
+    layers and the hardness (`digamma`) / penalty (`qpenalty`) schedule.
+
+    epoch_knots: (reach digamma 3, reach digamma max and start the penalty ramp, reach the maximum
+    penalty, stop cycling, total epochs)."""
+
+    _WARMUP = 7          # tmq/tmq.py:117
+    _CYCLE = 15          # tmq/tmq.py:141
+
+    def __init__(self, epoch_knots=None, digamma_range=(0.1, 6), qpenalty_range=None, quant_mode=QuantMode.TERNARY,
+                 post_scale=False, init_range=None, device="cpu"):
+        assert epoch_knots is None or len(epoch_knots) == 5
+        assert len(digamma_range) == 2, "Need to supply a start/end value for the digamma parameter of the softstep function"
+        assert digamma_range[0] >= 0.05, "Initial digamma value must be >= 0.05"
+        assert digamma_range[0] <= 1, "Initial digamma value must be <= 1"
+        assert digamma_range[1] <= 20.0, "Final digamma value must be <= 20"
+        assert digamma_range[1] >= 3, "Final digamma value must be >= 3"
+        assert digamma_range[0] <= digamma_range[1], "Please supply a valid range for digamma"
+        self._warmup_epochs = self._WARMUP
+        if epoch_knots is not None:
+            assert epoch_knots[0] >= self._warmup_epochs + 5, \
+                "At least %d epochs required to reach halfway point" % (self._warmup_epochs + 5)
+            self.max_epochs = epoch_knots[4]
+        else:
+            self.max_epochs = 0
+        self.quantization = quant_mode
+        self.epoch_knots = epoch_knots
+        self.post_scale = post_scale
+        self.digamma_start = max(0.05, digamma_range[0])
+        self.digamma_end = max(3, digamma_range[1])
+        self.digamma = self.digamma_start
+        self.qpenalty = qpenalty_range[0] if qpenalty_range is not None else 0
+        self.qpenalty_sharpness = 5.0
+        self.inference_mode = self.max_epochs == 0
+        self.device = device
+        self._registry = {}
+        self._last_cycle = -1
+        self._digamma_cycle_start = 0
+        self._digamma_cycle_end = 0
+        self._cycle_len = self._CYCLE
+        if quant_mode == QuantMode.TERNARY:
+            self.clamp_values = (-1., 1.)
+        else:
+            bits = int(quant_mode.value)
+            self.clamp_values = (-2 ** bits, (2 ** bits) - 1)
+        self.init_range = init_range if init_range is not None else self.clamp_values
+        if qpenalty_range is not None:
+            assert len(qpenalty_range) == 2, "Quantization penalty needs to supply a range"
+            self.qpenalty_range = qpenalty_range
+        else:
+            self.qpenalty_range = (0, 0)
+        self._table = None            # cached multi-tensor segment table (weights, grads)
+
+    # ---- schedule (host scalars only) -----------------------------------------------------------
+    @staticmethod
+    def _mix(lo_epoch, hi_epoch, epoch, start, end):
+        t = min(1, max(0, (epoch - lo_epoch) / (hi_epoch - lo_epoch)))
+        return t * end + (1 - t) * start
+
+    def _segment(self, epoch):
+        """Index of the knot interval an epoch falls into (0..4), tmq/tmq.py:176-181."""
+        kn = self.epoch_knots
+        if epoch >= kn[3]:
+            return 4
+        if epoch < kn[0]:
+            return 0
+        if epoch < kn[1]:
+            return 1
+        return 2 if epoch < kn[2] else 3
+
+    def _ramp(self, seg, epoch):
+        """The un-cycled hardness ramp: start -> 3 over [warm-up, knot 0], 3 -> end over
+        [knot 0, knot 1], end afterwards (tmq/tmq.py:183-190)."""
+        if seg >= 2:
+            return self.digamma_end
+        if seg == 0:
+            return self._mix(self._warmup_epochs, self.epoch_knots[0], epoch, self.digamma_start, 3.0)
+        return self._mix(self.epoch_knots[0], self.epoch_knots[1], epoch, 3.0, self.digamma_end)
+
+    def step(self, epoch):
+        """Advance the schedule; call once before every epoch, in order (the saw-tooth keeps state).
+
+        Behaviour of tmq/tmq.py:160-240: nothing changes through the warm-up; from knot 3 on the
+        hardness and the penalty sit at their final values; in between the hardness follows the
+        ramp, except that every 15 epochs it restarts at 0.45 x the ramp (never below the start
+        value) and climbs linearly to the ramp value 15 epochs ahead. The penalty ramps linearly
+        between knots 2 and 3."""
+        if self.epoch_knots is None:
+            return
+        if epoch >= self.epoch_knots[3]:
+            self.qpenalty = self.qpenalty_range[1]
+            self.digamma = self.digamma_end
+            return
+        if epoch <= self._warmup_epochs:
+            return
+        seg = self._segment(epoch)
+        first_window = self._warmup_epochs + self._cycle_len
+        in_cycle = self._last_cycle != -1
+        if seg < 4 or in_cycle:
+            ramp_now = self._ramp(seg, epoch)
+            may_restart = not in_cycle and seg < 4 and (seg != 0 or epoch >= first_window)
+            if may_restart:
+                ahead = self._segment(epoch + self._cycle_len)
+                if ahead < 4:
+                    self._digamma_cycle_start = max(self.digamma_start, ramp_now * 0.45)
+                    self._digamma_cycle_end = self._ramp(ahead, epoch + self._cycle_len)
+                    self._last_cycle = epoch
+                    self.digamma = self._digamma_cycle_start
+            elif epoch < first_window:
+                self.digamma = ramp_now
+            elif epoch <= self._last_cycle + self._cycle_len:
+                self.digamma = self._mix(self._last_cycle, self._last_cycle + self._cycle_len, epoch,
+                                         self._digamma_cycle_start, self._digamma_cycle_end)
+            else:
+                self._last_cycle = -1
+        else:
+            self.digamma = self._ramp(seg, epoch)
+        if seg >= 2:
+            self.qpenalty = self._mix(self.epoch_knots[2], self.epoch_knots[3], epoch, self.qpenalty_range[0],
+                                      self.qpenalty_range[1])
+
+    # ---- registry -----------------------------------------------------------------------------------
+    def inference(self):
+        """Run all TMQ layers in inference mode (tmq/tmq.py:243-249)."""
+        self.inference_mode = True
+
+    def register_node(self, name, node):
+        self._registry[name] = node
+        self._table = None
+
+    def collect_grad_norms(self):
+        return {name: node.weight.grad.norm() for name, node in self._registry.items()
+                if node.weight.grad is not None}
+
+    def _weights(self):
+        return [node.weight for node in self._registry.values()]
+
+    def _segment_table(self):
+        """Multi-tensor table over (weight, scratch gradient) of every registered layer; rebuilt
+        whenever a weight tensor has been reallocated."""
+        ws = [w.data for w in self._weights()]
+        for w in ws:
+            _require_gpu_weight(w, "QuantizationControl")
+            if w.dtype != torch.float32:
+                raise ValueError("Expected either a float16 or a float32 tensor as input/output")
+        key = tuple((w.data_ptr(), w.numel()) for w in ws)
+        if self._table is None or self._table[0] != key:
+            ws = [w if w.is_contiguous() else w.contiguous() for w in ws]
+            flat = torch.empty(sum(w.numel() for w in ws), dtype=torch.float32, device=ws[0].device)
+            grads, off = [], 0
+            for w in ws:
+                grads.append(flat[off:off + w.numel()])
+                off += w.numel()
+            self._table = (key, ops.SegmentTable(ws, aux=grads), grads, ws)
+        return self._table
+
+    # ---- tensor work: one launch for all layers ------------------------------------------------------
+    def clamp(self, slack=0):
+        """Clamp the weights of all registered layers into the quantization range (+- slack), in
+        place, in one launch (tmq/tmq.py:263-272 with 691-696 / 874-879)."""
+        if not self._registry:
+            return
+        lo, hi = self.clamp_values[0] - slack, self.clamp_values[1] + slack
+        _, table, _, _ = self._segment_table()
+        ops.clamp_multi_(table, lo, hi)
+
+    def quantize(self):
+        """Hard-quantize every registered layer: w <- round(SoftStep.map(w)) (tmq/tmq.py:284-295)."""
+        for node in self._registry.values():
+            w = node.weight.data
+            _require_gpu_weight(w, "QuantizationControl.quantize")
+            node.weight.data = ops.ternarize_(w.contiguous().clone(), self.digamma)
+
+    def quantization_loss(self, penalty=None):
+        """Sum over layers of mean(SoftStepDerivative(w, sharpness, p)) (tmq/tmq.py:298-310); one
+        multi-tensor launch forward, one backward. Returns None when no layer is registered."""
+        if not self._registry:
+            return None
+        p = penalty if penalty is not None else self.qpenalty
+        return _QuantizationLossAll.apply(self, float(p), float(self.qpenalty_sharpness), *self._weights())
+
+
+class _QuantizationLossAll(Function):
+    """total = sum_l mean_i q(w_l[i]); d total / d w_l = (g / n_l) * Q'(w_l) (tmq/tmq.py:456-493,
+    698-699) for every registered layer at once."""
+
+    @staticmethod
+    def forward(ctx, ctrl, strength, sharpness, *weights):
+        _, table, _, _ = ctrl._segment_table()
+        ctx.ctrl, ctx.strength, ctx.sharpness = ctrl, strength, sharpness
+        _, total = ops.qloss_multi(table, sharpness, strength)
+        return total.reshape(())
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        key, table, grads, ws = ctx.ctrl._segment_table()
+        g = grad_output.detach().to(torch.float32).reshape(1).contiguous()
+        ops.qloss_bwd_multi(table, ctx.sharpness, ctx.strength, accumulate=False, upstream=g)
+        out = tuple(gr.view(w.shape).clone() for gr, w in zip(grads, ws))
+        return (None, None, None) + out
+
+
+class SoftStep(Function):
+    """The differentiable staircase (tmq/tmq.py:315-438): y = sig(d frac(w) - d/2) / (2 sig(d/2)) +
+    1/2 + floor(w), sig a clamped cubic-over-quadratic. Forward and backward are single HIP kernels
+    with the fp32 arithmetic of the reference's CPU op chain."""
+
+    @staticmethod
+    @torch.no_grad()
+    def map(weight: torch.Tensor, ctrl: QuantizationControl) -> torch.Tensor:
+        """Soft-quantized image of a tensor, for logging and final ternarisation (tmq/tmq.py:328-338)."""
+        assert ctrl, "Control instance is required"
+        _require_gpu_weight(weight, "SoftStep.map")
+        return ops.softstep_map(weight.data, ctrl.digamma, derivative=False)
+
+    @staticmethod
+    @torch.no_grad()
+    def dmap(weight: torch.Tensor, ctrl: QuantizationControl) -> torch.Tensor:
+        """Slope of the staircase at a tensor (tmq/tmq.py:341-350)."""
+        assert ctrl, "Control instance is required"
+        _require_gpu_weight(weight, "SoftStep.dmap")
+        return ops.softstep_map(weight.data, ctrl.digamma, derivative=True)
+
+    @staticmethod
+    def sigmoid(input: torch.Tensor) -> torch.Tensor:
+        """tmq/tmq.py:353-360"""
+        _require_gpu_weight(input, "SoftStep.sigmoid")
+        return ops.sigmoid_piece(input, 0)
+
+    @staticmethod
+    def dsigmoid(input: torch.Tensor) -> torch.Tensor:
+        """tmq/tmq.py:363-370"""
+        _require_gpu_weight(input, "SoftStep.dsigmoid")
+        return ops.sigmoid_piece(input, 1)
+
+    @staticmethod
+    def d2sigmoid(input: torch.Tensor) -> torch.Tensor:
+        """tmq/tmq.py:373-381"""
+        _require_gpu_weight(input, "SoftStep.d2sigmoid")
+        return ops.sigmoid_piece(input, 2)
+
+    @staticmethod
+    def scalar_sigmoid(input: float) -> float:
+        """tmq/tmq.py:384-391"""
+        x = min(3.0, max(-3.0, input))
+        return x * (x * x + 27.0) / (27.0 + x * x * 9.0)
+
+    @staticmethod
+    def scalar_dsigmoid(input: float) -> float:
+        """tmq/tmq.py:394-401"""
+        x = min(3.0, max(-3.0, input))
+        x2 = x * x
+        return ((x2 - 9) * (x2 - 9)) / (9 * (3 + x2) * (3 + x2))
+
+    @staticmethod
+    def forward(ctx, weight, scale: float, ctrl: QuantizationControl):
+        _require_gpu_weight(weight, "SoftStep")
+        ctx.ctrl = ctrl
+        ctx.scale = scale            # only scales the gradient (tmq/tmq.py:412)
+        ctx.save_for_backward(weight)
+        return ops.fwd_softstep(weight.data, ctrl.digamma)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        weight = ctx.saved_tensors[0]
+        return ops.bwd_softstep(weight.data, ctx.ctrl.digamma, ctx.scale, grad_output), None, None
+
+
+class SoftStepDerivative(Function):
+    """First derivative of the staircase as an autograd function -- the quantization-loss
+    integrand (tmq/tmq.py:441-493)."""
+
+    @staticmethod
+    def forward(ctx, weight, digamma, strength):
+        _require_gpu_weight(weight, "SoftStepDerivative")
+        ctx.save_for_backward(weight)
+        ctx.digamma = digamma
+        ctx.strength = strength
+        return ops.fwd_softstep_derivative(weight.data, digamma, strength)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        weight = ctx.saved_tensors[0]
+        return ops.bwd_softstep_derivative(weight.data, ctx.digamma, ctx.strength, grad_output), None, None
+
+
+class TMQLayer:
+    """Bookkeeping shared by the quantization-aware layers (tmq/tmq.py:496-570)."""
+
+    _VARIANCE = {QuantMode.TERNARY: 2.0 / 3.0, QuantMode.TWO_BIT: (2 * 2 * 2 + 2 + 1) / 6.0,
+                 QuantMode.THREE_BIT: (2 * 4 * 4 + 4 + 1) / 6.0, QuantMode.FOUR_BIT: (2 * 8 * 8 + 8 + 1) / 6.0,
+                 QuantMode.FIVE_BIT: (2 * 16 * 16 + 16 + 1) / 6.0, QuantMode.SIX_BIT: (2 * 32 * 32 + 32 + 1) / 6.0,
+                 QuantMode.EIGHT_BIT: (2 * 128 * 128 + 128 + 1) / 6.0}
+
+    def __init__(self, ctrl=None, quant_mode=QuantMode.NONE, tensor_type=TensorType.FLOAT_32BIT, device=None):
+        self._ctrl = ctrl
+        self.quantization = quant_mode
+        self.tensor_type = tensor_type
+        self._device = device
+        self.compact = False
+        self.original_shape = None
+        self.post_scale_imm = 1.0
+        self.post_scale = None
+        self.layer_name = None
+        self._scale_dirty = True
+        self._native = None          # cached kernel-native weights for compact inference
+        self._scale_vec = None
+
+    def compact_inference_mode(self):
+        self.training = False
+        self.compact = True
+
+    def quantization_loss(self, strength, sharpness):
+        """mean(SoftStepDerivative(w, sharpness, strength)) (tmq/tmq.py:698-699, 889-891)."""
+        return torch.mean(SoftStepDerivative.apply(self.weight, sharpness, strength))
+
+    def quantize(self):
+        """Round the fp32 weights to the nearest integers, half to even (tmq/tmq.py:599-603, 882-886)."""
+        _require_gpu_weight(self.weight.data, "quantize")
+        self.weight.data = ops.ternarize_(self.weight.data.contiguous().clone())
+
+    @torch.no_grad()
+    def clamp(self, limits=(-1., 1.)):
+        """Clamp the weights (not the bias) in place (tmq/tmq.py:691-696, 874-879)."""
+        _require_gpu_weight(self.weight.data, "clamp")
+        if not self.weight.data.is_contiguous():
+            self.weight.data = self.weight.data.contiguous()
+        ops.clamp_(self.weight.data, limits[0], limits[1])
+
+    def _update_scale(self):
+        if self._scale_dirty and self.post_scale is not None:
+            self.post_scale_imm = self.post_scale.item()
+            self._scale_dirty = False
+
+    def _variance_estimate(self) -> float:
+        """Output variance of a unit-variance input under the layer's quantization levels
+        (tmq/tmq.py:550-570)."""
+        return self._VARIANCE.get(self.quantization, 1.0)
+
+    def _soft_weight(self):
+        use = self._ctrl is not None and not self._ctrl.inference_mode
+        return SoftStep.apply(self.weight, 1.0, self._ctrl) if use else self.weight
+
+    def _native_weights(self, conv_kernel=None):
+        w = self.weight.data
+        key = (w.data_ptr(), tuple(w.shape), w._version)
+        if self._native is None or self._native[0] != key:
+            self._native = (key, ops.NativeWeights(w, self.original_shape[0], conv_kernel))
+        return self._native[1]
+
+    def _epilogue_scale(self, n, device):
+        """Per-channel scale vector carrying the scalar post-scale (None when it is 1)."""
+        if self.post_scale_imm == 1.0:
+            return None
+        if self._scale_vec is None or self._scale_vec[0] != (self.post_scale_imm, n, device):
+            self._scale_vec = ((self.post_scale_imm, n, device),
+                               torch.full((n,), self.post_scale_imm, dtype=torch.float32, device=device))
+        return self._scale_vec[1]
+
+    def _adopt_stored_weight(self, state_dict, prefix, local_metadata):
+        """Shared tail of _load_from_state_dict (tmq/tmq.py:748-765, 956-973): interpret the
+        tmq.* metadata written by compressed_state_dict."""
+        if "tmq.quant" in local_metadata and "tmq.tensor_type" in local_metadata:
+            self.tensor_type = TensorType(local_metadata["tmq.tensor_type"])
+            self.original_shape = local_metadata["tmq.shape"]
+            if self.tensor_type == TensorType.COMPRESSED_TERNARY_32BIT:
+                stored = state_dict[prefix + "weight"]
+                dev = self.weight.device
+                self.weight = nn.Parameter(ops.decompress_ternary(stored.cpu(), self.original_shape).to(dev),
+                                           requires_grad=False)
+                self.tensor_type = TensorType.COMPACT_TERNARY_32BIT
+                self.compact = True
+            elif self.tensor_type == TensorType.COMPACT_TERNARY_32BIT:
+                self.weight = nn.Parameter(state_dict[prefix + "weight"].to(self.weight.device), requires_grad=False)
+                self.compact = True
+            else:
+                self.compact = False
+            self.quantization = QuantMode(local_metadata["tmq.quant"])
+            self.training = False if self.compact else self.training
+            self._native = None
+        else:
+            self.compact = False
+
+
+def _uniform_init(*shape):
+    # U(-1, 1) drawn exactly like the reference (one torch.rand call on the CPU generator), so
+    # seeded runs start from the same weights (tmq/tmq.py:723-725, 919-927).
+    return 2.0 * (torch.rand(*shape) - 0.5)
+
+
+class Linear(nn.Module, TMQLayer):
+    """Quantization-aware drop-in for nn.Linear (tmq/tmq.py:573-765)."""
+
+    def __init__(self, in_features: int, out_features: int, bias: bool = True, device=None,
+                 ctrl: QuantizationControl = None, quant_mode=QuantMode.NONE, post_scale=False):
+        nn.Module.__init__(self)
+        TMQLayer.__init__(self, ctrl, quant_mode, TensorType.FLOAT_32BIT, device)
+        self.weight = nn.Parameter()
+        self._in_features = in_features
+        self._out_features = out_features
+        self._init_weights(bias, device)
+        self.original_shape = self.weight.shape
+        self.post_scale_imm = 1.0 / (self._in_features * self._variance_estimate()) if post_scale else 1.0
+        self.post_scale = nn.Parameter(torch.tensor(self.post_scale_imm), requires_grad=False)
+        self.bn = None
+
+    def __repr__(self):
+        if len(self.original_shape) == 2:
+            return "Linear(%d,%d) [tmq]" % tuple(self.original_shape) + " <%s>" % self.layer_name
+        return "Linear(???) [tmq] <%s>" % self.layer_name
+
+    def disable_bias(self):
+        self.bias = None
+
+    def implicit_bn(self):
+        """Attach an internal BatchNorm1d that rescales the layer output (tmq/tmq.py:611-622)."""
+        self.bn = nn.BatchNorm1d(self._out_features)
+
+    def forward(self, x):
+        """Training / fp32 path: F.linear on the soft-quantized weights; compact path when packed
+        weights are loaded (tmq/tmq.py:637-659; the reference's debug dump of 624-635 is not kept)."""
+        if self.compact:
+            return self.compact_forward(x)
+        assert self._ctrl or not self.training, "Quantization controller required for training"
+        self._update_scale()
+        w = self._soft_weight()
+        if self.post_scale != 1.0:
+            out = self.post_scale * nn.functional.linear(x, w, None)
+            final = self.bias + out if self.bias is not None else out
+        else:
+            final = nn.functional.linear(x, w, self.bias)
+        return self.bn(final) if self.bn is not None else final
+
+    forward_wrap = forward
+
+    @torch.no_grad()
+    def compact_forward(self, x):
+        """Inference straight from the 2-bit packed weights (tmq/tmq.py:662-688), any batch shape."""
+        assert self.training == False, "Compact inference is not supported in training mode"
+        assert self.weight.data.dtype == torch.int32, "Compact inference requires 32-bit integer words"
+        self._update_scale()
+        if x.dim() == 4:
+            assert x.shape[1] == 1, "Illegal shape supplied"
+        nw = self._native_weights()
+        xin = x if x.is_contiguous() else x.contiguous()
+        out = ops.ternary_linear(xin, nw, scale=self._epilogue_scale(nw.N, x.device),
+                                 bias=self.bias.data.float() if self.bias is not None else None)
+        return self.bn(out) if self.bn is not None else out
+
+    @classmethod
+    def from_linear(cls, source: nn.Linear, name: str, ctrl: QuantizationControl):
+        assert ctrl, "Control instance is required"
+        obj = cls(source.in_features, source.out_features, source.bias is not None, ctrl=ctrl,
+                  device=source.weight.device, quant_mode=ctrl.quantization, post_scale=ctrl.post_scale)
+        obj.layer_name = name
+        ctrl.register_node(name, obj)
+        return obj
+
+    @torch.no_grad()
+    def _init_weights(self, bias, device):
+        if bias:
+            self.bias = nn.Parameter(torch.zeros(self._out_features).to(device), requires_grad=True)
+        else:
+            self.bias = None
+        self.weight = nn.Parameter(_uniform_init(self._out_features, self._in_features).to(device),
+                                   requires_grad=True)
+
+    def _load_from_state_dict(self, state_dict, prefix, local_metadata, strict, missing_keys, unexpected_keys,
+                              error_msgs):
+        super()._load_from_state_dict(state_dict, prefix, local_metadata, strict, missing_keys, unexpected_keys,
+                                      error_msgs)
+        self._adopt_stored_weight(state_dict, prefix, local_metadata)
+
+
+def _pair(v):
+    return tuple(v) if isinstance(v, (tuple, list)) else (v, v)
+
+
+class Conv2d(nn.Module, TMQLayer):
+    """Quantization-aware drop-in for nn.Conv2d (tmq/tmq.py:769-973)."""
+
+    _transposed = False
+
+    def __init__(self, in_channels, out_channels, kernel, stride=1, padding=0, groups=1, dilation=1, bias=True,
+                 device=None, ctrl=None, quant_mode=QuantMode.NONE, post_scale=False):
+        nn.Module.__init__(self)
+        TMQLayer.__init__(self, ctrl, quant_mode, TensorType.FLOAT_32BIT, device)
+        self.in_channels = in_channels
+        self.out_channels = out_channels
+        self.kernel = kernel
+        self.stride = stride
+        self.padding = padding
+        self.groups = groups
+        self.dilation = dilation
+        self._init_weights(bias, device)
+        self.original_shape = self.weight.shape
+        self.post_scale_imm = 1.0 / (self._fan_in * self._variance_estimate()) if post_scale else 1.0
+        self.post_scale = nn.Parameter(torch.tensor(self.post_scale_imm), requires_grad=False)
+
+    def __repr__(self):
+        return "Conv2d(%d,%d,%d,%d) [tmq]" % tuple(self.original_shape) + " <%s>" % self.layer_name
+
+    def to(self, *args, **kwargs):
+        me = super().to(*args, **kwargs)
+        me.post_scale_imm = me.post_scale.item()
+        return me
+
+    def _conv(self, x, w, bias):
+        return nn.functional.conv2d(x, w, bias, self.stride, self.padding, dilation=self.dilation, groups=self.groups)
+
+    def forward(self, x):
+        """tmq/tmq.py:805-819"""
+        if self.compact:
+            return self.compact_forward(x)
+        assert self._ctrl or not self.training, "Quantization controller required for training"
+        self._update_scale()
+        w = self._soft_weight()
+        if self.post_scale != 1.0:
+            out = self.post_scale * self._conv(x, w, None)
+            return self.bias + out if self.bias is not None else out
+        return self._conv(x, w, self.bias)
+
+    @torch.no_grad()
+    def compact_forward(self, x):
+        """Implicit-GEMM convolution from the packed weights (replaces the unfold / GEMM / fold
+        sequence of tmq/tmq.py:822-871). Output extents follow PyTorch's formula. Returns fp32
+        [B, N, Ho, Wo] (channels_last memory); a 3-D input gives a 3-D output."""
+        assert not self.training, "Compact inference is not supported in training mode"
+        assert self.weight.data.dtype == torch.int32, "Compact inference requires 32-bit integer words"
+        self._update_scale()
+        if x.dim() == 3:
+            return self.compact_forward(x.unsqueeze(0)).squeeze(0)
+        if x.dim() != 4:
+            raise Exception("Expected a 3D tensor")
+        assert self.groups == 1 or self.groups == self.original_shape[0], \
+            "Grouped convolutions are only supported for group == channels"
+        if self.groups != 1:
+            raise NotImplementedError("depthwise compact inference is not part of this build")
+        ky, kx = _pair(self.kernel)
+        nw = self._native_weights(conv_kernel=(ky, kx))
+        bias = self.bias.data.float() if self.bias is not None else None
+        return ops.ternary_conv2d(x, nw, _pair(self.stride), _pair(self.padding), _pair(self.dilation),
+                                  scale=self._epilogue_scale(nw.N, x.device), bias=bias)
+
+    @classmethod
+    def from_conv2d(cls, source: nn.Conv2d, name: str, ctrl: QuantizationControl):
+        assert ctrl, "Controller required"
+        obj = cls(source.in_channels, source.out_channels, source.kernel_size, stride=source.stride,
+                  padding=source.padding, groups=source.groups, dilation=source.dilation,
+                  bias=source.bias is not None, device=source.weight.device, ctrl=ctrl,
+                  quant_mode=ctrl.quantization, post_scale=ctrl.post_scale)
+        obj.layer_name = name
+        ctrl.register_node(name, obj)
+        return obj
+
+    def _weight_shape(self, ky, kx):
+        return [self.out_channels, self.in_channels // self.groups, ky, kx]
+
+    @torch.no_grad()
+    def _init_weights(self, bias, device):
+        ky, kx = _pair(self.kernel)
+        self._fan_in = ky * kx * self.in_channels
+        self._fan_out = ky * kx * self.out_channels
+        self.weight = nn.Parameter(_uniform_init(self._weight_shape(ky, kx)).to(device), requires_grad=True)
+        if bias:
+            self.bias = nn.Parameter(torch.zeros(self.out_channels).to(device), requires_grad=True)
+        else:
+            self.bias = None
+
+    def _load_from_state_dict(self, state_dict, prefix, local_metadata, strict, missing_keys, unexpected_keys,
+                              error_msgs):
+        super()._load_from_state_dict(state_dict, prefix, local_metadata, strict, missing_keys, unexpected_keys,
+                                      error_msgs)
+        self._adopt_stored_weight(state_dict, prefix, local_metadata)
+
+
+class ConvTranspose2d(Conv2d):
+    """Quantization-aware drop-in for nn.ConvTranspose2d (tmq/tmq.py:978-1087). Training path only:
+    the reference's compact path for this layer cannot pass its own shape checks, and no compact
+    kernel is provided here."""
+
+    _transposed = True
+
+    def __init__(self, in_channels, out_channels, kernel, stride=1, padding=0, output_padding=0, groups=1, bias=True,
+                 dilation=1, device=None, ctrl=None, quant_mode=QuantMode.NONE, post_scale=False):
+        super().__init__(in_channels, out_channels, kernel, stride, padding, groups, dilation, bias, device, ctrl,
+                         quant_mode, post_scale)
+        self.output_padding = output_padding
+
+    def __repr__(self):
+        return "ConvTranspose2d(%d,%d,%d,%d) [tmq] " % tuple(self.original_shape) + " <%s>" % self.layer_name
+
+    def _conv(self, x, w, bias):
+        return nn.functional.conv_transpose2d(x, w, bias, self.stride, self.padding, dilation=self.dilation,
+                                              groups=self.groups)
+
+    def _weight_shape(self, ky, kx):
+        return [self.in_channels, self.out_channels // self.groups, ky, kx]
+
+    @torch.no_grad()
+    def compact_forward(self, x):
+        raise NotImplementedError("compact inference for ConvTranspose2d is not part of this build")
+
+    @classmethod
+    def from_transconv2d(cls, source: nn.ConvTranspose2d, name: str, ctrl: QuantizationControl):
+        assert ctrl, "Controller required"
+        obj = cls(source.in_channels, source.out_channels, source.kernel_size, stride=source.stride,
+                  padding=source.padding, output_padding=source.output_padding, groups=source.groups,
+                  dilation=source.dilation, bias=source.bias is not None, device=ctrl.device, ctrl=ctrl,
+                  quant_mode=ctrl.quantization, post_scale=ctrl.post_scale)
+        obj.layer_name = name
+        ctrl.register_node(name, obj)
+        return obj
+
+
+# ---- model / state utilities (tmq/tmq.py:1090-1319) -------------------------------------------------------
+def _tmq_layers(module: nn.Module, prefix=""):
+    """(qualified name, parent, child name, layer) for every TMQ layer below `module`, depth first
+    in registration order; does not descend into TMQ layers."""
+    for name, sub in module.named_children():
+        full = prefix + "." + name if prefix != "" else name
+        if isinstance(sub, TMQLayer):
+            yield full, module, name, sub
+        else:
+            yield from _tmq_layers(sub, full)
+
+
+def quantize_weights(module: nn.Module):
+    """Snap the fp32 weights of every TMQ layer to integers in place (tmq/tmq.py:1090-1111)."""
+    for name, sub in module.named_children():
+        if isinstance(sub, TMQLayer):
+            if sub.weight.data.dtype == torch.float16:
+                raise Exception("FP16 data is currently not supported")
+            if sub.weight.data.dtype == torch.float32:
+                _require_gpu_weight(sub.weight.data, "quantize_weights")
+                rounded = ops.ternarize_(sub.weight.data.contiguous().clone())
+                sub.weight = nn.Parameter(rounded, requires_grad=sub.weight.requires_grad)
+        quantize_weights(sub)
+
+
+def quantize_model(module: nn.Module, ctrl: QuantizationControl, prefix="", exclude=[]):
+    """Swap nn.Linear / nn.Conv2d / nn.ConvTranspose2d for their quantization-aware versions in
+    place (tmq/tmq.py:1114-1180). `exclude` holds qualified names or '*' wildcards. The original
+    parameters are discarded and re-initialised U(-1, 1)."""
+    assert ctrl, "Must supply a quantization control instance"
+    exact = [p for p in exclude if "*" not in p]
+    globs = [p for p in exclude if "*" in p]
+    _swap_layers(module, ctrl, prefix, exact, globs)
+
+
+_FACTORIES = ((nn.Linear, lambda s, n, c: Linear.from_linear(s, n, c)),
+              (nn.Conv2d, lambda s, n, c: Conv2d.from_conv2d(s, n, c)),
+              (nn.ConvTranspose2d, lambda s, n, c: ConvTranspose2d.from_transconv2d(s, n, c)))
+
+
+def _swap_layers(module, ctrl, prefix, exact, globs):
+    for name, sub in module.named_children():
+        if sub is module:
+            continue
+        path = prefix + "." + name if prefix != "" else name
+        if path in exact:
+            print("Skipping excluded layer %s" % path)
+            continue                                   # an exactly excluded module is not descended into
+        if any(fnmatch.fnmatch(path, g) for g in globs):
+            print("Skipping excluded layer %s" % path)
+        else:
+            for kind, make in _FACTORIES:
+                if isinstance(sub, kind):
+                    # registered under prefix + "." + name: a leading dot for an empty prefix, as in
+                    # the reference (tmq/tmq.py:1171)
+                    sub = make(sub, prefix + "." + name, ctrl)
+                    setattr(module, name, sub)
+        _swap_layers(sub, ctrl, path, exact, globs)
+
+
+def compressed_state_dict(module: nn.Module, strong=False, remove_prefix=""):
+    """State dict with TMQ weights bit-stuffed (2 bit / weight) or, with strong=True, range coded;
+    the layers are switched to compact inference as a side effect (tmq/tmq.py:1183-1248)."""
+    for _, _, _, layer in _tmq_layers(module):
+        if not hasattr(layer, "tensor_type"):
+            continue
+        if getattr(layer, "original_shape", None) is None:
+            layer.original_shape = layer.weight.shape
+        if not strong and layer.tensor_type != TensorType.COMPACT_TERNARY_32BIT:
+            layer.weight = nn.Parameter(ops.compactify_ternary(layer.weight.data), requires_grad=False)
+            layer.tensor_type = TensorType.COMPACT_TERNARY_32BIT
+        elif strong and layer.tensor_type != TensorType.COMPRESSED_TERNARY_32BIT:
+            from_compact = layer.tensor_type == TensorType.COMPACT_TERNARY_32BIT
+            stream = ops.compress_ternary(layer.weight.data, layer.original_shape, from_compact)
+            layer._stream_device = layer.weight.device
+            layer.weight = nn.Parameter(stream, requires_grad=False)
+            layer.tensor_type = TensorType.COMPRESSED_TERNARY_32BIT
+        layer._native = None
+    state = module.state_dict()
+    for full, _, _, layer in _tmq_layers(module):
+        layer.compact_inference_mode()
+        meta = state._metadata[full]
+        meta["tmq.tensor_type"] = layer.tensor_type.value
+        meta["tmq.shape"] = layer.original_shape
+        meta["tmq.quant"] = layer.quantization.value
+        if layer.tensor_type == TensorType.COMPRESSED_TERNARY_32BIT:
+            # keep the model usable right away: back to the compact form in memory
+            dev = getattr(layer, "_stream_device", layer.weight.device)
+            layer.weight = nn.Parameter(ops.decompress_ternary(layer.weight.data.cpu(), layer.original_shape).to(dev),
+                                        requires_grad=False)
+            layer.tensor_type = TensorType.COMPACT_TERNARY_32BIT
+    return state
+
+
+def prepare_compressed_load(module: nn.Module, state_dict):
+    """tmq/tmq.py:1251-1252"""
+    _presize_weights(module, state_dict, "")
+
+
+def load_compressed_state_dict(module: nn.Module, state_dict):
+    """Load a compact / compressed state dict; entropy-coded weights end up in the compact form
+    in memory (tmq/tmq.py:1256-1268)."""
+    _presize_weights(module, state_dict)
+    module.load_state_dict(state_dict, strict=False)
+
+
+def _presize_weights(module: nn.Module, state_dict, prefix=""):
+    """Give every TMQ layer an empty weight of the stored shape and dtype so that load_state_dict
+    accepts the packed tensors (tmq/tmq.py:1271-1293)."""
+    meta = state_dict._metadata
+    for full, _, _, layer in _tmq_layers(module, prefix):
+        layer.layer_name = full
+        if full not in meta or "tmq.tensor_type" not in meta[full]:
+            continue
+        kind = TensorType(meta[full]["tmq.tensor_type"])
+        if kind in (TensorType.COMPACT_TERNARY_32BIT, TensorType.COMPRESSED_TERNARY_32BIT):
+            stored = state_dict[full + ".weight"]
+            layer.weight = nn.Parameter(torch.empty(stored.shape, dtype=stored.dtype, device=layer.weight.device),
+                                        requires_grad=False)
+        else:
+            layer.compact = False
+
+
+def expand_compact_layers(module: nn.Module, for_training=False):
+    """Expand compact TMQ layers back to fp32 weights in place (tmq/tmq.py:1296-1319)."""
+    for name, sub in module.named_children():
+        if isinstance(sub, TMQLayer) and hasattr(sub, "tensor_type") and getattr(sub, "original_shape", None) is not None:
+            if sub.tensor_type in (TensorType.COMPRESSED_TERNARY_32BIT, TensorType.COMPACT_TERNARY_32BIT):
+                entropy = sub.tensor_type == TensorType.COMPRESSED_TERNARY_32BIT
+                full = ops.expand_ternary(sub.weight.data, sub.original_shape, entropy)
+                sub.weight = nn.Parameter(full, requires_grad=for_training)
+                sub.tensor_type = TensorType.FLOAT_32BIT
+                sub.compact = False
+                sub._native = None
+        expand_compact_layers(sub, for_training)
