@@ -23,7 +23,10 @@ namespace tmq {
 namespace {
 
 constexpr int kBK = 64;          // k-tile
-constexpr int kPitch = 72;       // LDS row pitch in halfs (64 + 8 pad = 144 bytes)
+constexpr int kPitch = 64;       // LDS row pitch in halfs: 128 bytes = 8 chunks of 16 bytes, no padding.
+// Chunk c of row r is stored at position c ^ (r & 7): a wavefront's stores cover whole rows
+// (contiguous kilobytes) and the operand reads of 8 consecutive rows at one k offset land in 8
+// different 16-byte bank groups.
 
 struct Epilogue {
     const float *scale;      // [N] or null
@@ -37,14 +40,18 @@ struct Epilogue {
 // ---- loaders ------------------------------------------------------------------------------------------
 // A loader hands every thread CH 16-byte chunks (8 fp16) of the BM x 64 activation tile:
 // chunk i of thread t is row (t / 8 + i * T / 8), k offset (t % 8) * 8.
+//
+// FAST = rows are 16-byte aligned and K is a multiple of the k-tile: no guards in the hot loop
+// (rows past M are clamped to the last row; their results are never stored).
+template <bool FAST>
 struct DenseLoader {
     const _Float16 *x;
     int64_t M, K;
-    int vec;   // rows are 16-byte aligned (K % 8 == 0 and aligned base)
 
     template <int CH, int T>
     struct State {
         const _Float16 *row[CH];
+        bool live[CH];
         int kc;
     };
     template <int CH, int T>
@@ -53,7 +60,8 @@ struct DenseLoader {
 #pragma unroll
         for (int i = 0; i < CH; i++) {
             const int64_t m = m0 + (tid >> 3) + i * (T / 8);
-            st.row[i] = m < M ? x + m * K : nullptr;
+            st.live[i] = m < M;
+            st.row[i] = x + (m < M ? m : M - 1) * K;
         }
     }
     template <int CH, int T>
@@ -61,19 +69,17 @@ struct DenseLoader {
         const int64_t k = k0 + st.kc;
 #pragma unroll
         for (int i = 0; i < CH; i++) {
-            u32x4 v = {0u, 0u, 0u, 0u};
-            if (st.row[i] && k < K) {
-                if (vec && k + 8 <= K) {
-                    v = *reinterpret_cast<const u32x4 *>(st.row[i] + k);
-                } else {
-                    half8 h = {0, 0, 0, 0, 0, 0, 0, 0};
+            if constexpr (FAST) {
+                out[i] = *reinterpret_cast<const u32x4 *>(st.row[i] + k);
+            } else {
+                half8 h = {0, 0, 0, 0, 0, 0, 0, 0};
+                if (st.live[i]) {
 #pragma unroll
                     for (int e = 0; e < 8; e++)
                         if (k + e < K) h[e] = st.row[i][k + e];
-                    v = __builtin_bit_cast(u32x4, h);
                 }
+                out[i] = __builtin_bit_cast(u32x4, h);
             }
-            out[i] = v;
         }
     }
     template <int CH, int T>
@@ -81,11 +87,12 @@ struct DenseLoader {
 };
 
 // im2col view of an NHWC fp16 tensor: row m = (b, oh, ow), k = (i * kx + j) * C + c.
+// VEC = C is a multiple of 8 and the base is 16-byte aligned: a chunk is 8 channels of one tap.
+template <bool VEC>
 struct ConvLoader {
     const _Float16 *x;
     int64_t M, K;
     int B, C, H, W, Ho, Wo, ky, kx, sy, sx, py, px, dy, dx;
-    int vec;   // C % 8 == 0 and aligned base: a chunk is 8 channels of one tap
 
     template <int CH, int T>
     struct State {
@@ -132,13 +139,12 @@ struct ConvLoader {
         for (int q = 0; q < CH; q++) {
             u32x4 v = {0u, 0u, 0u, 0u};
             if (st.img[q] && k < K) {
-                if (vec) {
+                if constexpr (VEC) {
                     const int ih = st.ih0[q] + st.i * dy, iw = st.iw0[q] + st.j * dx;
                     if (ih >= 0 && ih < H && iw >= 0 && iw < W)
                         v = *reinterpret_cast<const u32x4 *>(st.img[q] + ((int64_t)ih * W + iw) * C + st.c);
                 } else {
                     half8 h;
-#pragma unroll
                     for (int e = 0; e < 8; e++) h[e] = at(st.img[q], st.ih0[q], st.iw0[q], k + e);
                     v = __builtin_bit_cast(u32x4, h);
                 }
@@ -158,12 +164,13 @@ struct ConvLoader {
 
 // ---- the tile kernel ---------------------------------------------------------------------------------
 template <int WM, int WN, int WGM, int WGN, class Loader>
-__global__ __launch_bounds__(64 * WGM * WGN) void tile_kernel(Loader ld, const uint32_t *__restrict__ native,
+__global__ __launch_bounds__(64 * WGM * WGN, 2) void tile_kernel(Loader ld, const uint32_t *__restrict__ native,
                                                               int64_t M, int64_t K, int64_t N, int64_t Kb, int64_t Nb,
                                                               Epilogue ep, int tiles_m, int tiles_n) {
     constexpr int T = 64 * WGM * WGN, BM = 16 * WM * WGM, BN = 16 * WN * WGN, CH = BM * 8 / T;
     static_assert(BM * 8 % T == 0, "chunks must divide evenly");
-    __shared__ __attribute__((aligned(16))) _Float16 As[BM * kPitch];
+    // two stages: the next k-tile is written while the current one is multiplied (one barrier per tile)
+    __shared__ __attribute__((aligned(16))) _Float16 As[2][BM * kPitch];
 
     // XCD-aware tile order: workgroup ids go round-robin over the 8 XCDs; give each XCD a
     // contiguous run of tiles, n fastest, so its L2 sees the same activation rows.
@@ -186,78 +193,150 @@ __global__ __launch_bounds__(64 * WGM * WGN) void tile_kernel(Loader ld, const u
 #pragma unroll
         for (int j = 0; j < WN; j++) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-    // per n-fragment pointer into the native layout (dword index lane * 4 + d inside a block)
+    // per n-fragment pointer into the native layout (dword index lane * 4 + d inside a block);
+    // fragments past N read block 0 of the last valid fragment (finite bits, never stored)
     const uint32_t *wptr[WN];
 #pragma unroll
     for (int j = 0; j < WN; j++) {
-        const int64_t nb = n0 / 16 + wn * WN + j;
-        wptr[j] = nb < Nb ? native + (nb * Kb) * 256 + lane * 4 : nullptr;
+        int64_t nb = n0 / 16 + wn * WN + j;
+        if (nb >= Nb) nb = Nb - 1;
+        wptr[j] = native + (nb * Kb) * 256 + lane * 4;
     }
     const int KT = (int)((K + kBK - 1) / kBK);
 
     u32x4 stage[CH];
     uint32_t wcur[WN], wnext[WN];
+    const int srow = tid >> 3;
+    const int scol = (((tid & 7) ^ (srow & 7)) * 8);   // (T / 8) is a multiple of 8, so row & 7 == srow & 7 for every chunk
+    // prologue: weight words first, activations last, so that the wait in front of the LDS store
+    // retires every outstanding load and the loop starts with a clean memory counter
+#pragma unroll
+    for (int j = 0; j < WN; j++) wcur[j] = wptr[j][0];
     ld.template fetch<CH, T>(st, 0, stage);
 #pragma unroll
-    for (int j = 0; j < WN; j++) wcur[j] = wptr[j] ? wptr[j][0] : 0u;
-
-    const int srow = tid >> 3, scol = (tid & 7) * 8;
-    for (int kt = 0; kt < KT; kt++) {
-        __syncthreads();   // every wave is done reading the previous tile
+    for (int i = 0; i < CH; i++) *reinterpret_cast<u32x4 *>(&As[0][(srow + i * (T / 8)) * kPitch + scol]) = stage[i];
 #pragma unroll
-        for (int i = 0; i < CH; i++)
-            *reinterpret_cast<u32x4 *>(&As[(srow + i * (T / 8)) * kPitch + scol]) = stage[i];
-        __syncthreads();
-        if (kt + 1 < KT) {
+    for (int j = 0; j < WN; j++) asm volatile("" ::"v"(wcur[j]));   // pin the weight loads in front of the loop
+    __syncthreads();
+
+    // per-column epilogue constants, fetched now so their latency hides behind the main loop
+    const int64_t nw0 = n0 + (int64_t)wn * WN * 16;        // first column of this wave
+    float sc[WN], bi[WN];
+#pragma unroll
+    for (int j = 0; j < WN; j++) {
+        const int64_t n = nw0 + j * 16 + r16;
+        sc[j] = (n < N && ep.scale ? ep.scale[n] : 1.0f) * (1.0f / kWeightUnit);
+        bi[j] = (n < N && ep.bias) ? ep.bias[n] : 0.0f;
+    }
+
+    const int arow = (wm * WM * 16 + r16) * kPitch;
+    // operand read of m-fragment i, k-step s: chunk (4 s + g) of row (.. + 16 i + r16); 16 i keeps row & 7
+    auto swz = [&](int i, int s) { return i * 16 * kPitch + (((4 * s + g) ^ (r16 & 7)) * 8); };
+    for (int kt = 0; kt < KT; kt++) {
+        const int cur = kt & 1;
+        const bool more = kt + 1 < KT;
+        if (more) {   // global loads of the next tile fly during the math
             ld.template advance<CH, T>(st);
             ld.template fetch<CH, T>(st, (int64_t)(kt + 1) * kBK, stage);
             const int kn = kt + 1;
 #pragma unroll
-            for (int j = 0; j < WN; j++) wnext[j] = wptr[j] ? wptr[j][(int64_t)(kn >> 2) * 256 + (kn & 3)] : 0u;
+            for (int j = 0; j < WN; j++) wnext[j] = wptr[j][(int64_t)(kn >> 2) * 256 + (kn & 3)];
         }
+        const _Float16 *abase = &As[cur][arow];
+        // Software pipeline over the 2 WM operand reads of the tile (fragment i, k-step s): kAhead reads
+        // are in flight ahead of the MFMAs that consume them, so LDS latency hides behind matrix
+        // work of this wave. sched_barrier pins the order; the compiler only adds the waits.
+        constexpr int NQ = 2 * WM, kAhead = NQ < 4 ? NQ : 4;
+        half8 a[NQ];
+        half8 bfr[2][WN];
 #pragma unroll
-        for (int s = 0; s < 2; s++) {
-            half8 b[WN];
+        for (int q = 0; q < kAhead; q++) a[q] = *reinterpret_cast<const half8 *>(abase + swz(q >> 1, q & 1));
 #pragma unroll
-            for (int j = 0; j < WN; j++) b[j] = decode_step(wcur[j], s);
+        for (int j = 0; j < WN; j++) bfr[0][j] = decode_step(wcur[j], 0);
 #pragma unroll
-            for (int i = 0; i < WM; i++) {
-                const half8 a = *reinterpret_cast<const half8 *>(
-                    &As[(wm * WM * 16 + i * 16 + r16) * kPitch + s * 32 + g * 8]);
+        for (int j = 0; j < WN; j++) bfr[1][j] = decode_step(wcur[j], 1);
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int j = 0; j < WN; j++) acc[i][j] = mfma16(a, b[j], acc[i][j]);
-            }
+        for (int q = 0; q < NQ; q++) {
+#pragma unroll
+            for (int j = 0; j < WN; j++) acc[q >> 1][j] = mfma16(a[q], bfr[q & 1][j], acc[q >> 1][j]);
+            if (q + kAhead < NQ)
+                a[q + kAhead] = *reinterpret_cast<const half8 *>(abase + swz((q + kAhead) >> 1, (q + kAhead) & 1));
+            __builtin_amdgcn_sched_barrier(0);
         }
+        if (more) {
 #pragma unroll
-        for (int j = 0; j < WN; j++) wcur[j] = wnext[j];
+            for (int i = 0; i < CH; i++)
+                *reinterpret_cast<u32x4 *>(&As[cur ^ 1][(srow + i * (T / 8)) * kPitch + scol]) = stage[i];
+#pragma unroll
+            for (int j = 0; j < WN; j++) wcur[j] = wnext[j];
+        }
+        __syncthreads();
     }
 
-    // epilogue: lane holds rows m = .. + 4g + r (r = 0..3), column n = .. + r16
+    // Epilogue. A lane holds rows 4g + r, column r16 of each 16 x 16 accumulator -- 64-byte row
+    // pieces if stored directly. Instead every wave transposes one 16-row slab (16 x 16 WN values)
+    // at a time through its own slice of the (now idle) activation buffer and writes whole rows:
+    // 16 lanes x 16 bytes = 256 contiguous bytes per row and store instruction.
+    constexpr int kEP = 16 * WN + 4;                       // slab row pitch in floats (+4: conflict-free)
+    static_assert(WGM * WGN * 16 * kEP * 4 <= 2 * BM * kPitch * 2, "epilogue slab does not fit the LDS buffer");
+    float *slab = reinterpret_cast<float *>(&As[0][0]) + wv * 16 * kEP;
+    const bool vec = (N % 4 == 0) && ((reinterpret_cast<uintptr_t>(ep.y) | reinterpret_cast<uintptr_t>(ep.residual)) & 15u) == 0;
 #pragma unroll
-    for (int j = 0; j < WN; j++) {
-        const int64_t n = n0 + (wn * WN + j) * 16 + r16;
-        if (n >= N) continue;
-        const float sc = (ep.scale ? ep.scale[n] : 1.0f) * (1.0f / kWeightUnit);
-        const float bi = ep.bias ? ep.bias[n] : 0.0f;
+    for (int i = 0; i < WM; i++) {
 #pragma unroll
-        for (int i = 0; i < WM; i++) {
+        for (int j = 0; j < WN; j++)
 #pragma unroll
-            for (int r = 0; r < 4; r++) {
-                const int64_t m = m0 + (wm * WM + i) * 16 + g * 4 + r;
-                if (m >= M) continue;
-                float v = acc[i][j][r] * sc + bi;
-                const int64_t o = m * N + n;
+            for (int r = 0; r < 4; r++) slab[(g * 4 + r) * kEP + j * 16 + r16] = acc[i][j][r] * sc[j] + bi[j];
+        __builtin_amdgcn_wave_barrier();
+        const int64_t mrow0 = m0 + (int64_t)(wm * WM + i) * 16;
+#pragma unroll
+        for (int t = 0; t < WN; t++) {                     // 16 rows x (16 WN / 4) float4 = 64 WN float4 per slab
+            const int idx = t * 64 + lane, row = idx / (4 * WN), c4 = idx % (4 * WN);
+            const int64_t m = mrow0 + row, n = nw0 + c4 * 4;
+            floatx4 v = *reinterpret_cast<const floatx4 *>(&slab[row * kEP + c4 * 4]);
+            if (m >= M || n >= N) continue;
+            const int64_t o = m * N + n;
+            if (vec) {
                 if (ep.y_f16) {
-                    if (ep.residual) v += (float)static_cast<const _Float16 *>(ep.residual)[o];
-                    if (ep.relu) v = v > 0.f ? v : 0.f;
-                    static_cast<_Float16 *>(ep.y)[o] = (_Float16)v;
+                    if (ep.residual) {
+                        const half4 rs = *reinterpret_cast<const half4 *>(static_cast<const _Float16 *>(ep.residual) + o);
+#pragma unroll
+                        for (int e = 0; e < 4; e++) v[e] += (float)rs[e];
+                    }
+                    half4 h;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) h[e] = (_Float16)((ep.relu && v[e] < 0.f) ? 0.f : v[e]);
+                    *reinterpret_cast<half4 *>(static_cast<_Float16 *>(ep.y) + o) = h;
                 } else {
-                    if (ep.residual) v += static_cast<const float *>(ep.residual)[o];
-                    if (ep.relu) v = v > 0.f ? v : 0.f;
-                    static_cast<float *>(ep.y)[o] = v;
+                    if (ep.residual) {
+                        const floatx4 rs = *reinterpret_cast<const floatx4 *>(static_cast<const float *>(ep.residual) + o);
+                        v += rs;
+                    }
+                    if (ep.relu) {
+#pragma unroll
+                        for (int e = 0; e < 4; e++) v[e] = v[e] > 0.f ? v[e] : 0.f;
+                    }
+                    __builtin_nontemporal_store(v, reinterpret_cast<floatx4 *>(static_cast<float *>(ep.y) + o));
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    if (n + e >= N) break;
+                    float f = v[e];
+                    if (ep.y_f16) {
+                        if (ep.residual) f += (float)static_cast<const _Float16 *>(ep.residual)[o + e];
+                        if (ep.relu) f = f > 0.f ? f : 0.f;
+                        static_cast<_Float16 *>(ep.y)[o + e] = (_Float16)f;
+                    } else {
+                        if (ep.residual) f += static_cast<const float *>(ep.residual)[o + e];
+                        if (ep.relu) f = f > 0.f ? f : 0.f;
+                        static_cast<float *>(ep.y)[o + e] = f;
+                    }
                 }
             }
         }
+        __builtin_amdgcn_wave_barrier();
     }
 }
 
@@ -278,6 +357,7 @@ template <class Loader>
 int dispatch_tile(const Loader &ld, const void *native, int64_t M, int64_t K, int64_t N, const Epilogue &ep,
                   void *stream) {
     auto wgs = [&](int bm, int bn) { return ((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
+    if (N > 128 && wgs(128, 256) >= 512) return launch_tile<8, 4, 1, 4>(ld, native, M, K, N, ep, stream);
     if (N > 128 && wgs(256, 256) >= 256) return launch_tile<8, 4, 2, 4>(ld, native, M, K, N, ep, stream);
     if (N > 64 && wgs(256, 128) >= 384) return launch_tile<8, 4, 2, 2>(ld, native, M, K, N, ep, stream);
     if (N > 64 && wgs(128, 128) >= 256) return launch_tile<4, 4, 2, 2>(ld, native, M, K, N, ep, stream);
@@ -289,9 +369,10 @@ int dispatch_tile(const Loader &ld, const void *native, int64_t M, int64_t K, in
 
 int launch_gemm_dense(const void *x, int64_t M, int64_t K, const void *native, int64_t N, const float *scale,
                       const float *bias, const void *residual, int relu, void *y, int y_f16, void *stream) {
-    DenseLoader ld{static_cast<const _Float16 *>(x), M, K, (K % 8 == 0) && aligned16(x) ? 1 : 0};
     Epilogue ep{scale, bias, residual, y, relu, y_f16};
-    return dispatch_tile(ld, native, M, K, N, ep, stream);
+    if ((K % kBK == 0) && aligned16(x))
+        return dispatch_tile(DenseLoader<true>{static_cast<const _Float16 *>(x), M, K}, native, M, K, N, ep, stream);
+    return dispatch_tile(DenseLoader<false>{static_cast<const _Float16 *>(x), M, K}, native, M, K, N, ep, stream);
 }
 
 }  // namespace tmq
@@ -324,10 +405,13 @@ int tmq_ternary_conv2d(const void *x, const tmq_conv_shape *s, const void *nativ
     if (ho <= 0 || wo <= 0) return TMQ_ERR_INVALID_ARG;
     const int64_t M = (int64_t)s->B * ho * wo, K = (int64_t)s->C * s->ky * s->kx;
     if (M == 0) return TMQ_OK;
-    ConvLoader ld{static_cast<const _Float16 *>(x), M, K, s->B, s->C, s->H, s->W, ho, wo, s->ky, s->kx, s->sy, s->sx,
-                  s->py, s->px, s->dy, s->dx, (s->C % 8 == 0) && aligned16(x) ? 1 : 0};
     Epilogue ep{scale, bias, residual, y, relu, y_dtype == TMQ_F16 ? 1 : 0};
-    return dispatch_tile(ld, native, M, K, s->N, ep, stream);
+    const _Float16 *xp = static_cast<const _Float16 *>(x);
+    if ((s->C % 8 == 0) && aligned16(x))
+        return dispatch_tile(ConvLoader<true>{xp, M, K, s->B, s->C, s->H, s->W, ho, wo, s->ky, s->kx, s->sy, s->sx,
+                                              s->py, s->px, s->dy, s->dx}, native, M, K, s->N, ep, stream);
+    return dispatch_tile(ConvLoader<false>{xp, M, K, s->B, s->C, s->H, s->W, ho, wo, s->ky, s->kx, s->sy, s->sx, s->py,
+                                           s->px, s->dy, s->dx}, native, M, K, s->N, ep, stream);
 }
 
 }  // extern "C"
