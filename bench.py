@@ -190,6 +190,79 @@ def bench_linear(args, torch):
             "value": out.get("4096", {}).get("tflops"), "by_M": out}
 
 
+def bench_resnet_infer(args, torch):
+    """BASELINE configs[3]: ResNet-18 (102 classes) ternary inference, batch 64 of 3x224x224 fp16."""
+    import tmq_amd as t
+    from bench_models import ResNet18, randomize_ternary_, FusedTernaryResNet18
+    dev = torch.device("cuda:0")
+    torch.manual_seed(20)
+    model = ResNet18(102)
+    ctrl = t.QuantizationControl()
+    t.quantize_model(model, ctrl)
+    randomize_ternary_(model, torch.Generator().manual_seed(20))
+    model.to(dev).eval()
+    t.compressed_state_dict(model, strong=False)              # switches every layer to compact weights
+    B = args.batch or 64
+    x = torch.randn(B, 3, 224, 224, generator=torch.Generator().manual_seed(20)).half().to(dev)
+    fused = FusedTernaryResNet18(model)
+    out = {}
+    for name, fn, reps in (("fused", lambda: fused(x), args.steps), ("drop_in", lambda: model(x), max(3, args.steps // 4))):
+        with torch.no_grad():
+            for _ in range(max(2, args.warmup // 4)):
+                fn()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(reps):
+                fn()
+            torch.cuda.synchronize()
+        dt = (time.perf_counter() - t0) / reps
+        out[name] = {"ms": round(dt * 1e3, 4), "img_s": round(B / dt, 1), "tflops": round(3.627e9 * B / dt / 1e12, 2)}
+    return {"metric": "ResNet-18 img/s", "value": out["fused"]["img_s"], "unit": "img/s", "n_gpus": 1, "dtype": "f16",
+            "data": "synthetic", "config": {"workload": "configs[3]: ResNet-18/102 ternary inference", "batch": B},
+            "modes": out}
+
+
+def bench_resnet_qat(args, torch):
+    """BASELINE configs[4]: one ResNet-18 QAT step, batch 128 fp32, hardness 2.236133, penalty 5e-4."""
+    import tmq_amd as t
+    from bench_models import ResNet18
+    from torch import nn
+    dev = torch.device("cuda:0")
+    torch.manual_seed(30)
+    model = ResNet18(102)
+    ctrl = t.QuantizationControl(epoch_knots=t.QuantizationScheduleBuilder.default_schedule(150),
+                                 qpenalty_range=(5e-4, 5e-4))
+    t.quantize_model(model, ctrl)
+    model.to(dev).train()
+    for e in range(76):
+        ctrl.step(e)
+    B = args.batch or 128
+    x = torch.randn(B, 3, 224, 224, generator=torch.Generator().manual_seed(30)).to(dev)
+    labels = torch.randint(0, 102, (B,), generator=torch.Generator().manual_seed(31)).to(dev)
+    opt = torch.optim.Adam(model.parameters(), lr=0.1)
+
+    def step():
+        opt.zero_grad(set_to_none=True)
+        loss = nn.functional.cross_entropy(model(x), labels) + ctrl.quantization_loss()
+        loss.backward()
+        opt.step()
+        ctrl.clamp()
+
+    reps = max(3, args.steps // 10)
+    for _ in range(3):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        step()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / reps
+    return {"metric": "ResNet-18 QAT step time", "value": round(dt * 1e3, 3), "unit": "ms", "higher_is_better": False,
+            "n_gpus": 1, "dtype": "f32", "data": "synthetic",
+            "config": {"workload": "configs[4]: ResNet-18 QAT step", "batch": B, "digamma": ctrl.digamma,
+                       "qpenalty": ctrl.qpenalty, "quantized_weights": 11219136}}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -203,6 +276,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--m-list", default="1,16,256,4096")
     ap.add_argument("--rotate", type=int, default=1)
+    ap.add_argument("--batch", type=int, default=0)
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build targets one GPU; --gpus N with N > 1 is not supported (the path has no "
@@ -216,6 +290,10 @@ def main():
         res = bench_softstep(args, torch)
     elif args.workload == "linear":
         res = bench_linear(args, torch)
+    elif args.workload == "resnet_infer":
+        res = bench_resnet_infer(args, torch)
+    elif args.workload == "resnet_qat":
+        res = bench_resnet_qat(args, torch)
     else:
         print(f"bench.py: unknown workload {args.workload}", file=sys.stderr)
         sys.exit(2)

@@ -1,0 +1,123 @@
+"""ResNet-18 for the inference / QAT workloads of BASELINE.json (configs[3] and configs[4]).
+
+torchvision is not available offline, so the network is defined here: the standard BasicBlock
+[2, 2, 2, 2] layout with plain nn.Conv2d / nn.Linear layers (bias-free convolutions, BatchNorm
+after every convolution), so that tmq_amd.quantize_model swaps them exactly as it would swap
+torchvision's. `FusedTernaryResNet18` is the deployment form: it reads the compact weights of
+a quantized model and runs every convolution as one ternary implicit-GEMM launch with the
+eval-mode BatchNorm folded into the per-channel epilogue, ReLU and the residual add fused, and fp16
+channels_last activations between layers.
+"""
+import torch
+from torch import nn
+
+
+class BasicBlock(nn.Module):
+    def __init__(self, cin, cout, stride):
+        super().__init__()
+        self.conv1 = nn.Conv2d(cin, cout, 3, stride, 1, bias=False)
+        self.bn1 = nn.BatchNorm2d(cout)
+        self.conv2 = nn.Conv2d(cout, cout, 3, 1, 1, bias=False)
+        self.bn2 = nn.BatchNorm2d(cout)
+        self.downsample = None
+        if stride != 1 or cin != cout:
+            self.downsample = nn.Sequential(nn.Conv2d(cin, cout, 1, stride, 0, bias=False), nn.BatchNorm2d(cout))
+
+    def forward(self, x):
+        idt = x if self.downsample is None else self.downsample(x)
+        out = torch.relu(self.bn1(self.conv1(x)))
+        out = self.bn2(self.conv2(out))
+        return torch.relu(out + idt)
+
+
+class ResNet18(nn.Module):
+    def __init__(self, num_classes=102):
+        super().__init__()
+        self.conv1 = nn.Conv2d(3, 64, 7, 2, 3, bias=False)
+        self.bn1 = nn.BatchNorm2d(64)
+        self.maxpool = nn.MaxPool2d(3, 2, 1)
+        chans, layers, cin = (64, 128, 256, 512), [], 64
+        for li, c in enumerate(chans):
+            layers.append(nn.Sequential(BasicBlock(cin, c, 1 if li == 0 else 2), BasicBlock(c, c, 1)))
+            cin = c
+        self.layer1, self.layer2, self.layer3, self.layer4 = layers
+        self.avgpool = nn.AdaptiveAvgPool2d(1)
+        self.fc = nn.Linear(512, num_classes)
+
+    def forward(self, x):
+        x = self.maxpool(torch.relu(self.bn1(self.conv1(x))))
+        x = self.layer4(self.layer3(self.layer2(self.layer1(x))))
+        return self.fc(torch.flatten(self.avgpool(x), 1))
+
+
+def randomize_ternary_(model, generator, p0=0.5):
+    """Fill every conv / linear weight with i.i.d. ternary values, P(0) = p0, and every BatchNorm
+    with running_mean ~ N(0, 0.1), running_var ~ U(0.5, 2), gamma 1, beta 0 (BASELINE configs[3])."""
+    with torch.no_grad():
+        for m in model.modules():
+            w = getattr(m, "weight", None)
+            if isinstance(m, nn.BatchNorm2d):
+                m.running_mean.copy_(0.1 * torch.randn(m.num_features, generator=generator))
+                m.running_var.copy_(0.5 + 1.5 * torch.rand(m.num_features, generator=generator))
+                m.weight.fill_(1.0)
+                m.bias.zero_()
+            elif w is not None and w.dim() in (2, 4) and w.dtype == torch.float32:
+                u = torch.rand(w.shape, generator=generator)
+                w.copy_(torch.where(u < (1 - p0) / 2, 1.0, torch.where(u < 1 - p0, -1.0, 0.0)))
+
+
+class FusedTernaryResNet18:
+    """Deployment runner over a tmq_amd-quantized ResNet18 whose layers hold compact weights."""
+
+    def __init__(self, model: ResNet18, pad_stem_channels=8):
+        from tmq_amd import ops
+        self.ops = ops
+        self.dev = model.fc.weight.device
+        self.stem_c = pad_stem_channels
+        self.stem = self._conv(model.conv1, model.bn1, pad_c=pad_stem_channels)
+        self.blocks = []
+        for layer in (model.layer1, model.layer2, model.layer3, model.layer4):
+            for blk in layer:
+                ds = None if blk.downsample is None else self._conv(blk.downsample[0], blk.downsample[1])
+                self.blocks.append((self._conv(blk.conv1, blk.bn1), self._conv(blk.conv2, blk.bn2), ds))
+        self.fc = (ops.NativeWeights(model.fc.weight.data, model.fc.original_shape[0]),
+                   model.fc.bias.data.float() if model.fc.bias is not None else None)
+
+    def _conv(self, conv, bn, pad_c=None):
+        ops = self.ops
+        N, C, ky, kx = (int(v) for v in conv.original_shape)
+        words = conv.weight.data
+        if pad_c is not None and C < pad_c:
+            # zero-pad the input channels so that im2col rows are whole 16-byte chunks
+            w = ops.expand_ternary(words, [N, C, ky, kx])
+            wp = torch.zeros(N, pad_c, ky, kx, device=w.device)
+            wp[:, :C] = w
+            words, C = ops.compactify_ternary(wp), pad_c
+        nw = ops.NativeWeights(words, N, conv_kernel=(ky, kx))
+        # eval-mode BatchNorm folded into the epilogue: y = gamma (acc - mean) / sqrt(var + eps) + beta
+        inv = (bn.running_var + bn.eps).rsqrt() * bn.weight
+        scale = inv.float().contiguous()
+        bias = (bn.bias - bn.running_mean * inv).float().contiguous()
+        pair = lambda v: tuple(v) if isinstance(v, (tuple, list)) else (v, v)
+        return nw, scale, bias, pair(conv.stride), pair(conv.padding)
+
+    def _run(self, x, layer, relu, residual=None):
+        nw, scale, bias, stride, pad = layer
+        return self.ops.ternary_conv2d(x, nw, stride, pad, 1, scale, bias, residual=residual, relu=relu,
+                                       out_dtype=torch.float16)
+
+    @torch.no_grad()
+    def __call__(self, x):
+        B, C, H, W = x.shape
+        xs = torch.empty((B, self.stem_c, H, W), dtype=torch.float16, device=x.device,
+                         memory_format=torch.channels_last).zero_()
+        xs[:, :C] = x
+        y = self._run(xs, self.stem, relu=True)
+        y = torch.nn.functional.max_pool2d(y, 3, 2, 1)
+        for c1, c2, ds in self.blocks:
+            idt = y if ds is None else self._run(y, ds, relu=False)
+            h = self._run(y, c1, relu=True)
+            y = self._run(h, c2, relu=True, residual=idt)
+        feat = y.float().mean(dim=(2, 3)).half().contiguous()
+        nw, bias = self.fc
+        return self.ops.ternary_linear(feat, nw, bias=bias)

@@ -1,0 +1,97 @@
+"""ResNet-18 (102 classes) compact inference and one QAT step on the GPU (BASELINE configs[3], [4])."""
+import numpy as np
+import pytest
+import torch
+from torch import nn
+
+pytestmark = pytest.mark.gpu
+
+
+def _build(cuda, seed=20):
+    import tmq_amd as t
+    from bench_models import ResNet18, randomize_ternary_
+    torch.manual_seed(seed)
+    model = ResNet18(102)
+    ctrl = t.QuantizationControl(epoch_knots=t.QuantizationScheduleBuilder.default_schedule(150),
+                                 qpenalty_range=(5e-4, 5e-4))
+    t.quantize_model(model, ctrl)
+    assert len(ctrl._registry) == 21
+    assert sum(n.weight.numel() for n in ctrl._registry.values()) == 11_219_136
+    randomize_ternary_(model, torch.Generator().manual_seed(seed))
+    return t, model.to(cuda), ctrl
+
+
+def test_compact_inference_matches_fp32_reference(cuda):
+    t, model, ctrl = _build(cuda)
+    ctrl.inference()
+    x = torch.randn(4, 3, 224, 224, generator=torch.Generator().manual_seed(1)).to(cuda)
+    # Unscaled ternary weights multiply the activation scale by ~sqrt(fan_in / 2) per layer; calibrate
+    # the BatchNorm statistics on the batch so that activations stay O(1) and fp16 does not overflow.
+    for m in model.modules():
+        if isinstance(m, nn.BatchNorm2d):
+            m.momentum = 1.0
+    model.train()
+    with torch.no_grad():
+        model(x)
+    model.eval()
+    # fp32 reference on the ternary-valued weights, with each conv / fc input rounded to fp16 like the
+    # compact kernels see it (so only the summation order differs)
+    hooks = [m.register_forward_pre_hook(lambda mod, inp: (inp[0].half().float(),))
+             for m in model.modules() if isinstance(m, (t.Conv2d, t.Linear))]
+    with torch.no_grad():
+        ref = model(x)
+    for h in hooks:
+        h.remove()
+    with torch.no_grad():
+        ref_plain = model(x)
+    sd = t.compressed_state_dict(model, strong=False)
+    packed_bytes = sum(v.numel() * 4 for k, v in sd.items() if v.dtype == torch.int32)
+    assert packed_bytes == sum(((n.original_shape[0] + 15) // 16) * 4 * int(np.prod(n.original_shape[1:]))
+                               for n in ctrl._registry.values())
+    with torch.no_grad():
+        out = model(x)                                  # drop-in path: compact conv + PyTorch BN / ReLU / pooling
+    err = (out - ref).abs().max().item() / ref.abs().max().item()
+    assert err <= 1e-3, err
+    assert (out - ref_plain).abs().max().item() / ref_plain.abs().max().item() <= 3e-2
+    # deployment path: folded BatchNorm, fused ReLU / residual, fp16 activations
+    from bench_models import FusedTernaryResNet18
+    fused = FusedTernaryResNet18(model)
+    yf = fused(x.half())
+    assert tuple(yf.shape) == (4, 102)
+    errf = (yf - ref_plain).abs().max().item() / ref_plain.abs().max().item()
+    assert errf <= 3e-2, errf
+    assert (yf.argmax(1) == ref_plain.argmax(1)).float().mean().item() >= 0.75
+
+
+def test_qat_step_runs_and_matches_unfused_losses(cuda):
+    t, model, ctrl = _build(cuda, seed=30)
+    with torch.no_grad():                                  # back to U(-1, 1) training weights
+        for n in ctrl._registry.values():
+            n.weight.copy_(2 * torch.rand(n.weight.shape, generator=torch.Generator().manual_seed(5)) - 1)
+    for e in range(76):
+        ctrl.step(e)
+    assert abs(ctrl.digamma - 2.236133) < 1e-6
+    model.train()
+    x = torch.randn(8, 3, 224, 224, generator=torch.Generator().manual_seed(2)).to(cuda)
+    labels = torch.randint(0, 102, (8,), generator=torch.Generator().manual_seed(3)).to(cuda)
+    opt = torch.optim.Adam(model.parameters(), lr=0.1)
+    opt.zero_grad()
+    loss = nn.functional.cross_entropy(model(x), labels)
+    ql = ctrl.quantization_loss()
+    per_layer = sum(n.quantization_loss(ctrl.qpenalty, ctrl.qpenalty_sharpness) for n in ctrl._registry.values())
+    assert abs(ql.item() - per_layer.item()) <= 1e-5 * abs(per_layer.item())
+    (loss + ql).backward()
+    g_fused = {k: n.weight.grad.clone() for k, n in ctrl._registry.items()}
+    # the same gradients through the per-layer autograd functions
+    opt.zero_grad()
+    loss2 = nn.functional.cross_entropy(model(x), labels)
+    (loss2 + sum(n.quantization_loss(ctrl.qpenalty, ctrl.qpenalty_sharpness) for n in ctrl._registry.values())).backward()
+    for k, n in ctrl._registry.items():
+        assert torch.isfinite(n.weight.grad).all()
+        d = (n.weight.grad - g_fused[k]).abs().max().item()
+        # PyTorch's convolution backward is not bit-reproducible from run to run; the TMQ part is
+        assert d <= 2e-3 * max(1e-6, g_fused[k].abs().max().item()), (k, d)
+    opt.step()
+    ctrl.clamp()
+    for n in ctrl._registry.values():
+        assert n.weight.data.abs().max().item() <= 1.0
