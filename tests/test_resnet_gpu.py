@@ -81,16 +81,16 @@ def test_qat_step_runs_and_matches_unfused_losses(cuda):
     per_layer = sum(n.quantization_loss(ctrl.qpenalty, ctrl.qpenalty_sharpness) for n in ctrl._registry.values())
     assert abs(ql.item() - per_layer.item()) <= 1e-5 * abs(per_layer.item())
     (loss + ql).backward()
-    g_fused = {k: n.weight.grad.clone() for k, n in ctrl._registry.items()}
-    # the same gradients through the per-layer autograd functions
-    opt.zero_grad()
-    loss2 = nn.functional.cross_entropy(model(x), labels)
-    (loss2 + sum(n.quantization_loss(ctrl.qpenalty, ctrl.qpenalty_sharpness) for n in ctrl._registry.values())).backward()
-    for k, n in ctrl._registry.items():
+    for n in ctrl._registry.values():
         assert torch.isfinite(n.weight.grad).all()
-        d = (n.weight.grad - g_fused[k]).abs().max().item()
-        # PyTorch's convolution backward is not bit-reproducible from run to run; the TMQ part is
-        assert d <= 2e-3 * max(1e-6, g_fused[k].abs().max().item()), (k, d)
+    # the quantization-loss gradient alone: one multi-tensor launch vs the per-layer autograd functions
+    # (PyTorch's convolution backward is not reproducible run to run, so it is kept out of this comparison)
+    ws = [n.weight for n in ctrl._registry.values()]
+    g_fused = torch.autograd.grad(ctrl.quantization_loss(), ws)
+    g_layer = torch.autograd.grad(sum(n.quantization_loss(ctrl.qpenalty, ctrl.qpenalty_sharpness)
+                                      for n in ctrl._registry.values()), ws)
+    for k, a, b in zip(ctrl._registry, g_fused, g_layer):
+        assert torch.equal(a, b), k
     opt.step()
     ctrl.clamp()
     for n in ctrl._registry.values():
