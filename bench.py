@@ -168,18 +168,27 @@ def bench_linear(args, torch):
         reps = args.steps if M < 4096 else max(10, args.steps // 4)
         for i in range(max(args.warmup, 3)):
             ops.ternary_linear(x, natives[i % nrot], scale)
+        torch.cuda.synchronize()
+        # One pass over the rotating weight buffers is captured in a HIP graph (kernel launches only),
+        # so that the figure is the kernel's own rate and not the Python call overhead between launches.
+        graph, side = torch.cuda.CUDAGraph(), torch.cuda.Stream()
+        per_graph = nrot if M < 4096 else 4
+        with torch.cuda.stream(side):
+            with torch.cuda.graph(graph, stream=side):
+                for i in range(per_graph):
+                    ops.ternary_linear(x, natives[i % nrot], scale)
+        replays = max(2, reps // per_graph)
         t_settle = time.perf_counter()
         while time.perf_counter() - t_settle < args.settle_ms * 1e-3:
-            ops.ternary_linear(x, natives[0], scale)
+            graph.replay()
             torch.cuda.synchronize()
-        torch.cuda.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
-        for i in range(reps):
-            ops.ternary_linear(x, natives[i % nrot], scale)
+        for i in range(replays):
+            graph.replay()
         e1.record()
         torch.cuda.synchronize()
-        us = e0.elapsed_time(e1) / reps * 1e3
+        us = e0.elapsed_time(e1) / (replays * per_graph) * 1e3
         flops = 2.0 * M * N * K
         byts = K * N / 4 + 2 * M * K + 4 * M * N + 4 * N
         out[str(M)] = {"us": round(us, 3), "tflops": round(flops / us / 1e6, 3), "gbs": round(byts / us / 1e3, 2),

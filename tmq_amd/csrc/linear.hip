@@ -93,98 +93,211 @@ __device__ __forceinline__ XFrag<X32> load_x(const void *x, int64_t m, int64_t M
 }
 
 // ---- skinny kernel --------------------------------------------------------------------------------
-// grid.x = ceil(N/16); blockDim.x = 64 * waves; wave w owns the weight blocks kb = w, w + waves, ...
-// MT = number of 16-row activation tiles (M <= 16 MT). D[n][m]: weights are the A operand.
-template <int MT, bool X32, bool VEC>
+// grid.x = ceil(Nb / G) workgroups of `waves` wavefronts; a workgroup owns G consecutive blocks of 16
+// output channels. Wavefront w works on channel block (w % G) and on the weight blocks
+// kb = w / G, w / G + waves / G, ... of it. MT = number of 16-row activation tiles (M <= 16 MT).
+// D[n][m]: the weights are the A operand of the MFMA.
+//
+// The kernel is a weight stream; what counts is the number of bytes in flight and the VALU work
+// per byte. Every wavefront keeps kAhead 1 KiB weight blocks outstanding in a rolling pipeline (a
+// register is reloaded as soon as its block has been consumed). XLDS: the activations are staged
+// once per workgroup in LDS -- fp32 activations already split into their two fp16 terms -- padded
+// with zeros to whole weight blocks, so that the inner loop has no edge handling at all: an operand
+// read is one ds_read_b128 at (lane base + block offset + immediate). Lanes whose activation row
+// does not exist (m >= M) read from a 512-byte zero region with a block stride of 0.
+constexpr int kAhead = 4;
+constexpr size_t kSkinnyLdsMax = 152 * 1024;
+
+template <int MT, bool X32, bool VEC, bool XLDS>
 __global__ __launch_bounds__(1024) void skinny_kernel(const void *__restrict__ x, int64_t M, int64_t K,
-                                                      const u32x4 *__restrict__ native, int64_t Kb, int64_t N,
-                                                      const float *__restrict__ scale, const float *__restrict__ bias,
-                                                      const void *__restrict__ residual, int relu, void *__restrict__ y,
-                                                      int y_f16) {
-    extern __shared__ float red[];   // [waves][MT][64][4]
+                                                      const u32x4 *__restrict__ native, int Kb, int64_t N, int64_t Nb,
+                                                      int G, const float *__restrict__ scale,
+                                                      const float *__restrict__ bias, const void *__restrict__ residual,
+                                                      int relu, void *__restrict__ y, int y_f16) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6, waves = blockDim.x >> 6;
     const int j = lane & 15, g = lane >> 4;
-    const int64_t nb = blockIdx.x;
+    const int sub = wv % G, ks = wv / G, nks = waves / G;
+    const int64_t nb = (int64_t)blockIdx.x * G + sub;
+    const bool valid = nb < Nb;
+    constexpr int kPlanes = X32 ? 2 : 1;
+    const int pitch = (Kb * kKB + 8) * 2;                              // bytes per staged activation row
+    const size_t plane = (size_t)M * pitch;
+    unsigned char *zeros = smem + (XLDS ? kPlanes * plane : 0);
+    floatx4 *slot = reinterpret_cast<floatx4 *>(zeros + (XLDS ? 512 : 0));
+
+    // epilogue constants: fetched first so that their latency hides behind the weight stream
+    float sc4[4] = {1.f, 1.f, 1.f, 1.f}, bi4[4] = {0.f, 0.f, 0.f, 0.f};
+    if (wv < G && valid) {
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int64_t n = nb * 16 + g * 4 + r;
+            if (n < N) {
+                if (scale) sc4[r] = scale[n];
+                if (bias) bi4[r] = bias[n];
+            }
+        }
+    }
+
     floatx4 acc[MT];
 #pragma unroll
     for (int t = 0; t < MT; t++) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-    for (int64_t kb = wv; kb < Kb; kb += waves) {
-        const u32x4 wq = __builtin_nontemporal_load(native + (nb * Kb + kb) * 64 + lane);
+    const u32x4 *wbase = native + (valid ? nb * Kb : 0) * 64 + lane;
+    const int nt = valid && Kb > ks ? (Kb - ks + nks - 1) / nks : 0;   // weight blocks of this wavefront
+    u32x4 cur[kAhead];
 #pragma unroll
-        for (int d = 0; d < 4; d++) {
+    for (int u = 0; u < kAhead; u++)
+        if (u < nt) cur[u] = __builtin_nontemporal_load(wbase + (ks + u * nks) * 64);
+
+    // per-lane operand base and block stride (bytes)
+    const unsigned char *xl[MT];
+    int stepb[MT];
+    if constexpr (XLDS) {
+        const int cpr = Kb * (kKB / 8), total = (int)M * cpr;          // 8-element chunks per row, in all
+        for (int id = threadIdx.x; id < total; id += blockDim.x) {
+            const int row = id / cpr, c = id - row * cpr;
+            const XFrag<X32> f = load_x<X32, VEC>(x, row, M, K, (int64_t)c * 8);
+            *reinterpret_cast<half8 *>(smem + (size_t)row * pitch + c * 16) = f.hi;
+            if constexpr (X32) *reinterpret_cast<half8 *>(smem + plane + (size_t)row * pitch + c * 16) = f.lo;
+        }
+        if (threadIdx.x < 32) reinterpret_cast<u32x4 *>(zeros)[threadIdx.x] = u32x4{0u, 0u, 0u, 0u};
 #pragma unroll
-            for (int s = 0; s < 2; s++) {
-                const int64_t k0 = kb * kKB + d * 64 + s * 32;
-                if (k0 >= K) continue;   // wave-uniform
-                const half8 a = decode_step(wq[d], s);
+        for (int t = 0; t < MT; t++) {
+            const int m = t * 16 + j;
+            xl[t] = m < M ? smem + (size_t)m * pitch + g * 16 : zeros + g * 16;
+            stepb[t] = m < M ? kKB * 2 : 0;
+        }
+        __syncthreads();
+    }
+
+    for (int t0 = 0; t0 < nt; t0 += kAhead) {
 #pragma unroll
-                for (int t = 0; t < MT; t++) {
-                    const XFrag<X32> xf = load_x<X32, VEC>(x, t * 16 + j, M, K, k0 + g * 8);
-                    acc[t] = mfma16(a, xf.hi, acc[t]);
-                    if constexpr (X32) acc[t] = mfma16(a, xf.lo, acc[t]);
+        for (int u = 0; u < kAhead; u++) {
+            if (t0 + u < nt) {   // wave-uniform
+                const int kb = ks + (t0 + u) * nks;
+                if constexpr (XLDS) {
+                    const unsigned char *xp[MT];
+#pragma unroll
+                    for (int t = 0; t < MT; t++) xp[t] = xl[t] + kb * stepb[t];
+#pragma unroll
+                    for (int d = 0; d < 4; d++) {
+#pragma unroll
+                        for (int s = 0; s < 2; s++) {
+                            const half8 a = decode_step(cur[u][d], s);
+#pragma unroll
+                            for (int t = 0; t < MT; t++) {
+                                acc[t] = mfma16(a, *reinterpret_cast<const half8 *>(xp[t] + d * 128 + s * 64), acc[t]);
+                                if constexpr (X32) {
+                                    // the zero region serves both terms: stepb == 0 marks such a lane
+                                    const unsigned char *lo = xp[t] + (stepb[t] ? plane : 0);
+                                    acc[t] = mfma16(a, *reinterpret_cast<const half8 *>(lo + d * 128 + s * 64), acc[t]);
+                                }
+                            }
+                        }
+                    }
+                } else {
+#pragma unroll
+                    for (int d = 0; d < 4; d++) {
+#pragma unroll
+                        for (int s = 0; s < 2; s++) {
+                            const int64_t k0 = (int64_t)kb * kKB + d * 64 + s * 32;
+                            if (k0 >= K) continue;   // wave-uniform
+                            const half8 a = decode_step(cur[u][d], s);
+#pragma unroll
+                            for (int t = 0; t < MT; t++) {
+                                const XFrag<X32> xf = load_x<X32, VEC>(x, t * 16 + j, M, K, k0 + g * 8);
+                                acc[t] = mfma16(a, xf.hi, acc[t]);
+                                if constexpr (X32) acc[t] = mfma16(a, xf.lo, acc[t]);
+                            }
+                        }
+                    }
                 }
             }
+            if (t0 + kAhead + u < nt) cur[u] = __builtin_nontemporal_load(wbase + (ks + (t0 + kAhead + u) * nks) * 64);
         }
     }
     // cross-wave reduction in wave order, then epilogue: lane slot (t, lane) holds
     // y[m = 16 t + j][n = 16 nb + 4 g + r], r = 0..3.
-    floatx4 *slot = reinterpret_cast<floatx4 *>(red);
 #pragma unroll
     for (int t = 0; t < MT; t++) slot[(wv * MT + t) * 64 + lane] = acc[t];
     __syncthreads();
-    for (int id = threadIdx.x; id < MT * 64; id += blockDim.x) {
-        const int t = id >> 6, l = id & 63, jj = l & 15, gg = l >> 4;
-        floatx4 s = slot[id];
-        for (int w = 1; w < waves; w++) {
-            const floatx4 p = slot[(w * MT + t) * 64 + l];
-            s[0] += p[0]; s[1] += p[1]; s[2] += p[2]; s[3] += p[3];
-        }
-        const int64_t m = t * 16 + jj, n0 = nb * 16 + gg * 4;
-        if (m >= M) continue;
+    if (wv < G && valid) {
+        for (int t = 0; t < MT; t++) {
+            floatx4 s = slot[(wv * MT + t) * 64 + lane];
+            for (int w = wv + G; w < waves; w += G) {
+                const floatx4 p = slot[(w * MT + t) * 64 + lane];
+                s[0] += p[0]; s[1] += p[1]; s[2] += p[2]; s[3] += p[3];
+            }
+            const int64_t m = t * 16 + j, n0 = nb * 16 + g * 4;
+            if (m >= M) continue;
 #pragma unroll
-        for (int r = 0; r < 4; r++) {
-            const int64_t n = n0 + r;
-            if (n < N) {
-                const float sc = (scale ? scale[n] : 1.0f) * (1.0f / kWeightUnit);
-                float v = s[r] * sc;
-                if (bias) v += bias[n];
-                const int64_t o = m * N + n;
-                if (y_f16) {
-                    if (residual) v += (float)static_cast<const _Float16 *>(residual)[o];
-                    if (relu) v = v > 0.f ? v : 0.f;
-                    static_cast<_Float16 *>(y)[o] = (_Float16)v;
-                } else {
-                    if (residual) v += static_cast<const float *>(residual)[o];
-                    if (relu) v = v > 0.f ? v : 0.f;
-                    static_cast<float *>(y)[o] = v;
+            for (int r = 0; r < 4; r++) {
+                const int64_t n = n0 + r;
+                if (n < N) {
+                    float v = s[r] * (sc4[r] * (1.0f / kWeightUnit)) + bi4[r];
+                    const int64_t o = m * N + n;
+                    if (y_f16) {
+                        if (residual) v += (float)static_cast<const _Float16 *>(residual)[o];
+                        if (relu) v = v > 0.f ? v : 0.f;
+                        static_cast<_Float16 *>(y)[o] = (_Float16)v;
+                    } else {
+                        if (residual) v += static_cast<const float *>(residual)[o];
+                        if (relu) v = v > 0.f ? v : 0.f;
+                        static_cast<float *>(y)[o] = v;
+                    }
                 }
             }
         }
     }
 }
 
-template <int MT, bool X32>
-int launch_skinny(const void *x, int64_t M, int64_t K, const void *native, int64_t N, const tmq_epilogue &ep,
-                  void *y, void *stream) {
+template <int MT, bool X32, bool VEC, bool XLDS>
+int launch_skinny_as(dim3 grid, dim3 block, size_t lds, void *stream, const void *x, int64_t M, int64_t K,
+                     const u32x4 *nat, int Kb, int64_t N, int64_t Nb, int G, const tmq_epilogue &ep, void *y) {
+    auto kernel = skinny_kernel<MT, X32, VEC, XLDS>;
+    if (lds > 64 * 1024) {
+        // opt in to the full 160 KiB of LDS (per device; the attribute is sticky, setting it again is cheap)
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)kSkinnyLdsMax);
+        if (e != hipSuccess) return note_hip_error(e);
+    }
     const float *scale = ep.scale, *bias = ep.bias;
     const void *residual = ep.residual;
     const int relu = ep.relu, y_f16 = ep.y_dtype == TMQ_F16;
-    const int64_t Nb = native_blocks_n(N), Kb = native_blocks_k(K);
-    int waves = 16;
-    while (waves > 1 && (waves > Kb || waves * MT > 32)) waves >>= 1;
-    const size_t lds = (size_t)waves * MT * 64 * sizeof(floatx4);
-    const bool vec = (K % 8 == 0) && aligned16(x);
-    if (Nb > 0x7FFFFFFF) return TMQ_ERR_TOO_LARGE;
-    dim3 grid((uint32_t)Nb), block(64 * waves);
-    const u32x4 *nat = static_cast<const u32x4 *>(native);
-    if (vec)
-        hipLaunchKernelGGL((skinny_kernel<MT, X32, true>), grid, block, lds, as_stream(stream), x, M, K, nat, Kb, N, scale,
-                           bias, residual, relu, y, y_f16);
-    else
-        hipLaunchKernelGGL((skinny_kernel<MT, X32, false>), grid, block, lds, as_stream(stream), x, M, K, nat, Kb, N,
-                           scale, bias, residual, relu, y, y_f16);
+    hipLaunchKernelGGL(kernel, grid, block, lds, as_stream(stream), x, M, K, nat, Kb, N, Nb, G, scale, bias, residual,
+                       relu, y, y_f16);
     return check_launch();
+}
+
+template <int MT, bool X32>
+int launch_skinny(const void *x, int64_t M, int64_t K, const void *native, int64_t N, const tmq_epilogue &ep,
+                  void *y, void *stream) {
+    const int64_t Nb = native_blocks_n(N), Kb = native_blocks_k(K);
+    if (Kb > (1 << 20)) return TMQ_ERR_TOO_LARGE;
+    // Geometry: 16 wavefronts where the reduction slots allow; short reductions give their spare
+    // wavefronts to more channel blocks (G) as long as >= 256 workgroups remain, else shrink.
+    int waves = 16, G = 1;
+    while (waves * MT > 32) waves >>= 1;
+    while (waves / G > Kb && waves / G > 1) {
+        if (Nb >= 512 * (int64_t)G) G <<= 1;
+        else waves >>= 1;
+    }
+    if (G == 1 && waves == 16 && Nb >= 1024 && Kb >= 32) G = 2;   // long streams: halve the staging per byte
+    const size_t red = (size_t)waves * MT * 64 * sizeof(floatx4);
+    const bool vec = (K % 8 == 0) && aligned16(x);
+    const size_t xbytes = (size_t)(X32 ? 2 : 1) * (size_t)M * (size_t)(Kb * kKB + 8) * 2 + 512;
+    const bool xlds = xbytes + red <= kSkinnyLdsMax;
+    const int64_t wgs = (Nb + G - 1) / G;
+    if (wgs > 0x7FFFFFFF) return TMQ_ERR_TOO_LARGE;
+    dim3 grid((uint32_t)wgs), block(64 * waves);
+    const u32x4 *nat = static_cast<const u32x4 *>(native);
+    if (xlds) {
+        if (vec) return launch_skinny_as<MT, X32, true, true>(grid, block, xbytes + red, stream, x, M, K, nat, (int)Kb, N, Nb, G, ep, y);
+        return launch_skinny_as<MT, X32, false, true>(grid, block, xbytes + red, stream, x, M, K, nat, (int)Kb, N, Nb, G, ep, y);
+    }
+    if (vec) return launch_skinny_as<MT, X32, true, false>(grid, block, red, stream, x, M, K, nat, (int)Kb, N, Nb, G, ep, y);
+    return launch_skinny_as<MT, X32, false, false>(grid, block, red, stream, x, M, K, nat, (int)Kb, N, Nb, G, ep, y);
 }
 
 template <bool X32>
