@@ -87,6 +87,35 @@ def test_exactness_on_integers(cuda, oracle):
         assert np.array_equal(y, ref)
 
 
+WIDE = [  # (M, K, N, fp32 activations): wide layers take the register-blocked variants of the skinny kernel
+    (1, 1024, 8192, False), (3, 520, 8200, False), (1, 16384, 16384, False), (1, 16640, 16400, False),
+    (7, 16384, 16464, True), (16, 4096, 16384, False), (2, 33000, 16384, False), (1, 4096, 8192, True),
+]
+
+
+@pytest.mark.parametrize("M,K,N,x32", WIDE)
+def test_wide_layers_exact_on_integers(cuda, M, K, N, x32):
+    """Small-integer activations, power-of-two scales and integer biases: every intermediate is
+    exact in fp32, so the output must equal the integer matrix product bit for bit. The expected
+    value comes from an fp32 library matmul on the expanded weights (exact for the same reason)."""
+    from tmq_amd import ops
+    g = torch.Generator(device=cuda).manual_seed(M + K + N)
+    W = torch.randint(-1, 2, (N, K), dtype=torch.int8, device=cuda, generator=g)
+    x = torch.randint(-8, 9, (M, K), device=cuda, generator=g).float()
+    scale = torch.pow(2.0, torch.randint(-2, 3, (N,), device=cuda, generator=g).float())
+    bias = torch.randint(-50, 51, (N,), device=cuda, generator=g).float()
+    nw = ops.NativeWeights(ops.compactify_ternary(W), N)
+    y = ops.ternary_linear(x if x32 else x.half(), nw, scale, bias)
+    ref = (x @ W.float().T) * scale + bias
+    assert torch.equal(y, ref)
+    # one hot rows pick single weights: catches any permutation between channel blocks
+    e = torch.zeros(2, K, device=cuda)
+    e[0, K - 1] = 1.0
+    e[1, K // 2 + 3] = 1.0
+    ye = ops.ternary_linear(e.half(), nw)
+    assert torch.equal(ye, torch.stack([W[:, K - 1], W[:, K // 2 + 3]]).float())
+
+
 def test_code_11_decodes_to_zero_and_linearity(cuda, oracle):
     from tmq_amd import ops
     rng = np.random.default_rng(5)

@@ -56,15 +56,15 @@ struct XFrag {
     half8 hi, lo;
 };
 
-template <bool X32, bool VEC>
-__device__ __forceinline__ XFrag<X32> load_x(const void *x, int64_t m, int64_t M, int64_t K, int64_t k) {
+template <bool X32>
+__device__ __forceinline__ XFrag<X32> load_x(const void *x, int64_t m, int64_t M, int64_t K, int64_t k, bool vec) {
     XFrag<X32> f;
     f.hi = half8{0, 0, 0, 0, 0, 0, 0, 0};
     f.lo = f.hi;
     if (m >= M || k >= K) return f;
     if constexpr (!X32) {
         const _Float16 *p = static_cast<const _Float16 *>(x) + m * K + k;
-        if (VEC && k + 8 <= K) {
+        if (vec && k + 8 <= K) {
             f.hi = *reinterpret_cast<const half8 *>(p);
         } else {
 #pragma unroll
@@ -74,7 +74,7 @@ __device__ __forceinline__ XFrag<X32> load_x(const void *x, int64_t m, int64_t M
     } else {
         const float *p = static_cast<const float *>(x) + m * K + k;
         float v[8];
-        if (VEC && k + 8 <= K) {
+        if (vec && k + 8 <= K) {
             floatx4 a = *reinterpret_cast<const floatx4 *>(p), b = *reinterpret_cast<const floatx4 *>(p + 4);
 #pragma unroll
             for (int e = 0; e < 4; e++) { v[e] = a[e]; v[4 + e] = b[e]; }
@@ -93,45 +93,48 @@ __device__ __forceinline__ XFrag<X32> load_x(const void *x, int64_t m, int64_t M
 }
 
 // ---- skinny kernel --------------------------------------------------------------------------------
-// grid.x = ceil(Nb / G) workgroups of `waves` wavefronts; a workgroup owns G consecutive blocks of 16
-// output channels. Wavefront w works on channel block (w % G) and on the weight blocks
-// kb = w / G, w / G + waves / G, ... of it. MT = number of 16-row activation tiles (M <= 16 MT).
-// D[n][m]: the weights are the A operand of the MFMA.
+// A workgroup of `waves` wavefronts owns GW consecutive blocks of 16 output channels. Wavefront w
+// works on channel block (w % GW) and, of it, on the weight blocks kb = w / GW, w / GW + waves / GW,
+// ... MT = number of 16-row activation tiles (M <= 16 MT). D[n][m]: the weights are the A operand of
+// the MFMA.
 //
-// The kernel is a weight stream; what counts is the number of bytes in flight and the VALU work
-// per byte. Every wavefront keeps kAhead 1 KiB weight blocks outstanding in a rolling pipeline (a
-// register is reloaded as soon as its block has been consumed). XLDS: the activations are staged
-// once per workgroup in LDS -- fp32 activations already split into their two fp16 terms -- padded
-// with zeros to whole weight blocks, so that the inner loop has no edge handling at all: an operand
-// read is one ds_read_b128 at (lane base + block offset + immediate). Lanes whose activation row
-// does not exist (m >= M) read from a 512-byte zero region with a block stride of 0.
-constexpr int kAhead = 4;
+// The kernel is a weight stream; besides HBM two things bound it:
+//   * bytes in flight: every wavefront keeps kAhead 1 KiB blocks outstanding in a rolling pipeline
+//     (a block's registers are reloaded as soon as it has been consumed);
+//   * VALU: two operations per operand register to expand the 2-bit codes -- nothing else is left
+//     in the inner loop. XLDS: the activations are staged once per workgroup in LDS, fp32
+//     activations already split into their two fp16 terms, zero-padded to whole weight blocks, so an
+//     operand read is one ds_read_b128 at (lane base + block offset + immediate) with no edge cases.
+// Lanes whose activation row does not exist (m >= M) read row M - 1: columns of D are independent,
+// and those columns are never stored.
 constexpr size_t kSkinnyLdsMax = 152 * 1024;
+constexpr int kAhead = 4;
 
-template <int MT, bool X32, bool VEC, bool XLDS>
-__global__ __launch_bounds__(1024) void skinny_kernel(const void *__restrict__ x, int64_t M, int64_t K,
+template <int MT, bool X32, bool XLDS>
+__global__ __launch_bounds__(1024) void skinny_kernel(const void *__restrict__ x, int64_t M, int64_t K, int vec,
                                                       const u32x4 *__restrict__ native, int Kb, int64_t N, int64_t Nb,
-                                                      int G, const float *__restrict__ scale,
+                                                      int GW, const float *__restrict__ scale,
                                                       const float *__restrict__ bias, const void *__restrict__ residual,
                                                       int relu, void *__restrict__ y, int y_f16) {
-    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6, waves = blockDim.x >> 6;
-    const int j = lane & 15, g = lane >> 4;
-    const int sub = wv % G, ks = wv / G, nks = waves / G;
-    const int64_t nb = (int64_t)blockIdx.x * G + sub;
-    const bool valid = nb < Nb;
     constexpr int kPlanes = X32 ? 2 : 1;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    // the wavefront index is uniform: telling the compiler keeps the loop control in scalar registers
+    const int lane = threadIdx.x & 63, wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), waves = blockDim.x >> 6;
+    const int j = lane & 15, g = lane >> 4;
+    const int sub = wv % GW, ks = wv / GW, nks = waves / GW;
+    const int64_t nb0 = (int64_t)blockIdx.x * GW + sub;
+    const bool valid = nb0 < Nb;
     const int pitch = (Kb * kKB + 8) * 2;                              // bytes per staged activation row
     const size_t plane = (size_t)M * pitch;
-    unsigned char *zeros = smem + (XLDS ? kPlanes * plane : 0);
-    floatx4 *slot = reinterpret_cast<floatx4 *>(zeros + (XLDS ? 512 : 0));
+    floatx4 *slot = reinterpret_cast<floatx4 *>(smem + (XLDS ? kPlanes * plane : 0));
 
-    // epilogue constants: fetched first so that their latency hides behind the weight stream
+    // The first GW wavefronts run the epilogue of one channel block each; its constants are fetched
+    // now so that their latency hides behind the weight stream.
     float sc4[4] = {1.f, 1.f, 1.f, 1.f}, bi4[4] = {0.f, 0.f, 0.f, 0.f};
-    if (wv < G && valid) {
+    if (wv < GW && valid) {
 #pragma unroll
         for (int r = 0; r < 4; r++) {
-            const int64_t n = nb * 16 + g * 4 + r;
+            const int64_t n = nb0 * 16 + g * 4 + r;
             if (n < N) {
                 if (scale) sc4[r] = scale[n];
                 if (bias) bi4[r] = bias[n];
@@ -143,89 +146,122 @@ __global__ __launch_bounds__(1024) void skinny_kernel(const void *__restrict__ x
 #pragma unroll
     for (int t = 0; t < MT; t++) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-    const u32x4 *wbase = native + (valid ? nb * Kb : 0) * 64 + lane;
+    const u32x4 *wb = native + (valid ? nb0 * Kb : 0) * 64 + lane;
     const int nt = valid && Kb > ks ? (Kb - ks + nks - 1) / nks : 0;   // weight blocks of this wavefront
-    u32x4 cur[kAhead];
-#pragma unroll
-    for (int u = 0; u < kAhead; u++)
-        if (u < nt) cur[u] = __builtin_nontemporal_load(wbase + (ks + u * nks) * 64);
 
-    // per-lane operand base and block stride (bytes)
+    // Prologue loads. A long stream issues them unconditionally: only then can the compiler count the
+    // loads behind the one it waits for in the steady-state loop below.
+    u32x4 cur[kAhead];
+    auto fetch = [&](int u, int t) { cur[u] = __builtin_nontemporal_load(wb + (ks + t * nks) * 64); };
+    const bool steady = nt >= 2 * kAhead;
+    if (steady) {
+#pragma unroll
+        for (int u = 0; u < kAhead; u++) fetch(u, u);
+    } else {
+#pragma unroll
+        for (int u = 0; u < kAhead; u++)
+            if (u < nt) fetch(u, u);
+    }
+
+    // per-lane operand base (row m, or the last row for lanes past M)
     const unsigned char *xl[MT];
-    int stepb[MT];
     if constexpr (XLDS) {
         const int cpr = Kb * (kKB / 8), total = (int)M * cpr;          // 8-element chunks per row, in all
         for (int id = threadIdx.x; id < total; id += blockDim.x) {
             const int row = id / cpr, c = id - row * cpr;
-            const XFrag<X32> f = load_x<X32, VEC>(x, row, M, K, (int64_t)c * 8);
+            const XFrag<X32> f = load_x<X32>(x, row, M, K, (int64_t)c * 8, vec);
             *reinterpret_cast<half8 *>(smem + (size_t)row * pitch + c * 16) = f.hi;
             if constexpr (X32) *reinterpret_cast<half8 *>(smem + plane + (size_t)row * pitch + c * 16) = f.lo;
         }
-        if (threadIdx.x < 32) reinterpret_cast<u32x4 *>(zeros)[threadIdx.x] = u32x4{0u, 0u, 0u, 0u};
 #pragma unroll
         for (int t = 0; t < MT; t++) {
             const int m = t * 16 + j;
-            xl[t] = m < M ? smem + (size_t)m * pitch + g * 16 : zeros + g * 16;
-            stepb[t] = m < M ? kKB * 2 : 0;
+            xl[t] = smem + (size_t)(m < M ? m : (int)M - 1) * pitch + g * 16;
         }
         __syncthreads();
     }
 
-    for (int t0 = 0; t0 < nt; t0 += kAhead) {
+    // One weight block against the activations: 8 MFMA steps of 32 reduction indices.
+    auto contract = [&](const u32x4 &wq, int kb) {
+        if constexpr (XLDS && MT == 1) {
+            // all operand reads of the block are issued ahead of the decode work
+            const unsigned char *xp = xl[0] + kb * (kKB * 2);
+            half8 xv[8], xw[X32 ? 8 : 1];
 #pragma unroll
-        for (int u = 0; u < kAhead; u++) {
-            if (t0 + u < nt) {   // wave-uniform
-                const int kb = ks + (t0 + u) * nks;
-                if constexpr (XLDS) {
-                    const unsigned char *xp[MT];
+            for (int i = 0; i < 8; i++) {
+                xv[i] = *reinterpret_cast<const half8 *>(xp + i * 64);
+                if constexpr (X32) xw[i] = *reinterpret_cast<const half8 *>(xp + plane + i * 64);
+            }
 #pragma unroll
-                    for (int t = 0; t < MT; t++) xp[t] = xl[t] + kb * stepb[t];
+            for (int i = 0; i < 8; i++) {
+                const half8 a = decode_step(wq[i >> 1], i & 1);
+                acc[0] = mfma16(a, xv[i], acc[0]);
+                if constexpr (X32) acc[0] = mfma16(a, xw[i], acc[0]);
+            }
+        } else if constexpr (XLDS) {
 #pragma unroll
-                    for (int d = 0; d < 4; d++) {
+            for (int i = 0; i < 8; i++) {
+                const half8 a = decode_step(wq[i >> 1], i & 1);
 #pragma unroll
-                        for (int s = 0; s < 2; s++) {
-                            const half8 a = decode_step(cur[u][d], s);
-#pragma unroll
-                            for (int t = 0; t < MT; t++) {
-                                acc[t] = mfma16(a, *reinterpret_cast<const half8 *>(xp[t] + d * 128 + s * 64), acc[t]);
-                                if constexpr (X32) {
-                                    // the zero region serves both terms: stepb == 0 marks such a lane
-                                    const unsigned char *lo = xp[t] + (stepb[t] ? plane : 0);
-                                    acc[t] = mfma16(a, *reinterpret_cast<const half8 *>(lo + d * 128 + s * 64), acc[t]);
-                                }
-                            }
-                        }
-                    }
-                } else {
-#pragma unroll
-                    for (int d = 0; d < 4; d++) {
-#pragma unroll
-                        for (int s = 0; s < 2; s++) {
-                            const int64_t k0 = (int64_t)kb * kKB + d * 64 + s * 32;
-                            if (k0 >= K) continue;   // wave-uniform
-                            const half8 a = decode_step(cur[u][d], s);
-#pragma unroll
-                            for (int t = 0; t < MT; t++) {
-                                const XFrag<X32> xf = load_x<X32, VEC>(x, t * 16 + j, M, K, k0 + g * 8);
-                                acc[t] = mfma16(a, xf.hi, acc[t]);
-                                if constexpr (X32) acc[t] = mfma16(a, xf.lo, acc[t]);
-                            }
-                        }
-                    }
+                for (int t = 0; t < MT; t++) {
+                    const unsigned char *xp = xl[t] + kb * (kKB * 2) + i * 64;
+                    acc[t] = mfma16(a, *reinterpret_cast<const half8 *>(xp), acc[t]);
+                    if constexpr (X32) acc[t] = mfma16(a, *reinterpret_cast<const half8 *>(xp + plane), acc[t]);
                 }
             }
-            if (t0 + kAhead + u < nt) cur[u] = __builtin_nontemporal_load(wbase + (ks + (t0 + kAhead + u) * nks) * 64);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const int64_t k0 = (int64_t)kb * kKB + i * 32;
+                if (k0 >= K) continue;   // wave-uniform
+                const half8 a = decode_step(wq[i >> 1], i & 1);
+#pragma unroll
+                for (int t = 0; t < MT; t++) {
+                    const XFrag<X32> xf = load_x<X32>(x, t * 16 + j, M, K, k0 + g * 8, vec);
+                    acc[t] = mfma16(a, xf.hi, acc[t]);
+                    if constexpr (X32) acc[t] = mfma16(a, xf.lo, acc[t]);
+                }
+            }
+        }
+    };
+
+    // Steady state: every slot is consumed and refilled unconditionally, so the number of loads
+    // behind the one being waited for is known at compile time.
+    int t0 = 0;
+    if (steady) {
+        // Start from a known state (nothing outstanding): paths that skipped the staging waits above
+        // would otherwise make the compiler wait for every load at the loop header.
+        __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
+        do {
+#pragma unroll
+            for (int u = 0; u < kAhead; u++) {
+                contract(cur[u], ks + (t0 + u) * nks);
+                __builtin_amdgcn_sched_barrier(0);   // keep the refill here, not batched at the loop end
+                fetch(u, t0 + kAhead + u);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            t0 += kAhead;
+        } while (t0 + 2 * kAhead <= nt);
+    }
+    // Drain: at most two rounds with wave-uniform guards.
+    for (; t0 < nt; t0 += kAhead) {
+#pragma unroll
+        for (int u = 0; u < kAhead; u++) {
+            if (t0 + u < nt) contract(cur[u], ks + (t0 + u) * nks);
+            if (t0 + kAhead + u < nt) fetch(u, t0 + kAhead + u);
         }
     }
-    // cross-wave reduction in wave order, then epilogue: lane slot (t, lane) holds
-    // y[m = 16 t + j][n = 16 nb + 4 g + r], r = 0..3.
+
+    // Cross-wave reduction in wave order, then the epilogue. Lane slot (w, t, lane) holds
+    // y[m = 16 t + j][n = 16 nb + 4 g + r], r = 0..3, of wavefront w's channel block.
 #pragma unroll
     for (int t = 0; t < MT; t++) slot[(wv * MT + t) * 64 + lane] = acc[t];
     __syncthreads();
-    if (wv < G && valid) {
+    if (wv < GW && valid) {
+        const int64_t nb = nb0;
         for (int t = 0; t < MT; t++) {
             floatx4 s = slot[(wv * MT + t) * 64 + lane];
-            for (int w = wv + G; w < waves; w += G) {
+            for (int w = wv + GW; w < waves; w += GW) {
                 const floatx4 p = slot[(w * MT + t) * 64 + lane];
                 s[0] += p[0]; s[1] += p[1]; s[2] += p[2]; s[3] += p[3];
             }
@@ -252,21 +288,33 @@ __global__ __launch_bounds__(1024) void skinny_kernel(const void *__restrict__ x
     }
 }
 
-template <int MT, bool X32, bool VEC, bool XLDS>
-int launch_skinny_as(dim3 grid, dim3 block, size_t lds, void *stream, const void *x, int64_t M, int64_t K,
-                     const u32x4 *nat, int Kb, int64_t N, int64_t Nb, int G, const tmq_epilogue &ep, void *y) {
-    auto kernel = skinny_kernel<MT, X32, VEC, XLDS>;
+struct SkinnyArgs {
+    const void *x;
+    int64_t M, K;
+    int vec;
+    const u32x4 *native;
+    int Kb;
+    int64_t N, Nb;
+    int GW;
+    const tmq_epilogue *ep;
+    void *y;
+};
+
+template <int MT, bool X32, bool XLDS>
+int launch_skinny_as(dim3 grid, dim3 block, size_t lds, void *stream, const SkinnyArgs &a) {
+    auto kernel = skinny_kernel<MT, X32, XLDS>;
     if (lds > 64 * 1024) {
-        // opt in to the full 160 KiB of LDS (per device; the attribute is sticky, setting it again is cheap)
+        // opt in to the large LDS (per device; the attribute is sticky, setting it again is cheap)
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)kSkinnyLdsMax);
         if (e != hipSuccess) return note_hip_error(e);
     }
+    const tmq_epilogue &ep = *a.ep;
     const float *scale = ep.scale, *bias = ep.bias;
     const void *residual = ep.residual;
     const int relu = ep.relu, y_f16 = ep.y_dtype == TMQ_F16;
-    hipLaunchKernelGGL(kernel, grid, block, lds, as_stream(stream), x, M, K, nat, Kb, N, Nb, G, scale, bias, residual,
-                       relu, y, y_f16);
+    hipLaunchKernelGGL(kernel, grid, block, lds, as_stream(stream), a.x, a.M, a.K, a.vec, a.native, a.Kb, a.N, a.Nb,
+                       a.GW, scale, bias, residual, relu, a.y, y_f16);
     return check_launch();
 }
 
@@ -276,28 +324,27 @@ int launch_skinny(const void *x, int64_t M, int64_t K, const void *native, int64
     const int64_t Nb = native_blocks_n(N), Kb = native_blocks_k(K);
     if (Kb > (1 << 20)) return TMQ_ERR_TOO_LARGE;
     // Geometry: 16 wavefronts where the reduction slots allow; short reductions give their spare
-    // wavefronts to more channel blocks (G) as long as >= 256 workgroups remain, else shrink.
-    int waves = 16, G = 1;
+    // wavefronts to more channel blocks (GW) as long as >= 256 workgroups remain, else shrink.
+    int waves = 16, GW = 1;
     while (waves * MT > 32) waves >>= 1;
-    while (waves / G > Kb && waves / G > 1) {
-        if (Nb >= 512 * (int64_t)G) G <<= 1;
+    while (waves / GW > Kb && waves / GW > 1) {
+        if (Nb >= 512 * (int64_t)GW) GW <<= 1;
         else waves >>= 1;
     }
-    if (G == 1 && waves == 16 && Nb >= 1024 && Kb >= 32) G = 2;   // long streams: halve the staging per byte
+    const size_t xbytes = (size_t)(X32 ? 2 : 1) * (size_t)M * (size_t)(Kb * kKB + 8) * 2;
+    const bool xlds = xbytes + (size_t)waves * MT * 64 * sizeof(floatx4) <= kSkinnyLdsMax;
+    // Wide single-tile layers: half-size workgroups that own two channel blocks each. Several of
+    // them fit a CU, so one group's staging and reduction overlap another's streaming (measured best
+    // among {4, 8, 16} wavefronts x {1, 2, 4} blocks at 8192^2 .. 32768 x 16384), and each group
+    // stages the activations for twice the weights.
+    if (MT == 1 && xlds && waves == 16 && GW == 1 && Nb >= 512 && Kb >= 32) { waves = 8; GW = 2; }
     const size_t red = (size_t)waves * MT * 64 * sizeof(floatx4);
-    const bool vec = (K % 8 == 0) && aligned16(x);
-    const size_t xbytes = (size_t)(X32 ? 2 : 1) * (size_t)M * (size_t)(Kb * kKB + 8) * 2 + 512;
-    const bool xlds = xbytes + red <= kSkinnyLdsMax;
-    const int64_t wgs = (Nb + G - 1) / G;
+    const int64_t wgs = (Nb + GW - 1) / GW;
     if (wgs > 0x7FFFFFFF) return TMQ_ERR_TOO_LARGE;
     dim3 grid((uint32_t)wgs), block(64 * waves);
-    const u32x4 *nat = static_cast<const u32x4 *>(native);
-    if (xlds) {
-        if (vec) return launch_skinny_as<MT, X32, true, true>(grid, block, xbytes + red, stream, x, M, K, nat, (int)Kb, N, Nb, G, ep, y);
-        return launch_skinny_as<MT, X32, false, true>(grid, block, xbytes + red, stream, x, M, K, nat, (int)Kb, N, Nb, G, ep, y);
-    }
-    if (vec) return launch_skinny_as<MT, X32, true, false>(grid, block, red, stream, x, M, K, nat, (int)Kb, N, Nb, G, ep, y);
-    return launch_skinny_as<MT, X32, false, false>(grid, block, red, stream, x, M, K, nat, (int)Kb, N, Nb, G, ep, y);
+    const SkinnyArgs a{x, M, K, (K % 8 == 0) && aligned16(x), static_cast<const u32x4 *>(native), (int)Kb, N, Nb, GW, &ep, y};
+    if (!xlds) return launch_skinny_as<MT, X32, false>(grid, block, red, stream, a);
+    return launch_skinny_as<MT, X32, true>(grid, block, xbytes + red, stream, a);
 }
 
 template <bool X32>
