@@ -93,7 +93,14 @@ WIDE = [  # (M, K, N, fp32 activations): wide layers take the register-blocked v
 ]
 
 
-@pytest.mark.parametrize("M,K,N,x32", WIDE)
+MID = [  # batches between the skinny kernel and the big-tile kernel, both activation types
+    (65, 4096, 4096, False), (256, 4096, 4096, False), (256, 4096, 4096, True), (128, 4096, 4096, False),
+    (100, 1000, 4100, False), (777, 2304, 520, False), (300, 4096, 96, True), (1024, 1024, 1024, False),
+    (2048, 512, 4096, False), (96, 8192, 2048, True), (65, 264, 40, False), (513, 4096, 1000, True),
+]
+
+
+@pytest.mark.parametrize("M,K,N,x32", WIDE + MID)
 def test_wide_layers_exact_on_integers(cuda, M, K, N, x32):
     """Small-integer activations, power-of-two scales and integer biases: every intermediate is
     exact in fp32, so the output must equal the integer matrix product bit for bit. The expected

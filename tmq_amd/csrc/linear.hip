@@ -358,6 +358,443 @@ int skinny_rows(const void *x, int64_t M, int64_t K, const void *native, int64_t
     }
 }
 
+// ---- mid kernel -----------------------------------------------------------------------------------
+// Batches between the skinny case and the big-tile GEMM (64 < M <~ 2048): too few output tiles to
+// fill 256 CUs with large tiles, too many rows to stage in LDS. A workgroup of 16 wavefronts owns a
+// (16 WM WGM) x (16 WN) output tile and splits the reduction over its wavefronts: wavefront
+// (wgm, kg) multiplies rows [16 WM wgm, +16 WM) by the weight blocks kb = kg, kg + KG, ...
+// (KG = 16 / WGM). Both operands come straight from global memory -- the weights as whole 1 KiB
+// native blocks (one coalesced dwordx4 per block), the activations as 16-byte row pieces two MFMA
+// steps ahead of their use -- and the partial tiles are summed through LDS in a fixed order, so the
+// result does not depend on scheduling. No activation byte is read twice by a workgroup.
+//
+// FAST: K is a multiple of 256 and rows are 16-byte aligned (no edge handling in the loop; rows past
+// M are clamped to the last row, their columns of D are never stored).
+template <int WM, int WN, int WGM, int WAVES, int D, bool X32, bool FAST>
+__global__ __launch_bounds__(64 * WAVES) void mid_kernel(const void *__restrict__ x, int64_t M, int64_t K,
+                                                   const u32x4 *__restrict__ native, int Kb, int64_t N, int64_t Nb,
+                                                   int tiles_n, const float *__restrict__ scale,
+                                                   const float *__restrict__ bias, const void *__restrict__ residual,
+                                                   int relu, void *__restrict__ y, int y_f16) {
+    constexpr int KG = WAVES / WGM, NF = WM * WN;
+    static_assert(8 % D == 0, "the window must divide a weight block");
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    floatx4 *red = reinterpret_cast<floatx4 *>(smem);
+    const int lane = threadIdx.x & 63, wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int j = lane & 15, g = lane >> 4;
+    const int wgm = wv % WGM, kg = wv / WGM;
+    const int tm = blockIdx.x / tiles_n, tn = blockIdx.x % tiles_n;
+    const int64_t mw = ((int64_t)tm * WGM + wgm) * (16 * WM);      // first row of this wavefront
+    const int64_t n0 = (int64_t)tn * (16 * WN);
+
+    // epilogue constants of the first fragment this wavefront finalises (fragment kg), fetched early
+    float sc4[4] = {1.f, 1.f, 1.f, 1.f}, bi4[4] = {0.f, 0.f, 0.f, 0.f};
+    auto load_consts = [&](int f) {
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int64_t n = n0 + (f % WN) * 16 + g * 4 + r;
+            sc4[r] = (n < N && scale) ? scale[n] : 1.f;
+            bi4[r] = (n < N && bias) ? bias[n] : 0.f;
+        }
+    };
+    if (kg < NF) load_consts(kg);
+
+    floatx4 acc[WM][WN];
+#pragma unroll
+    for (int mi = 0; mi < WM; mi++)
+#pragma unroll
+        for (int nj = 0; nj < WN; nj++) acc[mi][nj] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+    const u32x4 *wb[WN];
+#pragma unroll
+    for (int nj = 0; nj < WN; nj++) {
+        int64_t nb = n0 / 16 + nj;
+        if (nb >= Nb) nb = Nb - 1;                                  // finite bits, never stored
+        wb[nj] = native + (nb * Kb) * 64 + lane;
+    }
+    int64_t xoff[WM];                                               // element offset of the lane's row piece
+#pragma unroll
+    for (int mi = 0; mi < WM; mi++) {
+        int64_t m = mw + mi * 16 + j;
+        if (m >= M) m = M - 1;
+        xoff[mi] = m * K + g * 8;
+    }
+    const int nt = Kb > kg ? (Kb - kg + KG - 1) / KG : 0;           // weight blocks of this wavefront
+
+    // activation window: raw 16 (fp16) or 32 (fp32) bytes per fragment, D steps ahead
+    u32x4 xa[D][WM], xb[X32 ? D : 1][X32 ? WM : 1];
+    auto issue = [&](int slot, int s) {
+        const int64_t k0 = (int64_t)(kg + (s >> 3) * KG) * kKB + (s & 7) * 32;
+#pragma unroll
+        for (int mi = 0; mi < WM; mi++) {
+            if constexpr (FAST) {
+                if constexpr (X32) {
+                    const float *p = static_cast<const float *>(x) + xoff[mi] + k0;
+                    xa[slot][mi] = *reinterpret_cast<const u32x4 *>(p);
+                    xb[slot][mi] = *reinterpret_cast<const u32x4 *>(p + 4);
+                } else {
+                    xa[slot][mi] = *reinterpret_cast<const u32x4 *>(static_cast<const _Float16 *>(x) + xoff[mi] + k0);
+                }
+            } else {
+                int64_t m = mw + mi * 16 + j;
+                if (m >= M) m = M - 1;
+                const XFrag<X32> f = load_x<X32>(x, m, M, K, k0 + g * 8, false);
+                xa[slot][mi] = __builtin_bit_cast(u32x4, f.hi);
+                if constexpr (X32) xb[slot][mi] = __builtin_bit_cast(u32x4, f.lo);
+            }
+        }
+    };
+    auto consume = [&](int slot, const u32x4 (&wq)[WN], int i) {
+        half8 hi[WM], lo[X32 ? WM : 1];
+#pragma unroll
+        for (int mi = 0; mi < WM; mi++) {
+            if constexpr (X32 && FAST) {
+                const floatx4 a = __builtin_bit_cast(floatx4, xa[slot][mi]), b = __builtin_bit_cast(floatx4, xb[slot][mi]);
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    const float v = e < 4 ? a[e] : b[e - 4];
+                    const _Float16 h = (_Float16)v;
+                    hi[mi][e] = h;
+                    lo[mi][e] = (_Float16)(v - (float)h);
+                }
+            } else {
+                hi[mi] = __builtin_bit_cast(half8, xa[slot][mi]);
+                if constexpr (X32) lo[mi] = __builtin_bit_cast(half8, xb[slot][mi]);
+            }
+        }
+#pragma unroll
+        for (int nj = 0; nj < WN; nj++) {
+            const half8 a = decode_step(wq[nj][i >> 1], i & 1);
+#pragma unroll
+            for (int mi = 0; mi < WM; mi++) {
+                acc[mi][nj] = mfma16(a, hi[mi], acc[mi][nj]);
+                if constexpr (X32) acc[mi][nj] = mfma16(a, lo[mi], acc[mi][nj]);
+            }
+        }
+    };
+
+    if (nt > 0) {
+        u32x4 wq[WN], wn[WN];
+#pragma unroll
+        for (int nj = 0; nj < WN; nj++) wq[nj] = __builtin_nontemporal_load(wb[nj] + kg * 64);
+#pragma unroll
+        for (int d = 0; d < D; d++) issue(d, d);
+        for (int t = 0; t + 1 < nt; t++) {
+#pragma unroll
+            for (int nj = 0; nj < WN; nj++) wn[nj] = __builtin_nontemporal_load(wb[nj] + (kg + (t + 1) * KG) * 64);
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                consume(i % D, wq, i);
+                issue(i % D, t * 8 + i + D);
+            }
+#pragma unroll
+            for (int nj = 0; nj < WN; nj++) wq[nj] = wn[nj];
+        }
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            consume(i % D, wq, i);
+            if (i + D < 8) issue(i % D, (nt - 1) * 8 + i + D);
+        }
+    }
+
+    // Sum the KG partial tiles in wavefront order; fragment f = (mi, nj) of row group wgm is finalised
+    // by wavefront (wgm, kg = f mod KG). Lane (j, g) of a fragment holds y[16 mi + j][16 nj + 4 g + r].
+#pragma unroll
+    for (int mi = 0; mi < WM; mi++)
+#pragma unroll
+        for (int nj = 0; nj < WN; nj++) red[(wv * NF + mi * WN + nj) * 64 + lane] = acc[mi][nj];
+    __syncthreads();
+    for (int f = kg; f < NF; f += KG) {
+        if (f != kg) load_consts(f);
+        floatx4 s = red[(wgm * NF + f) * 64 + lane];
+        for (int q = 1; q < KG; q++) {
+            const floatx4 p = red[((q * WGM + wgm) * NF + f) * 64 + lane];
+            s[0] += p[0]; s[1] += p[1]; s[2] += p[2]; s[3] += p[3];
+        }
+        const int64_t m = mw + (f / WN) * 16 + j, nq = n0 + (f % WN) * 16 + g * 4;
+        if (m >= M) continue;
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int64_t n = nq + r;
+            if (n < N) {
+                float v = s[r] * (sc4[r] * (1.0f / kWeightUnit)) + bi4[r];
+                const int64_t o = m * N + n;
+                if (y_f16) {
+                    if (residual) v += (float)static_cast<const _Float16 *>(residual)[o];
+                    if (relu) v = v > 0.f ? v : 0.f;
+                    static_cast<_Float16 *>(y)[o] = (_Float16)v;
+                } else {
+                    if (residual) v += static_cast<const float *>(residual)[o];
+                    if (relu) v = v > 0.f ? v : 0.f;
+                    static_cast<float *>(y)[o] = v;
+                }
+            }
+        }
+    }
+}
+
+template <int WM, int WN, int WGM, int WAVES, int D, bool X32>
+int launch_mid(const void *x, int64_t M, int64_t K, const void *native, int64_t N, const tmq_epilogue &ep, void *y,
+               void *stream) {
+    constexpr int BM = 16 * WM * WGM, BN = 16 * WN;
+    const int64_t tm = (M + BM - 1) / BM, tn = (N + BN - 1) / BN, Kb = native_blocks_k(K);
+    if (tm * tn > 0x7FFFFFFF || Kb > (1 << 20)) return TMQ_ERR_TOO_LARGE;
+    const size_t lds = (size_t)WAVES * WM * WN * 64 * sizeof(floatx4);
+    const bool fast = (K % kKB == 0) && aligned16(x);
+    const float *scale = ep.scale, *bias = ep.bias;
+    const void *residual = ep.residual;
+    const int relu = ep.relu, y_f16 = ep.y_dtype == TMQ_F16;
+    auto go = [&](auto kernel) -> int {
+        if (lds > 64 * 1024) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            if (e != hipSuccess) return note_hip_error(e);
+        }
+        hipLaunchKernelGGL(kernel, dim3((uint32_t)(tm * tn)), dim3(64 * WAVES), lds, as_stream(stream), x, M, K,
+                           static_cast<const u32x4 *>(native), (int)Kb, N, native_blocks_n(N), (int)tn, scale, bias,
+                           residual, relu, y, y_f16);
+        return check_launch();
+    };
+    if (fast) return go(mid_kernel<WM, WN, WGM, WAVES, D, X32, true>);
+    return go(mid_kernel<WM, WN, WGM, WAVES, D, X32, false>);
+}
+
+// ---- mid kernel, staged -----------------------------------------------------------------------------
+// Same work split as mid_kernel with WGM = 1 (every wavefront owns the whole (16 WM) x (16 WN) tile
+// for its share of the reduction), but the activations take the detour an MFMA operand needs: a
+// lane wants 16 bytes of row (lane % 16), and 16 neighbouring lanes reading 16 different rows cost
+// the texture path a cache-line access each. Here a wavefront loads whole 128-byte row pieces (8
+// lanes per row), writes them to a private LDS window and reads them back in operand order. The
+// window belongs to one wavefront, so the loop has no workgroup barrier: LDS operations of a
+// wavefront execute in order, a wave barrier keeps the compiler from reordering them.
+//
+// Unit of the pipeline: a "pair" = 64 reduction indices = one dword of every native weight block =
+// two MFMA steps. While pair p is multiplied, pair p + 1 already sits in the other LDS slot and
+// pairs p + 2, p + 3 are in flight from global memory into registers.
+// Requires K % 256 == 0 and 16-byte aligned rows. fp32 activations are split into their two fp16
+// terms when they are written to LDS.
+template <int WM, int WN, int WAVES, bool X32>
+__global__ __launch_bounds__(64 * WAVES) void mid_lds_kernel(const void *__restrict__ x, int64_t M, int64_t K,
+                                                             const u32x4 *__restrict__ native, int Kb, int64_t N,
+                                                             int64_t Nb, int tiles_n, const float *__restrict__ scale,
+                                                             const float *__restrict__ bias,
+                                                             const void *__restrict__ residual, int relu,
+                                                             void *__restrict__ y, int y_f16) {
+    constexpr int NF = WM * WN, kPlanes = X32 ? 2 : 1;
+    constexpr int kRow = 144;                                  // LDS bytes per 64-index row piece (+16: conflict-free reads)
+    constexpr int kFrag = 16 * kRow, kSlot = kPlanes * WM * kFrag, kWave = 2 * kSlot;
+    constexpr int NL = X32 ? 4 : 2;                            // 1 KiB global loads per fragment and pair
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    floatx4 *red = reinterpret_cast<floatx4 *>(smem);
+    const int lane = threadIdx.x & 63, kg = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int j = lane & 15, g = lane >> 4;
+    unsigned char *win = smem + kg * kWave;
+    const int tm = blockIdx.x / tiles_n, tn = blockIdx.x % tiles_n;
+    const int64_t m0 = (int64_t)tm * (16 * WM), n0 = (int64_t)tn * (16 * WN);
+
+    float sc4[4] = {1.f, 1.f, 1.f, 1.f}, bi4[4] = {0.f, 0.f, 0.f, 0.f};
+    auto load_consts = [&](int f) {
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int64_t n = n0 + (f % WN) * 16 + g * 4 + r;
+            sc4[r] = (n < N && scale) ? scale[n] : 1.f;
+            bi4[r] = (n < N && bias) ? bias[n] : 0.f;
+        }
+    };
+
+    floatx4 acc[WM][WN];
+#pragma unroll
+    for (int mi = 0; mi < WM; mi++)
+#pragma unroll
+        for (int nj = 0; nj < WN; nj++) acc[mi][nj] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+    const uint32_t *wb[WN];                                       // dword d of block kb: wb[nj][kb * 256 + d]
+#pragma unroll
+    for (int nj = 0; nj < WN; nj++) {
+        int64_t nb = n0 / 16 + nj;
+        if (nb >= Nb) nb = Nb - 1;                                  // finite bits, never stored
+        wb[nj] = reinterpret_cast<const uint32_t *>(native + (nb * Kb) * 64 + lane);
+    }
+    // global side: load c of a fragment covers rows [c * 16 / NL, +16 / NL), whole row pieces;
+    // 32-bit byte offsets from x (the host checks that the matrix is smaller than 4 GiB)
+    constexpr int kLanesPerRow = 64 * NL / 16;                     // 8 (fp16) or 16 (fp32)
+    const int lrow = lane / kLanesPerRow, lchunk = lane % kLanesPerRow;
+    uint32_t goff[WM][NL];
+#pragma unroll
+    for (int mi = 0; mi < WM; mi++)
+#pragma unroll
+        for (int c = 0; c < NL; c++) {
+            int64_t m = m0 + mi * 16 + c * (16 / NL) + lrow;
+            if (m >= M) m = M - 1;
+            goff[mi][c] = (uint32_t)((m * K) * (X32 ? 4 : 2) + lchunk * 16);
+        }
+    const int nt = Kb > kg ? (Kb - kg + WAVES - 1) / WAVES : 0;      // weight blocks of this wavefront
+    auto pair_k = [&](int p) { return (int64_t)(kg + (p >> 2) * WAVES) * kKB + (p & 3) * 64; };
+
+    u32x4 stage[2][WM][NL];
+    auto gload = [&](int set, int p) {
+        const unsigned char *base = static_cast<const unsigned char *>(x) + pair_k(p) * (X32 ? 4 : 2);   // uniform
+#pragma unroll
+        for (int mi = 0; mi < WM; mi++)
+#pragma unroll
+            for (int c = 0; c < NL; c++) stage[set][mi][c] = *reinterpret_cast<const u32x4 *>(base + goff[mi][c]);
+    };
+    auto lwrite = [&](int set, int slot) {
+#pragma unroll
+        for (int mi = 0; mi < WM; mi++)
+#pragma unroll
+            for (int c = 0; c < NL; c++) {
+                unsigned char *dst = win + slot * kSlot + mi * kFrag + (c * (16 / NL) + lrow) * kRow;
+                if constexpr (X32) {
+                    const floatx4 v = __builtin_bit_cast(floatx4, stage[set][mi][c]);
+                    half4 hi, lo;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        hi[e] = (_Float16)v[e];
+                        lo[e] = (_Float16)(v[e] - (float)hi[e]);
+                    }
+                    *reinterpret_cast<half4 *>(dst + lchunk * 8) = hi;
+                    *reinterpret_cast<half4 *>(dst + WM * kFrag + lchunk * 8) = lo;
+                } else {
+                    *reinterpret_cast<u32x4 *>(dst + lchunk * 16) = stage[set][mi][c];
+                }
+            }
+    };
+    auto compute = [&](int slot, const uint32_t (&wq)[WN][4], int q) {
+        const unsigned char *src = win + slot * kSlot + j * kRow + g * 16;
+#pragma unroll
+        for (int st = 0; st < 2; st++) {
+            half8 hi[WM], lo[X32 ? WM : 1];
+#pragma unroll
+            for (int mi = 0; mi < WM; mi++) {
+                hi[mi] = *reinterpret_cast<const half8 *>(src + mi * kFrag + st * 64);
+                if constexpr (X32) lo[mi] = *reinterpret_cast<const half8 *>(src + (WM + mi) * kFrag + st * 64);
+            }
+#pragma unroll
+            for (int nj = 0; nj < WN; nj++) {
+                const half8 a = decode_step(wq[nj][q], st);
+#pragma unroll
+                for (int mi = 0; mi < WM; mi++) {
+                    acc[mi][nj] = mfma16(a, hi[mi], acc[mi][nj]);
+                    if constexpr (X32) acc[mi][nj] = mfma16(a, lo[mi], acc[mi][nj]);
+                }
+            }
+        }
+    };
+
+    if (nt > 0) {
+        // weight dwords: dword q of a block is only used by pair q and is refilled from the next
+        // block right after (the 1 KiB blocks stay in L1 / L2 between the four dword loads)
+        uint32_t wq[WN][4];
+#pragma unroll
+        for (int nj = 0; nj < WN; nj++)
+#pragma unroll
+            for (int q = 0; q < 4; q++) wq[nj][q] = wb[nj][(int64_t)kg * 256 + q];
+        gload(0, 0);
+        gload(1, 1);
+        lwrite(0, 0);
+        gload(0, 2);
+        lwrite(1, 1);
+        gload(1, 3);
+        __builtin_amdgcn_wave_barrier();
+        for (int t = 0; t + 1 < nt; t++) {
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                compute(q & 1, wq, q);
+                __builtin_amdgcn_wave_barrier();
+#pragma unroll
+                for (int nj = 0; nj < WN; nj++) wq[nj][q] = wb[nj][(int64_t)(kg + (t + 1) * WAVES) * 256 + q];
+                lwrite(q & 1, q & 1);                 // pair p + 2 replaces pair p
+                gload(q & 1, t * 4 + q + 4);
+                __builtin_amdgcn_wave_barrier();
+            }
+        }
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            compute(q & 1, wq, q);
+            __builtin_amdgcn_wave_barrier();
+            if (q < 2) lwrite(q & 1, q & 1);
+            __builtin_amdgcn_wave_barrier();
+        }
+    }
+
+    // Sum the WAVES partial tiles in wavefront order (the windows are dead by now); fragment f is
+    // finalised by wavefront f mod WAVES. Lane (j, g) holds y[16 mi + j][16 nj + 4 g + r].
+    __syncthreads();
+#pragma unroll
+    for (int mi = 0; mi < WM; mi++)
+#pragma unroll
+        for (int nj = 0; nj < WN; nj++) red[(kg * NF + mi * WN + nj) * 64 + lane] = acc[mi][nj];
+    __syncthreads();
+    for (int f = kg; f < NF; f += WAVES) {
+        load_consts(f);
+        floatx4 s = red[f * 64 + lane];
+        for (int q = 1; q < WAVES; q++) {
+            const floatx4 p = red[(q * NF + f) * 64 + lane];
+            s[0] += p[0]; s[1] += p[1]; s[2] += p[2]; s[3] += p[3];
+        }
+        const int64_t m = m0 + (f / WN) * 16 + j, nq = n0 + (f % WN) * 16 + g * 4;
+        if (m >= M) continue;
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int64_t n = nq + r;
+            if (n < N) {
+                float v = s[r] * (sc4[r] * (1.0f / kWeightUnit)) + bi4[r];
+                const int64_t o = m * N + n;
+                if (y_f16) {
+                    if (residual) v += (float)static_cast<const _Float16 *>(residual)[o];
+                    if (relu) v = v > 0.f ? v : 0.f;
+                    static_cast<_Float16 *>(y)[o] = (_Float16)v;
+                } else {
+                    if (residual) v += static_cast<const float *>(residual)[o];
+                    if (relu) v = v > 0.f ? v : 0.f;
+                    static_cast<float *>(y)[o] = v;
+                }
+            }
+        }
+    }
+}
+
+template <int WM, int WN, int WAVES, bool X32>
+int launch_mid_lds(const void *x, int64_t M, int64_t K, const void *native, int64_t N, const tmq_epilogue &ep, void *y,
+                   void *stream) {
+    constexpr int BM = 16 * WM, BN = 16 * WN;
+    const int64_t tm = (M + BM - 1) / BM, tn = (N + BN - 1) / BN, Kb = native_blocks_k(K);
+    if (tm * tn > 0x7FFFFFFF || Kb > (1 << 20)) return TMQ_ERR_TOO_LARGE;
+    constexpr size_t win = (size_t)WAVES * 2 * (X32 ? 2 : 1) * WM * 16 * 144;
+    constexpr size_t redb = (size_t)WAVES * WM * WN * 64 * sizeof(floatx4);
+    constexpr size_t lds = win > redb ? win : redb;
+    static_assert(lds <= kSkinnyLdsMax, "mid kernel LDS");
+    auto kernel = mid_lds_kernel<WM, WN, WAVES, X32>;
+    if (lds > 64 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return note_hip_error(e);
+    }
+    const float *scale = ep.scale, *bias = ep.bias;
+    const void *residual = ep.residual;
+    const int relu = ep.relu, y_f16 = ep.y_dtype == TMQ_F16;
+    hipLaunchKernelGGL(kernel, dim3((uint32_t)(tm * tn)), dim3(64 * WAVES), lds, as_stream(stream), x, M, K,
+                       static_cast<const u32x4 *>(native), (int)Kb, N, native_blocks_n(N), (int)tn, scale, bias,
+                       residual, relu, y, y_f16);
+    return check_launch();
+}
+
+// Tile choice of the mid kernel: the largest tile that yields at least one workgroup per CU.
+template <bool X32>
+int mid_rows(const void *x, int64_t M, int64_t K, const void *native, int64_t N, const tmq_epilogue &ep, void *y,
+             void *stream) {
+    auto wgs = [&](int bm, int bn) { return ((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
+    if ((K % kKB == 0) && aligned16(x) && (uint64_t)M * (uint64_t)K * (X32 ? 4 : 2) < (1ull << 32)) {
+        if constexpr (!X32) {
+            if (wgs(64, 64) >= 256) return launch_mid_lds<4, 4, 8, false>(x, M, K, native, N, ep, y, stream);
+        }
+        return launch_mid_lds<2, 4, 8, X32>(x, M, K, native, N, ep, y, stream);
+    }
+    if (wgs(64, 32) >= 256) return launch_mid<2, 2, 2, 16, 2, X32>(x, M, K, native, N, ep, y, stream);
+    return launch_mid<2, 1, 2, 16, 2, X32>(x, M, K, native, N, ep, y, stream);
+}
+
 }  // namespace
 
 // gemm.hip: the MFMA-bound tile kernel for large M (fp16 activations).
@@ -400,21 +837,13 @@ int tmq_ternary_linear(const void *x, int x_dtype, int64_t M, int64_t K, const v
     const bool x32 = x_dtype == TMQ_F32;
     if (M <= 64) return x32 ? skinny_rows<true>(x, M, K, native, N, ep, y, stream)
                             : skinny_rows<false>(x, M, K, native, N, ep, y, stream);
-    if (!x32)
-        return launch_gemm_dense(x, M, K, native, N, ep.scale, ep.bias, ep.residual, ep.relu, y,
-                                 ep.y_dtype == TMQ_F16, stream);
-    // fp32 activations with M > 64: 64-row slabs through the two-term skinny kernel (keeps fp32
-    // accuracy; the fp16 tile kernel is the fast path).
-    const size_t ysz = ep.y_dtype == TMQ_F16 ? 2 : 4;
-    for (int64_t m0 = 0; m0 < M; m0 += 64) {
-        const int64_t mm = M - m0 < 64 ? M - m0 : 64;
-        tmq_epilogue e2 = ep;
-        if (ep.residual) e2.residual = static_cast<const char *>(ep.residual) + (size_t)m0 * N * ysz;
-        int rc = skinny_rows<true>(static_cast<const char *>(x) + (size_t)m0 * K * 4, mm, K, native, N, e2,
-                                   static_cast<char *>(y) + (size_t)m0 * N * ysz, stream);
-        if (rc != TMQ_OK) return rc;
-    }
-    return TMQ_OK;
+    // fp32 activations always take the mid kernel (two fp16 terms per value keep fp32 accuracy; the
+    // tile kernel is fp16 only). For fp16 the big-tile kernel wins once there are more than about
+    // 2.5 tiles of 64 x 64 per CU (measured crossover at K = N = 4096: M between 512 and 768).
+    if (x32) return mid_rows<true>(x, M, K, native, N, ep, y, stream);
+    if (((M + 63) / 64) * ((N + 63) / 64) <= 640) return mid_rows<false>(x, M, K, native, N, ep, y, stream);
+    return launch_gemm_dense(x, M, K, native, N, ep.scale, ep.bias, ep.residual, ep.relu, y, ep.y_dtype == TMQ_F16,
+                             stream);
 }
 
 }  // extern "C"
