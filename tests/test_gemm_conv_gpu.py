@@ -66,6 +66,9 @@ CONV_CASES = [  # B, C, H, W, N, k, stride, pad, dil
     (3, 3, 20, 20, 64, 7, 2, 3, 1), (2, 64, 7, 7, 128, 1, 2, 0, 1), (1, 24, 10, 11, 20, (3, 2), (2, 1), (1, 0), 1),
     (1, 8, 12, 12, 17, 3, 1, 2, 2), (2, 5, 9, 9, 10, 3, 1, 1, 1), (1, 128, 14, 14, 256, 3, 1, 1, 1),
     (4, 64, 16, 16, 64, 3, 1, 1, 1), (1, 8, 7, 7, 8, 3, 2, 0, 1),
+    # channel counts that are multiples of 64 take the uniform-tap loader
+    (2, 64, 13, 11, 48, 3, 2, 1, 1), (1, 128, 9, 10, 70, (3, 5), (1, 2), (2, 1), (2, 1)), (3, 192, 6, 6, 64, 1, 1, 0, 1),
+    (2, 256, 7, 7, 512, 3, 1, 1, 1), (1, 64, 5, 5, 32, 5, 1, 4, 2), (2, 512, 7, 7, 512, 3, 1, 1, 1),
 ]
 
 

@@ -20,6 +20,12 @@
 #include "mfma.h"
 
 namespace tmq {
+
+// mid.hip: split-reduction kernel for outputs of a few hundred 64 x 64 tiles
+bool mid_conv_ok(const void *x, const tmq_conv_shape *s);
+int launch_mid_conv(const void *x, const tmq_conv_shape *s, int ho, int wo, const void *native, const float *scale,
+                    const float *bias, const void *residual, int relu, void *y, int y_f16, void *stream);
+
 namespace {
 
 constexpr int kBK = 64;          // k-tile
@@ -159,6 +165,69 @@ struct ConvLoader {
             st.c -= C;
             if (++st.j == kx) { st.j = 0; ++st.i; }
         }
+    }
+};
+
+// im2col view for C % 64 == 0 (and at most 64 taps, fewer than 2^31 elements): a 64-wide k-tile is
+// 64 consecutive channels of ONE filter tap, so tap and channel offset are the same for the whole
+// workgroup and live in scalar registers. Per row the loader keeps one 32-bit element offset and a
+// bit mask of the taps that fall inside the image; a fetch is one add, one bit test and the load.
+struct ConvLoader64 {
+    const _Float16 *x;
+    int64_t M, K;
+    int B, C, H, W, Ho, Wo, ky, kx, sy, sx, py, px, dy, dx;
+
+    template <int CH, int T>
+    struct State {
+        int32_t off0[CH];          // element offset of (b, ih0, iw0, channel kc); may be negative
+        uint64_t inside[CH];       // bit t: tap t of this row reads inside the image
+        int tap, i, j, c0;         // uniform
+        int32_t delta;             // uniform: element offset of (tap, c0) relative to off0
+    };
+    template <int CH, int T>
+    __device__ __forceinline__ void init(State<CH, T> &st, int64_t m0, int tid) const {
+        st.tap = st.i = st.j = st.c0 = 0;
+        st.delta = 0;
+        const int kc = (tid & 7) * 8;
+#pragma unroll
+        for (int q = 0; q < CH; q++) {
+            const int64_t m = m0 + (tid >> 3) + q * (T / 8);
+            st.inside[q] = 0;
+            st.off0[q] = 0;
+            if (m < M) {
+                const int ow = (int)(m % Wo);
+                const int64_t t = m / Wo;
+                const int oh = (int)(t % Ho), b = (int)(t / Ho);
+                const int ih0 = oh * sy - py, iw0 = ow * sx - px;
+                st.off0[q] = ((b * H + ih0) * W + iw0) * C + kc;
+                uint64_t mask = 0;
+                for (int i = 0; i < ky; i++)
+                    for (int j = 0; j < kx; j++) {
+                        const int ih = ih0 + i * dy, iw = iw0 + j * dx;
+                        if (ih >= 0 && ih < H && iw >= 0 && iw < W) mask |= 1ull << (i * kx + j);
+                    }
+                st.inside[q] = mask;
+            }
+        }
+    }
+    template <int CH, int T>
+    __device__ __forceinline__ void fetch(State<CH, T> &st, int64_t, u32x4 (&out)[CH]) const {
+#pragma unroll
+        for (int q = 0; q < CH; q++) {
+            u32x4 v = {0u, 0u, 0u, 0u};
+            if ((st.inside[q] >> st.tap) & 1) v = *reinterpret_cast<const u32x4 *>(x + (st.off0[q] + st.delta));
+            out[q] = v;
+        }
+    }
+    template <int CH, int T>
+    __device__ __forceinline__ void advance(State<CH, T> &st) const {   // next k-tile: 64 channels on
+        st.c0 += kBK;
+        if (st.c0 == C) {
+            st.c0 = 0;
+            st.tap++;
+            if (++st.j == kx) { st.j = 0; ++st.i; }
+        }
+        st.delta = (st.i * dy * W + st.j * dx) * C + st.c0;
     }
 };
 
@@ -352,16 +421,15 @@ int launch_tile(const Loader &ld, const void *native, int64_t M, int64_t K, int6
     return check_launch();
 }
 
-// Tile choice: the largest tile that still yields at least ~2 workgroups per CU, else smaller.
+// Tile choice, from a sweep over M x K x N (4096^2 weights at M = 768 .. 4096 and the ResNet-18 layer
+// shapes): 128 x 256 once it gives 1.5 workgroups per CU, 128 x 128 down to one per CU, else
+// 64 x 64. Larger tiles (256 x 256, 256 x 128) and 128 x 64 never won.
 template <class Loader>
 int dispatch_tile(const Loader &ld, const void *native, int64_t M, int64_t K, int64_t N, const Epilogue &ep,
                   void *stream) {
     auto wgs = [&](int bm, int bn) { return ((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
-    if (N > 128 && wgs(128, 256) >= 512) return launch_tile<8, 4, 1, 4>(ld, native, M, K, N, ep, stream);
-    if (N > 128 && wgs(256, 256) >= 256) return launch_tile<8, 4, 2, 4>(ld, native, M, K, N, ep, stream);
-    if (N > 64 && wgs(256, 128) >= 384) return launch_tile<8, 4, 2, 2>(ld, native, M, K, N, ep, stream);
+    if (N > 128 && wgs(128, 256) >= 384) return launch_tile<8, 4, 1, 4>(ld, native, M, K, N, ep, stream);
     if (N > 64 && wgs(128, 128) >= 256) return launch_tile<4, 4, 2, 2>(ld, native, M, K, N, ep, stream);
-    if (wgs(128, 64) >= 512) return launch_tile<4, 4, 2, 1>(ld, native, M, K, N, ep, stream);
     return launch_tile<2, 4, 2, 1>(ld, native, M, K, N, ep, stream);
 }
 
@@ -407,6 +475,13 @@ int tmq_ternary_conv2d(const void *x, const tmq_conv_shape *s, const void *nativ
     if (M == 0) return TMQ_OK;
     Epilogue ep{scale, bias, residual, y, relu, y_dtype == TMQ_F16 ? 1 : 0};
     const _Float16 *xp = static_cast<const _Float16 *>(x);
+    // few output tiles and a long reduction: split the reduction inside the workgroup (mid.hip)
+    if (mid_conv_ok(x, s) && K >= 2048 && ((M + 63) / 64) * (((int64_t)s->N + 63) / 64) <= 640)
+        return launch_mid_conv(x, s, ho, wo, native, scale, bias, residual, relu, y, y_dtype == TMQ_F16 ? 1 : 0, stream);
+    if ((s->C % kBK == 0) && aligned16(x) && s->ky * s->kx <= 64 &&
+        (int64_t)s->B * s->H * s->W * s->C < (int64_t)0x7FFFFFFF)
+        return dispatch_tile(ConvLoader64{xp, M, K, s->B, s->C, s->H, s->W, ho, wo, s->ky, s->kx, s->sy, s->sx, s->py,
+                                          s->px, s->dy, s->dx}, native, M, K, s->N, ep, stream);
     if ((s->C % 8 == 0) && aligned16(x))
         return dispatch_tile(ConvLoader<true>{xp, M, K, s->B, s->C, s->H, s->W, ho, wo, s->ky, s->kx, s->sy, s->sx,
                                               s->py, s->px, s->dy, s->dx}, native, M, K, s->N, ep, stream);

@@ -12,6 +12,12 @@
 #include "mfma.h"
 
 namespace tmq {
+
+// mid.hip: staged split-reduction kernel for mid-size fp16 problems
+bool mid_dense_ok(const void *x, int64_t M, int64_t K);
+int launch_mid_dense(const void *x, int64_t M, int64_t K, const void *native, int64_t N, const float *scale,
+                     const float *bias, const void *residual, int relu, void *y, int y_f16, void *stream);
+
 namespace {
 
 // ---- prepack ------------------------------------------------------------------------------------
@@ -785,11 +791,13 @@ template <bool X32>
 int mid_rows(const void *x, int64_t M, int64_t K, const void *native, int64_t N, const tmq_epilogue &ep, void *y,
              void *stream) {
     auto wgs = [&](int bm, int bn) { return ((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
-    if ((K % kKB == 0) && aligned16(x) && (uint64_t)M * (uint64_t)K * (X32 ? 4 : 2) < (1ull << 32)) {
-        if constexpr (!X32) {
-            if (wgs(64, 64) >= 256) return launch_mid_lds<4, 4, 8, false>(x, M, K, native, N, ep, y, stream);
-        }
-        return launch_mid_lds<2, 4, 8, X32>(x, M, K, native, N, ep, y, stream);
+    if constexpr (X32) {
+        if ((K % kKB == 0) && aligned16(x) && (uint64_t)M * (uint64_t)K * 4 < (1ull << 32))
+            return launch_mid_lds<2, 4, 8, true>(x, M, K, native, N, ep, y, stream);
+    } else {
+        if (K >= 2048 && mid_dense_ok(x, M, K))
+            return launch_mid_dense(x, M, K, native, N, ep.scale, ep.bias, ep.residual, ep.relu, y,
+                                    ep.y_dtype == TMQ_F16, stream);
     }
     if (wgs(64, 32) >= 256) return launch_mid<2, 2, 2, 16, 2, X32>(x, M, K, native, N, ep, y, stream);
     return launch_mid<2, 1, 2, 16, 2, X32>(x, M, K, native, N, ep, y, stream);

@@ -1,0 +1,338 @@
+// Ternary GEMM / implicit-GEMM convolution for outputs too small to fill the chip with big tiles
+// (a few hundred 64 x 64 tiles): the reduction is split over the wavefronts of a workgroup.
+//
+// A workgroup of WAVES wavefronts owns a (16 WM) x (16 WN) output tile; wavefront kg multiplies the
+// whole tile over the weight blocks kb = kg, kg + WAVES, ... (256 reduction indices each) and the
+// partial tiles are summed through LDS in wavefront order, so the result does not depend on
+// scheduling and needs no workspace.
+//
+//   * Weights: the dword of the kernel-native layout (mfma.h) a lane needs, straight from global
+//     memory (the blocks stay in L1 / L2 between the four dword loads), expanded in two VALU ops
+//     per operand register.
+//   * Activations: an MFMA operand wants 16 bytes of row (lane % 16) in every lane -- loaded
+//     directly, 16 neighbouring lanes would touch 16 different rows and cost the texture path one
+//     cache line each. Instead a wavefront fetches whole 128-byte row pieces (8 lanes per row, 8
+//     rows per instruction) with global_load_lds_dwordx4 straight into a private LDS window and
+//     reads them back in operand order. The load writes lane l to byte 16 l of its destination, so
+//     the bank swizzle is applied on the global side: lane (row r, position p) fetches chunk
+//     p ^ ((r / 2) % 8) of its row piece; the reader undoes it. Operand reads of 16 rows then fall
+//     into 16 different 16-byte bank groups.
+//   * Pipeline unit: a "pair" = 64 reduction indices = one dword of every weight block = two MFMA
+//     steps. While pair p is multiplied out of one LDS slot, the loads of pair p + 1 fill the
+//     other. The window belongs to one wavefront: no workgroup barrier inside the loop.
+//   * Rows: a dense row-major matrix, or the im2col view of an NHWC tensor with C % 64 == 0 (a pair
+//     is then 64 consecutive channels of one filter tap; taps outside the image and reduction
+//     indices past K read a zero chunk instead).
+#include "common.h"
+#include "mfma.h"
+
+namespace tmq {
+namespace {
+
+__device__ const u32x4 kZeroChunk[8] = {};   // 128 zero bytes: the source of padding taps / the K tail
+
+struct MidEpilogue {
+    const float *scale, *bias;
+    const void *residual;
+    void *y;
+    int relu, y_f16;
+};
+
+// Row providers. `prepare` fixes what a lane needs for its 2 WM row pieces (load c of fragment mi
+// covers rows 8 c .. 8 c + 7; the lane's row is R = 8 c + lane / 8); `source` returns the address
+// of the lane's 16-byte chunk of pair starting at reduction index k0 (uniform).
+struct DenseRows {
+    const _Float16 *x;
+    int64_t M, K;
+
+    template <int WM>
+    struct State {
+        uint32_t off[WM][2];     // element offset of the row + swizzled chunk (host: M K < 2^31)
+    };
+    template <int WM>
+    __device__ __forceinline__ void prepare(State<WM> &st, int64_t m0, int lane) const {
+#pragma unroll
+        for (int mi = 0; mi < WM; mi++)
+#pragma unroll
+            for (int c = 0; c < 2; c++) {
+                const int R = c * 8 + (lane >> 3);
+                int64_t m = m0 + mi * 16 + R;
+                if (m >= M) m = M - 1;                      // rows past M: finite data, never stored
+                st.off[mi][c] = (uint32_t)(m * K) + (((lane & 7) ^ ((R >> 1) & 7)) * 8);
+            }
+    }
+    struct Pair { int64_t k0; bool live; };
+    __device__ __forceinline__ Pair pair(int64_t k0) const { return {k0, k0 < K}; }
+    template <int WM>
+    __device__ __forceinline__ const void *source(const State<WM> &st, const Pair &p, int mi, int c, int lane) const {
+        return p.live ? static_cast<const void *>(x + (p.k0 + st.off[mi][c]))
+                      : static_cast<const void *>(kZeroChunk + (lane & 7));
+    }
+};
+
+struct ConvRows {
+    const _Float16 *x;
+    int64_t M, K;
+    int B, C, H, W, Ho, Wo, ky, kx, sy, sx, py, px, dy, dx;
+
+    template <int WM>
+    struct State {
+        int32_t off[WM][2];      // element offset of (b, ih0, iw0, swizzled chunk); may be negative
+        int32_t ih0[WM][2], iw0[WM][2];
+    };
+    template <int WM>
+    __device__ __forceinline__ void prepare(State<WM> &st, int64_t m0, int lane) const {
+#pragma unroll
+        for (int mi = 0; mi < WM; mi++)
+#pragma unroll
+            for (int c = 0; c < 2; c++) {
+                const int R = c * 8 + (lane >> 3);
+                int64_t m = m0 + mi * 16 + R;
+                if (m >= M) m = M - 1;
+                const int ow = (int)(m % Wo);
+                const int64_t t = m / Wo;
+                const int oh = (int)(t % Ho), b = (int)(t / Ho);
+                st.ih0[mi][c] = oh * sy - py;
+                st.iw0[mi][c] = ow * sx - px;
+                st.off[mi][c] = ((b * H + st.ih0[mi][c]) * W + st.iw0[mi][c]) * C + (((lane & 7) ^ ((R >> 1) & 7)) * 8);
+            }
+    }
+    struct Pair { int di, dj, delta; bool live; };
+    __device__ __forceinline__ Pair pair(int64_t k0) const {       // uniform
+        const int tap = (int)((uint32_t)k0 / (uint32_t)C), c0 = (int)k0 - tap * C;   // K < 2^31
+        const int i = tap / kx, j = tap - i * kx;
+        return {i * dy, j * dx, (i * dy * W + j * dx) * C + c0, k0 < K};
+    }
+    template <int WM>
+    __device__ __forceinline__ const void *source(const State<WM> &st, const Pair &p, int mi, int c, int lane) const {
+        const bool in = p.live && (unsigned)(st.ih0[mi][c] + p.di) < (unsigned)H &&
+                        (unsigned)(st.iw0[mi][c] + p.dj) < (unsigned)W;
+        return in ? static_cast<const void *>(x + (st.off[mi][c] + p.delta))
+                  : static_cast<const void *>(kZeroChunk + (lane & 7));
+    }
+};
+
+// 16 bytes per lane from global memory straight into LDS: lane l lands at dst + 16 l (dst uniform).
+// The host pass of the compiler does not know the builtin and would drop every kernel that uses it,
+// so it only sees an empty body.
+__device__ __forceinline__ void load_to_lds(const void *src, unsigned char *dst) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    typedef __attribute__((address_space(3))) void *lds_ptr;
+    __builtin_amdgcn_global_load_lds(src, (lds_ptr)dst, 16, 0, 0);
+#endif
+}
+
+template <int WM, int WN, int WAVES, class Rows>
+__global__ __launch_bounds__(64 * WAVES) void mid_kernel(Rows rows, const u32x4 *__restrict__ native, int64_t M, int Kb,
+                                                         int64_t N, int64_t Nb, int tiles_n, MidEpilogue ep) {
+    constexpr int NF = WM * WN;
+    constexpr int kFrag = 16 * 128, kSlot = WM * kFrag, kWave = 2 * kSlot;   // bytes: 16 rows x 128 B per fragment
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    floatx4 *red = reinterpret_cast<floatx4 *>(smem);
+    const int lane = threadIdx.x & 63, kg = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int j = lane & 15, g = lane >> 4;
+    unsigned char *win = smem + kg * kWave;
+    const int tm = blockIdx.x / tiles_n, tn = blockIdx.x % tiles_n;
+    const int64_t m0 = (int64_t)tm * (16 * WM), n0 = (int64_t)tn * (16 * WN);
+
+    floatx4 acc[WM][WN];
+#pragma unroll
+    for (int mi = 0; mi < WM; mi++)
+#pragma unroll
+        for (int nj = 0; nj < WN; nj++) acc[mi][nj] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+    const uint32_t *wb[WN];                                       // dword d of block kb: wb[nj][kb * 256 + d]
+#pragma unroll
+    for (int nj = 0; nj < WN; nj++) {
+        int64_t nb = n0 / 16 + nj;
+        if (nb >= Nb) nb = Nb - 1;                                  // finite bits, never stored
+        wb[nj] = reinterpret_cast<const uint32_t *>(native + (nb * Kb) * 64 + lane);
+    }
+    typename Rows::template State<WM> st;
+    rows.template prepare<WM>(st, m0, lane);
+
+    const int nt = Kb > kg ? (Kb - kg + WAVES - 1) / WAVES : 0;      // weight blocks of this wavefront
+    const int np = nt * 4;                                          // pairs of this wavefront
+    auto pair_k = [&](int p) { return (int64_t)(kg + (p >> 2) * WAVES) * kKB + (p & 3) * 64; };
+
+    // asynchronous fill of one LDS slot with pair p: 2 WM loads of 1 KiB, lane l -> byte 16 l
+    auto fill = [&](int slot, int p) {
+        const typename Rows::Pair pr = rows.pair(pair_k(p));
+#pragma unroll
+        for (int mi = 0; mi < WM; mi++)
+#pragma unroll
+            for (int c = 0; c < 2; c++)
+                load_to_lds(rows.template source<WM>(st, pr, mi, c, lane), win + slot * kSlot + mi * kFrag + c * 1024);
+    };
+    // operand (row j, chunk ch) of a fragment sits at position ch ^ ((j / 2) % 8) of its row
+    const int key = (j >> 1) & 7;
+    const unsigned char *rd = win + j * 128;
+
+    if (np > 0) {
+        uint32_t wq[WN][4];
+#pragma unroll
+        for (int nj = 0; nj < WN; nj++)
+#pragma unroll
+            for (int q = 0; q < 4; q++) wq[nj][q] = wb[nj][(int64_t)kg * 256 + q];
+        fill(0, 0);
+        for (int t = 0; t < nt; t++) {
+            const bool last = t + 1 == nt;
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const int slot = q & 1;
+                // the fill of this slot (and the weight dwords) must have landed
+                __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
+                __builtin_amdgcn_sched_barrier(0);
+                half8 a[2][WM];                        // all operand reads of the pair
+#pragma unroll
+                for (int s = 0; s < 2; s++)
+#pragma unroll
+                    for (int mi = 0; mi < WM; mi++)
+                        a[s][mi] = *reinterpret_cast<const half8 *>(rd + slot * kSlot + mi * kFrag + (((4 * s + g) ^ key) * 16));
+                __builtin_amdgcn_sched_barrier(0);
+                // the other slot was read out one pair ago: start filling it with the next pair
+                if (!(last && q == 3)) fill(slot ^ 1, t * 4 + q + 1);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int s = 0; s < 2; s++)
+#pragma unroll
+                    for (int nj = 0; nj < WN; nj++) {
+                        const half8 w = decode_step(wq[nj][q], s);
+#pragma unroll
+                        for (int mi = 0; mi < WM; mi++) acc[mi][nj] = mfma16(w, a[s][mi], acc[mi][nj]);
+                    }
+                if (!last) {
+#pragma unroll
+                    for (int nj = 0; nj < WN; nj++) wq[nj][q] = wb[nj][(int64_t)(kg + (t + 1) * WAVES) * 256 + q];
+                }
+            }
+        }
+    }
+
+    // Sum the WAVES partial tiles in wavefront order (the windows are dead by now); fragment f is
+    // finalised by wavefront f mod WAVES. Lane (j, g) holds y[16 mi + j][16 nj + 4 g + r].
+    __syncthreads();
+#pragma unroll
+    for (int mi = 0; mi < WM; mi++)
+#pragma unroll
+        for (int nj = 0; nj < WN; nj++) red[(kg * NF + mi * WN + nj) * 64 + lane] = acc[mi][nj];
+    __syncthreads();
+    for (int f = kg; f < NF; f += WAVES) {
+        const int64_t m = m0 + (f / WN) * 16 + j, nq = n0 + (f % WN) * 16 + g * 4;
+        float sc4[4], bi4[4];
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            sc4[r] = (nq + r < N && ep.scale) ? ep.scale[nq + r] : 1.f;
+            bi4[r] = (nq + r < N && ep.bias) ? ep.bias[nq + r] : 0.f;
+        }
+        floatx4 s = red[f * 64 + lane];
+        for (int q = 1; q < WAVES; q++) {
+            const floatx4 p = red[(q * NF + f) * 64 + lane];
+            s[0] += p[0]; s[1] += p[1]; s[2] += p[2]; s[3] += p[3];
+        }
+        if (m >= M) continue;
+        const int64_t o = m * N + nq;
+        float v[4];
+#pragma unroll
+        for (int r = 0; r < 4; r++) v[r] = s[r] * (sc4[r] * (1.0f / kWeightUnit)) + bi4[r];
+        const bool vec = nq + 4 <= N && (N % 4 == 0) &&
+                         ((reinterpret_cast<uintptr_t>(ep.y) | reinterpret_cast<uintptr_t>(ep.residual)) & 15u) == 0;
+        if (ep.y_f16) {
+            _Float16 *yp = static_cast<_Float16 *>(ep.y) + o;
+            const _Float16 *rp = static_cast<const _Float16 *>(ep.residual) + o;
+            if (vec) {
+                if (ep.residual) {
+                    const half4 rs = *reinterpret_cast<const half4 *>(rp);
+#pragma unroll
+                    for (int r = 0; r < 4; r++) v[r] += (float)rs[r];
+                }
+                half4 h;
+#pragma unroll
+                for (int r = 0; r < 4; r++) h[r] = (_Float16)((ep.relu && v[r] < 0.f) ? 0.f : v[r]);
+                *reinterpret_cast<half4 *>(yp) = h;
+            } else {
+#pragma unroll
+                for (int r = 0; r < 4; r++)
+                    if (nq + r < N) {
+                        float f32 = v[r] + (ep.residual ? (float)rp[r] : 0.f);
+                        yp[r] = (_Float16)((ep.relu && f32 < 0.f) ? 0.f : f32);
+                    }
+            }
+        } else {
+            float *yp = static_cast<float *>(ep.y) + o;
+            const float *rp = static_cast<const float *>(ep.residual) + o;
+            if (vec) {
+                floatx4 out = {v[0], v[1], v[2], v[3]};
+                if (ep.residual) out += *reinterpret_cast<const floatx4 *>(rp);
+                if (ep.relu) {
+#pragma unroll
+                    for (int r = 0; r < 4; r++) out[r] = out[r] > 0.f ? out[r] : 0.f;
+                }
+                *reinterpret_cast<floatx4 *>(yp) = out;
+            } else {
+#pragma unroll
+                for (int r = 0; r < 4; r++)
+                    if (nq + r < N) {
+                        float f32 = v[r] + (ep.residual ? rp[r] : 0.f);
+                        yp[r] = (ep.relu && f32 < 0.f) ? 0.f : f32;
+                    }
+            }
+        }
+    }
+}
+
+template <int WM, int WN, int WAVES, class Rows>
+int launch(const Rows &rows, const void *native, int64_t M, int64_t K, int64_t N, const MidEpilogue &ep, void *stream) {
+    constexpr int BM = 16 * WM, BN = 16 * WN;
+    const int64_t tm = (M + BM - 1) / BM, tn = (N + BN - 1) / BN, Kb = native_blocks_k(K);
+    if (tm * tn > 0x7FFFFFFF || Kb > (1 << 20)) return TMQ_ERR_TOO_LARGE;
+    constexpr size_t win = (size_t)WAVES * 2 * WM * 16 * 128;
+    constexpr size_t redb = (size_t)WAVES * WM * WN * 64 * sizeof(floatx4);
+    constexpr size_t lds = win > redb ? win : redb;
+    static_assert(lds <= 152 * 1024, "LDS budget");
+    auto kernel = mid_kernel<WM, WN, WAVES, Rows>;
+    if (lds > 64 * 1024) {
+        // opt in to the large LDS (per device; the attribute is sticky, setting it again is cheap)
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return note_hip_error(e);
+    }
+    hipLaunchKernelGGL(kernel, dim3((uint32_t)(tm * tn)), dim3(64 * WAVES), lds, as_stream(stream), rows,
+                       static_cast<const u32x4 *>(native), M, (int)Kb, N, native_blocks_n(N), (int)tn, ep);
+    return check_launch();
+}
+
+// 64 x 64 tiles once they give a workgroup per CU, else 32 x 64.
+template <class Rows>
+int dispatch(const Rows &rows, const void *native, int64_t M, int64_t K, int64_t N, const MidEpilogue &ep,
+             void *stream) {
+    if (((M + 63) / 64) * ((N + 63) / 64) >= 256) return launch<4, 4, 8, Rows>(rows, native, M, K, N, ep, stream);
+    return launch<2, 4, 8, Rows>(rows, native, M, K, N, ep, stream);
+}
+
+}  // namespace
+
+// True when the staged split-reduction kernel can take a dense fp16 problem.
+bool mid_dense_ok(const void *x, int64_t M, int64_t K) {
+    return (K % 64 == 0) && aligned16(x) && M * K < (int64_t)0x7FFFFFFF;
+}
+
+int launch_mid_dense(const void *x, int64_t M, int64_t K, const void *native, int64_t N, const float *scale,
+                     const float *bias, const void *residual, int relu, void *y, int y_f16, void *stream) {
+    MidEpilogue ep{scale, bias, residual, y, relu, y_f16};
+    return dispatch(DenseRows{static_cast<const _Float16 *>(x), M, K}, native, M, K, N, ep, stream);
+}
+
+bool mid_conv_ok(const void *x, const tmq_conv_shape *s) {
+    return (s->C % 64 == 0) && aligned16(x) && (int64_t)s->B * s->H * s->W * s->C < (int64_t)0x7FFFFFFF;
+}
+
+int launch_mid_conv(const void *x, const tmq_conv_shape *s, int ho, int wo, const void *native, const float *scale,
+                    const float *bias, const void *residual, int relu, void *y, int y_f16, void *stream) {
+    const int64_t M = (int64_t)s->B * ho * wo, K = (int64_t)s->C * s->ky * s->kx;
+    MidEpilogue ep{scale, bias, residual, y, relu, y_f16};
+    return dispatch(ConvRows{static_cast<const _Float16 *>(x), M, K, s->B, s->C, s->H, s->W, ho, wo, s->ky, s->kx, s->sy,
+                             s->sx, s->py, s->px, s->dy, s->dx}, native, M, K, s->N, ep, stream);
+}
+
+}  // namespace tmq
