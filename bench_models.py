@@ -69,12 +69,11 @@ def randomize_ternary_(model, generator, p0=0.5):
 class FusedTernaryResNet18:
     """Deployment runner over a tmq_amd-quantized ResNet18 whose layers hold compact weights."""
 
-    def __init__(self, model: ResNet18, pad_stem_channels=8):
+    def __init__(self, model: ResNet18):
         from tmq_amd import ops
         self.ops = ops
         self.dev = model.fc.weight.device
-        self.stem_c = pad_stem_channels
-        self.stem = self._conv(model.conv1, model.bn1, pad_c=pad_stem_channels)
+        self.stem = self._stem(model.conv1, model.bn1)
         self.blocks = []
         for layer in (model.layer1, model.layer2, model.layer3, model.layer4):
             for blk in layer:
@@ -83,17 +82,31 @@ class FusedTernaryResNet18:
         self.fc = (ops.NativeWeights(model.fc.weight.data, model.fc.original_shape[0]),
                    model.fc.bias.data.float() if model.fc.bias is not None else None)
 
-    def _conv(self, conv, bn, pad_c=None):
+    def _stem(self, conv, bn):
+        """The 7x7 / stride 2 / pad 3 stem on 3 channels as a 7x4 / stride (2, 1) convolution on
+        "super-pixels": the image is stored NHWC with 4 channels (3 + one zero), and two neighbouring
+        pixels are read as one pixel of 8 channels. Output column ow reads pixels 2 ow - 3 .. 2 ow + 3,
+        i.e. super-pixels ow - 2 .. ow + 1 (8 pixels; the extra one, 2 ow - 4, gets zero weights), so
+        the reduction is 7 x 4 x 8 = 224 long instead of 7 x 7 x 8 = 392 with channels padded to 8."""
         ops = self.ops
         N, C, ky, kx = (int(v) for v in conv.original_shape)
-        words = conv.weight.data
-        if pad_c is not None and C < pad_c:
-            # zero-pad the input channels so that im2col rows are whole 16-byte chunks
-            w = ops.expand_ternary(words, [N, C, ky, kx])
-            wp = torch.zeros(N, pad_c, ky, kx, device=w.device)
-            wp[:, :C] = w
-            words, C = ops.compactify_ternary(wp), pad_c
-        nw = ops.NativeWeights(words, N, conv_kernel=(ky, kx))
+        pair = lambda v: tuple(v) if isinstance(v, (tuple, list)) else (v, v)
+        assert (C, ky, kx) == (3, 7, 7) and pair(conv.stride) == (2, 2) and pair(conv.padding) == (3, 3)
+        w = ops.expand_ternary(conv.weight.data, [N, C, ky, kx])
+        wp = torch.zeros(N, 8, ky, 4, device=w.device)
+        for q in range(4):
+            for par in range(2):
+                k = 2 * q + par - 1
+                if 0 <= k < kx:
+                    wp[:, par * 4:par * 4 + C, :, q] = w[:, :, :, k]
+        nw = ops.NativeWeights(ops.compactify_ternary(wp), N, conv_kernel=(ky, 4))
+        inv = (bn.running_var + bn.eps).rsqrt() * bn.weight
+        return nw, inv.float().contiguous(), (bn.bias - bn.running_mean * inv).float().contiguous(), (2, 1), ((3, 3), (2, 1))
+
+    def _conv(self, conv, bn):
+        ops = self.ops
+        N, C, ky, kx = (int(v) for v in conv.original_shape)
+        nw = ops.NativeWeights(conv.weight.data, N, conv_kernel=(ky, kx))
         # eval-mode BatchNorm folded into the epilogue: y = gamma (acc - mean) / sqrt(var + eps) + beta
         inv = (bn.running_var + bn.eps).rsqrt() * bn.weight
         scale = inv.float().contiguous()
@@ -109,9 +122,10 @@ class FusedTernaryResNet18:
     @torch.no_grad()
     def __call__(self, x):
         B, C, H, W = x.shape
-        xs = torch.empty((B, self.stem_c, H, W), dtype=torch.float16, device=x.device,
-                         memory_format=torch.channels_last).zero_()
-        xs[:, :C] = x
+        nhwc4 = torch.empty((B, H, W, 4), dtype=torch.float16, device=x.device)
+        nhwc4[..., :C] = x.permute(0, 2, 3, 1)
+        nhwc4[..., C:] = 0
+        xs = nhwc4.view(B, H, W // 2, 8).permute(0, 3, 1, 2)      # [B, 8, H, W / 2], channels_last memory
         y = self._run(xs, self.stem, relu=True)
         y = torch.nn.functional.max_pool2d(y, 3, 2, 1)
         for c1, c2, ds in self.blocks:

@@ -220,10 +220,14 @@ typedef struct tmq_conv_shape {
     int32_t B, C, H, W;   /* input extents (batch, channels, height, width) */
     int32_t N;            /* output channels */
     int32_t ky, kx, sy, sx, py, px, dy, dx;
+    int32_t py_end, px_end; /* zero rows / columns after the last input row / column; py, px
+                             * count those before the first. Equal to py, px for the usual
+                             * symmetric padding.                                           */
 } tmq_conv_shape;
 
-/* Output extents (PyTorch's formula floor((h + 2p - d(k-1) - 1)/s) + 1; the reference's own
- * expression at tmq/tmq.py:842-845 agrees with it on every ResNet shape).                     */
+/* Output extents, floor((h + p + p_end - d(k-1) - 1)/s) + 1 (PyTorch's formula for symmetric
+ * padding; the reference's own expression at tmq/tmq.py:842-845 agrees with it on every ResNet
+ * shape).                                                                                     */
 int tmq_conv2d_out_hw(const tmq_conv_shape *s, int32_t *ho, int32_t *wo);
 
 /* Ternary implicit-GEMM convolution, no materialised im2col. x: fp16 NHWC [B][H][W][C]

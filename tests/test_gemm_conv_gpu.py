@@ -106,6 +106,30 @@ def test_conv2d_matches_oracle(cuda, oracle, B, C, H, W, N, k, stride, pad, dil)
     assert _rel_err(y16.float().cpu().numpy(), want16) <= 1e-3
 
 
+@pytest.mark.parametrize("C,H,W,N,k,stride,pad,dil", [
+    (8, 20, 13, 24, (7, 4), (2, 1), ((3, 3), (2, 1)), (1, 1)),     # the super-pixel stem
+    (8, 9, 9, 16, (3, 3), (1, 1), ((0, 2), (1, 0)), (1, 1)),
+    (16, 11, 10, 40, (3, 5), (2, 2), ((2, 1), (0, 3)), (1, 2)),
+    (32, 8, 8, 64, (3, 3), (1, 1), ((1, 1), (1, 1)), (2, 2)),
+    (64, 9, 7, 32, (3, 3), (1, 2), ((1, 0), (2, 1)), (1, 1)),
+    (128, 6, 6, 512, (3, 3), (1, 1), ((0, 1), (1, 0)), (1, 1)),
+    (5, 7, 8, 10, (2, 3), (1, 1), ((1, 0), (0, 2)), (1, 1)),
+])
+def test_conv2d_asymmetric_padding(cuda, C, H, W, N, k, stride, pad, dil):
+    """Padding given per side, checked against torch's convolution of the explicitly padded input
+    on the expanded weights (small integers: every product and sum is exact, so bit for bit)."""
+    from tmq_amd import ops
+    g = torch.Generator(device=cuda).manual_seed(C + H + N)
+    Wt = torch.randint(-1, 2, (N, C, k[0], k[1]), device=cuda, generator=g).float()
+    x = torch.randint(-4, 5, (3, C, H, W), device=cuda, generator=g).float()
+    nw = ops.NativeWeights(ops.compactify_ternary(Wt), N, conv_kernel=k)
+    y = ops.ternary_conv2d(x.half(), nw, stride, pad, dil)
+    (pt, pb), (pl, pr) = pad
+    ref = torch.nn.functional.conv2d(torch.nn.functional.pad(x, (pl, pr, pt, pb)), Wt, None, stride, 0, dil)
+    assert y.shape == ref.shape
+    assert torch.equal(y, ref)
+
+
 def test_resnet_layer_shapes_against_torch(cuda):
     """Full-size ResNet-18 layer shapes (batch 8): checked against torch's fp32 convolution on the
     expanded weights, which the small cases above tie to the oracle."""

@@ -29,7 +29,7 @@ class Segment(ctypes.Structure):
 class ConvShape(ctypes.Structure):
     """tmq_conv_shape of include/tmq_hip.h."""
     _fields_ = [(k, ctypes.c_int32) for k in
-                ("B", "C", "H", "W", "N", "ky", "kx", "sy", "sx", "py", "px", "dy", "dx")]
+                ("B", "C", "H", "W", "N", "ky", "kx", "sy", "sx", "py", "px", "dy", "dx", "py_end", "px_end")]
 
 
 class Epilogue(ctypes.Structure):

@@ -168,10 +168,10 @@ struct ConvLoader {
     }
 };
 
-// im2col view for C % 64 == 0 (and at most 64 taps, fewer than 2^31 elements): a 64-wide k-tile is
+// im2col view for C % 64 == 0 (fewer than 2^31 elements): a 64-wide k-tile is
 // 64 consecutive channels of ONE filter tap, so tap and channel offset are the same for the whole
-// workgroup and live in scalar registers. Per row the loader keeps one 32-bit element offset and a
-// bit mask of the taps that fall inside the image; a fetch is one add, one bit test and the load.
+// workgroup and live in scalar registers. Per row the loader keeps one 32-bit element offset and the
+// window's top-left coordinate; a fetch is two unsigned compares, one add and the load.
 struct ConvLoader64 {
     const _Float16 *x;
     int64_t M, K;
@@ -180,42 +180,38 @@ struct ConvLoader64 {
     template <int CH, int T>
     struct State {
         int32_t off0[CH];          // element offset of (b, ih0, iw0, channel kc); may be negative
-        uint64_t inside[CH];       // bit t: tap t of this row reads inside the image
-        int tap, i, j, c0;         // uniform
+        int32_t ih0[CH], iw0[CH];  // top-left input coordinate of the row's window (rows past M: far outside)
+        int i, j, c0;              // uniform: tap and first channel of the current k-tile
         int32_t delta;             // uniform: element offset of (tap, c0) relative to off0
     };
     template <int CH, int T>
     __device__ __forceinline__ void init(State<CH, T> &st, int64_t m0, int tid) const {
-        st.tap = st.i = st.j = st.c0 = 0;
+        st.i = st.j = st.c0 = 0;
         st.delta = 0;
         const int kc = (tid & 7) * 8;
 #pragma unroll
         for (int q = 0; q < CH; q++) {
             const int64_t m = m0 + (tid >> 3) + q * (T / 8);
-            st.inside[q] = 0;
             st.off0[q] = 0;
+            st.ih0[q] = st.iw0[q] = INT32_MIN / 2;
             if (m < M) {
                 const int ow = (int)(m % Wo);
                 const int64_t t = m / Wo;
                 const int oh = (int)(t % Ho), b = (int)(t / Ho);
-                const int ih0 = oh * sy - py, iw0 = ow * sx - px;
-                st.off0[q] = ((b * H + ih0) * W + iw0) * C + kc;
-                uint64_t mask = 0;
-                for (int i = 0; i < ky; i++)
-                    for (int j = 0; j < kx; j++) {
-                        const int ih = ih0 + i * dy, iw = iw0 + j * dx;
-                        if (ih >= 0 && ih < H && iw >= 0 && iw < W) mask |= 1ull << (i * kx + j);
-                    }
-                st.inside[q] = mask;
+                st.ih0[q] = oh * sy - py;
+                st.iw0[q] = ow * sx - px;
+                st.off0[q] = ((b * H + st.ih0[q]) * W + st.iw0[q]) * C + kc;
             }
         }
     }
     template <int CH, int T>
     __device__ __forceinline__ void fetch(State<CH, T> &st, int64_t, u32x4 (&out)[CH]) const {
+        const int di = st.i * dy, dj = st.j * dx;
 #pragma unroll
         for (int q = 0; q < CH; q++) {
             u32x4 v = {0u, 0u, 0u, 0u};
-            if ((st.inside[q] >> st.tap) & 1) v = *reinterpret_cast<const u32x4 *>(x + (st.off0[q] + st.delta));
+            if ((unsigned)(st.ih0[q] + di) < (unsigned)H && (unsigned)(st.iw0[q] + dj) < (unsigned)W)
+                v = *reinterpret_cast<const u32x4 *>(x + (st.off0[q] + st.delta));
             out[q] = v;
         }
     }
@@ -224,10 +220,64 @@ struct ConvLoader64 {
         st.c0 += kBK;
         if (st.c0 == C) {
             st.c0 = 0;
-            st.tap++;
-            if (++st.j == kx) { st.j = 0; ++st.i; }
+            if (++st.j == kx) { st.j = 0; ++st.i; }   // past the last tap only in the zero-padded K tail: i >= ky
         }
         st.delta = (st.i * dy * W + st.j * dx) * C + st.c0;
+    }
+};
+
+// im2col view for few channels (C = 8, 16 or 32; fewer than 2^31 elements): a
+// 16-byte chunk is 8 channels of one tap and a 64-wide k-tile covers 64 / C taps. A thread's chunk
+// keeps its channel offset for the whole reduction and its tap advances by 64 / C per k-tile, so the
+// loader carries its tap (i, j) per thread, one 32-bit offset and the window's top-left coordinate per row.
+struct ConvLoaderFewC {
+    const _Float16 *x;
+    int64_t M, K;
+    int B, C, H, W, Ho, Wo, ky, kx, sy, sx, py, px, dy, dx;
+
+    template <int CH, int T>
+    struct State {
+        int32_t off0[CH];          // element offset of (b, ih0, iw0, this thread's channel offset)
+        int32_t ih0[CH], iw0[CH];  // top-left input coordinate of the row's window (rows past M: far outside)
+        int i, j;                  // this thread's tap in the current k-tile
+    };
+    template <int CH, int T>
+    __device__ __forceinline__ void init(State<CH, T> &st, int64_t m0, int tid) const {
+        const int kc = (tid & 7) * 8, tap = kc / C;
+        st.i = tap / kx;
+        st.j = tap - st.i * kx;
+#pragma unroll
+        for (int q = 0; q < CH; q++) {
+            const int64_t m = m0 + (tid >> 3) + q * (T / 8);
+            st.off0[q] = 0;
+            st.ih0[q] = st.iw0[q] = INT32_MIN / 2;
+            if (m < M) {
+                const int ow = (int)(m % Wo);
+                const int64_t t = m / Wo;
+                const int oh = (int)(t % Ho), b = (int)(t / Ho);
+                st.ih0[q] = oh * sy - py;
+                st.iw0[q] = ow * sx - px;
+                st.off0[q] = ((b * H + st.ih0[q]) * W + st.iw0[q]) * C + kc % C;
+            }
+        }
+    }
+    template <int CH, int T>
+    __device__ __forceinline__ void fetch(State<CH, T> &st, int64_t, u32x4 (&out)[CH]) const {
+        const int di = st.i * dy, dj = st.j * dx;
+        const int32_t delta = (di * W + dj) * C;
+        const bool tap_ok = st.i < ky;                       // taps past the last one: the zero-padded K tail
+#pragma unroll
+        for (int q = 0; q < CH; q++) {
+            u32x4 v = {0u, 0u, 0u, 0u};
+            if (tap_ok && (unsigned)(st.ih0[q] + di) < (unsigned)H && (unsigned)(st.iw0[q] + dj) < (unsigned)W)
+                v = *reinterpret_cast<const u32x4 *>(x + (st.off0[q] + delta));
+            out[q] = v;
+        }
+    }
+    template <int CH, int T>
+    __device__ __forceinline__ void advance(State<CH, T> &st) const {   // next k-tile: 64 / C taps on
+        st.j += kBK / C;
+        while (st.j >= kx) { st.j -= kx; ++st.i; }
     }
 };
 
@@ -452,8 +502,11 @@ extern "C" {
 int tmq_conv2d_out_hw(const tmq_conv_shape *s, int32_t *ho, int32_t *wo) {
     if (!s || !ho || !wo || s->sy <= 0 || s->sx <= 0 || s->dy <= 0 || s->dx <= 0 || s->ky <= 0 || s->kx <= 0)
         return TMQ_ERR_INVALID_ARG;
-    *ho = (s->H + 2 * s->py - s->dy * (s->ky - 1) - 1) / s->sy + 1;
-    *wo = (s->W + 2 * s->px - s->dx * (s->kx - 1) - 1) / s->sx + 1;
+    if (s->py < 0 || s->px < 0 || s->py_end < 0 || s->px_end < 0) return TMQ_ERR_INVALID_ARG;
+    const int32_t eh = s->H + s->py + s->py_end - s->dy * (s->ky - 1) - 1;
+    const int32_t ew = s->W + s->px + s->px_end - s->dx * (s->kx - 1) - 1;
+    *ho = eh < 0 ? 0 : eh / s->sy + 1;
+    *wo = ew < 0 ? 0 : ew / s->sx + 1;
     return TMQ_OK;
 }
 
@@ -478,10 +531,14 @@ int tmq_ternary_conv2d(const void *x, const tmq_conv_shape *s, const void *nativ
     // few output tiles and a long reduction: split the reduction inside the workgroup (mid.hip)
     if (mid_conv_ok(x, s) && K >= 2048 && ((M + 63) / 64) * (((int64_t)s->N + 63) / 64) <= 640)
         return launch_mid_conv(x, s, ho, wo, native, scale, bias, residual, relu, y, y_dtype == TMQ_F16 ? 1 : 0, stream);
-    if ((s->C % kBK == 0) && aligned16(x) && s->ky * s->kx <= 64 &&
+    if ((s->C % kBK == 0) && aligned16(x) &&
         (int64_t)s->B * s->H * s->W * s->C < (int64_t)0x7FFFFFFF)
         return dispatch_tile(ConvLoader64{xp, M, K, s->B, s->C, s->H, s->W, ho, wo, s->ky, s->kx, s->sy, s->sx, s->py,
                                           s->px, s->dy, s->dx}, native, M, K, s->N, ep, stream);
+    if ((s->C == 8 || s->C == 16 || s->C == 32) && aligned16(x) &&
+        (int64_t)s->B * s->H * s->W * s->C < (int64_t)0x7FFFFFFF)
+        return dispatch_tile(ConvLoaderFewC{xp, M, K, s->B, s->C, s->H, s->W, ho, wo, s->ky, s->kx, s->sy, s->sx, s->py,
+                                            s->px, s->dy, s->dx}, native, M, K, s->N, ep, stream);
     if ((s->C % 8 == 0) && aligned16(x))
         return dispatch_tile(ConvLoader<true>{xp, M, K, s->B, s->C, s->H, s->W, ho, wo, s->ky, s->kx, s->sy, s->sx,
                                               s->py, s->px, s->dy, s->dx}, native, M, K, s->N, ep, stream);

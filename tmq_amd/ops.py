@@ -420,6 +420,8 @@ def ternary_conv2d(x: torch.Tensor, nw: NativeWeights, stride=1, padding=0, dila
     [B, N, Ho, Wo] in channels_last memory."""
     pair = lambda v: tuple(v) if isinstance(v, (tuple, list)) else (v, v)
     (sy, sx), (py, px), (dy, dx) = pair(stride), pair(padding), pair(dilation)
+    # padding may also be ((top, bottom), (left, right))
+    (py, py_end), (px, px_end) = pair(py), pair(px)
     if not x.is_cuda or x.dim() != 4:
         raise RuntimeError("ternary_conv2d: expected a 4-D GPU tensor")
     if x.shape[1] != nw.C:
@@ -427,7 +429,7 @@ def ternary_conv2d(x: torch.Tensor, nw: NativeWeights, stride=1, padding=0, dila
     if x.dtype != torch.float16 or not x.is_contiguous(memory_format=torch.channels_last):
         x = x.to(dtype=torch.float16, memory_format=torch.channels_last)
     B, C, H, W = x.shape
-    shp = _capi.ConvShape(B, C, H, W, nw.N, nw.ky, nw.kx, sy, sx, py, px, dy, dx)
+    shp = _capi.ConvShape(B, C, H, W, nw.N, nw.ky, nw.kx, sy, sx, py, px, dy, dx, py_end, px_end)
     ho, wo = ctypes.c_int32(0), ctypes.c_int32(0)
     lib = _lib()
     check(lib.tmq_conv2d_out_hw(ctypes.byref(shp), ctypes.byref(ho), ctypes.byref(wo)), "conv2d_out_hw")
