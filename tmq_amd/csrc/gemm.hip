@@ -18,6 +18,7 @@
 //     mod 8) cover neighbouring tiles and share activation rows in that XCD's L2.
 #include "common.h"
 #include "mfma.h"
+#include <type_traits>
 
 namespace tmq {
 
@@ -29,6 +30,16 @@ int launch_mid_conv(const void *x, const tmq_conv_shape *s, int ho, int wo, cons
 namespace {
 
 constexpr int kBK = 64;          // k-tile
+__device__ u32x4 kZeroChunk;              // zero-initialised, never written: what loads of padding taps / k-tiles past K are redirected to
+
+// One load from `p` if `ok`, else from the zero chunk. The empty asm keeps the selected address in a
+// register, so that the compiler issues exactly one load instead of a branch around two.
+__device__ __forceinline__ u32x4 load_or_zero(const u32x4 *p, bool ok) {
+    typedef const __attribute__((address_space(1))) u32x4 *global_ptr;   // stay in the global address space
+    global_ptr q = ok ? (global_ptr)p : (global_ptr)&kZeroChunk;
+    asm volatile("" : "+v"(q));
+    return *q;
+}
 constexpr int kPitch = 64;       // LDS row pitch in halfs: 128 bytes = 8 chunks of 16 bytes, no padding.
 // Chunk c of row r is stored at position c ^ (r & 7): a wavefront's stores cover whole rows
 // (contiguous kilobytes) and the operand reads of 8 consecutive rows at one k offset land in 8
@@ -72,7 +83,8 @@ struct DenseLoader {
     }
     template <int CH, int T>
     __device__ __forceinline__ void fetch(State<CH, T> &st, int64_t k0, u32x4 (&out)[CH]) const {
-        const int64_t k = k0 + st.kc;
+        // k-tiles past K are prefetched too (and never multiplied): FAST re-reads the last tile
+        const int64_t k = (FAST && k0 >= K ? K - kBK : k0) + st.kc;
 #pragma unroll
         for (int i = 0; i < CH; i++) {
             if constexpr (FAST) {
@@ -207,12 +219,13 @@ struct ConvLoader64 {
     template <int CH, int T>
     __device__ __forceinline__ void fetch(State<CH, T> &st, int64_t, u32x4 (&out)[CH]) const {
         const int di = st.i * dy, dj = st.j * dx;
+        const bool tap_ok = st.i < ky;                       // k-tiles past K are prefetched too
 #pragma unroll
         for (int q = 0; q < CH; q++) {
-            u32x4 v = {0u, 0u, 0u, 0u};
-            if ((unsigned)(st.ih0[q] + di) < (unsigned)H && (unsigned)(st.iw0[q] + dj) < (unsigned)W)
-                v = *reinterpret_cast<const u32x4 *>(x + (st.off0[q] + st.delta));
-            out[q] = v;
+            // every load is issued (padding reads the zero chunk), which keeps the compiler's count
+            // of outstanding loads exact
+            const bool in = tap_ok & ((unsigned)(st.ih0[q] + di) < (unsigned)H) & ((unsigned)(st.iw0[q] + dj) < (unsigned)W);
+            out[q] = load_or_zero(reinterpret_cast<const u32x4 *>(x + (st.off0[q] + st.delta)), in);
         }
     }
     template <int CH, int T>
@@ -268,10 +281,8 @@ struct ConvLoaderFewC {
         const bool tap_ok = st.i < ky;                       // taps past the last one: the zero-padded K tail
 #pragma unroll
         for (int q = 0; q < CH; q++) {
-            u32x4 v = {0u, 0u, 0u, 0u};
-            if (tap_ok && (unsigned)(st.ih0[q] + di) < (unsigned)H && (unsigned)(st.iw0[q] + dj) < (unsigned)W)
-                v = *reinterpret_cast<const u32x4 *>(x + (st.off0[q] + delta));
-            out[q] = v;
+            const bool in = tap_ok & ((unsigned)(st.ih0[q] + di) < (unsigned)H) & ((unsigned)(st.iw0[q] + dj) < (unsigned)W);
+            out[q] = load_or_zero(reinterpret_cast<const u32x4 *>(x + (st.off0[q] + delta)), in);
         }
     }
     template <int CH, int T>
@@ -282,7 +293,7 @@ struct ConvLoaderFewC {
 };
 
 // ---- the tile kernel ---------------------------------------------------------------------------------
-template <int WM, int WN, int WGM, int WGN, class Loader>
+template <int WM, int WN, int WGM, int WGN, int D, class Loader>
 __global__ __launch_bounds__(64 * WGM * WGN, 2) void tile_kernel(Loader ld, const uint32_t *__restrict__ native,
                                                               int64_t M, int64_t K, int64_t N, int64_t Kb, int64_t Nb,
                                                               Epilogue ep, int tiles_m, int tiles_n) {
@@ -323,19 +334,32 @@ __global__ __launch_bounds__(64 * WGM * WGN, 2) void tile_kernel(Loader ld, cons
     }
     const int KT = (int)((K + kBK - 1) / kBK);
 
-    u32x4 stage[CH];
-    uint32_t wcur[WN], wnext[WN];
+    // Register prefetch, D k-tiles deep: while tile kt is multiplied out of LDS, tiles kt + 1 .. kt + D
+    // are in flight from global memory (D = 1: fetched at the top of a pass, stored at its end) (a 64-wide k-tile of MFMA work is far shorter than a trip to
+    // L2 when the tile is small). Every load is issued unconditionally -- tiles past K read a zero
+    // chunk / the last weight dword -- so the compiler counts outstanding loads exactly.
+    u32x4 stage[D][CH];
+    uint32_t wcur[WN], wq[D][WN];
     const int srow = tid >> 3;
     const int scol = (((tid & 7) ^ (srow & 7)) * 8);   // (T / 8) is a multiple of 8, so row & 7 == srow & 7 for every chunk
-    // prologue: weight words first, activations last, so that the wait in front of the LDS store
-    // retires every outstanding load and the loop starts with a clean memory counter
+    auto wload = [&](uint32_t (&w)[WN], int kn) {
+        if (kn >= KT) kn = KT - 1;
 #pragma unroll
-    for (int j = 0; j < WN; j++) wcur[j] = wptr[j][0];
-    ld.template fetch<CH, T>(st, 0, stage);
+        for (int j = 0; j < WN; j++) w[j] = wptr[j][(int64_t)(kn >> 2) * 256 + (kn & 3)];
+    };
+    auto lds_store = [&](int buf, const u32x4 (&v)[CH]) {
 #pragma unroll
-    for (int i = 0; i < CH; i++) *reinterpret_cast<u32x4 *>(&As[0][(srow + i * (T / 8)) * kPitch + scol]) = stage[i];
+        for (int i = 0; i < CH; i++) *reinterpret_cast<u32x4 *>(&As[buf][(srow + i * (T / 8)) * kPitch + scol]) = v[i];
+    };
+    wload(wcur, 0);
+    ld.template fetch<CH, T>(st, 0, stage[0]);
+    lds_store(0, stage[0]);
 #pragma unroll
-    for (int j = 0; j < WN; j++) asm volatile("" ::"v"(wcur[j]));   // pin the weight loads in front of the loop
+    for (int d = 0; d + 1 < D; d++) {   // the last set is filled by the first pass of the loop
+        ld.template advance<CH, T>(st);
+        ld.template fetch<CH, T>(st, (int64_t)(d + 1) * kBK, stage[d]);
+        wload(wq[d], d + 1);
+    }
     __syncthreads();
 
     // per-column epilogue constants, fetched now so their latency hides behind the main loop
@@ -351,16 +375,15 @@ __global__ __launch_bounds__(64 * WGM * WGN, 2) void tile_kernel(Loader ld, cons
     const int arow = (wm * WM * 16 + r16) * kPitch;
     // operand read of m-fragment i, k-step s: chunk (4 s + g) of row (.. + 16 i + r16); 16 i keeps row & 7
     auto swz = [&](int i, int s) { return i * 16 * kPitch + (((4 * s + g) ^ (r16 & 7)) * 8); };
-    for (int kt = 0; kt < KT; kt++) {
+    // one k-tile; `slot` (static) is the register set that holds tile kt + 1
+    auto body = [&](int kt, auto slot_tag) {
+        constexpr int slot = decltype(slot_tag)::value, freed = (slot + D - 1) % D;
+        // the set written to LDS in the previous pass is refilled with tile kt + D; issued ahead of
+        // the matrix work so that address arithmetic and load issue overlap with it
+        ld.template advance<CH, T>(st);
+        ld.template fetch<CH, T>(st, (int64_t)(kt + D) * kBK, stage[freed]);
+        wload(wq[freed], kt + D);
         const int cur = kt & 1;
-        const bool more = kt + 1 < KT;
-        if (more) {   // global loads of the next tile fly during the math
-            ld.template advance<CH, T>(st);
-            ld.template fetch<CH, T>(st, (int64_t)(kt + 1) * kBK, stage);
-            const int kn = kt + 1;
-#pragma unroll
-            for (int j = 0; j < WN; j++) wnext[j] = wptr[j][(int64_t)(kn >> 2) * 256 + (kn & 3)];
-        }
         const _Float16 *abase = &As[cur][arow];
         // Software pipeline over the 2 WM operand reads of the tile (fragment i, k-step s): kAhead reads
         // are in flight ahead of the MFMAs that consume them, so LDS latency hides behind matrix
@@ -383,14 +406,31 @@ __global__ __launch_bounds__(64 * WGM * WGN, 2) void tile_kernel(Loader ld, cons
                 a[q + kAhead] = *reinterpret_cast<const half8 *>(abase + swz((q + kAhead) >> 1, (q + kAhead) & 1));
             __builtin_amdgcn_sched_barrier(0);
         }
-        if (more) {
+        // tile kt + 1 goes to the other LDS buffer
+        lds_store(cur ^ 1, stage[slot]);
+        // (a real move, pinned here: left to the compiler the copy drifts to the loop header and
+        // then waits for loads that are still in flight)
 #pragma unroll
-            for (int i = 0; i < CH; i++)
-                *reinterpret_cast<u32x4 *>(&As[cur ^ 1][(srow + i * (T / 8)) * kPitch + scol]) = stage[i];
-#pragma unroll
-            for (int j = 0; j < WN; j++) wcur[j] = wnext[j];
+        for (int j = 0; j < WN; j++) {
+            if constexpr (D > 1) asm volatile("v_mov_b32 %0, %1" : "=v"(wcur[j]) : "v"(wq[slot][j]));
+            else wcur[j] = wq[slot][j];
         }
         __syncthreads();
+    };
+    // enter the loop with nothing outstanding: the conditional loads above would otherwise make the
+    // compiler wait for every load at each use inside the loop
+    __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
+    int kt = 0;
+    for (; kt + D <= KT; kt += D) {
+        body(kt, std::integral_constant<int, 0>{});
+        if constexpr (D > 1) body(kt + 1, std::integral_constant<int, 1>{});
+        if constexpr (D > 2) body(kt + 2, std::integral_constant<int, 2>{});
+    }
+    if constexpr (D > 1) {
+        if (kt < KT) body(kt++, std::integral_constant<int, 0>{});
+    }
+    if constexpr (D > 2) {
+        if (kt < KT) body(kt++, std::integral_constant<int, 1>{});
     }
 
     // Epilogue. A lane holds rows 4g + r, column r16 of each 16 x 16 accumulator -- 64-byte row
@@ -459,13 +499,13 @@ __global__ __launch_bounds__(64 * WGM * WGN, 2) void tile_kernel(Loader ld, cons
     }
 }
 
-template <int WM, int WN, int WGM, int WGN, class Loader>
+template <int WM, int WN, int WGM, int WGN, int D, class Loader>
 int launch_tile(const Loader &ld, const void *native, int64_t M, int64_t K, int64_t N, const Epilogue &ep,
                 void *stream) {
     constexpr int BM = 16 * WM * WGM, BN = 16 * WN * WGN;
     const int64_t tm = (M + BM - 1) / BM, tn = (N + BN - 1) / BN;
     if (tm * tn > 0x7FFFFFFF) return TMQ_ERR_TOO_LARGE;
-    hipLaunchKernelGGL((tile_kernel<WM, WN, WGM, WGN, Loader>), dim3((uint32_t)(tm * tn)), dim3(64 * WGM * WGN), 0,
+    hipLaunchKernelGGL((tile_kernel<WM, WN, WGM, WGN, D, Loader>), dim3((uint32_t)(tm * tn)), dim3(64 * WGM * WGN), 0,
                        as_stream(stream), ld, static_cast<const uint32_t *>(native), M, K, N, native_blocks_k(K),
                        native_blocks_n(N), ep, (int)tm, (int)tn);
     return check_launch();
@@ -478,9 +518,17 @@ template <class Loader>
 int dispatch_tile(const Loader &ld, const void *native, int64_t M, int64_t K, int64_t N, const Epilogue &ep,
                   void *stream) {
     auto wgs = [&](int bm, int bn) { return ((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
-    if (N > 128 && wgs(128, 256) >= 384) return launch_tile<8, 4, 1, 4>(ld, native, M, K, N, ep, stream);
-    if (N > 64 && wgs(128, 128) >= 256) return launch_tile<4, 4, 2, 2>(ld, native, M, K, N, ep, stream);
-    return launch_tile<2, 4, 2, 1>(ld, native, M, K, N, ep, stream);
+    // Prefetch depth: the big tile has a k-tile of work long enough to cover a trip to L2 (and no
+    // registers to spare); the smaller ones fetch two tiles ahead once the reduction is long enough
+    // to pay for the extra tile in the prologue (measured on the ResNet-18 layers: K = 576 loses,
+    // K >= 1152 wins).
+    const bool deep = K >= 16 * kBK;
+    if (N > 128 && wgs(128, 256) >= 384) return launch_tile<8, 4, 1, 4, 1>(ld, native, M, K, N, ep, stream);
+    if (N > 64 && wgs(128, 128) >= 256)
+        return deep ? launch_tile<4, 4, 2, 2, 2>(ld, native, M, K, N, ep, stream)
+                    : launch_tile<4, 4, 2, 2, 1>(ld, native, M, K, N, ep, stream);
+    return deep ? launch_tile<2, 4, 2, 1, 2>(ld, native, M, K, N, ep, stream)
+                : launch_tile<2, 4, 2, 1, 1>(ld, native, M, K, N, ep, stream);
 }
 
 }  // namespace
