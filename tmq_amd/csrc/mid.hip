@@ -2,9 +2,11 @@
 // (a few hundred 64 x 64 tiles): the reduction is split over the wavefronts of a workgroup.
 //
 // A workgroup of WAVES wavefronts owns a (16 WM) x (16 WN) output tile; wavefront kg multiplies the
-// whole tile over the weight blocks kb = kg, kg + WAVES, ... (256 reduction indices each) and the
-// partial tiles are summed through LDS in wavefront order, so the result does not depend on
-// scheduling and needs no workspace.
+// whole tile over the "pairs" (64 reduction indices each) kg, kg + WAVES, ... and the partial tiles
+// are summed through LDS in wavefront order, so the result does not depend on scheduling and needs
+// no workspace. Every wavefront runs on its own: there is no workgroup barrier inside the loop, and
+// one wavefront expands each weight word for 64 rows (the expansion costs two VALU operations per
+// operand register whatever the number of rows).
 //
 //   * Weights: the dword of the kernel-native layout (mfma.h) a lane needs, straight from global
 //     memory (the blocks stay in L1 / L2 between the four dword loads), expanded in two VALU ops
@@ -25,6 +27,7 @@
 //     indices past K read a zero chunk instead).
 #include "common.h"
 #include "mfma.h"
+#include <type_traits>
 
 namespace tmq {
 namespace {
@@ -124,11 +127,11 @@ __device__ __forceinline__ void load_to_lds(const void *src, unsigned char *dst)
 
 template <int WM, int WN, int WAVES, class Rows>
 __global__ __launch_bounds__(64 * WAVES) void mid_kernel(Rows rows, const u32x4 *__restrict__ native, int64_t M, int Kb,
-                                                         int64_t N, int64_t Nb, int tiles_n, MidEpilogue ep) {
+                                                         int npairs, int64_t N, int64_t Nb, int tiles_n,
+                                                         MidEpilogue ep) {
     constexpr int NF = WM * WN;
     constexpr int kFrag = 16 * 128, kSlot = WM * kFrag, kWave = 2 * kSlot;   // bytes: 16 rows x 128 B per fragment
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-    floatx4 *red = reinterpret_cast<floatx4 *>(smem);
     const int lane = threadIdx.x & 63, kg = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int j = lane & 15, g = lane >> 4;
     unsigned char *win = smem + kg * kWave;
@@ -151,13 +154,16 @@ __global__ __launch_bounds__(64 * WAVES) void mid_kernel(Rows rows, const u32x4 
     typename Rows::template State<WM> st;
     rows.template prepare<WM>(st, m0, lane);
 
-    const int nt = Kb > kg ? (Kb - kg + WAVES - 1) / WAVES : 0;      // weight blocks of this wavefront
-    const int np = nt * 4;                                          // pairs of this wavefront
-    auto pair_k = [&](int p) { return (int64_t)(kg + (p >> 2) * WAVES) * kKB + (p & 3) * 64; };
-
-    // asynchronous fill of one LDS slot with pair p: 2 WM loads of 1 KiB, lane l -> byte 16 l
+    // the reduction is dealt out in pairs: wavefront kg takes pairs kg, kg + WAVES, ...
+    const int np = npairs > kg ? (npairs - kg + WAVES - 1) / WAVES : 0;
+    auto wload = [&](uint32_t (&w)[WN], int p) {
+        const int pi = kg + p * WAVES;
+#pragma unroll
+        for (int nj = 0; nj < WN; nj++) w[nj] = wb[nj][(int64_t)(pi >> 2) * 256 + (pi & 3)];
+    };
+    // asynchronous fill of one LDS slot with a pair: 2 WM loads of 1 KiB, lane l -> byte 16 l
     auto fill = [&](int slot, int p) {
-        const typename Rows::Pair pr = rows.pair(pair_k(p));
+        const typename Rows::Pair pr = rows.pair((int64_t)(kg + p * WAVES) * 64);
 #pragma unroll
         for (int mi = 0; mi < WM; mi++)
 #pragma unroll
@@ -169,113 +175,123 @@ __global__ __launch_bounds__(64 * WAVES) void mid_kernel(Rows rows, const u32x4 
     const unsigned char *rd = win + j * 128;
 
     if (np > 0) {
-        uint32_t wq[WN][4];
-#pragma unroll
-        for (int nj = 0; nj < WN; nj++)
-#pragma unroll
-            for (int q = 0; q < 4; q++) wq[nj][q] = wb[nj][(int64_t)kg * 256 + q];
+        uint32_t wq[2][WN];
+        wload(wq[0], 0);
         fill(0, 0);
-        for (int t = 0; t < nt; t++) {
-            const bool last = t + 1 == nt;
+        // one pair; `par` (static) = parity of p = LDS slot and weight register set of the pair
+        auto step = [&](int p, auto par_tag) {
+            constexpr int par = decltype(par_tag)::value;
+            // the fill of this slot (and the weight dwords) must have landed
+            __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
+            __builtin_amdgcn_sched_barrier(0);
+            half8 a[2][WM];                        // all operand reads of the pair
 #pragma unroll
-            for (int q = 0; q < 4; q++) {
-                const int slot = q & 1;
-                // the fill of this slot (and the weight dwords) must have landed
-                __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
-                __builtin_amdgcn_sched_barrier(0);
-                half8 a[2][WM];                        // all operand reads of the pair
+            for (int s = 0; s < 2; s++)
 #pragma unroll
-                for (int s = 0; s < 2; s++)
-#pragma unroll
-                    for (int mi = 0; mi < WM; mi++)
-                        a[s][mi] = *reinterpret_cast<const half8 *>(rd + slot * kSlot + mi * kFrag + (((4 * s + g) ^ key) * 16));
-                __builtin_amdgcn_sched_barrier(0);
-                // the other slot was read out one pair ago: start filling it with the next pair
-                if (!(last && q == 3)) fill(slot ^ 1, t * 4 + q + 1);
-                __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                for (int s = 0; s < 2; s++)
-#pragma unroll
-                    for (int nj = 0; nj < WN; nj++) {
-                        const half8 w = decode_step(wq[nj][q], s);
-#pragma unroll
-                        for (int mi = 0; mi < WM; mi++) acc[mi][nj] = mfma16(w, a[s][mi], acc[mi][nj]);
-                    }
-                if (!last) {
-#pragma unroll
-                    for (int nj = 0; nj < WN; nj++) wq[nj][q] = wb[nj][(int64_t)(kg + (t + 1) * WAVES) * 256 + q];
-                }
+                for (int mi = 0; mi < WM; mi++)
+                    a[s][mi] = *reinterpret_cast<const half8 *>(rd + par * kSlot + mi * kFrag + (((4 * s + g) ^ key) * 16));
+            __builtin_amdgcn_sched_barrier(0);
+            // the other slot was read out one pair ago: start filling it with the next pair
+            if (p + 1 < np) {
+                fill(par ^ 1, p + 1);
+                wload(wq[par ^ 1], p + 1);
             }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int s = 0; s < 2; s++)
+#pragma unroll
+                for (int nj = 0; nj < WN; nj++) {
+                    const half8 w = decode_step(wq[par][nj], s);
+#pragma unroll
+                    for (int mi = 0; mi < WM; mi++) acc[mi][nj] = mfma16(w, a[s][mi], acc[mi][nj]);
+                }
+        };
+        int p = 0;
+        for (; p + 2 <= np; p += 2) {
+            step(p, std::integral_constant<int, 0>{});
+            step(p + 1, std::integral_constant<int, 1>{});
         }
+        if (p < np) step(p, std::integral_constant<int, 0>{});
     }
 
-    // Sum the WAVES partial tiles in wavefront order (the windows are dead by now); fragment f is
-    // finalised by wavefront f mod WAVES. Lane (j, g) holds y[16 mi + j][16 nj + 4 g + r].
-    __syncthreads();
+    // Epilogue. Lane (j, g) of fragment (mi, nj) holds y[16 mi + j][16 nj + 4 g + r], r = 0..3. Every
+    // wavefront parks its fragments in LDS (the windows are dead by now) with the four g of a row
+    // next to each other; then the whole workgroup walks the tile row by row: 16 consecutive threads
+    // own one row (4 columns each), add the WAVES partial sums in wavefront order -- so the result
+    // does not depend on scheduling -- and write 128 or 256 contiguous bytes per row. A thread keeps
+    // its columns for all its rows, so scale and bias are fetched once.
+    constexpr int kFragPitch = 1024 + 64;                       // bytes; +64 spreads the nj over the banks
+    constexpr int T = 64 * WAVES, kC4 = 4 * WN;                 // threads; float4 columns per row
+    static_assert(T % kC4 == 0, "a thread must keep its columns");
+    if constexpr (WAVES > 1) __syncthreads();
+    else __builtin_amdgcn_wave_barrier();
 #pragma unroll
     for (int mi = 0; mi < WM; mi++)
 #pragma unroll
-        for (int nj = 0; nj < WN; nj++) red[(kg * NF + mi * WN + nj) * 64 + lane] = acc[mi][nj];
-    __syncthreads();
-    for (int f = kg; f < NF; f += WAVES) {
-        const int64_t m = m0 + (f / WN) * 16 + j, nq = n0 + (f % WN) * 16 + g * 4;
-        float sc4[4], bi4[4];
-#pragma unroll
-        for (int r = 0; r < 4; r++) {
-            sc4[r] = (nq + r < N && ep.scale) ? ep.scale[nq + r] : 1.f;
-            bi4[r] = (nq + r < N && ep.bias) ? ep.bias[nq + r] : 0.f;
-        }
-        floatx4 s = red[f * 64 + lane];
-        for (int q = 1; q < WAVES; q++) {
-            const floatx4 p = red[(q * NF + f) * 64 + lane];
-            s[0] += p[0]; s[1] += p[1]; s[2] += p[2]; s[3] += p[3];
-        }
-        if (m >= M) continue;
-        const int64_t o = m * N + nq;
-        float v[4];
-#pragma unroll
-        for (int r = 0; r < 4; r++) v[r] = s[r] * (sc4[r] * (1.0f / kWeightUnit)) + bi4[r];
-        const bool vec = nq + 4 <= N && (N % 4 == 0) &&
-                         ((reinterpret_cast<uintptr_t>(ep.y) | reinterpret_cast<uintptr_t>(ep.residual)) & 15u) == 0;
-        if (ep.y_f16) {
-            _Float16 *yp = static_cast<_Float16 *>(ep.y) + o;
-            const _Float16 *rp = static_cast<const _Float16 *>(ep.residual) + o;
-            if (vec) {
-                if (ep.residual) {
-                    const half4 rs = *reinterpret_cast<const half4 *>(rp);
-#pragma unroll
-                    for (int r = 0; r < 4; r++) v[r] += (float)rs[r];
-                }
-                half4 h;
-#pragma unroll
-                for (int r = 0; r < 4; r++) h[r] = (_Float16)((ep.relu && v[r] < 0.f) ? 0.f : v[r]);
-                *reinterpret_cast<half4 *>(yp) = h;
-            } else {
-#pragma unroll
-                for (int r = 0; r < 4; r++)
-                    if (nq + r < N) {
-                        float f32 = v[r] + (ep.residual ? (float)rp[r] : 0.f);
-                        yp[r] = (_Float16)((ep.relu && f32 < 0.f) ? 0.f : f32);
-                    }
-            }
+        for (int nj = 0; nj < WN; nj++)
+            *reinterpret_cast<floatx4 *>(smem + (size_t)(kg * NF + mi * WN + nj) * kFragPitch + (j * 4 + g) * 16) = acc[mi][nj];
+    if constexpr (WAVES > 1) __syncthreads();
+    else __builtin_amdgcn_wave_barrier();
+
+    const int tid = threadIdx.x, c4 = tid % kC4;
+    const int64_t n = n0 + c4 * 4;
+    const bool vec = (N % 4 == 0) && ((reinterpret_cast<uintptr_t>(ep.y) | reinterpret_cast<uintptr_t>(ep.residual) |
+                                       reinterpret_cast<uintptr_t>(ep.scale) | reinterpret_cast<uintptr_t>(ep.bias)) & 15u) == 0;
+    if (n < N) {
+        floatx4 sc = {1.f, 1.f, 1.f, 1.f}, bi = {0.f, 0.f, 0.f, 0.f};
+        if (vec) {
+            if (ep.scale) sc = *reinterpret_cast<const floatx4 *>(ep.scale + n);
+            if (ep.bias) bi = *reinterpret_cast<const floatx4 *>(ep.bias + n);
         } else {
-            float *yp = static_cast<float *>(ep.y) + o;
-            const float *rp = static_cast<const float *>(ep.residual) + o;
-            if (vec) {
-                floatx4 out = {v[0], v[1], v[2], v[3]};
-                if (ep.residual) out += *reinterpret_cast<const floatx4 *>(rp);
-                if (ep.relu) {
 #pragma unroll
-                    for (int r = 0; r < 4; r++) out[r] = out[r] > 0.f ? out[r] : 0.f;
+            for (int r = 0; r < 4; r++)
+                if (n + r < N) {
+                    if (ep.scale) sc[r] = ep.scale[n + r];
+                    if (ep.bias) bi[r] = ep.bias[n + r];
                 }
-                *reinterpret_cast<floatx4 *>(yp) = out;
+        }
+        sc *= 1.0f / kWeightUnit;
+        for (int row = tid / kC4; row < 16 * WM; row += T / kC4) {
+            const int64_t m = m0 + row;
+            if (m >= M) break;
+            const unsigned char *src = smem + (size_t)((row >> 4) * WN + (c4 >> 2)) * kFragPitch + ((row & 15) * 4 + (c4 & 3)) * 16;
+            floatx4 v = *reinterpret_cast<const floatx4 *>(src);
+#pragma unroll
+            for (int q = 1; q < WAVES; q++) v += *reinterpret_cast<const floatx4 *>(src + (size_t)q * NF * kFragPitch);
+            v = v * sc + bi;
+            const int64_t o = m * N + n;
+            if (vec) {
+                if (ep.y_f16) {
+                    if (ep.residual) {
+                        const half4 rs = *reinterpret_cast<const half4 *>(static_cast<const _Float16 *>(ep.residual) + o);
+#pragma unroll
+                        for (int r = 0; r < 4; r++) v[r] += (float)rs[r];
+                    }
+                    half4 h;
+#pragma unroll
+                    for (int r = 0; r < 4; r++) h[r] = (_Float16)((ep.relu && v[r] < 0.f) ? 0.f : v[r]);
+                    *reinterpret_cast<half4 *>(static_cast<_Float16 *>(ep.y) + o) = h;
+                } else {
+                    if (ep.residual) v += *reinterpret_cast<const floatx4 *>(static_cast<const float *>(ep.residual) + o);
+                    if (ep.relu) {
+#pragma unroll
+                        for (int r = 0; r < 4; r++) v[r] = v[r] > 0.f ? v[r] : 0.f;
+                    }
+                    *reinterpret_cast<floatx4 *>(static_cast<float *>(ep.y) + o) = v;
+                }
             } else {
 #pragma unroll
-                for (int r = 0; r < 4; r++)
-                    if (nq + r < N) {
-                        float f32 = v[r] + (ep.residual ? rp[r] : 0.f);
-                        yp[r] = (ep.relu && f32 < 0.f) ? 0.f : f32;
+                for (int r = 0; r < 4; r++) {
+                    if (n + r >= N) break;
+                    float f = v[r];
+                    if (ep.y_f16) {
+                        if (ep.residual) f += (float)static_cast<const _Float16 *>(ep.residual)[o + r];
+                        static_cast<_Float16 *>(ep.y)[o + r] = (_Float16)((ep.relu && f < 0.f) ? 0.f : f);
+                    } else {
+                        if (ep.residual) f += static_cast<const float *>(ep.residual)[o + r];
+                        static_cast<float *>(ep.y)[o + r] = (ep.relu && f < 0.f) ? 0.f : f;
                     }
+                }
             }
         }
     }
@@ -287,7 +303,7 @@ int launch(const Rows &rows, const void *native, int64_t M, int64_t K, int64_t N
     const int64_t tm = (M + BM - 1) / BM, tn = (N + BN - 1) / BN, Kb = native_blocks_k(K);
     if (tm * tn > 0x7FFFFFFF || Kb > (1 << 20)) return TMQ_ERR_TOO_LARGE;
     constexpr size_t win = (size_t)WAVES * 2 * WM * 16 * 128;
-    constexpr size_t redb = (size_t)WAVES * WM * WN * 64 * sizeof(floatx4);
+    constexpr size_t redb = (size_t)WAVES * WM * WN * (1024 + 64);
     constexpr size_t lds = win > redb ? win : redb;
     static_assert(lds <= 152 * 1024, "LDS budget");
     auto kernel = mid_kernel<WM, WN, WAVES, Rows>;
@@ -298,16 +314,35 @@ int launch(const Rows &rows, const void *native, int64_t M, int64_t K, int64_t N
         if (e != hipSuccess) return note_hip_error(e);
     }
     hipLaunchKernelGGL(kernel, dim3((uint32_t)(tm * tn)), dim3(64 * WAVES), lds, as_stream(stream), rows,
-                       static_cast<const u32x4 *>(native), M, (int)Kb, N, native_blocks_n(N), (int)tn, ep);
+                       static_cast<const u32x4 *>(native), M, (int)Kb, (int)((K + 63) / 64), N, native_blocks_n(N),
+                       (int)tn, ep);
     return check_launch();
 }
 
-// 64 x 64 tiles once they give a workgroup per CU, else 32 x 64.
+// Geometry: 64 x 64 tiles once they give a workgroup per CU, else 32 x 64; then as many wavefronts
+// per tile as it takes to put about ten on every CU, each with at least two pairs to multiply.
 template <class Rows>
 int dispatch(const Rows &rows, const void *native, int64_t M, int64_t K, int64_t N, const MidEpilogue &ep,
              void *stream) {
-    if (((M + 63) / 64) * ((N + 63) / 64) >= 256) return launch<4, 4, 8, Rows>(rows, native, M, K, N, ep, stream);
-    return launch<2, 4, 8, Rows>(rows, native, M, K, N, ep, stream);
+    const int64_t npairs = (K + 63) / 64, tn = (N + 63) / 64;
+    const bool big = ((M + 63) / 64) * tn >= 256;
+    const int64_t tiles = ((M + (big ? 63 : 31)) / (big ? 64 : 32)) * tn;
+    int waves = 1;
+    while (waves < 8 && tiles * waves < 2560 && npairs >= 4 * waves) waves *= 2;
+    if (big) {
+        switch (waves) {
+            case 1: return launch<4, 4, 1, Rows>(rows, native, M, K, N, ep, stream);
+            case 2: return launch<4, 4, 2, Rows>(rows, native, M, K, N, ep, stream);
+            case 4: return launch<4, 4, 4, Rows>(rows, native, M, K, N, ep, stream);
+            default: return launch<4, 4, 8, Rows>(rows, native, M, K, N, ep, stream);
+        }
+    }
+    switch (waves) {
+        case 1: return launch<2, 4, 1, Rows>(rows, native, M, K, N, ep, stream);
+        case 2: return launch<2, 4, 2, Rows>(rows, native, M, K, N, ep, stream);
+        case 4: return launch<2, 4, 4, Rows>(rows, native, M, K, N, ep, stream);
+        default: return launch<2, 4, 8, Rows>(rows, native, M, K, N, ep, stream);
+    }
 }
 
 }  // namespace
