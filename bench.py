@@ -194,9 +194,79 @@ def bench_linear(args, torch):
         out[str(M)] = {"us": round(us, 3), "tflops": round(flops / us / 1e6, 3), "gbs": round(byts / us / 1e3, 2),
                        "frac_hbm": round(byts / us / 1e3 / HBM_PEAK_GBS, 4),
                        "frac_mfma_fp16": round(flops / us / 1e6 / 2500.0, 4)}
+    extra = {}
+    if args.gemv_floor:
+        extra = _gemv_floor_and_large(args, torch, natives)
     return {"metric": "ternary-GEMM eff. TFLOP/s (K=N=4096)", "unit": "TFLOP/s", "n_gpus": 1, "dtype": "f16",
             "data": "synthetic", "config": {"workload": "configs[2]: ternary linear K=N=4096", "rotate_buffers": nrot},
-            "value": out.get("4096", {}).get("tflops"), "by_M": out}
+            "value": out.get("4096", {}).get("tflops"), "by_M": out, **extra}
+
+
+def _graph_time_us(torch, calls, replays, settle_ms):
+    """Capture the launches `calls` issue into one HIP graph and time its replays with events."""
+    graph, side = torch.cuda.CUDAGraph(), torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            n = calls()
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < settle_ms * 1e-3:
+        graph.replay()
+        torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(replays):
+        graph.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / (replays * n) * 1e3
+
+
+def _gemv_floor_and_large(args, torch, natives):
+    """Two reference points for the M = 1 figure: (1) the read floor -- a kernel that only streams the
+    same packed bytes with the same launch geometry (tmq_probe_stream_read) -- and (2) the same GEMV at
+    K = N = 16384 (64 MiB of packed weights per launch, rotating over 6 buffers), where a launch is
+    long enough for bandwidth rather than latency to decide."""
+    import ctypes
+    from tmq_amd import ops, _capi
+    dev = torch.device("cuda:0")
+    lib = _capi.load()
+    sink = torch.zeros(1, dtype=torch.int32, device=dev)
+    res = {}
+
+    def probe_calls(bufs):
+        def run():
+            s = _capi.stream_of(sink)
+            for b in bufs:
+                _capi.check(lib.tmq_probe_stream_read(_capi.ptr(b), ctypes.c_size_t(b.numel()), _capi.ptr(sink), s), "probe")
+            return len(bufs)
+        return run
+
+    small = [nw.buf for nw in natives]
+    run = probe_calls(small)
+    run()
+    res["read_floor_4MiB_us"] = round(_graph_time_us(torch, run, max(2, args.steps // len(small)), args.settle_ms), 3)
+
+    K = N = 16384
+    W = torch.randint(-1, 2, (N, K), dtype=torch.int8, device=dev)
+    packed = ops.compactify_ternary(W)
+    del W
+    big = [ops.NativeWeights(packed.clone(), N) for _ in range(6)]
+    x = torch.randn(1, K, device=dev).half()
+    scale = (0.5 + torch.rand(N, device=dev))
+
+    def gemv():
+        for nw in big:
+            ops.ternary_linear(x, nw, scale)
+        return len(big)
+    gemv()
+    us = _graph_time_us(torch, gemv, max(2, args.steps // 12), args.settle_ms)
+    byts = K * N / 4 + 2 * K + 8 * N
+    run = probe_calls([nw.buf for nw in big])
+    run()
+    floor = _graph_time_us(torch, run, max(2, args.steps // 12), args.settle_ms)
+    res["gemv_16384"] = {"us": round(us, 3), "gbs": round(byts / us / 1e3, 1), "frac_hbm": round(byts / us / 1e3 / HBM_PEAK_GBS, 4),
+                         "read_floor_us": round(floor, 3), "read_floor_gbs": round(K * N / 4 / floor / 1e3, 1)}
+    return res
 
 
 def bench_resnet_infer(args, torch):
@@ -285,6 +355,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--m-list", default="1,16,256,4096")
     ap.add_argument("--rotate", type=int, default=1)
+    ap.add_argument("--gemv-floor", type=int, default=1, help="linear workload: also time the read floor and a 16384^2 GEMV")
     ap.add_argument("--batch", type=int, default=0)
     args = ap.parse_args()
     if args.gpus != 1:

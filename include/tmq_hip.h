@@ -215,6 +215,13 @@ typedef struct tmq_epilogue {
 int tmq_ternary_linear(const void *x, int x_dtype, int64_t M, int64_t K, const void *native,
                        int64_t N, const tmq_epilogue *epilogue, void *y, void *stream);
 
+/* Measurement aid with no counterpart in the reference: streams `bytes` (a multiple of 1024)
+ * from src with the launch geometry of the M = 1 path of tmq_ternary_linear (1 KiB per
+ * wavefront and load, 16 wavefronts per workgroup) and does nothing else; *sink (device, 4
+ * bytes) is only written if the data has an impossible checksum. Its duration is the floor for
+ * a kernel that has to read that many bytes once: launch + one trip to memory.               */
+int tmq_probe_stream_read(const void *src, size_t bytes, uint32_t *sink, void *stream);
+
 /* Geometry of a 2-D convolution. */
 typedef struct tmq_conv_shape {
     int32_t B, C, H, W;   /* input extents (batch, channels, height, width) */

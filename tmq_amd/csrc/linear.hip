@@ -173,11 +173,23 @@ __global__ __launch_bounds__(1024) void skinny_kernel(const void *__restrict__ x
     const unsigned char *xl[MT];
     if constexpr (XLDS) {
         const int cpr = Kb * (kKB / 8), total = (int)M * cpr;          // 8-element chunks per row, in all
-        for (int id = threadIdx.x; id < total; id += blockDim.x) {
-            const int row = id / cpr, c = id - row * cpr;
-            const XFrag<X32> f = load_x<X32>(x, row, M, K, (int64_t)c * 8, vec);
-            *reinterpret_cast<half8 *>(smem + (size_t)row * pitch + c * 16) = f.hi;
-            if constexpr (X32) *reinterpret_cast<half8 *>(smem + plane + (size_t)row * pitch + c * 16) = f.lo;
+        // four chunks per pass: the loads of a pass are all issued before its LDS stores
+        constexpr int kBatch = 4;
+        for (int id0 = threadIdx.x; id0 < total; id0 += kBatch * blockDim.x) {
+            XFrag<X32> f[kBatch];
+#pragma unroll
+            for (int u = 0; u < kBatch; u++) {
+                const int id = id0 + u * blockDim.x, row = id / cpr, c = id - row * cpr;
+                f[u] = load_x<X32>(x, id < total ? row : M, M, K, (int64_t)c * 8, vec);   // past the end: zeros, not stored
+            }
+#pragma unroll
+            for (int u = 0; u < kBatch; u++) {
+                const int id = id0 + u * blockDim.x, row = id / cpr, c = id - row * cpr;
+                if (id < total) {
+                    *reinterpret_cast<half8 *>(smem + (size_t)row * pitch + c * 16) = f[u].hi;
+                    if constexpr (X32) *reinterpret_cast<half8 *>(smem + plane + (size_t)row * pitch + c * 16) = f[u].lo;
+                }
+            }
         }
 #pragma unroll
         for (int t = 0; t < MT; t++) {
@@ -294,6 +306,79 @@ __global__ __launch_bounds__(1024) void skinny_kernel(const void *__restrict__ x
     }
 }
 
+// ---- short GEMV -------------------------------------------------------------------------------------
+// M = 1 with at most two weight blocks per wavefront (K <= 8192 at 16 wavefronts): the whole job of a
+// wavefront is in flight at once -- its weight blocks and, straight into the operand registers, the
+// 512 bytes of the activation vector that go with each of them -- so a launch costs one trip to
+// memory, no staging through LDS and no barrier before the arithmetic. Lane (j, g) supplies column
+// j of the B operand; only column 0 is stored, so every lane simply loads the vector's chunk g.
+// Requires fp16 activations, K % 256 == 0, 16-byte aligned x.
+__global__ __launch_bounds__(1024) void gemv_short_kernel(const _Float16 *__restrict__ x, const u32x4 *__restrict__ native,
+                                                          int Kb, int64_t N, const float *__restrict__ scale,
+                                                          const float *__restrict__ bias, const void *__restrict__ residual,
+                                                          int relu, void *__restrict__ y, int y_f16) {
+    __shared__ floatx4 slot[16 * 64];
+    const int lane = threadIdx.x & 63, wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), waves = blockDim.x >> 6;
+    const int j = lane & 15, g = lane >> 4;
+    const int64_t nb = blockIdx.x;
+    const bool two = wv + waves < Kb;
+    const u32x4 *wp = native + (nb * Kb + wv) * 64 + lane;
+    const _Float16 *xp = x + (int64_t)wv * kKB + g * 8;
+    u32x4 w0 = __builtin_nontemporal_load(wp), w1 = {0u, 0u, 0u, 0u};
+    half8 x0[8], x1[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) x0[i] = *reinterpret_cast<const half8 *>(xp + i * 32);
+    if (two) {
+        w1 = __builtin_nontemporal_load(wp + (int64_t)waves * 64);
+#pragma unroll
+        for (int i = 0; i < 8; i++) x1[i] = *reinterpret_cast<const half8 *>(xp + (int64_t)waves * kKB + i * 32);
+    }
+    float sc4[4] = {1.f, 1.f, 1.f, 1.f}, bi4[4] = {0.f, 0.f, 0.f, 0.f};
+    if (wv == 0) {
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int64_t n = nb * 16 + g * 4 + r;
+            if (n < N) {
+                if (scale) sc4[r] = scale[n];
+                if (bias) bi4[r] = bias[n];
+            }
+        }
+    }
+    floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < 8; i++) acc = mfma16(decode_step(w0[i >> 1], i & 1), x0[i], acc);
+    if (two) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) acc = mfma16(decode_step(w1[i >> 1], i & 1), x1[i], acc);
+    }
+    // only column 0 (lanes j == 0) carries the result: 4 lanes x 4 channels per wavefront
+    if (j == 0) slot[wv * 4 + g] = acc;
+    __syncthreads();
+    if (wv == 0 && j == 0) {
+        floatx4 s = slot[g];
+        for (int w = 1; w < waves; w++) {
+            const floatx4 p = slot[w * 4 + g];
+            s[0] += p[0]; s[1] += p[1]; s[2] += p[2]; s[3] += p[3];
+        }
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int64_t n = nb * 16 + g * 4 + r;
+            if (n < N) {
+                float v = s[r] * (sc4[r] * (1.0f / kWeightUnit)) + bi4[r];
+                if (y_f16) {
+                    if (residual) v += (float)static_cast<const _Float16 *>(residual)[n];
+                    if (relu) v = v > 0.f ? v : 0.f;
+                    static_cast<_Float16 *>(y)[n] = (_Float16)v;
+                } else {
+                    if (residual) v += static_cast<const float *>(residual)[n];
+                    if (relu) v = v > 0.f ? v : 0.f;
+                    static_cast<float *>(y)[n] = v;
+                }
+            }
+        }
+    }
+}
+
 struct SkinnyArgs {
     const void *x;
     int64_t M, K;
@@ -329,6 +414,18 @@ int launch_skinny(const void *x, int64_t M, int64_t K, const void *native, int64
                   void *y, void *stream) {
     const int64_t Nb = native_blocks_n(N), Kb = native_blocks_k(K);
     if (Kb > (1 << 20)) return TMQ_ERR_TOO_LARGE;
+    if constexpr (MT == 1 && !X32) {
+        if (M == 1 && K % kKB == 0 && Kb <= 32 && aligned16(x) && Nb <= 0x7FFFFFFF) {
+            int waves = 16;
+            while (waves > Kb) waves >>= 1;
+            if (Kb <= 2 * waves) {
+                hipLaunchKernelGGL(gemv_short_kernel, dim3((uint32_t)Nb), dim3(64 * waves), 0, as_stream(stream),
+                                   static_cast<const _Float16 *>(x), static_cast<const u32x4 *>(native), (int)Kb, N,
+                                   ep.scale, ep.bias, ep.residual, ep.relu, y, ep.y_dtype == TMQ_F16);
+                return check_launch();
+            }
+        }
+    }
     // Geometry: 16 wavefronts where the reduction slots allow; short reductions give their spare
     // wavefronts to more channel blocks (GW) as long as >= 256 workgroups remain, else shrink.
     int waves = 16, GW = 1;
@@ -803,6 +900,17 @@ int mid_rows(const void *x, int64_t M, int64_t K, const void *native, int64_t N,
     return launch_mid<2, 1, 2, 16, 2, X32>(x, M, K, native, N, ep, y, stream);
 }
 
+// ---- read probe -------------------------------------------------------------------------------------
+// The weight stream of the skinny kernel and nothing else: wavefront w of a workgroup reads the
+// 1 KiB pieces w, w + 16, ... of the workgroup's share.
+__global__ __launch_bounds__(1024) void probe_read_kernel(const u32x4 *__restrict__ src, int per_wave, uint32_t *sink) {
+    const int lane = threadIdx.x & 63, wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const u32x4 *p = src + ((int64_t)blockIdx.x * 16 * per_wave + wv) * 64 + lane;
+    u32x4 acc = {0u, 0u, 0u, 0u};
+    for (int t = 0; t < per_wave; t++) acc ^= __builtin_nontemporal_load(p + (int64_t)t * 16 * 64);
+    if ((acc[0] ^ acc[1] ^ acc[2] ^ acc[3]) == 0x9E3779B9u && (acc[0] + acc[1]) == 0x7F4A7C15u) *sink = acc[2];
+}
+
 }  // namespace
 
 // gemm.hip: the MFMA-bound tile kernel for large M (fp16 activations).
@@ -833,6 +941,20 @@ int tmq_prepack_weights(const uint32_t *words, int64_t N, int64_t C, int64_t ky,
     return check_launch();
 }
 
+int tmq_probe_stream_read(const void *src, size_t bytes, uint32_t *sink, void *stream) {
+    if (!src || !sink || bytes == 0 || bytes % 1024 != 0 || !aligned16(src)) return TMQ_ERR_INVALID_ARG;
+    const size_t pieces = bytes / 1024;
+    // one piece per wavefront up to 4096 workgroups, then more pieces per wavefront
+    size_t per_wave = 1;
+    while (pieces / (16 * per_wave) > 4096 && pieces % (32 * per_wave) == 0) per_wave *= 2;
+    if (pieces % (16 * per_wave) != 0) return TMQ_ERR_INVALID_ARG;
+    const size_t wgs = pieces / (16 * per_wave);
+    if (wgs > 0x7FFFFFFF) return TMQ_ERR_TOO_LARGE;
+    hipLaunchKernelGGL(probe_read_kernel, dim3((uint32_t)wgs), dim3(1024), 0, as_stream(stream),
+                       static_cast<const u32x4 *>(src), (int)per_wave, sink);
+    return check_launch();
+}
+
 int tmq_ternary_linear(const void *x, int x_dtype, int64_t M, int64_t K, const void *native, int64_t N,
                        const tmq_epilogue *epilogue, void *y, void *stream) {
     if (M < 0 || K <= 0 || N <= 0) return TMQ_ERR_INVALID_ARG;
@@ -843,8 +965,12 @@ int tmq_ternary_linear(const void *x, int x_dtype, int64_t M, int64_t K, const v
     if (epilogue) ep = *epilogue;
     if (ep.y_dtype != TMQ_F16 && ep.y_dtype != TMQ_F32) return TMQ_ERR_UNSUPPORTED;
     const bool x32 = x_dtype == TMQ_F32;
-    if (M <= 64) return x32 ? skinny_rows<true>(x, M, K, native, N, ep, y, stream)
-                            : skinny_rows<false>(x, M, K, native, N, ep, y, stream);
+    // Up to 16 rows the weight-streaming kernel (activations staged in LDS); it also takes 17..64 rows
+    // when the split-reduction kernel cannot (fp32 input, short or ragged K, unaligned rows).
+    const bool mid_fp16 = !x32 && K >= 2048 && mid_dense_ok(x, M, K);
+    if (M <= 16 || (M <= 64 && !mid_fp16))
+        return x32 ? skinny_rows<true>(x, M, K, native, N, ep, y, stream)
+                   : skinny_rows<false>(x, M, K, native, N, ep, y, stream);
     // fp32 activations always take the mid kernel (two fp16 terms per value keep fp32 accuracy; the
     // tile kernel is fp16 only). For fp16 the big-tile kernel wins once there are more than about
     // 2.5 tiles of 64 x 64 per CU (measured crossover at K = N = 4096: M between 512 and 768).
