@@ -226,3 +226,20 @@ def test_library_exports_every_declared_symbol():
         assert name in _capi.SIGNATURES, f"{name} has no ctypes prototype"
     assert lib.tmq_version() >= 100
     assert lib.tmq_status_string(-5).decode().startswith("malformed")
+
+
+def test_torch_extension_exports_the_reference_names():
+    """tmq/tmq_cuda.cu:800-809 and tmq/tmq_native.cpp:550-555: the twelve names tmq.py imports."""
+    from tmq_amd import tmq_hip_ext as ext
+    for name in ("fwd_softstep", "bwd_softstep", "fwd_softstep_derivative", "bwd_softstep_derivative",
+                 "ternary_mmm_cuda", "ternary_mvm_cuda", "ternary_dwconv_cuda", "ternary_dwconvtrans_cuda",
+                 "compactify_ternary", "compress_ternary", "decompress_ternary", "expand_ternary"):
+        assert callable(getattr(ext, name)), name
+    # the host codec needs no GPU: a stream written by the reference's coder decodes to the same words
+    g = np.load(os.path.join(ROOT, "tests", "golden", "native_golden.npz"))
+    for i in range(3):
+        w, compact, stream = g[f"w{i}"], g[f"compact{i}"], g[f"stream{i}"]
+        words = ext.decompress_ternary(torch.from_numpy(stream.view(np.int8).copy()), list(w.shape)).numpy()
+        assert words.shape == compact.shape and np.array_equal(_u32(words), _u32(compact))
+        assert np.array_equal(ext.compress_ternary(torch.from_numpy(compact.view(np.int32).copy()), list(w.shape), True).numpy().view(np.uint8),
+                              stream.view(np.uint8))

@@ -478,3 +478,13 @@ def ternary_mvm_cuda(vector: torch.Tensor, weights: torch.Tensor, columns: int) 
     if vector.dim() < 1 or vector.dim() > 4 or any(s != 1 for s in vector.shape[:-1]):
         raise RuntimeError("ternary_mvm_cuda: expected a single vector (leading dimensions of 1)")
     return ternary_linear(vector.contiguous(), native_weights(weights, columns))
+
+
+# ---- the PyTorch extension with the reference's binding names --------------------------------------------
+# tmq_hip_ext (csrc/torch_ext.cpp, `make -C tmq_amd/csrc ext`) exposes the same twelve names as the
+# reference's tmq_cuda / tmq_native modules over the same C ABI; tmq.py calls through it when it has
+# been built and through the ctypes functions above otherwise. Either way the kernels are libtmq_hip's.
+try:
+    from . import tmq_hip_ext as ext
+except ImportError:
+    ext = None

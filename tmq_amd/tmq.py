@@ -27,6 +27,9 @@ from torch.autograd.function import Function
 from . import ops
 from ._capi import load as _load_native
 
+# the reference's binding names: the C++ extension when built, else the ctypes binding (same C ABI)
+_b = ops.ext if ops.ext is not None else ops
+
 # The reference exposes these two flags (tmq/tmq.py:28-46). Here the single native library is
 # mandatory: importing this module without it raises instead of degrading.
 _load_native()
@@ -330,12 +333,12 @@ class SoftStep(Function):
         ctx.ctrl = ctrl
         ctx.scale = scale            # only scales the gradient (tmq/tmq.py:412)
         ctx.save_for_backward(weight)
-        return ops.fwd_softstep(weight.data, ctrl.digamma)
+        return _b.fwd_softstep(weight.data, ctrl.digamma)
 
     @staticmethod
     def backward(ctx, grad_output):
         weight = ctx.saved_tensors[0]
-        return ops.bwd_softstep(weight.data, ctx.ctrl.digamma, ctx.scale, grad_output), None, None
+        return _b.bwd_softstep(weight.data, ctx.ctrl.digamma, ctx.scale, grad_output), None, None
 
 
 class SoftStepDerivative(Function):
@@ -348,12 +351,12 @@ class SoftStepDerivative(Function):
         ctx.save_for_backward(weight)
         ctx.digamma = digamma
         ctx.strength = strength
-        return ops.fwd_softstep_derivative(weight.data, digamma, strength)
+        return _b.fwd_softstep_derivative(weight.data, digamma, strength)
 
     @staticmethod
     def backward(ctx, grad_output):
         weight = ctx.saved_tensors[0]
-        return ops.bwd_softstep_derivative(weight.data, ctx.digamma, ctx.strength, grad_output), None, None
+        return _b.bwd_softstep_derivative(weight.data, ctx.digamma, ctx.strength, grad_output), None, None
 
 
 class TMQLayer:
@@ -438,7 +441,7 @@ class TMQLayer:
             if self.tensor_type == TensorType.COMPRESSED_TERNARY_32BIT:
                 stored = state_dict[prefix + "weight"]
                 dev = self.weight.device
-                self.weight = nn.Parameter(ops.decompress_ternary(stored.cpu(), self.original_shape).to(dev),
+                self.weight = nn.Parameter(_b.decompress_ternary(stored.cpu(), self.original_shape).to(dev),
                                            requires_grad=False)
                 self.tensor_type = TensorType.COMPACT_TERNARY_32BIT
                 self.compact = True
@@ -754,11 +757,11 @@ def compressed_state_dict(module: nn.Module, strong=False, remove_prefix=""):
         if getattr(layer, "original_shape", None) is None:
             layer.original_shape = layer.weight.shape
         if not strong and layer.tensor_type != TensorType.COMPACT_TERNARY_32BIT:
-            layer.weight = nn.Parameter(ops.compactify_ternary(layer.weight.data), requires_grad=False)
+            layer.weight = nn.Parameter(_b.compactify_ternary(layer.weight.data), requires_grad=False)
             layer.tensor_type = TensorType.COMPACT_TERNARY_32BIT
         elif strong and layer.tensor_type != TensorType.COMPRESSED_TERNARY_32BIT:
             from_compact = layer.tensor_type == TensorType.COMPACT_TERNARY_32BIT
-            stream = ops.compress_ternary(layer.weight.data, layer.original_shape, from_compact)
+            stream = _b.compress_ternary(layer.weight.data, layer.original_shape, from_compact)
             layer._stream_device = layer.weight.device
             layer.weight = nn.Parameter(stream, requires_grad=False)
             layer.tensor_type = TensorType.COMPRESSED_TERNARY_32BIT
@@ -773,7 +776,7 @@ def compressed_state_dict(module: nn.Module, strong=False, remove_prefix=""):
         if layer.tensor_type == TensorType.COMPRESSED_TERNARY_32BIT:
             # keep the model usable right away: back to the compact form in memory
             dev = getattr(layer, "_stream_device", layer.weight.device)
-            layer.weight = nn.Parameter(ops.decompress_ternary(layer.weight.data.cpu(), layer.original_shape).to(dev),
+            layer.weight = nn.Parameter(_b.decompress_ternary(layer.weight.data.cpu(), layer.original_shape).to(dev),
                                         requires_grad=False)
             layer.tensor_type = TensorType.COMPACT_TERNARY_32BIT
     return state
@@ -814,7 +817,7 @@ def expand_compact_layers(module: nn.Module, for_training=False):
         if isinstance(sub, TMQLayer) and hasattr(sub, "tensor_type") and getattr(sub, "original_shape", None) is not None:
             if sub.tensor_type in (TensorType.COMPRESSED_TERNARY_32BIT, TensorType.COMPACT_TERNARY_32BIT):
                 entropy = sub.tensor_type == TensorType.COMPRESSED_TERNARY_32BIT
-                full = ops.expand_ternary(sub.weight.data, sub.original_shape, entropy)
+                full = _b.expand_ternary(sub.weight.data, sub.original_shape, entropy)
                 sub.weight = nn.Parameter(full, requires_grad=for_training)
                 sub.tensor_type = TensorType.FLOAT_32BIT
                 sub.compact = False
