@@ -245,6 +245,21 @@ int tmq_conv2d_out_hw(const tmq_conv_shape *s, int32_t *ho, int32_t *wo);
 int tmq_ternary_conv2d(const void *x, const tmq_conv_shape *shape, const void *native,
                        const tmq_epilogue *epilogue, void *y, void *stream);
 
+/* Depthwise ternary convolution (groups == channels; shape->N must equal shape->C). x: fp16 NHWC;
+ * words: the reference packing of a [C][1][ky][kx] weight tensor, words[ky*kx][ceil(C/16)]
+ * (tmq_pack_ternary with N = C, K = ky*kx) -- read directly, no re-tiling; y: NHWC in
+ * epilogue->y_dtype. Replaces the unfold + ternary_dwconv_cuda + fold branch of
+ * Conv2d.compact_forward (tmq/tmq.py:849-853; kernel tmq/tmq_cuda.cu:166-238, host 607-642) without
+ * materialising the patches.                                                                    */
+int tmq_ternary_dwconv2d(const void *x, const tmq_conv_shape *shape, const uint32_t *words,
+                         const tmq_epilogue *epilogue, void *y, void *stream);
+
+/* The same arithmetic on unfolded patches, the calling convention of ternary_dwconv_cuda
+ * (tmq/tmq_cuda.cu:607-642): x [P][taps][C] (TMQ_F32 or TMQ_F16), y fp32 [P][C],
+ * y[p][c] = sum_t x[p][t][c] * T[c][t].                                                         */
+int tmq_ternary_dwconv_patches(const void *x, int x_dtype, int64_t P, int32_t taps, int64_t C,
+                               const uint32_t *words, float *y, void *stream);
+
 /* ------------------------------------------------------------------------------------------
  * Host entropy codec for packed tensors (host memory in, host memory out; no GPU involved).
  * ---------------------------------------------------------------------------------------- */

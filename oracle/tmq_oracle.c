@@ -353,6 +353,24 @@ void tmq_oracle_gemm(const float *x, int64_t M, int64_t K, const uint32_t *wp, i
     free(t);
 }
 
+/* Depthwise convolution on unfolded patches, the arithmetic of ternaryDWConvFP32
+ * (tmq/tmq_cuda.cu:166-238): x [P][T][C], weights packed as words[t][ceil(C/16)] (the layout
+ * compactTernaryConvKernel, tmq/tmq_native.cpp:279-294, gives a [C][1][ky][kx] tensor), y [P][C]:
+ * y[p][c] = sum_t x[p][t][c] * T[c][t]. fp64 accumulation.                                      */
+void tmq_oracle_dwconv_patches(const float *x, int64_t P, int64_t T, int64_t C, const uint32_t *wp, double *y) {
+    int64_t Q = (C + 15) / 16;
+    for (int64_t p = 0; p < P; p++)
+        for (int64_t c = 0; c < C; c++) {
+            double acc = 0.0;
+            for (int64_t t = 0; t < T; t++) {
+                uint32_t word = wp[t * Q + c / 16];
+                float w = value_from_code((int)((word >> (2 * (15 - (c % 16)))) & 3u), 0);
+                acc += (double)x[(p * T + t) * C + c] * (double)w;
+            }
+            y[p * C + c] = acc;
+        }
+}
+
 /* Direct convolution, NCHW input, weights packed as [C*ky*kx][ceil(N/16)] with row
  * (c*ky + y)*kx + x -- the ordering of F.unfold used at tmq/tmq.py:857-859. Output NCHW fp64.
  * Output size is PyTorch's floor((h + 2p - d(k-1) - 1)/s) + 1.                               */

@@ -44,6 +44,7 @@ def lib():
         L.tmq_oracle_gemm.argtypes = [_f32p, _i64, _i64, _u32p, _i64, ctypes.c_void_p, ctypes.c_void_p, _f64p]
         L.tmq_oracle_conv2d.argtypes = [_f32p] + [_i64] * 4 + [_u32p] + [_i64] * 9 + [ctypes.c_void_p,
                                                                                      ctypes.c_void_p, _f64p]
+        L.tmq_oracle_dwconv_patches.argtypes = [_f32p, _i64, _i64, _i64, _u32p, _f64p]
         L.tmq_oracle_compress.argtypes = [_u32p, _i64, _i64, ctypes.POINTER(ctypes.POINTER(ctypes.c_uint8))]
         L.tmq_oracle_compress.restype = _i64
         L.tmq_oracle_free.argtypes = [ctypes.c_void_p]
@@ -167,6 +168,16 @@ def conv2d(x, words, N, k, stride, pad, dil=(1, 1), scale=None, bias=None):
     s, sp = _opt(scale); b, bp = _opt(bias)
     lib().tmq_oracle_conv2d(x.reshape(-1), B, C, H, W, words.reshape(-1), N, ky, kx, sy, sx, py, px, dy, dx, sp, bp,
                             y.reshape(-1))
+    return y
+
+
+def dwconv_patches(x, words):
+    """x [P][T][C] -> fp64 [P][C] (depthwise: one ternary filter of T taps per channel)."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    P, T, C = x.shape
+    words = np.ascontiguousarray(words, dtype=np.uint32)
+    y = np.empty((P, C), dtype=np.float64)
+    lib().tmq_oracle_dwconv_patches(x.reshape(-1), P, T, C, words.reshape(-1), y.reshape(-1))
     return y
 
 

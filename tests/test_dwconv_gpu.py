@@ -1,0 +1,84 @@
+"""Depthwise ternary convolution (groups == channels) through the C ABI: the patch form against the CPU
+oracle, the image form against the patch form / torch's grouped convolution, the layer API end to end."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _ternary(rng, shape, p0=0.5):
+    u = rng.random(shape)
+    return np.where(u < (1 - p0) / 2, 1.0, np.where(u < 1 - p0, -1.0, 0.0)).astype(np.float32)
+
+
+@pytest.mark.parametrize("P,T,C", [(1, 1, 1), (7, 9, 16), (50, 9, 40), (33, 25, 8), (100, 4, 5), (64, 9, 96)])
+def test_patches_form_matches_oracle(cuda, oracle, P, T, C):
+    from tmq_amd import ops
+    rng = np.random.default_rng(P + T + C)
+    W = _ternary(rng, (C, 1, T, 1))
+    words = oracle.pack(W.reshape(C, T))                         # [T][ceil(C/16)]
+    x = rng.standard_normal((P, T, C)).astype(np.float32)
+    want = oracle.dwconv_patches(x, words)
+    tw = torch.from_numpy(words.view(np.int32)).to(cuda)
+    assert torch.equal(ops.compactify_ternary(torch.from_numpy(W).to(cuda)).view(-1), tw.view(-1))
+    for tx, tol in ((torch.from_numpy(x), 2e-6), (torch.from_numpy(x).half(), 1e-3)):
+        got = ops.ternary_dwconv_cuda(tx.to(cuda).view(1, P, T * C), tw, 1, T, C)
+        assert tuple(got.shape) == (1, P, C) and got.dtype == torch.float32
+        err = np.max(np.abs(got.cpu().numpy().reshape(P, C) - want)) / max(1e-30, np.max(np.abs(want)))
+        assert err <= tol
+    ext = ops.ext
+    if ext is not None:
+        assert torch.equal(ext.ternary_dwconv_cuda(torch.from_numpy(x).to(cuda).view(1, P, T * C), tw, 1, T, C),
+                           ops.ternary_dwconv_cuda(torch.from_numpy(x).to(cuda).view(1, P, T * C), tw, 1, T, C))
+
+
+@pytest.mark.parametrize("B,C,H,W,k,stride,pad,dil", [
+    (2, 16, 9, 9, 3, 1, 1, 1), (1, 40, 12, 11, (3, 5), (2, 1), (1, 2), 1), (3, 8, 7, 7, 3, 2, 0, 1),
+    (2, 5, 6, 6, 3, 1, 1, 1), (1, 96, 14, 14, 3, 1, 2, 2), (2, 32, 8, 8, 5, 1, ((2, 1), (0, 3)), 1),
+])
+def test_image_form_exact_on_integers(cuda, B, C, H, W, k, stride, pad, dil):
+    """Small-integer activations: every product and sum is exact, so the result must equal torch's
+    grouped convolution on the expanded weights bit for bit; then scale / bias / residual / ReLU / fp16."""
+    from tmq_amd import ops
+    pair = lambda v: tuple(v) if isinstance(v, (tuple, list)) else (v, v)
+    k, stride, dil = pair(k), pair(stride), pair(dil)
+    g = torch.Generator(device=cuda).manual_seed(B + C + H)
+    Wt = torch.randint(-1, 2, (C, 1, k[0], k[1]), device=cuda, generator=g).float()
+    x = torch.randint(-4, 5, (B, C, H, W), device=cuda, generator=g).float()
+    words = ops.compactify_ternary(Wt)
+    assert tuple(words.shape) == (1, k[0], k[1], (C + 15) // 16)
+    y = ops.ternary_dwconv2d(x.half(), words, k, stride, pad, dil)
+    if isinstance(pad, tuple) and isinstance(pad[0], tuple):
+        (pt, pb), (pl, pr) = pad
+        ref = torch.nn.functional.conv2d(torch.nn.functional.pad(x, (pl, pr, pt, pb)), Wt, None, stride, 0, dil, groups=C)
+    else:
+        ref = torch.nn.functional.conv2d(x, Wt, None, stride, pad, dil, groups=C)
+    assert y.shape == ref.shape and y.is_contiguous(memory_format=torch.channels_last)
+    assert torch.equal(y, ref)
+    scale = torch.pow(2.0, torch.randint(-2, 3, (C,), device=cuda, generator=g).float())
+    bias = torch.randint(-9, 10, (C,), device=cuda, generator=g).float()
+    res = torch.randint(-5, 6, ref.shape, device=cuda, generator=g).half().contiguous(memory_format=torch.channels_last)
+    y16 = ops.ternary_dwconv2d(x.half(), words, k, stride, pad, dil, scale, bias, residual=res, relu=True,
+                               out_dtype=torch.float16)
+    want = torch.relu(ref * scale.view(1, -1, 1, 1) + bias.view(1, -1, 1, 1) + res.float())
+    assert y16.dtype == torch.float16 and torch.equal(y16.float(), want.half().float())
+
+
+def test_depthwise_layer_compact_inference(cuda):
+    """quantize_model -> ternarise -> compressed_state_dict switches a depthwise Conv2d to compact
+    weights; its compact forward must equal the float forward on the ternarised weights."""
+    import tmq_amd as t
+    torch.manual_seed(3)
+    net = torch.nn.Sequential(torch.nn.Conv2d(24, 24, 3, 1, 1, groups=24, bias=True), torch.nn.ReLU(),
+                              torch.nn.Conv2d(24, 10, 1, bias=False))
+    ctrl = t.QuantizationControl()
+    t.quantize_model(net, ctrl)
+    net.to(cuda).eval()
+    x = torch.randint(-3, 4, (2, 24, 10, 10), device=cuda).float()
+    ctrl.quantize()
+    want = net(x)
+    t.compressed_state_dict(net, strong=False)
+    assert net[0].weight.dtype == torch.int32
+    got = net(x)
+    assert torch.allclose(got, want, rtol=1e-3, atol=1e-3)

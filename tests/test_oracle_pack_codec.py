@@ -243,3 +243,15 @@ def test_torch_extension_exports_the_reference_names():
         assert words.shape == compact.shape and np.array_equal(_u32(words), _u32(compact))
         assert np.array_equal(ext.compress_ternary(torch.from_numpy(compact.view(np.int32).copy()), list(w.shape), True).numpy().view(np.uint8),
                               stream.view(np.uint8))
+
+
+def test_oracle_depthwise_patches_is_the_textbook_sum(oracle):
+    """y[p][c] = sum_t x[p][t][c] T[c][t] against numpy's einsum on the unpacked weights, ragged C."""
+    rng = np.random.default_rng(9)
+    for (P, T, C) in [(5, 9, 16), (3, 4, 5), (11, 25, 40), (2, 1, 1)]:
+        u = rng.random((C, T))
+        W = np.where(u < .25, 1.0, np.where(u < .5, -1.0, 0.0)).astype(np.float32)
+        words = oracle.pack(W)                                   # [T][ceil(C/16)]
+        x = rng.standard_normal((P, T, C)).astype(np.float32)
+        want = np.einsum("ptc,ct->pc", x.astype(np.float64), W.astype(np.float64))
+        assert np.allclose(oracle.dwconv_patches(x, words), want, rtol=0, atol=1e-12)

@@ -1,0 +1,197 @@
+// Depthwise ternary convolution (groups == channels) on 2-bit packed weights, gfx950.
+//
+//   y[p][c] = epilogue( sum_t x(p, t, c) * T[c][t] ),   t = (i, j) over the ky x kx taps
+//
+// The weight tensor [C][1][ky][kx] is packed by the reference as words[t][ceil(C/16)]
+// (tmq/tmq_native.cpp:279-294 with one input channel): word (t, q) holds the codes of channels
+// 16 q .. 16 q + 15 at tap t, first channel in bits 31:30. The kernels read that format directly.
+//
+// One multiply-add per input element: the op is bound by HBM traffic (2 B in / output element and
+// tap on a cold cache, far less with the taps' overlap served from L2), not by arithmetic. A thread
+// owns 8 consecutive channels of one output position -- 16-byte fp16 loads, neighbouring threads on
+// neighbouring channel groups -- and applies a weight as two selects on the sign / nonzero bits.
+//
+// Two sources of x:
+//   * NHWC image (tmq_ternary_dwconv2d): taps are gathered on the fly, padding reads as zero;
+//   * unfolded patches [P][T][C] fp32, the calling convention of the reference's
+//     ternary_dwconv_cuda (tmq/tmq_cuda.cu:166-238, host 607-642; caller tmq/tmq.py:849-853).
+#include "common.h"
+#include "mfma.h"
+
+namespace tmq {
+namespace {
+
+struct DwEpilogue {
+    const float *scale, *bias;
+    const void *residual;
+    void *y;
+    int relu, y_f16;
+};
+
+// codes of 8 consecutive channels starting at c0 (a multiple of 8) from the word that holds them:
+// returns them left-aligned, channel c0 in bits 31:30
+__device__ __forceinline__ uint32_t codes8(const uint32_t *__restrict__ words, int64_t Q, int t, int64_t c0) {
+    const uint32_t w = words[(int64_t)t * Q + (c0 >> 4)];
+    return (c0 & 8) ? (w << 16) : w;
+}
+
+// value * {+1, -1, 0} for the code in bits 31:30 of `codes` (01 -> +1, 10 -> -1, 00 / 11 -> 0)
+__device__ __forceinline__ float apply_code(float v, uint32_t codes) {
+    const uint32_t c = codes >> 30;
+    return c == 1u ? v : (c == 2u ? -v : 0.0f);
+}
+
+__device__ __forceinline__ void store8(const DwEpilogue &ep, int64_t o, int64_t c0, int64_t C, float (&acc)[8], bool vec) {
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+        if (c0 + e >= C) break;
+        float v = acc[e];
+        if (ep.scale) v *= ep.scale[c0 + e];
+        if (ep.bias) v += ep.bias[c0 + e];
+        if (ep.residual)
+            v += ep.y_f16 ? (float)static_cast<const _Float16 *>(ep.residual)[o + e] : static_cast<const float *>(ep.residual)[o + e];
+        if (ep.relu) v = v > 0.f ? v : 0.f;
+        acc[e] = v;
+    }
+    if (vec) {
+        if (ep.y_f16) {
+            half8 h;
+#pragma unroll
+            for (int e = 0; e < 8; e++) h[e] = (_Float16)acc[e];
+            *reinterpret_cast<half8 *>(static_cast<_Float16 *>(ep.y) + o) = h;
+        } else {
+            float *yp = static_cast<float *>(ep.y) + o;
+            *reinterpret_cast<floatx4 *>(yp) = floatx4{acc[0], acc[1], acc[2], acc[3]};
+            *reinterpret_cast<floatx4 *>(yp + 4) = floatx4{acc[4], acc[5], acc[6], acc[7]};
+        }
+    } else {
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            if (c0 + e >= C) break;
+            if (ep.y_f16) static_cast<_Float16 *>(ep.y)[o + e] = (_Float16)acc[e];
+            else static_cast<float *>(ep.y)[o + e] = acc[e];
+        }
+    }
+}
+
+// NHWC fp16 image. grid.x covers P * ceil(C / 8) threads.
+__global__ __launch_bounds__(256) void dwconv_image_kernel(const _Float16 *__restrict__ x, const uint32_t *__restrict__ words,
+                                                           int B, int C, int H, int W, int Ho, int Wo, int ky, int kx,
+                                                           int sy, int sx, int py, int px, int dy, int dx, int vec,
+                                                           DwEpilogue ep) {
+    const int64_t G = (C + 7) / 8, Q = (C + 15) / 16;
+    const int64_t id = (int64_t)blockIdx.x * 256 + threadIdx.x, total = (int64_t)B * Ho * Wo * G;
+    if (id >= total) return;
+    const int64_t p = id / G, c0 = (id - p * G) * 8;
+    const int ow = (int)(p % Wo);
+    const int64_t r = p / Wo;
+    const int oh = (int)(r % Ho), b = (int)(r / Ho);
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    for (int i = 0; i < ky; i++) {
+        const int ih = oh * sy - py + i * dy;
+        if (ih < 0 || ih >= H) continue;
+        for (int j = 0; j < kx; j++) {
+            const int iw = ow * sx - px + j * dx;
+            if (iw < 0 || iw >= W) continue;
+            const _Float16 *src = x + (((int64_t)b * H + ih) * W + iw) * C + c0;
+            uint32_t codes = codes8(words, Q, i * kx + j, c0);
+            if (vec) {
+                const half8 v = *reinterpret_cast<const half8 *>(src);
+#pragma unroll
+                for (int e = 0; e < 8; e++) acc[e] += apply_code((float)v[e], codes << (2 * e));
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; e++)
+                    if (c0 + e < C) acc[e] += apply_code((float)src[e], codes << (2 * e));
+            }
+        }
+    }
+    store8(ep, p * C + c0, c0, C, acc, vec);
+}
+
+// Unfolded patches [P][T][C], fp32 (the reference's calling convention) or fp16.
+template <typename T>
+__global__ __launch_bounds__(256) void dwconv_patches_kernel(const T *__restrict__ x, const uint32_t *__restrict__ words,
+                                                             int64_t P, int taps, int64_t C, int vec, DwEpilogue ep) {
+    const int64_t G = (C + 7) / 8, Q = (C + 15) / 16;
+    const int64_t id = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (id >= P * G) return;
+    const int64_t p = id / G, c0 = (id - p * G) * 8;
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    for (int t = 0; t < taps; t++) {
+        const T *src = x + (p * taps + t) * C + c0;
+        const uint32_t codes = codes8(words, Q, t, c0);
+        float v[8];
+        if (vec) {
+            if constexpr (sizeof(T) == 4) {
+                const floatx4 a = *reinterpret_cast<const floatx4 *>(src), b = *reinterpret_cast<const floatx4 *>(src + 4);
+#pragma unroll
+                for (int e = 0; e < 4; e++) { v[e] = a[e]; v[4 + e] = b[e]; }
+            } else {
+                const half8 h = *reinterpret_cast<const half8 *>(src);
+#pragma unroll
+                for (int e = 0; e < 8; e++) v[e] = (float)h[e];
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; e++) v[e] = c0 + e < C ? (float)src[e] : 0.f;
+        }
+#pragma unroll
+        for (int e = 0; e < 8; e++) acc[e] += apply_code(v[e], codes << (2 * e));
+    }
+    store8(ep, p * C + c0, c0, C, acc, vec);
+}
+
+bool aligned_for(const void *p, size_t bytes) { return (reinterpret_cast<uintptr_t>(p) % bytes) == 0; }
+
+}  // namespace
+}  // namespace tmq
+
+using namespace tmq;
+
+extern "C" {
+
+int tmq_ternary_dwconv2d(const void *x, const tmq_conv_shape *s, const uint32_t *words, const tmq_epilogue *epilogue,
+                         void *y, void *stream) {
+    if (!s || !x || !words || !y) return TMQ_ERR_INVALID_ARG;
+    if (s->N != s->C) return TMQ_ERR_INVALID_ARG;                 // depthwise: one filter per channel
+    tmq_epilogue e = {nullptr, nullptr, nullptr, 0, TMQ_F32};
+    if (epilogue) e = *epilogue;
+    if (e.y_dtype != TMQ_F16 && e.y_dtype != TMQ_F32) return TMQ_ERR_UNSUPPORTED;
+    int32_t ho, wo;
+    int rc = tmq_conv2d_out_hw(s, &ho, &wo);
+    if (rc != TMQ_OK) return rc;
+    if (s->B < 0 || s->C <= 0 || s->H <= 0 || s->W <= 0 || ho <= 0 || wo <= 0) return TMQ_ERR_INVALID_ARG;
+    const int64_t total = (int64_t)s->B * ho * wo * ((s->C + 7) / 8), blocks = (total + 255) / 256;
+    if (total == 0) return TMQ_OK;
+    if (blocks > 0x7FFFFFFF) return TMQ_ERR_TOO_LARGE;
+    const int y_f16 = e.y_dtype == TMQ_F16;
+    const size_t ya = y_f16 ? 16 : 16;
+    const int vec = (s->C % 8 == 0) && aligned_for(x, 16) && aligned_for(y, ya) && (!e.residual || aligned_for(e.residual, ya));
+    DwEpilogue ep{e.scale, e.bias, e.residual, y, e.relu, y_f16};
+    hipLaunchKernelGGL(dwconv_image_kernel, dim3((uint32_t)blocks), dim3(256), 0, as_stream(stream),
+                       static_cast<const _Float16 *>(x), words, s->B, s->C, s->H, s->W, ho, wo, s->ky, s->kx, s->sy, s->sx,
+                       s->py, s->px, s->dy, s->dx, vec, ep);
+    return check_launch();
+}
+
+int tmq_ternary_dwconv_patches(const void *x, int x_dtype, int64_t P, int32_t taps, int64_t C, const uint32_t *words,
+                               float *y, void *stream) {
+    if (P < 0 || taps <= 0 || C <= 0) return TMQ_ERR_INVALID_ARG;
+    if (P == 0) return TMQ_OK;
+    if (!x || !words || !y) return TMQ_ERR_INVALID_ARG;
+    if (x_dtype != TMQ_F32 && x_dtype != TMQ_F16) return TMQ_ERR_UNSUPPORTED;
+    const int64_t total = P * ((C + 7) / 8), blocks = (total + 255) / 256;
+    if (blocks > 0x7FFFFFFF) return TMQ_ERR_TOO_LARGE;
+    const int vec = (C % 8 == 0) && aligned_for(x, 16) && aligned_for(y, 16);
+    DwEpilogue ep{nullptr, nullptr, nullptr, y, 0, 0};
+    if (x_dtype == TMQ_F32)
+        hipLaunchKernelGGL(dwconv_patches_kernel<float>, dim3((uint32_t)blocks), dim3(256), 0, as_stream(stream),
+                           static_cast<const float *>(x), words, P, (int)taps, C, vec, ep);
+    else
+        hipLaunchKernelGGL(dwconv_patches_kernel<_Float16>, dim3((uint32_t)blocks), dim3(256), 0, as_stream(stream),
+                           static_cast<const _Float16 *>(x), words, P, (int)taps, C, vec, ep);
+    return check_launch();
+}
+
+}  // extern "C"

@@ -147,11 +147,33 @@ torch::Tensor ternary_mvm_cuda(torch::Tensor vector, torch::Tensor weights, int6
     return y;
 }
 
-// Depthwise variants (tmq/tmq_cuda.cu:607-686): the reference's own hosts mis-size their outputs and are
-// not reachable from a working model; not built here.
-torch::Tensor ternary_dwconv_cuda(torch::Tensor, torch::Tensor, int64_t, int64_t, int64_t) {
-    TORCH_CHECK(false, "ternary_dwconv_cuda: not implemented on this build");
+// Depthwise convolution on the unfolded input (tmq/tmq_cuda.cu:607-642, caller tmq/tmq.py:849-853):
+// in [..., positions, ky * kx * channels] (tap-major, channel fastest), weights = compact words of the
+// [channels, 1, ky, kx] kernel; out [..., positions, channels], out[p][c] = sum_t in[p][t C + c] T[c][t].
+torch::Tensor ternary_dwconv_cuda(torch::Tensor input, torch::Tensor weights, int64_t kx, int64_t ky, int64_t channels) {
+    TORCH_CHECK(input.device().is_cuda() && weights.device().is_cuda(), "ternary_dwconv_cuda: expected tensors on the GPU");
+    TORCH_CHECK(input.scalar_type() == torch::kFloat32 || input.scalar_type() == torch::kFloat16,
+                "ternary_dwconv_cuda: expected fp32 (or fp16) input");
+    const int64_t taps = kx * ky;
+    TORCH_CHECK(weights.scalar_type() == torch::kInt32 && weights.numel() == taps * ((channels + 15) / 16),
+                "ternary_dwconv_cuda: compact weights do not match kernel size and channels");
+    TORCH_CHECK(input.dim() >= 2 && input.size(-1) == taps * channels,
+                "ternary_dwconv_cuda: the last dimension must be ky * kx * channels");
+    const c10::DeviceGuard guard(input.device());
+    auto x = input.contiguous();
+    auto w = weights.contiguous();
+    std::vector<int64_t> shape = input.sizes().vec();
+    shape.back() = channels;
+    auto y = torch::empty(shape, input.options().dtype(torch::kFloat32));
+    const int64_t P = x.numel() / (taps * channels);
+    check(tmq_ternary_dwconv_patches(x.data_ptr(), x.scalar_type() == torch::kFloat16 ? TMQ_F16 : TMQ_F32, P, (int32_t)taps,
+                                     channels, reinterpret_cast<const uint32_t *>(w.data_ptr<int32_t>()),
+                                     y.data_ptr<float>(), stream_of(x)), "ternary_dwconv_cuda");
+    return y;
 }
+
+// Transposed depthwise variant (tmq/tmq_cuda.cu:645-686): the reference's host mis-sizes its output and
+// no working model reaches it; not built here.
 torch::Tensor ternary_dwconvtrans_cuda(torch::Tensor, torch::Tensor, int64_t, int64_t) {
     TORCH_CHECK(false, "ternary_dwconvtrans_cuda: not implemented on this build");
 }

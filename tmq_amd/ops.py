@@ -444,6 +444,67 @@ def ternary_conv2d(x: torch.Tensor, nw: NativeWeights, stride=1, padding=0, dila
     return y
 
 
+class _Channels:
+    """What _epilogue needs to know about a depthwise layer: its channel count."""
+    def __init__(self, n):
+        self.N = n
+
+
+def ternary_dwconv2d(x: torch.Tensor, words: torch.Tensor, kernel, stride=1, padding=0, dilation=1, scale=None,
+                     bias=None, residual=None, relu=False, out_dtype=torch.float32) -> torch.Tensor:
+    """Depthwise ternary convolution (groups == channels) straight from the compact words of a
+    [C, 1, ky, kx] weight tensor (int32 [1, ky, kx, ceil(C/16)] as compactify_ternary returns them).
+    x: fp16 [B, C, H, W] in channels_last memory (anything else is converted first); returns
+    [B, C, Ho, Wo] in channels_last memory."""
+    pair = lambda v: tuple(v) if isinstance(v, (tuple, list)) else (v, v)
+    (ky, kx), (sy, sx), (py, px), (dy, dx) = pair(kernel), pair(stride), pair(padding), pair(dilation)
+    (py, py_end), (px, px_end) = pair(py), pair(px)
+    if not x.is_cuda or x.dim() != 4:
+        raise RuntimeError("ternary_dwconv2d: expected a 4-D GPU tensor")
+    B, C, H, W = x.shape
+    _capi.require_gpu(words, "words")
+    if words.dtype != torch.int32 or words.numel() != ky * kx * ((C + 15) // 16):
+        raise RuntimeError("ternary_dwconv2d: expected the int32 compact words of a [C, 1, ky, kx] weight tensor")
+    if x.dtype != torch.float16 or not x.is_contiguous(memory_format=torch.channels_last):
+        x = x.to(dtype=torch.float16, memory_format=torch.channels_last)
+    words = words.contiguous()
+    shp = _capi.ConvShape(B, C, H, W, C, ky, kx, sy, sx, py, px, dy, dx, py_end, px_end)
+    ho, wo = ctypes.c_int32(0), ctypes.c_int32(0)
+    lib = _lib()
+    check(lib.tmq_conv2d_out_hw(ctypes.byref(shp), ctypes.byref(ho), ctypes.byref(wo)), "conv2d_out_hw")
+    if ho.value <= 0 or wo.value <= 0:
+        raise RuntimeError("ternary_dwconv2d: empty output")
+    y = torch.empty((B, C, ho.value, wo.value), dtype=out_dtype, device=x.device, memory_format=torch.channels_last)
+    ep = _epilogue(_Channels(C), scale, bias, residual, relu, out_dtype, y)
+    with torch.cuda.device(x.device):
+        check(lib.tmq_ternary_dwconv2d(ptr(x), ctypes.byref(shp), ptr(words), ctypes.byref(ep), ptr(y), stream_of(x)),
+              "ternary_dwconv2d")
+    return y
+
+
+def ternary_dwconv_cuda(input: torch.Tensor, weights: torch.Tensor, kx: int, ky: int, channels: int) -> torch.Tensor:
+    """The reference's binding (tmq/tmq_cuda.cu:607-642, caller tmq/tmq.py:849-853): input is the
+    unfolded tensor [..., positions, ky * kx * channels] (tap-major, channel fastest), weights the
+    compact words of the [channels, 1, ky, kx] kernel; returns [..., positions, channels] fp32 with
+    out[p][c] = sum_t input[p][t * channels + c] * T[c][t]."""
+    if not input.is_cuda or not weights.is_cuda:
+        raise RuntimeError("ternary_dwconv_cuda: expected tensors on the GPU")
+    if input.dtype not in (torch.float32, torch.float16):
+        raise RuntimeError("ternary_dwconv_cuda: expected fp32 (or fp16) input")
+    taps = int(kx) * int(ky)
+    if weights.dtype != torch.int32 or weights.numel() != taps * ((channels + 15) // 16):
+        raise RuntimeError("ternary_dwconv_cuda: compact weights do not match kernel size and channels")
+    if input.dim() < 2 or input.shape[-1] != taps * channels:
+        raise RuntimeError("ternary_dwconv_cuda: the last dimension must be ky * kx * channels")
+    x = input.contiguous()
+    P = x.numel() // (taps * channels)
+    y = torch.empty(tuple(input.shape[:-1]) + (channels,), dtype=torch.float32, device=x.device)
+    with torch.cuda.device(x.device):
+        check(_lib().tmq_ternary_dwconv_patches(ptr(x), _capi.dtype_code(x), P, taps, channels, ptr(weights.contiguous()),
+                                                ptr(y), stream_of(x)), "ternary_dwconv_cuda")
+    return y
+
+
 def _check_mm_args(lhs, weights, columns, name):
     # tmq/tmq_cuda.cu:480-490, 566-575
     if not lhs.is_cuda or not weights.is_cuda:

@@ -609,9 +609,14 @@ class Conv2d(nn.Module, TMQLayer):
             raise Exception("Expected a 3D tensor")
         assert self.groups == 1 or self.groups == self.original_shape[0], \
             "Grouped convolutions are only supported for group == channels"
-        if self.groups != 1:
-            raise NotImplementedError("depthwise compact inference is not part of this build")
         ky, kx = _pair(self.kernel)
+        if self.groups != 1:
+            # depthwise (tmq/tmq.py:849-853): the compact words are read as they are, no re-tiling
+            if self.original_shape[1] != 1 or x.shape[1] != self.original_shape[0]:
+                raise RuntimeError("depthwise compact inference needs one filter per input channel")
+            bias = self.bias.data.float() if self.bias is not None else None
+            return ops.ternary_dwconv2d(x, self.weight.data, (ky, kx), _pair(self.stride), _pair(self.padding),
+                                        _pair(self.dilation), scale=self._epilogue_scale(x.shape[1], x.device), bias=bias)
         nw = self._native_weights(conv_kernel=(ky, kx))
         bias = self.bias.data.float() if self.bias is not None else None
         return ops.ternary_conv2d(x, nw, _pair(self.stride), _pair(self.padding), _pair(self.dilation),
