@@ -82,3 +82,25 @@ def test_depthwise_layer_compact_inference(cuda):
     assert net[0].weight.dtype == torch.int32
     got = net(x)
     assert torch.allclose(got, want, rtol=1e-3, atol=1e-3)
+
+
+@pytest.mark.parametrize("cin,cout,k,stride,pad,opad,dil", [(16, 8, 3, 2, 1, 1, 1), (24, 40, 2, 2, 0, 0, 1),
+                                                            (8, 8, 3, 1, 1, 0, 1), (32, 5, (3, 2), (2, 1), (1, 0), 0, 1)])
+def test_transposed_layer_compact_inference(cuda, cin, cout, k, stride, pad, opad, dil):
+    """ConvTranspose2d: the compact forward (GEMM on re-packed weights + fold) must equal the float
+    forward on the ternarised weights; small integers make that exact."""
+    import tmq_amd as t
+    torch.manual_seed(cin + cout)
+    net = torch.nn.Sequential(torch.nn.ConvTranspose2d(cin, cout, k, stride, pad, output_padding=opad, bias=True, dilation=dil))
+    ctrl = t.QuantizationControl()
+    t.quantize_model(net, ctrl)
+    net.to(cuda).eval()
+    with torch.no_grad():
+        net[0].bias.copy_(torch.randint(-4, 5, (cout,)).float())
+    x = torch.randint(-3, 4, (2, cin, 6, 5), device=cuda).float()
+    ctrl.quantize()
+    want = net(x)
+    t.compressed_state_dict(net, strong=False)
+    assert net[0].weight.dtype == torch.int32
+    got = net(x)
+    assert got.shape == want.shape and torch.equal(got, want)

@@ -655,9 +655,8 @@ class Conv2d(nn.Module, TMQLayer):
 
 
 class ConvTranspose2d(Conv2d):
-    """Quantization-aware drop-in for nn.ConvTranspose2d (tmq/tmq.py:978-1087). Training path only:
-    the reference's compact path for this layer cannot pass its own shape checks, and no compact
-    kernel is provided here."""
+    """Quantization-aware drop-in for nn.ConvTranspose2d (tmq/tmq.py:978-1087), with a working compact
+    path for groups == 1 (the reference's own cannot pass its shape checks)."""
 
     _transposed = True
 
@@ -671,15 +670,50 @@ class ConvTranspose2d(Conv2d):
         return "ConvTranspose2d(%d,%d,%d,%d) [tmq] " % tuple(self.original_shape) + " <%s>" % self.layer_name
 
     def _conv(self, x, w, bias):
-        return nn.functional.conv_transpose2d(x, w, bias, self.stride, self.padding, dilation=self.dilation,
-                                              groups=self.groups)
+        # output_padding is honoured (the reference's forward drops it, tmq/tmq.py:989-1003, and then
+        # disagrees with the nn.ConvTranspose2d it replaced)
+        return nn.functional.conv_transpose2d(x, w, bias, self.stride, self.padding, self.output_padding,
+                                              groups=self.groups, dilation=self.dilation)
 
     def _weight_shape(self, ky, kx):
         return [self.in_channels, self.out_channels // self.groups, ky, kx]
 
     @torch.no_grad()
     def compact_forward(self, x):
-        raise NotImplementedError("compact inference for ConvTranspose2d is not part of this build")
+        """Transposed convolution from the packed weights as GEMM + col2im: cols[b, (co, i, j), p] =
+        sum_ci x[b, ci, p] W[ci, co, i, j], then F.fold scatters the columns (the plan of
+        tmq/tmq.py:1005-1038, whose own shape checks reject its weight view). The compact tensor of a
+        [Cin, Cout, ky, kx] kernel packs along Cin, the reduction index here, so it is unpacked and
+        re-packed along (co, i, j) once per layer. groups == 1 only."""
+        assert not self.training, "Compact inference is not supported in training mode"
+        assert self.weight.data.dtype == torch.int32, "Compact inference requires 32-bit integer words"
+        self._update_scale()
+        if x.dim() == 3:
+            return self.compact_forward(x.unsqueeze(0)).squeeze(0)
+        if self.groups != 1:
+            raise NotImplementedError("grouped transposed compact inference is not part of this build")
+        cin, cout, ky, kx = (int(v) for v in self.original_shape)
+        w = self.weight.data
+        key = (w.data_ptr(), tuple(w.shape), w._version)
+        if self._native is None or self._native[0] != key:
+            full = ops.expand_ternary(w, [cin, cout, ky, kx])                     # [Cin, Cout, ky, kx]
+            words = ops.compactify_ternary(full.reshape(cin, cout * ky * kx).t().contiguous())   # [Cin][ceil(N/16)]
+            self._native = (key, ops.NativeWeights(words, cout * ky * kx))
+        nw = self._native[1]
+        B, C, H, W = x.shape
+        sy, sx = _pair(self.stride)
+        py, px = _pair(self.padding)
+        oy, ox = _pair(self.output_padding)
+        dy, dx = _pair(self.dilation)
+        h_out = (H - 1) * sy - 2 * py + dy * (ky - 1) + 1 + oy
+        w_out = (W - 1) * sx - 2 * px + dx * (kx - 1) + 1 + ox
+        lhs = x.permute(0, 2, 3, 1).reshape(B * H * W, C)
+        cols = ops.ternary_linear(lhs.contiguous(), nw, scale=self._epilogue_scale(nw.N, x.device))
+        final = nn.functional.fold(cols.view(B, H * W, nw.N).permute(0, 2, 1), output_size=(h_out, w_out),
+                                   kernel_size=(ky, kx), dilation=(dy, dx), stride=(sy, sx), padding=(py, px))
+        if self.bias is not None:
+            final = final + self.bias.view(1, -1, 1, 1)
+        return final
 
     @classmethod
     def from_transconv2d(cls, source: nn.ConvTranspose2d, name: str, ctrl: QuantizationControl):
