@@ -336,10 +336,38 @@ def bench_resnet_qat(args, torch):
         step()
     torch.cuda.synchronize()
     dt = (time.perf_counter() - t0) / reps
+
+    # The TMQ kernels of one step on their own (GPU time between events): soft-step forward and backward
+    # of each of the 21 layers, the multi-tensor quantization loss and its gradient, the multi-tensor clamp.
+    from tmq_amd import tmq as tmq_mod
+    b = tmq_mod._b
+    ws = [node.weight for node in ctrl._registry.values()]
+    gs = [torch.randn_like(w) for w in ws]
+
+    def tmq_only():
+        for w, g in zip(ws, gs):
+            b.fwd_softstep(w.data, ctrl.digamma)
+            b.bwd_softstep(w.data, ctrl.digamma, 1.0, g)
+        ctrl.quantization_loss().backward()
+        ctrl.clamp()
+
+    for _ in range(3):
+        tmq_only()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        tmq_only()
+    e1.record()
+    torch.cuda.synchronize()
+    tmq_ms = e0.elapsed_time(e1) / reps
+    nbytes = sum(w.numel() for w in ws) * (8 + 12 + 4 + 12 + 8)   # fwd, bwd, loss, loss gradient (accumulating), clamp
     return {"metric": "ResNet-18 QAT step time", "value": round(dt * 1e3, 3), "unit": "ms", "higher_is_better": False,
             "n_gpus": 1, "dtype": "f32", "data": "synthetic",
             "config": {"workload": "configs[4]: ResNet-18 QAT step", "batch": B, "digamma": ctrl.digamma,
-                       "qpenalty": ctrl.qpenalty, "quantized_weights": 11219136}}
+                       "qpenalty": ctrl.qpenalty, "quantized_weights": 11219136},
+            "tmq_kernels_ms": round(tmq_ms, 4), "tmq_share": round(tmq_ms / (dt * 1e3), 4),
+            "tmq_algorithmic_bytes": nbytes, "tmq_gbs": round(nbytes / tmq_ms / 1e6, 1)}
 
 
 def main():
