@@ -4,10 +4,11 @@
 //
 // Work split: a workgroup owns a BM x BN output tile; its WGM x WGN wavefronts each own
 // (16 WM) x (16 WN) of it as WM x WN accumulators of v_mfma_f32_16x16x32_f16 (fp32 accumulate).
-//   * Activations: staged global -> registers -> LDS one 64-wide k-tile ahead of the math (the
-//     next tile's global loads are in flight while the current one is multiplied); LDS rows are
-//     padded to 144 bytes so the 16-byte operand reads of a wavefront are conflict-free. The A
-//     tile is shared by every wavefront of the workgroup.
+//   * Activations: one 64-wide k-tile ahead of the math in LDS, shared by every wavefront of the
+//     workgroup. Aligned shapes (dense rows with K % 64 == 0, convolutions with 8, 16, 32 or a
+//     multiple of 64 channels) are loaded global -> LDS directly (tile_dma_kernel); everything else
+//     goes global -> registers -> LDS with per-element guards (tile_kernel). LDS rows are 128 bytes,
+//     chunks XOR-swizzled so the 16-byte operand reads of a wavefront are conflict-free.
 //   * Weights: never touch LDS. Each lane loads the dword of the kernel-native layout (mfma.h)
 //     that holds exactly its own operand bits and expands it in two VALU ops per register to
 //     +-2/0 fp16. The 2-bit weights are a few hundred KiB per workgroup and stay in L2.
@@ -32,14 +33,6 @@ namespace {
 constexpr int kBK = 64;          // k-tile
 __device__ u32x4 kZeroChunk;              // zero-initialised, never written: what loads of padding taps / k-tiles past K are redirected to
 
-// One load from `p` if `ok`, else from the zero chunk. The empty asm keeps the selected address in a
-// register, so that the compiler issues exactly one load instead of a branch around two.
-__device__ __forceinline__ u32x4 load_or_zero(const u32x4 *p, bool ok) {
-    typedef const __attribute__((address_space(1))) u32x4 *global_ptr;   // stay in the global address space
-    global_ptr q = ok ? (global_ptr)p : (global_ptr)&kZeroChunk;
-    asm volatile("" : "+v"(q));
-    return *q;
-}
 constexpr int kPitch = 64;       // LDS row pitch in halfs: 128 bytes = 8 chunks of 16 bytes, no padding.
 // Chunk c of row r is stored at position c ^ (r & 7): a wavefront's stores cover whole rows
 // (contiguous kilobytes) and the operand reads of 8 consecutive rows at one k offset land in 8
@@ -55,13 +48,17 @@ struct Epilogue {
 };
 
 // ---- loaders ------------------------------------------------------------------------------------------
-// A loader hands every thread CH 16-byte chunks (8 fp16) of the BM x 64 activation tile:
-// chunk i of thread t is row (t / 8 + i * T / 8), k offset (t % 8) * 8.
-//
-// FAST = rows are 16-byte aligned and K is a multiple of the k-tile: no guards in the hot loop
-// (rows past M are clamped to the last row; their results are never stored).
-template <bool FAST>
+// A loader hands every thread CH 16-byte chunks (8 fp16) of the BM x 64 activation tile: chunk i of
+// thread t belongs to row (t / 8 + i * T / 8). Two kinds:
+//   * register loaders (fetch): any shape; values pass through registers, guards in the loop. The
+//     thread's chunk sits at k offset (t % 8) * 8.
+//   * direct loaders (addr): rows are 16-byte aligned and a chunk never straddles the end of K or of a
+//     tap, so a chunk is one address -- the zero chunk for padding -- and can be loaded straight into
+//     LDS. The kernel tells init() which of the row's 8 chunks the thread fetches.
+
+// Dense rows, any K / alignment.
 struct DenseLoader {
+    static constexpr bool kDirect = false;
     const _Float16 *x;
     int64_t M, K;
 
@@ -83,22 +80,47 @@ struct DenseLoader {
     }
     template <int CH, int T>
     __device__ __forceinline__ void fetch(State<CH, T> &st, int64_t k0, u32x4 (&out)[CH]) const {
-        // k-tiles past K are prefetched too (and never multiplied): FAST re-reads the last tile
-        const int64_t k = (FAST && k0 >= K ? K - kBK : k0) + st.kc;
+        const int64_t k = k0 + st.kc;
 #pragma unroll
         for (int i = 0; i < CH; i++) {
-            if constexpr (FAST) {
-                out[i] = *reinterpret_cast<const u32x4 *>(st.row[i] + k);
-            } else {
-                half8 h = {0, 0, 0, 0, 0, 0, 0, 0};
-                if (st.live[i]) {
+            half8 h = {0, 0, 0, 0, 0, 0, 0, 0};
+            if (st.live[i]) {
 #pragma unroll
-                    for (int e = 0; e < 8; e++)
-                        if (k + e < K) h[e] = st.row[i][k + e];
-                }
-                out[i] = __builtin_bit_cast(u32x4, h);
+                for (int e = 0; e < 8; e++)
+                    if (k + e < K) h[e] = st.row[i][k + e];
             }
+            out[i] = __builtin_bit_cast(u32x4, h);
         }
+    }
+    template <int CH, int T>
+    __device__ __forceinline__ void advance(State<CH, T> &) const {}
+};
+
+// Dense rows, 16-byte aligned, K a multiple of the k-tile. Rows past M are clamped to the last row
+// (their results are never stored); k-tiles past K, which the pipeline prefetches and never multiplies,
+// re-read the last tile.
+struct DenseDirect {
+    static constexpr bool kDirect = true;
+    const _Float16 *x;
+    int64_t M, K;
+
+    template <int CH, int T>
+    struct State {
+        const _Float16 *row[CH];
+        int kc;
+    };
+    template <int CH, int T>
+    __device__ __forceinline__ void init(State<CH, T> &st, int64_t m0, int tid, int chunk) const {
+        st.kc = chunk * 8;
+#pragma unroll
+        for (int i = 0; i < CH; i++) {
+            const int64_t m = m0 + (tid >> 3) + i * (T / 8);
+            st.row[i] = x + (m < M ? m : M - 1) * K;
+        }
+    }
+    template <int CH, int T>
+    __device__ __forceinline__ const void *addr(const State<CH, T> &st, int64_t k0, int i) const {
+        return st.row[i] + ((k0 >= K ? K - kBK : k0) + st.kc);
     }
     template <int CH, int T>
     __device__ __forceinline__ void advance(State<CH, T> &) const {}
@@ -108,6 +130,7 @@ struct DenseLoader {
 // VEC = C is a multiple of 8 and the base is 16-byte aligned: a chunk is 8 channels of one tap.
 template <bool VEC>
 struct ConvLoader {
+    static constexpr bool kDirect = false;
     const _Float16 *x;
     int64_t M, K;
     int B, C, H, W, Ho, Wo, ky, kx, sy, sx, py, px, dy, dx;
@@ -185,6 +208,7 @@ struct ConvLoader {
 // workgroup and live in scalar registers. Per row the loader keeps one 32-bit element offset and the
 // window's top-left coordinate; a fetch is two unsigned compares, one add and the load.
 struct ConvLoader64 {
+    static constexpr bool kDirect = true;
     const _Float16 *x;
     int64_t M, K;
     int B, C, H, W, Ho, Wo, ky, kx, sy, sx, py, px, dy, dx;
@@ -197,10 +221,10 @@ struct ConvLoader64 {
         int32_t delta;             // uniform: element offset of (tap, c0) relative to off0
     };
     template <int CH, int T>
-    __device__ __forceinline__ void init(State<CH, T> &st, int64_t m0, int tid) const {
+    __device__ __forceinline__ void init(State<CH, T> &st, int64_t m0, int tid, int chunk) const {
         st.i = st.j = st.c0 = 0;
         st.delta = 0;
-        const int kc = (tid & 7) * 8;
+        const int kc = chunk * 8;
 #pragma unroll
         for (int q = 0; q < CH; q++) {
             const int64_t m = m0 + (tid >> 3) + q * (T / 8);
@@ -217,16 +241,10 @@ struct ConvLoader64 {
         }
     }
     template <int CH, int T>
-    __device__ __forceinline__ void fetch(State<CH, T> &st, int64_t, u32x4 (&out)[CH]) const {
-        const int di = st.i * dy, dj = st.j * dx;
-        const bool tap_ok = st.i < ky;                       // k-tiles past K are prefetched too
-#pragma unroll
-        for (int q = 0; q < CH; q++) {
-            // every load is issued (padding reads the zero chunk), which keeps the compiler's count
-            // of outstanding loads exact
-            const bool in = tap_ok & ((unsigned)(st.ih0[q] + di) < (unsigned)H) & ((unsigned)(st.iw0[q] + dj) < (unsigned)W);
-            out[q] = load_or_zero(reinterpret_cast<const u32x4 *>(x + (st.off0[q] + st.delta)), in);
-        }
+    __device__ __forceinline__ const void *addr(const State<CH, T> &st, int64_t, int q) const {
+        const bool in = (st.i < ky) & ((unsigned)(st.ih0[q] + st.i * dy) < (unsigned)H) &
+                        ((unsigned)(st.iw0[q] + st.j * dx) < (unsigned)W);
+        return in ? static_cast<const void *>(x + (st.off0[q] + st.delta)) : static_cast<const void *>(&kZeroChunk);
     }
     template <int CH, int T>
     __device__ __forceinline__ void advance(State<CH, T> &st) const {   // next k-tile: 64 channels on
@@ -244,6 +262,7 @@ struct ConvLoader64 {
 // keeps its channel offset for the whole reduction and its tap advances by 64 / C per k-tile, so the
 // loader carries its tap (i, j) per thread, one 32-bit offset and the window's top-left coordinate per row.
 struct ConvLoaderFewC {
+    static constexpr bool kDirect = true;
     const _Float16 *x;
     int64_t M, K;
     int B, C, H, W, Ho, Wo, ky, kx, sy, sx, py, px, dy, dx;
@@ -255,8 +274,8 @@ struct ConvLoaderFewC {
         int i, j;                  // this thread's tap in the current k-tile
     };
     template <int CH, int T>
-    __device__ __forceinline__ void init(State<CH, T> &st, int64_t m0, int tid) const {
-        const int kc = (tid & 7) * 8, tap = kc / C;
+    __device__ __forceinline__ void init(State<CH, T> &st, int64_t m0, int tid, int chunk) const {
+        const int kc = chunk * 8, tap = kc / C;
         st.i = tap / kx;
         st.j = tap - st.i * kx;
 #pragma unroll
@@ -275,15 +294,10 @@ struct ConvLoaderFewC {
         }
     }
     template <int CH, int T>
-    __device__ __forceinline__ void fetch(State<CH, T> &st, int64_t, u32x4 (&out)[CH]) const {
+    __device__ __forceinline__ const void *addr(const State<CH, T> &st, int64_t, int q) const {
         const int di = st.i * dy, dj = st.j * dx;
-        const int32_t delta = (di * W + dj) * C;
-        const bool tap_ok = st.i < ky;                       // taps past the last one: the zero-padded K tail
-#pragma unroll
-        for (int q = 0; q < CH; q++) {
-            const bool in = tap_ok & ((unsigned)(st.ih0[q] + di) < (unsigned)H) & ((unsigned)(st.iw0[q] + dj) < (unsigned)W);
-            out[q] = load_or_zero(reinterpret_cast<const u32x4 *>(x + (st.off0[q] + delta)), in);
-        }
+        const bool in = (st.i < ky) & ((unsigned)(st.ih0[q] + di) < (unsigned)H) & ((unsigned)(st.iw0[q] + dj) < (unsigned)W);
+        return in ? static_cast<const void *>(x + (st.off0[q] + (di * W + dj) * C)) : static_cast<const void *>(&kZeroChunk);
     }
     template <int CH, int T>
     __device__ __forceinline__ void advance(State<CH, T> &st) const {   // next k-tile: 64 / C taps on
@@ -291,6 +305,76 @@ struct ConvLoaderFewC {
         while (st.j >= kx) { st.j -= kx; ++st.i; }
     }
 };
+
+// Epilogue of one wavefront's (16 WM) x (16 WN) accumulator block. A lane holds rows 4g + r, column
+// r16 of each 16 x 16 accumulator -- 64-byte row pieces if stored directly. Instead the wavefront
+// transposes one 16-row slab (16 x 16 WN values) at a time through its own slice of LDS (`slab`, the
+// idle activation buffer) and writes whole rows: 16 lanes x 16 bytes = 256 contiguous bytes per row and
+// store instruction. sc / bi: per-column scale (weight unit folded in) and bias of column r16 of fragment j.
+template <int WM, int WN>
+__device__ __forceinline__ void write_tile(float *slab, const floatx4 (&acc)[WM][WN], const float (&sc)[WN],
+                                           const float (&bi)[WN], int lane, int64_t mw0, int64_t nw0, int64_t M,
+                                           int64_t N, const Epilogue &ep) {
+    constexpr int kEP = 16 * WN + 4;                       // slab row pitch in floats (+4: conflict-free)
+    const int r16 = lane & 15, g = lane >> 4;
+    const bool vec = (N % 4 == 0) && ((reinterpret_cast<uintptr_t>(ep.y) | reinterpret_cast<uintptr_t>(ep.residual)) & 15u) == 0;
+#pragma unroll
+    for (int i = 0; i < WM; i++) {
+#pragma unroll
+        for (int j = 0; j < WN; j++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) slab[(g * 4 + r) * kEP + j * 16 + r16] = acc[i][j][r] * sc[j] + bi[j];
+        __builtin_amdgcn_wave_barrier();
+        const int64_t mrow0 = mw0 + (int64_t)i * 16;
+#pragma unroll
+        for (int t = 0; t < WN; t++) {                     // 16 rows x (16 WN / 4) float4 = 64 WN float4 per slab
+            const int idx = t * 64 + lane, row = idx / (4 * WN), c4 = idx % (4 * WN);
+            const int64_t m = mrow0 + row, n = nw0 + c4 * 4;
+            floatx4 v = *reinterpret_cast<const floatx4 *>(&slab[row * kEP + c4 * 4]);
+            if (m >= M || n >= N) continue;
+            const int64_t o = m * N + n;
+            if (vec) {
+                if (ep.y_f16) {
+                    if (ep.residual) {
+                        const half4 rs = *reinterpret_cast<const half4 *>(static_cast<const _Float16 *>(ep.residual) + o);
+#pragma unroll
+                        for (int e = 0; e < 4; e++) v[e] += (float)rs[e];
+                    }
+                    half4 h;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) h[e] = (_Float16)((ep.relu && v[e] < 0.f) ? 0.f : v[e]);
+                    *reinterpret_cast<half4 *>(static_cast<_Float16 *>(ep.y) + o) = h;
+                } else {
+                    if (ep.residual) {
+                        const floatx4 rs = *reinterpret_cast<const floatx4 *>(static_cast<const float *>(ep.residual) + o);
+                        v += rs;
+                    }
+                    if (ep.relu) {
+#pragma unroll
+                        for (int e = 0; e < 4; e++) v[e] = v[e] > 0.f ? v[e] : 0.f;
+                    }
+                    __builtin_nontemporal_store(v, reinterpret_cast<floatx4 *>(static_cast<float *>(ep.y) + o));
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    if (n + e >= N) break;
+                    float f = v[e];
+                    if (ep.y_f16) {
+                        if (ep.residual) f += (float)static_cast<const _Float16 *>(ep.residual)[o + e];
+                        if (ep.relu) f = f > 0.f ? f : 0.f;
+                        static_cast<_Float16 *>(ep.y)[o + e] = (_Float16)f;
+                    } else {
+                        if (ep.residual) f += static_cast<const float *>(ep.residual)[o + e];
+                        if (ep.relu) f = f > 0.f ? f : 0.f;
+                        static_cast<float *>(ep.y)[o + e] = f;
+                    }
+                }
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+    }
+}
 
 // ---- the tile kernel ---------------------------------------------------------------------------------
 template <int WM, int WN, int WGM, int WGN, int D, class Loader>
@@ -335,9 +419,8 @@ __global__ __launch_bounds__(64 * WGM * WGN, 2) void tile_kernel(Loader ld, cons
     const int KT = (int)((K + kBK - 1) / kBK);
 
     // Register prefetch, D k-tiles deep: while tile kt is multiplied out of LDS, tiles kt + 1 .. kt + D
-    // are in flight from global memory (D = 1: fetched at the top of a pass, stored at its end) (a 64-wide k-tile of MFMA work is far shorter than a trip to
-    // L2 when the tile is small). Every load is issued unconditionally -- tiles past K read a zero
-    // chunk / the last weight dword -- so the compiler counts outstanding loads exactly.
+    // are in flight from global memory (D = 1: fetched at the top of a pass, stored at its end); a
+    // 64-wide k-tile of MFMA work is far shorter than a trip to L2 when the tile is small.
     u32x4 stage[D][CH];
     uint32_t wcur[WN], wq[D][WN];
     const int srow = tid >> 3;
@@ -433,70 +516,171 @@ __global__ __launch_bounds__(64 * WGM * WGN, 2) void tile_kernel(Loader ld, cons
         if (kt < KT) body(kt++, std::integral_constant<int, 1>{});
     }
 
-    // Epilogue. A lane holds rows 4g + r, column r16 of each 16 x 16 accumulator -- 64-byte row
-    // pieces if stored directly. Instead every wave transposes one 16-row slab (16 x 16 WN values)
-    // at a time through its own slice of the (now idle) activation buffer and writes whole rows:
-    // 16 lanes x 16 bytes = 256 contiguous bytes per row and store instruction.
-    constexpr int kEP = 16 * WN + 4;                       // slab row pitch in floats (+4: conflict-free)
+    // the k-loop is over: its LDS buffers become the epilogue's transpose slabs
+    constexpr int kEP = 16 * WN + 4;
     static_assert(WGM * WGN * 16 * kEP * 4 <= 2 * BM * kPitch * 2, "epilogue slab does not fit the LDS buffer");
-    float *slab = reinterpret_cast<float *>(&As[0][0]) + wv * 16 * kEP;
-    const bool vec = (N % 4 == 0) && ((reinterpret_cast<uintptr_t>(ep.y) | reinterpret_cast<uintptr_t>(ep.residual)) & 15u) == 0;
+    write_tile<WM, WN>(reinterpret_cast<float *>(&As[0][0]) + wv * 16 * kEP, acc, sc, bi, lane, m0 + (int64_t)wm * WM * 16,
+                       nw0, M, N, ep);
+}
+
+// ---- the tile kernel with direct-to-LDS activation loads ----------------------------------------------
+// Same tiling and arithmetic as tile_kernel; the activation tile goes global -> LDS without passing
+// through registers (global_load_lds_dwordx4) into a ring of S buffers, S - 1 k-tiles ahead of the
+// math. That removes the staging registers and the LDS store instructions, and the prefetch depth no
+// longer costs VGPRs. The load writes lane l of a wavefront to byte 16 l of its destination, which is
+// exactly "row tid / 8, position tid % 8" of the 128-byte rows; the XOR swizzle is applied on the
+// global side (the thread at position p of row r fetches chunk p ^ (r % 8)).
+// The compiler does not order these loads against the operand reads: the wait for "tile kt has landed"
+// is written by hand -- every pass issues CH tile loads and WN weight loads, S - 2 passes may stay
+// outstanding -- and is followed by the pass's one barrier.
+// 16 bytes per lane from global memory straight into LDS (the host pass does not know the builtin).
+__device__ __forceinline__ void load_to_lds(const void *src, unsigned char *dst) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    typedef __attribute__((address_space(3))) void *lds_ptr;
+    __builtin_amdgcn_global_load_lds(src, (lds_ptr)dst, 16, 0, 0);
+#endif
+}
+
+template <int WM, int WN, int WGM, int WGN, int S, class Loader>
+__global__ __launch_bounds__(64 * WGM * WGN, 2) void tile_dma_kernel(Loader ld, const uint32_t *__restrict__ native,
+                                                                  int64_t M, int64_t K, int64_t N, int64_t Kb,
+                                                                  int64_t Nb, Epilogue ep, int tiles_m, int tiles_n) {
+    constexpr int T = 64 * WGM * WGN, BM = 16 * WM * WGM, BN = 16 * WN * WGN, CH = BM * 8 / T, D = S - 1;
+    static_assert(BM * 8 % T == 0 && S >= 2 && S <= 4, "geometry");
+    __shared__ __attribute__((aligned(16))) _Float16 As[S][BM * kPitch];
+
+    int id = blockIdx.x;
+    const int G = tiles_m * tiles_n;
+    if ((G & 7) == 0) id = (id & 7) * (G >> 3) + (id >> 3);
+    const int tm = id / tiles_n, tn = id % tiles_n;
+    const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
+
+    const int tid = threadIdx.x, lane = tid & 63, wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wv / WGN, wn = wv % WGN;
+    const int r16 = lane & 15, g = lane >> 4;
+
+    typename Loader::template State<CH, T> st;
+    ld.template init<CH, T>(st, m0, tid, (tid & 7) ^ ((tid >> 3) & 7));
+
+    floatx4 acc[WM][WN];
 #pragma unroll
-    for (int i = 0; i < WM; i++) {
+    for (int i = 0; i < WM; i++)
 #pragma unroll
-        for (int j = 0; j < WN; j++)
+        for (int j = 0; j < WN; j++) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+    const uint32_t *wptr[WN];
 #pragma unroll
-            for (int r = 0; r < 4; r++) slab[(g * 4 + r) * kEP + j * 16 + r16] = acc[i][j][r] * sc[j] + bi[j];
-        __builtin_amdgcn_wave_barrier();
-        const int64_t mrow0 = m0 + (int64_t)(wm * WM + i) * 16;
-#pragma unroll
-        for (int t = 0; t < WN; t++) {                     // 16 rows x (16 WN / 4) float4 = 64 WN float4 per slab
-            const int idx = t * 64 + lane, row = idx / (4 * WN), c4 = idx % (4 * WN);
-            const int64_t m = mrow0 + row, n = nw0 + c4 * 4;
-            floatx4 v = *reinterpret_cast<const floatx4 *>(&slab[row * kEP + c4 * 4]);
-            if (m >= M || n >= N) continue;
-            const int64_t o = m * N + n;
-            if (vec) {
-                if (ep.y_f16) {
-                    if (ep.residual) {
-                        const half4 rs = *reinterpret_cast<const half4 *>(static_cast<const _Float16 *>(ep.residual) + o);
-#pragma unroll
-                        for (int e = 0; e < 4; e++) v[e] += (float)rs[e];
-                    }
-                    half4 h;
-#pragma unroll
-                    for (int e = 0; e < 4; e++) h[e] = (_Float16)((ep.relu && v[e] < 0.f) ? 0.f : v[e]);
-                    *reinterpret_cast<half4 *>(static_cast<_Float16 *>(ep.y) + o) = h;
-                } else {
-                    if (ep.residual) {
-                        const floatx4 rs = *reinterpret_cast<const floatx4 *>(static_cast<const float *>(ep.residual) + o);
-                        v += rs;
-                    }
-                    if (ep.relu) {
-#pragma unroll
-                        for (int e = 0; e < 4; e++) v[e] = v[e] > 0.f ? v[e] : 0.f;
-                    }
-                    __builtin_nontemporal_store(v, reinterpret_cast<floatx4 *>(static_cast<float *>(ep.y) + o));
-                }
-            } else {
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    if (n + e >= N) break;
-                    float f = v[e];
-                    if (ep.y_f16) {
-                        if (ep.residual) f += (float)static_cast<const _Float16 *>(ep.residual)[o + e];
-                        if (ep.relu) f = f > 0.f ? f : 0.f;
-                        static_cast<_Float16 *>(ep.y)[o + e] = (_Float16)f;
-                    } else {
-                        if (ep.residual) f += static_cast<const float *>(ep.residual)[o + e];
-                        if (ep.relu) f = f > 0.f ? f : 0.f;
-                        static_cast<float *>(ep.y)[o + e] = f;
-                    }
-                }
-            }
-        }
-        __builtin_amdgcn_wave_barrier();
+    for (int j = 0; j < WN; j++) {
+        int64_t nb = n0 / 16 + wn * WN + j;
+        if (nb >= Nb) nb = Nb - 1;
+        wptr[j] = native + (nb * Kb) * 256 + lane * 4;
     }
+    const int KT = (int)((K + kBK - 1) / kBK);
+
+    uint32_t wcur[WN], wq[D][WN];
+    auto wload = [&](uint32_t (&w)[WN], int kn) {
+        if (kn >= KT) kn = KT - 1;
+#pragma unroll
+        for (int j = 0; j < WN; j++) w[j] = wptr[j][(int64_t)(kn >> 2) * 256 + (kn & 3)];
+    };
+    // tile `kn` -> ring buffer kn % S; the loader's state moves on to the next tile
+    unsigned char *const lds0 = reinterpret_cast<unsigned char *>(&As[0][0]) + wv * 1024;
+    auto fill = [&](int kn) {
+        unsigned char *dst = lds0 + (kn % S) * (BM * kPitch * 2);
+#pragma unroll
+        for (int i = 0; i < CH; i++) load_to_lds(ld.template addr<CH, T>(st, (int64_t)kn * kBK, i), dst + i * (T * 16));
+        ld.template advance<CH, T>(st);
+    };
+
+    // per-column epilogue constants first (conditional loads: keep them out of the counted stream)
+    const int64_t nw0 = n0 + (int64_t)wn * WN * 16;
+    float sc[WN], bi[WN];
+#pragma unroll
+    for (int j = 0; j < WN; j++) {
+        const int64_t n = nw0 + j * 16 + r16;
+        sc[j] = (n < N && ep.scale ? ep.scale[n] : 1.0f) * (1.0f / kWeightUnit);
+        bi[j] = (n < N && ep.bias) ? ep.bias[n] : 0.0f;
+    }
+    wload(wcur, 0);
+    __builtin_amdgcn_s_waitcnt(0x0F70);            // vmcnt(0): start counting from a clean state
+    __builtin_amdgcn_sched_barrier(0);
+    // prologue: tiles 0 .. S-2 and the weights of tiles 1 .. D-1; from here on the order of issue is
+    // (S-1) x CH tile loads, (D-1) x WN weight loads, then per pass CH + WN
+#pragma unroll
+    for (int s = 0; s < S - 1; s++) fill(s);
+#pragma unroll
+    for (int d = 0; d + 1 < D; d++) wload(wq[d], d + 1);
+    __builtin_amdgcn_sched_barrier(0);
+
+    const int arow = (wm * WM * 16 + r16) * kPitch;
+    auto swz = [&](int i, int s) { return i * 16 * kPitch + (((4 * s + g) ^ (r16 & 7)) * 8); };
+    // vmcnt(N): at most N loads outstanding. Tile kt's loads are followed by those of S - 2 passes.
+    constexpr int kN = (S - 2) * (CH + WN);
+    constexpr int kWaitImm = (kN & 15) | (7 << 4) | (15 << 8) | ((kN >> 4) << 14);
+    static_assert(kN < 64, "vmcnt range");
+
+    auto body = [&](int kt, auto slot_tag) {
+        constexpr int slot = decltype(slot_tag)::value, freed = (slot + D - 1) % D;
+        __builtin_amdgcn_s_waitcnt(kWaitImm);       // this thread's part of tile kt is in LDS
+        __syncthreads();                             // ... and everybody's; buffer (kt - 1) % S is free
+        __builtin_amdgcn_sched_barrier(0);
+        fill(kt + S - 1);
+        wload(wq[freed], kt + D);
+        __builtin_amdgcn_sched_barrier(0);
+        const _Float16 *abase = &As[kt % S][arow];
+        constexpr int NQ = 2 * WM, kAhead = NQ < 4 ? NQ : 4;
+        half8 a[NQ];
+        half8 bfr[2][WN];
+#pragma unroll
+        for (int q = 0; q < kAhead; q++) a[q] = *reinterpret_cast<const half8 *>(abase + swz(q >> 1, q & 1));
+#pragma unroll
+        for (int j = 0; j < WN; j++) bfr[0][j] = decode_step(wcur[j], 0);
+#pragma unroll
+        for (int j = 0; j < WN; j++) bfr[1][j] = decode_step(wcur[j], 1);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int q = 0; q < NQ; q++) {
+#pragma unroll
+            for (int j = 0; j < WN; j++) acc[q >> 1][j] = mfma16(a[q], bfr[q & 1][j], acc[q >> 1][j]);
+            if (q + kAhead < NQ)
+                a[q + kAhead] = *reinterpret_cast<const half8 *>(abase + swz((q + kAhead) >> 1, (q + kAhead) & 1));
+            __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int j = 0; j < WN; j++) asm volatile("v_mov_b32 %0, %1" : "=v"(wcur[j]) : "v"(wq[slot][j]));
+    };
+    int kt = 0;
+    for (; kt + D <= KT; kt += D) {
+        body(kt, std::integral_constant<int, 0>{});
+        if constexpr (D > 1) body(kt + 1, std::integral_constant<int, 1>{});
+        if constexpr (D > 2) body(kt + 2, std::integral_constant<int, 2>{});
+    }
+    if constexpr (D > 1) {
+        if (kt < KT) body(kt++, std::integral_constant<int, 0>{});
+    }
+    if constexpr (D > 2) {
+        if (kt < KT) body(kt++, std::integral_constant<int, 1>{});
+    }
+    // drain the prefetches past K before the buffers are reused as transpose slabs
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();
+
+    constexpr int kEP = 16 * WN + 4;
+    static_assert(WGM * WGN * 16 * kEP * 4 <= S * BM * kPitch * 2, "epilogue slab does not fit the LDS buffer");
+    write_tile<WM, WN>(reinterpret_cast<float *>(&As[0][0]) + wv * 16 * kEP, acc, sc, bi, lane, m0 + (int64_t)wm * WM * 16,
+                       nw0, M, N, ep);
+}
+
+template <int WM, int WN, int WGM, int WGN, int S, class Loader>
+int launch_tile_dma(const Loader &ld, const void *native, int64_t M, int64_t K, int64_t N, const Epilogue &ep,
+                    void *stream) {
+    constexpr int BM = 16 * WM * WGM, BN = 16 * WN * WGN;
+    const int64_t tm = (M + BM - 1) / BM, tn = (N + BN - 1) / BN;
+    if (tm * tn > 0x7FFFFFFF) return TMQ_ERR_TOO_LARGE;
+    hipLaunchKernelGGL((tile_dma_kernel<WM, WN, WGM, WGN, S, Loader>), dim3((uint32_t)(tm * tn)), dim3(64 * WGM * WGN), 0,
+                       as_stream(stream), ld, static_cast<const uint32_t *>(native), M, K, N, native_blocks_k(K),
+                       native_blocks_n(N), ep, (int)tm, (int)tn);
+    return check_launch();
 }
 
 template <int WM, int WN, int WGM, int WGN, int D, class Loader>
@@ -518,17 +702,24 @@ template <class Loader>
 int dispatch_tile(const Loader &ld, const void *native, int64_t M, int64_t K, int64_t N, const Epilogue &ep,
                   void *stream) {
     auto wgs = [&](int bm, int bn) { return ((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
-    // Prefetch depth: the big tile has a k-tile of work long enough to cover a trip to L2 (and no
-    // registers to spare); the smaller ones fetch two tiles ahead once the reduction is long enough
-    // to pay for the extra tile in the prologue (measured on the ResNet-18 layers: K = 576 loses,
-    // K >= 1152 wins).
-    const bool deep = K >= 16 * kBK;
-    if (N > 128 && wgs(128, 256) >= 384) return launch_tile<8, 4, 1, 4, 1>(ld, native, M, K, N, ep, stream);
-    if (N > 64 && wgs(128, 128) >= 256)
-        return deep ? launch_tile<4, 4, 2, 2, 2>(ld, native, M, K, N, ep, stream)
-                    : launch_tile<4, 4, 2, 2, 1>(ld, native, M, K, N, ep, stream);
-    return deep ? launch_tile<2, 4, 2, 1, 2>(ld, native, M, K, N, ep, stream)
-                : launch_tile<2, 4, 2, 1, 1>(ld, native, M, K, N, ep, stream);
+    if constexpr (Loader::kDirect) {
+        // direct-to-LDS kernel, one k-tile ahead (deeper rings measured slower at every shape: the
+        // extra address registers cost more occupancy than the longer prefetch gains)
+        if (N > 128 && wgs(128, 256) >= 384) return launch_tile_dma<8, 4, 1, 4, 2>(ld, native, M, K, N, ep, stream);
+        if (N > 64 && wgs(128, 128) >= 256) return launch_tile_dma<4, 4, 2, 2, 2>(ld, native, M, K, N, ep, stream);
+        return launch_tile_dma<2, 4, 2, 1, 2>(ld, native, M, K, N, ep, stream);
+    } else {
+        // Register prefetch depth: the big tile has a k-tile of work long enough to cover a trip to L2
+        // (and no registers to spare); the smaller ones fetch two tiles ahead once the reduction is
+        // long enough to pay for the extra tile in the prologue.
+        const bool deep = K >= 16 * kBK;
+        if (N > 128 && wgs(128, 256) >= 384) return launch_tile<8, 4, 1, 4, 1>(ld, native, M, K, N, ep, stream);
+        if (N > 64 && wgs(128, 128) >= 256)
+            return deep ? launch_tile<4, 4, 2, 2, 2>(ld, native, M, K, N, ep, stream)
+                        : launch_tile<4, 4, 2, 2, 1>(ld, native, M, K, N, ep, stream);
+        return deep ? launch_tile<2, 4, 2, 1, 2>(ld, native, M, K, N, ep, stream)
+                    : launch_tile<2, 4, 2, 1, 1>(ld, native, M, K, N, ep, stream);
+    }
 }
 
 }  // namespace
@@ -537,8 +728,8 @@ int launch_gemm_dense(const void *x, int64_t M, int64_t K, const void *native, i
                       const float *bias, const void *residual, int relu, void *y, int y_f16, void *stream) {
     Epilogue ep{scale, bias, residual, y, relu, y_f16};
     if ((K % kBK == 0) && aligned16(x))
-        return dispatch_tile(DenseLoader<true>{static_cast<const _Float16 *>(x), M, K}, native, M, K, N, ep, stream);
-    return dispatch_tile(DenseLoader<false>{static_cast<const _Float16 *>(x), M, K}, native, M, K, N, ep, stream);
+        return dispatch_tile(DenseDirect{static_cast<const _Float16 *>(x), M, K}, native, M, K, N, ep, stream);
+    return dispatch_tile(DenseLoader{static_cast<const _Float16 *>(x), M, K}, native, M, K, N, ep, stream);
 }
 
 }  // namespace tmq
