@@ -260,6 +260,25 @@ int tmq_ternary_dwconv2d(const void *x, const tmq_conv_shape *shape, const uint3
 int tmq_ternary_dwconv_patches(const void *x, int x_dtype, int64_t P, int32_t taps, int64_t C,
                                const uint32_t *words, float *y, void *stream);
 
+/* Depthwise transposed convolution (groups == channels, one filter per channel), fused:
+ *   y[b][oh][ow][c] = sum_{i,j} x[b][ih][iw][c] * T[c][i][j],  oh = ih*sy - py + i*dy, ow likewise.
+ * x: fp16 NHWC [B][H][W][C]; shape describes the transposed convolution (N == C; py_end / px_end are
+ * ignored); out_pad_*: PyTorch's output_padding; words: the reference packing of the
+ * [C][1][ky][kx] weight, words[ky*kx][ceil(C/16)]; y: NHWC [B][Ho][Wo][C] in epilogue->y_dtype with
+ * Ho = (H-1)*sy - 2*py + dy*(ky-1) + 1 + out_pad_y. Replaces ternary_dwconvtrans_cuda + F.fold in
+ * ConvTranspose2d.compact_forward (tmq/tmq.py:1025-1029) without materialising the columns.      */
+int tmq_convtranspose2d_out_hw(const tmq_conv_shape *shape, int32_t out_pad_y, int32_t out_pad_x,
+                               int32_t *ho, int32_t *wo);
+int tmq_ternary_dwconvtrans2d(const void *x, const tmq_conv_shape *shape, int32_t out_pad_y, int32_t out_pad_x,
+                              const uint32_t *words, const tmq_epilogue *epilogue, void *y, void *stream);
+
+/* The column form, the calling convention of ternary_dwconvtrans_cuda (tmq/tmq_cuda.cu:645-686,
+ * kernel 118-162): x fp32 [B][P][C], y fp32 [B][C*taps][P], y[b][c*taps + t][p] = x[b][p][c] * T[c][t]
+ * (the caller scatters y with F.fold). Every batch entry is processed (the reference's launch covers
+ * the first only).                                                                                */
+int tmq_ternary_dwconvtrans_cols(const float *x, int64_t B, int64_t P, int32_t taps, int64_t C,
+                                 const uint32_t *words, float *y, void *stream);
+
 /* ------------------------------------------------------------------------------------------
  * Host entropy codec for packed tensors (host memory in, host memory out; no GPU involved).
  * ---------------------------------------------------------------------------------------- */

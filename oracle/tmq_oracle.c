@@ -371,6 +371,22 @@ void tmq_oracle_dwconv_patches(const float *x, int64_t P, int64_t T, int64_t C, 
         }
 }
 
+/* Transposed depthwise convolution in column form, the arithmetic of ternaryDWConvTransFP32
+ * (tmq/tmq_cuda.cu:118-162): x [B][P][C], words[t][ceil(C/16)], y [B][C*T][P] with
+ * y[b][c*T + t][p] = x[b][p][c] * T[c][t] as an fp32 product (a zero weight gives a zero that keeps
+ * the sign of x, like the reference's multiply by 0.f). The reference's launch has no batch index
+ * (host, 645-686) and so fills batch entry 0 only; here every entry follows the same formula.   */
+void tmq_oracle_dwconvtrans_cols(const float *x, int64_t B, int64_t P, int64_t T, int64_t C, const uint32_t *wp, float *y) {
+    int64_t Q = (C + 15) / 16;
+    for (int64_t b = 0; b < B; b++)
+        for (int64_t c = 0; c < C; c++)
+            for (int64_t t = 0; t < T; t++) {
+                uint32_t word = wp[t * Q + c / 16];
+                float w = value_from_code((int)((word >> (2 * (15 - (c % 16)))) & 3u), 0);
+                for (int64_t p = 0; p < P; p++) y[(b * C * T + c * T + t) * P + p] = x[(b * P + p) * C + c] * w;
+            }
+}
+
 /* Direct convolution, NCHW input, weights packed as [C*ky*kx][ceil(N/16)] with row
  * (c*ky + y)*kx + x -- the ordering of F.unfold used at tmq/tmq.py:857-859. Output NCHW fp64.
  * Output size is PyTorch's floor((h + 2p - d(k-1) - 1)/s) + 1.                               */

@@ -45,6 +45,7 @@ def lib():
         L.tmq_oracle_conv2d.argtypes = [_f32p] + [_i64] * 4 + [_u32p] + [_i64] * 9 + [ctypes.c_void_p,
                                                                                      ctypes.c_void_p, _f64p]
         L.tmq_oracle_dwconv_patches.argtypes = [_f32p, _i64, _i64, _i64, _u32p, _f64p]
+        L.tmq_oracle_dwconvtrans_cols.argtypes = [_f32p, _i64, _i64, _i64, _i64, _u32p, _f32p]
         L.tmq_oracle_compress.argtypes = [_u32p, _i64, _i64, ctypes.POINTER(ctypes.POINTER(ctypes.c_uint8))]
         L.tmq_oracle_compress.restype = _i64
         L.tmq_oracle_free.argtypes = [ctypes.c_void_p]
@@ -178,6 +179,16 @@ def dwconv_patches(x, words):
     words = np.ascontiguousarray(words, dtype=np.uint32)
     y = np.empty((P, C), dtype=np.float64)
     lib().tmq_oracle_dwconv_patches(x.reshape(-1), P, T, C, words.reshape(-1), y.reshape(-1))
+    return y
+
+
+def dwconvtrans_cols(x, words, taps):
+    """x [B][P][C] fp32 -> fp32 [B][C*taps][P], y[b][c*taps + t][p] = x[b][p][c] * T[c][t]."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    B, P, C = x.shape
+    words = np.ascontiguousarray(words, dtype=np.uint32)
+    y = np.empty((B, C * taps, P), dtype=np.float32)
+    lib().tmq_oracle_dwconvtrans_cols(x.reshape(-1), B, P, taps, C, words.reshape(-1), y.reshape(-1))
     return y
 
 

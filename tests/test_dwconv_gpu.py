@@ -104,3 +104,87 @@ def test_transposed_layer_compact_inference(cuda, cin, cout, k, stride, pad, opa
     assert net[0].weight.dtype == torch.int32
     got = net(x)
     assert got.shape == want.shape and torch.equal(got, want)
+
+
+@pytest.mark.parametrize("B,P,T,C", [(1, 1, 1, 1), (1, 7, 9, 16), (3, 50, 9, 40), (2, 130, 4, 5), (2, 64, 25, 96), (1, 200, 6, 70)])
+def test_transposed_column_form_matches_oracle(cuda, oracle, B, P, T, C):
+    """out[b][c T + t][p] = in[b][p][c] * T[c][t]: a product with +1 / -1 / 0, bit-identical to the oracle
+    (signed zeros included), for every batch entry; 2-, 3- and 4-D calling conventions; the extension."""
+    from tmq_amd import ops
+    rng = np.random.default_rng(B + P + T + C)
+    W = _ternary(rng, (C, T))
+    words = oracle.pack(W)                                       # [T][ceil(C/16)]
+    x = rng.standard_normal((B, P, C)).astype(np.float32)
+    x[0, 0, 0] = -0.0
+    want = oracle.dwconvtrans_cols(x, words, T)
+    # the restatement itself against the textbook outer product
+    assert np.array_equal(want, np.einsum("bpc,ct->bctp", x, W).reshape(B, C * T, P))
+    tw = torch.from_numpy(words.view(np.int32)).to(cuda).view(1, T, 1, -1)
+    tx = torch.from_numpy(x).to(cuda)
+    got = ops.ternary_dwconvtrans_cuda(tx, tw, 1, T)
+    assert tuple(got.shape) == (B, C * T, P) and got.dtype == torch.float32
+    assert np.array_equal(got.cpu().numpy().view(np.uint32), want.view(np.uint32))
+    got4 = ops.ternary_dwconvtrans_cuda(tx.view(B, 1, P, C), tw, T, 1)
+    assert tuple(got4.shape) == (B, 1, C * T, P) and torch.equal(got4.view(B, C * T, P), got)
+    got2 = ops.ternary_dwconvtrans_cuda(tx[0], tw, 1, T)
+    assert tuple(got2.shape) == (C * T, P) and torch.equal(got2, got[0])
+    ext = ops.ext
+    if ext is not None:
+        assert torch.equal(ext.ternary_dwconvtrans_cuda(tx, tw, 1, T), got)
+        assert torch.equal(ext.ternary_dwconvtrans_cuda(tx.view(B, 1, P, C), tw, 1, T), got4)
+        with pytest.raises(RuntimeError):
+            ext.ternary_dwconvtrans_cuda(tx, tw, 2, T)          # taps do not match the words
+    with pytest.raises(RuntimeError):
+        ops.ternary_dwconvtrans_cuda(tx.half(), tw, 1, T)
+
+
+@pytest.mark.parametrize("B,C,H,W,k,stride,pad,opad,dil", [
+    (2, 16, 5, 5, 3, 2, 1, 1, 1), (1, 40, 6, 7, (3, 2), (2, 3), (1, 0), (1, 2), 1), (3, 8, 4, 4, 3, 1, 1, 0, 1),
+    (2, 5, 6, 6, 2, 2, 0, 0, 1), (1, 96, 7, 7, 3, 2, 2, 1, 2), (2, 32, 3, 8, 4, (3, 1), 0, 0, (1, 2)),
+])
+def test_transposed_image_form_exact_on_integers(cuda, B, C, H, W, k, stride, pad, opad, dil):
+    """Small-integer activations: the gathered transposed convolution must equal torch's grouped
+    conv_transpose2d on the expanded weights bit for bit, and equal columns + F.fold; then the epilogue."""
+    from tmq_amd import ops
+    pair = lambda v: tuple(v) if isinstance(v, (tuple, list)) else (v, v)
+    k, stride, pad, opad, dil = pair(k), pair(stride), pair(pad), pair(opad), pair(dil)
+    g = torch.Generator(device=cuda).manual_seed(B + C + H)
+    Wt = torch.randint(-1, 2, (C, 1, k[0], k[1]), device=cuda, generator=g).float()
+    x = torch.randint(-4, 5, (B, C, H, W), device=cuda, generator=g).float()
+    words = ops.compactify_ternary(Wt)
+    y = ops.ternary_dwconvtrans2d(x.half(), words, k, stride, pad, opad, dil)
+    ref = torch.nn.functional.conv_transpose2d(x, Wt, None, stride, pad, opad, groups=C, dilation=dil)
+    assert y.shape == ref.shape and y.is_contiguous(memory_format=torch.channels_last)
+    assert torch.equal(y, ref)
+    # the reference's route: columns, then col2im
+    cols = ops.ternary_dwconvtrans_cuda(x.reshape(B, C, H * W).transpose(1, 2).contiguous(), words, k[1], k[0])
+    folded = torch.nn.functional.fold(cols, output_size=tuple(ref.shape[-2:]), kernel_size=k, dilation=dil, stride=stride,
+                                      padding=pad)
+    if opad == (0, 0):
+        assert torch.equal(folded, ref)
+    scale = torch.pow(2.0, torch.randint(-2, 3, (C,), device=cuda, generator=g).float())
+    bias = torch.randint(-9, 10, (C,), device=cuda, generator=g).float()
+    res = torch.randint(-5, 6, ref.shape, device=cuda, generator=g).half().contiguous(memory_format=torch.channels_last)
+    y2 = ops.ternary_dwconvtrans2d(x.half(), words, k, stride, pad, opad, dil, scale=scale, bias=bias, residual=res, relu=True,
+                                   out_dtype=torch.float16)
+    want = torch.relu(ref * scale.view(1, -1, 1, 1) + bias.view(1, -1, 1, 1) + res.float()).half()
+    assert torch.equal(y2, want)
+
+
+def test_depthwise_transposed_layer_compact_inference(cuda):
+    """A depthwise nn.ConvTranspose2d through quantize_model -> ternarise -> compact weights."""
+    import tmq_amd as t
+    torch.manual_seed(5)
+    net = torch.nn.Sequential(torch.nn.ConvTranspose2d(24, 24, 3, 2, 1, output_padding=1, groups=24, bias=True))
+    ctrl = t.QuantizationControl()
+    t.quantize_model(net, ctrl)
+    net.to(cuda).eval()
+    with torch.no_grad():
+        net[0].bias.copy_(torch.randint(-4, 5, (24,)).float())
+    x = torch.randint(-3, 4, (2, 24, 6, 5), device=cuda).float()
+    ctrl.quantize()
+    want = net(x)
+    t.compressed_state_dict(net, strong=False)
+    assert net[0].weight.dtype == torch.int32 and tuple(net[0].weight.shape) == (1, 3, 3, 2)
+    got = net(x)
+    assert got.shape == want.shape and torch.equal(got, want)

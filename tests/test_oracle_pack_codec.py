@@ -255,3 +255,16 @@ def test_oracle_depthwise_patches_is_the_textbook_sum(oracle):
         x = rng.standard_normal((P, T, C)).astype(np.float32)
         want = np.einsum("ptc,ct->pc", x.astype(np.float64), W.astype(np.float64))
         assert np.allclose(oracle.dwconv_patches(x, words), want, rtol=0, atol=1e-12)
+
+
+def test_oracle_transposed_depthwise_columns_are_the_outer_product(oracle):
+    """y[b][c T + t][p] = x[b][p][c] * T[c][t] against numpy on the unpacked weights (bit for bit: the
+    products are exact), ragged C, several batch entries."""
+    rng = np.random.default_rng(10)
+    for (B, P, T, C) in [(1, 5, 9, 16), (2, 3, 4, 5), (3, 11, 6, 40), (1, 1, 1, 1)]:
+        u = rng.random((C, T))
+        W = np.where(u < .25, 1.0, np.where(u < .5, -1.0, 0.0)).astype(np.float32)
+        words = oracle.pack(W)
+        x = rng.standard_normal((B, P, C)).astype(np.float32)
+        want = (x.transpose(0, 2, 1)[:, :, None, :] * W[None, :, :, None]).reshape(B, C * T, P)
+        assert np.array_equal(oracle.dwconvtrans_cols(x, words, T).view(np.uint32), want.view(np.uint32))

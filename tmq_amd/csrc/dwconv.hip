@@ -15,6 +15,14 @@
 //   * NHWC image (tmq_ternary_dwconv2d): taps are gathered on the fly, padding reads as zero;
 //   * unfolded patches [P][T][C] fp32, the calling convention of the reference's
 //     ternary_dwconv_cuda (tmq/tmq_cuda.cu:166-238, host 607-642; caller tmq/tmq.py:849-853).
+//
+// Depthwise transposed convolution, y[b][oh][ow][c] = sum over (ih, i), (iw, j) with
+// oh = ih sy - py + i dy, ow = iw sx - px + j dx of x[b][ih][iw][c] * T[c][i][j], in the same two forms:
+//   * NHWC image (tmq_ternary_dwconvtrans2d): each output position gathers the inputs that reach it
+//     (no columns, no col2im scatter);
+//   * columns: y[b][c T + t][p] = x[b][p][c] * T[c][t], the calling convention of the reference's
+//     ternary_dwconvtrans_cuda (tmq/tmq_cuda.cu:118-162, host 645-686; caller tmq/tmq.py:1026-1029),
+//     whose result the caller scatters with F.fold. Pure data movement: 4 B in, 4 T B out per element.
 #include "common.h"
 #include "mfma.h"
 
@@ -142,6 +150,74 @@ __global__ __launch_bounds__(256) void dwconv_patches_kernel(const T *__restrict
     store8(ep, p * C + c0, c0, C, acc, vec);
 }
 
+// Transposed depthwise convolution on an NHWC fp16 image: a thread owns 8 channels of one OUTPUT
+// position and visits the taps whose source coordinate (oh + py - i dy) / sy is integral and inside.
+__global__ __launch_bounds__(256) void dwconvtrans_image_kernel(const _Float16 *__restrict__ x,
+                                                                const uint32_t *__restrict__ words, int B, int C, int H,
+                                                                int W, int Ho, int Wo, int ky, int kx, int sy, int sx,
+                                                                int py, int px, int dy, int dx, int vec, DwEpilogue ep) {
+    const int64_t G = (C + 7) / 8, Q = (C + 15) / 16;
+    const int64_t id = (int64_t)blockIdx.x * 256 + threadIdx.x, total = (int64_t)B * Ho * Wo * G;
+    if (id >= total) return;
+    const int64_t p = id / G, c0 = (id - p * G) * 8;
+    const int ow = (int)(p % Wo);
+    const int64_t r = p / Wo;
+    const int oh = (int)(r % Ho), b = (int)(r / Ho);
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    for (int i = 0; i < ky; i++) {
+        const int ny = oh + py - i * dy;
+        if (ny < 0 || ny % sy) continue;
+        const int ih = ny / sy;
+        if (ih >= H) continue;
+        for (int j = 0; j < kx; j++) {
+            const int nx = ow + px - j * dx;
+            if (nx < 0 || nx % sx) continue;
+            const int iw = nx / sx;
+            if (iw >= W) continue;
+            const _Float16 *src = x + (((int64_t)b * H + ih) * W + iw) * C + c0;
+            const uint32_t codes = codes8(words, Q, i * kx + j, c0);
+            if (vec) {
+                const half8 v = *reinterpret_cast<const half8 *>(src);
+#pragma unroll
+                for (int e = 0; e < 8; e++) acc[e] += apply_code((float)v[e], codes << (2 * e));
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; e++)
+                    if (c0 + e < C) acc[e] += apply_code((float)src[e], codes << (2 * e));
+            }
+        }
+    }
+    store8(ep, p * C + c0, c0, C, acc, vec);
+}
+
+// Column form. A workgroup transposes a 64-patch x 64-channel tile of one batch entry through LDS:
+// reads run along channels, writes along patches (256 contiguous bytes per (channel, tap) row).
+// The product is formed as x * {+1, -1, 0} in fp32 like the reference's (a zero weight keeps the sign
+// of x in the zero it writes).
+__global__ __launch_bounds__(256) void dwconvtrans_cols_kernel(const float *__restrict__ x, const uint32_t *__restrict__ words,
+                                                               int64_t P, int taps, int64_t C, float *__restrict__ y) {
+    __shared__ float tile[64][65];
+    const int64_t p0 = (int64_t)blockIdx.x * 64, c0 = (int64_t)blockIdx.y * 64, b = blockIdx.z;
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const float *xb = x + b * P * C;
+    for (int r = wv; r < 64; r += 4) {
+        const int64_t p = p0 + r, c = c0 + lane;
+        tile[r][lane] = (p < P && c < C) ? xb[p * C + c] : 0.f;
+    }
+    __syncthreads();
+    const int64_t Q = (C + 15) / 16;
+    float *yb = y + b * C * taps * P;
+    const int64_t p = p0 + lane;
+    const int nc = (int)((C - c0) < 64 ? (C - c0) : 64);
+    for (int pair = wv; pair < nc * taps; pair += 4) {       // (channel, tap) rows, dealt to the 4 wavefronts
+        const int cc = pair / taps, t = pair - cc * taps;
+        const int64_t c = c0 + cc;
+        const uint32_t code = (words[(int64_t)t * Q + (c >> 4)] >> (30 - 2 * (int)(c & 15))) & 3u;
+        const float coef = code == 1u ? 1.0f : (code == 2u ? -1.0f : 0.0f);
+        if (p < P) yb[(c * taps + t) * P + p] = tile[lane][cc] * coef;
+    }
+}
+
 bool aligned_for(const void *p, size_t bytes) { return (reinterpret_cast<uintptr_t>(p) % bytes) == 0; }
 
 }  // namespace
@@ -191,6 +267,53 @@ int tmq_ternary_dwconv_patches(const void *x, int x_dtype, int64_t P, int32_t ta
     else
         hipLaunchKernelGGL(dwconv_patches_kernel<_Float16>, dim3((uint32_t)blocks), dim3(256), 0, as_stream(stream),
                            static_cast<const _Float16 *>(x), words, P, (int)taps, C, vec, ep);
+    return check_launch();
+}
+
+int tmq_convtranspose2d_out_hw(const tmq_conv_shape *s, int32_t out_pad_y, int32_t out_pad_x, int32_t *ho, int32_t *wo) {
+    if (!s || !ho || !wo) return TMQ_ERR_INVALID_ARG;
+    if (s->ky <= 0 || s->kx <= 0 || s->sy <= 0 || s->sx <= 0 || s->dy <= 0 || s->dx <= 0 || s->py < 0 || s->px < 0 ||
+        out_pad_y < 0 || out_pad_x < 0 || s->H <= 0 || s->W <= 0)
+        return TMQ_ERR_INVALID_ARG;
+    const int64_t h = ((int64_t)s->H - 1) * s->sy - 2 * (int64_t)s->py + (int64_t)s->dy * (s->ky - 1) + 1 + out_pad_y;
+    const int64_t w = ((int64_t)s->W - 1) * s->sx - 2 * (int64_t)s->px + (int64_t)s->dx * (s->kx - 1) + 1 + out_pad_x;
+    if (h <= 0 || w <= 0 || h > 0x7FFFFFFF || w > 0x7FFFFFFF) return TMQ_ERR_INVALID_ARG;
+    *ho = (int32_t)h;
+    *wo = (int32_t)w;
+    return TMQ_OK;
+}
+
+int tmq_ternary_dwconvtrans2d(const void *x, const tmq_conv_shape *s, int32_t out_pad_y, int32_t out_pad_x,
+                              const uint32_t *words, const tmq_epilogue *epilogue, void *y, void *stream) {
+    if (!s || !x || !words || !y) return TMQ_ERR_INVALID_ARG;
+    if (s->N != s->C || s->C <= 0 || s->B < 0) return TMQ_ERR_INVALID_ARG;
+    tmq_epilogue e = {nullptr, nullptr, nullptr, 0, TMQ_F32};
+    if (epilogue) e = *epilogue;
+    if (e.y_dtype != TMQ_F16 && e.y_dtype != TMQ_F32) return TMQ_ERR_UNSUPPORTED;
+    int32_t ho, wo;
+    int rc = tmq_convtranspose2d_out_hw(s, out_pad_y, out_pad_x, &ho, &wo);
+    if (rc != TMQ_OK) return rc;
+    const int64_t total = (int64_t)s->B * ho * wo * ((s->C + 7) / 8), blocks = (total + 255) / 256;
+    if (total == 0) return TMQ_OK;
+    if (blocks > 0x7FFFFFFF) return TMQ_ERR_TOO_LARGE;
+    const int y_f16 = e.y_dtype == TMQ_F16;
+    const int vec = (s->C % 8 == 0) && aligned_for(x, 16) && aligned_for(y, 16) && (!e.residual || aligned_for(e.residual, 16));
+    DwEpilogue ep{e.scale, e.bias, e.residual, y, e.relu, y_f16};
+    hipLaunchKernelGGL(dwconvtrans_image_kernel, dim3((uint32_t)blocks), dim3(256), 0, as_stream(stream),
+                       static_cast<const _Float16 *>(x), words, s->B, s->C, s->H, s->W, ho, wo, s->ky, s->kx, s->sy, s->sx,
+                       s->py, s->px, s->dy, s->dx, vec, ep);
+    return check_launch();
+}
+
+int tmq_ternary_dwconvtrans_cols(const float *x, int64_t B, int64_t P, int32_t taps, int64_t C, const uint32_t *words,
+                                 float *y, void *stream) {
+    if (B < 0 || P < 0 || taps <= 0 || C <= 0) return TMQ_ERR_INVALID_ARG;
+    if (B == 0 || P == 0) return TMQ_OK;
+    if (!x || !words || !y) return TMQ_ERR_INVALID_ARG;
+    const int64_t gx = (P + 63) / 64, gy = (C + 63) / 64;
+    if (gx > 0x7FFFFFFF || gy > 65535 || B > 65535) return TMQ_ERR_TOO_LARGE;
+    hipLaunchKernelGGL(dwconvtrans_cols_kernel, dim3((uint32_t)gx, (uint32_t)gy, (uint32_t)B), dim3(256), 0, as_stream(stream),
+                       x, words, P, (int)taps, C, y);
     return check_launch();
 }
 

@@ -172,10 +172,32 @@ torch::Tensor ternary_dwconv_cuda(torch::Tensor input, torch::Tensor weights, in
     return y;
 }
 
-// Transposed depthwise variant (tmq/tmq_cuda.cu:645-686): the reference's host mis-sizes its output and
-// no working model reaches it; not built here.
-torch::Tensor ternary_dwconvtrans_cuda(torch::Tensor, torch::Tensor, int64_t, int64_t) {
-    TORCH_CHECK(false, "ternary_dwconvtrans_cuda: not implemented on this build");
+// Transposed depthwise variant in column form (tmq/tmq_cuda.cu:645-686, caller tmq/tmq.py:1026-1029):
+// in fp32 [P, C], [B, P, C] or [B, 1, P, C]; weights = compact words of the [C, 1, ky, kx] kernel shaped
+// [1, *, *, ceil(C/16)]; out [.., C * taps, P], out[c taps + t][p] = in[p][c] T[c][t], ready for F.fold.
+// Every batch entry is computed and a 4-D input gives the 4-D output (the reference's launch has no
+// batch index and its 4-D result is overwritten by a 2-D one, tmq/tmq_cuda.cu:677-682).
+torch::Tensor ternary_dwconvtrans_cuda(torch::Tensor input, torch::Tensor weights, int64_t kx, int64_t ky) {
+    TORCH_CHECK(input.device().is_cuda() && weights.device().is_cuda(), "ternary_dwconvtrans_cuda: expected tensors on the GPU");
+    TORCH_CHECK(input.scalar_type() == torch::kFloat32, "ternary_dwconvtrans_cuda: expected fp32 input");
+    TORCH_CHECK(input.dim() >= 2 && input.dim() <= 4 && (input.dim() != 4 || input.size(1) == 1),
+                "ternary_dwconvtrans_cuda: expected [P, C], [B, P, C] or [B, 1, P, C]");
+    const int64_t taps = kx * ky, P = input.size(-2), C = input.size(-1), B = input.dim() > 2 ? input.size(0) : 1;
+    TORCH_CHECK(weights.scalar_type() == torch::kInt32 && weights.dim() == 4 && weights.size(0) == 1 &&
+                    weights.size(1) * weights.size(2) == taps && weights.size(3) == (C + 15) / 16,
+                "ternary_dwconvtrans_cuda: compact weights do not match kernel size and channels");
+    const c10::DeviceGuard guard(input.device());
+    auto x = input.contiguous();
+    auto w = weights.contiguous();
+    std::vector<int64_t> shape = input.sizes().vec();
+    shape[shape.size() - 2] = C * taps;
+    shape.back() = P;
+    auto y = torch::empty(shape, input.options());
+    if (y.numel())
+        check(tmq_ternary_dwconvtrans_cols(x.data_ptr<float>(), B, P, (int32_t)taps, C,
+                                           reinterpret_cast<const uint32_t *>(w.data_ptr<int32_t>()), y.data_ptr<float>(),
+                                           stream_of(x)), "ternary_dwconvtrans_cuda");
+    return y;
 }
 
 // ---- pack / unpack / codec (tmq/tmq_native.cpp:418-544) -------------------------------------------------

@@ -505,6 +505,65 @@ def ternary_dwconv_cuda(input: torch.Tensor, weights: torch.Tensor, kx: int, ky:
     return y
 
 
+def ternary_dwconvtrans2d(x: torch.Tensor, words: torch.Tensor, kernel, stride=1, padding=0, output_padding=0, dilation=1,
+                          scale=None, bias=None, residual=None, relu=False, out_dtype=torch.float32) -> torch.Tensor:
+    """Depthwise transposed ternary convolution (groups == channels, one filter per channel) straight
+    from the compact words of a [C, 1, ky, kx] weight tensor, gathered per output position -- no
+    columns, no fold. x: fp16 [B, C, H, W] in channels_last memory (anything else is converted first);
+    returns [B, C, Ho, Wo] in channels_last memory, extents by nn.ConvTranspose2d's formula."""
+    pair = lambda v: tuple(v) if isinstance(v, (tuple, list)) else (v, v)
+    (ky, kx), (sy, sx), (py, px), (oy, ox), (dy, dx) = (pair(kernel), pair(stride), pair(padding), pair(output_padding),
+                                                       pair(dilation))
+    if not x.is_cuda or x.dim() != 4:
+        raise RuntimeError("ternary_dwconvtrans2d: expected a 4-D GPU tensor")
+    B, C, H, W = x.shape
+    _capi.require_gpu(words, "words")
+    if words.dtype != torch.int32 or words.numel() != ky * kx * ((C + 15) // 16):
+        raise RuntimeError("ternary_dwconvtrans2d: expected the int32 compact words of a [C, 1, ky, kx] weight tensor")
+    if x.dtype != torch.float16 or not x.is_contiguous(memory_format=torch.channels_last):
+        x = x.to(dtype=torch.float16, memory_format=torch.channels_last)
+    words = words.contiguous()
+    shp = _capi.ConvShape(B, C, H, W, C, ky, kx, sy, sx, py, px, dy, dx, py, px)
+    ho, wo = ctypes.c_int32(0), ctypes.c_int32(0)
+    lib = _lib()
+    check(lib.tmq_convtranspose2d_out_hw(ctypes.byref(shp), oy, ox, ctypes.byref(ho), ctypes.byref(wo)),
+          "convtranspose2d_out_hw")
+    y = torch.empty((B, C, ho.value, wo.value), dtype=out_dtype, device=x.device, memory_format=torch.channels_last)
+    ep = _epilogue(_Channels(C), scale, bias, residual, relu, out_dtype, y)
+    with torch.cuda.device(x.device):
+        check(lib.tmq_ternary_dwconvtrans2d(ptr(x), ctypes.byref(shp), oy, ox, ptr(words), ctypes.byref(ep), ptr(y),
+                                            stream_of(x)), "ternary_dwconvtrans2d")
+    return y
+
+
+def ternary_dwconvtrans_cuda(input: torch.Tensor, weights: torch.Tensor, kx: int, ky: int) -> torch.Tensor:
+    """The reference's binding (tmq/tmq_cuda.cu:645-686, caller tmq/tmq.py:1026-1029): input fp32
+    [P, C], [B, P, C] or [B, 1, P, C]; weights the compact words of the [C, 1, ky, kx] kernel, shaped
+    [1, *, *, ceil(C/16)]; returns fp32 [C*ky*kx, P], [B, C*ky*kx, P] or [B, 1, C*ky*kx, P] with
+    out[c*taps + t][p] = input[p][c] * T[c][t], ready for F.fold. Every batch entry is computed and a
+    4-D input gives the 4-D output (the reference's host fills entry 0 only and overwrites the 4-D
+    result with a 2-D one, tmq/tmq_cuda.cu:677-682)."""
+    if not input.is_cuda or not weights.is_cuda:
+        raise RuntimeError("ternary_dwconvtrans_cuda: expected tensors on the GPU")
+    if input.dtype != torch.float32:
+        raise RuntimeError("ternary_dwconvtrans_cuda: expected fp32 input")
+    if input.dim() not in (2, 3, 4) or (input.dim() == 4 and input.shape[1] != 1):
+        raise RuntimeError("ternary_dwconvtrans_cuda: expected [P, C], [B, P, C] or [B, 1, P, C]")
+    taps = int(kx) * int(ky)
+    P, C = int(input.shape[-2]), int(input.shape[-1])
+    B = int(input.shape[0]) if input.dim() > 2 else 1
+    if weights.dtype != torch.int32 or weights.dim() != 4 or weights.shape[0] != 1 or \
+            weights.shape[1] * weights.shape[2] != taps or weights.shape[3] != (C + 15) // 16:
+        raise RuntimeError("ternary_dwconvtrans_cuda: compact weights do not match kernel size and channels")
+    x = input.contiguous()
+    y = torch.empty(tuple(input.shape[:-2]) + (C * taps, P), dtype=torch.float32, device=x.device)
+    if y.numel():
+        with torch.cuda.device(x.device):
+            check(_lib().tmq_ternary_dwconvtrans_cols(ptr(x), B, P, taps, C, ptr(weights.contiguous()), ptr(y), stream_of(x)),
+                  "ternary_dwconvtrans_cuda")
+    return y
+
+
 def _check_mm_args(lhs, weights, columns, name):
     # tmq/tmq_cuda.cu:480-490, 566-575
     if not lhs.is_cuda or not weights.is_cuda:

@@ -655,8 +655,8 @@ class Conv2d(nn.Module, TMQLayer):
 
 
 class ConvTranspose2d(Conv2d):
-    """Quantization-aware drop-in for nn.ConvTranspose2d (tmq/tmq.py:978-1087), with a working compact
-    path for groups == 1 (the reference's own cannot pass its shape checks)."""
+    """Quantization-aware drop-in for nn.ConvTranspose2d (tmq/tmq.py:978-1087), with working compact
+    paths for groups == 1 (the reference's own cannot pass its shape checks) and groups == channels."""
 
     _transposed = True
 
@@ -684,15 +684,23 @@ class ConvTranspose2d(Conv2d):
         sum_ci x[b, ci, p] W[ci, co, i, j], then F.fold scatters the columns (the plan of
         tmq/tmq.py:1005-1038, whose own shape checks reject its weight view). The compact tensor of a
         [Cin, Cout, ky, kx] kernel packs along Cin, the reduction index here, so it is unpacked and
-        re-packed along (co, i, j) once per layer. groups == 1 only."""
+        re-packed along (co, i, j) once per layer. groups == channels takes the depthwise kernel instead."""
         assert not self.training, "Compact inference is not supported in training mode"
         assert self.weight.data.dtype == torch.int32, "Compact inference requires 32-bit integer words"
         self._update_scale()
         if x.dim() == 3:
             return self.compact_forward(x.unsqueeze(0)).squeeze(0)
-        if self.groups != 1:
-            raise NotImplementedError("grouped transposed compact inference is not part of this build")
         cin, cout, ky, kx = (int(v) for v in self.original_shape)
+        if self.groups != 1:
+            # depthwise (tmq/tmq.py:1025-1029, columns + F.fold there): gathered per output position
+            # straight from the compact words
+            assert self.groups == cin, "Grouped transpose convolutions are only supported for channels == groupsize"
+            if cout != 1 or x.shape[1] != cin:
+                raise RuntimeError("depthwise transposed compact inference needs one filter per input channel")
+            bias = self.bias.data.float() if self.bias is not None else None
+            return ops.ternary_dwconvtrans2d(x, self.weight.data, (ky, kx), _pair(self.stride), _pair(self.padding),
+                                             _pair(self.output_padding), _pair(self.dilation),
+                                             scale=self._epilogue_scale(cin, x.device), bias=bias)
         w = self.weight.data
         key = (w.data_ptr(), tuple(w.shape), w._version)
         if self._native is None or self._native[0] != key:
