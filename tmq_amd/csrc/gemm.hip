@@ -19,6 +19,7 @@
 //     mod 8) cover neighbouring tiles and share activation rows in that XCD's L2.
 #include "common.h"
 #include "mfma.h"
+#include "tile_epilogue.h"
 #include <type_traits>
 
 namespace tmq {
@@ -37,15 +38,6 @@ constexpr int kPitch = 64;       // LDS row pitch in halfs: 128 bytes = 8 chunks
 // Chunk c of row r is stored at position c ^ (r & 7): a wavefront's stores cover whole rows
 // (contiguous kilobytes) and the operand reads of 8 consecutive rows at one k offset land in 8
 // different 16-byte bank groups.
-
-struct Epilogue {
-    const float *scale;      // [N] or null
-    const float *bias;       // [N] or null
-    const void *residual;    // same shape/dtype as y, or null
-    void *y;
-    int relu;
-    int y_f16;
-};
 
 // ---- loaders ------------------------------------------------------------------------------------------
 // A loader hands every thread CH 16-byte chunks (8 fp16) of the BM x 64 activation tile: chunk i of
@@ -305,76 +297,6 @@ struct ConvLoaderFewC {
         while (st.j >= kx) { st.j -= kx; ++st.i; }
     }
 };
-
-// Epilogue of one wavefront's (16 WM) x (16 WN) accumulator block. A lane holds rows 4g + r, column
-// r16 of each 16 x 16 accumulator -- 64-byte row pieces if stored directly. Instead the wavefront
-// transposes one 16-row slab (16 x 16 WN values) at a time through its own slice of LDS (`slab`, the
-// idle activation buffer) and writes whole rows: 16 lanes x 16 bytes = 256 contiguous bytes per row and
-// store instruction. sc / bi: per-column scale (weight unit folded in) and bias of column r16 of fragment j.
-template <int WM, int WN>
-__device__ __forceinline__ void write_tile(float *slab, const floatx4 (&acc)[WM][WN], const float (&sc)[WN],
-                                           const float (&bi)[WN], int lane, int64_t mw0, int64_t nw0, int64_t M,
-                                           int64_t N, const Epilogue &ep) {
-    constexpr int kEP = 16 * WN + 4;                       // slab row pitch in floats (+4: conflict-free)
-    const int r16 = lane & 15, g = lane >> 4;
-    const bool vec = (N % 4 == 0) && ((reinterpret_cast<uintptr_t>(ep.y) | reinterpret_cast<uintptr_t>(ep.residual)) & 15u) == 0;
-#pragma unroll
-    for (int i = 0; i < WM; i++) {
-#pragma unroll
-        for (int j = 0; j < WN; j++)
-#pragma unroll
-            for (int r = 0; r < 4; r++) slab[(g * 4 + r) * kEP + j * 16 + r16] = acc[i][j][r] * sc[j] + bi[j];
-        __builtin_amdgcn_wave_barrier();
-        const int64_t mrow0 = mw0 + (int64_t)i * 16;
-#pragma unroll
-        for (int t = 0; t < WN; t++) {                     // 16 rows x (16 WN / 4) float4 = 64 WN float4 per slab
-            const int idx = t * 64 + lane, row = idx / (4 * WN), c4 = idx % (4 * WN);
-            const int64_t m = mrow0 + row, n = nw0 + c4 * 4;
-            floatx4 v = *reinterpret_cast<const floatx4 *>(&slab[row * kEP + c4 * 4]);
-            if (m >= M || n >= N) continue;
-            const int64_t o = m * N + n;
-            if (vec) {
-                if (ep.y_f16) {
-                    if (ep.residual) {
-                        const half4 rs = *reinterpret_cast<const half4 *>(static_cast<const _Float16 *>(ep.residual) + o);
-#pragma unroll
-                        for (int e = 0; e < 4; e++) v[e] += (float)rs[e];
-                    }
-                    half4 h;
-#pragma unroll
-                    for (int e = 0; e < 4; e++) h[e] = (_Float16)((ep.relu && v[e] < 0.f) ? 0.f : v[e]);
-                    *reinterpret_cast<half4 *>(static_cast<_Float16 *>(ep.y) + o) = h;
-                } else {
-                    if (ep.residual) {
-                        const floatx4 rs = *reinterpret_cast<const floatx4 *>(static_cast<const float *>(ep.residual) + o);
-                        v += rs;
-                    }
-                    if (ep.relu) {
-#pragma unroll
-                        for (int e = 0; e < 4; e++) v[e] = v[e] > 0.f ? v[e] : 0.f;
-                    }
-                    __builtin_nontemporal_store(v, reinterpret_cast<floatx4 *>(static_cast<float *>(ep.y) + o));
-                }
-            } else {
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    if (n + e >= N) break;
-                    float f = v[e];
-                    if (ep.y_f16) {
-                        if (ep.residual) f += (float)static_cast<const _Float16 *>(ep.residual)[o + e];
-                        if (ep.relu) f = f > 0.f ? f : 0.f;
-                        static_cast<_Float16 *>(ep.y)[o + e] = (_Float16)f;
-                    } else {
-                        if (ep.residual) f += static_cast<const float *>(ep.residual)[o + e];
-                        if (ep.relu) f = f > 0.f ? f : 0.f;
-                        static_cast<float *>(ep.y)[o + e] = f;
-                    }
-                }
-            }
-        }
-        __builtin_amdgcn_wave_barrier();
-    }
-}
 
 // ---- the tile kernel ---------------------------------------------------------------------------------
 template <int WM, int WN, int WGM, int WGN, int D, class Loader>
