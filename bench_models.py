@@ -122,16 +122,14 @@ class FusedTernaryResNet18:
     @torch.no_grad()
     def __call__(self, x):
         B, C, H, W = x.shape
-        nhwc4 = torch.empty((B, H, W, 4), dtype=torch.float16, device=x.device)
-        nhwc4[..., :C] = x.permute(0, 2, 3, 1)
-        nhwc4[..., C:] = 0
+        nhwc4 = self.ops.nchw_to_nhwc4(x)
         xs = nhwc4.view(B, H, W // 2, 8).permute(0, 3, 1, 2)      # [B, 8, H, W / 2], channels_last memory
         y = self._run(xs, self.stem, relu=True)
-        y = torch.nn.functional.max_pool2d(y, 3, 2, 1)
+        y = self.ops.maxpool2d_nhwc(y, 3, 2, 1)
         for c1, c2, ds in self.blocks:
             idt = y if ds is None else self._run(y, ds, relu=False)
             h = self._run(y, c1, relu=True)
             y = self._run(h, c2, relu=True, residual=idt)
-        feat = y.float().mean(dim=(2, 3)).half().contiguous()
+        feat = self.ops.avgpool_global_nhwc(y)
         nw, bias = self.fc
         return self.ops.ternary_linear(feat, nw, bias=bias)

@@ -280,6 +280,27 @@ int tmq_ternary_dwconvtrans_cols(const float *x, int64_t B, int64_t P, int32_t t
                                  const uint32_t *words, float *y, void *stream);
 
 /* ------------------------------------------------------------------------------------------
+ * Memory-bound companions of the convolutions on fp16 NHWC feature maps. No counterpart in the
+ * reference, whose ResNet sample (samples/resnet_test.py:91-118) leaves pooling to PyTorch on NCHW
+ * fp32 tensors; a network that keeps fp16 NHWC between the ternary convolutions needs them.
+ * ---------------------------------------------------------------------------------------- */
+
+/* Max-pool, PyTorch's nn.MaxPool2d(kernel, stride, padding) with dilation 1 and floor mode:
+ * x [B][H][W][C] fp16 -> y [B][Ho][Wo][C] fp16, Ho = floor((H + 2 py - ky) / sy) + 1. Padding takes
+ * no part in the maximum (needs 2 p <= k).                                                       */
+int tmq_maxpool2d_nhwc(const void *x, int32_t B, int32_t C, int32_t H, int32_t W, int32_t ky, int32_t kx,
+                       int32_t sy, int32_t sx, int32_t py, int32_t px, void *y, void *stream);
+
+/* Global average pool: x [B][HW][C] fp16 -> y [B][C] (TMQ_F16 or TMQ_F32), fp32 accumulation.    */
+int tmq_avgpool_global_nhwc(const void *x, int64_t B, int64_t HW, int64_t C, void *y, int y_dtype,
+                            void *stream);
+
+/* Network input repack: x [B][C][H][W] (TMQ_F16 or TMQ_F32, C <= 4, W % 4 == 0) -> y [B][H][W][4]
+ * fp16, channels C..3 zero (the layout the few-channel convolution loader wants).               */
+int tmq_nchw_to_nhwc4(const void *x, int x_dtype, int64_t B, int32_t C, int64_t H, int64_t W, void *y,
+                      void *stream);
+
+/* ------------------------------------------------------------------------------------------
  * Host entropy codec for packed tensors (host memory in, host memory out; no GPU involved).
  * ---------------------------------------------------------------------------------------- */
 

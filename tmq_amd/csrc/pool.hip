@@ -1,0 +1,169 @@
+// Memory-bound companions of the ternary convolutions for fp16 NHWC feature maps, gfx950: max-pool,
+// global average pool, and the NCHW -> NHWC repack of a few-channel network input. Each is one pass
+// with 16-byte accesses (8 fp16 channels per thread); arithmetic is negligible, the bound is HBM.
+// The reference has no kernels for these: its ResNet sample (samples/resnet_test.py:91-118) runs
+// torchvision's NCHW fp32 model and so uses PyTorch's pooling.
+#include "common.h"
+#include "mfma.h"
+
+namespace tmq {
+namespace {
+
+// y[b][oh][ow][c] = max over the window of x[b][oh sy - py + i][ow sx - px + j][c]; taps outside the
+// image do not take part (PyTorch's implicit -inf padding). Thread = 8 channels of one output pixel.
+// NaN inputs: the packed fp16 maximum returns the other operand (IEEE maxNum), where PyTorch would
+// propagate the NaN.
+__global__ __launch_bounds__(256) void maxpool_nhwc_kernel(const _Float16 *__restrict__ x, int B, int C, int H, int W, int Ho,
+                                                           int Wo, int ky, int kx, int sy, int sx, int py, int px, int vec,
+                                                           _Float16 *__restrict__ y) {
+    const int64_t G = (C + 7) / 8;
+    const int64_t id = (int64_t)blockIdx.x * 256 + threadIdx.x, total = (int64_t)B * Ho * Wo * G;
+    if (id >= total) return;
+    const int64_t p = id / G, c0 = (id - p * G) * 8;
+    const int ow = (int)(p % Wo);
+    const int64_t r = p / Wo;
+    const int oh = (int)(r % Ho), b = (int)(r / Ho);
+    const _Float16 ninf = (_Float16)(-__builtin_inff());
+    half8 best = {ninf, ninf, ninf, ninf, ninf, ninf, ninf, ninf};
+    for (int i = 0; i < ky; i++) {
+        const int ih = oh * sy - py + i;
+        if (ih < 0 || ih >= H) continue;
+        for (int j = 0; j < kx; j++) {
+            const int iw = ow * sx - px + j;
+            if (iw < 0 || iw >= W) continue;
+            const _Float16 *src = x + (((int64_t)b * H + ih) * W + iw) * C + c0;
+            half8 v = best;
+            if (vec) {
+                v = *reinterpret_cast<const half8 *>(src);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; e++)
+                    if (c0 + e < C) v[e] = src[e];
+            }
+            best = __builtin_elementwise_max(best, v);
+        }
+    }
+    _Float16 *dst = y + p * C + c0;
+    if (vec) {
+        *reinterpret_cast<half8 *>(dst) = best;
+    } else {
+#pragma unroll
+        for (int e = 0; e < 8; e++)
+            if (c0 + e < C) dst[e] = best[e];
+    }
+}
+
+// y[b][c] = mean over the HW positions of x[b][.][c], fp32 accumulation in position order.
+// Thread = 8 channels of one image.
+__global__ __launch_bounds__(64) void avgpool_global_nhwc_kernel(const _Float16 *__restrict__ x, int64_t B, int64_t HW, int64_t C,
+                                                                 int vec, void *__restrict__ y, int y_f16) {
+    const int64_t G = (C + 7) / 8;
+    const int64_t id = (int64_t)blockIdx.x * 64 + threadIdx.x;
+    if (id >= B * G) return;
+    const int64_t b = id / G, c0 = (id - b * G) * 8;
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    const _Float16 *src = x + b * HW * C + c0;
+    for (int64_t p = 0; p < HW; p++, src += C) {
+        if (vec) {
+            const half8 v = *reinterpret_cast<const half8 *>(src);
+#pragma unroll
+            for (int e = 0; e < 8; e++) acc[e] += (float)v[e];
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; e++)
+                if (c0 + e < C) acc[e] += (float)src[e];
+        }
+    }
+    const float inv = 1.0f / (float)HW;
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+        if (c0 + e >= C) break;
+        const float m = acc[e] * inv;
+        if (y_f16) static_cast<_Float16 *>(y)[b * C + c0 + e] = (_Float16)m;
+        else static_cast<float *>(y)[b * C + c0 + e] = m;
+    }
+}
+
+// NCHW (fp16 or fp32, C <= 4) -> NHWC fp16 with 4 channels, the missing ones zero.
+// Thread = 4 neighbouring pixels of one row (W % 4 == 0): reads along W, writes 32 contiguous bytes.
+template <typename T>
+__global__ __launch_bounds__(256) void nchw_to_nhwc4_kernel(const T *__restrict__ x, int64_t B, int C, int64_t H, int64_t W,
+                                                            _Float16 *__restrict__ y) {
+    const int64_t W4 = W / 4;
+    const int64_t id = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (id >= B * H * W4) return;
+    const int64_t w0 = (id % W4) * 4, bh = id / W4, h = bh % H, b = bh / H;
+    _Float16 px[4][4];
+#pragma unroll
+    for (int c = 0; c < 4; c++) {
+        if (c < C) {
+            const T *src = x + ((b * C + c) * H + h) * W + w0;
+#pragma unroll
+            for (int q = 0; q < 4; q++) px[q][c] = (_Float16)src[q];
+        } else {
+#pragma unroll
+            for (int q = 0; q < 4; q++) px[q][c] = (_Float16)0;
+        }
+    }
+    half8 lo = {px[0][0], px[0][1], px[0][2], px[0][3], px[1][0], px[1][1], px[1][2], px[1][3]};
+    half8 hi = {px[2][0], px[2][1], px[2][2], px[2][3], px[3][0], px[3][1], px[3][2], px[3][3]};
+    half8 *dst = reinterpret_cast<half8 *>(y + ((b * H + h) * W + w0) * 4);
+    dst[0] = lo;
+    dst[1] = hi;
+}
+
+}  // namespace
+}  // namespace tmq
+
+using namespace tmq;
+
+extern "C" {
+
+int tmq_maxpool2d_nhwc(const void *x, int32_t B, int32_t C, int32_t H, int32_t W, int32_t ky, int32_t kx, int32_t sy,
+                       int32_t sx, int32_t py, int32_t px, void *y, void *stream) {
+    if (B < 0 || C <= 0 || H <= 0 || W <= 0 || ky <= 0 || kx <= 0 || sy <= 0 || sx <= 0 || py < 0 || px < 0)
+        return TMQ_ERR_INVALID_ARG;
+    if (2 * py > ky || 2 * px > kx) return TMQ_ERR_INVALID_ARG;          // PyTorch's rule: pad at most half the window
+    const int64_t ho = ((int64_t)H + 2 * py - ky) / sy + 1, wo = ((int64_t)W + 2 * px - kx) / sx + 1;
+    if ((int64_t)H + 2 * py < ky || (int64_t)W + 2 * px < kx) return TMQ_ERR_INVALID_ARG;
+    if (B == 0) return TMQ_OK;
+    if (!x || !y) return TMQ_ERR_INVALID_ARG;
+    const int64_t total = (int64_t)B * ho * wo * ((C + 7) / 8), blocks = (total + 255) / 256;
+    if (blocks > 0x7FFFFFFF) return TMQ_ERR_TOO_LARGE;
+    const int vec = (C % 8 == 0) && aligned16(x) && aligned16(y);
+    hipLaunchKernelGGL(maxpool_nhwc_kernel, dim3((uint32_t)blocks), dim3(256), 0, as_stream(stream),
+                       static_cast<const _Float16 *>(x), B, C, H, W, (int)ho, (int)wo, ky, kx, sy, sx, py, px, vec,
+                       static_cast<_Float16 *>(y));
+    return check_launch();
+}
+
+int tmq_avgpool_global_nhwc(const void *x, int64_t B, int64_t HW, int64_t C, void *y, int y_dtype, void *stream) {
+    if (B < 0 || HW <= 0 || C <= 0) return TMQ_ERR_INVALID_ARG;
+    if (y_dtype != TMQ_F16 && y_dtype != TMQ_F32) return TMQ_ERR_UNSUPPORTED;
+    if (B == 0) return TMQ_OK;
+    if (!x || !y) return TMQ_ERR_INVALID_ARG;
+    const int64_t total = B * ((C + 7) / 8), blocks = (total + 63) / 64;
+    if (blocks > 0x7FFFFFFF) return TMQ_ERR_TOO_LARGE;
+    const int vec = (C % 8 == 0) && aligned16(x);
+    hipLaunchKernelGGL(avgpool_global_nhwc_kernel, dim3((uint32_t)blocks), dim3(64), 0, as_stream(stream),
+                       static_cast<const _Float16 *>(x), B, HW, C, vec, y, y_dtype == TMQ_F16 ? 1 : 0);
+    return check_launch();
+}
+
+int tmq_nchw_to_nhwc4(const void *x, int x_dtype, int64_t B, int32_t C, int64_t H, int64_t W, void *y, void *stream) {
+    if (B < 0 || C <= 0 || C > 4 || H <= 0 || W <= 0 || W % 4 != 0) return TMQ_ERR_INVALID_ARG;
+    if (x_dtype != TMQ_F16 && x_dtype != TMQ_F32) return TMQ_ERR_UNSUPPORTED;
+    if (B == 0) return TMQ_OK;
+    if (!x || !y || !aligned16(y)) return TMQ_ERR_INVALID_ARG;
+    const int64_t total = B * H * (W / 4), blocks = (total + 255) / 256;
+    if (blocks > 0x7FFFFFFF) return TMQ_ERR_TOO_LARGE;
+    if (x_dtype == TMQ_F16)
+        hipLaunchKernelGGL(nchw_to_nhwc4_kernel<_Float16>, dim3((uint32_t)blocks), dim3(256), 0, as_stream(stream),
+                           static_cast<const _Float16 *>(x), B, (int)C, H, W, static_cast<_Float16 *>(y));
+    else
+        hipLaunchKernelGGL(nchw_to_nhwc4_kernel<float>, dim3((uint32_t)blocks), dim3(256), 0, as_stream(stream),
+                           static_cast<const float *>(x), B, (int)C, H, W, static_cast<_Float16 *>(y));
+    return check_launch();
+}
+
+}  // extern "C"

@@ -564,6 +564,55 @@ def ternary_dwconvtrans_cuda(input: torch.Tensor, weights: torch.Tensor, kx: int
     return y
 
 
+def maxpool2d_nhwc(x: torch.Tensor, kernel, stride=None, padding=0) -> torch.Tensor:
+    """nn.MaxPool2d(kernel, stride, padding) on an fp16 [B, C, H, W] tensor in channels_last memory
+    (anything else is converted first); returns [B, C, Ho, Wo] fp16 in channels_last memory."""
+    pair = lambda v: tuple(v) if isinstance(v, (tuple, list)) else (v, v)
+    (ky, kx), (py, px) = pair(kernel), pair(padding)
+    sy, sx = pair(stride) if stride is not None else (ky, kx)
+    if not x.is_cuda or x.dim() != 4:
+        raise RuntimeError("maxpool2d_nhwc: expected a 4-D GPU tensor")
+    if x.dtype != torch.float16 or not x.is_contiguous(memory_format=torch.channels_last):
+        x = x.to(dtype=torch.float16, memory_format=torch.channels_last)
+    B, C, H, W = x.shape
+    if 2 * py > ky or 2 * px > kx or H + 2 * py < ky or W + 2 * px < kx:
+        raise RuntimeError("maxpool2d_nhwc: pad should be at most half of the kernel size and the window must fit")
+    ho, wo = (H + 2 * py - ky) // sy + 1, (W + 2 * px - kx) // sx + 1
+    y = torch.empty((B, C, ho, wo), dtype=torch.float16, device=x.device, memory_format=torch.channels_last)
+    with torch.cuda.device(x.device):
+        check(_lib().tmq_maxpool2d_nhwc(ptr(x), B, C, H, W, ky, kx, sy, sx, py, px, ptr(y), stream_of(x)), "maxpool2d_nhwc")
+    return y
+
+
+def avgpool_global_nhwc(x: torch.Tensor, out_dtype=torch.float16) -> torch.Tensor:
+    """Mean over H x W of an fp16 [B, C, H, W] tensor in channels_last memory -> [B, C]."""
+    if not x.is_cuda or x.dim() != 4:
+        raise RuntimeError("avgpool_global_nhwc: expected a 4-D GPU tensor")
+    if x.dtype != torch.float16 or not x.is_contiguous(memory_format=torch.channels_last):
+        x = x.to(dtype=torch.float16, memory_format=torch.channels_last)
+    B, C, H, W = x.shape
+    y = torch.empty((B, C), dtype=out_dtype, device=x.device)
+    with torch.cuda.device(x.device):
+        check(_lib().tmq_avgpool_global_nhwc(ptr(x), B, H * W, C, ptr(y), _capi.dtype_code(y), stream_of(x)),
+              "avgpool_global_nhwc")
+    return y
+
+
+def nchw_to_nhwc4(x: torch.Tensor) -> torch.Tensor:
+    """Contiguous NCHW network input (fp16 or fp32, at most 4 channels, W a multiple of 4) -> fp16
+    [B, H, W, 4] with the missing channels zero."""
+    if not x.is_cuda or x.dim() != 4 or x.dtype not in (torch.float16, torch.float32):
+        raise RuntimeError("nchw_to_nhwc4: expected a 4-D fp16 / fp32 GPU tensor")
+    x = x.contiguous()
+    B, C, H, W = x.shape
+    if C > 4 or W % 4:
+        raise RuntimeError("nchw_to_nhwc4: at most 4 channels, width a multiple of 4")
+    y = torch.empty((B, H, W, 4), dtype=torch.float16, device=x.device)
+    with torch.cuda.device(x.device):
+        check(_lib().tmq_nchw_to_nhwc4(ptr(x), _capi.dtype_code(x), B, C, H, W, ptr(y), stream_of(x)), "nchw_to_nhwc4")
+    return y
+
+
 def _check_mm_args(lhs, weights, columns, name):
     # tmq/tmq_cuda.cu:480-490, 566-575
     if not lhs.is_cuda or not weights.is_cuda:
