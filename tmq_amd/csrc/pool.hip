@@ -53,32 +53,51 @@ __global__ __launch_bounds__(256) void maxpool_nhwc_kernel(const _Float16 *__res
     }
 }
 
-// y[b][c] = mean over the HW positions of x[b][.][c], fp32 accumulation in position order.
-// Thread = 8 channels of one image.
-__global__ __launch_bounds__(64) void avgpool_global_nhwc_kernel(const _Float16 *__restrict__ x, int64_t B, int64_t HW, int64_t C,
-                                                                 int vec, void *__restrict__ y, int y_f16) {
-    const int64_t G = (C + 7) / 8;
-    const int64_t id = (int64_t)blockIdx.x * 64 + threadIdx.x;
-    if (id >= B * G) return;
-    const int64_t b = id / G, c0 = (id - b * G) * 8;
+// y[b][c] = mean over the HW positions of x[b][.][c], fp32 accumulation. A workgroup = one image x 64
+// groups of 8 channels; its four wavefronts take every fourth position each (loads of a wavefront are
+// one contiguous KiB, several in flight), then the four partial sums are added in wavefront order.
+__global__ __launch_bounds__(256) void avgpool_global_nhwc_kernel(const _Float16 *__restrict__ x, int64_t B, int64_t HW, int64_t C,
+                                                                  int vec, void *__restrict__ y, int y_f16) {
+    __shared__ float part[4][64][9];
+    const int64_t G = (C + 7) / 8, GB = (G + 63) / 64;
+    const int64_t b = blockIdx.x / GB, cg = (blockIdx.x % GB) * 64 + (threadIdx.x & 63);
+    const int lane = threadIdx.x & 63, slice = threadIdx.x >> 6;
+    const int64_t c0 = cg * 8;
     float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    const _Float16 *src = x + b * HW * C + c0;
-    for (int64_t p = 0; p < HW; p++, src += C) {
+    if (cg < G) {
+        const _Float16 *src = x + b * HW * C + c0;
         if (vec) {
-            const half8 v = *reinterpret_cast<const half8 *>(src);
+            int64_t p = slice;
+            for (; p + 12 < HW; p += 16) {             // four loads in flight
+                half8 v[4];
 #pragma unroll
-            for (int e = 0; e < 8; e++) acc[e] += (float)v[e];
+                for (int u = 0; u < 4; u++) v[u] = *reinterpret_cast<const half8 *>(src + (p + 4 * u) * C);
+#pragma unroll
+                for (int u = 0; u < 4; u++)
+#pragma unroll
+                    for (int e = 0; e < 8; e++) acc[e] += (float)v[u][e];
+            }
+            for (; p < HW; p += 4) {
+                const half8 v = *reinterpret_cast<const half8 *>(src + p * C);
+#pragma unroll
+                for (int e = 0; e < 8; e++) acc[e] += (float)v[e];
+            }
         } else {
+            for (int64_t p = slice; p < HW; p += 4)
 #pragma unroll
-            for (int e = 0; e < 8; e++)
-                if (c0 + e < C) acc[e] += (float)src[e];
+                for (int e = 0; e < 8; e++)
+                    if (c0 + e < C) acc[e] += (float)src[p * C + e];
         }
     }
+#pragma unroll
+    for (int e = 0; e < 8; e++) part[slice][lane][e] = acc[e];
+    __syncthreads();
+    if (slice != 0 || cg >= G) return;
     const float inv = 1.0f / (float)HW;
 #pragma unroll
     for (int e = 0; e < 8; e++) {
         if (c0 + e >= C) break;
-        const float m = acc[e] * inv;
+        const float m = (((part[0][lane][e] + part[1][lane][e]) + part[2][lane][e]) + part[3][lane][e]) * inv;
         if (y_f16) static_cast<_Float16 *>(y)[b * C + c0 + e] = (_Float16)m;
         else static_cast<float *>(y)[b * C + c0 + e] = m;
     }
@@ -142,10 +161,10 @@ int tmq_avgpool_global_nhwc(const void *x, int64_t B, int64_t HW, int64_t C, voi
     if (y_dtype != TMQ_F16 && y_dtype != TMQ_F32) return TMQ_ERR_UNSUPPORTED;
     if (B == 0) return TMQ_OK;
     if (!x || !y) return TMQ_ERR_INVALID_ARG;
-    const int64_t total = B * ((C + 7) / 8), blocks = (total + 63) / 64;
+    const int64_t blocks = B * (((C + 7) / 8 + 63) / 64);
     if (blocks > 0x7FFFFFFF) return TMQ_ERR_TOO_LARGE;
     const int vec = (C % 8 == 0) && aligned16(x);
-    hipLaunchKernelGGL(avgpool_global_nhwc_kernel, dim3((uint32_t)blocks), dim3(64), 0, as_stream(stream),
+    hipLaunchKernelGGL(avgpool_global_nhwc_kernel, dim3((uint32_t)blocks), dim3(256), 0, as_stream(stream),
                        static_cast<const _Float16 *>(x), B, HW, C, vec, y, y_dtype == TMQ_F16 ? 1 : 0);
     return check_launch();
 }

@@ -617,10 +617,55 @@ class Conv2d(nn.Module, TMQLayer):
             bias = self.bias.data.float() if self.bias is not None else None
             return ops.ternary_dwconv2d(x, self.weight.data, (ky, kx), _pair(self.stride), _pair(self.padding),
                                         _pair(self.dilation), scale=self._epilogue_scale(x.shape[1], x.device), bias=bias)
-        nw = self._native_weights(conv_kernel=(ky, kx))
         bias = self.bias.data.float() if self.bias is not None else None
+        sp = self._superpixel_plan(x)
+        if sp is not None:
+            # a network's first layer (at most 4 input channels, horizontal stride 2): two neighbouring
+            # pixels of the 4-channel NHWC image are read as one pixel of 8 channels, see _superpixel_plan
+            nw, kxs, pl, pr = sp
+            B, C, H, W = x.shape
+            xs = ops.nchw_to_nhwc4(x).view(B, H, W // 2, 8).permute(0, 3, 1, 2)
+            (sy, _), (py, _) = _pair(self.stride), _pair(self.padding)
+            return ops.ternary_conv2d(xs, nw, (sy, 1), ((py, py), (pl, pr)), 1,
+                                      scale=self._epilogue_scale(nw.N, x.device), bias=bias)
+        nw = self._native_weights(conv_kernel=(ky, kx))
         return ops.ternary_conv2d(x, nw, _pair(self.stride), _pair(self.padding), _pair(self.dilation),
                                   scale=self._epilogue_scale(nw.N, x.device), bias=bias)
+
+    def _superpixel_plan(self, x):
+        """For a convolution with at most 4 input channels, horizontal stride 2 and no dilation on an
+        NCHW fp16 / fp32 input of even width: the equivalent stride-1 convolution over "super-pixels"
+        (pixels 2u and 2u + 1 of the image stored NHWC with 4 channels, read as one pixel of 8
+        channels). Output column ow reads image columns 2 ow - px + j = 2 (ow + t) + v with
+        t = floor((j - px) / 2), v = (j - px) mod 2, so super-pixel tap t, channel 4 v + c carries the
+        weight of (c, j) and the taps t_min .. t_max replace the kx image taps: the reduction is
+        ky * kxs * 8 long (224 for a 7 x 7 / 2 stem) where padding 3 channels to 8 would make it
+        ky * kx * 8 (392), and the 16-byte loader applies instead of the scalar one.
+        Returns (native weights, kxs, pad left, pad right) or None when the layer does not qualify."""
+        N, C, ky, kx = (int(v) for v in self.original_shape)
+        (sy, sx), (py, px), (dy, dx) = _pair(self.stride), _pair(self.padding), _pair(self.dilation)
+        W = int(x.shape[-1])
+        if C > 4 or x.shape[1] != C or sx != 2 or (dy, dx) != (1, 1) or W % 4 or x.dtype not in (torch.float16, torch.float32) or \
+                isinstance(py, (tuple, list)) or isinstance(px, (tuple, list)):
+            return None
+        t_min, t_max = (-px) // 2, (kx - 1 - px) // 2
+        kxs, pl = t_max - t_min + 1, -t_min
+        wo = (W + 2 * px - kx) // 2 + 1
+        pr = wo - 1 + kxs - W // 2 - pl
+        if wo < 1 or pr < 0:
+            return None
+        w = self.weight.data
+        key = (w.data_ptr(), tuple(w.shape), w._version, "superpixel")
+        if self._native is None or self._native[0] != key:
+            full = ops.expand_ternary(w, [N, C, ky, kx])
+            wsp = torch.zeros((N, 8, ky, kxs), dtype=full.dtype, device=full.device)
+            for t in range(kxs):
+                for v in range(2):
+                    j = 2 * (t + t_min) + v + px
+                    if 0 <= j < kx:
+                        wsp[:, 4 * v:4 * v + C, :, t] = full[:, :, :, j]
+            self._native = (key, ops.NativeWeights(ops.compactify_ternary(wsp), N, (ky, kxs)))
+        return self._native[1], kxs, pl, pr
 
     @classmethod
     def from_conv2d(cls, source: nn.Conv2d, name: str, ctrl: QuantizationControl):
