@@ -285,7 +285,10 @@ def bench_resnet_infer(args, torch):
     x = torch.randn(B, 3, 224, 224, generator=torch.Generator().manual_seed(20)).half().to(dev)
     fused = FusedTernaryResNet18(model)
     out = {}
-    for name, fn, reps in (("fused", lambda: fused(x), args.steps), ("drop_in", lambda: model(x), max(3, args.steps // 4))):
+    for name, fn, reps in (("fused", lambda: fused(x), args.steps), ("drop_in", lambda: model(x), max(3, args.steps // 4)),
+                           ("drop_in_bn_folded", lambda: model(x), max(3, args.steps // 4))):
+        if name == "drop_in_bn_folded":
+            t.fold_batchnorm(model)                           # BatchNorm into the convolutions' epilogues
         with torch.no_grad():
             for _ in range(max(2, args.warmup // 4)):
                 fn()

@@ -1,0 +1,77 @@
+"""fold_batchnorm: eval-mode BatchNorm folded into the compact layers' epilogues must give the
+unfolded model's outputs (fp32 rounding apart), replace the BatchNorm modules and refuse misuse."""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _randomize_bn(net, g):
+    for m in net.modules():
+        if isinstance(m, (torch.nn.BatchNorm1d, torch.nn.BatchNorm2d)):
+            m.running_mean.copy_(torch.randn(m.num_features, generator=g) * 0.3)
+            m.running_var.copy_(torch.rand(m.num_features, generator=g) + 0.5)
+            m.weight.data.copy_(torch.rand(m.num_features, generator=g) + 0.5)
+            m.bias.data.copy_(torch.randn(m.num_features, generator=g) * 0.2)
+
+
+def test_fold_into_conv_and_linear(cuda):
+    import tmq_amd as t
+    g = torch.Generator().manual_seed(1)
+    torch.manual_seed(1)
+    net = torch.nn.Sequential(torch.nn.Conv2d(3, 16, 3, 2, 1, bias=True), torch.nn.BatchNorm2d(16), torch.nn.ReLU(),
+                              torch.nn.Conv2d(16, 64, 3, 1, 1, bias=False), torch.nn.BatchNorm2d(64), torch.nn.ReLU(),
+                              torch.nn.Conv2d(64, 64, 3, 1, 1, groups=64, bias=False), torch.nn.BatchNorm2d(64),
+                              torch.nn.AdaptiveAvgPool2d(1), torch.nn.Flatten(),
+                              torch.nn.Linear(64, 10), torch.nn.BatchNorm1d(10))
+    ctrl = t.QuantizationControl(post_scale=True)
+    t.quantize_model(net, ctrl)
+    _randomize_bn(net, g)
+    net.to(cuda).eval()
+    ctrl.quantize()
+    t.compressed_state_dict(net, strong=False)
+    x = torch.randn(4, 3, 16, 16, device=cuda)
+    with torch.no_grad():
+        want = net(x)
+        done = t.fold_batchnorm(net)
+        assert done == [("0", "1"), ("3", "4"), ("6", "7"), ("10", "11")]
+        assert all(isinstance(net[i], torch.nn.Identity) for i in (1, 4, 7, 11))
+        got = net(x)
+    assert torch.allclose(got, want, rtol=2e-3, atol=2e-3)
+    assert t.fold_batchnorm(net) == []                                        # nothing left to fold
+    with pytest.raises(RuntimeError):
+        t.expand_compact_layers(net)
+
+
+def test_fold_resnet_and_explicit_pairs(cuda):
+    import tmq_amd as t
+    from bench_models import ResNet18, randomize_ternary_
+    torch.manual_seed(2)
+    model = ResNet18(10)
+    ctrl = t.QuantizationControl()
+    t.quantize_model(model, ctrl)
+    randomize_ternary_(model, torch.Generator().manual_seed(2))
+    model.to(cuda)
+    ctrl.inference()
+    x = torch.randn(2, 3, 64, 64, device=cuda)
+    # unscaled ternary weights blow the activation scale up layer by layer: calibrate the BatchNorm
+    # statistics on the batch so that the fp16 inputs of the compact convolutions stay finite
+    for m in model.modules():
+        if isinstance(m, torch.nn.BatchNorm2d):
+            m.momentum = 1.0
+    model.train()
+    with torch.no_grad():
+        model(x)
+    model.eval()
+    t.compressed_state_dict(model, strong=False)
+    with torch.no_grad():
+        want = model(x)
+        assert torch.isfinite(want).all()
+        with pytest.raises(RuntimeError):
+            t.fold_batchnorm(model, pairs=[("layer1.0.conv1", "layer2.0.bn1")])   # 64 outputs, 128 features
+        assert t.fold_batchnorm(model, pairs=[("conv1", "bn1")]) == [("conv1", "bn1")]
+        done = t.fold_batchnorm(model)
+        assert len(done) == 19 and ("layer2.0.downsample.0", "layer2.0.downsample.1") in done
+        assert not any(isinstance(m, torch.nn.BatchNorm2d) for m in model.modules())
+        got = model(x)
+    assert torch.allclose(got, want, rtol=5e-3, atol=5e-3 * want.abs().max().item())

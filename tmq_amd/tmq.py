@@ -380,6 +380,7 @@ class TMQLayer:
         self._scale_dirty = True
         self._native = None          # cached kernel-native weights for compact inference
         self._scale_vec = None
+        self._fold = None            # (scale [N], bias [N]) of a BatchNorm folded into the compact epilogue
 
     def compact_inference_mode(self):
         self.training = False
@@ -431,6 +432,22 @@ class TMQLayer:
             self._scale_vec = ((self.post_scale_imm, n, device),
                                torch.full((n,), self.post_scale_imm, dtype=torch.float32, device=device))
         return self._scale_vec[1]
+
+    def _epilogue(self, n, device):
+        """(per-channel scale or None, bias or None) of the compact forward: the scalar post-scale and
+        the layer's bias, then the affine map of a folded BatchNorm (fold_batchnorm) on top:
+        bn(ps * acc + b) = (g * ps) * acc + (g * b + h)."""
+        scale = self._epilogue_scale(n, device)
+        bias = self.bias.data.float() if getattr(self, "bias", None) is not None else None
+        if self._fold is None:
+            return scale, bias
+        g, h = self._fold
+        if g.device != device:
+            g, h = g.to(device), h.to(device)
+            self._fold = (g, h)
+        scale = g * self.post_scale_imm if self.post_scale_imm != 1.0 else g
+        bias = h if bias is None else g * bias + h
+        return scale, bias
 
     def _adopt_stored_weight(self, state_dict, prefix, local_metadata):
         """Shared tail of _load_from_state_dict (tmq/tmq.py:748-765, 956-973): interpret the
@@ -518,8 +535,8 @@ class Linear(nn.Module, TMQLayer):
             assert x.shape[1] == 1, "Illegal shape supplied"
         nw = self._native_weights()
         xin = x if x.is_contiguous() else x.contiguous()
-        out = ops.ternary_linear(xin, nw, scale=self._epilogue_scale(nw.N, x.device),
-                                 bias=self.bias.data.float() if self.bias is not None else None)
+        scale, bias = self._epilogue(nw.N, x.device)
+        out = ops.ternary_linear(xin, nw, scale=scale, bias=bias)
         return self.bn(out) if self.bn is not None else out
 
     @classmethod
@@ -614,10 +631,10 @@ class Conv2d(nn.Module, TMQLayer):
             # depthwise (tmq/tmq.py:849-853): the compact words are read as they are, no re-tiling
             if self.original_shape[1] != 1 or x.shape[1] != self.original_shape[0]:
                 raise RuntimeError("depthwise compact inference needs one filter per input channel")
-            bias = self.bias.data.float() if self.bias is not None else None
+            scale, bias = self._epilogue(x.shape[1], x.device)
             return ops.ternary_dwconv2d(x, self.weight.data, (ky, kx), _pair(self.stride), _pair(self.padding),
-                                        _pair(self.dilation), scale=self._epilogue_scale(x.shape[1], x.device), bias=bias)
-        bias = self.bias.data.float() if self.bias is not None else None
+                                        _pair(self.dilation), scale=scale, bias=bias)
+        scale, bias = self._epilogue(int(self.original_shape[0]), x.device)
         sp = self._superpixel_plan(x)
         if sp is not None:
             # a network's first layer (at most 4 input channels, horizontal stride 2): two neighbouring
@@ -626,11 +643,10 @@ class Conv2d(nn.Module, TMQLayer):
             B, C, H, W = x.shape
             xs = ops.nchw_to_nhwc4(x).view(B, H, W // 2, 8).permute(0, 3, 1, 2)
             (sy, _), (py, _) = _pair(self.stride), _pair(self.padding)
-            return ops.ternary_conv2d(xs, nw, (sy, 1), ((py, py), (pl, pr)), 1,
-                                      scale=self._epilogue_scale(nw.N, x.device), bias=bias)
+            return ops.ternary_conv2d(xs, nw, (sy, 1), ((py, py), (pl, pr)), 1, scale=scale, bias=bias)
         nw = self._native_weights(conv_kernel=(ky, kx))
-        return ops.ternary_conv2d(x, nw, _pair(self.stride), _pair(self.padding), _pair(self.dilation),
-                                  scale=self._epilogue_scale(nw.N, x.device), bias=bias)
+        return ops.ternary_conv2d(x, nw, _pair(self.stride), _pair(self.padding), _pair(self.dilation), scale=scale,
+                                  bias=bias)
 
     def _superpixel_plan(self, x):
         """For a convolution with at most 4 input channels, horizontal stride 2 and no dilation on an
@@ -903,11 +919,59 @@ def _presize_weights(module: nn.Module, state_dict, prefix=""):
             layer.compact = False
 
 
+@torch.no_grad()
+def fold_batchnorm(module: nn.Module, pairs=None):
+    """Fold eval-mode BatchNorm layers into the epilogue of the compact TMQ layer that feeds them (the
+    reference's README lists this fusion as future work, README.md:150-155): the layer then computes
+    gamma * (y - mean) / sqrt(var + eps) + beta in its own per-channel scale / bias and the BatchNorm
+    module is replaced by nn.Identity. For inference only; call it after the layers went compact
+    (compressed_state_dict / load_compressed_state_dict).
+
+    pairs: [(qualified layer name, qualified BatchNorm name), ...]. None = every BatchNorm that is
+    registered right after a compact Linear / Conv2d in the same parent and has as many features as
+    that layer has outputs (the conv1 / bn1, Sequential(conv, bn) idiom) -- pass explicit pairs when
+    registration order is not execution order. Returns the list of folded pairs."""
+    def fits(layer, bn):
+        return (isinstance(layer, (Linear, Conv2d)) and not isinstance(layer, ConvTranspose2d) and layer.compact and
+                isinstance(bn, (nn.BatchNorm1d, nn.BatchNorm2d)) and bn.track_running_stats and
+                bn.num_features == int(layer.original_shape[0]))
+
+    todo = []
+    if pairs is None:
+        for pname, parent in module.named_modules():
+            kids = list(parent.named_children())
+            for (ln, layer), (bname, bn) in zip(kids, kids[1:]):
+                if fits(layer, bn) and layer._fold is None:
+                    todo.append((parent, bname, layer, bn, (pname + "." if pname else "") + ln, (pname + "." if pname else "") + bname))
+    else:
+        mods = dict(module.named_modules())
+        for ln, bname in pairs:
+            layer, bn = mods[ln], mods[bname]
+            if not fits(layer, bn):
+                raise RuntimeError(f"fold_batchnorm: {ln} / {bname} is not a compact TMQ layer followed by a matching BatchNorm")
+            parent = mods[bname.rpartition(".")[0]] if "." in bname else module
+            todo.append((parent, bname.rpartition(".")[2], layer, bn, ln, bname))
+    done = []
+    for parent, child, layer, bn, ln, bname in todo:
+        if bn.training:
+            raise RuntimeError("fold_batchnorm: BatchNorm layers must be in eval mode")
+        inv = (bn.running_var.float() + bn.eps).rsqrt()
+        g = inv * bn.weight.float() if bn.affine else inv
+        h = (bn.bias.float() if bn.affine else 0.0) - bn.running_mean.float() * g
+        layer._fold = (g.contiguous(), h.contiguous())
+        setattr(parent, child, nn.Identity())
+        done.append((ln, bname))
+    return done
+
+
 def expand_compact_layers(module: nn.Module, for_training=False):
     """Expand compact TMQ layers back to fp32 weights in place (tmq/tmq.py:1296-1319)."""
     for name, sub in module.named_children():
         if isinstance(sub, TMQLayer) and hasattr(sub, "tensor_type") and getattr(sub, "original_shape", None) is not None:
             if sub.tensor_type in (TensorType.COMPRESSED_TERNARY_32BIT, TensorType.COMPACT_TERNARY_32BIT):
+                if sub._fold is not None:
+                    raise RuntimeError("expand_compact_layers: a BatchNorm was folded into this layer (fold_batchnorm); "
+                                       "reload the model instead")
                 entropy = sub.tensor_type == TensorType.COMPRESSED_TERNARY_32BIT
                 full = _b.expand_ternary(sub.weight.data, sub.original_shape, entropy)
                 sub.weight = nn.Parameter(full, requires_grad=for_training)
