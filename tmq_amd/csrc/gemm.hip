@@ -446,15 +446,15 @@ __global__ __launch_bounds__(64 * WGM * WGN, 2) void tile_kernel(Loader ld, cons
 }
 
 // ---- the tile kernel with direct-to-LDS activation loads ----------------------------------------------
-// Same tiling and arithmetic as tile_kernel; the activation tile goes global -> LDS without passing
-// through registers (global_load_lds_dwordx4) into a ring of S buffers, S - 1 k-tiles ahead of the
-// math. That removes the staging registers and the LDS store instructions, and the prefetch depth no
-// longer costs VGPRs. The load writes lane l of a wavefront to byte 16 l of its destination, which is
+// Same tiling and arithmetic as tile_kernel; the activation tiles go global -> LDS without passing
+// through registers (global_load_lds_dwordx4). That removes the staging registers and the LDS store
+// instructions. The load writes lane l of a wavefront to byte 16 l of its destination, which is
 // exactly "row tid / 8, position tid % 8" of the 128-byte rows; the XOR swizzle is applied on the
 // global side (the thread at position p of row r fetches chunk p ^ (r % 8)).
-// The compiler does not order these loads against the operand reads: the wait for "tile kt has landed"
-// is written by hand -- every pass issues CH tile loads and WN weight loads, S - 2 passes may stay
-// outstanding -- and is followed by the pass's one barrier.
+// A pass multiplies P k-tiles out of one half of a ring of 2 P buffers while the next P tiles (and
+// their weight dwords) are on their way into the other half. The compiler does not order these loads
+// against the operand reads: each pass starts with a hand-written s_waitcnt vmcnt(0) -- everything the
+// previous pass issued has landed -- followed by the pass's one barrier.
 // 16 bytes per lane from global memory straight into LDS (the host pass does not know the builtin).
 __device__ __forceinline__ void load_to_lds(const void *src, unsigned char *dst) {
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -463,12 +463,13 @@ __device__ __forceinline__ void load_to_lds(const void *src, unsigned char *dst)
 #endif
 }
 
-template <int WM, int WN, int WGM, int WGN, int S, class Loader>
+template <int WM, int WN, int WGM, int WGN, int P, class Loader>
 __global__ __launch_bounds__(64 * WGM * WGN, 2) void tile_dma_kernel(Loader ld, const uint32_t *__restrict__ native,
                                                                   int64_t M, int64_t K, int64_t N, int64_t Kb,
                                                                   int64_t Nb, Epilogue ep, int tiles_m, int tiles_n) {
-    constexpr int T = 64 * WGM * WGN, BM = 16 * WM * WGM, BN = 16 * WN * WGN, CH = BM * 8 / T, D = S - 1;
-    static_assert(BM * 8 % T == 0 && S >= 2 && S <= 4, "geometry");
+    constexpr int T = 64 * WGM * WGN, BM = 16 * WM * WGM, BN = 16 * WN * WGN, CH = BM * 8 / T, S = 2 * P;
+    constexpr int kTileBytes = BM * kPitch * 2;
+    static_assert(BM * 8 % T == 0 && P >= 1 && P <= 2, "geometry");
     __shared__ __attribute__((aligned(16))) _Float16 As[S][BM * kPitch];
 
     int id = blockIdx.x;
@@ -499,22 +500,23 @@ __global__ __launch_bounds__(64 * WGM * WGN, 2) void tile_dma_kernel(Loader ld, 
     }
     const int KT = (int)((K + kBK - 1) / kBK);
 
-    uint32_t wcur[WN], wq[D][WN];
+    uint32_t wcur[P][WN], wnext[P][WN];
     auto wload = [&](uint32_t (&w)[WN], int kn) {
         if (kn >= KT) kn = KT - 1;
 #pragma unroll
         for (int j = 0; j < WN; j++) w[j] = wptr[j][(int64_t)(kn >> 2) * 256 + (kn & 3)];
     };
-    // tile `kn` -> ring buffer kn % S; the loader's state moves on to the next tile
+    // tile `kn` -> ring buffer `slot`; the loader's state moves on to the next tile (tiles past K, which
+    // the last pass prefetches and nobody multiplies, read whatever the loader substitutes)
     unsigned char *const lds0 = reinterpret_cast<unsigned char *>(&As[0][0]) + wv * 1024;
-    auto fill = [&](int kn) {
-        unsigned char *dst = lds0 + (kn % S) * (BM * kPitch * 2);
+    auto fill = [&](int kn, int slot) {
+        unsigned char *dst = lds0 + slot * kTileBytes;
 #pragma unroll
         for (int i = 0; i < CH; i++) load_to_lds(ld.template addr<CH, T>(st, (int64_t)kn * kBK, i), dst + i * (T * 16));
         ld.template advance<CH, T>(st);
     };
 
-    // per-column epilogue constants first (conditional loads: keep them out of the counted stream)
+    // per-column epilogue constants first (conditional loads: keep them out of the main loop)
     const int64_t nw0 = n0 + (int64_t)wn * WN * 16;
     float sc[WN], bi[WN];
 #pragma unroll
@@ -523,42 +525,28 @@ __global__ __launch_bounds__(64 * WGM * WGN, 2) void tile_dma_kernel(Loader ld, 
         sc[j] = (n < N && ep.scale ? ep.scale[n] : 1.0f) * (1.0f / kWeightUnit);
         bi[j] = (n < N && ep.bias) ? ep.bias[n] : 0.0f;
     }
-    wload(wcur, 0);
-    __builtin_amdgcn_s_waitcnt(0x0F70);            // vmcnt(0): start counting from a clean state
+#pragma unroll
+    for (int i = 0; i < P; i++) wload(wcur[i], i);
+    __builtin_amdgcn_s_waitcnt(0x0F70);            // vmcnt(0): a clean state for the compiler's own counting
     __builtin_amdgcn_sched_barrier(0);
-    // prologue: tiles 0 .. S-2 and the weights of tiles 1 .. D-1; from here on the order of issue is
-    // (S-1) x CH tile loads, (D-1) x WN weight loads, then per pass CH + WN
 #pragma unroll
-    for (int s = 0; s < S - 1; s++) fill(s);
-#pragma unroll
-    for (int d = 0; d + 1 < D; d++) wload(wq[d], d + 1);
+    for (int i = 0; i < P; i++) fill(i, i);
     __builtin_amdgcn_sched_barrier(0);
 
     const int arow = (wm * WM * 16 + r16) * kPitch;
     auto swz = [&](int i, int s) { return i * 16 * kPitch + (((4 * s + g) ^ (r16 & 7)) * 8); };
-    // vmcnt(N): at most N loads outstanding. Tile kt's loads are followed by those of S - 2 passes.
-    constexpr int kN = (S - 2) * (CH + WN);
-    constexpr int kWaitImm = (kN & 15) | (7 << 4) | (15 << 8) | ((kN >> 4) << 14);
-    static_assert(kN < 64, "vmcnt range");
-
-    auto body = [&](int kt, auto slot_tag) {
-        constexpr int slot = decltype(slot_tag)::value, freed = (slot + D - 1) % D;
-        __builtin_amdgcn_s_waitcnt(kWaitImm);       // this thread's part of tile kt is in LDS
-        __syncthreads();                             // ... and everybody's; buffer (kt - 1) % S is free
-        __builtin_amdgcn_sched_barrier(0);
-        fill(kt + S - 1);
-        wload(wq[freed], kt + D);
-        __builtin_amdgcn_sched_barrier(0);
-        const _Float16 *abase = &As[kt % S][arow];
+    // one k-tile out of ring buffer `slot`: operand reads four ahead of the MFMAs that use them
+    auto multiply = [&](int slot, const uint32_t (&w)[WN]) {
+        const _Float16 *abase = &As[0][0] + slot * (BM * kPitch) + arow;
         constexpr int NQ = 2 * WM, kAhead = NQ < 4 ? NQ : 4;
         half8 a[NQ];
         half8 bfr[2][WN];
 #pragma unroll
         for (int q = 0; q < kAhead; q++) a[q] = *reinterpret_cast<const half8 *>(abase + swz(q >> 1, q & 1));
 #pragma unroll
-        for (int j = 0; j < WN; j++) bfr[0][j] = decode_step(wcur[j], 0);
+        for (int j = 0; j < WN; j++) bfr[0][j] = decode_step(w[j], 0);
 #pragma unroll
-        for (int j = 0; j < WN; j++) bfr[1][j] = decode_step(wcur[j], 1);
+        for (int j = 0; j < WN; j++) bfr[1][j] = decode_step(w[j], 1);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int q = 0; q < NQ; q++) {
@@ -568,38 +556,44 @@ __global__ __launch_bounds__(64 * WGM * WGN, 2) void tile_dma_kernel(Loader ld, 
                 a[q + kAhead] = *reinterpret_cast<const half8 *>(abase + swz((q + kAhead) >> 1, (q + kAhead) & 1));
             __builtin_amdgcn_sched_barrier(0);
         }
-#pragma unroll
-        for (int j = 0; j < WN; j++) asm volatile("v_mov_b32 %0, %1" : "=v"(wcur[j]) : "v"(wq[slot][j]));
     };
-    int kt = 0;
-    for (; kt + D <= KT; kt += D) {
-        body(kt, std::integral_constant<int, 0>{});
-        if constexpr (D > 1) body(kt + 1, std::integral_constant<int, 1>{});
-        if constexpr (D > 2) body(kt + 2, std::integral_constant<int, 2>{});
-    }
-    if constexpr (D > 1) {
-        if (kt < KT) body(kt++, std::integral_constant<int, 0>{});
-    }
-    if constexpr (D > 2) {
-        if (kt < KT) body(kt++, std::integral_constant<int, 1>{});
+
+    int half = 0;                                    // which half of the ring is being multiplied
+    for (int kt = 0; kt < KT; kt += P) {
+        __builtin_amdgcn_s_waitcnt(0x0F70);         // this thread's part of tiles kt .. kt + P - 1 is in LDS
+        __syncthreads();                             // ... and everybody's; the other half of the ring is free
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < P; i++) fill(kt + P + i, (half ^ 1) * P + i);
+#pragma unroll
+        for (int i = 0; i < P; i++) wload(wnext[i], kt + P + i);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < P; i++)
+            if (i == 0 || kt + i < KT) multiply(half * P + i, wcur[i]);
+#pragma unroll
+        for (int i = 0; i < P; i++)
+#pragma unroll
+            for (int j = 0; j < WN; j++) asm volatile("v_mov_b32 %0, %1" : "=v"(wcur[i][j]) : "v"(wnext[i][j]));
+        half ^= 1;
     }
     // drain the prefetches past K before the buffers are reused as transpose slabs
     __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();
 
     constexpr int kEP = 16 * WN + 4;
-    static_assert(WGM * WGN * 16 * kEP * 4 <= S * BM * kPitch * 2, "epilogue slab does not fit the LDS buffer");
+    static_assert(WGM * WGN * 16 * kEP * 4 <= S * kTileBytes, "epilogue slab does not fit the LDS buffer");
     write_tile<WM, WN>(reinterpret_cast<float *>(&As[0][0]) + wv * 16 * kEP, acc, sc, bi, lane, m0 + (int64_t)wm * WM * 16,
                        nw0, M, N, ep);
 }
 
-template <int WM, int WN, int WGM, int WGN, int S, class Loader>
+template <int WM, int WN, int WGM, int WGN, int P, class Loader>
 int launch_tile_dma(const Loader &ld, const void *native, int64_t M, int64_t K, int64_t N, const Epilogue &ep,
                     void *stream) {
     constexpr int BM = 16 * WM * WGM, BN = 16 * WN * WGN;
     const int64_t tm = (M + BM - 1) / BM, tn = (N + BN - 1) / BN;
     if (tm * tn > 0x7FFFFFFF) return TMQ_ERR_TOO_LARGE;
-    hipLaunchKernelGGL((tile_dma_kernel<WM, WN, WGM, WGN, S, Loader>), dim3((uint32_t)(tm * tn)), dim3(64 * WGM * WGN), 0,
+    hipLaunchKernelGGL((tile_dma_kernel<WM, WN, WGM, WGN, P, Loader>), dim3((uint32_t)(tm * tn)), dim3(64 * WGM * WGN), 0,
                        as_stream(stream), ld, static_cast<const uint32_t *>(native), M, K, N, native_blocks_k(K),
                        native_blocks_n(N), ep, (int)tm, (int)tn);
     return check_launch();
@@ -625,11 +619,19 @@ int dispatch_tile(const Loader &ld, const void *native, int64_t M, int64_t K, in
                   void *stream) {
     auto wgs = [&](int bm, int bn) { return ((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
     if constexpr (Loader::kDirect) {
-        // direct-to-LDS kernel, one k-tile ahead (deeper rings measured slower at every shape: the
-        // extra address registers cost more occupancy than the longer prefetch gains)
-        if (N > 128 && wgs(128, 256) >= 384) return launch_tile_dma<8, 4, 1, 4, 2>(ld, native, M, K, N, ep, stream);
-        if (N > 64 && wgs(128, 128) >= 256) return launch_tile_dma<4, 4, 2, 2, 2>(ld, native, M, K, N, ep, stream);
-        return launch_tile_dma<2, 4, 2, 1, 2>(ld, native, M, K, N, ep, stream);
+        // Tiles per pass: two (half the barriers, a whole extra tile of time for the loads to land) pay
+        // on long reductions when the doubled ring does not cost residency -- the 128 x 256 tile, which
+        // runs two workgroups per CU either way, and 128 x 128 when there is at most one per CU
+        // (measured at K = 4096: M = 4096 100 -> 93.5 us, M = 1024 52.5 -> 46.6, but M = 2048, two
+        // 128 x 128 tiles per CU, 59 -> 64; every 64 x 64 case loses).
+        const bool two = K >= 2048;
+        if (N > 128 && wgs(128, 256) >= 384)
+            return two ? launch_tile_dma<8, 4, 1, 4, 2>(ld, native, M, K, N, ep, stream)
+                       : launch_tile_dma<8, 4, 1, 4, 1>(ld, native, M, K, N, ep, stream);
+        if (N > 64 && wgs(128, 128) >= 256)
+            return two && wgs(128, 128) <= 256 ? launch_tile_dma<4, 4, 2, 2, 2>(ld, native, M, K, N, ep, stream)
+                                               : launch_tile_dma<4, 4, 2, 2, 1>(ld, native, M, K, N, ep, stream);
+        return launch_tile_dma<2, 4, 2, 1, 1>(ld, native, M, K, N, ep, stream);
     } else {
         // Register prefetch depth: the big tile has a k-tile of work long enough to cover a trip to L2
         // (and no registers to spare); the smaller ones fetch two tiles ahead once the reduction is
