@@ -97,6 +97,9 @@ MID = [  # batches between the skinny kernel and the big-tile kernel, both activ
     (65, 4096, 4096, False), (256, 4096, 4096, False), (256, 4096, 4096, True), (128, 4096, 4096, False),
     (100, 1000, 4100, False), (777, 2304, 520, False), (300, 4096, 96, True), (1024, 1024, 1024, False),
     (2048, 512, 4096, False), (96, 8192, 2048, True), (65, 264, 40, False), (513, 4096, 1000, True),
+    # the big-tile kernel at the full benchmark shape and around its tile-choice boundaries
+    (4096, 4096, 4096, False), (1024, 4096, 4096, False), (2048, 4096, 4096, False), (3000, 2112, 1000, False),
+    (40, 512, 102, False), (64, 512, 102, True), (33, 256, 4096, False),
 ]
 
 
