@@ -286,9 +286,12 @@ def bench_resnet_infer(args, torch):
     fused = FusedTernaryResNet18(model)
     out = {}
     for name, fn, reps in (("fused", lambda: fused(x), args.steps), ("drop_in", lambda: model(x), max(3, args.steps // 4)),
-                           ("drop_in_bn_folded", lambda: model(x), max(3, args.steps // 4))):
+                           ("drop_in_bn_folded", lambda: model(x), max(3, args.steps // 4)),
+                           ("drop_in_bn_folded_fp16", lambda: model(x), max(3, args.steps // 4))):
         if name == "drop_in_bn_folded":
             t.fold_batchnorm(model)                           # BatchNorm into the convolutions' epilogues
+        if name == "drop_in_bn_folded_fp16":
+            t.set_compact_output_dtype(torch.float16)         # fp16 channels_last between the layers
         with torch.no_grad():
             for _ in range(max(2, args.warmup // 4)):
                 fn()
@@ -299,6 +302,7 @@ def bench_resnet_infer(args, torch):
             torch.cuda.synchronize()
         dt = (time.perf_counter() - t0) / reps
         out[name] = {"ms": round(dt * 1e3, 4), "img_s": round(B / dt, 1), "tflops": round(3.627e9 * B / dt / 1e12, 2)}
+    t.set_compact_output_dtype(torch.float32)
     return {"metric": "ResNet-18 img/s", "value": out["fused"]["img_s"], "unit": "img/s", "n_gpus": 1, "dtype": "f16",
             "data": "synthetic", "config": {"workload": "configs[3]: ResNet-18/102 ternary inference", "batch": B},
             "modes": out}

@@ -74,4 +74,13 @@ def test_fold_resnet_and_explicit_pairs(cuda):
         assert len(done) == 19 and ("layer2.0.downsample.0", "layer2.0.downsample.1") in done
         assert not any(isinstance(m, torch.nn.BatchNorm2d) for m in model.modules())
         got = model(x)
+        # fp16 between the layers: same network within fp16 rounding of the activations
+        prev = t.set_compact_output_dtype(torch.float16)
+        try:
+            got16 = model(x)
+        finally:
+            t.set_compact_output_dtype(prev)
     assert torch.allclose(got, want, rtol=5e-3, atol=5e-3 * want.abs().max().item())
+    assert got16.dtype == torch.float16 and torch.allclose(got16.float(), want, rtol=3e-2, atol=3e-2 * want.abs().max().item())
+    with pytest.raises(ValueError):
+        t.set_compact_output_dtype(torch.bfloat16)
