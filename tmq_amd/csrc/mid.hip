@@ -319,12 +319,23 @@ int launch(const Rows &rows, const void *native, int64_t M, int64_t K, int64_t N
     return check_launch();
 }
 
-// Geometry: 64 x 64 tiles once they give a workgroup per CU, else 32 x 64; then as many wavefronts
-// per tile as it takes to put about ten on every CU, each with at least two pairs to multiply.
+// Geometry: 64 x 128 tiles where they save a pass over the CUs (below); else 64 x 64 tiles once they
+// give a workgroup per CU, else 32 x 64; then as many wavefronts per tile as it takes to put about
+// ten on every CU, each with at least two pairs to multiply.
 template <class Rows>
 int dispatch(const Rows &rows, const void *native, int64_t M, int64_t K, int64_t N, const MidEpilogue &ep,
              void *stream) {
     const int64_t npairs = (K + 63) / 64, tn = (N + 63) / 64;
+    // 64 x 128 tiles with four wavefronts read each activation row half as often (the weights are
+    // 2 bits, so a wide tile is the cheap direction) but a pass over them takes ~1.7 times as long as
+    // one over 64 x 64 tiles with eight wavefronts; both run one workgroup per CU. They win when they
+    // save a whole pass: M = 512 at K = N = 4096 27.5 -> 23.9 us, the 512-channel 7 x 7 convolutions
+    // of ResNet-18 33 -> 29.6 us; with a single pass of 64 x 64 tiles (M = 256) they lose.
+    {
+        const int64_t tm = (M + 63) / 64, passes64 = (tm * tn + 255) / 256, passes128 = (tm * ((N + 127) / 128) + 255) / 256;
+        if (npairs >= 16 && passes64 >= 2 && 17 * passes128 < 10 * passes64)
+            return launch<4, 8, 4, Rows>(rows, native, M, K, N, ep, stream);
+    }
     const bool big = ((M + 63) / 64) * tn >= 256;
     const int64_t tiles = ((M + (big ? 63 : 31)) / (big ? 64 : 32)) * tn;
     int waves = 1;
