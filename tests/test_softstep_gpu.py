@@ -252,3 +252,42 @@ def test_full_size_properties(cuda, oracle):
     assert_same(y[idx.to(cuda)], oy, "sample y")
     assert_same(dw[idx.to(cuda)], odw, "sample dw")
     assert_same(wc[idx.to(cuda)], owc, "sample clamp")
+
+
+@pytest.mark.parametrize("d", HARDNESS)
+def test_ternarize_over_every_float_in_range(cuda, oracle, d):
+    """Every fp32 value in [-1.02, 1.02] (2 x 1 065 520 989 bit patterns, both zeros included): ternarising
+    through the soft staircase (tmq/tmq.py:284-295 with map, 328-338) is expected to equal plain
+    round-half-even of the weight -- map is monotone and fixes k and k + 1/2 -- but the reference computes
+    it through map's own fp32 op order. Wherever the two differ in value, the kernel must agree with
+    the CPU restatement of that op order bit for bit; the test reports how often that happens, and how
+    often only the sign of a zero differs (map's arithmetic does not keep it)."""
+    from tmq_amd import ops
+    top = int(np.float32(1.02).view(np.uint32))                 # 0x3F828F5C
+    chunk = 1 << 26
+    differ = signs = 0
+    for base in range(0, top + 1, chunk):
+        n = min(chunk, top + 1 - base)
+        bits = torch.arange(base, base + n, dtype=torch.int64, device=cuda).to(torch.int32)
+        for sign in (0, -(1 << 31)):
+            w = (bits | sign).view(torch.float32) if sign else bits.view(torch.float32)
+            t = w.clone()
+            ops.ternarize_(t, d)
+            r = torch.round(w)
+            bad = (t != r).nonzero().flatten()                       # by value: -0.0 == +0.0
+            signs += int((t.view(torch.int32) != r.view(torch.int32)).sum().item()) - bad.numel()
+            if bad.numel():
+                differ += bad.numel()
+                sel = bad[:100000]
+                wm = w[sel].cpu().numpy()
+                assert np.array_equal(t[sel].cpu().numpy().view(np.uint32), oracle.ternarize(wm, d).view(np.uint32))
+    # a sample of the whole range against the oracle as well (the mismatch set may be empty)
+    g = torch.Generator(device=cuda).manual_seed(int(d * 1000))
+    sample = torch.randint(0, top + 1, (1 << 20,), device=cuda, generator=g, dtype=torch.int64).to(torch.int32)
+    sample[::2] |= -(1 << 31)
+    ws = sample.view(torch.float32)
+    ts = ws.clone()
+    ops.ternarize_(ts, d)
+    assert np.array_equal(ts.cpu().numpy().view(np.uint32), oracle.ternarize(ws.cpu().numpy(), d).view(np.uint32))
+    print(f"hardness {d}: ternarise differs from round-half-even in value on {differ} of {2 * (top + 1)} inputs "
+          f"and only in the sign of a zero on {signs}")
