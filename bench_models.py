@@ -83,25 +83,17 @@ class FusedTernaryResNet18:
                    model.fc.bias.data.float() if model.fc.bias is not None else None)
 
     def _stem(self, conv, bn):
-        """The 7x7 / stride 2 / pad 3 stem on 3 channels as a 7x4 / stride (2, 1) convolution on
-        "super-pixels": the image is stored NHWC with 4 channels (3 + one zero), and two neighbouring
-        pixels are read as one pixel of 8 channels. Output column ow reads pixels 2 ow - 3 .. 2 ow + 3,
-        i.e. super-pixels ow - 2 .. ow + 1 (8 pixels; the extra one, 2 ow - 4, gets zero weights), so
-        the reduction is 7 x 4 x 8 = 224 long instead of 7 x 7 x 8 = 392 with channels padded to 8."""
-        ops = self.ops
-        N, C, ky, kx = (int(v) for v in conv.original_shape)
+        """The 7x7 / stride 2 / pad 3 stem on 3 channels as the layer's own super-pixel rewrite
+        (tmq_amd.Conv2d._superpixel_plan): a 7x4 / stride (2, 1) convolution over pairs of RGB0 pixels
+        read as one pixel of 8 channels; the reduction is 7 x 4 x 8 = 224 long."""
+        probe = torch.empty((1, 3, 224, 224), dtype=torch.float16, device=self.dev)
+        plan = conv._superpixel_plan(probe)
+        assert plan is not None, "the stem does not qualify for the super-pixel rewrite"
+        nw, kxs, pl, pr = plan
         pair = lambda v: tuple(v) if isinstance(v, (tuple, list)) else (v, v)
-        assert (C, ky, kx) == (3, 7, 7) and pair(conv.stride) == (2, 2) and pair(conv.padding) == (3, 3)
-        w = ops.expand_ternary(conv.weight.data, [N, C, ky, kx])
-        wp = torch.zeros(N, 8, ky, 4, device=w.device)
-        for q in range(4):
-            for par in range(2):
-                k = 2 * q + par - 1
-                if 0 <= k < kx:
-                    wp[:, par * 4:par * 4 + C, :, q] = w[:, :, :, k]
-        nw = ops.NativeWeights(ops.compactify_ternary(wp), N, conv_kernel=(ky, 4))
+        (sy, _), (py, _) = pair(conv.stride), pair(conv.padding)
         inv = (bn.running_var + bn.eps).rsqrt() * bn.weight
-        return nw, inv.float().contiguous(), (bn.bias - bn.running_mean * inv).float().contiguous(), (2, 1), ((3, 3), (2, 1))
+        return nw, inv.float().contiguous(), (bn.bias - bn.running_mean * inv).float().contiguous(), (sy, 1), ((py, py), (pl, pr))
 
     def _conv(self, conv, bn):
         ops = self.ops
