@@ -500,11 +500,14 @@ __global__ __launch_bounds__(64 * WGM * WGN, 2) void tile_dma_kernel(Loader ld, 
     }
     const int KT = (int)((K + kBK - 1) / kBK);
 
-    uint32_t wcur[P][WN], wnext[P][WN];
-    auto wload = [&](uint32_t (&w)[WN], int kn) {
-        if (kn >= KT) kn = KT - 1;
+    // Weights: a lane's dwords of a whole native block (4 k-tiles) per n-fragment in one 16-byte load,
+    // fetched one block ahead -- one vector-memory instruction per k-tile instead of WN.
+    const int KB = (KT + 3) >> 2;
+    u32x4 wblk[WN], wnext[WN];
+    auto wload = [&](u32x4 (&w)[WN], int kb) {
+        if (kb >= KB) kb = KB - 1;
 #pragma unroll
-        for (int j = 0; j < WN; j++) w[j] = wptr[j][(int64_t)(kn >> 2) * 256 + (kn & 3)];
+        for (int j = 0; j < WN; j++) w[j] = *reinterpret_cast<const u32x4 *>(wptr[j] + (int64_t)kb * 256);
     };
     // tile `kn` -> ring buffer `slot`; the loader's state moves on to the next tile (tiles past K, which
     // the last pass prefetches and nobody multiplies, read whatever the loader substitutes)
@@ -516,7 +519,10 @@ __global__ __launch_bounds__(64 * WGM * WGN, 2) void tile_dma_kernel(Loader ld, 
         ld.template advance<CH, T>(st);
     };
 
-    // per-column epilogue constants first (conditional loads: keep them out of the main loop)
+    // the first tiles are requested before anything else waits on memory
+#pragma unroll
+    for (int i = 0; i < P; i++) fill(i, i);
+    wload(wblk, 0);
     const int64_t nw0 = n0 + (int64_t)wn * WN * 16;
     float sc[WN], bi[WN];
 #pragma unroll
@@ -525,12 +531,6 @@ __global__ __launch_bounds__(64 * WGM * WGN, 2) void tile_dma_kernel(Loader ld, 
         sc[j] = (n < N && ep.scale ? ep.scale[n] : 1.0f) * (1.0f / kWeightUnit);
         bi[j] = (n < N && ep.bias) ? ep.bias[n] : 0.0f;
     }
-#pragma unroll
-    for (int i = 0; i < P; i++) wload(wcur[i], i);
-    __builtin_amdgcn_s_waitcnt(0x0F70);            // vmcnt(0): a clean state for the compiler's own counting
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int i = 0; i < P; i++) fill(i, i);
     __builtin_amdgcn_sched_barrier(0);
 
     const int arow = (wm * WM * 16 + r16) * kPitch;
@@ -559,23 +559,33 @@ __global__ __launch_bounds__(64 * WGM * WGN, 2) void tile_dma_kernel(Loader ld, 
     };
 
     int half = 0;                                    // which half of the ring is being multiplied
-    for (int kt = 0; kt < KT; kt += P) {
-        __builtin_amdgcn_s_waitcnt(0x0F70);         // this thread's part of tiles kt .. kt + P - 1 is in LDS
-        __syncthreads();                             // ... and everybody's; the other half of the ring is free
-        __builtin_amdgcn_sched_barrier(0);
+    for (int kb = 0; kb < KB; kb++) {
 #pragma unroll
-        for (int i = 0; i < P; i++) fill(kt + P + i, (half ^ 1) * P + i);
+        for (int q = 0; q < 4; q += P) {             // the passes over this block's k-tiles
+            const int kt = kb * 4 + q;
+            if (kt < KT) {
+                __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this thread's part of tiles kt .. kt + P - 1 is in LDS
+                __syncthreads();                      // ... and everybody's; the other half of the ring is free
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int i = 0; i < P; i++) wload(wnext[i], kt + P + i);
-        __builtin_amdgcn_sched_barrier(0);
+                for (int i = 0; i < P; i++) fill(kt + P + i, (half ^ 1) * P + i);
+                if (q == 0) wload(wnext, kb + 1);
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int i = 0; i < P; i++)
-            if (i == 0 || kt + i < KT) multiply(half * P + i, wcur[i]);
+                for (int i = 0; i < P; i++)
+                    if (i == 0 || kt + i < KT) {
+                        uint32_t w[WN];
 #pragma unroll
-        for (int i = 0; i < P; i++)
+                        for (int j = 0; j < WN; j++) w[j] = wblk[j][q + i];
+                        multiply(half * P + i, w);
+                    }
+                half ^= 1;
+            }
+        }
 #pragma unroll
-            for (int j = 0; j < WN; j++) asm volatile("v_mov_b32 %0, %1" : "=v"(wcur[i][j]) : "v"(wnext[i][j]));
-        half ^= 1;
+        for (int j = 0; j < WN; j++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) asm volatile("v_mov_b32 %0, %1" : "=v"(wblk[j][e]) : "v"(wnext[j][e]));
     }
     // drain the prefetches past K before the buffers are reused as transpose slabs
     __builtin_amdgcn_s_waitcnt(0x0F70);
