@@ -23,6 +23,20 @@ inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 
 constexpr int kWave = 64;
 
 #if defined(__HIPCC__)
+// a / b and a % b for 0 <= a, 0 < b. The GPU has no integer divider: a 64-bit division expands to
+// ~100 instructions, a 32-bit one to ~20, and index arithmetic (pixel -> batch, row, column) sits in
+// the prologue of every workgroup -- so take the 32-bit route whenever the dividend fits.
+__device__ __forceinline__ int64_t div_rem(int64_t a, int b, int &rem) {
+    if (a < ((int64_t)1 << 32)) {
+        const uint32_t q = (uint32_t)a / (uint32_t)b;
+        rem = (int)((uint32_t)a - q * (uint32_t)b);
+        return q;
+    }
+    const int64_t q = a / b;
+    rem = (int)(a - q * b);
+    return q;
+}
+
 // Sum over the 64 lanes of a wavefront with DPP row operations (no LDS traffic): butterfly
 // inside each row of 16 lanes, then the four row sums are fetched with v_readlane.
 __device__ __forceinline__ float wave_sum(float v) {

@@ -90,10 +90,10 @@ __global__ __launch_bounds__(256) void dwconv_image_kernel(const _Float16 *__res
     const int64_t G = (C + 7) / 8, Q = (C + 15) / 16;
     const int64_t id = (int64_t)blockIdx.x * 256 + threadIdx.x, total = (int64_t)B * Ho * Wo * G;
     if (id >= total) return;
-    const int64_t p = id / G, c0 = (id - p * G) * 8;
-    const int ow = (int)(p % Wo);
-    const int64_t r = p / Wo;
-    const int oh = (int)(r % Ho), b = (int)(r / Ho);
+    int cg, ow, oh;
+    const int64_t p = div_rem(id, (int)G, cg), c0 = (int64_t)cg * 8;
+    const int64_t r = div_rem(p, Wo, ow);
+    const int b = (int)div_rem(r, Ho, oh);
     float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     for (int i = 0; i < ky; i++) {
         const int ih = oh * sy - py + i * dy;
@@ -124,7 +124,8 @@ __global__ __launch_bounds__(256) void dwconv_patches_kernel(const T *__restrict
     const int64_t G = (C + 7) / 8, Q = (C + 15) / 16;
     const int64_t id = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (id >= P * G) return;
-    const int64_t p = id / G, c0 = (id - p * G) * 8;
+    int cg;
+    const int64_t p = div_rem(id, (int)G, cg), c0 = (int64_t)cg * 8;
     float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     for (int t = 0; t < taps; t++) {
         const T *src = x + (p * taps + t) * C + c0;
@@ -159,10 +160,10 @@ __global__ __launch_bounds__(256) void dwconvtrans_image_kernel(const _Float16 *
     const int64_t G = (C + 7) / 8, Q = (C + 15) / 16;
     const int64_t id = (int64_t)blockIdx.x * 256 + threadIdx.x, total = (int64_t)B * Ho * Wo * G;
     if (id >= total) return;
-    const int64_t p = id / G, c0 = (id - p * G) * 8;
-    const int ow = (int)(p % Wo);
-    const int64_t r = p / Wo;
-    const int oh = (int)(r % Ho), b = (int)(r / Ho);
+    int cg, ow, oh;
+    const int64_t p = div_rem(id, (int)G, cg), c0 = (int64_t)cg * 8;
+    const int64_t r = div_rem(p, Wo, ow);
+    const int b = (int)div_rem(r, Ho, oh);
     float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     for (int i = 0; i < ky; i++) {
         const int ny = oh + py - i * dy;

@@ -144,10 +144,9 @@ struct ConvLoader {
         for (int q = 0; q < CH; q++) {
             const int64_t m = m0 + (tid >> 3) + q * (T / 8);
             if (m < M) {
-                const int ow = (int)(m % Wo);
-                const int64_t t = m / Wo;
-                const int oh = (int)(t % Ho);
-                const int64_t b = t / Ho;
+                int ow, oh;
+                const int64_t t = div_rem(m, Wo, ow);
+                const int64_t b = div_rem(t, Ho, oh);
                 st.img[q] = x + b * (int64_t)H * W * C;
                 st.ih0[q] = oh * sy - py;
                 st.iw0[q] = ow * sx - px;
@@ -223,9 +222,9 @@ struct ConvLoader64 {
             st.off0[q] = 0;
             st.ih0[q] = st.iw0[q] = INT32_MIN / 2;
             if (m < M) {
-                const int ow = (int)(m % Wo);
-                const int64_t t = m / Wo;
-                const int oh = (int)(t % Ho), b = (int)(t / Ho);
+                int ow, oh;
+                const int64_t t = div_rem(m, Wo, ow);
+                const int b = (int)div_rem(t, Ho, oh);
                 st.ih0[q] = oh * sy - py;
                 st.iw0[q] = ow * sx - px;
                 st.off0[q] = ((b * H + st.ih0[q]) * W + st.iw0[q]) * C + kc;
@@ -276,9 +275,9 @@ struct ConvLoaderFewC {
             st.off0[q] = 0;
             st.ih0[q] = st.iw0[q] = INT32_MIN / 2;
             if (m < M) {
-                const int ow = (int)(m % Wo);
-                const int64_t t = m / Wo;
-                const int oh = (int)(t % Ho), b = (int)(t / Ho);
+                int ow, oh;
+                const int64_t t = div_rem(m, Wo, ow);
+                const int b = (int)div_rem(t, Ho, oh);
                 st.ih0[q] = oh * sy - py;
                 st.iw0[q] = ow * sx - px;
                 st.off0[q] = ((b * H + st.ih0[q]) * W + st.iw0[q]) * C + kc % C;

@@ -92,9 +92,9 @@ struct ConvRows {
                 const int R = c * 8 + (lane >> 3);
                 int64_t m = m0 + mi * 16 + R;
                 if (m >= M) m = M - 1;
-                const int ow = (int)(m % Wo);
-                const int64_t t = m / Wo;
-                const int oh = (int)(t % Ho), b = (int)(t / Ho);
+                int ow, oh;
+                const int64_t t = div_rem(m, Wo, ow);
+                const int b = (int)div_rem(t, Ho, oh);
                 st.ih0[mi][c] = oh * sy - py;
                 st.iw0[mi][c] = ow * sx - px;
                 st.off[mi][c] = ((b * H + st.ih0[mi][c]) * W + st.iw0[mi][c]) * C + (((lane & 7) ^ ((R >> 1) & 7)) * 8);

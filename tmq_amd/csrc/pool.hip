@@ -19,10 +19,10 @@ __global__ __launch_bounds__(256) void maxpool_nhwc_kernel(const _Float16 *__res
     const int64_t G = (C + 7) / 8;
     const int64_t id = (int64_t)blockIdx.x * 256 + threadIdx.x, total = (int64_t)B * Ho * Wo * G;
     if (id >= total) return;
-    const int64_t p = id / G, c0 = (id - p * G) * 8;
-    const int ow = (int)(p % Wo);
-    const int64_t r = p / Wo;
-    const int oh = (int)(r % Ho), b = (int)(r / Ho);
+    int cg, ow, oh;
+    const int64_t p = div_rem(id, (int)G, cg), c0 = (int64_t)cg * 8;
+    const int64_t r = div_rem(p, Wo, ow);
+    const int b = (int)div_rem(r, Ho, oh);
     const _Float16 ninf = (_Float16)(-__builtin_inff());
     half8 best = {ninf, ninf, ninf, ninf, ninf, ninf, ninf, ninf};
     for (int i = 0; i < ky; i++) {
@@ -60,7 +60,7 @@ __global__ __launch_bounds__(256) void avgpool_global_nhwc_kernel(const _Float16
                                                                   int vec, void *__restrict__ y, int y_f16) {
     __shared__ float part[4][64][9];
     const int64_t G = (C + 7) / 8, GB = (G + 63) / 64;
-    const int64_t b = blockIdx.x / GB, cg = (blockIdx.x % GB) * 64 + (threadIdx.x & 63);
+    const int64_t b = (uint32_t)blockIdx.x / (uint32_t)GB, cg = (int64_t)((uint32_t)blockIdx.x % (uint32_t)GB) * 64 + (threadIdx.x & 63);
     const int lane = threadIdx.x & 63, slice = threadIdx.x >> 6;
     const int64_t c0 = cg * 8;
     float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
@@ -111,7 +111,9 @@ __global__ __launch_bounds__(256) void nchw_to_nhwc4_kernel(const T *__restrict_
     const int64_t W4 = W / 4;
     const int64_t id = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (id >= B * H * W4) return;
-    const int64_t w0 = (id % W4) * 4, bh = id / W4, h = bh % H, b = bh / H;
+    int wq, hh;
+    const int64_t bh = div_rem(id, (int)W4, wq), w0 = (int64_t)wq * 4;
+    const int64_t b = div_rem(bh, (int)H, hh), h = hh;
     _Float16 px[4][4];
 #pragma unroll
     for (int c = 0; c < 4; c++) {
@@ -172,6 +174,7 @@ int tmq_avgpool_global_nhwc(const void *x, int64_t B, int64_t HW, int64_t C, voi
 int tmq_nchw_to_nhwc4(const void *x, int x_dtype, int64_t B, int32_t C, int64_t H, int64_t W, void *y, void *stream) {
     if (B < 0 || C <= 0 || C > 4 || H <= 0 || W <= 0 || W % 4 != 0) return TMQ_ERR_INVALID_ARG;
     if (x_dtype != TMQ_F16 && x_dtype != TMQ_F32) return TMQ_ERR_UNSUPPORTED;
+    if (H > 0x7FFFFFFF || W > 0x7FFFFFFF) return TMQ_ERR_TOO_LARGE;
     if (B == 0) return TMQ_OK;
     if (!x || !y || !aligned16(y)) return TMQ_ERR_INVALID_ARG;
     const int64_t total = B * H * (W / 4), blocks = (total + 255) / 256;
