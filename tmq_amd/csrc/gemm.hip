@@ -368,13 +368,8 @@ __global__ __launch_bounds__(64 * WGM * WGN, 2) void tile_kernel(Loader ld, cons
 
     // per-column epilogue constants, fetched now so their latency hides behind the main loop
     const int64_t nw0 = n0 + (int64_t)wn * WN * 16;        // first column of this wave
-    float sc[WN], bi[WN];
-#pragma unroll
-    for (int j = 0; j < WN; j++) {
-        const int64_t n = nw0 + j * 16 + r16;
-        sc[j] = (n < N && ep.scale ? ep.scale[n] : 1.0f) * (1.0f / kWeightUnit);
-        bi[j] = (n < N && ep.bias) ? ep.bias[n] : 0.0f;
-    }
+    floatx4 sc, bi;
+    load_scale_bias<WN>(ep, lane, nw0, N, sc, bi);
 
     const int arow = (wm * WM * 16 + r16) * kPitch;
     // operand read of m-fragment i, k-step s: chunk (4 s + g) of row (.. + 16 i + r16); 16 i keeps row & 7
@@ -523,13 +518,8 @@ __global__ __launch_bounds__(64 * WGM * WGN, 2) void tile_dma_kernel(Loader ld, 
     for (int i = 0; i < P; i++) fill(i, i);
     wload(wblk, 0);
     const int64_t nw0 = n0 + (int64_t)wn * WN * 16;
-    float sc[WN], bi[WN];
-#pragma unroll
-    for (int j = 0; j < WN; j++) {
-        const int64_t n = nw0 + j * 16 + r16;
-        sc[j] = (n < N && ep.scale ? ep.scale[n] : 1.0f) * (1.0f / kWeightUnit);
-        bi[j] = (n < N && ep.bias) ? ep.bias[n] : 0.0f;
-    }
+    floatx4 sc, bi;
+    load_scale_bias<WN>(ep, lane, nw0, N, sc, bi);
     __builtin_amdgcn_sched_barrier(0);
 
     const int arow = (wm * WM * 16 + r16) * kPitch;

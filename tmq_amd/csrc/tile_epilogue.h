@@ -17,14 +17,39 @@ struct Epilogue {
 
 #if defined(__HIPCC__)
 
+// Per-column scale (the weight unit folded in) and bias of the four consecutive columns a lane writes in
+// write_tile: lane -> columns nw0 + 4 (lane % (4 WN)) .. + 3. Two 16-byte loads where the vectors allow
+// it -- a load instruction costs the CU's address unit the same 16 cycles for 4 or for 16 bytes per lane.
+template <int WN>
+__device__ __forceinline__ void load_scale_bias(const Epilogue &ep, int lane, int64_t nw0, int64_t N, floatx4 &sc, floatx4 &bi) {
+    const int64_t n = nw0 + (lane % (4 * WN)) * 4;
+    sc = floatx4{1.f, 1.f, 1.f, 1.f};
+    bi = floatx4{0.f, 0.f, 0.f, 0.f};
+    const bool vec = (N % 4 == 0) && ((reinterpret_cast<uintptr_t>(ep.scale) | reinterpret_cast<uintptr_t>(ep.bias)) & 15u) == 0;
+    if (vec) {
+        if (n < N) {
+            if (ep.scale) sc = *reinterpret_cast<const floatx4 *>(ep.scale + n);
+            if (ep.bias) bi = *reinterpret_cast<const floatx4 *>(ep.bias + n);
+        }
+    } else {
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+            if (n + e < N) {
+                if (ep.scale) sc[e] = ep.scale[n + e];
+                if (ep.bias) bi[e] = ep.bias[n + e];
+            }
+    }
+    sc *= 1.0f / kWeightUnit;
+}
+
 // Epilogue of one wavefront's (16 WM) x (16 WN) accumulator block. A lane holds rows 4g + r, column
 // r16 of each 16 x 16 accumulator -- 64-byte row pieces if stored directly. Instead the wavefront
 // transposes one 16-row slab (16 x 16 WN values) at a time through its own slice of LDS (`slab`, the
 // idle activation buffer) and writes whole rows: 16 lanes x 16 bytes = 256 contiguous bytes per row and
-// store instruction. sc / bi: per-column scale (weight unit folded in) and bias of column r16 of fragment j.
+// store instruction. sc / bi: scale and bias of the lane's four columns (load_scale_bias).
 template <int WM, int WN>
-__device__ __forceinline__ void write_tile(float *slab, const floatx4 (&acc)[WM][WN], const float (&sc)[WN],
-                                           const float (&bi)[WN], int lane, int64_t mw0, int64_t nw0, int64_t M,
+__device__ __forceinline__ void write_tile(float *slab, const floatx4 (&acc)[WM][WN], const floatx4 &sc,
+                                           const floatx4 &bi, int lane, int64_t mw0, int64_t nw0, int64_t M,
                                            int64_t N, const Epilogue &ep) {
     constexpr int kEP = 16 * WN + 4;                       // slab row pitch in floats (+4: conflict-free)
     const int r16 = lane & 15, g = lane >> 4;
@@ -34,14 +59,14 @@ __device__ __forceinline__ void write_tile(float *slab, const floatx4 (&acc)[WM]
 #pragma unroll
         for (int j = 0; j < WN; j++)
 #pragma unroll
-            for (int r = 0; r < 4; r++) slab[(g * 4 + r) * kEP + j * 16 + r16] = acc[i][j][r] * sc[j] + bi[j];
+            for (int r = 0; r < 4; r++) slab[(g * 4 + r) * kEP + j * 16 + r16] = acc[i][j][r];
         __builtin_amdgcn_wave_barrier();
         const int64_t mrow0 = mw0 + (int64_t)i * 16;
 #pragma unroll
         for (int t = 0; t < WN; t++) {                     // 16 rows x (16 WN / 4) float4 = 64 WN float4 per slab
             const int idx = t * 64 + lane, row = idx / (4 * WN), c4 = idx % (4 * WN);
             const int64_t m = mrow0 + row, n = nw0 + c4 * 4;
-            floatx4 v = *reinterpret_cast<const floatx4 *>(&slab[row * kEP + c4 * 4]);
+            floatx4 v = *reinterpret_cast<const floatx4 *>(&slab[row * kEP + c4 * 4]) * sc + bi;
             if (m >= M || n >= N) continue;
             const int64_t o = m * N + n;
             if (vec) {
