@@ -368,8 +368,8 @@ __global__ __launch_bounds__(64 * WGM * WGN, 2) void tile_kernel(Loader ld, cons
 
     // per-column epilogue constants, fetched now so their latency hides behind the main loop
     const int64_t nw0 = n0 + (int64_t)wn * WN * 16;        // first column of this wave
-    floatx4 sc, bi;
-    load_scale_bias<WN>(ep, lane, nw0, N, sc, bi);
+    ColumnConstants cc;
+    load_scale_bias<WN>(ep, lane, nw0, N, cc);
 
     const int arow = (wm * WM * 16 + r16) * kPitch;
     // operand read of m-fragment i, k-step s: chunk (4 s + g) of row (.. + 16 i + r16); 16 i keeps row & 7
@@ -435,7 +435,7 @@ __global__ __launch_bounds__(64 * WGM * WGN, 2) void tile_kernel(Loader ld, cons
     // the k-loop is over: its LDS buffers become the epilogue's transpose slabs
     constexpr int kEP = 16 * WN + 4;
     static_assert(WGM * WGN * 16 * kEP * 4 <= 2 * BM * kPitch * 2, "epilogue slab does not fit the LDS buffer");
-    write_tile<WM, WN>(reinterpret_cast<float *>(&As[0][0]) + wv * 16 * kEP, acc, sc, bi, lane, m0 + (int64_t)wm * WM * 16,
+    write_tile<WM, WN>(reinterpret_cast<float *>(&As[0][0]) + wv * 16 * kEP, acc, cc, lane, m0 + (int64_t)wm * WM * 16,
                        nw0, M, N, ep);
 }
 
@@ -518,8 +518,8 @@ __global__ __launch_bounds__(64 * WGM * WGN, 2) void tile_dma_kernel(Loader ld, 
     for (int i = 0; i < P; i++) fill(i, i);
     wload(wblk, 0);
     const int64_t nw0 = n0 + (int64_t)wn * WN * 16;
-    floatx4 sc, bi;
-    load_scale_bias<WN>(ep, lane, nw0, N, sc, bi);
+    ColumnConstants cc;
+    load_scale_bias<WN>(ep, lane, nw0, N, cc);
     __builtin_amdgcn_sched_barrier(0);
 
     const int arow = (wm * WM * 16 + r16) * kPitch;
@@ -582,7 +582,7 @@ __global__ __launch_bounds__(64 * WGM * WGN, 2) void tile_dma_kernel(Loader ld, 
 
     constexpr int kEP = 16 * WN + 4;
     static_assert(WGM * WGN * 16 * kEP * 4 <= S * kTileBytes, "epilogue slab does not fit the LDS buffer");
-    write_tile<WM, WN>(reinterpret_cast<float *>(&As[0][0]) + wv * 16 * kEP, acc, sc, bi, lane, m0 + (int64_t)wm * WM * 16,
+    write_tile<WM, WN>(reinterpret_cast<float *>(&As[0][0]) + wv * 16 * kEP, acc, cc, lane, m0 + (int64_t)wm * WM * 16,
                        nw0, M, N, ep);
 }
 

@@ -17,43 +17,60 @@ struct Epilogue {
 
 #if defined(__HIPCC__)
 
-// Per-column scale (the weight unit folded in) and bias of the four consecutive columns a lane writes in
-// write_tile: lane -> columns nw0 + 4 (lane % (4 WN)) .. + 3. Two 16-byte loads where the vectors allow
-// it -- a load instruction costs the CU's address unit the same 16 cycles for 4 or for 16 bytes per lane.
+// fp16 results whose rows are whole 16-byte pieces are written 8 columns (16 bytes) per lane, everything
+// else 4 columns per lane: a store instruction costs the CU's address unit the same 16 cycles either way.
+__device__ __forceinline__ bool wide_rows(const Epilogue &ep, int64_t N) {
+    return ep.y_f16 && (N % 8 == 0) &&
+           ((reinterpret_cast<uintptr_t>(ep.y) | reinterpret_cast<uintptr_t>(ep.residual)) & 15u) == 0;
+}
+
+// Per-column scale (the weight unit folded in) and bias of the columns a lane writes in write_tile:
+// columns nw0 + 4 (lane % (4 WN)) .. + 3 in sc[0] / bi[0], or, for wide rows, nw0 + 8 (lane % (2 WN)) .. + 7
+// in sc[0..1] / bi[0..1]. 16-byte loads where the vectors allow it.
+struct ColumnConstants {
+    floatx4 sc[2], bi[2];
+};
+
 template <int WN>
-__device__ __forceinline__ void load_scale_bias(const Epilogue &ep, int lane, int64_t nw0, int64_t N, floatx4 &sc, floatx4 &bi) {
-    const int64_t n = nw0 + (lane % (4 * WN)) * 4;
-    sc = floatx4{1.f, 1.f, 1.f, 1.f};
-    bi = floatx4{0.f, 0.f, 0.f, 0.f};
+__device__ __forceinline__ void load_scale_bias(const Epilogue &ep, int lane, int64_t nw0, int64_t N, ColumnConstants &cc) {
+    const bool wide = wide_rows(ep, N);
+    const int64_t n = wide ? nw0 + (lane % (2 * WN)) * 8 : nw0 + (lane % (4 * WN)) * 4;
     const bool vec = (N % 4 == 0) && ((reinterpret_cast<uintptr_t>(ep.scale) | reinterpret_cast<uintptr_t>(ep.bias)) & 15u) == 0;
-    if (vec) {
-        if (n < N) {
-            if (ep.scale) sc = *reinterpret_cast<const floatx4 *>(ep.scale + n);
-            if (ep.bias) bi = *reinterpret_cast<const floatx4 *>(ep.bias + n);
-        }
-    } else {
 #pragma unroll
-        for (int e = 0; e < 4; e++)
-            if (n + e < N) {
-                if (ep.scale) sc[e] = ep.scale[n + e];
-                if (ep.bias) bi[e] = ep.bias[n + e];
+    for (int h = 0; h < 2; h++) {
+        cc.sc[h] = floatx4{1.f, 1.f, 1.f, 1.f};
+        cc.bi[h] = floatx4{0.f, 0.f, 0.f, 0.f};
+        if (h == 1 && !wide) break;
+        const int64_t nh = n + 4 * h;
+        if (vec) {
+            if (nh < N) {
+                if (ep.scale) cc.sc[h] = *reinterpret_cast<const floatx4 *>(ep.scale + nh);
+                if (ep.bias) cc.bi[h] = *reinterpret_cast<const floatx4 *>(ep.bias + nh);
             }
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+                if (nh + e < N) {
+                    if (ep.scale) cc.sc[h][e] = ep.scale[nh + e];
+                    if (ep.bias) cc.bi[h][e] = ep.bias[nh + e];
+                }
+        }
+        cc.sc[h] *= 1.0f / kWeightUnit;
     }
-    sc *= 1.0f / kWeightUnit;
 }
 
 // Epilogue of one wavefront's (16 WM) x (16 WN) accumulator block. A lane holds rows 4g + r, column
 // r16 of each 16 x 16 accumulator -- 64-byte row pieces if stored directly. Instead the wavefront
 // transposes one 16-row slab (16 x 16 WN values) at a time through its own slice of LDS (`slab`, the
-// idle activation buffer) and writes whole rows: 16 lanes x 16 bytes = 256 contiguous bytes per row and
-// store instruction. sc / bi: scale and bias of the lane's four columns (load_scale_bias).
+// idle activation buffer) and writes whole rows, 16 bytes per lane: 4 fp32 or, for wide rows, 8 fp16
+// values. cc: scale and bias of the lane's columns (load_scale_bias).
 template <int WM, int WN>
-__device__ __forceinline__ void write_tile(float *slab, const floatx4 (&acc)[WM][WN], const floatx4 &sc,
-                                           const floatx4 &bi, int lane, int64_t mw0, int64_t nw0, int64_t M,
-                                           int64_t N, const Epilogue &ep) {
+__device__ __forceinline__ void write_tile(float *slab, const floatx4 (&acc)[WM][WN], const ColumnConstants &cc, int lane,
+                                           int64_t mw0, int64_t nw0, int64_t M, int64_t N, const Epilogue &ep) {
     constexpr int kEP = 16 * WN + 4;                       // slab row pitch in floats (+4: conflict-free)
     const int r16 = lane & 15, g = lane >> 4;
     const bool vec = (N % 4 == 0) && ((reinterpret_cast<uintptr_t>(ep.y) | reinterpret_cast<uintptr_t>(ep.residual)) & 15u) == 0;
+    const bool wide = wide_rows(ep, N);
 #pragma unroll
     for (int i = 0; i < WM; i++) {
 #pragma unroll
@@ -62,11 +79,37 @@ __device__ __forceinline__ void write_tile(float *slab, const floatx4 (&acc)[WM]
             for (int r = 0; r < 4; r++) slab[(g * 4 + r) * kEP + j * 16 + r16] = acc[i][j][r];
         __builtin_amdgcn_wave_barrier();
         const int64_t mrow0 = mw0 + (int64_t)i * 16;
+        if (wide) {
+#pragma unroll
+            for (int t = 0; t < (WN + 1) / 2; t++) {           // 16 rows x 2 WN pieces of 8 columns per slab
+                const int idx = t * 64 + lane, row = idx / (2 * WN), c8 = idx % (2 * WN);
+                if (idx >= 32 * WN) continue;
+                const int64_t m = mrow0 + row, n = nw0 + c8 * 8;
+                floatx4 v0 = *reinterpret_cast<const floatx4 *>(&slab[row * kEP + c8 * 8]) * cc.sc[0] + cc.bi[0];
+                floatx4 v1 = *reinterpret_cast<const floatx4 *>(&slab[row * kEP + c8 * 8 + 4]) * cc.sc[1] + cc.bi[1];
+                if (m >= M || n >= N) continue;
+                const int64_t o = m * N + n;
+                if (ep.residual) {
+                    const half8 rs = *reinterpret_cast<const half8 *>(static_cast<const _Float16 *>(ep.residual) + o);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) { v0[e] += (float)rs[e]; v1[e] += (float)rs[4 + e]; }
+                }
+                half8 h;
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    h[e] = (_Float16)((ep.relu && v0[e] < 0.f) ? 0.f : v0[e]);
+                    h[4 + e] = (_Float16)((ep.relu && v1[e] < 0.f) ? 0.f : v1[e]);
+                }
+                *reinterpret_cast<half8 *>(static_cast<_Float16 *>(ep.y) + o) = h;
+            }
+            __builtin_amdgcn_wave_barrier();
+            continue;
+        }
 #pragma unroll
         for (int t = 0; t < WN; t++) {                     // 16 rows x (16 WN / 4) float4 = 64 WN float4 per slab
             const int idx = t * 64 + lane, row = idx / (4 * WN), c4 = idx % (4 * WN);
             const int64_t m = mrow0 + row, n = nw0 + c4 * 4;
-            floatx4 v = *reinterpret_cast<const floatx4 *>(&slab[row * kEP + c4 * 4]) * sc + bi;
+            floatx4 v = *reinterpret_cast<const floatx4 *>(&slab[row * kEP + c4 * 4]) * cc.sc[0] + cc.bi[0];
             if (m >= M || n >= N) continue;
             const int64_t o = m * N + n;
             if (vec) {
