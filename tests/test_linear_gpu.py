@@ -100,6 +100,9 @@ MID = [  # batches between the skinny kernel and the big-tile kernel, both activ
     # the big-tile kernel at the full benchmark shape and around its tile-choice boundaries
     (4096, 4096, 4096, False), (1024, 4096, 4096, False), (2048, 4096, 4096, False), (3000, 2112, 1000, False),
     (40, 512, 102, False), (64, 512, 102, True), (33, 256, 4096, False),
+    # 2 .. 16 rows with whole blocks and at most two per wavefront: private activation windows
+    (3, 256, 70, False), (5, 1024, 1000, False), (15, 4096, 4096, False), (16, 4096, 4096, False), (2, 2048, 8192, False),
+    (4, 8192, 1024, False), (16, 8192, 1024, False), (9, 768, 48, False), (16, 2048, 8192, False),
     # 64 x 128 split-reduction tiles (chosen where they save a pass over the CUs), ragged N included
     (512, 4096, 4096, False), (384, 1024, 4100, False), (256, 8192, 8192, False),
 ]

@@ -390,6 +390,102 @@ __global__ __launch_bounds__(1024) void gemv_short_kernel(const _Float16 *__rest
     }
 }
 
+// ---- short reductions, up to 16 rows -----------------------------------------------------------------
+// The same plan as gemv_short_kernel for 2 <= M <= 16 (one row tile): a wavefront owns one or two weight
+// blocks and fetches, together with them, its own 512-byte slice of every activation row -- two rows per
+// 16-byte-per-lane load -- into a private LDS window. No workgroup-wide staging of all of x and no
+// barrier before the arithmetic: a launch is one trip to memory, the MFMAs, one reduction.
+// Rows of a window are 528 bytes apart (512 + 16) to spread the operand reads of 16 rows over the banks.
+// Requires fp16 activations, K % 256 == 0, 16-byte aligned x, at most two blocks per wavefront.
+constexpr int kShortRowPitch = kKB * 2 + 16;
+
+__global__ __launch_bounds__(1024) void short_rows_kernel(const _Float16 *__restrict__ x, int M, int64_t K,
+                                                          const u32x4 *__restrict__ native, int Kb, int64_t N,
+                                                          const float *__restrict__ scale, const float *__restrict__ bias,
+                                                          const void *__restrict__ residual, int relu, void *__restrict__ y,
+                                                          int y_f16) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    const int lane = threadIdx.x & 63, wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), waves = blockDim.x >> 6;
+    const int j = lane & 15, g = lane >> 4;
+    const int64_t nb = blockIdx.x;
+    const bool two = wv + waves < Kb;
+    const int win_bytes = M * kShortRowPitch;                       // one block's window
+    floatx4 *slot = reinterpret_cast<floatx4 *>(smem);               // [waves][64] partial sums, then the windows
+    unsigned char *win = smem + waves * 64 * sizeof(floatx4) + (size_t)wv * (Kb > waves ? 2 : 1) * win_bytes;
+
+    const u32x4 *wp = native + (nb * Kb + wv) * 64 + lane;
+    u32x4 w0 = __builtin_nontemporal_load(wp), w1 = {0u, 0u, 0u, 0u};
+    if (two) w1 = __builtin_nontemporal_load(wp + (int64_t)waves * 64);
+    // lane -> (row r0 + lane / 32, 16-byte chunk lane % 32) of the slice; rows past M repeat the last one
+    const int lr = lane >> 5, lc = lane & 31;
+    for (int r0 = 0; r0 < M; r0 += 2) {
+        const int r = r0 + lr < M ? r0 + lr : M - 1;
+        const _Float16 *src = x + (int64_t)r * K + (int64_t)wv * kKB + lc * 8;
+        const u32x4 a = *reinterpret_cast<const u32x4 *>(src);
+        u32x4 b = {0u, 0u, 0u, 0u};
+        if (two) b = *reinterpret_cast<const u32x4 *>(src + (int64_t)waves * kKB);
+        *reinterpret_cast<u32x4 *>(win + r * kShortRowPitch + lc * 16) = a;
+        if (two) *reinterpret_cast<u32x4 *>(win + win_bytes + r * kShortRowPitch + lc * 16) = b;
+    }
+    float sc4[4] = {1.f, 1.f, 1.f, 1.f}, bi4[4] = {0.f, 0.f, 0.f, 0.f};
+    if (wv == 0) {
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int64_t n = nb * 16 + g * 4 + r;
+            if (n < N) {
+                if (scale) sc4[r] = scale[n];
+                if (bias) bi4[r] = bias[n];
+            }
+        }
+    }
+    __builtin_amdgcn_wave_barrier();
+    // B operand: lane (j, g) supplies row j (rows past M: the last row, never stored)
+    const unsigned char *xr = win + (j < M ? j : M - 1) * kShortRowPitch + g * 16;
+    floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+    {
+        half8 xv[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) xv[i] = *reinterpret_cast<const half8 *>(xr + i * 64);
+#pragma unroll
+        for (int i = 0; i < 8; i++) acc = mfma16(decode_step(w0[i >> 1], i & 1), xv[i], acc);
+    }
+    if (two) {
+        half8 xv[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) xv[i] = *reinterpret_cast<const half8 *>(xr + win_bytes + i * 64);
+#pragma unroll
+        for (int i = 0; i < 8; i++) acc = mfma16(decode_step(w1[i >> 1], i & 1), xv[i], acc);
+    }
+    // lane (j, g) holds y[m = j][n = 16 nb + 4 g + r], r = 0..3, of this wavefront's share of K
+    slot[wv * 64 + lane] = acc;
+    __syncthreads();
+    if (wv == 0 && j < M) {
+        floatx4 s = slot[lane];
+        for (int w = 1; w < waves; w++) {
+            const floatx4 p = slot[w * 64 + lane];
+            s[0] += p[0]; s[1] += p[1]; s[2] += p[2]; s[3] += p[3];
+        }
+        const int64_t n0 = nb * 16 + g * 4;
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int64_t n = n0 + r;
+            if (n < N) {
+                float v = s[r] * (sc4[r] * (1.0f / kWeightUnit)) + bi4[r];
+                const int64_t o = (int64_t)j * N + n;
+                if (y_f16) {
+                    if (residual) v += (float)static_cast<const _Float16 *>(residual)[o];
+                    if (relu) v = v > 0.f ? v : 0.f;
+                    static_cast<_Float16 *>(y)[o] = (_Float16)v;
+                } else {
+                    if (residual) v += static_cast<const float *>(residual)[o];
+                    if (relu) v = v > 0.f ? v : 0.f;
+                    static_cast<float *>(y)[o] = v;
+                }
+            }
+        }
+    }
+}
+
 struct SkinnyArgs {
     const void *x;
     int64_t M, K;
@@ -432,6 +528,27 @@ int launch_skinny(const void *x, int64_t M, int64_t K, const void *native, int64
             if (Kb <= 2 * waves) {
                 hipLaunchKernelGGL(gemv_short_kernel, dim3((uint32_t)Nb), dim3(64 * waves), 0, as_stream(stream),
                                    static_cast<const _Float16 *>(x), static_cast<const u32x4 *>(native), (int)Kb, N,
+                                   ep.scale, ep.bias, ep.residual, ep.relu, y, ep.y_dtype == TMQ_F16);
+                return check_launch();
+            }
+        }
+    }
+    if constexpr (MT == 1 && !X32) {
+        // 2 .. 16 rows with at most two weight blocks per wavefront: private windows instead of staging all of x
+        // (M = 16 at K = N = 4096: 7.4 -> 5.6 us; M = 2 .. 8: 5.5-5.9 -> 4.3-4.8 us)
+        if (M >= 2 && K % kKB == 0 && Kb <= 32 && aligned16(x) && Nb <= 0x7FFFFFFF) {
+            int waves = Kb > 16 ? 16 : 8;
+            while (waves > Kb) waves >>= 1;
+            const int per_wave = Kb > waves ? 2 : 1;      // windows (weight blocks) per wavefront
+            const size_t lds = (size_t)waves * 64 * sizeof(floatx4) + (size_t)waves * per_wave * M * kShortRowPitch;
+            if (Kb <= 2 * waves && lds <= kSkinnyLdsMax) {
+                if (lds > 64 * 1024) {
+                    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(short_rows_kernel),
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)kSkinnyLdsMax);
+                    if (e != hipSuccess) return note_hip_error(e);
+                }
+                hipLaunchKernelGGL(short_rows_kernel, dim3((uint32_t)Nb), dim3(64 * waves), lds, as_stream(stream),
+                                   static_cast<const _Float16 *>(x), (int)M, K, static_cast<const u32x4 *>(native), (int)Kb, N,
                                    ep.scale, ep.bias, ep.residual, ep.relu, y, ep.y_dtype == TMQ_F16);
                 return check_launch();
             }
