@@ -69,6 +69,11 @@ CONV_CASES = [  # B, C, H, W, N, k, stride, pad, dil
     # channel counts that are multiples of 64 take the uniform-tap loader
     (2, 64, 13, 11, 48, 3, 2, 1, 1), (1, 128, 9, 10, 70, (3, 5), (1, 2), (2, 1), (2, 1)), (3, 192, 6, 6, 64, 1, 1, 0, 1),
     (2, 256, 7, 7, 512, 3, 1, 1, 1), (1, 64, 5, 5, 32, 5, 1, 4, 2), (2, 512, 7, 7, 512, 3, 1, 1, 1),
+    # small batches of ResNet-sized layers: split-reduction kernel with 32 x 32 / 16 x 32 / 32 x 64 tiles
+    (1, 64, 56, 56, 64, 3, 1, 1, 1), (1, 128, 28, 28, 128, 3, 1, 1, 1), (4, 64, 56, 56, 64, 3, 1, 1, 1),
+    (2, 128, 28, 28, 256, 1, 2, 0, 1),
+    # a short reduction with many tiles stays on the tile kernel
+    (8, 64, 40, 40, 128, 1, 1, 0, 1),
 ]
 
 

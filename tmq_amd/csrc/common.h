@@ -22,6 +22,15 @@ inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 
 
 constexpr int kWave = 64;
 
+// Whether a GEMM of M x N outputs over K reduction indices goes to the split-reduction kernels (mid.hip)
+// rather than the big-tile kernel. Measured crossovers: with K >= 512 the split reduction wins or ties up
+// to about 2.5 tiles of 64 x 64 per CU (K = N = 4096: M between 512 and 768); with shorter reductions
+// its per-tile cost shows earlier (K = 256: up to ~128 tiles, K = 128: ~64).
+inline bool split_reduction_pays(int64_t M, int64_t K, int64_t N) {
+    const int64_t tiles64 = ((M + 63) / 64) * ((N + 63) / 64);
+    return K >= 512 ? tiles64 <= 640 : tiles64 <= K / 2;
+}
+
 #if defined(__HIPCC__)
 // a / b and a % b for 0 <= a, 0 < b. The GPU has no integer divider: a 64-bit division expands to
 // ~100 instructions, a 32-bit one to ~20, and index arithmetic (pixel -> batch, row, column) sits in

@@ -690,8 +690,8 @@ int tmq_ternary_conv2d(const void *x, const tmq_conv_shape *s, const void *nativ
     if (M == 0) return TMQ_OK;
     Epilogue ep{scale, bias, residual, y, relu, y_dtype == TMQ_F16 ? 1 : 0};
     const _Float16 *xp = static_cast<const _Float16 *>(x);
-    // few output tiles and a long reduction: split the reduction inside the workgroup (mid.hip)
-    if (mid_conv_ok(x, s) && K >= 2048 && ((M + 63) / 64) * (((int64_t)s->N + 63) / 64) <= 640)
+    // few output tiles: split the reduction inside the workgroup (mid.hip)
+    if (mid_conv_ok(x, s) && split_reduction_pays(M, K, s->N))
         return launch_mid_conv(x, s, ho, wo, native, scale, bias, residual, relu, y, y_dtype == TMQ_F16 ? 1 : 0, stream);
     if ((s->C % kBK == 0) && aligned16(x) &&
         (int64_t)s->B * s->H * s->W * s->C < (int64_t)0x7FFFFFFF)

@@ -1020,7 +1020,7 @@ int mid_rows(const void *x, int64_t M, int64_t K, const void *native, int64_t N,
         if ((K % kKB == 0) && aligned16(x) && (uint64_t)M * (uint64_t)K * 4 < (1ull << 32))
             return launch_mid_lds<2, 4, 8, true>(x, M, K, native, N, ep, y, stream);
     } else {
-        if (K >= 2048 && mid_dense_ok(x, M, K))
+        if (mid_dense_ok(x, M, K))
             return launch_mid_dense(x, M, K, native, N, ep.scale, ep.bias, ep.residual, ep.relu, y,
                                     ep.y_dtype == TMQ_F16, stream);
     }
@@ -1102,10 +1102,9 @@ int tmq_ternary_linear(const void *x, int x_dtype, int64_t M, int64_t K, const v
         return x32 ? skinny_rows<true>(x, M, K, native, N, ep, y, stream)
                    : skinny_rows<false>(x, M, K, native, N, ep, y, stream);
     // fp32 activations always take the mid kernel (two fp16 terms per value keep fp32 accuracy; the
-    // tile kernel is fp16 only). For fp16 the big-tile kernel wins once there are more than about
-    // 2.5 tiles of 64 x 64 per CU (measured crossover at K = N = 4096: M between 512 and 768).
+    // tile kernel is fp16 only).
     if (x32) return mid_rows<true>(x, M, K, native, N, ep, y, stream);
-    if (((M + 63) / 64) * ((N + 63) / 64) <= 640) return mid_rows<false>(x, M, K, native, N, ep, y, stream);
+    if (split_reduction_pays(M, K, N)) return mid_rows<false>(x, M, K, native, N, ep, y, stream);
     return launch_gemm_dense(x, M, K, native, N, ep.scale, ep.bias, ep.residual, ep.relu, y, ep.y_dtype == TMQ_F16,
                              stream);
 }

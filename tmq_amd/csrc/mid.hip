@@ -319,9 +319,9 @@ int launch(const Rows &rows, const void *native, int64_t M, int64_t K, int64_t N
     return check_launch();
 }
 
-// Geometry: 64 x 128 tiles where they save a pass over the CUs (below); else 64 x 64 tiles once they
-// give a workgroup per CU, else 32 x 64; then as many wavefronts per tile as it takes to put about
-// ten on every CU, each with at least two pairs to multiply.
+// Geometry: 64 x 128 tiles where they save a pass over the CUs (below); else the largest smaller tile
+// that keeps most CUs busy; then as many wavefronts per tile as it takes to put about ten on every CU,
+// each with at least two pairs to multiply.
 template <class Rows>
 int dispatch(const Rows &rows, const void *native, int64_t M, int64_t K, int64_t N, const MidEpilogue &ep,
              void *stream) {
@@ -336,24 +336,29 @@ int dispatch(const Rows &rows, const void *native, int64_t M, int64_t K, int64_t
         if (npairs >= 16 && passes64 >= 2 && 17 * passes128 < 10 * passes64)
             return launch<4, 8, 4, Rows>(rows, native, M, K, N, ep, stream);
     }
-    const bool big = ((M + 63) / 64) * tn >= 256;
-    const int64_t tiles = ((M + (big ? 63 : 31)) / (big ? 64 : 32)) * tn;
+    // Otherwise the largest of 64 x 64, 32 x 64, 32 x 32, 16 x 32 that still gives most CUs a tile (measured
+    // at K = N = 4096: M = 64 10.0 -> 7.6 us with 32 x 32, M = 17 9.7 -> 6.4 us with 16 x 32, while
+    // M = 96 .. 128 stay best on 32 x 64).
+    auto tiles = [&](int bm, int bn) { return ((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
+    int bm = 16, bn = 32;
+    if (tiles(64, 64) >= 256) { bm = 64; bn = 64; }
+    else if (tiles(32, 64) >= 192) { bm = 32; bn = 64; }
+    else if (tiles(32, 32) >= 192) { bm = 32; bn = 32; }
     int waves = 1;
-    while (waves < 8 && tiles * waves < 2560 && npairs >= 4 * waves) waves *= 2;
-    if (big) {
+    while (waves < 8 && tiles(bm, bn) * waves < 2560 && npairs >= 4 * waves) waves *= 2;
+    auto go = [&](auto wm_tag, auto wn_tag) {
+        constexpr int WM = decltype(wm_tag)::value, WN = decltype(wn_tag)::value;
         switch (waves) {
-            case 1: return launch<4, 4, 1, Rows>(rows, native, M, K, N, ep, stream);
-            case 2: return launch<4, 4, 2, Rows>(rows, native, M, K, N, ep, stream);
-            case 4: return launch<4, 4, 4, Rows>(rows, native, M, K, N, ep, stream);
-            default: return launch<4, 4, 8, Rows>(rows, native, M, K, N, ep, stream);
+            case 1: return launch<WM, WN, 1, Rows>(rows, native, M, K, N, ep, stream);
+            case 2: return launch<WM, WN, 2, Rows>(rows, native, M, K, N, ep, stream);
+            case 4: return launch<WM, WN, 4, Rows>(rows, native, M, K, N, ep, stream);
+            default: return launch<WM, WN, 8, Rows>(rows, native, M, K, N, ep, stream);
         }
-    }
-    switch (waves) {
-        case 1: return launch<2, 4, 1, Rows>(rows, native, M, K, N, ep, stream);
-        case 2: return launch<2, 4, 2, Rows>(rows, native, M, K, N, ep, stream);
-        case 4: return launch<2, 4, 4, Rows>(rows, native, M, K, N, ep, stream);
-        default: return launch<2, 4, 8, Rows>(rows, native, M, K, N, ep, stream);
-    }
+    };
+    if (bm == 64) return go(std::integral_constant<int, 4>{}, std::integral_constant<int, 4>{});
+    if (bn == 64) return go(std::integral_constant<int, 2>{}, std::integral_constant<int, 4>{});
+    if (bm == 32) return go(std::integral_constant<int, 2>{}, std::integral_constant<int, 2>{});
+    return go(std::integral_constant<int, 1>{}, std::integral_constant<int, 2>{});
 }
 
 }  // namespace
