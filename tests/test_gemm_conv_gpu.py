@@ -18,7 +18,9 @@ def _rel_err(got, want):
 
 
 GEMM_SHAPES = [(65, 64, 16), (128, 512, 64), (256, 4096, 256), (300, 147, 64), (1000, 576, 128), (513, 1000, 130),
-               (4096, 512, 512), (777, 2304, 256), (3136, 256, 102), (2048, 64, 64)]
+               (4096, 512, 512), (777, 2304, 256), (3136, 256, 102), (2048, 64, 64),
+               # few rows over a long reduction: the weight-stream kernel with every epilogue
+               (4, 2048, 520), (16, 2304, 1000), (1, 4096, 96)]
 
 
 @pytest.mark.parametrize("M,K,N", GEMM_SHAPES)

@@ -111,7 +111,14 @@ MID = [  # batches between the skinny kernel and the big-tile kernel, both activ
 ]
 
 
-@pytest.mark.parametrize("M,K,N,x32", WIDE + MID)
+STREAM = [  # at most 16 fp16 rows, K a multiple of 256 and >= 2048: every geometry of the weight-stream kernel
+    (1, 2048, 70, False), (2, 4096, 1000, False), (3, 2304, 520, False), (4, 2048, 8200, False), (4, 2560, 4096, False),
+    (5, 4096, 12300, False), (7, 2048, 8200, False), (8, 3072, 4100, False), (9, 4096, 12304, False), (12, 2048, 8192, False),
+    (16, 16384, 4096, False), (13, 2304, 48, False), (6, 8192, 28672, False), (1, 28672, 8192, False),
+]
+
+
+@pytest.mark.parametrize("M,K,N,x32", WIDE + MID + STREAM)
 def test_wide_layers_exact_on_integers(cuda, M, K, N, x32):
     """Small-integer activations, power-of-two scales and integer biases: every intermediate is
     exact in fp32, so the output must equal the integer matrix product bit for bit. The expected

@@ -15,6 +15,9 @@ namespace tmq {
 
 // mid.hip: staged split-reduction kernel for mid-size fp16 problems
 bool mid_dense_ok(const void *x, int64_t M, int64_t K);
+bool stream_dense_ok(const void *x, int64_t M, int64_t K);
+int launch_stream_dense(const void *x, int64_t M, int64_t K, const void *native, int64_t N, const float *scale,
+                        const float *bias, const void *residual, int relu, void *y, int y_f16, void *stream);
 int launch_mid_dense(const void *x, int64_t M, int64_t K, const void *native, int64_t N, const float *scale,
                      const float *bias, const void *residual, int relu, void *y, int y_f16, void *stream);
 
@@ -1098,6 +1101,11 @@ int tmq_ternary_linear(const void *x, int x_dtype, int64_t M, int64_t K, const v
     // kernels are as fast at K = 4096 and two to three times faster at short K, where staging all of
     // x in every workgroup dominates (M = 64, K = 512: 11.2 -> 4.6 us; fp32 input at K = 4096: 33 -> 14 us).
     const bool blocks_ok = (K % kKB == 0) && aligned16(x);
+    // At most 16 fp16 rows against eight or more weight blocks per channel: the weight-stream kernel (mid.hip).
+    // Against the kernels below: M = 16 at 16384^2 67 -> 20 us, M = 8 at 8192 x 28672 34 -> 17 us, M = 1 at
+    // 11008 x 4096 7.2 -> 6.2 us, even at 4096^2.
+    if (!x32 && stream_dense_ok(x, M, K) && K >= 8 * kKB)
+        return launch_stream_dense(x, M, K, native, N, ep.scale, ep.bias, ep.residual, ep.relu, y, ep.y_dtype == TMQ_F16, stream);
     if (M <= 16 || (M <= 64 && !blocks_ok))
         return x32 ? skinny_rows<true>(x, M, K, native, N, ep, y, stream)
                    : skinny_rows<false>(x, M, K, native, N, ep, y, stream);

@@ -125,11 +125,98 @@ __device__ __forceinline__ void load_to_lds(const void *src, unsigned char *dst)
 #endif
 }
 
+// Epilogue of the split-reduction kernels. Lane (j, g) of fragment (mi, nj) holds
+// y[16 mi + j][16 nj + 4 g + r], r = 0..3. Every wavefront parks its fragments in LDS (the windows are
+// dead by now) with the four g of a row next to each other; then the whole workgroup walks the tile row
+// by row: 16 consecutive threads own one row (4 columns each), add the WAVES partial sums in wavefront
+// order -- so the result does not depend on scheduling -- and write 128 or 256 contiguous bytes per row.
+// A thread keeps its columns for all its rows, so scale and bias are fetched once.
+template <int WM, int WN, int WAVES>
+__device__ __forceinline__ void reduce_and_store(unsigned char *smem, const floatx4 (&acc)[WM][WN], int kg, int lane,
+                                                 int64_t m0, int64_t n0, int64_t M, int64_t N, const MidEpilogue &ep) {
+    constexpr int NF = WM * WN;
+    const int j = lane & 15, g = lane >> 4;
+    constexpr int kFragPitch = 1024 + 64;                       // bytes; +64 spreads the nj over the banks
+    constexpr int T = 64 * WAVES, kC4 = 4 * WN;                 // threads; float4 columns per row
+    static_assert(T % kC4 == 0, "a thread must keep its columns");
+    if constexpr (WAVES > 1) __syncthreads();
+    else __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int mi = 0; mi < WM; mi++)
+#pragma unroll
+        for (int nj = 0; nj < WN; nj++)
+            *reinterpret_cast<floatx4 *>(smem + (size_t)(kg * NF + mi * WN + nj) * kFragPitch + (j * 4 + g) * 16) = acc[mi][nj];
+    if constexpr (WAVES > 1) __syncthreads();
+    else __builtin_amdgcn_wave_barrier();
+
+    const int tid = threadIdx.x, c4 = tid % kC4;
+    const int64_t n = n0 + c4 * 4;
+    const bool vec = (N % 4 == 0) && ((reinterpret_cast<uintptr_t>(ep.y) | reinterpret_cast<uintptr_t>(ep.residual) |
+                                       reinterpret_cast<uintptr_t>(ep.scale) | reinterpret_cast<uintptr_t>(ep.bias)) & 15u) == 0;
+    if (n < N) {
+        floatx4 sc = {1.f, 1.f, 1.f, 1.f}, bi = {0.f, 0.f, 0.f, 0.f};
+        if (vec) {
+            if (ep.scale) sc = *reinterpret_cast<const floatx4 *>(ep.scale + n);
+            if (ep.bias) bi = *reinterpret_cast<const floatx4 *>(ep.bias + n);
+        } else {
+#pragma unroll
+            for (int r = 0; r < 4; r++)
+                if (n + r < N) {
+                    if (ep.scale) sc[r] = ep.scale[n + r];
+                    if (ep.bias) bi[r] = ep.bias[n + r];
+                }
+        }
+        sc *= 1.0f / kWeightUnit;
+        for (int row = tid / kC4; row < 16 * WM; row += T / kC4) {
+            const int64_t m = m0 + row;
+            if (m >= M) break;
+            const unsigned char *src = smem + (size_t)((row >> 4) * WN + (c4 >> 2)) * kFragPitch + ((row & 15) * 4 + (c4 & 3)) * 16;
+            floatx4 v = *reinterpret_cast<const floatx4 *>(src);
+#pragma unroll
+            for (int q = 1; q < WAVES; q++) v += *reinterpret_cast<const floatx4 *>(src + (size_t)q * NF * kFragPitch);
+            v = v * sc + bi;
+            const int64_t o = m * N + n;
+            if (vec) {
+                if (ep.y_f16) {
+                    if (ep.residual) {
+                        const half4 rs = *reinterpret_cast<const half4 *>(static_cast<const _Float16 *>(ep.residual) + o);
+#pragma unroll
+                        for (int r = 0; r < 4; r++) v[r] += (float)rs[r];
+                    }
+                    half4 h;
+#pragma unroll
+                    for (int r = 0; r < 4; r++) h[r] = (_Float16)((ep.relu && v[r] < 0.f) ? 0.f : v[r]);
+                    *reinterpret_cast<half4 *>(static_cast<_Float16 *>(ep.y) + o) = h;
+                } else {
+                    if (ep.residual) v += *reinterpret_cast<const floatx4 *>(static_cast<const float *>(ep.residual) + o);
+                    if (ep.relu) {
+#pragma unroll
+                        for (int r = 0; r < 4; r++) v[r] = v[r] > 0.f ? v[r] : 0.f;
+                    }
+                    *reinterpret_cast<floatx4 *>(static_cast<float *>(ep.y) + o) = v;
+                }
+            } else {
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    if (n + r >= N) break;
+                    float f = v[r];
+                    if (ep.y_f16) {
+                        if (ep.residual) f += (float)static_cast<const _Float16 *>(ep.residual)[o + r];
+                        static_cast<_Float16 *>(ep.y)[o + r] = (_Float16)((ep.relu && f < 0.f) ? 0.f : f);
+                    } else {
+                        if (ep.residual) f += static_cast<const float *>(ep.residual)[o + r];
+                        static_cast<float *>(ep.y)[o + r] = (ep.relu && f < 0.f) ? 0.f : f;
+                    }
+                }
+            }
+        }
+    }
+}
+
 template <int WM, int WN, int WAVES, class Rows>
 __global__ __launch_bounds__(64 * WAVES) void mid_kernel(Rows rows, const u32x4 *__restrict__ native, int64_t M, int Kb,
                                                          int npairs, int64_t N, int64_t Nb, int tiles_n,
                                                          MidEpilogue ep) {
-    constexpr int NF = WM * WN;
     constexpr int kFrag = 16 * 128, kSlot = WM * kFrag, kWave = 2 * kSlot;   // bytes: 16 rows x 128 B per fragment
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const int lane = threadIdx.x & 63, kg = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -214,87 +301,7 @@ __global__ __launch_bounds__(64 * WAVES) void mid_kernel(Rows rows, const u32x4 
         if (p < np) step(p, std::integral_constant<int, 0>{});
     }
 
-    // Epilogue. Lane (j, g) of fragment (mi, nj) holds y[16 mi + j][16 nj + 4 g + r], r = 0..3. Every
-    // wavefront parks its fragments in LDS (the windows are dead by now) with the four g of a row
-    // next to each other; then the whole workgroup walks the tile row by row: 16 consecutive threads
-    // own one row (4 columns each), add the WAVES partial sums in wavefront order -- so the result
-    // does not depend on scheduling -- and write 128 or 256 contiguous bytes per row. A thread keeps
-    // its columns for all its rows, so scale and bias are fetched once.
-    constexpr int kFragPitch = 1024 + 64;                       // bytes; +64 spreads the nj over the banks
-    constexpr int T = 64 * WAVES, kC4 = 4 * WN;                 // threads; float4 columns per row
-    static_assert(T % kC4 == 0, "a thread must keep its columns");
-    if constexpr (WAVES > 1) __syncthreads();
-    else __builtin_amdgcn_wave_barrier();
-#pragma unroll
-    for (int mi = 0; mi < WM; mi++)
-#pragma unroll
-        for (int nj = 0; nj < WN; nj++)
-            *reinterpret_cast<floatx4 *>(smem + (size_t)(kg * NF + mi * WN + nj) * kFragPitch + (j * 4 + g) * 16) = acc[mi][nj];
-    if constexpr (WAVES > 1) __syncthreads();
-    else __builtin_amdgcn_wave_barrier();
-
-    const int tid = threadIdx.x, c4 = tid % kC4;
-    const int64_t n = n0 + c4 * 4;
-    const bool vec = (N % 4 == 0) && ((reinterpret_cast<uintptr_t>(ep.y) | reinterpret_cast<uintptr_t>(ep.residual) |
-                                       reinterpret_cast<uintptr_t>(ep.scale) | reinterpret_cast<uintptr_t>(ep.bias)) & 15u) == 0;
-    if (n < N) {
-        floatx4 sc = {1.f, 1.f, 1.f, 1.f}, bi = {0.f, 0.f, 0.f, 0.f};
-        if (vec) {
-            if (ep.scale) sc = *reinterpret_cast<const floatx4 *>(ep.scale + n);
-            if (ep.bias) bi = *reinterpret_cast<const floatx4 *>(ep.bias + n);
-        } else {
-#pragma unroll
-            for (int r = 0; r < 4; r++)
-                if (n + r < N) {
-                    if (ep.scale) sc[r] = ep.scale[n + r];
-                    if (ep.bias) bi[r] = ep.bias[n + r];
-                }
-        }
-        sc *= 1.0f / kWeightUnit;
-        for (int row = tid / kC4; row < 16 * WM; row += T / kC4) {
-            const int64_t m = m0 + row;
-            if (m >= M) break;
-            const unsigned char *src = smem + (size_t)((row >> 4) * WN + (c4 >> 2)) * kFragPitch + ((row & 15) * 4 + (c4 & 3)) * 16;
-            floatx4 v = *reinterpret_cast<const floatx4 *>(src);
-#pragma unroll
-            for (int q = 1; q < WAVES; q++) v += *reinterpret_cast<const floatx4 *>(src + (size_t)q * NF * kFragPitch);
-            v = v * sc + bi;
-            const int64_t o = m * N + n;
-            if (vec) {
-                if (ep.y_f16) {
-                    if (ep.residual) {
-                        const half4 rs = *reinterpret_cast<const half4 *>(static_cast<const _Float16 *>(ep.residual) + o);
-#pragma unroll
-                        for (int r = 0; r < 4; r++) v[r] += (float)rs[r];
-                    }
-                    half4 h;
-#pragma unroll
-                    for (int r = 0; r < 4; r++) h[r] = (_Float16)((ep.relu && v[r] < 0.f) ? 0.f : v[r]);
-                    *reinterpret_cast<half4 *>(static_cast<_Float16 *>(ep.y) + o) = h;
-                } else {
-                    if (ep.residual) v += *reinterpret_cast<const floatx4 *>(static_cast<const float *>(ep.residual) + o);
-                    if (ep.relu) {
-#pragma unroll
-                        for (int r = 0; r < 4; r++) v[r] = v[r] > 0.f ? v[r] : 0.f;
-                    }
-                    *reinterpret_cast<floatx4 *>(static_cast<float *>(ep.y) + o) = v;
-                }
-            } else {
-#pragma unroll
-                for (int r = 0; r < 4; r++) {
-                    if (n + r >= N) break;
-                    float f = v[r];
-                    if (ep.y_f16) {
-                        if (ep.residual) f += (float)static_cast<const _Float16 *>(ep.residual)[o + r];
-                        static_cast<_Float16 *>(ep.y)[o + r] = (_Float16)((ep.relu && f < 0.f) ? 0.f : f);
-                    } else {
-                        if (ep.residual) f += static_cast<const float *>(ep.residual)[o + r];
-                        static_cast<float *>(ep.y)[o + r] = (ep.relu && f < 0.f) ? 0.f : f;
-                    }
-                }
-            }
-        }
-    }
+    reduce_and_store<WM, WN, WAVES>(smem, acc, kg, lane, m0, n0, M, N, ep);
 }
 
 template <int WM, int WN, int WAVES, class Rows>
@@ -316,6 +323,173 @@ int launch(const Rows &rows, const void *native, int64_t M, int64_t K, int64_t N
     hipLaunchKernelGGL(kernel, dim3((uint32_t)(tm * tn)), dim3(64 * WAVES), lds, as_stream(stream), rows,
                        static_cast<const u32x4 *>(native), M, (int)Kb, (int)((K + 63) / 64), N, native_blocks_n(N),
                        (int)tn, ep);
+    return check_launch();
+}
+
+// ---- weight stream, at most 16 rows ------------------------------------------------------------------
+// Large layers with a handful of rows (batched decoding): the job is to read the weights once at HBM
+// speed. A workgroup of WAVES wavefronts owns 16 WN output channels and splits the reduction over its
+// wavefronts by whole weight blocks (256 reduction indices): wavefront kg takes blocks kg, kg + WAVES, ...
+// Unlike mid_kernel, whose pipeline unit is a 64-index pair loaded one step ahead, a wavefront here keeps
+// D of its blocks in flight -- the WN weight blocks as whole 1 KiB loads (one instruction per block
+// instead of four dword loads) in D register sets, and the R x 512 bytes of activations that go with
+// them in a private LDS window of D slots -- enough outstanding bytes to cover the latency of HBM. An
+// operand read from LDS feeds WN multiplications.
+//
+// R = 16, 8, 4 or 2 >= M rows are staged (fewer rows: smaller slots, deeper pipeline). One staging
+// instruction moves 1 KiB, lane l to byte 16 l of its destination: 8 rows x 128 bytes for R >= 8 (the
+// layout of mid_kernel), else R rows x 1024 / R bytes. Rows lie a multiple of 256 bytes apart, i.e. on the
+// same banks, so the 16-byte chunk c of row r is stored at position c ^ swz(r); the XOR is applied to the
+// source address and undone by the reader. Rows past M repeat row M - 1; MFMA columns past M read row
+// M - 1 too and are never stored. Requires K % 256 == 0.
+template <int R>
+struct StreamRows {
+    static constexpr int kLoads = R / 2;                             // staging instructions per block: R x 512 B / 1 KiB
+    static constexpr int kSlot = R * 512;                            // bytes of a block's activations
+    // element offset (without the block's k0) of what lane `lane` fetches in instruction i
+    __device__ static uint32_t source(int i, int lane, int64_t M, int64_t K) {
+        int row, k;
+        if constexpr (R >= 8) {                                        // instruction = (pair, half): 8 rows x 128 B
+            const int p = R == 16 ? i >> 1 : i, c = R == 16 ? i & 1 : 0;
+            row = 8 * c + (lane >> 3);
+            k = p * 64 + (((lane & 7) ^ ((row >> 1) & 7)) * 8);
+        } else {                                                       // R rows x (1024 / R) B
+            constexpr int kPieces = 64 / R;                            // 16-byte pieces per row and instruction
+            row = lane / kPieces;
+            k = i * (kPieces * 8) + (((lane % kPieces) ^ (row << 2)) * 8);
+        }
+        if (row >= M) row = (int)M - 1;
+        return (uint32_t)(row * K + k);
+    }
+    // LDS offset inside a slot of (row r, MFMA step i of the block, lane group g)
+    __device__ static int operand(int r, int i, int g) {
+        if constexpr (R >= 8) {
+            const int p = i >> 1, c = 4 * (i & 1) + g;                 // pair, chunk of the pair
+            return p * (R * 128) + r * 128 + ((c ^ ((r >> 1) & 7)) * 16);
+        } else {
+            constexpr int kPieces = 64 / R;
+            const int c = 4 * i + g;                                   // chunk of the block's 32
+            return (c / kPieces) * 1024 + r * (kPieces * 16) + (((c % kPieces) ^ (r << 2)) * 16);
+        }
+    }
+};
+
+template <int WN, int WAVES, int R, int D>
+__global__ __launch_bounds__(64 * WAVES) void stream_kernel(const _Float16 *__restrict__ x, const u32x4 *__restrict__ native,
+                                                            int64_t M, int64_t K, int Kb, int64_t N, int64_t Nb,
+                                                            MidEpilogue ep) {
+    using Rows = StreamRows<R>;
+    constexpr int kLoads = Rows::kLoads, kSlot = Rows::kSlot, kWave = D * kSlot, kPerBlock = WN + kLoads;
+    static_assert((D - 1) * kPerBlock < 64, "vmcnt is a 6-bit counter");
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    const int lane = threadIdx.x & 63, kg = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int j = lane & 15, g = lane >> 4;
+    unsigned char *win = smem + kg * kWave;
+    const int64_t n0 = (int64_t)blockIdx.x * (16 * WN);
+
+    floatx4 acc[1][WN];
+#pragma unroll
+    for (int nj = 0; nj < WN; nj++) acc[0][nj] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+    const u32x4 *wb[WN];                                          // block kb of channel block nj: wb[nj][kb * 64]
+#pragma unroll
+    for (int nj = 0; nj < WN; nj++) {
+        int64_t nb = n0 / 16 + nj;
+        if (nb >= Nb) nb = Nb - 1;                                  // finite bits, never stored
+        wb[nj] = native + (nb * Kb) * 64 + lane;
+    }
+    uint32_t src[kLoads];
+#pragma unroll
+    for (int i = 0; i < kLoads; i++) src[i] = Rows::source(i, lane, M, K);
+    int rd[8];                                                      // operand offsets of the 8 MFMA steps
+    {
+        const int r = j < M ? j : (int)M - 1;
+#pragma unroll
+        for (int i = 0; i < 8; i++) rd[i] = Rows::operand(r, i, g);
+    }
+
+    const int nt = Kb > kg ? (Kb - kg + WAVES - 1) / WAVES : 0;   // weight blocks of this wavefront
+    auto wload = [&](u32x4 (&w)[WN], int t) {
+        const int64_t kb = kg + (int64_t)t * WAVES;
+#pragma unroll
+        for (int nj = 0; nj < WN; nj++) w[nj] = __builtin_nontemporal_load(wb[nj] + kb * 64);
+    };
+    auto fill = [&](int slot, int t) {
+        const _Float16 *xb = x + (kg + (int64_t)t * WAVES) * kKB;
+#pragma unroll
+        for (int i = 0; i < kLoads; i++) load_to_lds(xb + src[i], win + slot * kSlot + i * 1024);
+    };
+    // wait until at most n blocks' loads are outstanding (loads complete in issue order)
+    auto wait_blocks = [&](int n) {
+        static_assert(D <= 4, "cases below");
+        constexpr auto enc = [](int c) { return (c & 15) | (7 << 4) | (15 << 8) | ((c >> 4) << 14); };
+        if (n >= 3 && D > 3) __builtin_amdgcn_s_waitcnt(enc(3 * kPerBlock));
+        else if (n == 2 && D > 2) __builtin_amdgcn_s_waitcnt(enc(2 * kPerBlock));
+        else if (n == 1) __builtin_amdgcn_s_waitcnt(enc(kPerBlock));
+        else __builtin_amdgcn_s_waitcnt(enc(0));
+    };
+
+    if (nt > 0) {
+        u32x4 wq[D][WN];
+#pragma unroll
+        for (int d = 0; d < D; d++)
+            if (d < nt) {
+                fill(d, d);
+                wload(wq[d], d);
+            }
+        // one block; `par` (static) = t % D = LDS slot and weight register set of the block
+        auto step = [&](int t, auto par_tag) {
+            constexpr int par = decltype(par_tag)::value;
+            const int ahead = nt - 1 - t;                         // blocks issued after this one
+            wait_blocks(ahead < D - 1 ? ahead : D - 1);
+            __builtin_amdgcn_sched_barrier(0);
+            half8 a[8];                                            // all operand reads of the block
+#pragma unroll
+            for (int i = 0; i < 8; i++) a[i] = *reinterpret_cast<const half8 *>(win + par * kSlot + rd[i]);
+            // the slot is free again once the reads have returned: refill it with the block D ahead
+            __builtin_amdgcn_s_waitcnt(0xC07F);                    // lgkmcnt(0)
+            __builtin_amdgcn_sched_barrier(0);
+            if (t + D < nt) fill(par, t + D);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int i = 0; i < 8; i++)
+#pragma unroll
+                for (int nj = 0; nj < WN; nj++)
+                    acc[0][nj] = mfma16(decode_step(wq[par][nj][i >> 1], i & 1), a[i], acc[0][nj]);
+            __builtin_amdgcn_sched_barrier(0);
+            if (t + D < nt) wload(wq[par], t + D);
+            __builtin_amdgcn_sched_barrier(0);
+        };
+        int t = 0;
+        for (; t + D <= nt; t += D) {
+            step(t, std::integral_constant<int, 0>{});
+            if constexpr (D > 1) step(t + 1, std::integral_constant<int, 1>{});
+            if constexpr (D > 2) step(t + 2, std::integral_constant<int, 2>{});
+            if constexpr (D > 3) step(t + 3, std::integral_constant<int, 3>{});
+        }
+        if (t < nt) step(t, std::integral_constant<int, 0>{});
+        if constexpr (D > 2) if (t + 1 < nt) step(t + 1, std::integral_constant<int, 1>{});
+        if constexpr (D > 3) if (t + 2 < nt) step(t + 2, std::integral_constant<int, 2>{});
+    }
+    reduce_and_store<1, WN, WAVES>(smem, acc, kg, lane, 0, n0, M, N, ep);
+}
+
+template <int WN, int WAVES, int R, int D>
+int launch_stream(const void *x, const void *native, int64_t M, int64_t K, int64_t N, const MidEpilogue &ep, void *stream) {
+    const int64_t tn = (N + 16 * WN - 1) / (16 * WN), Kb = native_blocks_k(K);
+    if (tn > 0x7FFFFFFF || Kb > (1 << 20)) return TMQ_ERR_TOO_LARGE;
+    constexpr size_t win = (size_t)WAVES * D * R * 512, redb = (size_t)WAVES * WN * (1024 + 64);
+    constexpr size_t lds = win > redb ? win : redb;
+    static_assert(lds <= 152 * 1024, "LDS budget");
+    auto kernel = stream_kernel<WN, WAVES, R, D>;
+    if (lds > 64 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return note_hip_error(e);
+    }
+    hipLaunchKernelGGL(kernel, dim3((uint32_t)tn), dim3(64 * WAVES), lds, as_stream(stream),
+                       static_cast<const _Float16 *>(x), static_cast<const u32x4 *>(native), M, K, (int)Kb, N,
+                       native_blocks_n(N), ep);
     return check_launch();
 }
 
@@ -372,6 +546,35 @@ int launch_mid_dense(const void *x, int64_t M, int64_t K, const void *native, in
                      const float *bias, const void *residual, int relu, void *y, int y_f16, void *stream) {
     MidEpilogue ep{scale, bias, residual, y, relu, y_f16};
     return dispatch(DenseRows{static_cast<const _Float16 *>(x), M, K}, native, M, K, N, ep, stream);
+}
+
+// True when the weight-stream kernel can take a dense fp16 problem of at most 16 rows.
+bool stream_dense_ok(const void *x, int64_t M, int64_t K) {
+    return M >= 1 && M <= 16 && (K % kKB == 0) && aligned16(x) && M * K < (int64_t)0x7FFFFFFF;
+}
+
+// Geometry of the weight-stream kernel (stream_dense_ok must hold). Rows staged: the power of two >= M. Tile
+// width: the fewer rows, the smaller the LDS windows and the more workgroups fit a CU, so narrow tiles
+// (more workgroups, less reuse of an operand read) win for M <= 2, wider ones once a row block costs as much
+// to stage as the weights it meets -- provided at least 256 workgroups remain (measured on 4096^2 ..
+// 16384^2, 8192 x 28672 and 28672 x 8192).
+int launch_stream_dense(const void *x, int64_t M, int64_t K, const void *native, int64_t N, const float *scale,
+                        const float *bias, const void *residual, int relu, void *y, int y_f16, void *stream) {
+    MidEpilogue ep{scale, bias, residual, y, relu, y_f16};
+    const int64_t Nb = native_blocks_n(N);
+    if (M <= 2) return launch_stream<1, 8, 2, 4>(x, native, M, K, N, ep, stream);
+    if (M <= 4) {
+        if (Nb >= 512) return launch_stream<2, 8, 4, 4>(x, native, M, K, N, ep, stream);
+        return launch_stream<1, 8, 4, 4>(x, native, M, K, N, ep, stream);
+    }
+    if (M <= 8) {
+        if (Nb >= 768) return launch_stream<4, 8, 8, 2>(x, native, M, K, N, ep, stream);
+        if (Nb >= 512) return launch_stream<2, 8, 8, 4>(x, native, M, K, N, ep, stream);
+        return launch_stream<1, 8, 8, 4>(x, native, M, K, N, ep, stream);
+    }
+    if (Nb >= 768) return launch_stream<4, 8, 16, 2>(x, native, M, K, N, ep, stream);
+    if (Nb >= 512) return launch_stream<2, 8, 16, 2>(x, native, M, K, N, ep, stream);
+    return launch_stream<1, 8, 16, 2>(x, native, M, K, N, ep, stream);
 }
 
 bool mid_conv_ok(const void *x, const tmq_conv_shape *s) {
