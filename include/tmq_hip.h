@@ -215,6 +215,20 @@ typedef struct tmq_epilogue {
 int tmq_ternary_linear(const void *x, int x_dtype, int64_t M, int64_t K, const void *native,
                        int64_t N, const tmq_epilogue *epilogue, void *y, void *stream);
 
+/* hi[i] = fp16(x[i]), lo[i] = fp16(x[i] - hi[i]) for n fp32 values (device pointers; hi, lo fp16).
+ * No counterpart in the reference, whose ternary_mmm_cuda (tmq/tmq_cuda.cu:478-549) multiplies fp32
+ * activations in fp32: for many rows a caller that may allocate runs the fp16 kernels on the two terms,
+ *   t = tmq_ternary_linear(hi, ..., scale, bias, residual)  (fp32 out, no ReLU)
+ *   y = tmq_ternary_linear(lo, ..., scale, residual = t, ReLU)
+ * which keeps ~fp32 accuracy at MFMA speed (M = 4096, K = N = 4096: 400 -> 238 us); the bindings in
+ * tmq_amd/ops.py and tmq_amd/csrc/torch_ext.cpp do so where tmq_fp32_rows_prefer_split says it pays. */
+int tmq_split_f32(const float *x, void *hi, void *lo, int64_t n, void *stream);
+
+/* 1 if M fp32 rows against a K x N layer are faster as two fp16 passes over tmq_split_f32's terms than
+ * as one tmq_ternary_linear call with x_dtype TMQ_F32 (many rows, or a few rows over a very large
+ * layer), else 0. Host-only arithmetic on the shape; no counterpart in the reference.               */
+int tmq_fp32_rows_prefer_split(int64_t M, int64_t K, int64_t N);
+
 /* Measurement aid with no counterpart in the reference: streams `bytes` (a multiple of 1024)
  * from src with the launch geometry of the M = 1 path of tmq_ternary_linear (1 KiB per
  * wavefront and load, 16 wavefronts per workgroup) and does nothing else; *sink (device, 4

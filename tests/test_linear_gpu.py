@@ -72,6 +72,49 @@ def test_linear_fp32_activations(cuda, oracle, M, K, N):
             assert _rel_err(v.cpu().numpy().reshape(1, N), ref) <= 5e-6
 
 
+def test_split_f32_terms(cuda):
+    """hi = fp16(x), lo = fp16(x - hi), bit for bit, on aligned, ragged and unaligned buffers."""
+    from tmq_amd import ops
+    g = torch.Generator(device=cuda).manual_seed(5)
+    base = torch.randn(1 << 16, device=cuda, generator=g) * torch.pow(10.0, torch.randint(-6, 4, (1 << 16,), device=cuda, generator=g).float())
+    base[:8] = torch.tensor([0.0, -0.0, 65504.0, -65504.0, 1e-8, 70000.0, 1.0 + 2.0 ** -12, -3.0], device=cuda)
+    for x in (base, base[:4099], base[1:2050], base[:5]):
+        hi, lo = ops.split_f32(x)
+        want_hi = x.half()
+        want_lo = (x - want_hi.float()).half()
+        assert torch.equal(hi.view(torch.int16), want_hi.view(torch.int16))
+        assert torch.equal(lo.view(torch.int16), want_lo.view(torch.int16))
+    fin = torch.isfinite(hi.float())
+    x = base[:5]
+    assert torch.all((hi.float() + lo.float() - x).abs()[fin] <= x.abs()[fin] * 2.0 ** -21 + 1e-7)
+
+
+@pytest.mark.parametrize("M,K,N", [(1024, 1024, 4096), (600, 4096, 2048), (5, 16384, 8192)])
+def test_linear_fp32_many_rows(cuda, M, K, N):
+    """Many fp32 rows run as two passes of the fp16 kernels over the two fp16 terms of the activations:
+    fp32-level accuracy against the fp64 product, with every epilogue option."""
+    from tmq_amd import ops
+    g = torch.Generator(device=cuda).manual_seed(M + K)
+    W = torch.randint(-1, 2, (N, K), dtype=torch.int8, device=cuda, generator=g)
+    nw = ops.NativeWeights(ops.compactify_ternary(W), N)
+    x = torch.randn(M, K, device=cuda, generator=g)
+    scale = 0.5 + torch.rand(N, device=cuda, generator=g)
+    bias = torch.randn(N, device=cuda, generator=g)
+    res = torch.randn(M, N, device=cuda, generator=g)
+    ref = x.double() @ W.double().T
+    y = ops.ternary_linear(x, nw)
+    assert ((y.double() - ref).abs().max() / ref.abs().max()).item() <= 5e-6
+    y2 = ops.ternary_linear(x, nw, scale, bias, residual=res, relu=True)
+    ref2 = torch.relu(ref * scale.double() + bias.double() + res.double())
+    assert ((y2.double() - ref2).abs().max() / ref2.abs().max()).item() <= 5e-6
+    # the fp16 product of the same activations is three orders of magnitude coarser
+    y16 = ops.ternary_linear(x.half(), nw)
+    assert ((y16.double() - ref).abs().max() / ref.abs().max()).item() > 5e-5
+    # integers: exact
+    xi = torch.randint(-8, 9, (M, K), device=cuda, generator=g).float()
+    assert torch.equal(ops.ternary_linear(xi, nw), xi @ W.float().T)
+
+
 def test_exactness_on_integers(cuda, oracle):
     """With small-integer activations every product and partial sum is exact in fp32, so the
     result must equal the integer matrix product bit for bit, whatever the summation order."""

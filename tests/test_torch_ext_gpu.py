@@ -61,7 +61,7 @@ def test_pack_codec_round_trip_and_oracle(cuda, ext, oracle):
 def test_ternary_products_match_ctypes_binding(cuda, ext):
     from tmq_amd import ops
     g = torch.Generator(device=cuda).manual_seed(2)
-    for (M, K, N) in [(1, 4096, 4096), (7, 512, 102), (300, 4096, 96), (64, 2304, 512)]:
+    for (M, K, N) in [(1, 4096, 4096), (7, 512, 102), (300, 4096, 96), (64, 2304, 512), (1024, 2048, 2048)]:
         W = torch.randint(-1, 2, (N, K), device=cuda, generator=g).float()
         words = ext.compactify_ternary(W)
         x = torch.randn(M, K, device=cuda, generator=g)

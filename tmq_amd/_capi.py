@@ -58,6 +58,8 @@ SIGNATURES = {
     "tmq_softstep_fused": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _dbl, _dbl, _dbl, _flt, _dbl, _dbl, _vp]),
     "tmq_selfcheck_division": (_int, [_dbl, _vp, _vp]),
     "tmq_probe_stream_read": (_int, [_vp, ctypes.c_size_t, _vp, _vp]),
+    "tmq_split_f32": (_int, [_vp, _vp, _vp, _i64, _vp]),
+    "tmq_fp32_rows_prefer_split": (_int, [_i64, _i64, _i64]),
     "tmq_multi_plan": (_int, [ctypes.POINTER(Segment), _int, ctypes.POINTER(_u32)]),
     "tmq_qloss_multi_workspace_bytes": (_sz, [_u32]),
     "tmq_qloss_multi": (_int, [_vp, _int, _u32, _dbl, _dbl, _vp, _vp, _vp, _vp]),

@@ -1031,6 +1031,35 @@ int mid_rows(const void *x, int64_t M, int64_t K, const void *native, int64_t N,
     return launch_mid<2, 1, 2, 16, 2, X32>(x, M, K, native, N, ep, y, stream);
 }
 
+// ---- two-term split ------------------------------------------------------------------------------
+// x = hi + lo with hi = fp16(x), lo = fp16(x - hi): 22 significant bits in two fp16 values. 8 elements per
+// thread (two 16-byte loads, a 16-byte store per term) when the pointers allow it.
+__global__ __launch_bounds__(256) void split_terms_kernel(const float *__restrict__ x, _Float16 *__restrict__ hi,
+                                                          _Float16 *__restrict__ lo, int64_t n, int vec) {
+    const int64_t i0 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 8;
+    if (i0 >= n) return;
+    if (vec && i0 + 8 <= n) {
+        const floatx4 a = __builtin_nontemporal_load(reinterpret_cast<const floatx4 *>(x + i0));
+        const floatx4 b = __builtin_nontemporal_load(reinterpret_cast<const floatx4 *>(x + i0 + 4));
+        half8 h, l;
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            h[e] = (_Float16)a[e];
+            h[4 + e] = (_Float16)b[e];
+            l[e] = (_Float16)(a[e] - (float)h[e]);
+            l[4 + e] = (_Float16)(b[e] - (float)h[4 + e]);
+        }
+        *reinterpret_cast<half8 *>(hi + i0) = h;
+        *reinterpret_cast<half8 *>(lo + i0) = l;
+    } else {
+        for (int64_t i = i0; i < n && i < i0 + 8; i++) {
+            const _Float16 h = (_Float16)x[i];
+            hi[i] = h;
+            lo[i] = (_Float16)(x[i] - (float)h);
+        }
+    }
+}
+
 // ---- read probe -------------------------------------------------------------------------------------
 // The weight stream of the skinny kernel and nothing else: wavefront w of a workgroup reads the
 // 1 KiB pieces w, w + 16, ... of the workgroup's share.
@@ -1069,6 +1098,27 @@ int tmq_prepack_weights(const uint32_t *words, int64_t N, int64_t C, int64_t ky,
     if (blocks > 0x7FFFFFFF) return TMQ_ERR_TOO_LARGE;
     hipLaunchKernelGGL(prepack_kernel, dim3((uint32_t)blocks), dim3(256), 0, as_stream(stream), words,
                        static_cast<uint32_t *>(native), N, K, C, ky, kx, Kb, total);
+    return check_launch();
+}
+
+int tmq_fp32_rows_prefer_split(int64_t M, int64_t K, int64_t N) {
+    // Measured: at K = N = 4096 the two fp16 passes win from about 512 rows (M = 4096: 400 -> 238 us), at
+    // K = N = 1024 from about 4096; over very large layers already from 3 rows (16384^2, M = 16: 118 -> 45 us),
+    // because the fp16 weight-stream and tile kernels have no fp32 form.
+    if (M <= 0 || K <= 0 || N <= 0) return 0;
+    const bool many_rows = M >= 512 && (double)M * (double)K * (double)N >= 4294967296.0;
+    const bool large_layer = M >= 3 && (double)K * (double)N >= 134217728.0;
+    return many_rows || large_layer;
+}
+
+int tmq_split_f32(const float *x, void *hi, void *lo, int64_t n, void *stream) {
+    if (n < 0 || (n > 0 && (!x || !hi || !lo))) return TMQ_ERR_INVALID_ARG;
+    if (n == 0) return TMQ_OK;
+    const int64_t blocks = (n + 2047) / 2048;
+    if (blocks > 0x7FFFFFFF) return TMQ_ERR_TOO_LARGE;
+    const int vec = aligned16(x) && aligned16(hi) && aligned16(lo);
+    hipLaunchKernelGGL(split_terms_kernel, dim3((uint32_t)blocks), dim3(256), 0, as_stream(stream), x,
+                       static_cast<_Float16 *>(hi), static_cast<_Float16 *>(lo), n, vec);
     return check_launch();
 }
 

@@ -126,6 +126,19 @@ torch::Tensor ternary_mmm_cuda(torch::Tensor lhs, torch::Tensor weights, int64_t
     shape.back() = columns;
     auto y = torch::empty(shape, lhs.options().dtype(torch::kFloat32));
     const int64_t M = K ? x.numel() / K : 0;
+    if (x.scalar_type() == torch::kFloat32 && tmq_fp32_rows_prefer_split(M, K, columns)) {
+        // many fp32 rows: the fp16 kernels over the two fp16 terms of the activations, y = W hi + W lo
+        auto hi = torch::empty_like(x, x.options().dtype(torch::kFloat16));
+        auto lo = torch::empty_like(hi);
+        check(tmq_split_f32(x.data_ptr<float>(), hi.data_ptr(), lo.data_ptr(), x.numel(), stream_of(x)), "ternary_mmm_cuda");
+        auto t = torch::empty_like(y);
+        check(tmq_ternary_linear(hi.data_ptr(), TMQ_F16, M, K, native.data_ptr(), columns, nullptr, t.data_ptr(),
+                                 stream_of(x)), "ternary_mmm_cuda");
+        tmq_epilogue ep = {nullptr, nullptr, t.data_ptr(), 0, TMQ_F32};
+        check(tmq_ternary_linear(lo.data_ptr(), TMQ_F16, M, K, native.data_ptr(), columns, &ep, y.data_ptr(),
+                                 stream_of(x)), "ternary_mmm_cuda");
+        return y;
+    }
     check(tmq_ternary_linear(x.data_ptr(), x.scalar_type() == torch::kFloat16 ? TMQ_F16 : TMQ_F32, M, K,
                              native.data_ptr(), columns, nullptr, y.data_ptr(), stream_of(x)), "ternary_mmm_cuda");
     return y;

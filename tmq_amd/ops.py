@@ -396,6 +396,18 @@ def _epilogue(nw, scale, bias, residual, relu, out_dtype, y):
     return ep
 
 
+def split_f32(x: torch.Tensor):
+    """(hi, lo) with hi = fp16(x), lo = fp16(x - hi): fp32 activations as two fp16 terms."""
+    _capi.require_gpu(x, "activations")
+    if x.dtype != torch.float32:
+        raise RuntimeError("split_f32: expected fp32")
+    x = x.contiguous()
+    hi, lo = torch.empty_like(x, dtype=torch.float16), torch.empty_like(x, dtype=torch.float16)
+    with torch.cuda.device(x.device):
+        check(_lib().tmq_split_f32(ptr(x), ptr(hi), ptr(lo), x.numel(), stream_of(x)), "split_f32")
+    return hi, lo
+
+
 def ternary_linear(x: torch.Tensor, nw: NativeWeights, scale=None, bias=None, residual=None, relu=False,
                    out_dtype=torch.float32) -> torch.Tensor:
     """y[..., n] = relu?(scale[n] * sum_k x[..., k] T[k][n] + bias[n] + residual); x fp16 or fp32."""
@@ -405,6 +417,13 @@ def ternary_linear(x: torch.Tensor, nw: NativeWeights, scale=None, bias=None, re
     if x.shape[-1] != nw.K:
         raise RuntimeError(f"ternary_linear: activations have {x.shape[-1]} features, weights expect {nw.K}")
     M = x.numel() // nw.K if nw.K else 0
+    if (x.dtype == torch.float32 and out_dtype == torch.float32 and (residual is None or residual.dtype == torch.float32)
+            and _lib().tmq_fp32_rows_prefer_split(M, nw.K, nw.N)):
+        # many fp32 rows (or a few over a very large layer): two passes of the fp16 kernels over the two
+        # fp16 terms of the activations beat the kernels that split them on the fly
+        hi, lo = split_f32(x)
+        t = ternary_linear(hi, nw, scale, bias, residual, False, torch.float32)
+        return ternary_linear(lo, nw, scale, None, t, relu, torch.float32)
     y = torch.empty(x.shape[:-1] + (nw.N,), dtype=out_dtype, device=x.device)
     ep = _epilogue(nw, scale, bias, residual, relu, out_dtype, y)
     with torch.cuda.device(x.device):
