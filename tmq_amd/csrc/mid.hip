@@ -553,11 +553,13 @@ bool stream_dense_ok(const void *x, int64_t M, int64_t K) {
     return M >= 1 && M <= 16 && (K % kKB == 0) && aligned16(x) && M * K < (int64_t)0x7FFFFFFF;
 }
 
-// Geometry of the weight-stream kernel (stream_dense_ok must hold). Rows staged: the power of two >= M. Tile
-// width: the fewer rows, the smaller the LDS windows and the more workgroups fit a CU, so narrow tiles
-// (more workgroups, less reuse of an operand read) win for M <= 2, wider ones once a row block costs as much
-// to stage as the weights it meets -- provided at least 256 workgroups remain (measured on 4096^2 ..
-// 16384^2, 8192 x 28672 and 28672 x 8192).
+// Geometry of the weight-stream kernel (stream_dense_ok must hold). Rows staged: the power of two >= M.
+// What decides is that all workgroups are resident at once: a second, partly filled pass over the CUs
+// costs more than running with fewer workgroups than CUs (N = 5120 at M = 16: 320 workgroups of one per CU
+// 9.0 us, 160 twice as wide 6.1 us). Residency per CU follows from the LDS windows: 4 workgroups at R = 2,
+// 2 at R = 4 and at R = 8 with two blocks in flight, 1 at R = 16 (2 with four wavefronts). So: the
+// narrowest tile whose workgroups fit in one pass (narrow tiles mean more wavefronts streaming), measured
+// on 4096 x {4096, 5120, 11008, 13824}, 8192 x {6144, 8192, 16384, 28672} and 16384^2.
 int launch_stream_dense(const void *x, int64_t M, int64_t K, const void *native, int64_t N, const float *scale,
                         const float *bias, const void *residual, int relu, void *y, int y_f16, void *stream) {
     MidEpilogue ep{scale, bias, residual, y, relu, y_f16};
@@ -568,13 +570,14 @@ int launch_stream_dense(const void *x, int64_t M, int64_t K, const void *native,
         return launch_stream<1, 8, 4, 4>(x, native, M, K, N, ep, stream);
     }
     if (M <= 8) {
-        if (Nb >= 768) return launch_stream<4, 8, 8, 2>(x, native, M, K, N, ep, stream);
-        if (Nb >= 512) return launch_stream<2, 8, 8, 4>(x, native, M, K, N, ep, stream);
-        return launch_stream<1, 8, 8, 4>(x, native, M, K, N, ep, stream);
+        if (Nb <= 256) return launch_stream<1, 8, 8, 4>(x, native, M, K, N, ep, stream);
+        if (Nb <= 1024) return launch_stream<2, 8, 8, 2>(x, native, M, K, N, ep, stream);
+        return launch_stream<4, 8, 8, 2>(x, native, M, K, N, ep, stream);
     }
-    if (Nb >= 768) return launch_stream<4, 8, 16, 2>(x, native, M, K, N, ep, stream);
-    if (Nb >= 512) return launch_stream<2, 8, 16, 2>(x, native, M, K, N, ep, stream);
-    return launch_stream<1, 8, 16, 2>(x, native, M, K, N, ep, stream);
+    if (Nb <= 256) return launch_stream<1, 8, 16, 2>(x, native, M, K, N, ep, stream);
+    if (Nb <= 512) return launch_stream<2, 8, 16, 2>(x, native, M, K, N, ep, stream);
+    if (Nb <= 1024) return launch_stream<4, 8, 16, 2>(x, native, M, K, N, ep, stream);
+    return launch_stream<4, 4, 16, 2>(x, native, M, K, N, ep, stream);
 }
 
 bool mid_conv_ok(const void *x, const tmq_conv_shape *s) {
