@@ -266,6 +266,19 @@ def _gemv_floor_and_large(args, torch, natives):
     floor = _graph_time_us(torch, run, max(2, args.steps // 12), args.settle_ms)
     res["gemv_16384"] = {"us": round(us, 3), "gbs": round(byts / us / 1e3, 1), "frac_hbm": round(byts / us / 1e3 / HBM_PEAK_GBS, 4),
                          "read_floor_us": round(floor, 3), "read_floor_gbs": round(K * N / 4 / floor / 1e3, 1)}
+    # the same layer against 4 and 16 rows (batched decoding): the weights are still read once
+    for rows in (4, 16):
+        xr = torch.randn(rows, K, device=dev).half()
+
+        def few(xr=xr):
+            for nw in big:
+                ops.ternary_linear(xr, nw, scale)
+            return len(big)
+        few()
+        us = _graph_time_us(torch, few, max(2, args.steps // 12), args.settle_ms)
+        byts = K * N / 4 + 2 * rows * K + 4 * N + 4 * rows * N
+        res["rows%d_16384" % rows] = {"us": round(us, 3), "gbs": round(byts / us / 1e3, 1),
+                                      "frac_hbm": round(byts / us / 1e3 / HBM_PEAK_GBS, 4)}
     return res
 
 
