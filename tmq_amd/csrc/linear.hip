@@ -1,13 +1,18 @@
 // Ternary linear layers on gfx950: y[m][n] = scale[n] * sum_k x[m][k] * T[k][n] + bias[n].
 //
-//   prepack_kernel : reference packing words[K][ceil(N/16)] -> kernel-native blocks (mfma.h)
-//   skinny_kernel  : M <= 64 (GEMV and small batches). Bound by streaming the 2-bit weights:
-//                    every wavefront fetches 1 KiB weight blocks with one coalesced dwordx4 load,
-//                    expands them in registers to exact +-2/0 fp16 MFMA operands (two VALU ops
-//                    per register), and contracts with the activations on
-//                    v_mfma_f32_16x16x32_f16 (fp32 accumulate). K is split over the wavefronts
-//                    of a workgroup and reduced through LDS in a fixed order (deterministic).
-//   The MFMA-bound large-M kernel lives in gemm.hip.
+//   prepack_kernel    : reference packing words[K][ceil(N/16)] -> kernel-native blocks (mfma.h)
+//   skinny_kernel     : M <= 64 rows of any shape and type (fp32 activations, ragged K, unaligned rows).
+//                       Bound by streaming the 2-bit weights: every wavefront fetches 1 KiB weight blocks
+//                       with one coalesced dwordx4 load, expands them in registers to exact +-2/0 fp16
+//                       MFMA operands (two VALU ops per register), and contracts with the activations on
+//                       v_mfma_f32_16x16x32_f16 (fp32 accumulate). K is split over the wavefronts of a
+//                       workgroup and reduced through LDS in a fixed order (deterministic).
+//   gemv_short_kernel, short_rows_kernel : M = 1 / 2..16 fp16 rows with K < 2048: everything in flight at once
+//   mid_kernel, mid_lds_kernel : older split-reduction kernels, kept for what mid.hip does not take
+//                       (K % 64 != 0, unaligned rows, fp32 activations)
+//   split_terms_kernel : fp32 -> two fp16 terms, for the two-pass route of fp32 activations
+//   tmq_ternary_linear : the dispatch. fp16 rows with whole blocks go to mid.hip (weight-stream kernel up to
+//                       16 rows, split-reduction kernel for few output tiles) or gemm.hip (MFMA-bound tiles).
 #include "common.h"
 #include "mfma.h"
 
@@ -1146,16 +1151,16 @@ int tmq_ternary_linear(const void *x, int x_dtype, int64_t M, int64_t K, const v
     if (epilogue) ep = *epilogue;
     if (ep.y_dtype != TMQ_F16 && ep.y_dtype != TMQ_F32) return TMQ_ERR_UNSUPPORTED;
     const bool x32 = x_dtype == TMQ_F32;
-    // Up to 16 rows the weight-streaming kernel (activations staged in LDS). It also takes 17 .. 64
-    // rows when K is ragged or the rows are unaligned; with whole 256-index blocks the split-reduction
-    // kernels are as fast at K = 4096 and two to three times faster at short K, where staging all of
-    // x in every workgroup dominates (M = 64, K = 512: 11.2 -> 4.6 us; fp32 input at K = 4096: 33 -> 14 us).
-    const bool blocks_ok = (K % kKB == 0) && aligned16(x);
     // At most 16 fp16 rows against eight or more weight blocks per channel: the weight-stream kernel (mid.hip).
     // Against the kernels below: M = 16 at 16384^2 67 -> 20 us, M = 8 at 8192 x 28672 34 -> 17 us, M = 1 at
     // 11008 x 4096 7.2 -> 6.2 us, even at 4096^2.
     if (!x32 && stream_dense_ok(x, M, K) && K >= 8 * kKB)
         return launch_stream_dense(x, M, K, native, N, ep.scale, ep.bias, ep.residual, ep.relu, y, ep.y_dtype == TMQ_F16, stream);
+    // Otherwise up to 16 rows take the skinny kernels (activations staged in LDS). They also take 17 .. 64
+    // rows when K is ragged or the rows are unaligned; with whole 256-index blocks the split-reduction
+    // kernels are as fast at K = 4096 and two to three times faster at short K, where staging all of
+    // x in every workgroup dominates (M = 64, K = 512: 11.2 -> 4.6 us; fp32 input at K = 4096: 33 -> 14 us).
+    const bool blocks_ok = (K % kKB == 0) && aligned16(x);
     if (M <= 16 || (M <= 64 && !blocks_ok))
         return x32 ? skinny_rows<true>(x, M, K, native, N, ep, y, stream)
                    : skinny_rows<false>(x, M, K, native, N, ep, y, stream);
