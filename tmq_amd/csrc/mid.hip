@@ -292,6 +292,9 @@ __global__ __launch_bounds__(64 * WAVES) void mid_kernel(Rows rows, const u32x4 
 #pragma unroll
                     for (int mi = 0; mi < WM; mi++) acc[mi][nj] = mfma16(w, a[s][mi], acc[mi][nj]);
                 }
+            // keeps the next pair's wait below these multiplications: hoisted above them it would make
+            // them wait for the loads just issued
+            __builtin_amdgcn_sched_barrier(0);
         };
         int p = 0;
         for (; p + 2 <= np; p += 2) {
