@@ -377,7 +377,7 @@ struct StreamRows {
     }
 };
 
-template <int WN, int WAVES, int R, int D>
+template <int WN, int WAVES, int R, int D, bool LONG>
 __global__ __launch_bounds__(64 * WAVES) void stream_kernel(const _Float16 *__restrict__ x, const u32x4 *__restrict__ native,
                                                             int64_t M, int64_t K, int Kb, int64_t N, int64_t Nb,
                                                             MidEpilogue ep) {
@@ -434,17 +434,19 @@ __global__ __launch_bounds__(64 * WAVES) void stream_kernel(const _Float16 *__re
 
     if (nt > 0) {
         u32x4 wq[D][WN];
-#pragma unroll
-        for (int d = 0; d < D; d++)
-            if (d < nt) {
-                fill(d, d);
-                wload(wq[d], d);
-            }
-        // one block; `par` (static) = t % D = LDS slot and weight register set of the block
-        auto step = [&](int t, auto par_tag) {
+        // one block; `par` (static) = t % D = LDS slot and weight register set of the block. In the steady
+        // state every step refills unconditionally, so the number of loads behind the one being waited for
+        // is a constant -- for the wait below and for the waits the compiler adds before it lets the
+        // weight registers be used (with a conditional refill it can only wait for everything).
+        auto step = [&](int t, auto par_tag, auto steady_tag) {
             constexpr int par = decltype(par_tag)::value;
-            const int ahead = nt - 1 - t;                         // blocks issued after this one
-            wait_blocks(ahead < D - 1 ? ahead : D - 1);
+            constexpr bool kSteady = decltype(steady_tag)::value;
+            if constexpr (kSteady) {
+                wait_blocks(D - 1);
+            } else {
+                const int ahead = nt - 1 - t;                     // blocks issued after this one
+                wait_blocks(ahead < D - 1 ? ahead : D - 1);
+            }
             __builtin_amdgcn_sched_barrier(0);
             half8 a[8];                                            // all operand reads of the block
 #pragma unroll
@@ -452,7 +454,7 @@ __global__ __launch_bounds__(64 * WAVES) void stream_kernel(const _Float16 *__re
             // the slot is free again once the reads have returned: refill it with the block D ahead
             __builtin_amdgcn_s_waitcnt(0xC07F);                    // lgkmcnt(0)
             __builtin_amdgcn_sched_barrier(0);
-            if (t + D < nt) fill(par, t + D);
+            if (kSteady || t + D < nt) fill(par, t + D);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int i = 0; i < 8; i++)
@@ -460,19 +462,43 @@ __global__ __launch_bounds__(64 * WAVES) void stream_kernel(const _Float16 *__re
                 for (int nj = 0; nj < WN; nj++)
                     acc[0][nj] = mfma16(decode_step(wq[par][nj][i >> 1], i & 1), a[i], acc[0][nj]);
             __builtin_amdgcn_sched_barrier(0);
-            if (t + D < nt) wload(wq[par], t + D);
+            if (kSteady || t + D < nt) wload(wq[par], t + D);
             __builtin_amdgcn_sched_barrier(0);
         };
+        auto round = [&](int t, auto steady_tag) {
+            step(t, std::integral_constant<int, 0>{}, steady_tag);
+            if constexpr (D > 1) step(t + 1, std::integral_constant<int, 1>{}, steady_tag);
+            if constexpr (D > 2) step(t + 2, std::integral_constant<int, 2>{}, steady_tag);
+            if constexpr (D > 3) step(t + 3, std::integral_constant<int, 3>{}, steady_tag);
+        };
         int t = 0;
-        for (; t + D <= nt; t += D) {
-            step(t, std::integral_constant<int, 0>{});
-            if constexpr (D > 1) step(t + 1, std::integral_constant<int, 1>{});
-            if constexpr (D > 2) step(t + 2, std::integral_constant<int, 2>{});
-            if constexpr (D > 3) step(t + 3, std::integral_constant<int, 3>{});
+        if constexpr (LONG) {
+            // every wavefront has at least 2 D blocks (the host checks): an unconditional prologue and at
+            // least one steady round, entered from one known sequence of outstanding loads
+#pragma unroll
+            for (int d = 0; d < D; d++) {
+                fill(d, d);
+                wload(wq[d], d);
+                __builtin_amdgcn_sched_barrier(0);                // the order of issue the waits count on
+            }
+            do {
+                round(t, std::true_type{});
+                t += D;
+            } while (t + 2 * D <= nt);
+        } else {
+#pragma unroll
+            for (int d = 0; d < D; d++)
+                if (d < nt) {
+                    fill(d, d);
+                    wload(wq[d], d);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
         }
-        if (t < nt) step(t, std::integral_constant<int, 0>{});
-        if constexpr (D > 2) if (t + 1 < nt) step(t + 1, std::integral_constant<int, 1>{});
-        if constexpr (D > 3) if (t + 2 < nt) step(t + 2, std::integral_constant<int, 2>{});
+        // drain: at most 2 D - 1 blocks with wave-uniform guards
+        for (; t + D <= nt; t += D) round(t, std::false_type{});
+        if (t < nt) step(t, std::integral_constant<int, 0>{}, std::false_type{});
+        if constexpr (D > 2) if (t + 1 < nt) step(t + 1, std::integral_constant<int, 1>{}, std::false_type{});
+        if constexpr (D > 3) if (t + 2 < nt) step(t + 2, std::integral_constant<int, 2>{}, std::false_type{});
     }
     reduce_and_store<1, WN, WAVES>(smem, acc, kg, lane, 0, n0, M, N, ep);
 }
@@ -484,7 +510,12 @@ int launch_stream(const void *x, const void *native, int64_t M, int64_t K, int64
     constexpr size_t win = (size_t)WAVES * D * R * 512, redb = (size_t)WAVES * WN * (1024 + 64);
     constexpr size_t lds = win > redb ? win : redb;
     static_assert(lds <= 152 * 1024, "LDS budget");
-    auto kernel = stream_kernel<WN, WAVES, R, D>;
+    // the variant with a steady-state loop needs 2 D blocks in every wavefront; with fewer, half the depth
+    // and a steady state beats the full depth without one
+    if constexpr (D == 4) {
+        if (Kb / WAVES < 2 * D && Kb / WAVES >= D) return launch_stream<WN, WAVES, R, 2>(x, native, M, K, N, ep, stream);
+    }
+    auto kernel = Kb / WAVES >= 2 * D ? stream_kernel<WN, WAVES, R, D, true> : stream_kernel<WN, WAVES, R, D, false>;
     if (lds > 64 * 1024) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
