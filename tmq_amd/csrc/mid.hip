@@ -377,8 +377,18 @@ struct StreamRows {
     }
 };
 
+// Wavefronts per SIMD the LDS windows leave room for: the register budget the compiler has to keep to.
+constexpr int stream_waves_per_simd(int WN, int WAVES, int R, int D) {
+    const int win = WAVES * D * R * 512, redb = WAVES * WN * (1024 + 64), lds = win > redb ? win : redb;
+    int wgs = (160 * 1024) / lds;
+    if (wgs > 32 / WAVES) wgs = 32 / WAVES;
+    if (wgs < 1) wgs = 1;
+    const int w = wgs * WAVES / 4;
+    return w < 1 ? 1 : (w > 4 ? 4 : w);
+}
+
 template <int WN, int WAVES, int R, int D, bool LONG>
-__global__ __launch_bounds__(64 * WAVES) void stream_kernel(const _Float16 *__restrict__ x, const u32x4 *__restrict__ native,
+__global__ __launch_bounds__(64 * WAVES, stream_waves_per_simd(WN, WAVES, R, D)) void stream_kernel(const _Float16 *__restrict__ x, const u32x4 *__restrict__ native,
                                                             int64_t M, int64_t K, int Kb, int64_t N, int64_t Nb,
                                                             MidEpilogue ep) {
     using Rows = StreamRows<R>;
@@ -422,83 +432,189 @@ __global__ __launch_bounds__(64 * WAVES) void stream_kernel(const _Float16 *__re
 #pragma unroll
         for (int i = 0; i < kLoads; i++) load_to_lds(xb + src[i], win + slot * kSlot + i * 1024);
     };
-    // wait until at most n blocks' loads are outstanding (loads complete in issue order)
-    auto wait_blocks = [&](int n) {
-        static_assert(D <= 4, "cases below");
-        constexpr auto enc = [](int c) { return (c & 15) | (7 << 4) | (15 << 8) | ((c >> 4) << 14); };
-        if (n >= 3 && D > 3) __builtin_amdgcn_s_waitcnt(enc(3 * kPerBlock));
-        else if (n == 2 && D > 2) __builtin_amdgcn_s_waitcnt(enc(2 * kPerBlock));
-        else if (n == 1) __builtin_amdgcn_s_waitcnt(enc(kPerBlock));
-        else __builtin_amdgcn_s_waitcnt(enc(0));
-    };
-
-    if (nt > 0) {
+    if constexpr (R == 16) {
+        // One block out of slot / register set PAR with at most BEHIND younger blocks still on their way (loads
+        // complete in issue order), refilling the slot with block t + D if REFILL. Everything about the pipeline
+        // state is a template argument: the wait below is exact, and so are the waits the compiler adds before it
+        // lets the weight registers be used -- after a conditional refill it could only wait for everything.
         u32x4 wq[D][WN];
-        // one block; `par` (static) = t % D = LDS slot and weight register set of the block. In the steady
-        // state every step refills unconditionally, so the number of loads behind the one being waited for
-        // is a constant -- for the wait below and for the waits the compiler adds before it lets the
-        // weight registers be used (with a conditional refill it can only wait for everything).
-        auto step = [&](int t, auto par_tag, auto steady_tag) {
-            constexpr int par = decltype(par_tag)::value;
-            constexpr bool kSteady = decltype(steady_tag)::value;
-            if constexpr (kSteady) {
-                wait_blocks(D - 1);
-            } else {
-                const int ahead = nt - 1 - t;                     // blocks issued after this one
-                wait_blocks(ahead < D - 1 ? ahead : D - 1);
-            }
+        auto step = [&](int t, auto par_tag, auto behind_tag, auto refill_tag) {
+            constexpr int PAR = decltype(par_tag)::value, BEHIND = decltype(behind_tag)::value;
+            constexpr bool REFILL = decltype(refill_tag)::value;
+            static_assert(BEHIND >= 0 && BEHIND < D && BEHIND * kPerBlock < 64, "vmcnt is a 6-bit counter");
+            constexpr int kCount = BEHIND * kPerBlock;
+            __builtin_amdgcn_s_waitcnt((kCount & 15) | (7 << 4) | (15 << 8) | ((kCount >> 4) << 14));   // vmcnt(kCount)
             __builtin_amdgcn_sched_barrier(0);
-            half8 a[8];                                            // all operand reads of the block
+            half8 a[8];                                                // all operand reads of the block
 #pragma unroll
-            for (int i = 0; i < 8; i++) a[i] = *reinterpret_cast<const half8 *>(win + par * kSlot + rd[i]);
-            // the slot is free again once the reads have returned: refill it with the block D ahead
-            __builtin_amdgcn_s_waitcnt(0xC07F);                    // lgkmcnt(0)
+            for (int i = 0; i < 8; i++) a[i] = *reinterpret_cast<const half8 *>(win + PAR * kSlot + rd[i]);
+            // the slot is free again once the reads have returned
+            __builtin_amdgcn_s_waitcnt(0xC07F);                        // lgkmcnt(0)
             __builtin_amdgcn_sched_barrier(0);
-            if (kSteady || t + D < nt) fill(par, t + D);
+            if constexpr (REFILL) fill(PAR, t + D);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int i = 0; i < 8; i++)
 #pragma unroll
                 for (int nj = 0; nj < WN; nj++)
-                    acc[0][nj] = mfma16(decode_step(wq[par][nj][i >> 1], i & 1), a[i], acc[0][nj]);
+                    acc[0][nj] = mfma16(decode_step(wq[PAR][nj][i >> 1], i & 1), a[i], acc[0][nj]);
             __builtin_amdgcn_sched_barrier(0);
-            if (kSteady || t + D < nt) wload(wq[par], t + D);
+            if constexpr (REFILL) wload(wq[PAR], t + D);
             __builtin_amdgcn_sched_barrier(0);
         };
-        auto round = [&](int t, auto steady_tag) {
-            step(t, std::integral_constant<int, 0>{}, steady_tag);
-            if constexpr (D > 1) step(t + 1, std::integral_constant<int, 1>{}, steady_tag);
-            if constexpr (D > 2) step(t + 2, std::integral_constant<int, 2>{}, steady_tag);
-            if constexpr (D > 3) step(t + 3, std::integral_constant<int, 3>{}, steady_tag);
-        };
-        int t = 0;
-        if constexpr (LONG) {
-            // every wavefront has at least 2 D blocks (the host checks): an unconditional prologue and at
-            // least one steady round, entered from one known sequence of outstanding loads
+        // the first COUNT blocks, in the order the waits count on
+        auto prologue = [&](auto count_tag) {
+            constexpr int COUNT = decltype(count_tag)::value;
 #pragma unroll
-            for (int d = 0; d < D; d++) {
+            for (int d = 0; d < COUNT; d++) {
                 fill(d, d);
                 wload(wq[d], d);
-                __builtin_amdgcn_sched_barrier(0);                // the order of issue the waits count on
+                __builtin_amdgcn_sched_barrier(0);
             }
-            do {
-                round(t, std::true_type{});
+        };
+        // the last D + REM blocks (t a multiple of D, blocks t .. t + D - 1 in flight): D steps of which the first
+        // REM still refill, then REM steps
+        auto drain = [&](int t, auto rem_tag) {
+            constexpr int REM = decltype(rem_tag)::value;
+            auto first = [&](auto j_tag) {
+                constexpr int J = decltype(j_tag)::value;
+                if constexpr (J < D)
+                    step(t + J, j_tag, std::integral_constant<int, D - 1 - J + (J < REM ? J : REM)>{}, std::bool_constant<(J < REM)>{});
+            };
+            first(std::integral_constant<int, 0>{});
+            first(std::integral_constant<int, 1>{});
+            first(std::integral_constant<int, 2>{});
+            first(std::integral_constant<int, 3>{});
+            auto second = [&](auto j_tag) {
+                constexpr int J = decltype(j_tag)::value;
+                if constexpr (J < REM) step(t + D + J, j_tag, std::integral_constant<int, REM - 1 - J>{}, std::false_type{});
+            };
+            second(std::integral_constant<int, 0>{});
+            second(std::integral_constant<int, 1>{});
+            second(std::integral_constant<int, 2>{});
+        };
+        // fewer than D blocks in all: everything in flight at once
+        auto few = [&](auto nt_tag) {
+            constexpr int NT = decltype(nt_tag)::value;
+            if constexpr (NT < D) {
+                prologue(nt_tag);
+                auto one = [&](auto j_tag) {
+                    constexpr int J = decltype(j_tag)::value;
+                    if constexpr (J < NT) step(J, j_tag, std::integral_constant<int, NT - 1 - J>{}, std::false_type{});
+                };
+                one(std::integral_constant<int, 0>{});
+                one(std::integral_constant<int, 1>{});
+                one(std::integral_constant<int, 2>{});
+            }
+        };
+        static_assert(D >= 1 && D <= 4, "cases below");
+
+        if (nt >= D) {
+            prologue(std::integral_constant<int, D>{});
+            int t = 0;
+            while (t + 2 * D <= nt) {                                  // steady state: D - 1 blocks behind, always refill
+                step(t, std::integral_constant<int, 0>{}, std::integral_constant<int, D - 1>{}, std::true_type{});
+                if constexpr (D > 1) step(t + 1, std::integral_constant<int, 1>{}, std::integral_constant<int, D - 1>{}, std::true_type{});
+                if constexpr (D > 2) step(t + 2, std::integral_constant<int, 2>{}, std::integral_constant<int, D - 1>{}, std::true_type{});
+                if constexpr (D > 3) step(t + 3, std::integral_constant<int, 3>{}, std::integral_constant<int, D - 1>{}, std::true_type{});
                 t += D;
-            } while (t + 2 * D <= nt);
+            }
+            switch (nt - t - D) {                                      // 0 .. D - 1 blocks not yet requested
+                case 0: drain(t, std::integral_constant<int, 0>{}); break;
+                case 1: if constexpr (D > 1) drain(t, std::integral_constant<int, 1>{}); break;
+                case 2: if constexpr (D > 2) drain(t, std::integral_constant<int, 2>{}); break;
+                default: if constexpr (D > 3) drain(t, std::integral_constant<int, 3>{}); break;
+            }
         } else {
+            switch (nt) {
+                case 1: few(std::integral_constant<int, 1>{}); break;
+                case 2: few(std::integral_constant<int, 2>{}); break;
+                case 3: few(std::integral_constant<int, 3>{}); break;
+                default: break;
+            }
+        }
+    } else {
+        // Fewer than 16 rows: several workgroups share a CU, and the fully static pipeline above costs the
+        // registers that residency depends on (measured slower). Here only the steady state is static (template
+        // argument LONG: every wavefront has at least 2 D blocks) and the drain works with guards.
+        // wait until at most n blocks' loads are outstanding (loads complete in issue order)
+        auto wait_blocks = [&](int n) {
+            static_assert(D <= 4, "cases below");
+            constexpr auto enc = [](int c) { return (c & 15) | (7 << 4) | (15 << 8) | ((c >> 4) << 14); };
+            if (n >= 3 && D > 3) __builtin_amdgcn_s_waitcnt(enc(3 * kPerBlock));
+            else if (n == 2 && D > 2) __builtin_amdgcn_s_waitcnt(enc(2 * kPerBlock));
+            else if (n == 1) __builtin_amdgcn_s_waitcnt(enc(kPerBlock));
+            else __builtin_amdgcn_s_waitcnt(enc(0));
+        };
+
+        if (nt > 0) {
+            u32x4 wq[D][WN];
+            // one block; `par` (static) = t % D = LDS slot and weight register set of the block. In the steady
+            // state every step refills unconditionally, so the number of loads behind the one being waited for
+            // is a constant -- for the wait below and for the waits the compiler adds before it lets the
+            // weight registers be used (with a conditional refill it can only wait for everything).
+            auto step = [&](int t, auto par_tag, auto steady_tag) {
+                constexpr int par = decltype(par_tag)::value;
+                constexpr bool kSteady = decltype(steady_tag)::value;
+                if constexpr (kSteady) {
+                    wait_blocks(D - 1);
+                } else {
+                    const int ahead = nt - 1 - t;                     // blocks issued after this one
+                    wait_blocks(ahead < D - 1 ? ahead : D - 1);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                half8 a[8];                                            // all operand reads of the block
 #pragma unroll
-            for (int d = 0; d < D; d++)
-                if (d < nt) {
+                for (int i = 0; i < 8; i++) a[i] = *reinterpret_cast<const half8 *>(win + par * kSlot + rd[i]);
+                // the slot is free again once the reads have returned: refill it with the block D ahead
+                __builtin_amdgcn_s_waitcnt(0xC07F);                    // lgkmcnt(0)
+                __builtin_amdgcn_sched_barrier(0);
+                if (kSteady || t + D < nt) fill(par, t + D);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int i = 0; i < 8; i++)
+#pragma unroll
+                    for (int nj = 0; nj < WN; nj++)
+                        acc[0][nj] = mfma16(decode_step(wq[par][nj][i >> 1], i & 1), a[i], acc[0][nj]);
+                __builtin_amdgcn_sched_barrier(0);
+                if (kSteady || t + D < nt) wload(wq[par], t + D);
+                __builtin_amdgcn_sched_barrier(0);
+            };
+            auto round = [&](int t, auto steady_tag) {
+                step(t, std::integral_constant<int, 0>{}, steady_tag);
+                if constexpr (D > 1) step(t + 1, std::integral_constant<int, 1>{}, steady_tag);
+                if constexpr (D > 2) step(t + 2, std::integral_constant<int, 2>{}, steady_tag);
+                if constexpr (D > 3) step(t + 3, std::integral_constant<int, 3>{}, steady_tag);
+            };
+            int t = 0;
+            if constexpr (LONG) {
+                // every wavefront has at least 2 D blocks (the host checks): an unconditional prologue and at
+                // least one steady round, entered from one known sequence of outstanding loads
+#pragma unroll
+                for (int d = 0; d < D; d++) {
                     fill(d, d);
                     wload(wq[d], d);
-                    __builtin_amdgcn_sched_barrier(0);
+                    __builtin_amdgcn_sched_barrier(0);                // the order of issue the waits count on
                 }
+                do {
+                    round(t, std::true_type{});
+                    t += D;
+                } while (t + 2 * D <= nt);
+            } else {
+#pragma unroll
+                for (int d = 0; d < D; d++)
+                    if (d < nt) {
+                        fill(d, d);
+                        wload(wq[d], d);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+            }
+            // drain: at most 2 D - 1 blocks with wave-uniform guards
+            for (; t + D <= nt; t += D) round(t, std::false_type{});
+            if (t < nt) step(t, std::integral_constant<int, 0>{}, std::false_type{});
+            if constexpr (D > 2) if (t + 1 < nt) step(t + 1, std::integral_constant<int, 1>{}, std::false_type{});
+            if constexpr (D > 3) if (t + 2 < nt) step(t + 2, std::integral_constant<int, 2>{}, std::false_type{});
         }
-        // drain: at most 2 D - 1 blocks with wave-uniform guards
-        for (; t + D <= nt; t += D) round(t, std::false_type{});
-        if (t < nt) step(t, std::integral_constant<int, 0>{}, std::false_type{});
-        if constexpr (D > 2) if (t + 1 < nt) step(t + 1, std::integral_constant<int, 1>{}, std::false_type{});
-        if constexpr (D > 3) if (t + 2 < nt) step(t + 2, std::integral_constant<int, 2>{}, std::false_type{});
     }
     reduce_and_store<1, WN, WAVES>(smem, acc, kg, lane, 0, n0, M, N, ep);
 }
@@ -515,7 +631,7 @@ int launch_stream(const void *x, const void *native, int64_t M, int64_t K, int64
     if constexpr (D == 4) {
         if (Kb / WAVES < 2 * D && Kb / WAVES >= D) return launch_stream<WN, WAVES, R, 2>(x, native, M, K, N, ep, stream);
     }
-    auto kernel = Kb / WAVES >= 2 * D ? stream_kernel<WN, WAVES, R, D, true> : stream_kernel<WN, WAVES, R, D, false>;
+    auto kernel = R != 16 && Kb / WAVES >= 2 * D ? stream_kernel<WN, WAVES, R, D, true> : stream_kernel<WN, WAVES, R, D, false>;
     if (lds > 64 * 1024) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
