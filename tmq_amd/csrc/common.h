@@ -31,6 +31,29 @@ inline bool split_reduction_pays(int64_t M, int64_t K, int64_t N) {
     return K >= 512 ? tiles64 <= 640 : tiles64 <= K / 2;
 }
 
+// Division of 0 <= n < 2^31 by a divisor known on the host (an image extent): q = umulhi(n, mul) >> shift,
+// two instructions instead of the ~25 of a 32-bit division. With s = ceil(log2 d) and mul = ceil(2^(31 + s) / d)
+// (< 2^32), n mul / 2^(31 + s) exceeds n / d by less than 2^-s <= 1 / d, so the floor is the same.
+struct FastDiv {
+    uint32_t mul, shift, d;
+    FastDiv() : mul(0), shift(0), d(1) {}
+    explicit FastDiv(uint32_t div) : mul(0), shift(0), d(div) {
+        if (div > 1) {
+            uint32_t s = 0;
+            while ((uint64_t(1) << s) < div) s++;
+            mul = (uint32_t)(((uint64_t(1) << (31 + s)) + div - 1) / div);
+            shift = s - 1;
+        }
+    }
+#if defined(__HIPCC__)
+    __device__ __forceinline__ uint32_t divmod(uint32_t n, int &rem) const {
+        const uint32_t q = d > 1 ? __umulhi(n, mul) >> shift : n;
+        rem = (int)(n - q * d);
+        return q;
+    }
+#endif
+};
+
 #if defined(__HIPCC__)
 // a / b and a % b for 0 <= a, 0 < b. The GPU has no integer divider: a 64-bit division expands to
 // ~100 instructions, a 32-bit one to ~20, and index arithmetic (pixel -> batch, row, column) sits in

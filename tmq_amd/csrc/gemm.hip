@@ -203,6 +203,7 @@ struct ConvLoader64 {
     const _Float16 *x;
     int64_t M, K;
     int B, C, H, W, Ho, Wo, ky, kx, sy, sx, py, px, dy, dx;
+    FastDiv by_wo, by_ho;      // set by with_divisors(); M < 2^31
 
     template <int CH, int T>
     struct State {
@@ -223,8 +224,8 @@ struct ConvLoader64 {
             st.ih0[q] = st.iw0[q] = INT32_MIN / 2;
             if (m < M) {
                 int ow, oh;
-                const int64_t t = div_rem(m, Wo, ow);
-                const int b = (int)div_rem(t, Ho, oh);
+                const uint32_t t = by_wo.divmod((uint32_t)m, ow);
+                const int b = (int)by_ho.divmod(t, oh);
                 st.ih0[q] = oh * sy - py;
                 st.iw0[q] = ow * sx - px;
                 st.off0[q] = ((b * H + st.ih0[q]) * W + st.iw0[q]) * C + kc;
@@ -257,6 +258,7 @@ struct ConvLoaderFewC {
     const _Float16 *x;
     int64_t M, K;
     int B, C, H, W, Ho, Wo, ky, kx, sy, sx, py, px, dy, dx;
+    FastDiv by_wo, by_ho;      // set by with_divisors(); M < 2^31
 
     template <int CH, int T>
     struct State {
@@ -276,8 +278,8 @@ struct ConvLoaderFewC {
             st.ih0[q] = st.iw0[q] = INT32_MIN / 2;
             if (m < M) {
                 int ow, oh;
-                const int64_t t = div_rem(m, Wo, ow);
-                const int b = (int)div_rem(t, Ho, oh);
+                const uint32_t t = by_wo.divmod((uint32_t)m, ow);
+                const int b = (int)by_ho.divmod(t, oh);
                 st.ih0[q] = oh * sy - py;
                 st.iw0[q] = ow * sx - px;
                 st.off0[q] = ((b * H + st.ih0[q]) * W + st.iw0[q]) * C + kc % C;
@@ -614,6 +616,13 @@ int launch_tile(const Loader &ld, const void *native, int64_t M, int64_t K, int6
 // shapes): 128 x 256 once it gives 1.5 workgroups per CU, 128 x 128 down to one per CU, else
 // 64 x 64. Larger tiles (256 x 256, 256 x 128) and 128 x 64 never won.
 template <class Loader>
+Loader with_divisors(Loader ld) {
+    ld.by_wo = FastDiv((uint32_t)ld.Wo);
+    ld.by_ho = FastDiv((uint32_t)ld.Ho);
+    return ld;
+}
+
+template <class Loader>
 int dispatch_tile(const Loader &ld, const void *native, int64_t M, int64_t K, int64_t N, const Epilogue &ep,
                   void *stream) {
     auto wgs = [&](int bm, int bn) { return ((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
@@ -693,14 +702,13 @@ int tmq_ternary_conv2d(const void *x, const tmq_conv_shape *s, const void *nativ
     // few output tiles: split the reduction inside the workgroup (mid.hip)
     if (mid_conv_ok(x, s) && split_reduction_pays(M, K, s->N))
         return launch_mid_conv(x, s, ho, wo, native, scale, bias, residual, relu, y, y_dtype == TMQ_F16 ? 1 : 0, stream);
-    if ((s->C % kBK == 0) && aligned16(x) &&
-        (int64_t)s->B * s->H * s->W * s->C < (int64_t)0x7FFFFFFF)
-        return dispatch_tile(ConvLoader64{xp, M, K, s->B, s->C, s->H, s->W, ho, wo, s->ky, s->kx, s->sy, s->sx, s->py,
-                                          s->px, s->dy, s->dx}, native, M, K, s->N, ep, stream);
-    if ((s->C == 8 || s->C == 16 || s->C == 32) && aligned16(x) &&
-        (int64_t)s->B * s->H * s->W * s->C < (int64_t)0x7FFFFFFF)
-        return dispatch_tile(ConvLoaderFewC{xp, M, K, s->B, s->C, s->H, s->W, ho, wo, s->ky, s->kx, s->sy, s->sx, s->py,
-                                            s->px, s->dy, s->dx}, native, M, K, s->N, ep, stream);
+    const bool small = (int64_t)s->B * s->H * s->W * s->C < (int64_t)0x7FFFFFFF && M < (int64_t)0x7FFFFFFF;   // 32-bit offsets and rows
+    if ((s->C % kBK == 0) && aligned16(x) && small)
+        return dispatch_tile(with_divisors(ConvLoader64{xp, M, K, s->B, s->C, s->H, s->W, ho, wo, s->ky, s->kx, s->sy,
+                                                        s->sx, s->py, s->px, s->dy, s->dx, {}, {}}), native, M, K, s->N, ep, stream);
+    if ((s->C == 8 || s->C == 16 || s->C == 32) && aligned16(x) && small)
+        return dispatch_tile(with_divisors(ConvLoaderFewC{xp, M, K, s->B, s->C, s->H, s->W, ho, wo, s->ky, s->kx, s->sy,
+                                                          s->sx, s->py, s->px, s->dy, s->dx, {}, {}}), native, M, K, s->N, ep, stream);
     if ((s->C % 8 == 0) && aligned16(x))
         return dispatch_tile(ConvLoader<true>{xp, M, K, s->B, s->C, s->H, s->W, ho, wo, s->ky, s->kx, s->sy, s->sx,
                                               s->py, s->px, s->dy, s->dx}, native, M, K, s->N, ep, stream);

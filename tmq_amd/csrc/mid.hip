@@ -77,6 +77,7 @@ struct ConvRows {
     const _Float16 *x;
     int64_t M, K;
     int B, C, H, W, Ho, Wo, ky, kx, sy, sx, py, px, dy, dx;
+    FastDiv by_wo, by_ho;      // M < 2^31
 
     template <int WM>
     struct State {
@@ -93,8 +94,8 @@ struct ConvRows {
                 int64_t m = m0 + mi * 16 + R;
                 if (m >= M) m = M - 1;
                 int ow, oh;
-                const int64_t t = div_rem(m, Wo, ow);
-                const int b = (int)div_rem(t, Ho, oh);
+                const uint32_t t = by_wo.divmod((uint32_t)m, ow);
+                const int b = (int)by_ho.divmod(t, oh);
                 st.ih0[mi][c] = oh * sy - py;
                 st.iw0[mi][c] = ow * sx - px;
                 st.off[mi][c] = ((b * H + st.ih0[mi][c]) * W + st.iw0[mi][c]) * C + (((lane & 7) ^ ((R >> 1) & 7)) * 8);
@@ -739,7 +740,8 @@ int launch_mid_conv(const void *x, const tmq_conv_shape *s, int ho, int wo, cons
     const int64_t M = (int64_t)s->B * ho * wo, K = (int64_t)s->C * s->ky * s->kx;
     MidEpilogue ep{scale, bias, residual, y, relu, y_f16};
     return dispatch(ConvRows{static_cast<const _Float16 *>(x), M, K, s->B, s->C, s->H, s->W, ho, wo, s->ky, s->kx, s->sy,
-                             s->sx, s->py, s->px, s->dy, s->dx}, native, M, K, s->N, ep, stream);
+                             s->sx, s->py, s->px, s->dy, s->dx, FastDiv((uint32_t)wo), FastDiv((uint32_t)ho)},
+                    native, M, K, s->N, ep, stream);
 }
 
 }  // namespace tmq
