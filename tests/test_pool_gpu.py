@@ -7,7 +7,8 @@ pytestmark = pytest.mark.gpu
 
 
 @pytest.mark.parametrize("B,C,H,W,k,s,p", [(2, 64, 112, 112, 3, 2, 1), (1, 8, 7, 9, 2, 2, 0), (3, 40, 13, 11, (3, 2), (2, 1), (1, 1)),
-                                           (2, 5, 9, 9, 3, 1, 1), (1, 16, 6, 6, 3, 3, 0), (2, 24, 5, 5, 5, 1, 2)])
+                                           (2, 5, 9, 9, 3, 1, 1), (1, 16, 6, 6, 3, 3, 0), (2, 24, 5, 5, 5, 1, 2),
+                                           (2, 8, 5, 7, 3, 1, 1), (1, 24, 3, 3, 3, 2, 1), (3, 16, 2, 9, 3, (1, 2), 1)])
 def test_maxpool_equals_torch(cuda, B, C, H, W, k, s, p):
     from tmq_amd import ops
     g = torch.Generator(device=cuda).manual_seed(B + C + H)

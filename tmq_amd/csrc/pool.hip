@@ -53,6 +53,39 @@ __global__ __launch_bounds__(256) void maxpool_nhwc_kernel(const _Float16 *__res
     }
 }
 
+// The common case -- a 3 x 3 window, whole groups of 8 channels, fewer than 2^31 threads: the index
+// arithmetic by multiply-high (FastDiv) and all nine loads in flight at once. Taps outside the image read
+// the clamped pixel and are replaced by -inf afterwards, so no load depends on a branch.
+__global__ __launch_bounds__(256) void maxpool3x3_nhwc_kernel(const _Float16 *__restrict__ x, uint32_t total, int C, int H, int W,
+                                                              FastDiv by_g, FastDiv by_wo, FastDiv by_ho, int sy, int sx,
+                                                              int py, int px, _Float16 *__restrict__ y) {
+    const uint32_t id = blockIdx.x * 256u + threadIdx.x;
+    if (id >= total) return;
+    int cg, ow, oh;
+    const uint32_t p = by_g.divmod(id, cg);
+    const uint32_t r = by_wo.divmod(p, ow);
+    const int b = (int)by_ho.divmod(r, oh);
+    const _Float16 ninf = (_Float16)(-__builtin_inff());
+    const half8 none = {ninf, ninf, ninf, ninf, ninf, ninf, ninf, ninf};
+    const _Float16 *img = x + (int64_t)b * H * W * C + cg * 8;
+    half8 v[9];
+    bool in[9];
+#pragma unroll
+    for (int i = 0; i < 3; i++) {
+        const int ih = oh * sy - py + i, ihc = ih < 0 ? 0 : (ih >= H ? H - 1 : ih);
+#pragma unroll
+        for (int j = 0; j < 3; j++) {
+            const int iw = ow * sx - px + j, iwc = iw < 0 ? 0 : (iw >= W ? W - 1 : iw);
+            in[i * 3 + j] = (ih == ihc) & (iw == iwc);
+            v[i * 3 + j] = *reinterpret_cast<const half8 *>(img + ((int64_t)ihc * W + iwc) * C);
+        }
+    }
+    half8 best = none;
+#pragma unroll
+    for (int t = 0; t < 9; t++) best = __builtin_elementwise_max(best, in[t] ? v[t] : none);
+    *reinterpret_cast<half8 *>(y + (int64_t)p * C + cg * 8) = best;
+}
+
 // y[b][c] = mean over the HW positions of x[b][.][c], fp32 accumulation. A workgroup = one image x 64
 // groups of 8 channels; its four wavefronts take every fourth position each (loads of a wavefront are
 // one contiguous KiB, several in flight), then the four partial sums are added in wavefront order.
@@ -152,6 +185,12 @@ int tmq_maxpool2d_nhwc(const void *x, int32_t B, int32_t C, int32_t H, int32_t W
     const int64_t total = (int64_t)B * ho * wo * ((C + 7) / 8), blocks = (total + 255) / 256;
     if (blocks > 0x7FFFFFFF) return TMQ_ERR_TOO_LARGE;
     const int vec = (C % 8 == 0) && aligned16(x) && aligned16(y);
+    if (vec && ky == 3 && kx == 3 && total < (int64_t)0x7FFFFFFF) {
+        hipLaunchKernelGGL(maxpool3x3_nhwc_kernel, dim3((uint32_t)blocks), dim3(256), 0, as_stream(stream),
+                           static_cast<const _Float16 *>(x), (uint32_t)total, C, H, W, FastDiv((uint32_t)(C / 8)),
+                           FastDiv((uint32_t)wo), FastDiv((uint32_t)ho), sy, sx, py, px, static_cast<_Float16 *>(y));
+        return check_launch();
+    }
     hipLaunchKernelGGL(maxpool_nhwc_kernel, dim3((uint32_t)blocks), dim3(256), 0, as_stream(stream),
                        static_cast<const _Float16 *>(x), B, C, H, W, (int)ho, (int)wo, ky, kx, sy, sx, py, px, vec,
                        static_cast<_Float16 *>(y));
