@@ -236,6 +236,12 @@ int tmq_fp32_rows_prefer_split(int64_t M, int64_t K, int64_t N);
  * a kernel that has to read that many bytes once: launch + one trip to memory.               */
 int tmq_probe_stream_read(const void *src, size_t bytes, uint32_t *sink, void *stream);
 
+/* Diagnostic with no counterpart in the reference, host only: the convolution and pooling kernels
+ * turn an output pixel's index into (batch, row, column) with a multiply-high by constants computed on
+ * the host instead of integer divisions. Returns how many of n[0 .. count) (host memory, each below
+ * 2^31) the same constants divide wrongly by `divisor` (1 <= divisor < 2^31): must be 0.            */
+int64_t tmq_selfcheck_fastdiv(uint32_t divisor, const uint32_t *n, int64_t count);
+
 /* Geometry of a 2-D convolution. */
 typedef struct tmq_conv_shape {
     int32_t B, C, H, W;   /* input extents (batch, channels, height, width) */

@@ -268,3 +268,25 @@ def test_oracle_transposed_depthwise_columns_are_the_outer_product(oracle):
         x = rng.standard_normal((B, P, C)).astype(np.float32)
         want = (x.transpose(0, 2, 1)[:, :, None, :] * W[None, :, :, None]).reshape(B, C * T, P)
         assert np.array_equal(oracle.dwconvtrans_cols(x, words, T).view(np.uint32), want.view(np.uint32))
+
+
+def test_pixel_index_division_constants():
+    """The convolution / pooling kernels divide an output pixel's index by image extents with a multiply-high
+    by host-computed constants. Host-only check of those constants against integer division: every divisor up
+    to 4096 and a few large ones, on multiples of the divisor and their neighbours, both ends of the 31-bit
+    range and random dividends."""
+    import ctypes
+    from tmq_amd import _capi
+    lib = _capi.load()
+    rng = np.random.default_rng(3)
+    big = np.uint64(2 ** 31 - 1)
+    for d in list(range(1, 4097)) + [65535, 65536, 65537, 1000003, 2 ** 30, 2 ** 30 + 1, 2 ** 31 - 1]:
+        k = rng.integers(0, int(big) // d + 1, 300, dtype=np.uint64)
+        mult = k * np.uint64(d)
+        n = np.concatenate([mult, mult + np.uint64(d - 1), np.maximum(mult, 1) - 1,
+                            rng.integers(0, 2 ** 31, 300, dtype=np.uint64),
+                            np.array([0, 1, d - 1, d, min(d + 1, int(big)), int(big), int(big) - 1], dtype=np.uint64)])
+        n = np.minimum(n, big).astype(np.uint32)
+        bad = lib.tmq_selfcheck_fastdiv(d, n.ctypes.data_as(ctypes.c_void_p), n.size)
+        assert bad == 0, f"divisor {d}: {bad} wrong quotients"
+    assert lib.tmq_selfcheck_fastdiv(0, n.ctypes.data_as(ctypes.c_void_p), 1) == -1

@@ -59,6 +59,7 @@ SIGNATURES = {
     "tmq_selfcheck_division": (_int, [_dbl, _vp, _vp]),
     "tmq_probe_stream_read": (_int, [_vp, ctypes.c_size_t, _vp, _vp]),
     "tmq_split_f32": (_int, [_vp, _vp, _vp, _i64, _vp]),
+    "tmq_selfcheck_fastdiv": (_i64, [_u32, _vp, _i64]),
     "tmq_fp32_rows_prefer_split": (_int, [_i64, _i64, _i64]),
     "tmq_multi_plan": (_int, [ctypes.POINTER(Segment), _int, ctypes.POINTER(_u32)]),
     "tmq_qloss_multi_workspace_bytes": (_sz, [_u32]),

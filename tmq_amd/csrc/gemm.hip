@@ -670,6 +670,17 @@ using namespace tmq;
 
 extern "C" {
 
+int64_t tmq_selfcheck_fastdiv(uint32_t divisor, const uint32_t *n, int64_t count) {
+    if (divisor == 0 || divisor >= 0x80000000u || !n || count < 0) return -1;
+    const FastDiv f(divisor);
+    int64_t bad = 0;
+    for (int64_t i = 0; i < count; i++) {
+        const uint32_t q = divisor > 1 ? (uint32_t)(((uint64_t)n[i] * f.mul) >> 32) >> f.shift : n[i];   // = FastDiv::divmod
+        if (n[i] >= 0x80000000u || q != n[i] / divisor) bad++;
+    }
+    return bad;
+}
+
 int tmq_conv2d_out_hw(const tmq_conv_shape *s, int32_t *ho, int32_t *wo) {
     if (!s || !ho || !wo || s->sy <= 0 || s->sx <= 0 || s->dy <= 0 || s->dx <= 0 || s->ky <= 0 || s->kx <= 0)
         return TMQ_ERR_INVALID_ARG;
