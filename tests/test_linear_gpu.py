@@ -53,7 +53,8 @@ def test_linear_fp16_matches_oracle(cuda, oracle, M, K, N):
     assert _rel_err(y0.cpu().numpy(), ref) <= 2e-6
 
 
-@pytest.mark.parametrize("M,K,N", [(1, 4096, 4096), (16, 4096, 4096), (5, 300, 70), (64, 1024, 256), (200, 512, 64)])
+@pytest.mark.parametrize("M,K,N", [(1, 4096, 4096), (16, 4096, 4096), (5, 300, 70), (64, 1024, 256), (200, 512, 64),
+                                   (2, 2048, 1000), (3, 4096, 70), (4, 2304, 520), (1, 16384, 4100)])
 def test_linear_fp32_activations(cuda, oracle, M, K, N):
     """fp32 activations (the reference's calling convention) keep fp32-level accuracy."""
     from tmq_amd import ops
@@ -158,6 +159,8 @@ STREAM = [  # at most 16 fp16 rows, K a multiple of 256 and >= 2048: every geome
     (1, 2048, 70, False), (2, 4096, 1000, False), (3, 2304, 520, False), (4, 2048, 8200, False), (4, 2560, 4096, False),
     (5, 4096, 12300, False), (7, 2048, 8200, False), (8, 3072, 4100, False), (9, 4096, 12304, False), (12, 2048, 8192, False),
     (16, 16384, 4096, False), (13, 2304, 48, False), (6, 8192, 28672, False), (1, 28672, 8192, False),
+    # at most 4 fp32 rows: the fp32 form of the weight-stream kernel
+    (4, 2048, 8200, True), (2, 8192, 1024, True), (3, 2560, 40, True), (1, 2048, 16, True),
 ]
 
 

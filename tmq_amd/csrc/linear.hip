@@ -21,6 +21,9 @@ namespace tmq {
 // mid.hip: staged split-reduction kernel for mid-size fp16 problems
 bool mid_dense_ok(const void *x, int64_t M, int64_t K);
 bool stream_dense_ok(const void *x, int64_t M, int64_t K);
+bool stream32_dense_ok(const void *x, int64_t M, int64_t K);
+int launch_stream32_dense(const void *x, int64_t M, int64_t K, const void *native, int64_t N, const float *scale,
+                          const float *bias, const void *residual, int relu, void *y, int y_f16, void *stream);
 int launch_stream_dense(const void *x, int64_t M, int64_t K, const void *native, int64_t N, const float *scale,
                         const float *bias, const void *residual, int relu, void *y, int y_f16, void *stream);
 int launch_mid_dense(const void *x, int64_t M, int64_t K, const void *native, int64_t N, const float *scale,
@@ -1156,6 +1159,9 @@ int tmq_ternary_linear(const void *x, int x_dtype, int64_t M, int64_t K, const v
     // 11008 x 4096 7.2 -> 6.2 us, even at 4096^2.
     if (!x32 && stream_dense_ok(x, M, K) && K >= 8 * kKB)
         return launch_stream_dense(x, M, K, native, N, ep.scale, ep.bias, ep.residual, ep.relu, y, ep.y_dtype == TMQ_F16, stream);
+    // ... and at most 4 fp32 rows (the reference's GEMV convention): its fp32 form (M = 1 at 4096^2: 6.0 -> 4.5 us)
+    if (x32 && stream32_dense_ok(x, M, K) && K >= 8 * kKB)
+        return launch_stream32_dense(x, M, K, native, N, ep.scale, ep.bias, ep.residual, ep.relu, y, ep.y_dtype == TMQ_F16, stream);
     // Otherwise up to 16 rows take the skinny kernels (activations staged in LDS). They also take 17 .. 64
     // rows when K is ragged or the rows are unaligned; with whole 256-index blocks the split-reduction
     // kernels are as fast at K = 4096 and two to three times faster at short K, where staging all of

@@ -644,6 +644,111 @@ int launch_stream(const void *x, const void *native, int64_t M, int64_t K, int64
     return check_launch();
 }
 
+// ---- weight stream, fp32 activations, at most 4 rows -------------------------------------------------
+// The reference's GEMV (ternary_mvm_cuda) takes an fp32 vector. Same plan as stream_kernel with 16 channels
+// per workgroup, but the activations of a block (256 fp32 = 1 KiB per row, one 16-byte load per lane) travel
+// through registers: each value is split into two fp16 terms (hi = fp16(x), lo = fp16(x - hi), together 22
+// significant bits), the terms go through a small wavefront-private LDS area into operand order, and
+// every weight fragment is multiplied with both. All loads are register loads, so the compiler counts the
+// waits itself -- exactly, as long as the steady state refills unconditionally (template argument LONG:
+// every wavefront has at least 2 D blocks; otherwise a guarded pipeline).
+template <int WAVES, int MR, int D, bool LONG>
+__global__ __launch_bounds__(64 * WAVES) void stream32_kernel(const float *__restrict__ x, const u32x4 *__restrict__ native,
+                                                              int64_t M, int64_t K, int Kb, int64_t N, int64_t Nb,
+                                                              MidEpilogue ep) {
+    constexpr int kRow = 1024 + 32;                                 // bytes per staged row: hi plane, lo plane, pad
+    constexpr int kWave = MR * kRow;
+    constexpr size_t kRed = (size_t)WAVES * (1024 + 64);
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    const int lane = threadIdx.x & 63, kg = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int j = lane & 15, g = lane >> 4;
+    unsigned char *win = smem + kRed + kg * kWave;                  // behind the reduction area: no reuse, no barrier
+    const int64_t n0 = (int64_t)blockIdx.x * 16;
+
+    floatx4 acc[1][1] = {{floatx4{0.f, 0.f, 0.f, 0.f}}};
+    int64_t nb = n0 / 16;
+    if (nb >= Nb) nb = Nb - 1;
+    const u32x4 *wb = native + (nb * Kb) * 64 + lane;
+    const float *xr[MR];                                            // this lane's four values of a block, per row
+#pragma unroll
+    for (int r = 0; r < MR; r++) xr[r] = x + (int64_t)(r < M ? r : M - 1) * K + lane * 4;
+    const int rrow = j < M ? j : (int)M - 1;                        // the row whose operand this lane supplies
+    const unsigned char *rd = win + rrow * kRow + g * 16;
+
+    const int nt = Kb > kg ? (Kb - kg + WAVES - 1) / WAVES : 0;   // weight blocks of this wavefront
+    u32x4 wq[D];
+    floatx4 xq[D][MR];
+    auto load = [&](int slot, int t) {
+        const int64_t kb = kg + (int64_t)t * WAVES;
+        wq[slot] = __builtin_nontemporal_load(wb + kb * 64);
+#pragma unroll
+        for (int r = 0; r < MR; r++) xq[slot][r] = *reinterpret_cast<const floatx4 *>(xr[r] + kb * kKB);
+    };
+    auto multiply = [&](int slot) {
+#pragma unroll
+        for (int r = 0; r < MR; r++) {
+            half4 hi, lo;
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                hi[e] = (_Float16)xq[slot][r][e];
+                lo[e] = (_Float16)(xq[slot][r][e] - (float)hi[e]);
+            }
+            *reinterpret_cast<half4 *>(win + r * kRow + lane * 8) = hi;
+            *reinterpret_cast<half4 *>(win + r * kRow + 512 + lane * 8) = lo;
+        }
+        __builtin_amdgcn_wave_barrier();
+        half8 a[8], b[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            a[i] = *reinterpret_cast<const half8 *>(rd + i * 64);
+            b[i] = *reinterpret_cast<const half8 *>(rd + 512 + i * 64);
+        }
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const half8 w = decode_step(wq[slot][i >> 1], i & 1);
+            acc[0][0] = mfma16(w, a[i], acc[0][0]);
+            acc[0][0] = mfma16(w, b[i], acc[0][0]);
+        }
+        __builtin_amdgcn_wave_barrier();
+    };
+    static_assert(D == 4, "unrolled by hand");
+    int t = 0;
+    if constexpr (LONG) {
+#pragma unroll
+        for (int d = 0; d < D; d++) load(d, d);
+        do {
+            multiply(0); load(0, t + D);
+            multiply(1); load(1, t + D + 1);
+            multiply(2); load(2, t + D + 2);
+            multiply(3); load(3, t + D + 3);
+            t += D;
+        } while (t + 2 * D <= nt);
+    } else {
+#pragma unroll
+        for (int d = 0; d < D; d++)
+            if (d < nt) load(d, d);
+    }
+    for (; t < nt; t += D) {
+        if (t < nt) { multiply(0); if (t + D < nt) load(0, t + D); }
+        if (t + 1 < nt) { multiply(1); if (t + D + 1 < nt) load(1, t + D + 1); }
+        if (t + 2 < nt) { multiply(2); if (t + D + 2 < nt) load(2, t + D + 2); }
+        if (t + 3 < nt) { multiply(3); if (t + D + 3 < nt) load(3, t + D + 3); }
+    }
+    reduce_and_store<1, 1, WAVES>(smem, acc, kg, lane, 0, n0, M, N, ep);
+}
+
+template <int MR>
+int launch_stream32(const void *x, const void *native, int64_t M, int64_t K, int64_t N, const MidEpilogue &ep, void *stream) {
+    constexpr int WAVES = 8, D = 4;
+    const int64_t tn = (N + 15) / 16, Kb = native_blocks_k(K);
+    if (tn > 0x7FFFFFFF || Kb > (1 << 20)) return TMQ_ERR_TOO_LARGE;
+    constexpr size_t lds = (size_t)WAVES * (1024 + 64) + (size_t)WAVES * MR * (1024 + 32);
+    auto kernel = Kb / WAVES >= 2 * D ? stream32_kernel<WAVES, MR, D, true> : stream32_kernel<WAVES, MR, D, false>;
+    hipLaunchKernelGGL(kernel, dim3((uint32_t)tn), dim3(64 * WAVES), lds, as_stream(stream), static_cast<const float *>(x),
+                       static_cast<const u32x4 *>(native), M, K, (int)Kb, N, native_blocks_n(N), ep);
+    return check_launch();
+}
+
 // Geometry: 64 x 128 tiles where they save a pass over the CUs (below); else the largest smaller tile
 // that keeps most CUs busy; then as many wavefronts per tile as it takes to put about ten on every CU,
 // each with at least two pairs to multiply.
@@ -702,6 +807,19 @@ int launch_mid_dense(const void *x, int64_t M, int64_t K, const void *native, in
 // True when the weight-stream kernel can take a dense fp16 problem of at most 16 rows.
 bool stream_dense_ok(const void *x, int64_t M, int64_t K) {
     return M >= 1 && M <= 16 && (K % kKB == 0) && aligned16(x) && M * K < (int64_t)0x7FFFFFFF;
+}
+
+// At most 4 fp32 rows with whole weight blocks: the fp32 weight-stream kernel.
+bool stream32_dense_ok(const void *x, int64_t M, int64_t K) {
+    return M >= 1 && M <= 4 && (K % kKB == 0) && aligned16(x);
+}
+
+int launch_stream32_dense(const void *x, int64_t M, int64_t K, const void *native, int64_t N, const float *scale,
+                          const float *bias, const void *residual, int relu, void *y, int y_f16, void *stream) {
+    MidEpilogue ep{scale, bias, residual, y, relu, y_f16};
+    if (M == 1) return launch_stream32<1>(x, native, M, K, N, ep, stream);
+    if (M == 2) return launch_stream32<2>(x, native, M, K, N, ep, stream);
+    return launch_stream32<4>(x, native, M, K, N, ep, stream);
 }
 
 // Geometry of the weight-stream kernel (stream_dense_ok must hold). Rows staged: the power of two >= M.
