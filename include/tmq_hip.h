@@ -225,7 +225,7 @@ int tmq_ternary_linear(const void *x, int x_dtype, int64_t M, int64_t K, const v
 int tmq_split_f32(const float *x, void *hi, void *lo, int64_t n, void *stream);
 
 /* 1 if M fp32 rows against a K x N layer are faster as two fp16 passes over tmq_split_f32's terms than
- * as one tmq_ternary_linear call with x_dtype TMQ_F32 (many rows, or a few rows over a very large
+ * as one tmq_ternary_linear call with x_dtype TMQ_F32 (many rows, or a few rows over a large
  * layer), else 0. Host-only arithmetic on the shape; no counterpart in the reference.               */
 int tmq_fp32_rows_prefer_split(int64_t M, int64_t K, int64_t N);
 

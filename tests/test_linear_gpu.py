@@ -54,7 +54,7 @@ def test_linear_fp16_matches_oracle(cuda, oracle, M, K, N):
 
 
 @pytest.mark.parametrize("M,K,N", [(1, 4096, 4096), (16, 4096, 4096), (5, 300, 70), (64, 1024, 256), (200, 512, 64),
-                                   (2, 2048, 1000), (3, 4096, 70), (4, 2304, 520), (1, 16384, 4100)])
+                                   (2, 2048, 1000), (3, 4096, 70), (4, 2304, 520), (1, 16384, 4100), (5, 2048, 200), (8, 4096, 1000), (7, 16384, 4096)])
 def test_linear_fp32_activations(cuda, oracle, M, K, N):
     """fp32 activations (the reference's calling convention) keep fp32-level accuracy."""
     from tmq_amd import ops
@@ -90,7 +90,7 @@ def test_split_f32_terms(cuda):
     assert torch.all((hi.float() + lo.float() - x).abs()[fin] <= x.abs()[fin] * 2.0 ** -21 + 1e-7)
 
 
-@pytest.mark.parametrize("M,K,N", [(1024, 1024, 4096), (600, 4096, 2048), (5, 16384, 8192)])
+@pytest.mark.parametrize("M,K,N", [(1024, 1024, 4096), (600, 4096, 2048), (10, 8192, 8192), (5, 16384, 8192)])
 def test_linear_fp32_many_rows(cuda, M, K, N):
     """Many fp32 rows run as two passes of the fp16 kernels over the two fp16 terms of the activations:
     fp32-level accuracy against the fp64 product, with every epilogue option."""
@@ -160,7 +160,7 @@ STREAM = [  # at most 16 fp16 rows, K a multiple of 256 and >= 2048: every geome
     (5, 4096, 12300, False), (7, 2048, 8200, False), (8, 3072, 4100, False), (9, 4096, 12304, False), (12, 2048, 8192, False),
     (16, 16384, 4096, False), (13, 2304, 48, False), (6, 8192, 28672, False), (1, 28672, 8192, False),
     # at most 4 fp32 rows: the fp32 form of the weight-stream kernel
-    (4, 2048, 8200, True), (2, 8192, 1024, True), (3, 2560, 40, True), (1, 2048, 16, True),
+    (4, 2048, 8200, True), (2, 8192, 1024, True), (3, 2560, 40, True), (1, 2048, 16, True), (8, 2048, 8200, True), (6, 4096, 100, True),
 ]
 
 

@@ -1111,11 +1111,14 @@ int tmq_prepack_weights(const uint32_t *words, int64_t N, int64_t C, int64_t ky,
 
 int tmq_fp32_rows_prefer_split(int64_t M, int64_t K, int64_t N) {
     // Measured: at K = N = 4096 the two fp16 passes win from about 512 rows (M = 4096: 400 -> 238 us), at
-    // K = N = 1024 from about 4096; over very large layers already from 3 rows (16384^2, M = 16: 118 -> 45 us),
-    // because the fp16 weight-stream and tile kernels have no fp32 form.
+    // K = N = 1024 from about 4096; over large layers already from 9 rows (8192^2, M = 16: 34 -> 23 us) or,
+    // beyond 2^27 weights, from 3 (16384^2, M = 4: 65 -> 39 us, M = 16: 118 -> 45 us): there the fp16
+    // weight-stream kernel run twice beats every kernel that splits on the fly.
     if (M <= 0 || K <= 0 || N <= 0) return 0;
     const bool many_rows = M >= 512 && (double)M * (double)K * (double)N >= 4294967296.0;
-    const bool large_layer = M >= 3 && (double)K * (double)N >= 134217728.0;
+    // up to 8 rows have an fp32 stream kernel, which holds its own up to about 2^26 weights
+    const double weights = (double)K * (double)N;
+    const bool large_layer = (M >= 9 && weights >= 67108864.0) || (M >= 3 && weights >= 134217728.0);
     return many_rows || large_layer;
 }
 
@@ -1159,7 +1162,8 @@ int tmq_ternary_linear(const void *x, int x_dtype, int64_t M, int64_t K, const v
     // 11008 x 4096 7.2 -> 6.2 us, even at 4096^2.
     if (!x32 && stream_dense_ok(x, M, K) && K >= 8 * kKB)
         return launch_stream_dense(x, M, K, native, N, ep.scale, ep.bias, ep.residual, ep.relu, y, ep.y_dtype == TMQ_F16, stream);
-    // ... and at most 4 fp32 rows (the reference's GEMV convention): its fp32 form (M = 1 at 4096^2: 6.0 -> 4.5 us)
+    // ... and at most 8 fp32 rows (the reference's GEMV convention): its fp32 form (M = 1 at 4096^2: 6.0 -> 4.5 us,
+    // M = 8 at 8192^2: 24 -> 17 us)
     if (x32 && stream32_dense_ok(x, M, K) && K >= 8 * kKB)
         return launch_stream32_dense(x, M, K, native, N, ep.scale, ep.bias, ep.residual, ep.relu, y, ep.y_dtype == TMQ_F16, stream);
     // Otherwise up to 16 rows take the skinny kernels (activations staged in LDS). They also take 17 .. 64

@@ -644,7 +644,7 @@ int launch_stream(const void *x, const void *native, int64_t M, int64_t K, int64
     return check_launch();
 }
 
-// ---- weight stream, fp32 activations, at most 4 rows -------------------------------------------------
+// ---- weight stream, fp32 activations, at most 8 rows -------------------------------------------------
 // The reference's GEMV (ternary_mvm_cuda) takes an fp32 vector. Same plan as stream_kernel with 16 channels
 // per workgroup, but the activations of a block (256 fp32 = 1 KiB per row, one 16-byte load per lane) travel
 // through registers: each value is split into two fp16 terms (hi = fp16(x), lo = fp16(x - hi), together 22
@@ -711,7 +711,7 @@ __global__ __launch_bounds__(64 * WAVES) void stream32_kernel(const float *__res
         }
         __builtin_amdgcn_wave_barrier();
     };
-    static_assert(D == 4, "unrolled by hand");
+    static_assert(D == 2 || D == 4, "unrolled by hand");
     int t = 0;
     if constexpr (LONG) {
 #pragma unroll
@@ -719,8 +719,10 @@ __global__ __launch_bounds__(64 * WAVES) void stream32_kernel(const float *__res
         do {
             multiply(0); load(0, t + D);
             multiply(1); load(1, t + D + 1);
-            multiply(2); load(2, t + D + 2);
-            multiply(3); load(3, t + D + 3);
+            if constexpr (D > 2) {
+                multiply(2); load(2, t + D + 2);
+                multiply(3); load(3, t + D + 3);
+            }
             t += D;
         } while (t + 2 * D <= nt);
     } else {
@@ -731,15 +733,17 @@ __global__ __launch_bounds__(64 * WAVES) void stream32_kernel(const float *__res
     for (; t < nt; t += D) {
         if (t < nt) { multiply(0); if (t + D < nt) load(0, t + D); }
         if (t + 1 < nt) { multiply(1); if (t + D + 1 < nt) load(1, t + D + 1); }
-        if (t + 2 < nt) { multiply(2); if (t + D + 2 < nt) load(2, t + D + 2); }
-        if (t + 3 < nt) { multiply(3); if (t + D + 3 < nt) load(3, t + D + 3); }
+        if constexpr (D > 2) {
+            if (t + 2 < nt) { multiply(2); if (t + D + 2 < nt) load(2, t + D + 2); }
+            if (t + 3 < nt) { multiply(3); if (t + D + 3 < nt) load(3, t + D + 3); }
+        }
     }
     reduce_and_store<1, 1, WAVES>(smem, acc, kg, lane, 0, n0, M, N, ep);
 }
 
 template <int MR>
 int launch_stream32(const void *x, const void *native, int64_t M, int64_t K, int64_t N, const MidEpilogue &ep, void *stream) {
-    constexpr int WAVES = 8, D = 4;
+    constexpr int WAVES = 8, D = MR <= 4 ? 4 : 2;                  // D x MR x 4 registers hold the activations
     const int64_t tn = (N + 15) / 16, Kb = native_blocks_k(K);
     if (tn > 0x7FFFFFFF || Kb > (1 << 20)) return TMQ_ERR_TOO_LARGE;
     constexpr size_t lds = (size_t)WAVES * (1024 + 64) + (size_t)WAVES * MR * (1024 + 32);
@@ -809,9 +813,10 @@ bool stream_dense_ok(const void *x, int64_t M, int64_t K) {
     return M >= 1 && M <= 16 && (K % kKB == 0) && aligned16(x) && M * K < (int64_t)0x7FFFFFFF;
 }
 
-// At most 4 fp32 rows with whole weight blocks: the fp32 weight-stream kernel.
+// At most 8 fp32 rows with whole weight blocks: the fp32 weight-stream kernel (with 9..16 rows its
+// activations no longer fit the registers: measured slower than the older kernel on large layers).
 bool stream32_dense_ok(const void *x, int64_t M, int64_t K) {
-    return M >= 1 && M <= 4 && (K % kKB == 0) && aligned16(x);
+    return M >= 1 && M <= 8 && (K % kKB == 0) && aligned16(x);
 }
 
 int launch_stream32_dense(const void *x, int64_t M, int64_t K, const void *native, int64_t N, const float *scale,
@@ -819,7 +824,8 @@ int launch_stream32_dense(const void *x, int64_t M, int64_t K, const void *nativ
     MidEpilogue ep{scale, bias, residual, y, relu, y_f16};
     if (M == 1) return launch_stream32<1>(x, native, M, K, N, ep, stream);
     if (M == 2) return launch_stream32<2>(x, native, M, K, N, ep, stream);
-    return launch_stream32<4>(x, native, M, K, N, ep, stream);
+    if (M <= 4) return launch_stream32<4>(x, native, M, K, N, ep, stream);
+    return launch_stream32<8>(x, native, M, K, N, ep, stream);
 }
 
 // Geometry of the weight-stream kernel (stream_dense_ok must hold). Rows staged: the power of two >= M.
