@@ -78,8 +78,17 @@ def test_fold_resnet_and_explicit_pairs(cuda):
         prev = t.set_compact_output_dtype(torch.float16)
         try:
             got16 = model(x)
+            # the library's own fp16 NHWC pooling in place of PyTorch's: the same values (max is exact, the
+            # mean accumulates in fp32 either way)
+            names = t.use_native_pooling(model)
+            assert names == ["maxpool", "avgpool"]
+            got16p = model(x)
         finally:
             t.set_compact_output_dtype(prev)
+        # fp32 tensors pass through the replaced modules to PyTorch's pooling
+        assert torch.allclose(model(x), got, rtol=1e-5, atol=1e-5 * want.abs().max().item())
+    assert got16p.dtype == torch.float16
+    assert torch.allclose(got16p.float(), got16.float(), rtol=2e-3, atol=2e-3 * want.abs().max().item())
     assert torch.allclose(got, want, rtol=5e-3, atol=5e-3 * want.abs().max().item())
     assert got16.dtype == torch.float16 and torch.allclose(got16.float(), want, rtol=3e-2, atol=3e-2 * want.abs().max().item())
     with pytest.raises(ValueError):

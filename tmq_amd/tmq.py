@@ -979,6 +979,51 @@ def fold_batchnorm(module: nn.Module, pairs=None):
     return done
 
 
+class _MaxPool2dNHWC(nn.Module):
+    """nn.MaxPool2d for fp16 channels_last GPU tensors (anything else goes to the module it replaced)."""
+
+    def __init__(self, inner: nn.MaxPool2d):
+        super().__init__()
+        self.inner = inner
+
+    def forward(self, x):
+        if x.is_cuda and x.dim() == 4 and x.dtype == torch.float16 and x.is_contiguous(memory_format=torch.channels_last):
+            return ops.maxpool2d_nhwc(x, self.inner.kernel_size, self.inner.stride, self.inner.padding)
+        return self.inner(x)
+
+
+class _GlobalAvgPoolNHWC(nn.Module):
+    """nn.AdaptiveAvgPool2d(1) for fp16 channels_last GPU tensors (anything else goes to the module it replaced)."""
+
+    def __init__(self, inner: nn.AdaptiveAvgPool2d):
+        super().__init__()
+        self.inner = inner
+
+    def forward(self, x):
+        if x.is_cuda and x.dim() == 4 and x.dtype == torch.float16 and x.is_contiguous(memory_format=torch.channels_last):
+            return ops.avgpool_global_nhwc(x, out_dtype=torch.float16).view(x.shape[0], x.shape[1], 1, 1)
+        return self.inner(x)
+
+
+def use_native_pooling(module: nn.Module):
+    """Replace the nn.MaxPool2d (no dilation, no ceil_mode, no indices) and nn.AdaptiveAvgPool2d(1) modules
+    below `module` by fp16 NHWC kernels of this library; they act only on fp16 channels_last GPU tensors --
+    what compact layers hand on after set_compact_output_dtype(torch.float16) -- and defer to the original
+    module otherwise. For inference. Returns the qualified names of the replaced modules."""
+    done = []
+    for pname, parent in list(module.named_modules()):
+        for cname, child in list(parent.named_children()):
+            name = (pname + "." if pname else "") + cname
+            if (isinstance(child, nn.MaxPool2d) and child.dilation in (1, (1, 1)) and not child.ceil_mode
+                    and not child.return_indices):
+                setattr(parent, cname, _MaxPool2dNHWC(child))
+                done.append(name)
+            elif isinstance(child, nn.AdaptiveAvgPool2d) and child.output_size in (1, (1, 1)):
+                setattr(parent, cname, _GlobalAvgPoolNHWC(child))
+                done.append(name)
+    return done
+
+
 def expand_compact_layers(module: nn.Module, for_training=False):
     """Expand compact TMQ layers back to fp32 weights in place (tmq/tmq.py:1296-1319)."""
     for name, sub in module.named_children():
