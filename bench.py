@@ -297,17 +297,20 @@ def bench_resnet_infer(args, torch):
     B = args.batch or 64
     x = torch.randn(B, 3, 224, 224, generator=torch.Generator().manual_seed(20)).half().to(dev)
     fused = FusedTernaryResNet18(model)
-    out = {}
+    out, graph = {}, [None]
     for name, fn, reps in (("fused", lambda: fused(x), args.steps), ("drop_in", lambda: model(x), max(3, args.steps // 4)),
                            ("drop_in_bn_folded", lambda: model(x), max(3, args.steps // 4)),
                            ("drop_in_bn_folded_fp16", lambda: model(x), max(3, args.steps // 4)),
-                           ("drop_in_bn_folded_fp16_pooling", lambda: model(x), max(3, args.steps // 4))):
+                           ("drop_in_bn_folded_fp16_pooling", lambda: model(x), max(3, args.steps // 4)),
+                           ("drop_in_fused_graph", lambda: graph[0](x), max(3, args.steps // 4))):
         if name == "drop_in_bn_folded":
             t.fold_batchnorm(model)                           # BatchNorm into the convolutions' epilogues
         if name == "drop_in_bn_folded_fp16":
             t.set_compact_output_dtype(torch.float16)         # fp16 channels_last between the layers
         if name == "drop_in_bn_folded_fp16_pooling":
             t.use_native_pooling(model)                       # the library's fp16 NHWC max-pool / average pool
+        if name == "drop_in_fused_graph":
+            graph[0] = t.fuse_epilogues(model)[0]             # ReLU / residual add into the kernels' epilogues (torch.fx)
         with torch.no_grad():
             for _ in range(max(2, args.warmup // 4)):
                 fn()

@@ -83,8 +83,18 @@ def test_fold_resnet_and_explicit_pairs(cuda):
             names = t.use_native_pooling(model)
             assert names == ["maxpool", "avgpool"]
             got16p = model(x)
+            # ReLU and residual additions into the convolutions' epilogues: 8 blocks x (relu(conv1), relu(conv2 + r))
+            # and the stem's relu
+            gm, sites = t.fuse_epilogues(model)
+            assert sites == 17
+            assert not any(n.op == "call_function" and n.target in (torch.relu, torch.add) for n in gm.graph.nodes)
+            got16f = gm(x)
         finally:
             t.set_compact_output_dtype(prev)
+        got32f = gm(x)                                     # the fused graph in fp32 as well
+        assert torch.allclose(got32f, got, rtol=1e-4, atol=1e-4 * want.abs().max().item())
+        assert got16f.dtype == torch.float16
+        assert torch.allclose(got16f.float(), got16.float(), rtol=5e-3, atol=5e-3 * want.abs().max().item())
         # fp32 tensors pass through the replaced modules to PyTorch's pooling
         assert torch.allclose(model(x), got, rtol=1e-5, atol=1e-5 * want.abs().max().item())
     assert got16p.dtype == torch.float16
@@ -93,3 +103,63 @@ def test_fold_resnet_and_explicit_pairs(cuda):
     assert got16.dtype == torch.float16 and torch.allclose(got16.float(), want, rtol=3e-2, atol=3e-2 * want.abs().max().item())
     with pytest.raises(ValueError):
         t.set_compact_output_dtype(torch.bfloat16)
+
+
+class _Patterns(torch.nn.Module):
+    """One site of every pattern fuse_epilogues recognises, and three it must leave alone."""
+
+    def __init__(self):
+        super().__init__()
+        nn = torch.nn
+        self.a = nn.Conv2d(8, 16, 3, 1, 1, bias=True)         # relu module
+        self.act = nn.ReLU(inplace=True)
+        self.b = nn.Conv2d(16, 16, 3, 1, 1, bias=False)        # += residual, then .relu()
+        self.c = nn.Conv2d(16, 16, 1, bias=False)              # residual on the left, no relu
+        self.d = nn.Conv2d(16, 16, 3, 1, 1, groups=16, bias=False)   # depthwise, F.relu
+        self.e = nn.Conv2d(16, 16, 1, bias=False)              # used twice: stays
+        self.f = nn.Conv2d(16, 16, 1, bias=False)              # BatchNorm in between: stays
+        self.bn = nn.BatchNorm2d(16)
+        self.g = nn.Conv2d(16, 16, 1, bias=False)              # x + x of its own output: stays
+        self.head = nn.Linear(16, 10)                          # torch.relu on a linear layer
+
+    def forward(self, x):
+        h = self.act(self.a(x))
+        y = self.b(h)
+        y += h
+        y = y.relu()
+        z = h + self.c(y)
+        z = torch.nn.functional.relu(self.d(z))
+        e = self.e(z)
+        z = e + torch.tanh(e)
+        z = torch.relu(self.bn(self.f(z)))
+        g = self.g(z)
+        z = g + g
+        return torch.relu(self.head(z.mean(dim=(2, 3))))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_fuse_epilogues_patterns(cuda, dtype):
+    import tmq_amd as t
+    torch.manual_seed(3)
+    net = _Patterns()
+    ctrl = t.QuantizationControl(post_scale=True)
+    t.quantize_model(net, ctrl)
+    _randomize_bn(net, torch.Generator().manual_seed(3))
+    net.to(cuda).eval()
+    ctrl.quantize()
+    t.compressed_state_dict(net, strong=False)
+    x = torch.randn(3, 8, 12, 10, device=cuda)
+    prev = t.set_compact_output_dtype(dtype)
+    try:
+        with torch.no_grad():
+            want = net(x)
+            gm, sites = t.fuse_epilogues(net)
+            got = gm(x)
+    finally:
+        t.set_compact_output_dtype(prev)
+    assert sites == 5                                          # a, b, c, d, head
+    calls = [n.target for n in gm.graph.nodes if n.op == "call_module"]
+    assert sum(str(c).startswith("_fused_") for c in calls) == 5
+    assert {"e", "f", "g", "bn"} <= set(calls) and not {"a", "b", "c", "d", "head", "act"} & set(calls)
+    tol = 2e-3 if dtype == torch.float16 else 1e-5
+    assert got.dtype == want.dtype and torch.allclose(got.float(), want.float(), rtol=tol, atol=tol * want.abs().max().item())

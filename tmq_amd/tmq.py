@@ -540,8 +540,9 @@ class Linear(nn.Module, TMQLayer):
     forward_wrap = forward
 
     @torch.no_grad()
-    def compact_forward(self, x):
-        """Inference straight from the 2-bit packed weights (tmq/tmq.py:662-688), any batch shape."""
+    def compact_forward(self, x, residual=None, relu=False):
+        """Inference straight from the 2-bit packed weights (tmq/tmq.py:662-688), any batch shape.
+        residual / relu: added / applied in the kernel's epilogue (fuse_epilogues)."""
         assert self.training == False, "Compact inference is not supported in training mode"
         assert self.weight.data.dtype == torch.int32, "Compact inference requires 32-bit integer words"
         self._update_scale()
@@ -550,7 +551,11 @@ class Linear(nn.Module, TMQLayer):
         nw = self._native_weights()
         xin = x if x.is_contiguous() else x.contiguous()
         scale, bias = self._epilogue(nw.N, x.device)
-        out = ops.ternary_linear(xin, nw, scale=scale, bias=bias, out_dtype=_compact_out)
+        if (residual is not None or relu) and self.bn is not None:
+            raise RuntimeError("compact_forward: the layer's own BatchNorm comes between the product and the fused epilogue")
+        if residual is not None:
+            residual = residual.to(_compact_out).contiguous()
+        out = ops.ternary_linear(xin, nw, scale=scale, bias=bias, residual=residual, relu=relu, out_dtype=_compact_out)
         return self.bn(out) if self.bn is not None else out
 
     @classmethod
@@ -627,15 +632,20 @@ class Conv2d(nn.Module, TMQLayer):
         return self._conv(x, w, self.bias)
 
     @torch.no_grad()
-    def compact_forward(self, x):
+    def compact_forward(self, x, residual=None, relu=False):
         """Implicit-GEMM convolution from the packed weights (replaces the unfold / GEMM / fold
         sequence of tmq/tmq.py:822-871). Output extents follow PyTorch's formula. Returns fp32
-        [B, N, Ho, Wo] (channels_last memory); a 3-D input gives a 3-D output."""
+        [B, N, Ho, Wo] (channels_last memory); a 3-D input gives a 3-D output.
+        residual / relu: added / applied in the kernel's epilogue (fuse_epilogues)."""
         assert not self.training, "Compact inference is not supported in training mode"
         assert self.weight.data.dtype == torch.int32, "Compact inference requires 32-bit integer words"
         self._update_scale()
         if x.dim() == 3:
-            return self.compact_forward(x.unsqueeze(0)).squeeze(0)
+            r3 = residual.unsqueeze(0) if residual is not None else None
+            return self.compact_forward(x.unsqueeze(0), r3, relu).squeeze(0)
+        if residual is not None and (residual.dtype != _compact_out or
+                                     not residual.is_contiguous(memory_format=torch.channels_last)):
+            residual = residual.to(dtype=_compact_out, memory_format=torch.channels_last)
         if x.dim() != 4:
             raise Exception("Expected a 3D tensor")
         assert self.groups == 1 or self.groups == self.original_shape[0], \
@@ -647,7 +657,8 @@ class Conv2d(nn.Module, TMQLayer):
                 raise RuntimeError("depthwise compact inference needs one filter per input channel")
             scale, bias = self._epilogue(x.shape[1], x.device)
             return ops.ternary_dwconv2d(x, self.weight.data, (ky, kx), _pair(self.stride), _pair(self.padding),
-                                        _pair(self.dilation), scale=scale, bias=bias, out_dtype=_compact_out)
+                                        _pair(self.dilation), scale=scale, bias=bias, residual=residual, relu=relu,
+                                        out_dtype=_compact_out)
         scale, bias = self._epilogue(int(self.original_shape[0]), x.device)
         sp = self._superpixel_plan(x)
         if sp is not None:
@@ -658,10 +669,10 @@ class Conv2d(nn.Module, TMQLayer):
             xs = ops.nchw_to_nhwc4(x).view(B, H, W // 2, 8).permute(0, 3, 1, 2)
             (sy, _), (py, _) = _pair(self.stride), _pair(self.padding)
             return ops.ternary_conv2d(xs, nw, (sy, 1), ((py, py), (pl, pr)), 1, scale=scale, bias=bias,
-                                      out_dtype=_compact_out)
+                                      residual=residual, relu=relu, out_dtype=_compact_out)
         nw = self._native_weights(conv_kernel=(ky, kx))
         return ops.ternary_conv2d(x, nw, _pair(self.stride), _pair(self.padding), _pair(self.dilation), scale=scale,
-                                  bias=bias, out_dtype=_compact_out)
+                                  bias=bias, residual=residual, relu=relu, out_dtype=_compact_out)
 
     def _superpixel_plan(self, x):
         """For a convolution with at most 4 input channels, horizontal stride 2 and no dilation on an
@@ -977,6 +988,111 @@ def fold_batchnorm(module: nn.Module, pairs=None):
         setattr(parent, child, nn.Identity())
         done.append((ln, bname))
     return done
+
+
+class _FusedEpilogue(nn.Module):
+    """A compact layer called with its residual input and / or a ReLU in the kernel's epilogue."""
+
+    def __init__(self, layer, relu):
+        super().__init__()
+        self.layer = layer
+        self.relu = bool(relu)
+
+    def forward(self, x, residual=None):
+        return self.layer.compact_forward(x, residual, self.relu)
+
+
+def fuse_epilogues(model: nn.Module):
+    """Move the ReLU and the residual addition that follow a compact Conv2d / Linear in the model's forward
+    into that layer's kernel epilogue (the reference's README lists this fusion as future work,
+    README.md:150-155). The model is traced with torch.fx (TMQ layers are leaves); recognised are, with any
+    number of nn.Identity modules (what fold_batchnorm leaves behind) in between,
+
+        relu(layer(x))      layer(x) + r      relu(layer(x) + r)
+
+    where `relu` is torch.relu / F.relu / x.relu() / an nn.ReLU module, `+` is +, += or torch.add, the
+    layer is a compact Conv2d or Linear without a BatchNorm of its own, and the intermediate values have no
+    other use. Everything else stays as traced. For inference, after the layers went compact and after
+    fold_batchnorm. Returns (GraphModule sharing the model's parameters, number of fused sites)."""
+    import operator
+    import torch.fx as fx
+
+    class Tracer(fx.Tracer):
+        def is_leaf_module(self, m, qualname):
+            # this module's own layers and wrappers branch on their input: never trace into them
+            return isinstance(m, TMQLayer) or type(m).__module__ == __name__ or super().is_leaf_module(m, qualname)
+
+    graph = Tracer().trace(model)
+    mods = dict(model.named_modules())
+
+    def is_relu(n):
+        if n.op == "call_function":
+            return n.target in (torch.relu, nn.functional.relu, torch.relu_) and len(n.args) >= 1
+        if n.op == "call_method":
+            return n.target in ("relu", "relu_")
+        return n.op == "call_module" and isinstance(mods.get(n.target), nn.ReLU)
+
+    def is_add(n):
+        if n.op == "call_function":
+            return n.target in (operator.add, operator.iadd, torch.add) and len(n.args) == 2 and not n.kwargs
+        return n.op == "call_method" and n.target in ("add", "add_") and len(n.args) == 2 and not n.kwargs
+
+    def only_user(n):
+        users = list(n.users)
+        return users[0] if len(users) == 1 else None
+
+    gm = fx.GraphModule(model, graph)
+    fused = 0
+    for node in list(graph.nodes):
+        if node.op != "call_module":
+            continue
+        layer = mods.get(node.target)
+        if not (isinstance(layer, (Linear, Conv2d)) and not isinstance(layer, ConvTranspose2d) and layer.compact
+                and getattr(layer, "bn", None) is None and len(node.args) == 1 and not node.kwargs):
+            continue
+        # follow the value through Identity modules
+        last = node
+        while True:
+            nxt = only_user(last)
+            if nxt is not None and nxt.op == "call_module" and isinstance(mods.get(nxt.target), nn.Identity):
+                last = nxt
+            else:
+                break
+        nxt = only_user(last)
+        if nxt is None:
+            continue
+        residual, end, relu = None, None, False
+        if is_add(nxt) and nxt.args[0] is not nxt.args[1] and isinstance(nxt.args[0], fx.Node) and isinstance(nxt.args[1], fx.Node):
+            residual = nxt.args[1] if nxt.args[0] is last else nxt.args[0]
+            end = nxt
+            after = only_user(nxt)
+            if after is not None and is_relu(after) and after.args[0] is nxt:
+                end, relu = after, True
+        elif is_relu(nxt) and nxt.args[0] is last:
+            end, relu = nxt, True
+        if end is None:
+            continue
+        name = "_fused_" + node.target.replace(".", "_")
+        k = 0
+        while hasattr(gm, name + (str(k) if k else "")):
+            k += 1
+        name += str(k) if k else ""
+        gm.add_submodule(name, _FusedEpilogue(layer, relu))
+        with graph.inserting_before(end):
+            args = (node.args[0],) if residual is None else (node.args[0], residual)
+            new = graph.call_module(name, args)
+        end.replace_all_uses_with(new)
+        # erase the replaced chain, consumers first
+        chain, cur = [end], end
+        while cur is not node:
+            cur = cur.args[0] if (cur.args[0] is not residual or not is_add(cur)) else cur.args[1]
+            chain.append(cur)
+        for n in chain:
+            graph.erase_node(n)
+        fused += 1
+    graph.lint()
+    gm.recompile()
+    return gm, fused
 
 
 class _MaxPool2dNHWC(nn.Module):
