@@ -117,6 +117,111 @@ __global__ __launch_bounds__(256) void dwconv_image_kernel(const _Float16 *__res
     store8(ep, p * C + c0, c0, C, acc, vec);
 }
 
+// The common case -- 3 x 3 taps, no dilation, whole groups of 8 channels, fewer than 2^31 threads. A thread owns
+// 8 channels of PX horizontally adjacent output positions: the columns their windows share are loaded once
+// (for stride 1, PX + 2 columns per row instead of 3 PX), the 8 weights of a tap are expanded to floats once
+// for all PX positions, and the index arithmetic is multiply-high (FastDiv). All loads of a row are in
+// flight together; taps outside the image read the clamped pixel and are replaced by zero. Per output the
+// taps are accumulated in the same order as in dwconv_image_kernel (fp32, every product exact).
+template <int PX, int SX>
+__global__ __launch_bounds__(256) void dwconv3x3_image_kernel(const _Float16 *__restrict__ x, const uint32_t *__restrict__ words,
+                                                              uint32_t total, int C, int H, int W, int Wo, FastDiv by_g,
+                                                              FastDiv by_wg, FastDiv by_ho, int sy, int py, int px,
+                                                              DwEpilogue ep) {
+    constexpr int NC = (PX - 1) * SX + 3;                          // input columns the PX windows cover
+    const uint32_t id = blockIdx.x * 256u + threadIdx.x;
+    if (id >= total) return;
+    int cg, wg, oh;
+    const uint32_t p = by_g.divmod(id, cg);                         // channel group fastest: neighbours share a pixel
+    const uint32_t r = by_wg.divmod(p, wg);
+    const int b = (int)by_ho.divmod(r, oh);
+    const int c0 = cg * 8, ow0 = wg * PX, iw0 = ow0 * SX - px;
+    const int64_t Q = (C + 15) / 16;
+    const _Float16 *img = x + (int64_t)b * H * W * C + c0;
+
+    float acc[PX][8];
+#pragma unroll
+    for (int q = 0; q < PX; q++)
+#pragma unroll
+        for (int e = 0; e < 8; e++) acc[q][e] = 0.f;
+
+#pragma unroll 1
+    for (int i = 0; i < 3; i++) {                                  // one row at a time: its NC loads in flight, few registers
+        const int ih = oh * sy - py + i;
+        const bool row_in = (unsigned)ih < (unsigned)H;
+        const int ihc = ih < 0 ? 0 : (ih >= H ? H - 1 : ih);
+        const _Float16 *row = img + (int64_t)ihc * W * C;
+        half8 v[NC];
+#pragma unroll
+        for (int c = 0; c < NC; c++) {
+            const int iw = iw0 + c, iwc = iw < 0 ? 0 : (iw >= W ? W - 1 : iw);
+            v[c] = *reinterpret_cast<const half8 *>(row + (int64_t)iwc * C);
+        }
+#pragma unroll
+        for (int c = 0; c < NC; c++) {
+            const int iw = iw0 + c;
+            if (!(row_in && (unsigned)iw < (unsigned)W)) v[c] = half8{0, 0, 0, 0, 0, 0, 0, 0};
+        }
+#pragma unroll
+        for (int j = 0; j < 3; j++) {
+            const uint32_t codes = codes8(words, Q, i * 3 + j, c0);
+            float w[8];
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const uint32_t cd = (codes >> (30 - 2 * e)) & 3u;   // 01 -> +1, 10 -> -1, 00 / 11 -> 0
+                w[e] = (float)((int)(cd & 1u) - (int)(cd >> 1));
+            }
+#pragma unroll
+            for (int q = 0; q < PX; q++)
+#pragma unroll
+                for (int e = 0; e < 8; e++) acc[q][e] = __builtin_fmaf((float)v[q * SX + j][e], w[e], acc[q][e]);
+        }
+    }
+    // epilogue: the 8 channels' scale and bias once for all PX positions, 16-byte accesses throughout
+    floatx4 sc[2] = {floatx4{1.f, 1.f, 1.f, 1.f}, floatx4{1.f, 1.f, 1.f, 1.f}};
+    floatx4 bi[2] = {floatx4{0.f, 0.f, 0.f, 0.f}, floatx4{0.f, 0.f, 0.f, 0.f}};
+    if (ep.scale) { sc[0] = *reinterpret_cast<const floatx4 *>(ep.scale + c0); sc[1] = *reinterpret_cast<const floatx4 *>(ep.scale + c0 + 4); }
+    if (ep.bias) { bi[0] = *reinterpret_cast<const floatx4 *>(ep.bias + c0); bi[1] = *reinterpret_cast<const floatx4 *>(ep.bias + c0 + 4); }
+#pragma unroll
+    for (int q = 0; q < PX; q++) {
+        if (ow0 + q >= Wo) break;
+        const int64_t o = ((int64_t)(r * (uint32_t)Wo) + ow0 + q) * C + c0;
+        float v[8];
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            v[e] = acc[q][e];
+            if (ep.scale) v[e] *= sc[e >> 2][e & 3];               // same operations, same order as store8
+            if (ep.bias) v[e] += bi[e >> 2][e & 3];
+        }
+        if (ep.residual) {
+            if (ep.y_f16) {
+                const half8 rs = *reinterpret_cast<const half8 *>(static_cast<const _Float16 *>(ep.residual) + o);
+#pragma unroll
+                for (int e = 0; e < 8; e++) v[e] += (float)rs[e];
+            } else {
+                const floatx4 r0 = *reinterpret_cast<const floatx4 *>(static_cast<const float *>(ep.residual) + o);
+                const floatx4 r1 = *reinterpret_cast<const floatx4 *>(static_cast<const float *>(ep.residual) + o + 4);
+#pragma unroll
+                for (int e = 0; e < 4; e++) { v[e] += r0[e]; v[4 + e] += r1[e]; }
+            }
+        }
+        if (ep.relu) {
+#pragma unroll
+            for (int e = 0; e < 8; e++) v[e] = v[e] > 0.f ? v[e] : 0.f;
+        }
+        if (ep.y_f16) {
+            half8 h;
+#pragma unroll
+            for (int e = 0; e < 8; e++) h[e] = (_Float16)v[e];
+            *reinterpret_cast<half8 *>(static_cast<_Float16 *>(ep.y) + o) = h;
+        } else {
+            float *yp = static_cast<float *>(ep.y) + o;
+            *reinterpret_cast<floatx4 *>(yp) = floatx4{v[0], v[1], v[2], v[3]};
+            *reinterpret_cast<floatx4 *>(yp + 4) = floatx4{v[4], v[5], v[6], v[7]};
+        }
+    }
+}
+
 // Unfolded patches [P][T][C], fp32 (the reference's calling convention) or fp16.
 template <typename T>
 __global__ __launch_bounds__(256) void dwconv_patches_kernel(const T *__restrict__ x, const uint32_t *__restrict__ words,
@@ -246,6 +351,23 @@ int tmq_ternary_dwconv2d(const void *x, const tmq_conv_shape *s, const uint32_t 
     const size_t ya = y_f16 ? 16 : 16;
     const int vec = (s->C % 8 == 0) && aligned_for(x, 16) && aligned_for(y, ya) && (!e.residual || aligned_for(e.residual, ya));
     DwEpilogue ep{e.scale, e.bias, e.residual, y, e.relu, y_f16};
+    if (vec && aligned_for(e.scale, 16) && aligned_for(e.bias, 16) && s->ky == 3 && s->kx == 3 && s->dy == 1 && s->dx == 1 &&
+        (s->sx == 1 || s->sx == 2) && total < (int64_t)0x7FFFFFFF &&
+        (int64_t)s->B * ho * wo < (int64_t)0x7FFFFFFF) {
+        const int px_per_thread = s->sx == 1 ? 4 : 2;
+        const int64_t wgroups = (wo + px_per_thread - 1) / px_per_thread, G = s->C / 8;
+        const int64_t threads = (int64_t)s->B * ho * wgroups * G, nblocks = (threads + 255) / 256;
+        const FastDiv by_g((uint32_t)G), by_wg((uint32_t)wgroups), by_ho((uint32_t)ho);
+        if (s->sx == 1)
+            hipLaunchKernelGGL((dwconv3x3_image_kernel<4, 1>), dim3((uint32_t)nblocks), dim3(256), 0, as_stream(stream),
+                               static_cast<const _Float16 *>(x), words, (uint32_t)threads, s->C, s->H, s->W, wo, by_g, by_wg,
+                               by_ho, s->sy, s->py, s->px, ep);
+        else
+            hipLaunchKernelGGL((dwconv3x3_image_kernel<2, 2>), dim3((uint32_t)nblocks), dim3(256), 0, as_stream(stream),
+                               static_cast<const _Float16 *>(x), words, (uint32_t)threads, s->C, s->H, s->W, wo, by_g, by_wg,
+                               by_ho, s->sy, s->py, s->px, ep);
+        return check_launch();
+    }
     hipLaunchKernelGGL(dwconv_image_kernel, dim3((uint32_t)blocks), dim3(256), 0, as_stream(stream),
                        static_cast<const _Float16 *>(x), words, s->B, s->C, s->H, s->W, ho, wo, s->ky, s->kx, s->sy, s->sx,
                        s->py, s->px, s->dy, s->dx, vec, ep);
