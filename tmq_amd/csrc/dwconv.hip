@@ -82,6 +82,58 @@ __device__ __forceinline__ void store8(const DwEpilogue &ep, int64_t o, int64_t 
     }
 }
 
+// The same epilogue as store8 for whole groups of 8 channels with 16-byte aligned tensors: scale and bias
+// come in as two 16-byte loads each (once per thread), residual and result move 16 bytes at a time. Same
+// operations in the same order as store8.
+struct ChannelConstants {
+    floatx4 sc[2], bi[2];
+};
+
+__device__ __forceinline__ ChannelConstants load_channel_constants(const DwEpilogue &ep, int64_t c0) {
+    ChannelConstants cc;
+    cc.sc[0] = cc.sc[1] = floatx4{1.f, 1.f, 1.f, 1.f};
+    cc.bi[0] = cc.bi[1] = floatx4{0.f, 0.f, 0.f, 0.f};
+    if (ep.scale) { cc.sc[0] = *reinterpret_cast<const floatx4 *>(ep.scale + c0); cc.sc[1] = *reinterpret_cast<const floatx4 *>(ep.scale + c0 + 4); }
+    if (ep.bias) { cc.bi[0] = *reinterpret_cast<const floatx4 *>(ep.bias + c0); cc.bi[1] = *reinterpret_cast<const floatx4 *>(ep.bias + c0 + 4); }
+    return cc;
+}
+
+__device__ __forceinline__ void store8_vec(const DwEpilogue &ep, const ChannelConstants &cc, int64_t o, const float (&acc)[8]) {
+    float v[8];
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+        v[e] = acc[e];
+        if (ep.scale) v[e] *= cc.sc[e >> 2][e & 3];
+        if (ep.bias) v[e] += cc.bi[e >> 2][e & 3];
+    }
+    if (ep.residual) {
+        if (ep.y_f16) {
+            const half8 rs = *reinterpret_cast<const half8 *>(static_cast<const _Float16 *>(ep.residual) + o);
+#pragma unroll
+            for (int e = 0; e < 8; e++) v[e] += (float)rs[e];
+        } else {
+            const floatx4 r0 = *reinterpret_cast<const floatx4 *>(static_cast<const float *>(ep.residual) + o);
+            const floatx4 r1 = *reinterpret_cast<const floatx4 *>(static_cast<const float *>(ep.residual) + o + 4);
+#pragma unroll
+            for (int e = 0; e < 4; e++) { v[e] += r0[e]; v[4 + e] += r1[e]; }
+        }
+    }
+    if (ep.relu) {
+#pragma unroll
+        for (int e = 0; e < 8; e++) v[e] = v[e] > 0.f ? v[e] : 0.f;
+    }
+    if (ep.y_f16) {
+        half8 h;
+#pragma unroll
+        for (int e = 0; e < 8; e++) h[e] = (_Float16)v[e];
+        *reinterpret_cast<half8 *>(static_cast<_Float16 *>(ep.y) + o) = h;
+    } else {
+        float *yp = static_cast<float *>(ep.y) + o;
+        *reinterpret_cast<floatx4 *>(yp) = floatx4{v[0], v[1], v[2], v[3]};
+        *reinterpret_cast<floatx4 *>(yp + 4) = floatx4{v[4], v[5], v[6], v[7]};
+    }
+}
+
 // NHWC fp16 image. grid.x covers P * ceil(C / 8) threads.
 __global__ __launch_bounds__(256) void dwconv_image_kernel(const _Float16 *__restrict__ x, const uint32_t *__restrict__ words,
                                                            int B, int C, int H, int W, int Ho, int Wo, int ky, int kx,
@@ -114,7 +166,8 @@ __global__ __launch_bounds__(256) void dwconv_image_kernel(const _Float16 *__res
             }
         }
     }
-    store8(ep, p * C + c0, c0, C, acc, vec);
+    if (vec & 2) store8_vec(ep, load_channel_constants(ep, c0), p * C + c0, acc);
+    else store8(ep, p * C + c0, c0, C, acc, vec);
 }
 
 // The common case -- 3 x 3 taps, no dilation, whole groups of 8 channels, fewer than 2^31 threads. A thread owns
@@ -178,47 +231,11 @@ __global__ __launch_bounds__(256) void dwconv3x3_image_kernel(const _Float16 *__
         }
     }
     // epilogue: the 8 channels' scale and bias once for all PX positions, 16-byte accesses throughout
-    floatx4 sc[2] = {floatx4{1.f, 1.f, 1.f, 1.f}, floatx4{1.f, 1.f, 1.f, 1.f}};
-    floatx4 bi[2] = {floatx4{0.f, 0.f, 0.f, 0.f}, floatx4{0.f, 0.f, 0.f, 0.f}};
-    if (ep.scale) { sc[0] = *reinterpret_cast<const floatx4 *>(ep.scale + c0); sc[1] = *reinterpret_cast<const floatx4 *>(ep.scale + c0 + 4); }
-    if (ep.bias) { bi[0] = *reinterpret_cast<const floatx4 *>(ep.bias + c0); bi[1] = *reinterpret_cast<const floatx4 *>(ep.bias + c0 + 4); }
+    const ChannelConstants cc = load_channel_constants(ep, c0);
 #pragma unroll
     for (int q = 0; q < PX; q++) {
         if (ow0 + q >= Wo) break;
-        const int64_t o = ((int64_t)(r * (uint32_t)Wo) + ow0 + q) * C + c0;
-        float v[8];
-#pragma unroll
-        for (int e = 0; e < 8; e++) {
-            v[e] = acc[q][e];
-            if (ep.scale) v[e] *= sc[e >> 2][e & 3];               // same operations, same order as store8
-            if (ep.bias) v[e] += bi[e >> 2][e & 3];
-        }
-        if (ep.residual) {
-            if (ep.y_f16) {
-                const half8 rs = *reinterpret_cast<const half8 *>(static_cast<const _Float16 *>(ep.residual) + o);
-#pragma unroll
-                for (int e = 0; e < 8; e++) v[e] += (float)rs[e];
-            } else {
-                const floatx4 r0 = *reinterpret_cast<const floatx4 *>(static_cast<const float *>(ep.residual) + o);
-                const floatx4 r1 = *reinterpret_cast<const floatx4 *>(static_cast<const float *>(ep.residual) + o + 4);
-#pragma unroll
-                for (int e = 0; e < 4; e++) { v[e] += r0[e]; v[4 + e] += r1[e]; }
-            }
-        }
-        if (ep.relu) {
-#pragma unroll
-            for (int e = 0; e < 8; e++) v[e] = v[e] > 0.f ? v[e] : 0.f;
-        }
-        if (ep.y_f16) {
-            half8 h;
-#pragma unroll
-            for (int e = 0; e < 8; e++) h[e] = (_Float16)v[e];
-            *reinterpret_cast<half8 *>(static_cast<_Float16 *>(ep.y) + o) = h;
-        } else {
-            float *yp = static_cast<float *>(ep.y) + o;
-            *reinterpret_cast<floatx4 *>(yp) = floatx4{v[0], v[1], v[2], v[3]};
-            *reinterpret_cast<floatx4 *>(yp + 4) = floatx4{v[4], v[5], v[6], v[7]};
-        }
+        store8_vec(ep, cc, ((int64_t)(r * (uint32_t)Wo) + ow0 + q) * C + c0, acc[q]);
     }
 }
 
@@ -349,9 +366,10 @@ int tmq_ternary_dwconv2d(const void *x, const tmq_conv_shape *s, const uint32_t 
     if (blocks > 0x7FFFFFFF) return TMQ_ERR_TOO_LARGE;
     const int y_f16 = e.y_dtype == TMQ_F16;
     const size_t ya = y_f16 ? 16 : 16;
-    const int vec = (s->C % 8 == 0) && aligned_for(x, 16) && aligned_for(y, ya) && (!e.residual || aligned_for(e.residual, ya));
+    int vec = (s->C % 8 == 0) && aligned_for(x, 16) && aligned_for(y, ya) && (!e.residual || aligned_for(e.residual, ya));
+    if (vec && aligned_for(e.scale, 16) && aligned_for(e.bias, 16)) vec |= 2;       // the 16-byte epilogue as well
     DwEpilogue ep{e.scale, e.bias, e.residual, y, e.relu, y_f16};
-    if (vec && aligned_for(e.scale, 16) && aligned_for(e.bias, 16) && s->ky == 3 && s->kx == 3 && s->dy == 1 && s->dx == 1 &&
+    if ((vec & 2) && s->ky == 3 && s->kx == 3 && s->dy == 1 && s->dx == 1 &&
         (s->sx == 1 || s->sx == 2) && total < (int64_t)0x7FFFFFFF &&
         (int64_t)s->B * ho * wo < (int64_t)0x7FFFFFFF) {
         const int px_per_thread = s->sx == 1 ? 4 : 2;
