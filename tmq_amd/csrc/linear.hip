@@ -1162,7 +1162,7 @@ int tmq_ternary_linear(const void *x, int x_dtype, int64_t M, int64_t K, const v
     // 11008 x 4096 7.2 -> 6.2 us, even at 4096^2.
     if (!x32 && stream_dense_ok(x, M, K) && K >= 8 * kKB)
         return launch_stream_dense(x, M, K, native, N, ep.scale, ep.bias, ep.residual, ep.relu, y, ep.y_dtype == TMQ_F16, stream);
-    // ... and at most 8 fp32 rows (the reference's GEMV convention): its fp32 form (M = 1 at 4096^2: 6.0 -> 4.5 us,
+    // ... and a few fp32 rows (the reference's GEMV convention; up to 8, up to 16 on short reductions): its fp32 form (M = 1 at 4096^2: 6.0 -> 4.5 us,
     // M = 8 at 8192^2: 24 -> 17 us)
     if (x32 && stream32_dense_ok(x, M, K) && K >= 8 * kKB)
         return launch_stream32_dense(x, M, K, native, N, ep.scale, ep.bias, ep.residual, ep.relu, y, ep.y_dtype == TMQ_F16, stream);

@@ -644,7 +644,7 @@ int launch_stream(const void *x, const void *native, int64_t M, int64_t K, int64
     return check_launch();
 }
 
-// ---- weight stream, fp32 activations, at most 8 rows -------------------------------------------------
+// ---- weight stream, fp32 activations, at most 16 rows -------------------------------------------------
 // The reference's GEMV (ternary_mvm_cuda) takes an fp32 vector. Same plan as stream_kernel with 16 channels
 // per workgroup, but the activations of a block (256 fp32 = 1 KiB per row, one 16-byte load per lane) travel
 // through registers: each value is split into two fp16 terms (hi = fp16(x), lo = fp16(x - hi), together 22
@@ -813,10 +813,11 @@ bool stream_dense_ok(const void *x, int64_t M, int64_t K) {
     return M >= 1 && M <= 16 && (K % kKB == 0) && aligned16(x) && M * K < (int64_t)0x7FFFFFFF;
 }
 
-// At most 8 fp32 rows with whole weight blocks: the fp32 weight-stream kernel (with 9..16 rows its
-// activations no longer fit the registers: measured slower than the older kernel on large layers).
+// fp32 rows with whole weight blocks that take the fp32 weight-stream kernel: up to 8, or up to 16 on short reductions.
 bool stream32_dense_ok(const void *x, int64_t M, int64_t K) {
-    return M >= 1 && M <= 8 && (K % kKB == 0) && aligned16(x);
+    // 9 .. 16 rows: the activations of two blocks (128 registers) only pay on short reductions -- measured faster
+    // than the older kernel at K = 2048 .. 5120 (K = N = 4096, M = 16: 11.4 -> 9.2 us), slower at K >= 8192
+    return M >= 1 && (M <= 8 || (M <= 16 && K <= 6144)) && (K % kKB == 0) && aligned16(x);
 }
 
 int launch_stream32_dense(const void *x, int64_t M, int64_t K, const void *native, int64_t N, const float *scale,
@@ -825,7 +826,8 @@ int launch_stream32_dense(const void *x, int64_t M, int64_t K, const void *nativ
     if (M == 1) return launch_stream32<1>(x, native, M, K, N, ep, stream);
     if (M == 2) return launch_stream32<2>(x, native, M, K, N, ep, stream);
     if (M <= 4) return launch_stream32<4>(x, native, M, K, N, ep, stream);
-    return launch_stream32<8>(x, native, M, K, N, ep, stream);
+    if (M <= 8) return launch_stream32<8>(x, native, M, K, N, ep, stream);
+    return launch_stream32<16>(x, native, M, K, N, ep, stream);
 }
 
 // Geometry of the weight-stream kernel (stream_dense_ok must hold). Rows staged: the power of two >= M.
