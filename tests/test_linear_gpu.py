@@ -159,7 +159,9 @@ STREAM = [  # at most 16 fp16 rows, K a multiple of 256 and >= 2048: every geome
     (1, 2048, 70, False), (2, 4096, 1000, False), (3, 2304, 520, False), (4, 2048, 8200, False), (4, 2560, 4096, False),
     (5, 4096, 12300, False), (7, 2048, 8200, False), (8, 3072, 4100, False), (9, 4096, 12304, False), (12, 2048, 8192, False),
     (16, 16384, 4096, False), (13, 2304, 48, False), (6, 8192, 28672, False), (1, 28672, 8192, False),
-    # at most 4 fp32 rows: the fp32 form of the weight-stream kernel
+    # fp32 rows on the small tiles of the register-staged split-reduction kernel
+    (17, 4096, 4096, True), (64, 4096, 1024, True), (100, 2048, 1000, True),
+    # a few fp32 rows: the fp32 form of the weight-stream kernel
     (4, 2048, 8200, True), (2, 8192, 1024, True), (3, 2560, 40, True), (1, 2048, 16, True), (8, 2048, 8200, True), (6, 4096, 100, True), (16, 4096, 1000, True), (11, 2304, 8200, True), (13, 6144, 64, True),
 ]
 

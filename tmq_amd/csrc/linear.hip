@@ -1028,8 +1028,13 @@ int mid_rows(const void *x, int64_t M, int64_t K, const void *native, int64_t N,
              void *stream) {
     auto wgs = [&](int bm, int bn) { return ((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
     if constexpr (X32) {
-        if ((K % kKB == 0) && aligned16(x) && (uint64_t)M * (uint64_t)K * 4 < (1ull << 32))
-            return launch_mid_lds<2, 4, 8, true>(x, M, K, native, N, ep, y, stream);
+        if ((K % kKB == 0) && aligned16(x) && (uint64_t)M * (uint64_t)K * 4 < (1ull << 32)) {
+            // the smallest tile that still fills one pass over the CUs, as for fp16 rows (mid.hip)
+            // (K = N = 4096, M = 17: 13.7 -> 8.3 us; K = 4096, N = 1024, M = 64: 13.8 -> 8.0 us)
+            if (wgs(32, 64) >= 192) return launch_mid_lds<2, 4, 8, true>(x, M, K, native, N, ep, y, stream);
+            if (wgs(32, 32) >= 192) return launch_mid_lds<2, 2, 8, true>(x, M, K, native, N, ep, y, stream);
+            return launch_mid_lds<1, 2, 8, true>(x, M, K, native, N, ep, y, stream);
+        }
     } else {
         if (mid_dense_ok(x, M, K))
             return launch_mid_dense(x, M, K, native, N, ep.scale, ep.bias, ep.residual, ep.relu, y,
