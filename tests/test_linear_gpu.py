@@ -159,6 +159,8 @@ STREAM = [  # at most 16 fp16 rows, K a multiple of 256 and >= 2048: every geome
     (1, 2048, 70, False), (2, 4096, 1000, False), (3, 2304, 520, False), (4, 2048, 8200, False), (4, 2560, 4096, False),
     (5, 4096, 12300, False), (7, 2048, 8200, False), (8, 3072, 4100, False), (9, 4096, 12304, False), (12, 2048, 8192, False),
     (16, 16384, 4096, False), (13, 2304, 48, False), (6, 8192, 28672, False), (1, 28672, 8192, False),
+    # 9 .. 16 rows with odd block counts per wavefront: every drain of the static pipeline
+    (12, 6144, 520, False), (16, 7168, 100, False), (10, 5120, 8200, False), (9, 12800, 64, False),
     # fp32 rows on the small tiles of the register-staged split-reduction kernel
     (17, 4096, 4096, True), (64, 4096, 1024, True), (100, 2048, 1000, True),
     # a few fp32 rows: the fp32 form of the weight-stream kernel
