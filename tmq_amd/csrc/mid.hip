@@ -214,7 +214,7 @@ __device__ __forceinline__ void reduce_and_store(unsigned char *smem, const floa
     }
 }
 
-template <int WM, int WN, int WAVES, class Rows>
+template <int WM, int WN, int WAVES, bool BLK, class Rows>
 __global__ __launch_bounds__(64 * WAVES) void mid_kernel(Rows rows, const u32x4 *__restrict__ native, int64_t M, int Kb,
                                                          int npairs, int64_t N, int64_t Nb, int tiles_n,
                                                          MidEpilogue ep) {
@@ -242,6 +242,84 @@ __global__ __launch_bounds__(64 * WAVES) void mid_kernel(Rows rows, const u32x4 
     typename Rows::template State<WM> st;
     rows.template prepare<WM>(st, m0, lane);
 
+    // operand (row j, chunk ch) of a fragment sits at position ch ^ ((j / 2) % 8) of its row
+    const int key = (j >> 1) & 7;
+    const unsigned char *rd = win + j * 128;
+
+    if constexpr (BLK) {
+        // The reduction dealt out in whole weight blocks (4 pairs): wavefront kg takes blocks kg, kg + WAVES, ...
+        // A lane's 16 bytes of a block arrive with one load per channel block (instead of four dword loads, one per
+        // pair: the CU's vector-memory pipeline is what this kernel keeps busiest), one block ahead; the
+        // activations go pair by pair through the two slots as below.
+        const u32x4 *wbb[WN];
+#pragma unroll
+        for (int nj = 0; nj < WN; nj++) wbb[nj] = reinterpret_cast<const u32x4 *>(wb[nj]);
+        const int nt = Kb > kg ? (Kb - kg + WAVES - 1) / WAVES : 0;
+        auto wloadb = [&](u32x4 (&w)[WN], int t) {
+            const int64_t kb = kg + (int64_t)t * WAVES;
+#pragma unroll
+            for (int nj = 0; nj < WN; nj++) w[nj] = wbb[nj][kb * 64];
+        };
+        auto fillb = [&](int slot, int t, int q) {
+            const typename Rows::Pair pr = rows.pair(((int64_t)(kg + t * WAVES) * 4 + q) * 64);
+#pragma unroll
+            for (int mi = 0; mi < WM; mi++)
+#pragma unroll
+                for (int c = 0; c < 2; c++)
+                    load_to_lds(rows.template source<WM>(st, pr, mi, c, lane), win + slot * kSlot + mi * kFrag + c * 1024);
+        };
+        if (nt > 0) {
+            u32x4 wq[2][WN];
+            wloadb(wq[0], 0);
+            fillb(0, 0, 0);
+            constexpr int kWaitW = (WN & 15) | (7 << 4) | (15 << 8) | ((WN >> 4) << 14);   // vmcnt(WN)
+            // pair q of block t; `par` = parity of t (weight register set), slot = q % 2
+            auto step = [&](int t, auto par_tag, auto q_tag) {
+                constexpr int par = decltype(par_tag)::value, q = decltype(q_tag)::value, slot = q & 1;
+                const bool more = t + 1 < nt;
+                // this pair's activations must have landed; at q == 3 the next block's weights, issued one
+                // step ago behind them, may still be on their way
+                if (q == 3 && more) __builtin_amdgcn_s_waitcnt(kWaitW);
+                else __builtin_amdgcn_s_waitcnt(0x0F70);
+                __builtin_amdgcn_sched_barrier(0);
+                half8 a[2][WM];
+#pragma unroll
+                for (int s2 = 0; s2 < 2; s2++)
+#pragma unroll
+                    for (int mi = 0; mi < WM; mi++)
+                        a[s2][mi] = *reinterpret_cast<const half8 *>(rd + slot * kSlot + mi * kFrag + (((4 * s2 + g) ^ key) * 16));
+                __builtin_amdgcn_sched_barrier(0);
+                if (q < 3) fillb(slot ^ 1, t, q + 1);
+                else if (more) fillb(slot ^ 1, t + 1, 0);
+                if (q == 2 && more) wloadb(wq[par ^ 1], t + 1);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int s2 = 0; s2 < 2; s2++)
+#pragma unroll
+                    for (int nj = 0; nj < WN; nj++) {
+                        const half8 w = decode_step(wq[par][nj][q], s2);
+#pragma unroll
+                        for (int mi = 0; mi < WM; mi++) acc[mi][nj] = mfma16(w, a[s2][mi], acc[mi][nj]);
+                    }
+                __builtin_amdgcn_sched_barrier(0);
+            };
+            auto block = [&](int t, auto par_tag) {
+                step(t, par_tag, std::integral_constant<int, 0>{});
+                step(t, par_tag, std::integral_constant<int, 1>{});
+                step(t, par_tag, std::integral_constant<int, 2>{});
+                step(t, par_tag, std::integral_constant<int, 3>{});
+            };
+            int t = 0;
+            for (; t + 2 <= nt; t += 2) {
+                block(t, std::integral_constant<int, 0>{});
+                block(t + 1, std::integral_constant<int, 1>{});
+            }
+            if (t < nt) block(t, std::integral_constant<int, 0>{});
+        }
+        reduce_and_store<WM, WN, WAVES>(smem, acc, kg, lane, m0, n0, M, N, ep);
+        return;
+    }
+
     // the reduction is dealt out in pairs: wavefront kg takes pairs kg, kg + WAVES, ...
     const int np = npairs > kg ? (npairs - kg + WAVES - 1) / WAVES : 0;
     auto wload = [&](uint32_t (&w)[WN], int p) {
@@ -258,10 +336,6 @@ __global__ __launch_bounds__(64 * WAVES) void mid_kernel(Rows rows, const u32x4 
             for (int c = 0; c < 2; c++)
                 load_to_lds(rows.template source<WM>(st, pr, mi, c, lane), win + slot * kSlot + mi * kFrag + c * 1024);
     };
-    // operand (row j, chunk ch) of a fragment sits at position ch ^ ((j / 2) % 8) of its row
-    const int key = (j >> 1) & 7;
-    const unsigned char *rd = win + j * 128;
-
     if (np > 0) {
         uint32_t wq[2][WN];
         wload(wq[0], 0);
@@ -308,7 +382,7 @@ __global__ __launch_bounds__(64 * WAVES) void mid_kernel(Rows rows, const u32x4 
     reduce_and_store<WM, WN, WAVES>(smem, acc, kg, lane, m0, n0, M, N, ep);
 }
 
-template <int WM, int WN, int WAVES, class Rows>
+template <int WM, int WN, int WAVES, class Rows, bool BLK = false>
 int launch(const Rows &rows, const void *native, int64_t M, int64_t K, int64_t N, const MidEpilogue &ep, void *stream) {
     constexpr int BM = 16 * WM, BN = 16 * WN;
     const int64_t tm = (M + BM - 1) / BM, tn = (N + BN - 1) / BN, Kb = native_blocks_k(K);
@@ -317,7 +391,7 @@ int launch(const Rows &rows, const void *native, int64_t M, int64_t K, int64_t N
     constexpr size_t redb = (size_t)WAVES * WM * WN * (1024 + 64);
     constexpr size_t lds = win > redb ? win : redb;
     static_assert(lds <= 152 * 1024, "LDS budget");
-    auto kernel = mid_kernel<WM, WN, WAVES, Rows>;
+    auto kernel = mid_kernel<WM, WN, WAVES, BLK, Rows>;
     if (lds > 64 * 1024) {
         // opt in to the large LDS (per device; the attribute is sticky, setting it again is cheap)
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
@@ -760,6 +834,12 @@ template <class Rows>
 int dispatch(const Rows &rows, const void *native, int64_t M, int64_t K, int64_t N, const MidEpilogue &ep,
              void *stream) {
     const int64_t npairs = (K + 63) / 64, tn = (N + 63) / 64;
+    // Whole weight blocks per wavefront (one 16-byte load per lane and block instead of four dword loads) when the
+    // blocks deal out evenly (or there are many); else pairs (K = 4608 over 4 wavefronts: 18 blocks would leave two
+    // wavefronts with five and two with four, which costs more than the loads save).
+    // M = 256 at K = N = 4096: 14.5 -> 13.1 us, M = 128 at K = 8192: 15.2 -> 12.3 us.
+    const int64_t Kb = native_blocks_k(K);
+    auto by_blocks = [&](int waves) { return K % 256 == 0 && (Kb % waves == 0 || Kb >= 8 * waves); };
     // 64 x 128 tiles with four wavefronts read each activation row half as often (the weights are
     // 2 bits, so a wide tile is the cheap direction) but a pass over them takes ~1.7 times as long as
     // one over 64 x 64 tiles with eight wavefronts; both run one workgroup per CU. They win when they
@@ -768,7 +848,8 @@ int dispatch(const Rows &rows, const void *native, int64_t M, int64_t K, int64_t
     {
         const int64_t tm = (M + 63) / 64, passes64 = (tm * tn + 255) / 256, passes128 = (tm * ((N + 127) / 128) + 255) / 256;
         if (npairs >= 16 && passes64 >= 2 && 17 * passes128 < 10 * passes64)
-            return launch<4, 8, 4, Rows>(rows, native, M, K, N, ep, stream);
+            return by_blocks(4) ? launch<4, 8, 4, Rows, true>(rows, native, M, K, N, ep, stream)
+                                : launch<4, 8, 4, Rows>(rows, native, M, K, N, ep, stream);
     }
     // Otherwise the largest of 64 x 64, 32 x 64, 32 x 32, 16 x 32 that still gives most CUs a tile (measured
     // at K = N = 4096: M = 64 10.0 -> 7.6 us with 32 x 32, M = 17 9.7 -> 6.4 us with 16 x 32, while
@@ -782,6 +863,14 @@ int dispatch(const Rows &rows, const void *native, int64_t M, int64_t K, int64_t
     while (waves < 8 && tiles(bm, bn) * waves < 2560 && npairs >= 4 * waves) waves *= 2;
     auto go = [&](auto wm_tag, auto wn_tag) {
         constexpr int WM = decltype(wm_tag)::value, WN = decltype(wn_tag)::value;
+        if (by_blocks(waves)) {
+            switch (waves) {
+                case 1: return launch<WM, WN, 1, Rows, true>(rows, native, M, K, N, ep, stream);
+                case 2: return launch<WM, WN, 2, Rows, true>(rows, native, M, K, N, ep, stream);
+                case 4: return launch<WM, WN, 4, Rows, true>(rows, native, M, K, N, ep, stream);
+                default: return launch<WM, WN, 8, Rows, true>(rows, native, M, K, N, ep, stream);
+            }
+        }
         switch (waves) {
             case 1: return launch<WM, WN, 1, Rows>(rows, native, M, K, N, ep, stream);
             case 2: return launch<WM, WN, 2, Rows>(rows, native, M, K, N, ep, stream);
