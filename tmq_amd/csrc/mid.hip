@@ -129,7 +129,7 @@ __device__ __forceinline__ void load_to_lds(const void *src, unsigned char *dst)
 // Scale (already divided by the weight unit) and bias of a thread's four output columns in the epilogue
 // below. Fetched before the main loop where registers allow: asked for only after it, the two loads are a
 // trip to memory that nothing overlaps.
-struct ColumnConstants {
+struct ThreadColumns {
     floatx4 sc, bi;
 };
 
@@ -139,9 +139,9 @@ __device__ __forceinline__ bool epilogue_vectorised(int64_t N, const MidEpilogue
 }
 
 template <int WN>
-__device__ __forceinline__ ColumnConstants load_column_constants(int64_t n0, int64_t N, const MidEpilogue &ep) {
+__device__ __forceinline__ ThreadColumns load_column_constants(int64_t n0, int64_t N, const MidEpilogue &ep) {
     const int64_t n = n0 + (int)(threadIdx.x % (4 * WN)) * 4;
-    ColumnConstants c{{1.f, 1.f, 1.f, 1.f}, {0.f, 0.f, 0.f, 0.f}};
+    ThreadColumns c{{1.f, 1.f, 1.f, 1.f}, {0.f, 0.f, 0.f, 0.f}};
     if (n < N) {
         if (epilogue_vectorised(N, ep)) {
             if (ep.scale) c.sc = *reinterpret_cast<const floatx4 *>(ep.scale + n);
@@ -170,7 +170,7 @@ __device__ __forceinline__ ColumnConstants load_column_constants(int64_t n0, int
 template <int WM, int WN, int WAVES>
 __device__ __forceinline__ void reduce_and_store(unsigned char *smem, const floatx4 (&acc)[WM][WN], int kg, int lane,
                                                  int64_t m0, int64_t n0, int64_t M, int64_t N, const MidEpilogue &ep,
-                                                 const ColumnConstants &cc) {
+                                                 const ThreadColumns &cc) {
     constexpr int NF = WM * WN;
     const int j = lane & 15, g = lane >> 4;
     constexpr int kFragPitch = 1024 + 64;                       // bytes; +64 spreads the nj over the banks
@@ -289,7 +289,7 @@ __global__ __launch_bounds__(64 * WAVES) void mid_kernel(Rows rows, const u32x4 
     }
     typename Rows::template State<WM> st;
     rows.template prepare<WM>(st, m0, lane);
-    const ColumnConstants cc = load_column_constants<WN>(n0, N, ep);
+    const ThreadColumns cc = load_column_constants<WN>(n0, N, ep);
 
     // operand (row j, chunk ch) of a fragment sits at position ch ^ ((j / 2) % 8) of its row
     const int key = (j >> 1) & 7;
