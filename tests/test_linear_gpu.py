@@ -149,6 +149,9 @@ MID = [  # batches between the skinny kernel and the big-tile kernel, both activ
     (4, 8192, 1024, False), (16, 8192, 1024, False), (9, 768, 48, False), (16, 2048, 8192, False),
     # 64 x 128 split-reduction tiles (chosen where they save a pass over the CUs), ragged N included
     (512, 4096, 4096, False), (384, 1024, 4100, False), (256, 8192, 8192, False),
+    # ... with pair-granular weights two pairs ahead (the weight blocks do not deal out evenly over four wavefronts):
+    # 18, 19 / 20 and 6 / 7 pairs per wavefront, i.e. every tail of the three-slot ring; ragged M and N
+    (512, 4608, 4096, False), (500, 4928, 4100, False), (512, 1600, 4096, False),
     # 32 x 32 and 16 x 32 split-reduction tiles (few rows: smaller tiles keep every CU busy), ragged shapes included
     (17, 4096, 4096, False), (64, 4096, 4096, True), (96, 2048, 2048, False), (128, 8192, 1024, False),
     (192, 8192, 1024, False), (50, 1000, 1001, False), (31, 192, 4100, True), (20, 64, 33, False),
