@@ -51,6 +51,7 @@ constexpr int kPitch = 64;       // LDS row pitch in halfs: 128 bytes = 8 chunks
 // Dense rows, any K / alignment.
 struct DenseLoader {
     static constexpr bool kDirect = false;
+    [[maybe_unused]] static constexpr bool kConv = false;
     const _Float16 *x;
     int64_t M, K;
 
@@ -93,6 +94,7 @@ struct DenseLoader {
 // re-read the last tile.
 struct DenseDirect {
     static constexpr bool kDirect = true;
+    [[maybe_unused]] static constexpr bool kConv = false;
     const _Float16 *x;
     int64_t M, K;
 
@@ -123,6 +125,7 @@ struct DenseDirect {
 template <bool VEC>
 struct ConvLoader {
     static constexpr bool kDirect = false;
+    [[maybe_unused]] static constexpr bool kConv = true;
     const _Float16 *x;
     int64_t M, K;
     int B, C, H, W, Ho, Wo, ky, kx, sy, sx, py, px, dy, dx;
@@ -200,6 +203,7 @@ struct ConvLoader {
 // window's top-left coordinate; a fetch is two unsigned compares, one add and the load.
 struct ConvLoader64 {
     static constexpr bool kDirect = true;
+    [[maybe_unused]] static constexpr bool kConv = true;
     const _Float16 *x;
     int64_t M, K;
     int B, C, H, W, Ho, Wo, ky, kx, sy, sx, py, px, dy, dx;
@@ -255,6 +259,7 @@ struct ConvLoader64 {
 // loader carries its tap (i, j) per thread, one 32-bit offset and the window's top-left coordinate per row.
 struct ConvLoaderFewC {
     static constexpr bool kDirect = true;
+    [[maybe_unused]] static constexpr bool kConv = true;
     const _Float16 *x;
     int64_t M, K;
     int B, C, H, W, Ho, Wo, ky, kx, sy, sx, py, px, dy, dx;
@@ -615,6 +620,13 @@ int launch_tile(const Loader &ld, const void *native, int64_t M, int64_t K, int6
 // Tile choice, from a sweep over M x K x N (4096^2 weights at M = 768 .. 4096 and the ResNet-18 layer
 // shapes): 128 x 256 once it gives 1.5 workgroups per CU, 128 x 128 down to one per CU, else
 // 64 x 64. Larger tiles (256 x 256, 256 x 128) and 128 x 64 never won.
+// How a tile is dealt to its wavefronts matters as much: every wavefront expands the weights of its own
+// columns (2 VALU operations per operand register), so the small tiles give each wavefront all rows and a
+// slice of the columns -- 64 x 32 of a 64 x 64 tile, 128 x 32 of a 128 x 128 tile -- instead of a square:
+// half the expansions per MFMA for twice the (cheap) operand reads from LDS. 3 x 3 convolution 64 -> 64 at
+// 56 x 56, batch 64: 31.4 -> 26.1 us (counters had shown 1500 VALU instructions per wavefront next to 144
+// MFMAs). Dense 128 x 128 tiles with two workgroups per CU are the exception (M = 2048 at K = N = 4096:
+// 51 -> 57 us, the LDS reads then cost more than the expansions save) and keep the square split.
 template <class Loader>
 Loader with_divisors(Loader ld) {
     ld.by_wo = FastDiv((uint32_t)ld.Wo);
@@ -636,10 +648,14 @@ int dispatch_tile(const Loader &ld, const void *native, int64_t M, int64_t K, in
         if (N > 128 && wgs(128, 256) >= 384)
             return two ? launch_tile_dma<8, 4, 1, 4, 2>(ld, native, M, K, N, ep, stream)
                        : launch_tile_dma<8, 4, 1, 4, 1>(ld, native, M, K, N, ep, stream);
-        if (N > 64 && wgs(128, 128) >= 256)
-            return two && wgs(128, 128) <= 256 ? launch_tile_dma<4, 4, 2, 2, 2>(ld, native, M, K, N, ep, stream)
-                                               : launch_tile_dma<4, 4, 2, 2, 1>(ld, native, M, K, N, ep, stream);
-        return launch_tile_dma<2, 4, 2, 1, 1>(ld, native, M, K, N, ep, stream);
+        if (N > 64 && wgs(128, 128) >= 256) {
+            const bool one = wgs(128, 128) <= 256;      // at most one workgroup per CU
+            if (Loader::kConv || one)
+                return two && one ? launch_tile_dma<8, 2, 1, 4, 2>(ld, native, M, K, N, ep, stream)
+                                  : launch_tile_dma<8, 2, 1, 4, 1>(ld, native, M, K, N, ep, stream);
+            return launch_tile_dma<4, 4, 2, 2, 1>(ld, native, M, K, N, ep, stream);
+        }
+        return launch_tile_dma<4, 2, 1, 2, 1>(ld, native, M, K, N, ep, stream);
     } else {
         // Register prefetch depth: the big tile has a k-tile of work long enough to cover a trip to L2
         // (and no registers to spare); the smaller ones fetch two tiles ahead once the reduction is
@@ -649,8 +665,8 @@ int dispatch_tile(const Loader &ld, const void *native, int64_t M, int64_t K, in
         if (N > 64 && wgs(128, 128) >= 256)
             return deep ? launch_tile<4, 4, 2, 2, 2>(ld, native, M, K, N, ep, stream)
                         : launch_tile<4, 4, 2, 2, 1>(ld, native, M, K, N, ep, stream);
-        return deep ? launch_tile<2, 4, 2, 1, 2>(ld, native, M, K, N, ep, stream)
-                    : launch_tile<2, 4, 2, 1, 1>(ld, native, M, K, N, ep, stream);
+        return deep ? launch_tile<4, 2, 1, 2, 2>(ld, native, M, K, N, ep, stream)
+                    : launch_tile<4, 2, 1, 2, 1>(ld, native, M, K, N, ep, stream);
     }
 }
 
