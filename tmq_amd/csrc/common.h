@@ -31,6 +31,30 @@ inline bool split_reduction_pays(int64_t M, int64_t K, int64_t N) {
     return K >= 512 ? tiles64 <= 640 : tiles64 <= K / 2;
 }
 
+// 16 bytes per lane from global memory straight into LDS through a buffer resource: lane l's 16 bytes at byte
+// `offset` of the buffer go to byte 16 l of the (uniform) destination; a lane whose offset lies past the end of
+// the buffer gets zeros. The padding taps of a convolution then cost a select of the offset instead of a select
+// between two 64-bit addresses. The host pass does not know the builtins and only sees empty bodies.
+constexpr uint32_t kPastTheEnd = 0xFFFFFFF0u;   // beyond any buffer these kernels wrap (hosts check: < 2^32 - 32 bytes)
+#if defined(__HIP_DEVICE_COMPILE__)
+typedef __amdgpu_buffer_rsrc_t BufferResource;
+#else
+struct BufferResource {};
+#endif
+__device__ __forceinline__ BufferResource make_buffer_resource(const void *base, uint32_t bytes) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)bytes, 0x00020000);   // raw buffer, 32-bit elements
+#else
+    return {};
+#endif
+}
+__device__ __forceinline__ void buffer_to_lds(BufferResource rsrc, uint32_t offset, unsigned char *dst) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    typedef __attribute__((address_space(3))) void *lds_ptr;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_ptr)dst, 16, offset, 0, 0, 0);
+#endif
+}
+
 // Division of 0 <= n < 2^31 by a divisor known on the host (an image extent): q = umulhi(n, mul) >> shift,
 // two instructions instead of the ~25 of a 32-bit division. With s = ceil(log2 d) and mul = ceil(2^(31 + s) / d)
 // (< 2^32), n mul / 2^(31 + s) exceeds n / d by less than 2^-s <= 1 / d, so the floor is the same.

@@ -52,6 +52,7 @@ constexpr int kPitch = 64;       // LDS row pitch in halfs: 128 bytes = 8 chunks
 struct DenseLoader {
     static constexpr bool kDirect = false;
     [[maybe_unused]] static constexpr bool kConv = false;
+    [[maybe_unused]] static constexpr bool kBuffer = false;
     const _Float16 *x;
     int64_t M, K;
 
@@ -95,6 +96,7 @@ struct DenseLoader {
 struct DenseDirect {
     static constexpr bool kDirect = true;
     [[maybe_unused]] static constexpr bool kConv = false;
+    [[maybe_unused]] static constexpr bool kBuffer = false;
     const _Float16 *x;
     int64_t M, K;
 
@@ -126,6 +128,7 @@ template <bool VEC>
 struct ConvLoader {
     static constexpr bool kDirect = false;
     [[maybe_unused]] static constexpr bool kConv = true;
+    [[maybe_unused]] static constexpr bool kBuffer = false;
     const _Float16 *x;
     int64_t M, K;
     int B, C, H, W, Ho, Wo, ky, kx, sy, sx, py, px, dy, dx;
@@ -204,6 +207,7 @@ struct ConvLoader {
 struct ConvLoader64 {
     static constexpr bool kDirect = true;
     [[maybe_unused]] static constexpr bool kConv = true;
+    [[maybe_unused]] static constexpr bool kBuffer = true;
     const _Float16 *x;
     int64_t M, K;
     int B, C, H, W, Ho, Wo, ky, kx, sy, sx, py, px, dy, dx;
@@ -242,6 +246,15 @@ struct ConvLoader64 {
                         ((unsigned)(st.iw0[q] + st.j * dx) < (unsigned)W);
         return in ? static_cast<const void *>(x + (st.off0[q] + st.delta)) : static_cast<const void *>(&kZeroChunk);
     }
+    // The same chunk as a byte offset into a buffer resource over x; padding taps and the K tail get an
+    // offset past its end, for which the load delivers zeros.
+    template <int CH, int T>
+    __device__ __forceinline__ uint32_t offset(const State<CH, T> &st, int q) const {
+        const bool in = (st.i < ky) & ((unsigned)(st.ih0[q] + st.i * dy) < (unsigned)H) &
+                        ((unsigned)(st.iw0[q] + st.j * dx) < (unsigned)W);
+        return in ? (uint32_t)(st.off0[q] + st.delta) * 2u : kPastTheEnd;
+    }
+    __device__ __forceinline__ uint32_t bytes() const { return (uint32_t)((int64_t)B * H * W * C * 2); }
     template <int CH, int T>
     __device__ __forceinline__ void advance(State<CH, T> &st) const {   // next k-tile: 64 channels on
         st.c0 += kBK;
@@ -260,6 +273,7 @@ struct ConvLoader64 {
 struct ConvLoaderFewC {
     static constexpr bool kDirect = true;
     [[maybe_unused]] static constexpr bool kConv = true;
+    [[maybe_unused]] static constexpr bool kBuffer = true;
     const _Float16 *x;
     int64_t M, K;
     int B, C, H, W, Ho, Wo, ky, kx, sy, sx, py, px, dy, dx;
@@ -297,6 +311,13 @@ struct ConvLoaderFewC {
         const bool in = (st.i < ky) & ((unsigned)(st.ih0[q] + di) < (unsigned)H) & ((unsigned)(st.iw0[q] + dj) < (unsigned)W);
         return in ? static_cast<const void *>(x + (st.off0[q] + (di * W + dj) * C)) : static_cast<const void *>(&kZeroChunk);
     }
+    template <int CH, int T>
+    __device__ __forceinline__ uint32_t offset(const State<CH, T> &st, int q) const {
+        const int di = st.i * dy, dj = st.j * dx;
+        const bool in = (st.i < ky) & ((unsigned)(st.ih0[q] + di) < (unsigned)H) & ((unsigned)(st.iw0[q] + dj) < (unsigned)W);
+        return in ? (uint32_t)(st.off0[q] + (di * W + dj) * C) * 2u : kPastTheEnd;
+    }
+    __device__ __forceinline__ uint32_t bytes() const { return (uint32_t)((int64_t)B * H * W * C * 2); }
     template <int CH, int T>
     __device__ __forceinline__ void advance(State<CH, T> &st) const {   // next k-tile: 64 / C taps on
         st.j += kBK / C;
@@ -513,10 +534,15 @@ __global__ __launch_bounds__(64 * WGM * WGN, 2) void tile_dma_kernel(Loader ld, 
     // tile `kn` -> ring buffer `slot`; the loader's state moves on to the next tile (tiles past K, which
     // the last pass prefetches and nobody multiplies, read whatever the loader substitutes)
     unsigned char *const lds0 = reinterpret_cast<unsigned char *>(&As[0][0]) + wv * 1024;
+    BufferResource rsrc;
+    if constexpr (Loader::kBuffer) rsrc = make_buffer_resource(ld.x, ld.bytes());
     auto fill = [&](int kn, int slot) {
         unsigned char *dst = lds0 + slot * kTileBytes;
 #pragma unroll
-        for (int i = 0; i < CH; i++) load_to_lds(ld.template addr<CH, T>(st, (int64_t)kn * kBK, i), dst + i * (T * 16));
+        for (int i = 0; i < CH; i++) {
+            if constexpr (Loader::kBuffer) buffer_to_lds(rsrc, ld.template offset<CH, T>(st, i), dst + i * (T * 16));
+            else load_to_lds(ld.template addr<CH, T>(st, (int64_t)kn * kBK, i), dst + i * (T * 16));
+        }
         ld.template advance<CH, T>(st);
     };
 
@@ -729,7 +755,7 @@ int tmq_ternary_conv2d(const void *x, const tmq_conv_shape *s, const void *nativ
     // few output tiles: split the reduction inside the workgroup (mid.hip)
     if (mid_conv_ok(x, s) && split_reduction_pays(M, K, s->N))
         return launch_mid_conv(x, s, ho, wo, native, scale, bias, residual, relu, y, y_dtype == TMQ_F16 ? 1 : 0, stream);
-    const bool small = (int64_t)s->B * s->H * s->W * s->C < (int64_t)0x7FFFFFFF && M < (int64_t)0x7FFFFFFF;   // 32-bit offsets and rows
+    const bool small = (int64_t)s->B * s->H * s->W * s->C < (int64_t)0x7FFFFFF0 && M < (int64_t)0x7FFFFFFF;   // 32-bit offsets and rows
     if ((s->C % kBK == 0) && aligned16(x) && small)
         return dispatch_tile(with_divisors(ConvLoader64{xp, M, K, s->B, s->C, s->H, s->W, ho, wo, s->ky, s->kx, s->sy,
                                                         s->sx, s->py, s->px, s->dy, s->dx, {}, {}}), native, M, K, s->N, ep, stream);

@@ -45,6 +45,7 @@ struct MidEpilogue {
 // covers rows 8 c .. 8 c + 7; the lane's row is R = 8 c + lane / 8); `source` returns the address
 // of the lane's 16-byte chunk of pair starting at reduction index k0 (uniform).
 struct DenseRows {
+    static constexpr bool kBuffer = false;
     const _Float16 *x;
     int64_t M, K;
 
@@ -74,6 +75,7 @@ struct DenseRows {
 };
 
 struct ConvRows {
+    static constexpr bool kBuffer = true;      // chunks are fetched through a buffer resource over x
     const _Float16 *x;
     int64_t M, K;
     int B, C, H, W, Ho, Wo, ky, kx, sy, sx, py, px, dy, dx;
@@ -114,6 +116,14 @@ struct ConvRows {
         return in ? static_cast<const void *>(x + (st.off[mi][c] + p.delta))
                   : static_cast<const void *>(kZeroChunk + (lane & 7));
     }
+    // the same chunk as a byte offset into the buffer; padding taps and the K tail: past its end (zeros)
+    template <int WM>
+    __device__ __forceinline__ uint32_t offset(const State<WM> &st, const Pair &p, int mi, int c) const {
+        const bool in = p.live && (unsigned)(st.ih0[mi][c] + p.di) < (unsigned)H &&
+                        (unsigned)(st.iw0[mi][c] + p.dj) < (unsigned)W;
+        return in ? (uint32_t)(st.off[mi][c] + p.delta) * 2u : kPastTheEnd;
+    }
+    __device__ __forceinline__ uint32_t bytes() const { return (uint32_t)((int64_t)B * H * W * C * 2); }
 };
 
 // 16 bytes per lane from global memory straight into LDS: lane l lands at dst + 16 l (dst uniform).
@@ -289,6 +299,8 @@ __global__ __launch_bounds__(64 * WAVES) void mid_kernel(Rows rows, const u32x4 
     }
     typename Rows::template State<WM> st;
     rows.template prepare<WM>(st, m0, lane);
+    BufferResource rsrc;
+    if constexpr (Rows::kBuffer) rsrc = make_buffer_resource(rows.x, rows.bytes());
     const ThreadColumns cc = load_column_constants<WN>(n0, N, ep);
 
     // operand (row j, chunk ch) of a fragment sits at position ch ^ ((j / 2) % 8) of its row
@@ -315,7 +327,10 @@ __global__ __launch_bounds__(64 * WAVES) void mid_kernel(Rows rows, const u32x4 
             for (int mi = 0; mi < WM; mi++)
 #pragma unroll
                 for (int c = 0; c < 2; c++)
-                    load_to_lds(rows.template source<WM>(st, pr, mi, c, lane), win + slot * kSlot + mi * kFrag + c * 1024);
+                    if constexpr (Rows::kBuffer)
+                        buffer_to_lds(rsrc, rows.template offset<WM>(st, pr, mi, c), win + slot * kSlot + mi * kFrag + c * 1024);
+                    else
+                        load_to_lds(rows.template source<WM>(st, pr, mi, c, lane), win + slot * kSlot + mi * kFrag + c * 1024);
         };
         if (nt > 0) {
             u32x4 wq[2][WN];
@@ -383,7 +398,10 @@ __global__ __launch_bounds__(64 * WAVES) void mid_kernel(Rows rows, const u32x4 
         for (int mi = 0; mi < WM; mi++)
 #pragma unroll
             for (int c = 0; c < 2; c++)
-                load_to_lds(rows.template source<WM>(st, pr, mi, c, lane), win + slot * kSlot + mi * kFrag + c * 1024);
+                if constexpr (Rows::kBuffer)
+                    buffer_to_lds(rsrc, rows.template offset<WM>(st, pr, mi, c), win + slot * kSlot + mi * kFrag + c * 1024);
+                else
+                    load_to_lds(rows.template source<WM>(st, pr, mi, c, lane), win + slot * kSlot + mi * kFrag + c * 1024);
     };
     if constexpr (RING == 3) {
         // Two pairs ahead instead of one: with one wavefront per SIMD (the 64 x 128 tile) a pair's multiplications
@@ -1050,7 +1068,7 @@ int launch_stream_dense(const void *x, int64_t M, int64_t K, const void *native,
 }
 
 bool mid_conv_ok(const void *x, const tmq_conv_shape *s) {
-    return (s->C % 64 == 0) && aligned16(x) && (int64_t)s->B * s->H * s->W * s->C < (int64_t)0x7FFFFFFF;
+    return (s->C % 64 == 0) && aligned16(x) && (int64_t)s->B * s->H * s->W * s->C < (int64_t)0x7FFFFFF0;
 }
 
 int launch_mid_conv(const void *x, const tmq_conv_shape *s, int ho, int wo, const void *native, const float *scale,
