@@ -36,6 +36,9 @@ def test_patches_form_matches_oracle(cuda, oracle, P, T, C):
 @pytest.mark.parametrize("B,C,H,W,k,stride,pad,dil", [
     (2, 16, 9, 9, 3, 1, 1, 1), (1, 40, 12, 11, (3, 5), (2, 1), (1, 2), 1), (3, 8, 7, 7, 3, 2, 0, 1),
     (2, 5, 6, 6, 3, 1, 1, 1), (1, 96, 14, 14, 3, 1, 2, 2), (2, 32, 8, 8, 5, 1, ((2, 1), (0, 3)), 1),
+    # square 5 x 5 and 7 x 7 windows on the several-positions-per-thread kernel: strides 1 and 2, ragged widths
+    (2, 24, 13, 11, 5, 1, 2, 1), (1, 16, 14, 15, 5, 2, 2, 1), (2, 8, 9, 10, 7, 1, 3, 1), (1, 40, 15, 13, 7, 2, 3, 1),
+    (1, 8, 3, 3, 7, 1, 3, 1), (1, 16, 20, 17, 5, (1, 2), (2, 0), 1),
 ])
 def test_image_form_exact_on_integers(cuda, B, C, H, W, k, stride, pad, dil):
     """Small-integer activations: every product and sum is exact, so the result must equal torch's

@@ -170,18 +170,18 @@ __global__ __launch_bounds__(256) void dwconv_image_kernel(const _Float16 *__res
     else store8(ep, p * C + c0, c0, C, acc, vec);
 }
 
-// The common case -- 3 x 3 taps, no dilation, whole groups of 8 channels, fewer than 2^31 threads. A thread owns
-// 8 channels of PX horizontally adjacent output positions: the columns their windows share are loaded once
-// (for stride 1, PX + 2 columns per row instead of 3 PX), the 8 weights of a tap are expanded to floats once
+// The common cases -- KS x KS taps (3, 5 or 7), no dilation, whole groups of 8 channels, fewer than 2^31 threads. A
+// thread owns 8 channels of PX horizontally adjacent output positions: the columns their windows share are loaded once
+// (for stride 1, PX + KS - 1 columns per row instead of KS PX), the 8 weights of a tap are expanded to floats once
 // for all PX positions, and the index arithmetic is multiply-high (FastDiv). All loads of a row are in
 // flight together; taps outside the image read the clamped pixel and are replaced by zero. Per output the
 // taps are accumulated in the same order as in dwconv_image_kernel (fp32, every product exact).
-template <int PX, int SX>
-__global__ __launch_bounds__(256) void dwconv3x3_image_kernel(const _Float16 *__restrict__ x, const uint32_t *__restrict__ words,
+template <int KS, int PX, int SX>
+__global__ __launch_bounds__(256) void dwconv_square_image_kernel(const _Float16 *__restrict__ x, const uint32_t *__restrict__ words,
                                                               uint32_t total, int C, int H, int W, int Wo, FastDiv by_g,
                                                               FastDiv by_wg, FastDiv by_ho, int sy, int py, int px,
                                                               DwEpilogue ep) {
-    constexpr int NC = (PX - 1) * SX + 3;                          // input columns the PX windows cover
+    constexpr int NC = (PX - 1) * SX + KS;                         // input columns the PX windows cover
     const uint32_t id = blockIdx.x * 256u + threadIdx.x;
     if (id >= total) return;
     int cg, wg, oh;
@@ -199,7 +199,7 @@ __global__ __launch_bounds__(256) void dwconv3x3_image_kernel(const _Float16 *__
         for (int e = 0; e < 8; e++) acc[q][e] = 0.f;
 
 #pragma unroll 1
-    for (int i = 0; i < 3; i++) {                                  // one row at a time: its NC loads in flight, few registers
+    for (int i = 0; i < KS; i++) {                                 // one row at a time: its NC loads in flight, few registers
         const int ih = oh * sy - py + i;
         const bool row_in = (unsigned)ih < (unsigned)H;
         const int ihc = ih < 0 ? 0 : (ih >= H ? H - 1 : ih);
@@ -216,8 +216,8 @@ __global__ __launch_bounds__(256) void dwconv3x3_image_kernel(const _Float16 *__
             if (!(row_in && (unsigned)iw < (unsigned)W)) v[c] = half8{0, 0, 0, 0, 0, 0, 0, 0};
         }
 #pragma unroll
-        for (int j = 0; j < 3; j++) {
-            const uint32_t codes = codes8(words, Q, i * 3 + j, c0);
+        for (int j = 0; j < KS; j++) {
+            const uint32_t codes = codes8(words, Q, i * KS + j, c0);
             float w[8];
 #pragma unroll
             for (int e = 0; e < 8; e++) {
@@ -369,22 +369,24 @@ int tmq_ternary_dwconv2d(const void *x, const tmq_conv_shape *s, const uint32_t 
     int vec = (s->C % 8 == 0) && aligned_for(x, 16) && aligned_for(y, ya) && (!e.residual || aligned_for(e.residual, ya));
     if (vec && aligned_for(e.scale, 16) && aligned_for(e.bias, 16)) vec |= 2;       // the 16-byte epilogue as well
     DwEpilogue ep{e.scale, e.bias, e.residual, y, e.relu, y_f16};
-    if ((vec & 2) && s->ky == 3 && s->kx == 3 && s->dy == 1 && s->dx == 1 &&
-        (s->sx == 1 || s->sx == 2) && total < (int64_t)0x7FFFFFFF &&
+    const bool square = s->ky == s->kx && (s->ky == 3 || s->ky == 5 || s->ky == 7);
+    if ((vec & 2) && square && s->dy == 1 && s->dx == 1 && (s->sx == 1 || s->sx == 2) && total < (int64_t)0x7FFFFFFF &&
         (int64_t)s->B * ho * wo < (int64_t)0x7FFFFFFF) {
-        const int px_per_thread = s->sx == 1 ? 4 : 2;
+        // output positions per thread, measured: 4 except at stride 2 with 3 x 3 or 5 x 5 windows (the windows then
+        // share few columns, and 4 positions would hold 9 or 11 columns of a row in registers)
+        const int px_per_thread = (s->sx == 1 || s->ky == 7) ? 4 : 2;
         const int64_t wgroups = (wo + px_per_thread - 1) / px_per_thread, G = s->C / 8;
         const int64_t threads = (int64_t)s->B * ho * wgroups * G, nblocks = (threads + 255) / 256;
         const FastDiv by_g((uint32_t)G), by_wg((uint32_t)wgroups), by_ho((uint32_t)ho);
-        if (s->sx == 1)
-            hipLaunchKernelGGL((dwconv3x3_image_kernel<4, 1>), dim3((uint32_t)nblocks), dim3(256), 0, as_stream(stream),
+        auto go = [&](auto kernel) {
+            hipLaunchKernelGGL(kernel, dim3((uint32_t)nblocks), dim3(256), 0, as_stream(stream),
                                static_cast<const _Float16 *>(x), words, (uint32_t)threads, s->C, s->H, s->W, wo, by_g, by_wg,
                                by_ho, s->sy, s->py, s->px, ep);
-        else
-            hipLaunchKernelGGL((dwconv3x3_image_kernel<2, 2>), dim3((uint32_t)nblocks), dim3(256), 0, as_stream(stream),
-                               static_cast<const _Float16 *>(x), words, (uint32_t)threads, s->C, s->H, s->W, wo, by_g, by_wg,
-                               by_ho, s->sy, s->py, s->px, ep);
-        return check_launch();
+            return check_launch();
+        };
+        if (s->ky == 3) return s->sx == 1 ? go(dwconv_square_image_kernel<3, 4, 1>) : go(dwconv_square_image_kernel<3, 2, 2>);
+        if (s->ky == 5) return s->sx == 1 ? go(dwconv_square_image_kernel<5, 4, 1>) : go(dwconv_square_image_kernel<5, 2, 2>);
+        return s->sx == 1 ? go(dwconv_square_image_kernel<7, 4, 1>) : go(dwconv_square_image_kernel<7, 4, 2>);
     }
     hipLaunchKernelGGL(dwconv_image_kernel, dim3((uint32_t)blocks), dim3(256), 0, as_stream(stream),
                        static_cast<const _Float16 *>(x), words, s->B, s->C, s->H, s->W, ho, wo, s->ky, s->kx, s->sy, s->sx,
