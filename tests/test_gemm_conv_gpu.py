@@ -76,6 +76,12 @@ CONV_CASES = [  # B, C, H, W, N, k, stride, pad, dil
     (2, 128, 28, 28, 256, 1, 2, 0, 1),
     # a short reduction with many tiles stays on the tile kernel
     (8, 64, 40, 40, 128, 1, 1, 0, 1),
+    # padding wider than the window's reach, dilation and strides on the direct-to-LDS loaders (taps outside the
+    # image are out-of-range buffer offsets there), last tile ragged in M; 64 / 8 / 16 / 32 channels
+    (3, 64, 9, 7, 64, 3, 1, 4, 1), (2, 64, 10, 10, 96, 3, 2, 3, 3), (1, 8, 11, 9, 40, 3, 1, 5, 2),
+    (5, 16, 7, 7, 64, (5, 3), (2, 1), (4, 3), (1, 2)), (2, 32, 6, 13, 24, 3, (1, 2), (3, 0), 1),
+    # ... and on the split-reduction kernel (many channels, few output tiles)
+    (1, 256, 5, 5, 128, 3, 1, 3, 1), (2, 512, 4, 6, 256, 3, 2, 2, 2),
 ]
 
 
