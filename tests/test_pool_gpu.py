@@ -41,7 +41,8 @@ def test_global_average_pool(cuda, B, C, H, W):
 
 
 @pytest.mark.parametrize("B,C,H,W,dtype", [(4, 3, 224, 224, torch.float16), (2, 3, 8, 12, torch.float32), (1, 1, 5, 4, torch.float16),
-                                           (3, 4, 6, 8, torch.float32)])
+                                           (3, 4, 6, 8, torch.float32), (2, 4, 6, 8, torch.float16), (3, 1, 5, 16, torch.float16),
+                                           (2, 3, 3, 8, torch.float16), (5, 2, 7, 24, torch.float16)])
 def test_input_repack(cuda, B, C, H, W, dtype):
     from tmq_amd import ops
     g = torch.Generator(device=cuda).manual_seed(B + C + H)
