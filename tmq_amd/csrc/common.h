@@ -26,10 +26,11 @@ constexpr int kWave = 64;
 // rather than the big-tile kernel. Measured crossovers: with K >= 512 the split reduction wins up to two
 // tiles of 64 x 64 per CU, which 64 x 128 tiles still cover in one pass (beyond that its second pass runs
 // partly empty: M = 4608, K = 4096, N = 512 takes 52 us there and 31 us on the big-tile kernel); with shorter
-// reductions its per-tile cost shows earlier (K = 256: up to ~128 tiles, K = 128: ~64).
+// reductions its per-tile cost shows earlier (K = 256: up to ~128 tiles, K = 128: ~64). Long reductions over
+// wide layers keep it a little longer (M = 576, K = 8192, N = 4096: 50 us against 58 us).
 inline bool split_reduction_pays(int64_t M, int64_t K, int64_t N) {
     const int64_t tiles64 = ((M + 63) / 64) * ((N + 63) / 64);
-    return K >= 512 ? tiles64 <= 512 : tiles64 <= K / 2;
+    return K >= 512 ? tiles64 <= ((K >= 8192 && N >= 2048) ? 640 : 512) : tiles64 <= K / 2;
 }
 
 // 16 bytes per lane from global memory straight into LDS through a buffer resource: lane l's 16 bytes at byte
