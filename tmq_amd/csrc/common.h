@@ -57,6 +57,14 @@ __device__ __forceinline__ void buffer_to_lds(BufferResource rsrc, uint32_t offs
 #endif
 }
 
+// Workgroup ids are dealt round-robin over the 8 XCDs, each with an L2 of its own. Position of workgroup `id` of `G`
+// in an order where the workgroups of one XCD are consecutive, so that a kernel can give them neighbouring tiles.
+// XCDs below G % 8 (all of them when that is 0) hold ceil(G / 8) workgroups, the others one fewer.
+__device__ __forceinline__ int xcd_contiguous(int id, int G) {
+    const int xcd = id & 7, per = (G + 7) >> 3, rem = G & 7;
+    return xcd * per - ((rem != 0 && xcd > rem) ? xcd - rem : 0) + (id >> 3);
+}
+
 // Division of 0 <= n < 2^31 by a divisor known on the host (an image extent): q = umulhi(n, mul) >> shift,
 // two instructions instead of the ~25 of a 32-bit division. With s = ceil(log2 d) and mul = ceil(2^(31 + s) / d)
 // (< 2^32), n mul / 2^(31 + s) exceeds n / d by less than 2^-s <= 1 / d, so the floor is the same.
