@@ -12,7 +12,8 @@
  *     caller holds them; the library rounds them to fp32 once, the way torch does when a Python
  *     scalar meets an fp32 tensor, so results are bit-identical to the reference's CPU chain
  *     of separately rounded fp32 operations.
- *   - Thread safe; no hidden mutable global state.
+ *   - Thread safe; no hidden mutable global state, with one documented exception: the static
+ *     scratch array of tmq_softstep_fused_noalloc.
  *
  * Each declaration cites the reference interface it replaces (paths relative to the reference
  * repository root).
@@ -105,6 +106,21 @@ int tmq_softstep_fused(const float *w, const float *g, float *y, float *dw, floa
                        double *loss_sum, void *workspace, size_t n, double digamma,
                        double sharpness, double strength, float gl, double lo, double hi,
                        void *stream);
+
+/* tmq_softstep_fused without a workspace argument and without any device allocation. It has no
+ * counterpart in the reference; it is for callers that cannot allocate device memory: code under HIP
+ * graph capture, tight serving / training loops, harnesses that forbid hipMalloc. The block partial
+ * sums of the loss reduction go to a 1 MiB array that is part of the library's device image (each
+ * GPU the library runs on holds its own copy until the process ends); its address is looked up once
+ * per device on the first call there. n may be at most tmq_softstep_fused_noalloc_max_elements()
+ * (2^29), larger tensors return TMQ_ERR_TOO_LARGE. Results are bit-identical to tmq_softstep_fused.
+ * All calls on one GPU share that GPU's array: calls that overlap in time on one GPU (different
+ * streams or threads) race on it and must be serialised by the caller; calls on one stream are
+ * ordered. Nothing in the array needs clearing between calls.                                   */
+size_t tmq_softstep_fused_noalloc_max_elements(void);
+int tmq_softstep_fused_noalloc(const float *w, const float *g, float *y, float *dw, float *wc,
+                               double *loss_sum, size_t n, double digamma, double sharpness,
+                               double strength, float gl, double lo, double hi, void *stream);
 
 /* Diagnostic with no counterpart in the reference: the kernels above replace IEEE division by
  * cheaper FMA sequences; this proves on the device that they are bit-identical to IEEE

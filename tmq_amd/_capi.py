@@ -56,6 +56,8 @@ SIGNATURES = {
     "tmq_ternarize_inplace": (_int, [_vp, _sz, _dbl, _vp]),
     "tmq_softstep_fused_workspace_bytes": (_sz, [_sz]),
     "tmq_softstep_fused": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _dbl, _dbl, _dbl, _flt, _dbl, _dbl, _vp]),
+    "tmq_softstep_fused_noalloc_max_elements": (_sz, []),
+    "tmq_softstep_fused_noalloc": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _sz, _dbl, _dbl, _dbl, _flt, _dbl, _dbl, _vp]),
     "tmq_selfcheck_division": (_int, [_dbl, _vp, _vp]),
     "tmq_probe_stream_read": (_int, [_vp, ctypes.c_size_t, _vp, _vp]),
     "tmq_split_f32": (_int, [_vp, _vp, _vp, _i64, _vp]),

@@ -13,6 +13,7 @@
 #include "softstep_math.h"
 
 #include <math.h>
+#include <mutex>
 #include <type_traits>
 
 namespace tmq {
@@ -432,6 +433,36 @@ __global__ __launch_bounds__(kThreads) void selfcheck_kernel(float c, float rc, 
 inline uint32_t blocks_for(uint64_t n) { return (uint32_t)((n + kChunk - 1) / kChunk); }
 constexpr uint64_t kMaxElems = (uint64_t)0x7FFFFFFFu * kChunk / 2;  // keeps block counts in 31 bits
 
+// Scratch of tmq_softstep_fused_noalloc: the block partial sums of the loss reduction live in a
+// file-scope device array instead of a caller-provided workspace, so that entry point never needs a
+// device allocation. Every GPU holds its own copy of the array at its own address; the name below is
+// only a host-side stand-in, the address comes from hipGetSymbolAddress once per device.
+constexpr uint64_t kNoAllocMaxElems = (uint64_t)1 << 29;
+constexpr size_t kScratchBytes = (size_t)(kNoAllocMaxElems / kChunk) * sizeof(float);   // 1 MiB
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void *g_scratch_ptr[kMaxDevices] = {};
+
+// Device address of `scratch` on the current device (looked up on the first call per device).
+int scratch_address(void **out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return note_hip_error(e);
+    if (dev < 0 || dev >= kMaxDevices) return TMQ_ERR_UNSUPPORTED;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void *p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return note_hip_error(e);
+        if (!p) return TMQ_ERR_LAUNCH;
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
+    return TMQ_OK;
+}
+
 template <class Op>
 int launch_single(const Op &op, const float *in0, const float *in1, float *o0, float *o1, float *o2, size_t n,
                   float *partials, void *stream) {
@@ -562,6 +593,23 @@ int tmq_softstep_fused(const float *w, const float *g, float *y, float *dw, floa
     }
     return rc;
 }
+
+int tmq_softstep_fused_noalloc(const float *w, const float *g, float *y, float *dw, float *wc, double *loss_sum,
+                               size_t n, double digamma, double sharpness, double strength, float gl, double lo,
+                               double hi, void *stream) {
+    if (n > kNoAllocMaxElems) return TMQ_ERR_TOO_LARGE;
+    void *ws = nullptr;
+    if (loss_sum) {
+        // Every block of this call writes its own partial sum before the finalisation reads exactly
+        // those, so nothing in the array has to start at zero; what earlier calls left behind it is
+        // never read.
+        const int rc = scratch_address(&ws);
+        if (rc != TMQ_OK) return rc;
+    }
+    return tmq_softstep_fused(w, g, y, dw, wc, loss_sum, ws, n, digamma, sharpness, strength, gl, lo, hi, stream);
+}
+
+size_t tmq_softstep_fused_noalloc_max_elements(void) { return (size_t)kNoAllocMaxElems; }
 
 int tmq_selfcheck_division(double digamma, uint64_t *counts, void *stream) {
     if (!counts || bad_hardness(digamma)) return TMQ_ERR_INVALID_ARG;
