@@ -168,6 +168,38 @@ int tmq_qloss_bwd_multi(const tmq_segment *segs_dev, int nseg, uint32_t total_bl
                         double sharpness, double strength, const float *upstream, int accumulate,
                         void *stream);
 
+/* The same for the tensors of a training step, whose outputs and gradients sit at new addresses in
+ * every step: the table is a HOST array that the library copies into the kernels' arguments, so
+ * nothing is uploaded or cached (up to 64 tensors per launch, more are split over several).
+ * Replaces the per-layer launches of SoftStep.forward / backward (tmq/tmq.py:404-438, called from
+ * Linear.forward_wrap 650 and Conv2d.forward 812 for every layer) together with the quantization loss
+ * (298-310, 456-493) and autograd's accumulation of the two gradient terms.                       */
+typedef struct tmq_step_tensor {
+    const float *w; /* weights (device, fp32) */
+    const float *g; /* backward only: dL/dy of this tensor (device), NULL if none arrived */
+    float *out;     /* forward: y = S(w); backward: dw */
+    uint64_t n;     /* elements */
+} tmq_step_tensor;
+
+/* Workspace (bytes) of tmq_softstep_fwd_multi when a loss output is requested. */
+size_t tmq_softstep_multi_workspace_bytes(const tmq_step_tensor *tensors_host, int ntensors);
+
+/* out_l = S(w_l; digamma) for every tensor; with loss_per_tensor / loss_total non-NULL also
+ * loss_per_tensor[l] = mean_i q(w_l[i]; sharpness, strength) and *loss_total = their fp32 sum in
+ * table order (as tmq_qloss_multi), from the same pass over the weights.                         */
+int tmq_softstep_fwd_multi(const tmq_step_tensor *tensors_host, int ntensors, double digamma,
+                           double sharpness, double strength, float *loss_per_tensor,
+                           float *loss_total, void *workspace, void *stream);
+
+/* out_l = g_l * S'(w_l; digamma) + (u / float(n_l)) * Q'(w_l; sharpness, strength): the weight
+ * gradient of a whole step, u = *loss_upstream (device, 1 float: the gradient arriving at the total
+ * quantization loss; NULL = the loss took no part, the second term is dropped). A tensor with g NULL
+ * gets the second term alone. Each term is rounded as the reference's backward functions round it
+ * (tmq/tmq.py:434-438, 488-493) and the two are added once, as autograd's accumulation would.    */
+int tmq_softstep_bwd_multi(const tmq_step_tensor *tensors_host, int ntensors, double digamma,
+                           double sharpness, double strength, const float *loss_upstream,
+                           void *stream);
+
 /* w_l <- clamp(w_l, lo, hi) for every segment, one launch. */
 int tmq_clamp_multi(const tmq_segment *segs_dev, int nseg, uint32_t total_blocks, double lo,
                     double hi, void *stream);

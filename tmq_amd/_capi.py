@@ -26,6 +26,11 @@ class Segment(ctypes.Structure):
                 ("block_begin", ctypes.c_uint32), ("scalar", ctypes.c_float)]
 
 
+class StepTensor(ctypes.Structure):
+    """tmq_step_tensor of include/tmq_hip.h (32 bytes)."""
+    _fields_ = [("w", ctypes.c_void_p), ("g", ctypes.c_void_p), ("out", ctypes.c_void_p), ("n", ctypes.c_uint64)]
+
+
 class ConvShape(ctypes.Structure):
     """tmq_conv_shape of include/tmq_hip.h."""
     _fields_ = [(k, ctypes.c_int32) for k in
@@ -68,6 +73,9 @@ SIGNATURES = {
     "tmq_qloss_multi": (_int, [_vp, _int, _u32, _dbl, _dbl, _vp, _vp, _vp, _vp]),
     "tmq_qloss_bwd_multi": (_int, [_vp, _int, _u32, _dbl, _dbl, _vp, _int, _vp]),
     "tmq_clamp_multi": (_int, [_vp, _int, _u32, _dbl, _dbl, _vp]),
+    "tmq_softstep_multi_workspace_bytes": (_sz, [ctypes.POINTER(StepTensor), _int]),
+    "tmq_softstep_fwd_multi": (_int, [ctypes.POINTER(StepTensor), _int, _dbl, _dbl, _dbl, _vp, _vp, _vp, _vp]),
+    "tmq_softstep_bwd_multi": (_int, [ctypes.POINTER(StepTensor), _int, _dbl, _dbl, _dbl, _vp, _vp]),
     "tmq_pack_ternary": (_int, [_vp, _int, _i64, _i64, _vp, _vp]),
     "tmq_unpack_ternary": (_int, [_vp, _i64, _i64, _vp, _vp]),
     "tmq_native_weight_bytes": (_sz, [_i64, _i64]),

@@ -218,6 +218,29 @@ struct FusedOp {
     }
 };
 
+// Backward of a whole QAT step for one tensor: out1 = g*S'(w) (HAS_G) + sc*Q'(w) (HAS_Q), each term
+// rounded as the reference's two backward functions round it (tmq/tmq.py:434-438 with scale 1.0,
+// 488-493) and summed once, as autograd's gradient accumulation would. sc is the per-tensor scalar.
+template <bool HAS_G, bool HAS_Q>
+struct StepBwdOp {
+    TMQ_OP_FLAGS(HAS_G, false, true, false, false, false);
+    StepK s, q;
+    template <bool CAREFUL>
+    __device__ __forceinline__ void apply(float w, float g, float sc, float &, float &o1, float &, float &) const {
+        Frac f = split(w);
+        float t1 = 0.f, t2 = 0.f;
+        if constexpr (HAS_G) {
+            Rational r(clamped_arg<CAREFUL>(f, s.d, s.h));
+            t1 = g * cdiv(s.d * r.dsig(), s.c, s.rc);
+        }
+        if constexpr (HAS_Q) {
+            Rational r5(clamped_arg<CAREFUL>(f, q.d, q.h));
+            t2 = sc * cdiv(q.k2 * r5.d2sig(), q.c, q.rc);
+        }
+        o1 = (HAS_G && HAS_Q) ? (t1 + t2) : (HAS_G ? t1 : t2);
+    }
+};
+
 // ---- tensor locators ------------------------------------------------------------------------
 struct View {
     const float *in0;
@@ -259,6 +282,37 @@ struct Multi {
         bool vec = ((reinterpret_cast<uintptr_t>(p) | reinterpret_cast<uintptr_t>(a)) & 15u) == 0;
         const float sc = upstream ? upstream[0] / (float)s.n : s.scalar;
         return View{p, nullptr, inplace ? p : nullptr, a, nullptr, s.n, b - s.block_begin, sc, vec};
+    }
+};
+
+// Multi-tensor with the table inside the kernel's arguments (nothing to upload: the pointers of a
+// training step's gradients change with every step). Up to kArgTensors tensors per launch.
+constexpr int kArgTensors = 64;
+struct ArgTable {
+    const float *w[kArgTensors];
+    const float *g[kArgTensors];
+    float *out[kArgTensors];
+    uint64_t n[kArgTensors];
+    uint32_t begin[kArgTensors + 1];   // first block of tensor l; begin[ntensors] = blocks of the launch
+    int ntensors;
+};
+struct MultiArg {
+    ArgTable t;
+    const float *upstream;   // device scalar u: the per-tensor scalar is u / float(n) (mean backward), or null
+    __device__ __forceinline__ View locate(uint32_t b) const {
+        int lo = 0, hi = t.ntensors - 1;
+        while (lo < hi) {
+            int mid = (lo + hi + 1) >> 1;
+            if (t.begin[mid] <= b) lo = mid;
+            else hi = mid - 1;
+        }
+        const float *w = t.w[lo];
+        const float *g = t.g[lo];
+        float *o = t.out[lo];
+        const uint64_t n = t.n[lo];
+        bool vec = ((reinterpret_cast<uintptr_t>(w) | reinterpret_cast<uintptr_t>(g) | reinterpret_cast<uintptr_t>(o)) & 15u) == 0;
+        const float sc = upstream ? upstream[0] / (float)n : 0.f;
+        return View{w, g, o, o, nullptr, n, b - t.begin[lo], sc, vec};
     }
 };
 
@@ -345,16 +399,39 @@ __device__ __forceinline__ double wave_sum_f64(double v) {
     return v;
 }
 
-__global__ __launch_bounds__(kFinThreads) void finalize_kernel(const tmq_segment *segs, int nseg,
-                                                              uint32_t total_blocks, const float *partials,
-                                                              double factor, float *per_tensor, float *total,
-                                                              double *sum_out) {
+// Block ranges of the tensors whose partial sums are finalised: from a device table, or by value.
+struct DevRanges {
+    const tmq_segment *segs;   // null: one range [0, total) without a mean
+    int nseg;
+    uint32_t total;
+    __device__ __forceinline__ int count() const { return nseg; }
+    __device__ __forceinline__ uint32_t begin(int l) const { return segs ? segs[l].block_begin : 0u; }
+    __device__ __forceinline__ uint32_t end(int l) const { return segs ? (l + 1 < nseg ? segs[l + 1].block_begin : total) : total; }
+    __device__ __forceinline__ bool has_mean() const { return segs != nullptr; }
+    __device__ __forceinline__ uint64_t elems(int l) const { return segs[l].n; }
+};
+struct ArgRanges {
+    uint64_t n[kArgTensors];
+    uint32_t first[kArgTensors + 1];
+    int ntensors;
+    __device__ __forceinline__ int count() const { return ntensors; }
+    __device__ __forceinline__ uint32_t begin(int l) const { return first[l]; }
+    __device__ __forceinline__ uint32_t end(int l) const { return first[l + 1]; }
+    __device__ __forceinline__ bool has_mean() const { return true; }
+    __device__ __forceinline__ uint64_t elems(int l) const { return n[l]; }
+};
+
+// carry (device, optional): the running total of the tensors finalised by an earlier launch.
+template <class R>
+__global__ __launch_bounds__(kFinThreads) void finalize_kernel(R rg, const float *partials, double factor,
+                                                              float *per_tensor, float *total, double *sum_out,
+                                                              const float *carry) {
     __shared__ double task_sum[kMaxTasks];
     const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const int nseg = rg.count();
     uint32_t task = 0;
     for (int l = 0; l < nseg; l++) {
-        const uint32_t b0 = segs ? segs[l].block_begin : 0u;
-        const uint32_t b1 = segs ? (l + 1 < nseg ? segs[l + 1].block_begin : total_blocks) : total_blocks;
+        const uint32_t b0 = rg.begin(l), b1 = rg.end(l);
         const uint32_t ntask = (b1 - b0 + kTaskLen - 1) / kTaskLen;
         for (uint32_t t = 0; t < ntask; t++, task++) {
             if ((int)(task % kFinWaves) != wv) continue;
@@ -368,21 +445,22 @@ __global__ __launch_bounds__(kFinThreads) void finalize_kernel(const tmq_segment
     }
     __syncthreads();
     if (threadIdx.x == 0) {
-        float running = 0.f;
+        float running = carry ? *carry : 0.f;
+        bool first = carry == nullptr;
         uint32_t tk = 0;
         for (int l = 0; l < nseg; l++) {
-            const uint32_t b0 = segs ? segs[l].block_begin : 0u;
-            const uint32_t b1 = segs ? (l + 1 < nseg ? segs[l + 1].block_begin : total_blocks) : total_blocks;
+            const uint32_t b0 = rg.begin(l), b1 = rg.end(l);
             const uint32_t ntask = (b1 - b0 + kTaskLen - 1) / kTaskLen;
             double sum = 0.0;
             for (uint32_t t = 0; t < ntask; t++) sum += task_sum[tk++];
             sum *= factor;   // partials hold sum dsig; factor = strength*sharpness/c
             if (sum_out) sum_out[l] = sum;
-            if (segs) {
-                const uint64_t n = segs[l].n;
+            if (rg.has_mean()) {
+                const uint64_t n = rg.elems(l);
                 float mean = (float)(sum / (double)n);   // n == 0 gives NaN like torch.mean of an empty tensor
                 if (per_tensor) per_tensor[l] = mean;
-                running = (l == 0) ? mean : running + mean;
+                running = first ? mean : running + mean;
+                first = false;
             }
         }
         if (total) *total = running;
@@ -488,6 +566,36 @@ int launch_multi(const Op &op, const tmq_segment *segs, int nseg, uint32_t total
 
 bool bad_hardness(double d) { return !(d > 0.0) || !(d <= 1.0e6); }
 
+// Fills an argument table with tensors [first, first + count) of `ts` that pass `keep`; returns the
+// launch's block count (0 = nothing to do) or a negative status.
+template <class Keep>
+int64_t fill_table(ArgTable &t, const tmq_step_tensor *ts, int first, int count, Keep keep) {
+    uint64_t b = 0;
+    int k = 0;
+    for (int i = first; i < first + count; i++) {
+        if (!keep(ts[i])) continue;
+        if (ts[i].n > kMaxElems) return TMQ_ERR_TOO_LARGE;
+        t.w[k] = ts[i].w;
+        t.g[k] = ts[i].g;
+        t.out[k] = ts[i].out;
+        t.n[k] = ts[i].n;
+        t.begin[k] = (uint32_t)b;
+        b += blocks_for(ts[i].n);
+        if (b > 0x7FFFFFFFull) return TMQ_ERR_TOO_LARGE;
+        k++;
+    }
+    t.begin[k] = (uint32_t)b;
+    t.ntensors = k;
+    return (int64_t)b;
+}
+
+template <class Op>
+int launch_args(const Op &op, const ArgTable &t, uint32_t blocks, const float *upstream, float *partials, void *stream) {
+    MultiArg loc{t, upstream};
+    hipLaunchKernelGGL((stream_kernel<Op, MultiArg>), dim3(blocks), dim3(kThreads), 0, as_stream(stream), loc, op, partials);
+    return check_launch();
+}
+
 }  // namespace
 }  // namespace tmq
 
@@ -587,8 +695,9 @@ int tmq_softstep_fused(const float *w, const float *g, float *y, float *dw, floa
         if (rc != TMQ_OK) return rc;
     }
     if (loss_sum) {
-        hipLaunchKernelGGL(finalize_kernel, dim3(1), dim3(kFinThreads), 0, as_stream(stream), nullptr, 1,
-                           blocks_for(n), partials, (double)q.k1 / (double)q.c, nullptr, nullptr, loss_sum);
+        hipLaunchKernelGGL(finalize_kernel<DevRanges>, dim3(1), dim3(kFinThreads), 0, as_stream(stream),
+                           DevRanges{nullptr, 1, blocks_for(n)}, partials, (double)q.k1 / (double)q.c, nullptr, nullptr,
+                           loss_sum, nullptr);
         rc = check_launch();
     }
     return rc;
@@ -645,8 +754,9 @@ int tmq_qloss_multi(const tmq_segment *segs, int nseg, uint32_t total_blocks, do
     QLossOp op{make_step(sharpness, strength)};
     int rc = launch_multi(op, segs, nseg, total_blocks, 0, partials, stream);
     if (rc != TMQ_OK) return rc;
-    hipLaunchKernelGGL(finalize_kernel, dim3(1), dim3(kFinThreads), 0, as_stream(stream), segs, nseg, total_blocks,
-                       partials, (double)op.q.k1 / (double)op.q.c, per_tensor, total, nullptr);
+    hipLaunchKernelGGL(finalize_kernel<DevRanges>, dim3(1), dim3(kFinThreads), 0, as_stream(stream),
+                       DevRanges{segs, nseg, total_blocks}, partials, (double)op.q.k1 / (double)op.q.c, per_tensor, total,
+                       nullptr, nullptr);
     return check_launch();
 }
 
@@ -656,6 +766,84 @@ int tmq_qloss_bwd_multi(const tmq_segment *segs, int nseg, uint32_t total_blocks
     const StepK q = make_step(sharpness, strength);
     if (accumulate) return launch_multi(QLossBwdOp<true>{q}, segs, nseg, total_blocks, 0, nullptr, stream, upstream);
     return launch_multi(QLossBwdOp<false>{q}, segs, nseg, total_blocks, 0, nullptr, stream, upstream);
+}
+
+size_t tmq_softstep_multi_workspace_bytes(const tmq_step_tensor *ts, int ntensors) {
+    uint64_t b = 0;
+    for (int i = 0; ts && i < ntensors; i++) b += blocks_for(ts[i].n);
+    return (size_t)b * sizeof(float) + 16;
+}
+
+int tmq_softstep_fwd_multi(const tmq_step_tensor *ts, int ntensors, double digamma, double sharpness, double strength,
+                           float *loss_per_tensor, float *loss_total, void *workspace, void *stream) {
+    if (ntensors < 0 || (ntensors > 0 && !ts)) return TMQ_ERR_INVALID_ARG;
+    const bool want_loss = loss_per_tensor || loss_total;
+    if (bad_hardness(digamma) || (want_loss && (bad_hardness(sharpness) || !workspace))) return TMQ_ERR_INVALID_ARG;
+    for (int i = 0; i < ntensors; i++)
+        if (ts[i].n && (!ts[i].w || !ts[i].out)) return TMQ_ERR_INVALID_ARG;
+    const StepK s = make_step(digamma, 0.0), q = make_step(want_loss ? sharpness : 1.0, want_loss ? strength : 0.0);
+    float *partials = static_cast<float *>(workspace);
+    bool carried = false;
+    if (ntensors == 0 && want_loss) return TMQ_ERR_INVALID_ARG;   // a sum over no tensors: nothing would write it
+    for (int first = 0; first < ntensors; first += kArgTensors) {
+        const int count = ntensors - first < kArgTensors ? ntensors - first : kArgTensors;
+        ArgTable t;
+        const int64_t blocks = fill_table(t, ts, first, count, [](const tmq_step_tensor &) { return true; });
+        if (blocks < 0) return (int)blocks;
+        if (want_loss && !finalize_fits(t.ntensors, (uint32_t)blocks)) return TMQ_ERR_TOO_LARGE;
+        int rc = TMQ_OK;
+        if (blocks > 0) {
+            if (want_loss) rc = launch_args(FusedOp<9>{s, q, 0.f, 0.f, 0.f}, t, (uint32_t)blocks, nullptr, partials, stream);
+            else rc = launch_args(FusedOp<1>{s, q, 0.f, 0.f, 0.f}, t, (uint32_t)blocks, nullptr, nullptr, stream);
+            if (rc != TMQ_OK) return rc;
+        }
+        if (want_loss) {
+            ArgRanges rg;
+            for (int k = 0; k < t.ntensors; k++) { rg.n[k] = t.n[k]; rg.first[k] = t.begin[k]; }
+            rg.first[t.ntensors] = t.begin[t.ntensors];
+            rg.ntensors = t.ntensors;
+            hipLaunchKernelGGL(finalize_kernel<ArgRanges>, dim3(1), dim3(kFinThreads), 0, as_stream(stream), rg, partials,
+                               (double)q.k1 / (double)q.c, loss_per_tensor ? loss_per_tensor + first : nullptr, loss_total,
+                               nullptr, carried ? loss_total : nullptr);
+            rc = check_launch();
+            if (rc != TMQ_OK) return rc;
+            carried = true;
+            partials += blocks;
+        }
+    }
+    return TMQ_OK;
+}
+
+int tmq_softstep_bwd_multi(const tmq_step_tensor *ts, int ntensors, double digamma, double sharpness, double strength,
+                           const float *loss_upstream, void *stream) {
+    if (ntensors < 0 || (ntensors > 0 && !ts)) return TMQ_ERR_INVALID_ARG;
+    if (bad_hardness(digamma) || (loss_upstream && bad_hardness(sharpness))) return TMQ_ERR_INVALID_ARG;
+    for (int i = 0; i < ntensors; i++) {
+        if (ts[i].n && (!ts[i].w || !ts[i].out)) return TMQ_ERR_INVALID_ARG;
+        if (!ts[i].g && !loss_upstream) return TMQ_ERR_INVALID_ARG;   // no gradient reaches this tensor: leave it out
+    }
+    const StepK s = make_step(digamma, 0.0), q = make_step(loss_upstream ? sharpness : 1.0, loss_upstream ? strength : 0.0);
+    for (int first = 0; first < ntensors; first += kArgTensors) {
+        const int count = ntensors - first < kArgTensors ? ntensors - first : kArgTensors;
+        ArgTable t;
+        int64_t blocks = fill_table(t, ts, first, count, [](const tmq_step_tensor &x) { return x.g != nullptr; });
+        if (blocks < 0) return (int)blocks;
+        int rc = TMQ_OK;
+        if (blocks > 0) {
+            if (loss_upstream) rc = launch_args(StepBwdOp<true, true>{s, q}, t, (uint32_t)blocks, loss_upstream, nullptr, stream);
+            else rc = launch_args(StepBwdOp<true, false>{s, q}, t, (uint32_t)blocks, nullptr, nullptr, stream);
+            if (rc != TMQ_OK) return rc;
+        }
+        if (loss_upstream) {   // tensors the forward pass did not use: the loss term alone
+            blocks = fill_table(t, ts, first, count, [](const tmq_step_tensor &x) { return x.g == nullptr; });
+            if (blocks < 0) return (int)blocks;
+            if (blocks > 0) {
+                rc = launch_args(StepBwdOp<false, true>{s, q}, t, (uint32_t)blocks, loss_upstream, nullptr, stream);
+                if (rc != TMQ_OK) return rc;
+            }
+        }
+    }
+    return TMQ_OK;
 }
 
 int tmq_clamp_multi(const tmq_segment *segs, int nseg, uint32_t total_blocks, double lo, double hi, void *stream) {

@@ -72,6 +72,105 @@ torch::Tensor bwd_softstep_derivative(torch::Tensor weights, double digamma, dou
     return y;
 }
 
+// ---- one launch for all layers of a training step -------------------------------------------------
+// Additive (no counterpart among the reference's bindings): SoftStep.forward / backward of every layer
+// (tmq/tmq.py:404-438), the quantization loss (298-310) and its gradient (475-493) as multi-tensor
+// launches. Outputs are carved from one flat buffer per call, each on a 256-byte boundary.
+struct Carved {
+    torch::Tensor flat;
+    std::vector<torch::Tensor> parts;
+};
+
+Carved carve(const std::vector<torch::Tensor> &like) {
+    int64_t total = 0;
+    std::vector<int64_t> offs;
+    for (const auto &t : like) {
+        offs.push_back(total);
+        total += (t.numel() + 63) / 64 * 64;
+    }
+    Carved c;
+    c.flat = torch::empty({total}, like[0].options());
+    for (size_t i = 0; i < like.size(); i++) {
+        auto part = torch::empty({0}, like[0].options());
+        part.set_(c.flat.storage(), offs[i], like[i].sizes(), like[i].strides());
+        c.parts.push_back(part);
+    }
+    return c;
+}
+
+std::vector<torch::Tensor> step_weights(const std::vector<torch::Tensor> &weights, const char *name) {
+    TORCH_CHECK(!weights.empty(), name, ": no tensors");
+    std::vector<torch::Tensor> ws;
+    for (const auto &w : weights) {
+        ws.push_back(f32_cuda(w.detach(), name));
+        TORCH_CHECK(ws.back().device() == ws[0].device(), name, ": all tensors must live on one device");
+    }
+    return ws;
+}
+
+std::tuple<std::vector<torch::Tensor>, c10::optional<torch::Tensor>> softstep_fwd_all(
+        std::vector<torch::Tensor> weights, double digamma, bool want_loss, double sharpness, double strength) {
+    auto ws = step_weights(weights, "softstep_fwd_all");
+    const c10::DeviceGuard guard(ws[0].device());
+    Carved ys = carve(ws);
+    std::vector<tmq_step_tensor> table(ws.size());
+    for (size_t i = 0; i < ws.size(); i++)
+        table[i] = tmq_step_tensor{ws[i].data_ptr<float>(), nullptr, ys.parts[i].data_ptr<float>(), (uint64_t)ws[i].numel()};
+    c10::optional<torch::Tensor> loss;
+    torch::Tensor workspace;
+    if (want_loss) {
+        loss = torch::empty({}, ws[0].options());
+        workspace = torch::empty({(int64_t)tmq_softstep_multi_workspace_bytes(table.data(), (int)table.size())},
+                                 ws[0].options().dtype(torch::kUInt8));
+    }
+    check(tmq_softstep_fwd_multi(table.data(), (int)table.size(), digamma, sharpness, strength, nullptr,
+                                 want_loss ? loss->data_ptr<float>() : nullptr, want_loss ? workspace.data_ptr() : nullptr,
+                                 stream_of(ws[0])), "softstep_fwd_all");
+    return {ys.parts, loss};
+}
+
+std::vector<c10::optional<torch::Tensor>> softstep_bwd_all(std::vector<torch::Tensor> weights,
+                                                           std::vector<c10::optional<torch::Tensor>> grads,
+                                                           c10::optional<torch::Tensor> loss_upstream, double digamma,
+                                                           double sharpness, double strength) {
+    auto ws = step_weights(weights, "softstep_bwd_all");
+    TORCH_CHECK(grads.size() == ws.size(), "softstep_bwd_all: one gradient (or None) per tensor");
+    const c10::DeviceGuard guard(ws[0].device());
+    torch::Tensor up;
+    if (loss_upstream.has_value()) {
+        TORCH_CHECK(loss_upstream->device().is_cuda() && loss_upstream->numel() == 1,
+                    "softstep_bwd_all: loss_upstream must be one value on the GPU");
+        up = loss_upstream->detach().to(torch::kFloat32).contiguous();
+    }
+    std::vector<size_t> live;
+    std::vector<torch::Tensor> like, gs;
+    for (size_t i = 0; i < ws.size(); i++)
+        if (grads[i].has_value() || up.defined()) {
+            live.push_back(i);
+            like.push_back(ws[i]);
+        }
+    std::vector<c10::optional<torch::Tensor>> out(ws.size());
+    if (live.empty()) return out;
+    Carved dws = carve(like);
+    std::vector<tmq_step_tensor> table(live.size());
+    for (size_t k = 0; k < live.size(); k++) {
+        const size_t i = live[k];
+        const float *gp = nullptr;
+        if (grads[i].has_value()) {
+            const auto &g = *grads[i];
+            TORCH_CHECK(g.device() == ws[i].device() && g.scalar_type() == torch::kFloat32 && g.numel() == ws[i].numel(),
+                        "softstep_bwd_all: a gradient must match its weights in device, dtype and size");
+            gs.push_back(g.detach().contiguous());
+            gp = gs.back().data_ptr<float>();
+        }
+        table[k] = tmq_step_tensor{ws[i].data_ptr<float>(), gp, dws.parts[k].data_ptr<float>(), (uint64_t)ws[i].numel()};
+        out[i] = dws.parts[k];
+    }
+    check(tmq_softstep_bwd_multi(table.data(), (int)table.size(), digamma, sharpness, strength,
+                                 up.defined() ? up.data_ptr<float>() : nullptr, stream_of(ws[0])), "softstep_bwd_all");
+    return out;
+}
+
 // ---- ternary inference -----------------------------------------------------------------------------
 // The reference hands the compact words to every call; the kernels want the re-tiled layout, built
 // once per weight tensor. A small LRU keeps (words -> native) pairs; an entry holds a reference to
@@ -311,6 +410,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("ternary_mvm_cuda", &ternary_mvm_cuda);
     m.def("ternary_dwconv_cuda", &ternary_dwconv_cuda);
     m.def("ternary_dwconvtrans_cuda", &ternary_dwconvtrans_cuda);
+    // additive: all layers of a training step in one launch
+    m.def("softstep_fwd_all", &softstep_fwd_all);
+    m.def("softstep_bwd_all", &softstep_bwd_all);
     // tmq_native (tmq/tmq_native.cpp:550-555)
     m.def("compactify_ternary", &compactify_ternary);
     m.def("compress_ternary", &compress_ternary);

@@ -196,6 +196,99 @@ def qloss_bwd_multi(table: SegmentTable, sharpness: float, strength: float, accu
                                          stream_of(table.table)), "qloss_bwd_multi")
 
 
+def _carve(flat, offsets, like):
+    """Tensors of the shapes of `like` on the storage of one flat buffer (not views of one another)."""
+    out = []
+    for off, t in zip(offsets, like):
+        out.append(torch.empty(0, dtype=flat.dtype, device=flat.device).set_(flat.untyped_storage(), off, t.shape))
+    return out
+
+
+def _flat_offsets(tensors):
+    """Element offsets of the tensors in one flat buffer, each starting on a 256-byte boundary."""
+    offs, total = [], 0
+    for t in tensors:
+        offs.append(total)
+        total += (t.numel() + 63) // 64 * 64
+    return offs, total
+
+
+def _step_weights(weights, name):
+    if not weights:
+        raise ValueError(f"{name}: no tensors")
+    dev = weights[0].device
+    ws = []
+    for w in weights:
+        w = _f32_cuda(w.detach(), name)
+        if w.device != dev:
+            raise RuntimeError(f"{name}: all tensors must live on one device")
+        ws.append(w)
+    return ws, dev
+
+
+def softstep_fwd_all(weights, digamma: float, want_loss: bool = False, sharpness: float = 5.0, strength: float = 0.0):
+    """y_l = S(w_l; digamma) for a list of fp32 GPU tensors in one launch (SoftStep.forward of every
+    layer of a model, tmq/tmq.py:404-419) and, with want_loss, the total quantization loss
+    sum_l mean(q(w_l; sharpness, strength)) (tmq/tmq.py:298-310) from the same pass over the weights.
+    Returns (list of y, 0-dim fp32 loss or None)."""
+    ws, dev = _step_weights(weights, "softstep_fwd_all")
+    offs, total = _flat_offsets(ws)
+    flat = torch.empty(total, dtype=torch.float32, device=dev)
+    ys = _carve(flat, offs, ws)
+    arr = (_capi.StepTensor * len(ws))()
+    for i, (w, y) in enumerate(zip(ws, ys)):
+        arr[i].w, arr[i].g, arr[i].out, arr[i].n = w.data_ptr(), None, y.data_ptr(), w.numel()
+    lib = _lib()
+    loss = wsp = None
+    if want_loss:
+        loss = torch.empty((), dtype=torch.float32, device=dev)
+        wsp = torch.empty(lib.tmq_softstep_multi_workspace_bytes(arr, len(ws)), dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        check(lib.tmq_softstep_fwd_multi(arr, len(ws), float(digamma), float(sharpness), float(strength), None, ptr(loss),
+                                         ptr(wsp), stream_of(flat)), "softstep_fwd_all")
+    return ys, loss
+
+
+def softstep_bwd_all(weights, grads, loss_upstream, digamma: float, sharpness: float = 5.0, strength: float = 0.0):
+    """dw_l = g_l * S'(w_l; digamma) + (u / n_l) * Q'(w_l; sharpness, strength) for a list of tensors in
+    one launch: the weight gradients of a whole step (tmq/tmq.py:422-438, 475-493 plus autograd's sum of
+    the two). grads[l] may be None (no gradient reached y_l), loss_upstream (one fp32 GPU value u, the
+    gradient arriving at the total quantization loss) may be None; a tensor that gets neither term
+    yields None."""
+    ws, dev = _step_weights(weights, "softstep_bwd_all")
+    if len(grads) != len(ws):
+        raise ValueError("softstep_bwd_all: one gradient (or None) per tensor")
+    if loss_upstream is not None:
+        _capi.require_gpu(loss_upstream, "loss_upstream")
+        if loss_upstream.numel() != 1:
+            raise RuntimeError("softstep_bwd_all: loss_upstream must be one value")
+        loss_upstream = loss_upstream.detach().to(torch.float32).contiguous()
+    live = [i for i in range(len(ws)) if grads[i] is not None or loss_upstream is not None]
+    out = [None] * len(ws)
+    if not live:
+        return out
+    offs, total = _flat_offsets([ws[i] for i in live])
+    flat = torch.empty(total, dtype=torch.float32, device=dev)
+    dws = _carve(flat, offs, [ws[i] for i in live])
+    arr = (_capi.StepTensor * len(live))()
+    keep = []
+    for k, i in enumerate(live):
+        g = grads[i]
+        if g is not None:
+            if not g.is_cuda or g.dtype != torch.float32 or g.numel() != ws[i].numel():
+                raise RuntimeError("softstep_bwd_all: a gradient must match its weights in device, dtype and size")
+            g = g.detach()
+            g = g if g.is_contiguous() else g.contiguous()
+            keep.append(g)
+        arr[k].w, arr[k].g, arr[k].out, arr[k].n = ws[i].data_ptr(), (g.data_ptr() if g is not None else None), \
+            dws[k].data_ptr(), ws[i].numel()
+        out[i] = dws[k]
+    with torch.cuda.device(dev):
+        check(_lib().tmq_softstep_bwd_multi(arr, len(live), float(digamma), float(sharpness), float(strength),
+                                            ptr(loss_upstream), stream_of(flat)), "softstep_bwd_all")
+    return out
+
+
 def softstep_map(weights: torch.Tensor, digamma: float, derivative: bool = False) -> torch.Tensor:
     """SoftStep.map / SoftStep.dmap (tmq/tmq.py:328-350) on an fp32 GPU tensor."""
     w = _f32_cuda(weights, "softstep_map")

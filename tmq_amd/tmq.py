@@ -138,7 +138,9 @@ class QuantizationControl:
             self.qpenalty_range = qpenalty_range
         else:
             self.qpenalty_range = (0, 0)
-        self._table = None            # cached multi-tensor segment table (weights, grads)
+        self._table = None            # cached multi-tensor segment table over the registered weights
+        self._step = None             # soft weights of the current forward pass (_StepState)
+        self._loss_wanted = False     # set by the first quantization_loss(): later passes fuse the loss
 
     # ---- schedule (host scalars only) -----------------------------------------------------------
     @staticmethod
@@ -216,6 +218,7 @@ class QuantizationControl:
     def register_node(self, name, node):
         self._registry[name] = node
         self._table = None
+        self._step = None
 
     def collect_grad_norms(self):
         return {name: node.weight.grad.norm() for name, node in self._registry.items()
@@ -225,8 +228,8 @@ class QuantizationControl:
         return [node.weight for node in self._registry.values()]
 
     def _segment_table(self):
-        """Multi-tensor table over (weight, scratch gradient) of every registered layer; rebuilt
-        whenever a weight tensor has been reallocated."""
+        """Multi-tensor table over the weights of every registered layer; rebuilt whenever a weight
+        tensor has been reallocated."""
         ws = [w.data for w in self._weights()]
         for w in ws:
             _require_gpu_weight(w, "QuantizationControl")
@@ -235,12 +238,7 @@ class QuantizationControl:
         key = tuple((w.data_ptr(), w.numel()) for w in ws)
         if self._table is None or self._table[0] != key:
             ws = [w if w.is_contiguous() else w.contiguous() for w in ws]
-            flat = torch.empty(sum(w.numel() for w in ws), dtype=torch.float32, device=ws[0].device)
-            grads, off = [], 0
-            for w in ws:
-                grads.append(flat[off:off + w.numel()])
-                off += w.numel()
-            self._table = (key, ops.SegmentTable(ws, aux=grads), grads, ws)
+            self._table = (key, ops.SegmentTable(ws), ws)
         return self._table
 
     # ---- tensor work: one launch for all layers ------------------------------------------------------
@@ -250,8 +248,9 @@ class QuantizationControl:
         if not self._registry:
             return
         lo, hi = self.clamp_values[0] - slack, self.clamp_values[1] + slack
-        _, table, _, _ = self._segment_table()
+        _, table, _ = self._segment_table()
         ops.clamp_multi_(table, lo, hi)
+        self._step = None
 
     def quantize(self):
         """Hard-quantize every registered layer: w <- round(SoftStep.map(w)) (tmq/tmq.py:284-295)."""
@@ -259,34 +258,142 @@ class QuantizationControl:
             w = node.weight.data
             _require_gpu_weight(w, "QuantizationControl.quantize")
             node.weight.data = ops.ternarize_(w.contiguous().clone(), self.digamma)
+        self._step = None
 
     def quantization_loss(self, penalty=None):
-        """Sum over layers of mean(SoftStepDerivative(w, sharpness, p)) (tmq/tmq.py:298-310); one
+        """Sum over layers of mean(SoftStepDerivative(w, sharpness, p)) (tmq/tmq.py:298-310). When the
+        model's forward pass of this step has already produced it (same weights, same penalty), that
+        value is returned and its gradient joins the soft-step backward in one launch; otherwise one
         multi-tensor launch forward, one backward. Returns None when no layer is registered."""
         if not self._registry:
             return None
-        p = penalty if penalty is not None else self.qpenalty
-        return _QuantizationLossAll.apply(self, float(p), float(self.qpenalty_sharpness), *self._weights())
+        p = float(penalty if penalty is not None else self.qpenalty)
+        self._loss_wanted = True
+        st = self._step
+        if (st is not None and st.loss is not None and st.strength == p and st.sharpness == float(self.qpenalty_sharpness)
+                and st.grad_mode == torch.is_grad_enabled() and st.covers(self._registry.values())):
+            return st.loss
+        return _QuantizationLossAll.apply(self, p, float(self.qpenalty_sharpness), *self._weights())
+
+    # ---- soft weights of a forward pass: one launch for all layers ------------------------------------
+    def _soft_weight_of(self, node):
+        """S(weight) of a registered layer for the forward pass that is under way. The first layer that
+        asks triggers one multi-tensor launch for every registered fp32 layer (and, once
+        quantization_loss() has been used, for the loss as well); each layer's result is handed out
+        once per pass, and a changed weight tensor, hardness or autograd mode starts a new pass.
+        Returns None for a layer this controller cannot serve (then SoftStep.apply does it)."""
+        st = self._step
+        i = st.index.get(id(node)) if st is not None else None
+        w = node.weight
+        if (i is None or st.used[i] or st.versions[i] != w._version or st.ptrs[i] != w.data_ptr()
+                or st.digamma != self.digamma or st.grad_mode != torch.is_grad_enabled()):
+            st = self._step = _StepState.run(self)
+            i = st.index.get(id(node)) if st is not None else None
+            if i is None:
+                return None
+        st.used[i] = True
+        return st.ys[i]
+
+
+class _StepState:
+    """Outputs of one multi-tensor soft-step forward launch and what they were computed from."""
+
+    __slots__ = ("index", "nodes", "ptrs", "versions", "used", "ys", "loss", "digamma", "sharpness", "strength", "grad_mode")
+
+    @classmethod
+    def run(cls, ctrl):
+        nodes, dev = [], None
+        for node in ctrl._registry.values():
+            w = getattr(node, "weight", None)
+            if w is None or node.compact or not w.is_cuda or w.dtype != torch.float32 or (dev is not None and w.device != dev):
+                continue
+            dev = w.device
+            nodes.append(node)
+        if not nodes:
+            return None
+        st = cls()
+        st.nodes = nodes
+        st.index = {id(n): i for i, n in enumerate(nodes)}
+        weights = [n.weight for n in nodes]
+        st.ptrs = [w.data_ptr() for w in weights]
+        st.versions = [w._version for w in weights]
+        st.used = [False] * len(nodes)
+        st.digamma, st.sharpness, st.strength = ctrl.digamma, float(ctrl.qpenalty_sharpness), float(ctrl.qpenalty)
+        st.grad_mode = torch.is_grad_enabled()
+        want_loss = ctrl._loss_wanted
+        outs = _SoftStepAll.apply(st.digamma, want_loss, st.sharpness, st.strength, *weights)
+        st.ys = outs[:len(nodes)]
+        st.loss = outs[len(nodes)] if want_loss else None
+        return st
+
+    def covers(self, registered):
+        """True when every registered layer took part and none of their weights changed since."""
+        registered = list(registered)
+        if len(registered) != len(self.nodes):
+            return False
+        for n, p, v in zip(self.nodes, self.ptrs, self.versions):
+            w = n.weight
+            if w.data_ptr() != p or w._version != v:
+                return False
+        return all(a is b for a, b in zip(registered, self.nodes))
+
+
+class _SoftStepAll(Function):
+    """(y_1 .. y_L [, loss]) = (S(w_1) .. S(w_L) [, sum_l mean q(w_l)]) as ONE autograd node: the forward
+    is one multi-tensor launch and, because autograd runs a node only when the gradients of all its
+    outputs are there, so is the backward, dw_l = g_l S'(w_l) + (g_loss / n_l) Q'(w_l) -- the two terms
+    the reference computes in SoftStep.backward and SoftStepDerivative.backward per layer and lets autograd
+    add (tmq/tmq.py:422-438, 475-493)."""
+
+    @staticmethod
+    def forward(ctx, digamma, want_loss, sharpness, strength, *weights):
+        ctx.args = (digamma, want_loss, sharpness, strength)
+        ctx.save_for_backward(*weights)
+        ctx.set_materialize_grads(False)
+        ys, loss = _b.softstep_fwd_all([w.data for w in weights], digamma, want_loss, sharpness, strength)
+        return (*ys, loss) if want_loss else tuple(ys)
+
+    @staticmethod
+    def backward(ctx, *grads):
+        digamma, want_loss, sharpness, strength = ctx.args
+        weights = ctx.saved_tensors
+        L = len(weights)
+        upstream = grads[L] if want_loss else None
+        need = ctx.needs_input_grad[4:]
+        live = [i for i in range(L) if need[i] and (grads[i] is not None or upstream is not None)]
+        out = [None] * L
+        if live:
+            dws = _b.softstep_bwd_all([weights[i].data for i in live], [grads[i] for i in live], upstream, digamma,
+                                      sharpness, strength)
+            for i, dw in zip(live, dws):
+                out[i] = dw
+        return (None, None, None, None) + tuple(out)
 
 
 class _QuantizationLossAll(Function):
     """total = sum_l mean_i q(w_l[i]); d total / d w_l = (g / n_l) * Q'(w_l) (tmq/tmq.py:456-493,
-    698-699) for every registered layer at once."""
+    698-699) for every registered layer at once, when the loss is asked for outside a forward pass."""
 
     @staticmethod
     def forward(ctx, ctrl, strength, sharpness, *weights):
-        _, table, _, _ = ctrl._segment_table()
-        ctx.ctrl, ctx.strength, ctx.sharpness = ctrl, strength, sharpness
+        _, table, _ = ctrl._segment_table()
+        ctx.strength, ctx.sharpness = strength, sharpness
+        ctx.save_for_backward(*weights)
         _, total = ops.qloss_multi(table, sharpness, strength)
         return total.reshape(())
 
     @staticmethod
     def backward(ctx, grad_output):
-        key, table, grads, ws = ctx.ctrl._segment_table()
-        g = grad_output.detach().to(torch.float32).reshape(1).contiguous()
-        ops.qloss_bwd_multi(table, ctx.sharpness, ctx.strength, accumulate=False, upstream=g)
-        out = tuple(gr.view(w.shape).clone() for gr, w in zip(grads, ws))
-        return (None, None, None) + out
+        weights = ctx.saved_tensors
+        need = ctx.needs_input_grad[3:]
+        live = [i for i in range(len(weights)) if need[i]]
+        out = [None] * len(weights)
+        if live:
+            dws = _b.softstep_bwd_all([weights[i].data for i in live], [None] * len(live), grad_output, 1.0,
+                                      ctx.sharpness, ctx.strength)
+            for i, dw in zip(live, dws):
+                out[i] = dw
+        return (None, None, None) + tuple(out)
 
 
 class SoftStep(Function):
@@ -428,8 +535,11 @@ class TMQLayer:
         return self._VARIANCE.get(self.quantization, 1.0)
 
     def _soft_weight(self):
-        use = self._ctrl is not None and not self._ctrl.inference_mode
-        return SoftStep.apply(self.weight, 1.0, self._ctrl) if use else self.weight
+        ctrl = self._ctrl
+        if ctrl is None or ctrl.inference_mode:
+            return self.weight
+        y = ctrl._soft_weight_of(self)
+        return y if y is not None else SoftStep.apply(self.weight, 1.0, ctrl)
 
     def _native_weights(self, conv_kernel=None):
         w = self.weight.data
