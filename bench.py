@@ -1,5 +1,7 @@
 #!/usr/bin/env python3
-"""Headline benchmark: the fused soft-staircase pass on one MI355X.
+"""Benchmark of TMQ's GPU hot path on one MI355X. The headline is the fused soft-staircase pass; the
+other legs of the metric (ternary GEMV / GEMM, ResNet-18 inference, the TMQ share of a ResNet-18 QAT
+step) ride along under "also", each with its own `roofline` and `cpu_baseline`.
 
 Workload (BASELINE.json configs[1]): a flat fp32 tensor of 2^26 weights, uniform in [-1,1] with
 10 % of the elements placed within +-0.02 of a ternary level, an N(0,1) upstream gradient, and a
@@ -12,7 +14,7 @@ Prints ONE JSON line: metric soft-step fwd+bwd GB/s on the algorithmic 20 B/elem
 object (the op-for-op torch CPU restatement of the reference path, timed on this host's cores
 on a bounded sample).
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload softstep|gemv|gemm|...]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload all|softstep|linear|resnet_infer|resnet_qat]
 """
 import argparse
 import json
@@ -26,6 +28,35 @@ sys.path.insert(0, ROOT)
 HARDNESS = [0.1, 1.1684210526315788, 3.0004, 4.72, 6.0]   # default schedule, epochs 0/21/79/88/149 of 150
 SHARPNESS, STRENGTH = 5.0, 5e-4
 HBM_PEAK_GBS = 8000.0
+MFMA_FP16_PEAK_TFLOPS = 2500.0
+
+
+def cpu_model():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def timed_cpu(torch, fn, threads, budget_s, min_reps=3, max_reps=15):
+    """Median seconds of fn() on `threads` host threads: one warm-up, then repetitions until the
+    budget is spent (at least min_reps)."""
+    prev = torch.get_num_threads()
+    torch.set_num_threads(threads)
+    try:
+        fn()
+        times, t_start = [], time.perf_counter()
+        while len(times) < min_reps or (time.perf_counter() - t_start < budget_s and len(times) < max_reps):
+            t0 = time.perf_counter()
+            fn()
+            times.append(time.perf_counter() - t0)
+    finally:
+        torch.set_num_threads(prev)
+    times.sort()
+    return times[len(times) // 2], len(times)
 BYTES_PER_ELEM = 20                                        # load w, g; store y, dw, clamp(w)
 
 
@@ -56,32 +87,24 @@ def make_inputs(n, torch):
     return w, g
 
 
-def cpu_baseline(torch, sample_n, budget_s=15.0):
+def cpu_baseline(torch, sample_n, budget_s=8.0):
     """The reference's CPU op chain (oracle/torch_path.py) on the first sample_n elements of the
-    same workload, all host cores torch uses; GB/s on the same 20 B/element."""
+    same workload, on all host threads torch uses and on one; GB/s on the same 20 B/element."""
     from oracle import torch_path as tp
     w, g = make_inputs(sample_n, torch)
     gl = 1.0 / sample_n
     threads = torch.get_num_threads()
-    times = []
-    t_start = time.perf_counter()
-    reps = 0
-    while True:
-        d = HARDNESS[reps % len(HARDNESS)]
-        t0 = time.perf_counter()
-        tp.fused_step(w, g, d, SHARPNESS, STRENGTH, gl, -1.0, 1.0)
-        dt = time.perf_counter() - t0
-        if reps >= 1:                      # first repetition is the warm-up
-            times.append(dt)
-        reps += 1
-        if (len(times) >= 5 and time.perf_counter() - t_start > budget_s) or len(times) >= 25:
-            break
-    times.sort()
-    med = times[len(times) // 2]
+    k = [0]
+
+    def one():
+        tp.fused_step(w, g, HARDNESS[k[0] % len(HARDNESS)], SHARPNESS, STRENGTH, gl, -1.0, 1.0)
+        k[0] += 1
+    med, reps = timed_cpu(torch, one, threads, budget_s, min_reps=5, max_reps=25)
+    med1, reps1 = timed_cpu(torch, one, 1, budget_s / 2, min_reps=3, max_reps=10)
     return {"value": round(sample_n * BYTES_PER_ELEM / med / 1e9, 3), "unit": "GB/s", "cores": threads,
-            "kind": "port",
-            "sample": f"first {sample_n} elements of the workload, {len(times)} timed fused steps over the hardness "
-                      f"sweep, median; torch {torch.__version__} CPU ops in the reference's op order"}
+            "kind": "port", "value_1_thread": round(sample_n * BYTES_PER_ELEM / med1 / 1e9, 3), "cpu": cpu_model(),
+            "sample": f"first {sample_n} elements of the workload, {reps} ({reps1} on one thread) timed fused steps over "
+                      f"the hardness sweep, median; torch {torch.__version__} CPU ops in the reference's op order"}
 
 
 def bench_softstep(args, torch):
@@ -197,9 +220,55 @@ def bench_linear(args, torch):
     extra = {}
     if args.gemv_floor:
         extra = _gemv_floor_and_large(args, torch, natives)
-    return {"metric": "ternary-GEMM eff. TFLOP/s (K=N=4096)", "unit": "TFLOP/s", "n_gpus": 1, "dtype": "f16",
-            "data": "synthetic", "config": {"workload": "configs[2]: ternary linear K=N=4096", "rotate_buffers": nrot},
-            "value": out.get("4096", {}).get("tflops"), "by_M": out, **extra}
+    res = {"metric": "ternary-GEMM eff. TFLOP/s (K=N=4096)", "unit": "TFLOP/s", "n_gpus": 1, "dtype": "f16",
+           "data": "synthetic", "config": {"workload": "configs[2]: ternary linear K=N=4096", "rotate_buffers": nrot},
+           "value": out.get("4096", {}).get("tflops"), "by_M": out, **extra}
+    if "4096" in out:
+        o = out["4096"]
+        res["roofline"] = {"bound": "mfma", "achieved": o["tflops"], "peak": MFMA_FP16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                           "frac": o["frac_mfma_fp16"], "traffic": None, "algorithmic_flops": 2.0 * 4096 * N * K,
+                           "kernel": "tile_dma_kernel<128 x 256> (M = 4096)", "avg_launch_us": o["us"]}
+    if "1" in out:
+        o = out["1"]
+        res["roofline_gemv"] = {"bound": "hbm", "achieved": o["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                "frac": o["frac_hbm"], "traffic": None,
+                                "algorithmic_bytes": int(K * N / 4 + 2 * K + 8 * N),
+                                "kernel": "weight-stream GEMV (M = 1), %d rotating weight buffers" % nrot,
+                                "avg_launch_us": o["us"]}
+    if "gemv_16384" in extra:
+        o = extra["gemv_16384"]
+        res["roofline_gemv_16384"] = {"bound": "hbm", "achieved": o["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                      "frac": o["frac_hbm"], "traffic": None,
+                                      "algorithmic_bytes": int(16384 * 16384 / 4 + 2 * 16384 + 8 * 16384),
+                                      "kernel": "weight-stream GEMV (M = 1, K = N = 16384), 6 rotating weight buffers",
+                                      "avg_launch_us": o["us"]}
+    if not args.no_cpu:
+        res["cpu_baseline"] = cpu_baseline_linear(torch, W, scale.cpu())
+    return res
+
+
+def cpu_baseline_linear(torch, W, scale):
+    """The reference's CPU inference of a ternary layer: fp32 F.linear on ternary-valued fp32 weights
+    (it has no CPU path for packed weights), then the per-channel scale. M = 4096 and M = 1 at
+    K = N = 4096, all host threads and one thread (one thread: 512 of the 4096 rows)."""
+    F = torch.nn.functional
+    K = W.shape[1]
+    threads = torch.get_num_threads()
+    gen = torch.Generator(device="cpu").manual_seed(12)
+    x = torch.randn(4096, K, generator=gen)
+    x1 = x[:1].contiguous()
+    xs = x[:512].contiguous()
+    t_all, r_all = timed_cpu(torch, lambda: F.linear(x, W) * scale, threads, 4.0)
+    t_one, r_one = timed_cpu(torch, lambda: F.linear(xs, W) * scale, 1, 4.0)
+    t_v, _ = timed_cpu(torch, lambda: F.linear(x1, W) * scale, threads, 1.0, min_reps=10, max_reps=50)
+    t_v1, _ = timed_cpu(torch, lambda: F.linear(x1, W) * scale, 1, 1.0, min_reps=10, max_reps=50)
+    fl = 2.0 * W.shape[0] * K
+    return {"value": round(fl * 4096 / t_all / 1e12, 4), "unit": "TFLOP/s", "cores": threads, "kind": "port",
+            "value_1_thread": round(fl * 512 / t_one / 1e12, 4), "cpu": cpu_model(),
+            "gemv_tflops": round(fl / t_v / 1e12, 5), "gemv_tflops_1_thread": round(fl / t_v1 / 1e12, 5),
+            "gemv_us": round(t_v * 1e6, 1),
+            "sample": f"fp32 F.linear on ternary-valued fp32 weights, K = N = 4096: M = 4096 on {threads} threads "
+                      f"({r_all} reps), M = 512 on one thread ({r_one} reps), M = 1 on both; medians; torch {torch.__version__}"}
 
 
 def _graph_time_us(torch, calls, replays, settle_ms):
@@ -315,16 +384,51 @@ def bench_resnet_infer(args, torch):
             for _ in range(max(2, args.warmup // 4)):
                 fn()
             torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             t0 = time.perf_counter()
+            e0.record()
             for _ in range(reps):
                 fn()
+            e1.record()
             torch.cuda.synchronize()
         dt = (time.perf_counter() - t0) / reps
-        out[name] = {"ms": round(dt * 1e3, 4), "img_s": round(B / dt, 1), "tflops": round(3.627e9 * B / dt / 1e12, 2)}
+        out[name] = {"ms": round(dt * 1e3, 4), "gpu_ms": round(e0.elapsed_time(e1) / reps, 4), "img_s": round(B / dt, 1),
+                     "tflops": round(3.627e9 * B / dt / 1e12, 2)}
     t.set_compact_output_dtype(torch.float32)
-    return {"metric": "ResNet-18 img/s", "value": out["fused"]["img_s"], "unit": "img/s", "n_gpus": 1, "dtype": "f16",
-            "data": "synthetic", "config": {"workload": "configs[3]: ResNet-18/102 ternary inference", "batch": B},
-            "modes": out}
+    best = max(out, key=lambda k: out[k]["img_s"])
+    res = {"metric": "ResNet-18 img/s", "value": out["fused"]["img_s"], "unit": "img/s", "n_gpus": 1, "dtype": "f16",
+           "data": "synthetic", "config": {"workload": "configs[3]: ResNet-18/102 ternary inference", "batch": B},
+           "modes": out,
+           "roofline": {"bound": "mfma", "achieved": out["fused"]["tflops"], "peak": MFMA_FP16_PEAK_TFLOPS,
+                        "unit": "TFLOP/s", "frac": round(out["fused"]["tflops"] / MFMA_FP16_PEAK_TFLOPS, 4), "traffic": None,
+                        "algorithmic_flops": 3.627e9 * B,
+                        "kernel": "whole forward of the fused runner: 20 ternary implicit-GEMM convolutions, fc, pooling, "
+                                  "input repack (23 launches)",
+                        "avg_launch_us": round(out["fused"]["gpu_ms"] * 1e3, 2)},
+           "fastest_mode": best}
+    if not args.no_cpu:
+        res["cpu_baseline"] = cpu_baseline_resnet(torch)
+    return res
+
+
+def cpu_baseline_resnet(torch):
+    """The reference's CPU inference mode for a ternarised network: the fp32 model with ternary-valued
+    weights through F.conv2d / F.linear (samples/resnet_train.py:255-264), eval-mode BatchNorm. A
+    bounded sample of the batch: 16 images on all host threads, 4 on one."""
+    from bench_models import ResNet18, randomize_ternary_
+    torch.manual_seed(20)
+    model = ResNet18(102)
+    randomize_ternary_(model, torch.Generator().manual_seed(20))
+    model.eval()
+    x = torch.randn(16, 3, 224, 224, generator=torch.Generator().manual_seed(20))
+    threads = torch.get_num_threads()
+    with torch.no_grad():
+        t_all, r_all = timed_cpu(torch, lambda: model(x), threads, 5.0)
+        t_one, r_one = timed_cpu(torch, lambda: model(x[:4]), 1, 5.0)
+    return {"value": round(16 / t_all, 2), "unit": "img/s", "cores": threads, "kind": "port",
+            "value_1_thread": round(4 / t_one, 2), "cpu": cpu_model(),
+            "sample": f"fp32 ResNet-18/102 with ternary-valued weights (F.conv2d / F.linear, eval BatchNorm): 16 images on "
+                      f"{threads} threads ({r_all} reps), 4 images on one thread ({r_one} reps), medians; torch {torch.__version__}"}
 
 
 def bench_resnet_qat(args, torch):
@@ -363,37 +467,75 @@ def bench_resnet_qat(args, torch):
     torch.cuda.synchronize()
     dt = (time.perf_counter() - t0) / reps
 
-    # The TMQ kernels of one step on their own (GPU time between events): soft-step forward and backward
-    # of each of the 21 layers, the multi-tensor quantization loss and its gradient, the multi-tensor clamp.
+    # The TMQ kernels of one step on their own, exactly the launches the step above issues: the
+    # multi-tensor soft-step forward with the quantization loss, the multi-tensor backward
+    # (g S'(w) + loss gradient), the multi-tensor clamp. Eager (Python call overhead included, what a
+    # loop of these calls alone costs) and as HIP-graph replays (the kernels' own time).
     from tmq_amd import tmq as tmq_mod
     b = tmq_mod._b
-    ws = [node.weight for node in ctrl._registry.values()]
+    ws = [node.weight.data for node in ctrl._registry.values()]
     gs = [torch.randn_like(w) for w in ws]
+    up = torch.ones((), device=dev)
+    d, sharp, p = ctrl.digamma, float(ctrl.qpenalty_sharpness), float(ctrl.qpenalty)
+    n_w = sum(w.numel() for w in ws)
+    parts = {"fwd_loss": (lambda: b.softstep_fwd_all(ws, d, True, sharp, p), 8),
+             "bwd": (lambda: b.softstep_bwd_all(ws, gs, up, d, sharp, p), 12),
+             "clamp": (lambda: ctrl.clamp(), 8)}
 
     def tmq_only():
-        for w, g in zip(ws, gs):
-            b.fwd_softstep(w.data, ctrl.digamma)
-            b.bwd_softstep(w.data, ctrl.digamma, 1.0, g)
-        ctrl.quantization_loss().backward()
-        ctrl.clamp()
+        for fn, _ in parts.values():
+            fn()
+        return 1
 
     for _ in range(3):
         tmq_only()
     torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     e0.record()
-    for _ in range(reps):
+    for _ in range(20):
         tmq_only()
     e1.record()
     torch.cuda.synchronize()
-    tmq_ms = e0.elapsed_time(e1) / reps
-    nbytes = sum(w.numel() for w in ws) * (8 + 12 + 4 + 12 + 8)   # fwd, bwd, loss, loss gradient (accumulating), clamp
-    return {"metric": "ResNet-18 QAT step time", "value": round(dt * 1e3, 3), "unit": "ms", "higher_is_better": False,
-            "n_gpus": 1, "dtype": "f32", "data": "synthetic",
-            "config": {"workload": "configs[4]: ResNet-18 QAT step", "batch": B, "digamma": ctrl.digamma,
-                       "qpenalty": ctrl.qpenalty, "quantized_weights": 11219136},
-            "tmq_kernels_ms": round(tmq_ms, 4), "tmq_share": round(tmq_ms / (dt * 1e3), 4),
-            "tmq_algorithmic_bytes": nbytes, "tmq_gbs": round(nbytes / tmq_ms / 1e6, 1)}
+    eager_ms = e0.elapsed_time(e1) / 20
+    tmq_ms = _graph_time_us(torch, tmq_only, 50, args.settle_ms) / 1e3
+    per = {}
+    for name, (fn, bpe) in parts.items():
+        us = _graph_time_us(torch, lambda fn=fn: (fn(), 1)[1], 50, 10.0)
+        per[name] = {"us": round(us, 2), "gbs": round(n_w * bpe / us / 1e3, 1)}
+    nbytes = n_w * 28
+    res = {"metric": "ResNet-18 QAT step time", "value": round(dt * 1e3, 3), "unit": "ms", "higher_is_better": False,
+           "n_gpus": 1, "dtype": "f32", "data": "synthetic",
+           "config": {"workload": "configs[4]: ResNet-18 QAT step", "batch": B, "digamma": ctrl.digamma,
+                      "qpenalty": ctrl.qpenalty, "quantized_weights": n_w, "layers": len(ws)},
+           "tmq_kernels_ms": round(tmq_ms, 4), "tmq_share": round(tmq_ms / (dt * 1e3), 5),
+           "tmq_calls_eager_ms": round(eager_ms, 4), "tmq_algorithmic_bytes": nbytes, "tmq_launches": per,
+           "roofline": {"bound": "hbm", "achieved": round(nbytes / tmq_ms / 1e6, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                        "frac": round(nbytes / tmq_ms / 1e6 / HBM_PEAK_GBS, 4), "traffic": None,
+                        "algorithmic_bytes": nbytes,
+                        "kernel": "the step's TMQ launches: multi-tensor soft-step forward + loss (8 B/weight), loss "
+                                  "finalisation, multi-tensor backward (12 B/weight), multi-tensor clamp (8 B/weight)",
+                        "avg_launch_us": round(tmq_ms * 1e3, 2)}}
+    if not args.no_cpu:
+        res["cpu_baseline"] = cpu_baseline_qat(torch, [w.cpu() for w in ws], d, sharp, p)
+    return res
+
+
+def cpu_baseline_qat(torch, ws, d, sharp, p):
+    """The TMQ part of the same step on the reference's CPU op chains (oracle/torch_path.py), layer by
+    layer: soft-step forward and backward, loss and its gradient, clamp."""
+    from oracle import torch_path as tp
+    gs = [torch.randn_like(w) for w in ws]
+    threads = torch.get_num_threads()
+
+    def one():
+        for w, g in zip(ws, gs):
+            tp.fused_step(w, g, d, sharp, p, 1.0 / w.numel(), -1.0, 1.0)
+    t_all, r_all = timed_cpu(torch, one, threads, 4.0)
+    t_one, r_one = timed_cpu(torch, one, 1, 4.0, min_reps=2)
+    return {"value": round(t_all * 1e3, 2), "unit": "ms of TMQ work per step", "cores": threads, "kind": "port",
+            "value_1_thread": round(t_one * 1e3, 2), "cpu": cpu_model(),
+            "sample": f"all {len(ws)} weight tensors of the network ({sum(w.numel() for w in ws)} weights), {r_all} reps on "
+                      f"{threads} threads, {r_one} on one; medians; torch {torch.__version__} CPU ops in the reference's op order"}
 
 
 def main():
@@ -403,7 +545,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--settle-ms", type=float, default=60.0)
     ap.add_argument("--copy-calibration", action="store_true")
-    ap.add_argument("--workload", default="softstep")
+    ap.add_argument("--workload", default="all")
     ap.add_argument("--elements", type=int, default=1 << 26)
     ap.add_argument("--cpu-sample", type=int, default=1 << 22)
     ap.add_argument("--no-cpu", action="store_true")
@@ -420,7 +562,15 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
-    if args.workload == "softstep":
+    if args.workload == "all":
+        # the headline line (soft-step) with the other legs of the metric riding along under "also"
+        res = bench_softstep(args, torch)
+        torch.cuda.empty_cache()
+        res["also"] = {}
+        for name, leg in (("linear", bench_linear), ("resnet_infer", bench_resnet_infer), ("resnet_qat", bench_resnet_qat)):
+            res["also"][name] = leg(args, torch)
+            torch.cuda.empty_cache()
+    elif args.workload == "softstep":
         res = bench_softstep(args, torch)
     elif args.workload == "linear":
         res = bench_linear(args, torch)
