@@ -444,27 +444,46 @@ __global__ __launch_bounds__(kFinThreads) void finalize_kernel(R rg, const float
         }
     }
     __syncthreads();
+    // One thread per tensor: its task sums in order, the factor, the mean. Then thread 0 adds the means
+    // in table order (the reference adds per-layer means one by one in fp32, tmq/tmq.py:309).
+    __shared__ float means[kFinThreads];
+    __shared__ float run_s;
+    __shared__ int first_s;
     if (threadIdx.x == 0) {
-        float running = carry ? *carry : 0.f;
-        bool first = carry == nullptr;
-        uint32_t tk = 0;
-        for (int l = 0; l < nseg; l++) {
-            const uint32_t b0 = rg.begin(l), b1 = rg.end(l);
-            const uint32_t ntask = (b1 - b0 + kTaskLen - 1) / kTaskLen;
+        run_s = carry ? *carry : 0.f;
+        first_s = carry == nullptr;
+    }
+    for (int l0 = 0; l0 < nseg; l0 += kFinThreads) {
+        const int l = l0 + threadIdx.x;
+        if (l < nseg) {
+            uint32_t tk = 0;
+            for (int j = 0; j < l; j++) tk += (rg.end(j) - rg.begin(j) + kTaskLen - 1) / kTaskLen;
+            const uint32_t ntask = (rg.end(l) - rg.begin(l) + kTaskLen - 1) / kTaskLen;
             double sum = 0.0;
-            for (uint32_t t = 0; t < ntask; t++) sum += task_sum[tk++];
+            for (uint32_t t = 0; t < ntask; t++) sum += task_sum[tk + t];
             sum *= factor;   // partials hold sum dsig; factor = strength*sharpness/c
             if (sum_out) sum_out[l] = sum;
             if (rg.has_mean()) {
-                const uint64_t n = rg.elems(l);
-                float mean = (float)(sum / (double)n);   // n == 0 gives NaN like torch.mean of an empty tensor
+                const float mean = (float)(sum / (double)rg.elems(l));   // n == 0 gives NaN like torch.mean of an empty tensor
                 if (per_tensor) per_tensor[l] = mean;
-                running = first ? mean : running + mean;
-                first = false;
+                means[threadIdx.x] = mean;
             }
         }
-        if (total) *total = running;
+        __syncthreads();
+        if (threadIdx.x == 0 && rg.has_mean()) {
+            float running = run_s;
+            bool first = first_s != 0;
+            const int cnt = nseg - l0 < kFinThreads ? nseg - l0 : kFinThreads;
+            for (int j = 0; j < cnt; j++) {
+                running = first ? means[j] : running + means[j];
+                first = false;
+            }
+            run_s = running;
+            first_s = 0;
+        }
+        __syncthreads();
     }
+    if (threadIdx.x == 0 && total && rg.has_mean()) *total = run_s;
 }
 
 inline bool finalize_fits(int nseg, uint32_t total_blocks) {
