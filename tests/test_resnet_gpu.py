@@ -44,6 +44,9 @@ def test_compact_inference_matches_fp32_reference(cuda):
         h.remove()
     with torch.no_grad():
         ref_plain = model(x)
+    import copy
+    from tests.test_exact_configs_gpu import _faithful_reference
+    ref16 = _faithful_reference(copy.deepcopy(model), x)      # activations rounded to fp16 where the fused kernels store them
     sd = t.compressed_state_dict(model, strong=False)
     packed_bytes = sum(v.numel() * 4 for k, v in sd.items() if v.dtype == torch.int32)
     assert packed_bytes == sum(((n.original_shape[0] + 15) // 16) * 4 * int(np.prod(n.original_shape[1:]))
@@ -58,9 +61,9 @@ def test_compact_inference_matches_fp32_reference(cuda):
     fused = FusedTernaryResNet18(model)
     yf = fused(x.half())
     assert tuple(yf.shape) == (4, 102)
-    errf = (yf - ref_plain).abs().max().item() / ref_plain.abs().max().item()
-    assert errf <= 3e-2, errf
-    assert (yf.argmax(1) == ref_plain.argmax(1)).float().mean().item() >= 0.75
+    errf = (yf.float() - ref16).abs().max().item() / ref16.abs().max().item()
+    assert errf <= 1e-3, errf
+    assert (yf.float() - ref_plain).abs().max().item() / ref_plain.abs().max().item() <= 3e-2   # fp16 vs fp32 activations
 
 
 def test_qat_step_runs_and_matches_unfused_losses(cuda):
