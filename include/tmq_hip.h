@@ -122,14 +122,6 @@ int tmq_softstep_fused_noalloc(const float *w, const float *g, float *y, float *
                                double *loss_sum, size_t n, double digamma, double sharpness,
                                double strength, float gl, double lo, double hi, void *stream);
 
-/* Diagnostic with no counterpart in the reference: the kernels above replace IEEE division by
- * cheaper FMA sequences; this proves on the device that they are bit-identical to IEEE
- * division. counts (device, 5 x uint64) receives: [0..2] mismatches of the three rational
- * pieces over every fp32 argument in [-3,3] (and NaN), [3] mismatches of x / c(digamma) over
- * every mantissa, both signs, three binades, [4] the number of arguments swept (a sanity
- * figure, 2*0x40400000 + 1 + NaNs). All mismatch counts must be 0.                           */
-int tmq_selfcheck_division(double digamma, uint64_t *counts, void *stream);
-
 /* ------------------------------------------------------------------------------------------
  * Multi-tensor (one launch for every registered layer) forms of the per-layer Python loops of
  * QuantizationControl.quantization_loss / clamp (tmq/tmq.py:298-310, 263-272).
@@ -255,40 +247,47 @@ typedef struct tmq_epilogue {
     int32_t y_dtype;
 } tmq_epilogue;
 
-/* x [M][K] row-major, x_dtype TMQ_F16 or TMQ_F32 (fp32 activations are split into two fp16 terms
- * so the product keeps ~fp32 accuracy); y [M][N].
+/* x [M][K] row-major, x_dtype TMQ_F16 or TMQ_F32; y [M][N].
+ * fp32 activations are carried as two fp16 terms (22 significant bits), so they must lie inside fp16's
+ * exponent range: max|x| at most 65504, and values below ~6e-5 lose precision. Tensors of any other
+ * magnitude go through tmq_f32_prescale first (exact power-of-two scaling, undone in the per-channel scale of
+ * the epilogue); the Python / PyTorch bindings of this library always do, because the reference multiplies
+ * fp32 activations in fp32 and has no such limit.
  * Replaces ternary_mvm_cuda (tmq/tmq_cuda.cu:563-603, kernel 242-286) for M == 1 and
  * ternary_mmm_cuda (tmq/tmq_cuda.cu:478-549, kernel 289-427) for M > 1, plus the post-scale /
  * bias passes of Linear.compact_forward (tmq/tmq.py:684-687). Any M, K, N (ragged tails masked). */
 int tmq_ternary_linear(const void *x, int x_dtype, int64_t M, int64_t K, const void *native,
                        int64_t N, const tmq_epilogue *epilogue, void *y, void *stream);
 
-/* hi[i] = fp16(x[i]), lo[i] = fp16(x[i] - hi[i]) for n fp32 values (device pointers; hi, lo fp16).
+/* Range handling for fp32 activations (no counterpart in the reference, whose kernels multiply fp32
+ * activations in fp32, tmq/tmq_cuda.cu:242-427). Scans n fp32 values and writes prescale[0] = s,
+ * prescale[1] = 1 / s (device, 2 floats): s is the power of two that brings the largest finite |x| into
+ * [1024, 2048) (s = 1 for an all-zero tensor). Optionally, in the same call:
+ *   xs (n floats)             xs[i] = s * x[i] (exact), the tensor to hand to tmq_ternary_linear;
+ *   scale_out (channels)      scale_out[c] = (scale_in ? scale_in[c] : 1) / s, the epilogue scale that
+ *                             undoes the prescale (bias and residual are added after it, unscaled).
+ * Up to 65536 values are handled by one launch; beyond that by two (three with xs) and `workspace` must
+ * hold tmq_f32_prescale_workspace_bytes(n) bytes.                                                  */
+size_t tmq_f32_prescale_workspace_bytes(int64_t n);
+int tmq_f32_prescale(const float *x, int64_t n, float *prescale, float *xs, const float *scale_in,
+                     float *scale_out, int64_t channels, void *workspace, void *stream);
+
+/* hi[i] = fp16(s x[i]), lo[i] = fp16(s x[i] - hi[i]) for n fp32 values (device pointers; hi, lo fp16), s =
+ * prescale[0] (device; NULL = 1). lo may be NULL when one term is enough (the convolutions take fp16).
  * No counterpart in the reference, whose ternary_mmm_cuda (tmq/tmq_cuda.cu:478-549) multiplies fp32
  * activations in fp32: for many rows a caller that may allocate runs the fp16 kernels on the two terms,
  *   t = tmq_ternary_linear(hi, ..., scale, bias, residual)  (fp32 out, no ReLU)
  *   y = tmq_ternary_linear(lo, ..., scale, residual = t, ReLU)
  * which keeps ~fp32 accuracy at MFMA speed (M = 4096, K = N = 4096: 400 -> 238 us); the bindings in
- * tmq_amd/ops.py and tmq_amd/csrc/torch_ext.cpp do so where tmq_fp32_rows_prefer_split says it pays. */
+ * tmq_amd/ops.py and tmq_amd/csrc/torch_ext.cpp do so where tmq_fp32_rows_prefer_split says it pays.
+ * tmq_split_f32 is the form without a prescale.                                                     */
+int tmq_split_f32_scaled(const float *x, const float *prescale, void *hi, void *lo, int64_t n, void *stream);
 int tmq_split_f32(const float *x, void *hi, void *lo, int64_t n, void *stream);
 
 /* 1 if M fp32 rows against a K x N layer are faster as two fp16 passes over tmq_split_f32's terms than
  * as one tmq_ternary_linear call with x_dtype TMQ_F32 (many rows, or a few rows over a large
  * layer), else 0. Host-only arithmetic on the shape; no counterpart in the reference.               */
 int tmq_fp32_rows_prefer_split(int64_t M, int64_t K, int64_t N);
-
-/* Measurement aid with no counterpart in the reference: streams `bytes` (a multiple of 1024)
- * from src with the launch geometry of the M = 1 path of tmq_ternary_linear (1 KiB per
- * wavefront and load, 16 wavefronts per workgroup) and does nothing else; *sink (device, 4
- * bytes) is only written if the data has an impossible checksum. Its duration is the floor for
- * a kernel that has to read that many bytes once: launch + one trip to memory.               */
-int tmq_probe_stream_read(const void *src, size_t bytes, uint32_t *sink, void *stream);
-
-/* Diagnostic with no counterpart in the reference, host only: the convolution and pooling kernels
- * turn an output pixel's index into (batch, row, column) with a multiply-high by constants computed on
- * the host instead of integer divisions. Returns how many of n[0 .. count) (host memory, each below
- * 2^31) the same constants divide wrongly by `divisor` (1 <= divisor < 2^31): must be 0.            */
-int64_t tmq_selfcheck_fastdiv(uint32_t divisor, const uint32_t *n, int64_t count);
 
 /* Geometry of a 2-D convolution. */
 typedef struct tmq_conv_shape {
@@ -367,6 +366,34 @@ int tmq_avgpool_global_nhwc(const void *x, int64_t B, int64_t HW, int64_t C, voi
  * fp16, channels C..3 zero (the layout the few-channel convolution loader wants).               */
 int tmq_nchw_to_nhwc4(const void *x, int x_dtype, int64_t B, int32_t C, int64_t H, int64_t W, void *y,
                       void *stream);
+
+/* ------------------------------------------------------------------------------------------
+ * DIAGNOSTICS AND MEASUREMENT AIDS. Not part of the product surface: nothing in the library's own
+ * call paths uses them and a caller never needs them. They exist for the test suite (device-side
+ * proofs about the kernels' arithmetic) and for the benchmark (a read-only stream as the floor a
+ * GEMV is compared with). None has a counterpart in the reference.
+ * ---------------------------------------------------------------------------------------- */
+
+/* Diagnostic with no counterpart in the reference: the kernels above replace IEEE division by
+ * cheaper FMA sequences; this proves on the device that they are bit-identical to IEEE
+ * division. counts (device, 5 x uint64) receives: [0..2] mismatches of the three rational
+ * pieces over every fp32 argument in [-3,3] (and NaN), [3] mismatches of x / c(digamma) over
+ * every mantissa, both signs, three binades, [4] the number of arguments swept (a sanity
+ * figure, 2*0x40400000 + 1 + NaNs). All mismatch counts must be 0.                           */
+int tmq_selfcheck_division(double digamma, uint64_t *counts, void *stream);
+
+/* Measurement aid with no counterpart in the reference: streams `bytes` (a multiple of 1024)
+ * from src with the launch geometry of the M = 1 path of tmq_ternary_linear (1 KiB per
+ * wavefront and load, 16 wavefronts per workgroup) and does nothing else; *sink (device, 4
+ * bytes) is only written if the data has an impossible checksum. Its duration is the floor for
+ * a kernel that has to read that many bytes once: launch + one trip to memory.               */
+int tmq_probe_stream_read(const void *src, size_t bytes, uint32_t *sink, void *stream);
+
+/* Diagnostic with no counterpart in the reference, host only: the convolution and pooling kernels
+ * turn an output pixel's index into (batch, row, column) with a multiply-high by constants computed on
+ * the host instead of integer divisions. Returns how many of n[0 .. count) (host memory, each below
+ * 2^31) the same constants divide wrongly by `divisor` (1 <= divisor < 2^31): must be 0.            */
+int64_t tmq_selfcheck_fastdiv(uint32_t divisor, const uint32_t *n, int64_t count);
 
 /* ------------------------------------------------------------------------------------------
  * Host entropy codec for packed tensors (host memory in, host memory out; no GPU involved).

@@ -1,6 +1,8 @@
 """Compiles the reference's own host codec / packer (tmq/tmq_native.cpp with rangecoder.h and
 bitstream.h) from the sources where they lie in the reference tree into oracle/_ref/ -- a
-checker for the tests, never committed and never shipped. One g++ command on the reference's own
+checker for the tests. The built library is kept out of version control; it travels to a GPU machine
+with the rest of the tree like the library's own binaries, where only the tests may load it (they run
+from the committed fixtures when it is absent). One g++ command on the reference's own
 file; the reference's build system is not run. The CUDA file needs nvcc and is not buildable
 in this image.
 

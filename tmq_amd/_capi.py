@@ -66,6 +66,9 @@ SIGNATURES = {
     "tmq_selfcheck_division": (_int, [_dbl, _vp, _vp]),
     "tmq_probe_stream_read": (_int, [_vp, ctypes.c_size_t, _vp, _vp]),
     "tmq_split_f32": (_int, [_vp, _vp, _vp, _i64, _vp]),
+    "tmq_split_f32_scaled": (_int, [_vp, _vp, _vp, _vp, _i64, _vp]),
+    "tmq_f32_prescale_workspace_bytes": (_sz, [_i64]),
+    "tmq_f32_prescale": (_int, [_vp, _i64, _vp, _vp, _vp, _vp, _i64, _vp, _vp]),
     "tmq_selfcheck_fastdiv": (_i64, [_u32, _vp, _i64]),
     "tmq_fp32_rows_prefer_split": (_int, [_i64, _i64, _i64]),
     "tmq_multi_plan": (_int, [ctypes.POINTER(Segment), _int, ctypes.POINTER(_u32)]),
@@ -148,3 +151,11 @@ def require_gpu(t, name="tensor"):
         raise RuntimeError(f"{name} must live on the GPU")
     if not t.is_contiguous():
         raise RuntimeError(f"{name} must be contiguous")
+
+
+def require_gpu_dense(t, name="tensor"):
+    """On the GPU and dense in memory (contiguous in the default or the channels_last format)."""
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must live on the GPU")
+    if not (t.is_contiguous() or (t.dim() == 4 and t.is_contiguous(memory_format=torch.channels_last))):
+        raise RuntimeError(f"{name} must be dense in memory")

@@ -58,7 +58,7 @@ __device__ __forceinline__ void store8(const DwEpilogue &ep, int64_t o, int64_t 
         if (ep.bias) v += ep.bias[c0 + e];
         if (ep.residual)
             v += ep.y_f16 ? (float)static_cast<const _Float16 *>(ep.residual)[o + e] : static_cast<const float *>(ep.residual)[o + e];
-        if (ep.relu) v = v > 0.f ? v : 0.f;
+        if (ep.relu) v = v < 0.f ? 0.f : v;
         acc[e] = v;
     }
     if (vec) {
@@ -120,7 +120,7 @@ __device__ __forceinline__ void store8_vec(const DwEpilogue &ep, const ChannelCo
     }
     if (ep.relu) {
 #pragma unroll
-        for (int e = 0; e < 8; e++) v[e] = v[e] > 0.f ? v[e] : 0.f;
+        for (int e = 0; e < 8; e++) v[e] = v[e] < 0.f ? 0.f : v[e];
     }
     if (ep.y_f16) {
         half8 h;

@@ -304,11 +304,11 @@ __global__ __launch_bounds__(1024) void skinny_kernel(const void *__restrict__ x
                     const int64_t o = m * N + n;
                     if (y_f16) {
                         if (residual) v += (float)static_cast<const _Float16 *>(residual)[o];
-                        if (relu) v = v > 0.f ? v : 0.f;
+                        if (relu) v = v < 0.f ? 0.f : v;
                         static_cast<_Float16 *>(y)[o] = (_Float16)v;
                     } else {
                         if (residual) v += static_cast<const float *>(residual)[o];
-                        if (relu) v = v > 0.f ? v : 0.f;
+                        if (relu) v = v < 0.f ? 0.f : v;
                         static_cast<float *>(y)[o] = v;
                     }
                 }
@@ -389,11 +389,11 @@ __global__ __launch_bounds__(1024) void gemv_short_kernel(const _Float16 *__rest
                 float v = s[r] * (sc4[r] * (1.0f / kWeightUnit)) + bi4[r];
                 if (y_f16) {
                     if (residual) v += (float)static_cast<const _Float16 *>(residual)[n];
-                    if (relu) v = v > 0.f ? v : 0.f;
+                    if (relu) v = v < 0.f ? 0.f : v;
                     static_cast<_Float16 *>(y)[n] = (_Float16)v;
                 } else {
                     if (residual) v += static_cast<const float *>(residual)[n];
-                    if (relu) v = v > 0.f ? v : 0.f;
+                    if (relu) v = v < 0.f ? 0.f : v;
                     static_cast<float *>(y)[n] = v;
                 }
             }
@@ -485,11 +485,11 @@ __global__ __launch_bounds__(1024) void short_rows_kernel(const _Float16 *__rest
                 const int64_t o = (int64_t)j * N + n;
                 if (y_f16) {
                     if (residual) v += (float)static_cast<const _Float16 *>(residual)[o];
-                    if (relu) v = v > 0.f ? v : 0.f;
+                    if (relu) v = v < 0.f ? 0.f : v;
                     static_cast<_Float16 *>(y)[o] = (_Float16)v;
                 } else {
                     if (residual) v += static_cast<const float *>(residual)[o];
-                    if (relu) v = v > 0.f ? v : 0.f;
+                    if (relu) v = v < 0.f ? 0.f : v;
                     static_cast<float *>(y)[o] = v;
                 }
             }
@@ -763,11 +763,11 @@ __global__ __launch_bounds__(64 * WAVES) void mid_kernel(const void *__restrict_
                 const int64_t o = m * N + n;
                 if (y_f16) {
                     if (residual) v += (float)static_cast<const _Float16 *>(residual)[o];
-                    if (relu) v = v > 0.f ? v : 0.f;
+                    if (relu) v = v < 0.f ? 0.f : v;
                     static_cast<_Float16 *>(y)[o] = (_Float16)v;
                 } else {
                     if (residual) v += static_cast<const float *>(residual)[o];
-                    if (relu) v = v > 0.f ? v : 0.f;
+                    if (relu) v = v < 0.f ? 0.f : v;
                     static_cast<float *>(y)[o] = v;
                 }
             }
@@ -985,11 +985,11 @@ __global__ __launch_bounds__(64 * WAVES) void mid_lds_kernel(const void *__restr
                 const int64_t o = m * N + n;
                 if (y_f16) {
                     if (residual) v += (float)static_cast<const _Float16 *>(residual)[o];
-                    if (relu) v = v > 0.f ? v : 0.f;
+                    if (relu) v = v < 0.f ? 0.f : v;
                     static_cast<_Float16 *>(y)[o] = (_Float16)v;
                 } else {
                     if (residual) v += static_cast<const float *>(residual)[o];
-                    if (relu) v = v > 0.f ? v : 0.f;
+                    if (relu) v = v < 0.f ? 0.f : v;
                     static_cast<float *>(y)[o] = v;
                 }
             }
@@ -1044,35 +1044,6 @@ int mid_rows(const void *x, int64_t M, int64_t K, const void *native, int64_t N,
     return launch_mid<2, 1, 2, 16, 2, X32>(x, M, K, native, N, ep, y, stream);
 }
 
-// ---- two-term split ------------------------------------------------------------------------------
-// x = hi + lo with hi = fp16(x), lo = fp16(x - hi): 22 significant bits in two fp16 values. 8 elements per
-// thread (two 16-byte loads, a 16-byte store per term) when the pointers allow it.
-__global__ __launch_bounds__(256) void split_terms_kernel(const float *__restrict__ x, _Float16 *__restrict__ hi,
-                                                          _Float16 *__restrict__ lo, int64_t n, int vec) {
-    const int64_t i0 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 8;
-    if (i0 >= n) return;
-    if (vec && i0 + 8 <= n) {
-        const floatx4 a = __builtin_nontemporal_load(reinterpret_cast<const floatx4 *>(x + i0));
-        const floatx4 b = __builtin_nontemporal_load(reinterpret_cast<const floatx4 *>(x + i0 + 4));
-        half8 h, l;
-#pragma unroll
-        for (int e = 0; e < 4; e++) {
-            h[e] = (_Float16)a[e];
-            h[4 + e] = (_Float16)b[e];
-            l[e] = (_Float16)(a[e] - (float)h[e]);
-            l[4 + e] = (_Float16)(b[e] - (float)h[4 + e]);
-        }
-        *reinterpret_cast<half8 *>(hi + i0) = h;
-        *reinterpret_cast<half8 *>(lo + i0) = l;
-    } else {
-        for (int64_t i = i0; i < n && i < i0 + 8; i++) {
-            const _Float16 h = (_Float16)x[i];
-            hi[i] = h;
-            lo[i] = (_Float16)(x[i] - (float)h);
-        }
-    }
-}
-
 // ---- read probe -------------------------------------------------------------------------------------
 // The weight stream of the skinny kernel and nothing else: wavefront w of a workgroup reads the
 // 1 KiB pieces w, w + 16, ... of the workgroup's share.
@@ -1125,17 +1096,6 @@ int tmq_fp32_rows_prefer_split(int64_t M, int64_t K, int64_t N) {
     const double weights = (double)K * (double)N;
     const bool large_layer = (M >= 9 && weights >= 67108864.0) || (M >= 3 && weights >= 134217728.0);
     return many_rows || large_layer;
-}
-
-int tmq_split_f32(const float *x, void *hi, void *lo, int64_t n, void *stream) {
-    if (n < 0 || (n > 0 && (!x || !hi || !lo))) return TMQ_ERR_INVALID_ARG;
-    if (n == 0) return TMQ_OK;
-    const int64_t blocks = (n + 2047) / 2048;
-    if (blocks > 0x7FFFFFFF) return TMQ_ERR_TOO_LARGE;
-    const int vec = aligned16(x) && aligned16(hi) && aligned16(lo);
-    hipLaunchKernelGGL(split_terms_kernel, dim3((uint32_t)blocks), dim3(256), 0, as_stream(stream), x,
-                       static_cast<_Float16 *>(hi), static_cast<_Float16 *>(lo), n, vec);
-    return check_launch();
 }
 
 int tmq_probe_stream_read(const void *src, size_t bytes, uint32_t *sink, void *stream) {

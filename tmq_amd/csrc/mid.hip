@@ -245,7 +245,7 @@ __device__ __forceinline__ void reduce_and_store(unsigned char *smem, const floa
                 if (ep.residual) v += res32[it];
                 if (ep.relu) {
 #pragma unroll
-                    for (int r = 0; r < 4; r++) v[r] = v[r] > 0.f ? v[r] : 0.f;
+                    for (int r = 0; r < 4; r++) v[r] = v[r] < 0.f ? 0.f : v[r];
                 }
                 *reinterpret_cast<floatx4 *>(static_cast<float *>(ep.y) + o) = v;
             }

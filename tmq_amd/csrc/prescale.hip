@@ -1,0 +1,230 @@
+// fp32 activations for the fp16 MFMA kernels: the power-of-two prescale that brings a tensor into fp16's
+// range, and the split of (prescaled) values into fp16 terms.
+//
+// The ternary kernels multiply fp16 operands. fp32 activations are carried as hi = fp16(x), lo = fp16(x - hi)
+// (22 significant bits), which only works while x sits inside fp16's exponent range: above 65504 hi
+// overflows, below ~6e-5 the terms are subnormal and lose their bits. The reference multiplies in fp32
+// (tmq/tmq_cuda.cu:242-427) and has no such limit. So a caller first scales the tensor by the power of two s
+// that puts max|x| into [1024, 2048) -- exact, whatever the magnitude -- and folds 1/s into the
+// per-channel scale of the epilogue; elements more than 2^14 below the maximum keep an absolute
+// precision of 2^-35 of that maximum, which is below the rounding of the fp32 accumulation.
+#include "common.h"
+#include "mfma.h"
+
+#include <math.h>
+
+namespace tmq {
+namespace {
+
+constexpr int kPartials = 1024;           // partial maxima of the multi-block scan
+constexpr int64_t kSingleMax = 1 << 16;   // up to here one workgroup does everything in one launch
+
+__device__ __forceinline__ float finite_abs(float v) {
+    const float a = __builtin_fabsf(v);
+    return a < INFINITY ? a : 0.f;          // NaN and Inf take no part in the maximum (they propagate anyway)
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+    return v;
+}
+
+// maximum over the workgroup, valid in every thread
+__device__ __forceinline__ float block_max(float v, float *lds /* >= 17 floats */) {
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
+    v = wave_max(v);
+    if (lane == 0) lds[wv] = v;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float t = 0.f;
+        for (int i = 0; i < nw; i++) t = fmaxf(t, lds[i]);
+        lds[16] = t;
+    }
+    __syncthreads();
+    return lds[16];
+}
+
+// s = 2^(11 - e) for amax in [2^(e-1), 2^e), kept inside the normal range together with its reciprocal.
+__device__ __forceinline__ void make_prescale(float amax, float &s, float &inv) {
+    s = 1.f;
+    inv = 1.f;
+    if (!(amax > 0.f)) return;
+    int e;
+    (void)frexpf(amax, &e);
+    int p = 11 - e;
+    p = p > 126 ? 126 : (p < -126 ? -126 : p);
+    s = ldexpf(1.f, p);
+    inv = ldexpf(1.f, -p);
+}
+
+__device__ __forceinline__ float scan_abs_max(const float *__restrict__ x, int64_t n, int64_t first, int64_t stride, bool vec) {
+    float m = 0.f;
+    if (vec) {
+        const int64_t n4 = n / 4;
+        for (int64_t i = first; i < n4; i += stride) {
+            const floatx4 v = *reinterpret_cast<const floatx4 *>(x + 4 * i);
+            m = fmaxf(fmaxf(m, fmaxf(finite_abs(v[0]), finite_abs(v[1]))), fmaxf(finite_abs(v[2]), finite_abs(v[3])));
+        }
+        for (int64_t i = 4 * n4 + first; i < n; i += stride) m = fmaxf(m, finite_abs(x[i]));
+    } else {
+        for (int64_t i = first; i < n; i += stride) m = fmaxf(m, finite_abs(x[i]));
+    }
+    return m;
+}
+
+__device__ __forceinline__ void write_scale(const float *scale_in, float *scale_out, int64_t channels, float inv) {
+    if (!scale_out) return;
+    for (int64_t c = threadIdx.x; c < channels; c += blockDim.x) scale_out[c] = (scale_in ? scale_in[c] : 1.f) * inv;
+}
+
+// Small tensors: one workgroup scans, derives the prescale, writes the scaled copy and the adjusted
+// per-channel scale -- one launch in front of a GEMV.
+__global__ __launch_bounds__(1024) void prescale_single_kernel(const float *__restrict__ x, int64_t n, float *prescale,
+                                                               float *__restrict__ xs, const float *scale_in,
+                                                               float *scale_out, int64_t channels, int vec) {
+    __shared__ float lds[17];
+    const float amax = block_max(scan_abs_max(x, n, threadIdx.x, blockDim.x, vec != 0), lds);
+    float s, inv;
+    make_prescale(amax, s, inv);
+    if (threadIdx.x == 0) {
+        prescale[0] = s;
+        prescale[1] = inv;
+    }
+    if (xs) {
+        if (vec) {
+            const int64_t n4 = n / 4;
+            for (int64_t i = threadIdx.x; i < n4; i += blockDim.x)
+                *reinterpret_cast<floatx4 *>(xs + 4 * i) = *reinterpret_cast<const floatx4 *>(x + 4 * i) * s;
+            for (int64_t i = 4 * n4 + threadIdx.x; i < n; i += blockDim.x) xs[i] = x[i] * s;
+        } else {
+            for (int64_t i = threadIdx.x; i < n; i += blockDim.x) xs[i] = x[i] * s;
+        }
+    }
+    write_scale(scale_in, scale_out, channels, inv);
+}
+
+__global__ __launch_bounds__(256) void absmax_partial_kernel(const float *__restrict__ x, int64_t n, float *partials, int vec) {
+    __shared__ float lds[17];
+    const float m = block_max(scan_abs_max(x, n, (int64_t)blockIdx.x * 256 + threadIdx.x, (int64_t)gridDim.x * 256, vec != 0), lds);
+    if (threadIdx.x == 0) partials[blockIdx.x] = m;
+}
+
+__global__ __launch_bounds__(1024) void prescale_finalize_kernel(const float *partials, int count, float *prescale,
+                                                                 const float *scale_in, float *scale_out, int64_t channels) {
+    __shared__ float lds[17];
+    const float amax = block_max((int)threadIdx.x < count ? partials[threadIdx.x] : 0.f, lds);
+    float s, inv;
+    make_prescale(amax, s, inv);
+    if (threadIdx.x == 0) {
+        prescale[0] = s;
+        prescale[1] = inv;
+    }
+    write_scale(scale_in, scale_out, channels, inv);
+}
+
+__global__ __launch_bounds__(256) void scale_copy_kernel(const float *__restrict__ x, const float *prescale,
+                                                         float *__restrict__ xs, int64_t n, int vec) {
+    const float s = prescale[0];
+    const int64_t i0 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i0 >= n) return;
+    if (vec && i0 + 4 <= n) {
+        *reinterpret_cast<floatx4 *>(xs + i0) = __builtin_nontemporal_load(reinterpret_cast<const floatx4 *>(x + i0)) * s;
+    } else {
+        for (int64_t i = i0; i < n && i < i0 + 4; i++) xs[i] = x[i] * s;
+    }
+}
+
+// x s = hi + lo with hi = fp16(x s), lo = fp16(x s - hi): 22 significant bits in two fp16 values (s = 1 without
+// a prescale; lo may be left out). 8 elements per thread (two 16-byte loads, a 16-byte store per term) when
+// the pointers allow it.
+template <bool LO, bool SCALED>
+__global__ __launch_bounds__(256) void split_terms_kernel(const float *__restrict__ x, const float *prescale,
+                                                          _Float16 *__restrict__ hi, _Float16 *__restrict__ lo, int64_t n,
+                                                          int vec) {
+    float s = 1.f;
+    if constexpr (SCALED) s = prescale[0];
+    const int64_t i0 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 8;
+    if (i0 >= n) return;
+    if (vec && i0 + 8 <= n) {
+        floatx4 a = __builtin_nontemporal_load(reinterpret_cast<const floatx4 *>(x + i0));
+        floatx4 b = __builtin_nontemporal_load(reinterpret_cast<const floatx4 *>(x + i0 + 4));
+        if constexpr (SCALED) {
+            a *= s;
+            b *= s;
+        }
+        half8 h, l;
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            h[e] = (_Float16)a[e];
+            h[4 + e] = (_Float16)b[e];
+            l[e] = (_Float16)(a[e] - (float)h[e]);
+            l[4 + e] = (_Float16)(b[e] - (float)h[4 + e]);
+        }
+        *reinterpret_cast<half8 *>(hi + i0) = h;
+        if constexpr (LO) *reinterpret_cast<half8 *>(lo + i0) = l;
+    } else {
+        for (int64_t i = i0; i < n && i < i0 + 8; i++) {
+            const float v = SCALED ? x[i] * s : x[i];
+            const _Float16 h = (_Float16)v;
+            hi[i] = h;
+            if constexpr (LO) lo[i] = (_Float16)(v - (float)h);
+        }
+    }
+}
+
+}  // namespace
+}  // namespace tmq
+
+using namespace tmq;
+
+extern "C" {
+
+size_t tmq_f32_prescale_workspace_bytes(int64_t n) { return n > kSingleMax ? kPartials * sizeof(float) : 0; }
+
+int tmq_f32_prescale(const float *x, int64_t n, float *prescale, float *xs, const float *scale_in, float *scale_out,
+                     int64_t channels, void *workspace, void *stream) {
+    if (n <= 0 || !x || !prescale || channels < 0 || (scale_out && channels == 0)) return TMQ_ERR_INVALID_ARG;
+    const int vec = aligned16(x) && (!xs || aligned16(xs));
+    if (n <= kSingleMax) {
+        hipLaunchKernelGGL(prescale_single_kernel, dim3(1), dim3(1024), 0, as_stream(stream), x, n, prescale, xs, scale_in,
+                           scale_out, channels, vec);
+        return check_launch();
+    }
+    if (!workspace) return TMQ_ERR_INVALID_ARG;
+    float *partials = static_cast<float *>(workspace);
+    int64_t blocks = (n + 8191) / 8192;                    // 32 values per thread and more
+    if (blocks > kPartials) blocks = kPartials;
+    hipLaunchKernelGGL(absmax_partial_kernel, dim3((uint32_t)blocks), dim3(256), 0, as_stream(stream), x, n, partials,
+                       (int)aligned16(x));
+    int rc = check_launch();
+    if (rc != TMQ_OK) return rc;
+    hipLaunchKernelGGL(prescale_finalize_kernel, dim3(1), dim3(1024), 0, as_stream(stream), partials, (int)blocks, prescale,
+                       scale_in, scale_out, channels);
+    rc = check_launch();
+    if (rc != TMQ_OK || !xs) return rc;
+    const int64_t cblocks = (n + 1023) / 1024;
+    if (cblocks > 0x7FFFFFFF) return TMQ_ERR_TOO_LARGE;
+    hipLaunchKernelGGL(scale_copy_kernel, dim3((uint32_t)cblocks), dim3(256), 0, as_stream(stream), x, prescale, xs, n, vec);
+    return check_launch();
+}
+
+int tmq_split_f32_scaled(const float *x, const float *prescale, void *hi, void *lo, int64_t n, void *stream) {
+    if (n < 0 || (n > 0 && (!x || !hi))) return TMQ_ERR_INVALID_ARG;
+    if (n == 0) return TMQ_OK;
+    const int64_t blocks = (n + 2047) / 2048;
+    if (blocks > 0x7FFFFFFF) return TMQ_ERR_TOO_LARGE;
+    const int vec = aligned16(x) && aligned16(hi) && aligned16(lo);
+    auto kernel = lo ? (prescale ? split_terms_kernel<true, true> : split_terms_kernel<true, false>)
+                     : (prescale ? split_terms_kernel<false, true> : split_terms_kernel<false, false>);
+    hipLaunchKernelGGL(kernel, dim3((uint32_t)blocks), dim3(256), 0, as_stream(stream), x, prescale,
+                       static_cast<_Float16 *>(hi), static_cast<_Float16 *>(lo), n, vec);
+    return check_launch();
+}
+
+int tmq_split_f32(const float *x, void *hi, void *lo, int64_t n, void *stream) {
+    if (n > 0 && !lo) return TMQ_ERR_INVALID_ARG;
+    return tmq_split_f32_scaled(x, nullptr, hi, lo, n, stream);
+}
+
+}  // extern "C"

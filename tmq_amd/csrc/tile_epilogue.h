@@ -130,7 +130,7 @@ __device__ __forceinline__ void write_tile(float *slab, const floatx4 (&acc)[WM]
                     }
                     if (ep.relu) {
 #pragma unroll
-                        for (int e = 0; e < 4; e++) v[e] = v[e] > 0.f ? v[e] : 0.f;
+                        for (int e = 0; e < 4; e++) v[e] = v[e] < 0.f ? 0.f : v[e];
                     }
                     __builtin_nontemporal_store(v, reinterpret_cast<floatx4 *>(static_cast<float *>(ep.y) + o));
                 }
@@ -141,11 +141,11 @@ __device__ __forceinline__ void write_tile(float *slab, const floatx4 (&acc)[WM]
                     float f = v[e];
                     if (ep.y_f16) {
                         if (ep.residual) f += (float)static_cast<const _Float16 *>(ep.residual)[o + e];
-                        if (ep.relu) f = f > 0.f ? f : 0.f;
+                        if (ep.relu) f = f < 0.f ? 0.f : f;
                         static_cast<_Float16 *>(ep.y)[o + e] = (_Float16)f;
                     } else {
                         if (ep.residual) f += static_cast<const float *>(ep.residual)[o + e];
-                        if (ep.relu) f = f > 0.f ? f : 0.f;
+                        if (ep.relu) f = f < 0.f ? 0.f : f;
                         static_cast<float *>(ep.y)[o + e] = f;
                     }
                 }

@@ -212,6 +212,38 @@ void check_mm_args(const torch::Tensor &lhs, const torch::Tensor &weights, int64
                 ": compact weight width does not match the number of columns");
 }
 
+// fp32 activations (the reference's convention). The kernels carry them as fp16 terms, so the tensor is first
+// scaled by the power of two that brings its largest value into fp16's range (tmq_f32_prescale; exact, undone
+// in the epilogue's per-channel scale): any magnitude works, as with the reference's fp32 arithmetic. Many
+// rows: the fp16 kernels over the two fp16 terms, y = W hi + W lo; few rows: the kernels that split on the fly.
+torch::Tensor linear_f32(const torch::Tensor &x, int64_t M, int64_t K, const torch::Tensor &native, int64_t columns,
+                         torch::Tensor &y, const char *name) {
+    const bool two_pass = tmq_fp32_rows_prefer_split(M, K, columns) != 0;
+    auto fopt = x.options().dtype(torch::kFloat32);
+    auto prescale = torch::empty({2}, fopt), scale = torch::empty({columns}, fopt);
+    torch::Tensor xs, workspace;
+    if (!two_pass) xs = torch::empty_like(x);
+    const size_t wsb = tmq_f32_prescale_workspace_bytes(x.numel());
+    if (wsb) workspace = torch::empty({(int64_t)wsb}, x.options().dtype(torch::kUInt8));
+    check(tmq_f32_prescale(x.data_ptr<float>(), x.numel(), prescale.data_ptr<float>(), two_pass ? nullptr : xs.data_ptr<float>(),
+                           nullptr, scale.data_ptr<float>(), columns, wsb ? workspace.data_ptr() : nullptr, stream_of(x)), name);
+    if (!two_pass) {
+        tmq_epilogue ep = {scale.data_ptr<float>(), nullptr, nullptr, 0, TMQ_F32};
+        check(tmq_ternary_linear(xs.data_ptr(), TMQ_F32, M, K, native.data_ptr(), columns, &ep, y.data_ptr(), stream_of(x)), name);
+        return y;
+    }
+    auto hi = torch::empty_like(x, x.options().dtype(torch::kFloat16));
+    auto lo = torch::empty_like(hi);
+    check(tmq_split_f32_scaled(x.data_ptr<float>(), prescale.data_ptr<float>(), hi.data_ptr(), lo.data_ptr(), x.numel(),
+                               stream_of(x)), name);
+    auto t = torch::empty_like(y);
+    tmq_epilogue ep1 = {scale.data_ptr<float>(), nullptr, nullptr, 0, TMQ_F32};
+    check(tmq_ternary_linear(hi.data_ptr(), TMQ_F16, M, K, native.data_ptr(), columns, &ep1, t.data_ptr(), stream_of(x)), name);
+    tmq_epilogue ep2 = {scale.data_ptr<float>(), nullptr, t.data_ptr(), 0, TMQ_F32};
+    check(tmq_ternary_linear(lo.data_ptr(), TMQ_F16, M, K, native.data_ptr(), columns, &ep2, y.data_ptr(), stream_of(x)), name);
+    return y;
+}
+
 torch::Tensor ternary_mmm_cuda(torch::Tensor lhs, torch::Tensor weights, int64_t columns) {   // tmq_cuda.cu:478-549
     check_mm_args(lhs, weights, columns, "ternary_mmm_cuda");
     TORCH_CHECK(lhs.dim() >= 1 && lhs.dim() <= 4, "ternary_mmm_cuda: expected 1 to 4 dimensions");
@@ -225,21 +257,10 @@ torch::Tensor ternary_mmm_cuda(torch::Tensor lhs, torch::Tensor weights, int64_t
     shape.back() = columns;
     auto y = torch::empty(shape, lhs.options().dtype(torch::kFloat32));
     const int64_t M = K ? x.numel() / K : 0;
-    if (x.scalar_type() == torch::kFloat32 && tmq_fp32_rows_prefer_split(M, K, columns)) {
-        // many fp32 rows: the fp16 kernels over the two fp16 terms of the activations, y = W hi + W lo
-        auto hi = torch::empty_like(x, x.options().dtype(torch::kFloat16));
-        auto lo = torch::empty_like(hi);
-        check(tmq_split_f32(x.data_ptr<float>(), hi.data_ptr(), lo.data_ptr(), x.numel(), stream_of(x)), "ternary_mmm_cuda");
-        auto t = torch::empty_like(y);
-        check(tmq_ternary_linear(hi.data_ptr(), TMQ_F16, M, K, native.data_ptr(), columns, nullptr, t.data_ptr(),
-                                 stream_of(x)), "ternary_mmm_cuda");
-        tmq_epilogue ep = {nullptr, nullptr, t.data_ptr(), 0, TMQ_F32};
-        check(tmq_ternary_linear(lo.data_ptr(), TMQ_F16, M, K, native.data_ptr(), columns, &ep, y.data_ptr(),
-                                 stream_of(x)), "ternary_mmm_cuda");
-        return y;
-    }
-    check(tmq_ternary_linear(x.data_ptr(), x.scalar_type() == torch::kFloat16 ? TMQ_F16 : TMQ_F32, M, K,
-                             native.data_ptr(), columns, nullptr, y.data_ptr(), stream_of(x)), "ternary_mmm_cuda");
+    if (M == 0) return y;
+    if (x.scalar_type() == torch::kFloat32) return linear_f32(x, M, K, native, columns, y, "ternary_mmm_cuda");
+    check(tmq_ternary_linear(x.data_ptr(), TMQ_F16, M, K, native.data_ptr(), columns, nullptr, y.data_ptr(), stream_of(x)),
+          "ternary_mmm_cuda");
     return y;
 }
 
@@ -254,8 +275,9 @@ torch::Tensor ternary_mvm_cuda(torch::Tensor vector, torch::Tensor weights, int6
     std::vector<int64_t> shape = vector.sizes().vec();
     shape.back() = columns;
     auto y = torch::empty(shape, vector.options().dtype(torch::kFloat32));
-    check(tmq_ternary_linear(x.data_ptr(), x.scalar_type() == torch::kFloat16 ? TMQ_F16 : TMQ_F32, 1, K,
-                             native.data_ptr(), columns, nullptr, y.data_ptr(), stream_of(x)), "ternary_mvm_cuda");
+    if (x.scalar_type() == torch::kFloat32) return linear_f32(x, 1, K, native, columns, y, "ternary_mvm_cuda");
+    check(tmq_ternary_linear(x.data_ptr(), TMQ_F16, 1, K, native.data_ptr(), columns, nullptr, y.data_ptr(), stream_of(x)),
+          "ternary_mvm_cuda");
     return y;
 }
 

@@ -457,7 +457,10 @@ def native_weights(words: torch.Tensor, columns: int, conv_kernel=None) -> Nativ
 
     The key is the storage address, shape and version counter of the compact tensor. The cache
     keeps a reference to that tensor, so its address cannot be handed to another tensor while the
-    entry lives; entries are evicted least-recently-used."""
+    entry lives; entries are evicted least-recently-used. Compact tensors are expected to be immutable:
+    a caller that passes `weight.data` (as the reference's layers do) hands over a tensor whose version
+    counter never moves, so words overwritten in place at the same address are not noticed --
+    clear_native_cache() after such a write."""
     key = (words.data_ptr(), tuple(words.shape), tuple(words.stride()), words._version, int(columns), conv_kernel,
            words.device.index)
     hit = _native_cache.pop(key, None)
@@ -467,6 +470,11 @@ def native_weights(words: torch.Tensor, columns: int, conv_kernel=None) -> Nativ
             _native_cache.pop(next(iter(_native_cache)))
     _native_cache[key] = hit
     return hit[0]
+
+
+def clear_native_cache():
+    """Forget every cached kernel-native weight buffer of the raw binding functions."""
+    _native_cache.clear()
 
 
 def _epilogue(nw, scale, bias, residual, relu, out_dtype, y):
@@ -489,16 +497,64 @@ def _epilogue(nw, scale, bias, residual, relu, out_dtype, y):
     return ep
 
 
-def split_f32(x: torch.Tensor):
-    """(hi, lo) with hi = fp16(x), lo = fp16(x - hi): fp32 activations as two fp16 terms."""
-    _capi.require_gpu(x, "activations")
+_fp32_prescale = True
+
+
+def set_fp32_prescale(flag: bool) -> bool:
+    """fp32 activations reach the fp16 MFMA kernels as fp16 terms. By default every fp32 tensor is first
+    scaled by the power of two that puts its largest value into fp16's comfortable range (one extra small
+    launch, exact, undone in the epilogue), so any magnitude works, as in the reference, which multiplies in
+    fp32. A caller who knows its activations are of order 1 (max|x| <= 65504, nothing of interest below ~1e-4)
+    can switch that off. Returns the previous setting."""
+    global _fp32_prescale
+    prev, _fp32_prescale = _fp32_prescale, bool(flag)
+    return prev
+
+
+def f32_prescale(x: torch.Tensor, scale=None, channels: int = 0, want_copy: bool = False):
+    """(prescale [2] = (s, 1 / s), s x or None, scale / s [channels] or None) for an fp32 GPU tensor: s is the
+    power of two that brings max|x| into [1024, 2048). x must be dense (any memory format)."""
+    _capi.require_gpu_dense(x, "activations")
+    if x.dtype != torch.float32:
+        raise RuntimeError("f32_prescale: expected fp32")
+    lib = _lib()
+    n = x.numel()
+    ps = torch.empty(2, dtype=torch.float32, device=x.device)
+    xs = torch.empty_like(x) if want_copy else None
+    adj = torch.empty(channels, dtype=torch.float32, device=x.device) if channels else None
+    if scale is not None and (scale.dtype != torch.float32 or scale.numel() != channels or not scale.is_cuda):
+        raise RuntimeError("scale must be fp32 with one entry per output channel")
+    wsb = lib.tmq_f32_prescale_workspace_bytes(n)
+    ws = torch.empty(wsb, dtype=torch.uint8, device=x.device) if wsb else None
+    with torch.cuda.device(x.device):
+        check(lib.tmq_f32_prescale(ptr(x), n, ptr(ps), ptr(xs), ptr(scale), ptr(adj), channels, ptr(ws), stream_of(x)),
+              "f32_prescale")
+    return ps, xs, adj
+
+
+def split_f32(x: torch.Tensor, prescale=None, want_lo: bool = True):
+    """(hi, lo) with hi = fp16(s x), lo = fp16(s x - hi): fp32 activations as two fp16 terms (s = prescale[0],
+    1 without). lo is None with want_lo=False. The terms keep x's shape and memory format."""
+    _capi.require_gpu_dense(x, "activations")
     if x.dtype != torch.float32:
         raise RuntimeError("split_f32: expected fp32")
-    x = x.contiguous()
-    hi, lo = torch.empty_like(x, dtype=torch.float16), torch.empty_like(x, dtype=torch.float16)
+    hi = torch.empty_like(x, dtype=torch.float16)
+    lo = torch.empty_like(x, dtype=torch.float16) if want_lo else None
     with torch.cuda.device(x.device):
-        check(_lib().tmq_split_f32(ptr(x), ptr(hi), ptr(lo), x.numel(), stream_of(x)), "split_f32")
+        check(_lib().tmq_split_f32_scaled(ptr(x), ptr(prescale), ptr(hi), ptr(lo), x.numel(), stream_of(x)), "split_f32")
     return hi, lo
+
+
+def f32_to_f16_prescaled(x: torch.Tensor, scale, channels: int):
+    """One fp16 term of an fp32 activation tensor for the convolution kernels: (fp16 tensor of x's shape and
+    memory format holding s x, scale / s) with the range prescale s, or (x.half(), scale) when the prescale
+    is switched off."""
+    if not _fp32_prescale:
+        return x.to(torch.float16), scale
+    if not (x.is_contiguous() or x.is_contiguous(memory_format=torch.channels_last)):
+        x = x.contiguous()
+    ps, _, adj = f32_prescale(x, scale, channels)
+    return split_f32(x, ps, want_lo=False)[0], adj
 
 
 def ternary_linear(x: torch.Tensor, nw: NativeWeights, scale=None, bias=None, residual=None, relu=False,
@@ -510,13 +566,22 @@ def ternary_linear(x: torch.Tensor, nw: NativeWeights, scale=None, bias=None, re
     if x.shape[-1] != nw.K:
         raise RuntimeError(f"ternary_linear: activations have {x.shape[-1]} features, weights expect {nw.K}")
     M = x.numel() // nw.K if nw.K else 0
-    if (x.dtype == torch.float32 and out_dtype == torch.float32 and (residual is None or residual.dtype == torch.float32)
-            and _lib().tmq_fp32_rows_prefer_split(M, nw.K, nw.N)):
-        # many fp32 rows (or a few over a very large layer): two passes of the fp16 kernels over the two
-        # fp16 terms of the activations beat the kernels that split them on the fly
-        hi, lo = split_f32(x)
-        t = ternary_linear(hi, nw, scale, bias, residual, False, torch.float32)
-        return ternary_linear(lo, nw, scale, None, t, relu, torch.float32)
+    if x.dtype == torch.float32 and M > 0:
+        two_pass = (out_dtype == torch.float32 and (residual is None or residual.dtype == torch.float32)
+                    and bool(_lib().tmq_fp32_rows_prefer_split(M, nw.K, nw.N)))
+        ps = None
+        if _fp32_prescale:
+            if scale is not None:
+                _capi.require_gpu(scale, "scale")
+            # any magnitude: the tensor times a power of two, undone in the per-channel scale
+            ps, xs, scale = f32_prescale(x, scale, nw.N, want_copy=not two_pass)
+            x = x if two_pass else xs
+        if two_pass:
+            # many fp32 rows (or a few over a very large layer): two passes of the fp16 kernels over the two
+            # fp16 terms of the activations beat the kernels that split them on the fly
+            hi, lo = split_f32(x, ps)
+            t = ternary_linear(hi, nw, scale, bias, residual, False, torch.float32)
+            return ternary_linear(lo, nw, scale, None, t, relu, torch.float32)
     y = torch.empty(x.shape[:-1] + (nw.N,), dtype=out_dtype, device=x.device)
     ep = _epilogue(nw, scale, bias, residual, relu, out_dtype, y)
     with torch.cuda.device(x.device):
@@ -538,6 +603,8 @@ def ternary_conv2d(x: torch.Tensor, nw: NativeWeights, stride=1, padding=0, dila
         raise RuntimeError("ternary_conv2d: expected a 4-D GPU tensor")
     if x.shape[1] != nw.C:
         raise RuntimeError(f"ternary_conv2d: input has {x.shape[1]} channels, weights expect {nw.C}")
+    if x.dtype == torch.float32:
+        x, scale = f32_to_f16_prescaled(x, scale, nw.N)
     if x.dtype != torch.float16 or not x.is_contiguous(memory_format=torch.channels_last):
         x = x.to(dtype=torch.float16, memory_format=torch.channels_last)
     B, C, H, W = x.shape
@@ -577,6 +644,8 @@ def ternary_dwconv2d(x: torch.Tensor, words: torch.Tensor, kernel, stride=1, pad
     _capi.require_gpu(words, "words")
     if words.dtype != torch.int32 or words.numel() != ky * kx * ((C + 15) // 16):
         raise RuntimeError("ternary_dwconv2d: expected the int32 compact words of a [C, 1, ky, kx] weight tensor")
+    if x.dtype == torch.float32:
+        x, scale = f32_to_f16_prescaled(x, scale, C)
     if x.dtype != torch.float16 or not x.is_contiguous(memory_format=torch.channels_last):
         x = x.to(dtype=torch.float16, memory_format=torch.channels_last)
     words = words.contiguous()
@@ -632,6 +701,8 @@ def ternary_dwconvtrans2d(x: torch.Tensor, words: torch.Tensor, kernel, stride=1
     _capi.require_gpu(words, "words")
     if words.dtype != torch.int32 or words.numel() != ky * kx * ((C + 15) // 16):
         raise RuntimeError("ternary_dwconvtrans2d: expected the int32 compact words of a [C, 1, ky, kx] weight tensor")
+    if x.dtype == torch.float32:
+        x, scale = f32_to_f16_prescaled(x, scale, C)
     if x.dtype != torch.float16 or not x.is_contiguous(memory_format=torch.channels_last):
         x = x.to(dtype=torch.float16, memory_format=torch.channels_last)
     words = words.contiguous()

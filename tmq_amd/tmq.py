@@ -541,11 +541,22 @@ class TMQLayer:
         y = ctrl._soft_weight_of(self)
         return y if y is not None else SoftStep.apply(self.weight, 1.0, ctrl)
 
+    def _weight_key(self, *extra):
+        """Identity of the compact weight tensor for the cache of its kernel-native form: storage address,
+        shape and the Parameter's version counter (weight.data has a counter of its own that never moves).
+        In-place writes that bypass autograd's bookkeeping (weight.data.copy_(...)) are not seen: call
+        invalidate_native() after them."""
+        w = self.weight
+        return (w.data_ptr(), tuple(w.shape), w._version) + extra
+
+    def invalidate_native(self):
+        """Drop the cached kernel-native form of the compact weights (rebuilt on the next forward)."""
+        self._native = None
+
     def _native_weights(self, conv_kernel=None):
-        w = self.weight.data
-        key = (w.data_ptr(), tuple(w.shape), w._version)
+        key = self._weight_key()
         if self._native is None or self._native[0] != key:
-            self._native = (key, ops.NativeWeights(w, self.original_shape[0], conv_kernel))
+            self._native = (key, ops.NativeWeights(self.weight.data, self.original_shape[0], conv_kernel))
         return self._native[1]
 
     def _epilogue_scale(self, n, device):
@@ -776,6 +787,8 @@ class Conv2d(nn.Module, TMQLayer):
             # pixels of the 4-channel NHWC image are read as one pixel of 8 channels, see _superpixel_plan
             nw, kxs, pl, pr = sp
             B, C, H, W = x.shape
+            if x.dtype == torch.float32:
+                x, scale = ops.f32_to_f16_prescaled(x, scale, int(self.original_shape[0]))
             xs = ops.nchw_to_nhwc4(x).view(B, H, W // 2, 8).permute(0, 3, 1, 2)
             (sy, _), (py, _) = _pair(self.stride), _pair(self.padding)
             return ops.ternary_conv2d(xs, nw, (sy, 1), ((py, py), (pl, pr)), 1, scale=scale, bias=bias,
@@ -807,7 +820,7 @@ class Conv2d(nn.Module, TMQLayer):
         if wo < 1 or pr < 0:
             return None
         w = self.weight.data
-        key = (w.data_ptr(), tuple(w.shape), w._version, "superpixel")
+        key = self._weight_key("superpixel")
         if self._native is None or self._native[0] != key:
             full = ops.expand_ternary(w, [N, C, ky, kx])
             wsp = torch.zeros((N, 8, ky, kxs), dtype=full.dtype, device=full.device)
@@ -899,7 +912,7 @@ class ConvTranspose2d(Conv2d):
                                              _pair(self.output_padding), _pair(self.dilation),
                                              scale=self._epilogue_scale(cin, x.device), bias=bias)
         w = self.weight.data
-        key = (w.data_ptr(), tuple(w.shape), w._version)
+        key = self._weight_key()
         if self._native is None or self._native[0] != key:
             full = ops.expand_ternary(w, [cin, cout, ky, kx])                     # [Cin, Cout, ky, kx]
             words = ops.compactify_ternary(full.reshape(cin, cout * ky * kx).t().contiguous())   # [Cin][ceil(N/16)]
@@ -1068,7 +1081,10 @@ def fold_batchnorm(module: nn.Module, pairs=None):
     that layer has outputs (the conv1 / bn1, Sequential(conv, bn) idiom) -- pass explicit pairs when
     registration order is not execution order. Returns the list of folded pairs."""
     def fits(layer, bn):
+        # a layer with a BatchNorm of its own (Linear.implicit_bn) applies it after the kernel's epilogue: an
+        # affine map folded into that epilogue would come before it instead of after
         return (isinstance(layer, (Linear, Conv2d)) and not isinstance(layer, ConvTranspose2d) and layer.compact and
+                getattr(layer, "bn", None) is None and
                 isinstance(bn, (nn.BatchNorm1d, nn.BatchNorm2d)) and bn.track_running_stats and
                 bn.num_features == int(layer.original_shape[0]))
 
