@@ -14,7 +14,7 @@ Prints ONE JSON line: metric soft-step fwd+bwd GB/s on the algorithmic 20 B/elem
 object (the op-for-op torch CPU restatement of the reference path, timed on this host's cores
 on a bounded sample).
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload all|softstep|linear|resnet_infer|resnet_qat]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload all|softstep|linear|pack|resnet_infer|resnet_qat]
 """
 import argparse
 import json
@@ -351,6 +351,47 @@ def _gemv_floor_and_large(args, torch, natives):
     return res
 
 
+def bench_pack(args, torch):
+    """2-bit pack / unpack of a 4096 x 4096 fp32 weight matrix (the layer of BASELINE configs[2]): 4.25 B per
+    weight (4 on the fp32 side, 1/4 on the packed side). Rotates over distinct fp32 buffers (> 256 MB in total)
+    so that nothing comes from L2 / Infinity Cache; HIP-graph replays, events on the launch stream."""
+    from tmq_amd import _capi
+    lib = _capi.load()
+    dev = torch.device("cuda:0")
+    N = K = 4096
+    nb = 7
+    Ws = [torch.randint(-1, 2, (N, K), device=dev).float() for _ in range(nb)]
+    outs = [torch.empty((K, N // 16), dtype=torch.int32, device=dev) for _ in range(nb)]
+    if args.copy_calibration:
+        Ws[1].copy_(Ws[0])          # a copy of known size (64 MiB read + 64 MiB written) for scaling the traffic counters
+
+    def pack():
+        s = _capi.stream_of(Ws[0])
+        for w, o in zip(Ws, outs):
+            _capi.check(lib.tmq_pack_ternary(_capi.ptr(w), _capi.F32, N, K, _capi.ptr(o), s), "pack")
+        return nb
+
+    def unpack():
+        s = _capi.stream_of(Ws[0])
+        for w, o in zip(Ws, outs):
+            _capi.check(lib.tmq_unpack_ternary(_capi.ptr(o), N, K, _capi.ptr(w), s), "unpack")
+        return nb
+    pack()
+    torch.cuda.synchronize()
+    byts = N * K * 4.25
+    res = {"metric": "2-bit pack / unpack GB/s", "unit": "GB/s", "n_gpus": 1, "dtype": "u32", "data": "synthetic",
+           "config": {"workload": "pack / unpack of a 4096 x 4096 fp32 matrix, %d rotating buffers" % nb}}
+    for name, fn in (("pack", pack), ("unpack", unpack)):
+        us = _graph_time_us(torch, fn, max(3, args.steps // nb), args.settle_ms)
+        res[name] = {"us": round(us, 3), "gbs": round(byts / us / 1e3, 1)}
+        res["roofline" if name == "pack" else "roofline_unpack"] = {
+            "bound": "hbm", "achieved": round(byts / us / 1e3, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": round(byts / us / 1e3 / HBM_PEAK_GBS, 4), "traffic": None, "algorithmic_bytes": int(byts),
+            "kernel": ("pack_wide_kernel<float, 4>" if name == "pack" else "unpack_wide_kernel<8>"), "avg_launch_us": round(us, 3)}
+    res["value"] = res["pack"]["gbs"]
+    return res
+
+
 def bench_resnet_infer(args, torch):
     """BASELINE configs[3]: ResNet-18 (102 classes) ternary inference, batch 64 of 3x224x224 fp16."""
     import tmq_amd as t
@@ -574,6 +615,8 @@ def main():
         res = bench_softstep(args, torch)
     elif args.workload == "linear":
         res = bench_linear(args, torch)
+    elif args.workload == "pack":
+        res = bench_pack(args, torch)
     elif args.workload == "resnet_infer":
         res = bench_resnet_infer(args, torch)
     elif args.workload == "resnet_qat":

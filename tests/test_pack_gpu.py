@@ -5,7 +5,8 @@ import torch
 
 pytestmark = pytest.mark.gpu
 
-SHAPES_2D = [(1, 1), (16, 1), (17, 3), (6, 5), (102, 512), (64, 147), (256, 64), (4096, 256), (300, 1000), (33, 65)]
+SHAPES_2D = [(1, 1), (16, 1), (17, 3), (6, 5), (102, 512), (64, 147), (256, 64), (4096, 256), (300, 1000), (33, 65),
+             (64, 4608), (520, 260), (48, 1024), (1, 256), (4100, 300), (130, 2052)]   # K >= 256, K % 4 == 0: the 256-k tiles
 SHAPES_4D = [(64, 3, 7, 7), (128, 64, 3, 3), (102, 16, 1, 1), (20, 5, 3, 2)]
 
 
@@ -52,11 +53,12 @@ def test_rounding_and_clamping_of_float_input(cuda, oracle):
     from tmq_amd import ops
     v = np.array([0.5, -0.5, 0.49999997, -0.49999997, 1.5, -1.5, 2.5, -2.5, 0.0, -0.0, 1e-30, 7.0, -7.0, 3e9, -3e9,
                   np.inf, -np.inf, np.nan, 2147483520.0, 2147483648.0, 0.50000006, 1e38], dtype=np.float32)
-    w = np.zeros((32, 3), dtype=np.float32)
-    w[:v.size, 1] = v
-    want = oracle.pack(w)
-    got = ops.compactify_ternary(torch.from_numpy(w).to(cuda)).cpu().numpy().view(np.uint32)
-    assert np.array_equal(got, want)
+    for K, col in ((3, 1), (256, 77), (516, 515)):            # the scalar tiles and the 256-k tiles
+        w = np.zeros((32, K), dtype=np.float32)
+        w[:v.size, col] = v
+        want = oracle.pack(w)
+        got = ops.compactify_ternary(torch.from_numpy(w).to(cuda)).cpu().numpy().view(np.uint32)
+        assert np.array_equal(got, want), K
     iv = np.array([0, 1, -1, 2, -2, 127, -128, 5, -5], dtype=np.int8)
     wi = np.zeros((16, 2), dtype=np.int8); wi[:iv.size, 0] = iv
     assert np.array_equal(ops.compactify_ternary(torch.from_numpy(wi).to(cuda)).cpu().numpy().view(np.uint32),
