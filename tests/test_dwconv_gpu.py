@@ -87,11 +87,17 @@ def test_depthwise_layer_compact_inference(cuda):
     assert torch.allclose(got, want, rtol=1e-3, atol=1e-3)
 
 
-@pytest.mark.parametrize("cin,cout,k,stride,pad,opad,dil", [(16, 8, 3, 2, 1, 1, 1), (24, 40, 2, 2, 0, 0, 1),
-                                                            (8, 8, 3, 1, 1, 0, 1), (32, 5, (3, 2), (2, 1), (1, 0), 0, 1)])
+@pytest.mark.parametrize("cin,cout,k,stride,pad,opad,dil", [
+    (16, 8, 3, 2, 1, 1, 1), (24, 40, 2, 2, 0, 0, 1), (8, 8, 3, 1, 1, 0, 1), (32, 5, (3, 2), (2, 1), (1, 0), 0, 1),
+    (16, 16, 4, 2, 1, 0, 1),            # the usual decoder layer: four phases of 2 x 2 taps
+    (8, 8, 2, 3, 0, 1, 1),              # kernel smaller than the stride: phases without any tap (bias only)
+    (8, 4, 3, 2, 2, 1, 1),              # padding as large as the kernel reaches
+    (4, 6, 3, 2, 1, 0, 2),              # dilation 2 at stride 2: every tap lands in the even phase
+    (8, 8, 5, 3, 2, 2, 1), (8, 8, 3, 1, 3, 0, 1),   # stride 3; padding beyond the kernel (results to skip)
+    (64, 24, (3, 5), (2, 3), (1, 2), (1, 2), (1, 2)), (5, 7, 4, 4, 0, 3, 1)])
 def test_transposed_layer_compact_inference(cuda, cin, cout, k, stride, pad, opad, dil):
-    """ConvTranspose2d: the compact forward (GEMM on re-packed weights + fold) must equal the float
-    forward on the ternarised weights; small integers make that exact."""
+    """ConvTranspose2d: the compact forward (one stride-1 implicit-GEMM convolution per phase of the output
+    grid) must equal the float forward on the ternarised weights; small integers make that exact."""
     import tmq_amd as t
     torch.manual_seed(cin + cout)
     net = torch.nn.Sequential(torch.nn.ConvTranspose2d(cin, cout, k, stride, pad, output_padding=opad, bias=True, dilation=dil))

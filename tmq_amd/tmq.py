@@ -708,6 +708,27 @@ def _pair(v):
     return tuple(v) if isinstance(v, (tuple, list)) else (v, v)
 
 
+def _phase_extent(r, s, p, n_out, n_in, geo):
+    """One axis of one phase of a transposed convolution (ConvTranspose2d._phase_weights): the output
+    positions o = s q + r - p inside [0, n_out) and the stride-1 convolution over the n_in input positions that
+    computes them. geo = (taps, largest e, step of e). Returns (first output position, count, padding before,
+    padding after, leading results to skip) or None when the phase has no output position."""
+    taps, e_max, step = geo
+    q_min = -((r - p) // s)                       # ceil((p - r) / s)
+    q_max = (n_out - 1 + p - r) // s
+    if q_max < q_min:
+        return None
+    count = q_max - q_min + 1
+    first = s * q_min + r - p
+    if taps == 0:
+        return first, count, 0, 0, 0
+    # result u of the convolution reads x[u - before + t step]; it stands for q = u + q_start with before = e_max - q_start
+    q_start = min(q_min, e_max)                   # no negative padding: start earlier and skip
+    before, skip = e_max - q_start, q_min - q_start
+    after = max(0, (skip + count) - n_in - before + step * (taps - 1))
+    return first, count, before, after, skip
+
+
 class Conv2d(nn.Module, TMQLayer):
     """Quantization-aware drop-in for nn.Conv2d (tmq/tmq.py:769-973)."""
 
@@ -890,11 +911,13 @@ class ConvTranspose2d(Conv2d):
 
     @torch.no_grad()
     def compact_forward(self, x):
-        """Transposed convolution from the packed weights as GEMM + col2im: cols[b, (co, i, j), p] =
-        sum_ci x[b, ci, p] W[ci, co, i, j], then F.fold scatters the columns (the plan of
-        tmq/tmq.py:1005-1038, whose own shape checks reject its weight view). The compact tensor of a
-        [Cin, Cout, ky, kx] kernel packs along Cin, the reduction index here, so it is unpacked and
-        re-packed along (co, i, j) once per layer. groups == channels takes the depthwise kernel instead."""
+        """Transposed convolution from the packed weights, gathered: every phase of the output grid is an
+        ordinary stride-1 ternary implicit-GEMM convolution with the sub-kernel of the taps that reach it
+        (_phase_weights), written into its strided share of the output. No columns and no F.fold, the useful
+        multiply-adds only (the reference's plan, tmq/tmq.py:1005-1038, is GEMM + F.fold over columns ky kx /
+        (sy sx) times the size of the output, and its own shape checks reject its weight view). The compact
+        tensor of a [Cin, Cout, ky, kx] kernel packs along Cin, the reduction index here, so the sub-kernels
+        are unpacked and re-packed along Cout once per layer. groups == channels takes the depthwise kernel."""
         assert not self.training, "Compact inference is not supported in training mode"
         assert self.weight.data.dtype == torch.int32, "Compact inference requires 32-bit integer words"
         self._update_scale()
@@ -911,13 +934,6 @@ class ConvTranspose2d(Conv2d):
             return ops.ternary_dwconvtrans2d(x, self.weight.data, (ky, kx), _pair(self.stride), _pair(self.padding),
                                              _pair(self.output_padding), _pair(self.dilation),
                                              scale=self._epilogue_scale(cin, x.device), bias=bias)
-        w = self.weight.data
-        key = self._weight_key()
-        if self._native is None or self._native[0] != key:
-            full = ops.expand_ternary(w, [cin, cout, ky, kx])                     # [Cin, Cout, ky, kx]
-            words = ops.compactify_ternary(full.reshape(cin, cout * ky * kx).t().contiguous())   # [Cin][ceil(N/16)]
-            self._native = (key, ops.NativeWeights(words, cout * ky * kx))
-        nw = self._native[1]
         B, C, H, W = x.shape
         sy, sx = _pair(self.stride)
         py, px = _pair(self.padding)
@@ -925,13 +941,63 @@ class ConvTranspose2d(Conv2d):
         dy, dx = _pair(self.dilation)
         h_out = (H - 1) * sy - 2 * py + dy * (ky - 1) + 1 + oy
         w_out = (W - 1) * sx - 2 * px + dx * (kx - 1) + 1 + ox
-        lhs = x.permute(0, 2, 3, 1).reshape(B * H * W, C)
-        cols = ops.ternary_linear(lhs.contiguous(), nw, scale=self._epilogue_scale(nw.N, x.device))
-        final = nn.functional.fold(cols.view(B, H * W, nw.N).permute(0, 2, 1), output_size=(h_out, w_out),
-                                   kernel_size=(ky, kx), dilation=(dy, dx), stride=(sy, sx), padding=(py, px))
-        if self.bias is not None:
-            final = final + self.bias.view(1, -1, 1, 1)
-        return final
+        if C != cin or h_out <= 0 or w_out <= 0:
+            raise RuntimeError("ConvTranspose2d.compact_forward: input does not match the layer")
+        phases = self._phase_weights(cin, cout, ky, kx, sy, sx, dy, dx)
+        scale = self._epilogue_scale(cout, x.device)
+        bias = self.bias.data.float() if self.bias is not None else None
+        if x.dtype == torch.float32:
+            x, scale = ops.f32_to_f16_prescaled(x, scale, cout)     # once for all phases
+        y = torch.empty((B, cout, h_out, w_out), dtype=_compact_out, device=x.device, memory_format=torch.channels_last)
+        for (rh, rw), (nw, geo_h, geo_w) in phases.items():
+            rows, cols = _phase_extent(rh, sy, py, h_out, H, geo_h), _phase_extent(rw, sx, px, w_out, W, geo_w)
+            if rows is None or cols is None:
+                continue                                             # no output position in this phase
+            (o0, cnt_h, pt, pb, skip_h), (p0, cnt_w, pl, pr, skip_w) = rows, cols
+            target = y[:, :, o0::sy, p0::sx]
+            if nw is None:                                           # no tap reaches this phase: bias only
+                target.zero_()
+                if bias is not None:
+                    target += bias.to(y.dtype).view(1, -1, 1, 1)
+                continue
+            part = ops.ternary_conv2d(x, nw, (1, 1), ((pt, pb), (pl, pr)), (geo_h[2], geo_w[2]), scale=scale, bias=bias,
+                                      out_dtype=_compact_out)
+            target.copy_(part[:, :, skip_h:skip_h + cnt_h, skip_w:skip_w + cnt_w])
+        return y
+
+    def _phase_weights(self, cin, cout, ky, kx, sy, sx, dy, dx):
+        """The transposed convolution as sy * sx ordinary stride-1 convolutions, one per phase
+        (r_h, r_w) = ((oh + py) mod sy, (ow + px) mod sx) of the output grid: an output row oh = sy q + r - py is
+        reached from input row ih = q - e by exactly the taps i with i dy = r (mod sy), e = (i dy - r) / sy. In
+        terms of q that is a convolution of x with those taps in reverse order, dilation (step of e), left padding
+        (largest e). Returns {(r_h, r_w): (native weights of the sub-kernel or None when it is empty,
+        (taps, largest e, step of e) along h, the same along w)}; cached with the weights."""
+        key = self._weight_key("phases", sy, sx, dy, dx)
+        if self._native is not None and self._native[0] == key:
+            return self._native[1]
+        full = ops.expand_ternary(self.weight.data, [cin, cout, ky, kx])          # [Cin, Cout, ky, kx]
+
+        def taps(k, s, d, r):
+            idx = [i for i in range(k) if (i * d - r) % s == 0 and i * d >= r]
+            if not idx:
+                return idx, 0, 1
+            e = [(i * d - r) // s for i in idx]
+            step = e[1] - e[0] if len(e) > 1 else 1
+            assert all(b - a == step for a, b in zip(e, e[1:]))
+            return idx, e[-1], step
+
+        phases = {}
+        for rh in range(sy):
+            ih, eh, dh = taps(ky, sy, dy, rh)
+            for rw in range(sx):
+                iw, ew, dw = taps(kx, sx, dx, rw)
+                nw = None
+                if ih and iw:
+                    sub = full[:, :, ih][:, :, :, iw].flip(2, 3).permute(1, 0, 2, 3).contiguous()   # [Cout, Cin, Th, Tw]
+                    nw = ops.NativeWeights(ops.compactify_ternary(sub), cout, (len(ih), len(iw)))
+                phases[(rh, rw)] = (nw, (len(ih), eh, dh), (len(iw), ew, dw))
+        self._native = (key, phases)
+        return phases
 
     @classmethod
     def from_transconv2d(cls, source: nn.ConvTranspose2d, name: str, ctrl: QuantizationControl):
