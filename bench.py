@@ -233,14 +233,14 @@ def bench_linear(args, torch):
         res["roofline_gemv"] = {"bound": "hbm", "achieved": o["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                                 "frac": o["frac_hbm"], "traffic": None,
                                 "algorithmic_bytes": int(K * N / 4 + 2 * K + 8 * N),
-                                "kernel": "weight-stream GEMV (M = 1), %d rotating weight buffers" % nrot,
+                                "kernel": "gemv8_kernel (M = 1, fp8 x bf8 MFMA), %d rotating weight buffers" % nrot,
                                 "avg_launch_us": o["us"]}
     if "gemv_16384" in extra:
         o = extra["gemv_16384"]
         res["roofline_gemv_16384"] = {"bound": "hbm", "achieved": o["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                                       "frac": o["frac_hbm"], "traffic": None,
                                       "algorithmic_bytes": int(16384 * 16384 / 4 + 2 * 16384 + 8 * 16384),
-                                      "kernel": "weight-stream GEMV (M = 1, K = N = 16384), 6 rotating weight buffers",
+                                      "kernel": "gemv8_kernel (M = 1, K = N = 16384, fp8 x bf8 MFMA), 6 rotating weight buffers",
                                       "avg_launch_us": o["us"]}
     if not args.no_cpu:
         res["cpu_baseline"] = cpu_baseline_linear(torch, W, scale.cpu())

@@ -253,6 +253,11 @@ typedef struct tmq_epilogue {
  * magnitude go through tmq_f32_prescale first (exact power-of-two scaling, undone in the per-channel scale of
  * the epilogue); the Python / PyTorch bindings of this library always do, because the reference multiplies
  * fp32 activations in fp32 and has no such limit.
+ * Arithmetic: exact products, fp32 accumulation. One fp16 row (M == 1) with K a multiple of 2048 up to 16384
+ * runs on the 8-bit matrix instructions (weights as fp8, the row as four exact bf8 terms); there the hardware adds
+ * 32 products at a time aligned to the largest of them, so the result can differ from an fp32 running sum by a few
+ * 1e-6 of the largest output (about 1e-4 when values near 65504 sit next to values of order one) -- inside the
+ * 1e-3 tolerance of this path, and exact whenever all partial sums are integers below 2^24.
  * Replaces ternary_mvm_cuda (tmq/tmq_cuda.cu:563-603, kernel 242-286) for M == 1 and
  * ternary_mmm_cuda (tmq/tmq_cuda.cu:478-549, kernel 289-427) for M > 1, plus the post-scale /
  * bias passes of Linear.compact_forward (tmq/tmq.py:684-687). Any M, K, N (ragged tails masked). */

@@ -1,0 +1,166 @@
+"""One fp16 activation row with K a multiple of 2048 (up to 16384) runs on the 8-bit matrix instructions:
+weights as fp8 +-2, the activation vector as four exact bf8 terms. Checked against an fp64 product of the
+expanded weights (not the library), through every epilogue, ragged N, every K the kernel takes, and on the
+inputs where its one numerical difference from an fp32 sum (the instruction's internal alignment window over
+32 products) would show. On normally distributed activations that difference is a few 1e-6 of the largest output
+(the fp16 kernels: below 1e-6); the bar for this path is 1e-3.
+"""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _ternary(rng, N, K, p0=0.5):
+    u = rng.random((N, K))
+    return np.where(u < (1 - p0) / 2, 1.0, np.where(u < 1 - p0, -1.0, 0.0)).astype(np.float32)
+
+
+def _rel_err(got, want):
+    want = np.asarray(want, np.float64)
+    got = np.asarray(got, np.float64)
+    return np.max(np.abs(got - want)) / max(1e-30, np.max(np.abs(want)))
+
+
+def _layer(cuda, oracle, rng, N, K, p0=0.5):
+    from tmq_amd import ops
+    W = _ternary(rng, N, K, p0)
+    words = oracle.pack(W)
+    return W, ops.NativeWeights(torch.from_numpy(words.view(np.int32)).to(cuda), N)
+
+
+@pytest.mark.parametrize("K", [2048 * i for i in range(1, 9)])
+@pytest.mark.parametrize("N", [16, 1000, 4100])
+def test_every_reduction_length_and_ragged_channels(cuda, oracle, K, N):
+    from tmq_amd import ops
+    rng = np.random.default_rng(K + N)
+    W, nw = _layer(cuda, oracle, rng, N, K)
+    x = rng.standard_normal((1, K)).astype(np.float16)
+    y = ops.ternary_linear(torch.from_numpy(x).to(cuda), nw)
+    ref = x.astype(np.float64) @ W.astype(np.float64).T
+    assert y.shape == (1, N) and y.dtype == torch.float32
+    assert _rel_err(y.cpu().numpy(), ref) <= 1e-5
+    assert torch.equal(ops.ternary_linear(torch.from_numpy(x).to(cuda), nw), y)   # run to run identical
+    # the reference's binding name on the compact words, a one-dimensional vector
+    words = torch.from_numpy(oracle.pack(W).view(np.int32)).to(cuda)
+    v = ops.ternary_mvm_cuda(torch.from_numpy(x[0]).to(cuda), words, N)
+    assert torch.equal(v.reshape(1, N), y)
+
+
+@pytest.mark.parametrize("y16", [False, True])
+def test_epilogues(cuda, oracle, y16):
+    from tmq_amd import ops
+    K, N = 4096, 1000
+    rng = np.random.default_rng(77)
+    W, nw = _layer(cuda, oracle, rng, N, K)
+    x = rng.standard_normal((1, K)).astype(np.float16)
+    scale = (0.01 + 0.02 * rng.random(N)).astype(np.float32)
+    bias = rng.standard_normal(N).astype(np.float32)
+    res = rng.standard_normal((1, N)).astype(np.float16 if y16 else np.float32)
+    acc = x.astype(np.float64) @ W.astype(np.float64).T
+    t = lambda a: torch.from_numpy(a).to(cuda)
+    odt = torch.float16 if y16 else torch.float32
+    tol = 1e-3 if y16 else 1e-5
+    y = ops.ternary_linear(t(x), nw, t(scale), t(bias), out_dtype=odt)
+    assert y.dtype == odt
+    assert _rel_err(y.float().cpu().numpy(), acc * scale + bias) <= tol
+    y = ops.ternary_linear(t(x), nw, t(scale), None, residual=t(res), relu=True, out_dtype=odt)
+    assert _rel_err(y.float().cpu().numpy(), np.maximum(acc * scale + res.astype(np.float64), 0)) <= tol
+    y = ops.ternary_linear(t(x), nw, None, t(bias), relu=True, out_dtype=odt)
+    assert _rel_err(y.float().cpu().numpy(), np.maximum(acc + bias, 0)) <= tol
+    assert (y >= 0).all()
+
+
+def test_exact_on_integers_and_on_every_fp16_mantissa(cuda, oracle):
+    """Small integers: every product and every partial sum is an integer below 2^24, so the result is exact
+    whatever the order. All 11 significant bits of the fp16 values must survive the four-term split: values
+    (1024 + m) for every m reach the last bit."""
+    from tmq_amd import ops
+    K, N = 2048, 256
+    rng = np.random.default_rng(3)
+    W, nw = _layer(cuda, oracle, rng, N, K)
+    x = rng.integers(-8, 9, size=(1, K)).astype(np.float16)
+    y = ops.ternary_linear(torch.from_numpy(x).to(cuda), nw)
+    assert np.array_equal(y.cpu().numpy().astype(np.float64), x.astype(np.float64) @ W.astype(np.float64).T)
+    m = (1024 + (np.arange(K) % 1024)).astype(np.float16) * np.where(rng.random(K) < .5, -1, 1).astype(np.float16)
+    y = ops.ternary_linear(torch.from_numpy(m[None]).to(cuda), nw)
+    assert np.array_equal(y.cpu().numpy().astype(np.float64), m[None].astype(np.float64) @ W.astype(np.float64).T)
+    # subnormal fp16 values: integers times 2^-24, so again exact whatever the order
+    tiny = (rng.integers(-1023, 1024, size=(1, K)).astype(np.float64) * 2.0 ** -24).astype(np.float16)
+    y = ops.ternary_linear(torch.from_numpy(tiny).to(cuda), nw)
+    assert np.array_equal(y.cpu().numpy().astype(np.float64), tiny.astype(np.float64) @ W.astype(np.float64).T)
+    # a layer whose activations are all of order 1e-3
+    small = (rng.standard_normal((1, K)) * 1e-3).astype(np.float16)
+    y = ops.ternary_linear(torch.from_numpy(small).to(cuda), nw)
+    assert _rel_err(y.cpu().numpy(), small.astype(np.float64) @ W.astype(np.float64).T) <= 1e-5
+
+
+def test_single_weight_selects_each_position(cuda, oracle):
+    """A weight matrix with one nonzero per channel picks single activations: catches any mismatch between the
+    byte order of the activation planes and the weight registers (a permuted k within a block)."""
+    from tmq_amd import ops
+    K, N = 2048, 2048
+    W = np.zeros((N, K), np.float32)
+    rng = np.random.default_rng(4)
+    sign = np.where(rng.random(N) < .5, -1.0, 1.0).astype(np.float32)
+    W[np.arange(N), np.arange(N)] = sign
+    nw = ops.NativeWeights(torch.from_numpy(oracle.pack(W).view(np.int32)).to(cuda), N)
+    x = rng.standard_normal((1, K)).astype(np.float16)
+    y = ops.ternary_linear(torch.from_numpy(x).to(cuda), nw)
+    assert np.array_equal(y.cpu().numpy()[0], x[0].astype(np.float32) * sign)
+
+
+def test_every_finite_fp16_value_passes_through_exactly(cuda, oracle):
+    """The activation vector reaches the 8-bit instruction as four scaled bf8 terms. With the identity as weights
+    the output must be the input, bit for bit, for each of the 63488 finite fp16 values (subnormals included)."""
+    from tmq_amd import ops
+    K = N = 4096
+    nw = ops.NativeWeights(torch.from_numpy(oracle.pack(np.eye(N, dtype=np.float32)).view(np.int32)).to(cuda), N)
+    bits = np.arange(65536, dtype=np.uint32).astype(np.uint16)
+    vals = bits.view(np.float16).copy()
+    vals[~np.isfinite(vals)] = 0
+    perm = np.random.default_rng(8).permutation(65536)          # neighbours of unrelated magnitude
+    vals = vals[perm]
+    for c in range(65536 // K):
+        x = vals[c * K:(c + 1) * K][None]
+        y = ops.ternary_linear(torch.from_numpy(x).to(cuda), nw).cpu().numpy()
+        assert np.array_equal(y, x.astype(np.float32)), c                  # by value: -0 comes back as +0
+
+
+def test_wide_dynamic_range_within_the_stated_tolerance(cuda, oracle):
+    """The 8-bit instruction aligns its 32 products to the largest before adding: next to 65504, values of order
+    one lose their low bits. The loss is bounded by ~2^-17 of the largest product per instruction -- far inside
+    the 1e-3 bar, and asserted here at 2e-4 of the largest output."""
+    from tmq_amd import ops
+    K, N = 4096, 512
+    rng = np.random.default_rng(5)
+    W, nw = _layer(cuda, oracle, rng, N, K)
+    x = rng.standard_normal((1, K)).astype(np.float16)
+    x[0, ::32] = np.float16(65504.0) * np.where(rng.random(K // 32) < .5, -1, 1)
+    x[0, 1::32] = (rng.standard_normal(K // 32) * 1e-4).astype(np.float16)
+    y = ops.ternary_linear(torch.from_numpy(x).to(cuda), nw)
+    ref = x.astype(np.float64) @ W.astype(np.float64).T
+    assert _rel_err(y.cpu().numpy(), ref) <= 2e-4
+    # ten orders of magnitude apart, elementwise random
+    x = (rng.standard_normal((1, K)) * 10.0 ** rng.integers(-6, 4, size=(1, K))).astype(np.float16)
+    y = ops.ternary_linear(torch.from_numpy(x).to(cuda), nw)
+    assert _rel_err(y.cpu().numpy(), x.astype(np.float64) @ W.astype(np.float64).T) <= 2e-4
+
+
+def test_agrees_with_the_fp16_kernels_on_neighbouring_shapes(cuda, oracle):
+    """M = 2 (fp16 weight-stream kernel) on two copies of the row, and an unaligned view of the row (skinny
+    kernel), give the same numbers to fp32 rounding."""
+    from tmq_amd import ops
+    K, N = 8192, 1024
+    rng = np.random.default_rng(6)
+    W, nw = _layer(cuda, oracle, rng, N, K)
+    buf = torch.from_numpy(rng.standard_normal(K + 8).astype(np.float16)).to(cuda)
+    x = buf[:K].clone()[None]
+    y1 = ops.ternary_linear(x, nw)
+    y2 = ops.ternary_linear(torch.cat([x, x]), nw)
+    assert torch.equal(y2[0], y2[1])
+    assert _rel_err(y1.cpu().numpy(), y2[:1].cpu().numpy()) <= 1e-5
+    buf[1:K + 1] = x[0]
+    y3 = ops.ternary_linear(buf[1:K + 1][None], nw)                     # 2-byte aligned: not the 8-bit kernel
+    assert _rel_err(y1.cpu().numpy(), y3.cpu().numpy()) <= 1e-5

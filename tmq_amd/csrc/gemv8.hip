@@ -1,0 +1,242 @@
+// M = 1 on the 8-bit matrix instructions: v_mfma_f32_16x16x32_fp8_bf8.
+//
+// The fp16 MFMA kernels expand every 2-bit code into an fp16 operand, one VALU lane-operation per weight,
+// and for a single activation row that expansion, not memory, is what a launch waits for. The fp8 operand
+// format takes four weights per register: the native layout's (sign, nonzero) pairs sit two bits apart, so
+// `(word << 2 f) & 0xC0C0C0C0` puts the pairs of four weights into the top two bits of the four bytes, which
+// read as e4m3 are +-2.0 or 0 -- half the VALU work per weight. The activation vector has to become 8-bit as
+// well, exactly: an fp16 value is a sum of four scaled bf8 (e5m2) terms, because the top byte of an fp16 number
+// IS a bf8 number (same sign and exponent, the two leading mantissa bits): take the top byte, subtract it
+// (exact), rescale the remainder, repeat -- three significant bits per term (bf8_terms below). The four term
+// vectors ride in rows 0..3 of the MFMA's sixteen activation columns, which a single row leaves unused anyway,
+// so the instruction count does not grow; the four result columns are added, with their scales, at the end. Products are exact
+// and the accumulation is fp32, as in the fp16 kernels. One difference remains: the hardware adds the 32
+// products of one instruction in a fixed-point window below the largest of them (measured: ~2^-17 of it), so a
+// vector whose neighbouring elements differ by more than five orders of magnitude loses the small ones'
+// contribution earlier than an fp32 sum would (1e-4 of the largest output in a constructed case with 65504
+// next to values of order one; 1.4e-6 on normally distributed data; exact on small integers).
+//
+// Structure: a workgroup of WAVES wavefronts owns CB blocks of 16 channels; KS = WAVES / CB wavefronts share a
+// channel block, wavefront ks taking the weight blocks ks, ks + KS, ... (NT of them, all in flight at once as
+// 16-byte-per-lane loads issued in the order they are used). The workgroup first turns the activation vector
+// into the four term planes in LDS, in the byte order the weight registers imply (a thread per 8 values: two
+// 8-byte loads, 28 operations for the terms, 8 byte permutes, four 8-byte LDS writes), while its weight loads
+// are on their way; then every MFMA takes its activation operand with one 8-byte LDS read. Sums of the KS
+// wavefronts meet in LDS in wavefront order (deterministic). Measured (HIP-graph replays over rotating weight
+// buffers): K = N = 4096 3.0 us (fp16 weight-stream kernel 3.75), 8192^2 5.5 us, 16384^2 15.6 us (17.7).
+//
+// Requires fp16 activations, M == 1, K a multiple of 2048 and at most 16384, 16-byte aligned x.
+#include "common.h"
+#include "mfma.h"
+
+#include <type_traits>
+
+namespace tmq {
+namespace {
+
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+
+// Four bf8 terms of the two fp16 values packed in one register: t[i] carries term i of both values in the high
+// byte of each half-word, and x = t0 + t1 / 4 + t2 / 32 + t3 / 256 exactly, for every finite fp16 x.
+//   t0 = the top byte of x (its three leading significant bits, truncated);
+//   r1 = 4 (x - t0), below |x| in magnitude;         t1 = r1 rounded to three significant bits;
+//   r2 = 8 (r1 - t1), at most |r1| (half an ulp x 8); t2 = r2 rounded;     r3 = 8 (r2 - t2);     t3 = r3, exact.
+// Rounding is an integer add on the bit patterns (half of the kept unit, then the mask): it carries into the
+// exponent correctly and treats subnormals like normals. The rescaling is what keeps small values exact: without
+// it a remainder below 2^-14 would be subnormal in its own right and lose everything under 2^-16 to the mask;
+// with it the four terms resolve 2^-16, 2^-18, 2^-21 and 2^-24, the smallest fp16 subnormal. Every difference
+// and product is exact in fp16 (each term holds leading bits of its remainder; the factors are powers of two and
+// nothing grows past |x|).
+__device__ __forceinline__ void bf8_terms(uint32_t x2, uint32_t (&t)[4]) {
+    const half2_t four = {(_Float16)4.0f, (_Float16)4.0f}, eight = {(_Float16)8.0f, (_Float16)8.0f};
+    t[0] = x2 & 0xFF00FF00u;
+    half2_t r = (__builtin_bit_cast(half2_t, x2) - __builtin_bit_cast(half2_t, t[0])) * four;
+#pragma unroll
+    for (int i = 1; i < 3; i++) {
+        t[i] = (__builtin_bit_cast(uint32_t, r) + 0x00800080u) & 0xFF00FF00u;
+        r = (r - __builtin_bit_cast(half2_t, t[i])) * eight;
+    }
+    t[3] = __builtin_bit_cast(uint32_t, r) & 0xFF00FF00u;
+}
+
+struct Gemv8Epilogue {
+    const float *scale, *bias;
+    const void *residual;
+    void *y;
+    int relu, y_f16;
+};
+
+// ORDER: what separates the activation loads from the weight loads. 0: nothing. 1: a workgroup barrier, so that
+// no wavefront's activation loads queue behind another's weight loads (8192^2: 5.65 -> 5.3 us). 2: the
+// wavefront waits for its activation values before it asks for weights, so they do not queue behind the weight
+// requests of the whole chip either (16384^2, where 64 MiB are requested at once: 16.7 -> 15.8 us).
+template <int WAVES, int CB, int NT, int ORDER>
+__global__ __launch_bounds__(64 * WAVES) void gemv8_kernel(const _Float16 *__restrict__ x, const u32x4 *__restrict__ native,
+                                                           int Kb, int64_t N, int64_t Nb, Gemv8Epilogue ep) {
+    constexpr int KS = WAVES / CB, kUnits = (KS * NT + 2 * WAVES - 1) / (2 * WAVES);   // units of 8 values per thread: ceil(32 Kb / threads)
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    const int K = Kb * kKB;
+    const int plane = K + 32;                                    // bytes per term plane; +32 puts the four planes on different banks
+    unsigned char *planes = smem;
+    float *red = reinterpret_cast<float *>(smem + 4 * plane);   // [WAVES][16]
+    const int lane = threadIdx.x & 63, wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int j = lane & 15, g = lane >> 4;
+    const int cb = wv / KS, ks = wv % KS;
+    int64_t nb = (int64_t)blockIdx.x * CB + cb;
+    if (nb >= Nb) nb = Nb - 1;                                   // finite bits, never stored
+
+    // The activation quads of this thread's units first, then the weight blocks, all in flight at once; loads
+    // return in issue order, so waiting for the quads leaves the weights on their way. Unit u = (kb, d, h, g')
+    // covers x[256 kb + 64 d + 8 g' + 4 h + {0..3}] (quad A) and the same 32 further on (quad B): the eight
+    // values whose weights lane group g' finds in one operand register pair of dword d.
+    u32x2 qa[kUnits], qb[kUnits];
+#pragma unroll
+    for (int i = 0; i < kUnits; i++) {
+        const int u = threadIdx.x + i * 64 * WAVES;
+        const int gq = u & 3, h = (u >> 2) & 1, d = (u >> 3) & 3, kb = u >> 5;
+        const int k0 = kKB * kb + 64 * d + 8 * gq + 4 * h;
+        qa[i] = qb[i] = u32x2{0u, 0u};
+        if (u < K / 8) {
+            qa[i] = *reinterpret_cast<const u32x2 *>(x + k0);
+            qb[i] = *reinterpret_cast<const u32x2 *>(x + k0 + 32);
+        }
+    }
+    if (ORDER == 1) {
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    if (ORDER == 2) {
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_waitcnt(0x0F70);                      // vmcnt(0)
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    const u32x4 *wp = native + (nb * Kb + ks) * 64 + lane;
+    u32x4 wq[NT];
+#pragma unroll
+    for (int t = 0; t < NT; t++) {
+        wq[t] = __builtin_nontemporal_load(wp + (int64_t)t * KS * 64);
+        __builtin_amdgcn_sched_barrier(0);                       // issue order = use order: the waits below count on it
+    }
+    // per-channel constants of the threads that will store, asked for now
+    float sc = 1.f, bi = 0.f;
+    uint32_t res_bits = 0;                                       // converted where it is used: no wait for it here
+    const int64_t n_out = ((int64_t)blockIdx.x * CB + (threadIdx.x >> 4)) * 16 + (threadIdx.x & 15);
+    const bool stores = threadIdx.x < 16 * CB && n_out < N;
+    if (stores) {
+        if (ep.scale) sc = ep.scale[n_out];
+        if (ep.bias) bi = ep.bias[n_out];
+        if (ep.residual) res_bits = ep.y_f16 ? (uint32_t)static_cast<const uint16_t *>(ep.residual)[n_out]
+                                             : static_cast<const uint32_t *>(ep.residual)[n_out];
+    }
+#pragma unroll
+    for (int i = 0; i < kUnits; i++) {
+        const int u = threadIdx.x + i * 64 * WAVES;
+        if (u < K / 8) {
+            uint32_t ta0[4], ta1[4], tb0[4], tb1[4];
+            bf8_terms(qa[i][0], ta0);
+            bf8_terms(qa[i][1], ta1);
+            bf8_terms(qb[i][0], tb0);
+            bf8_terms(qb[i][1], tb1);
+#pragma unroll
+            for (int m = 0; m < 4; m++) {
+                // An operand register pair of dword d holds, byte by byte, the weights of (step 1, e), (step 0, e),
+                // (step 1, e + 1), (step 0, e + 1), ...: quad B and quad A interleaved, B first.
+                const uint32_t lo = __builtin_amdgcn_perm(ta0[m], tb0[m], 0x07030501u);
+                const uint32_t hi = __builtin_amdgcn_perm(ta1[m], tb1[m], 0x07030501u);
+                *reinterpret_cast<u32x2 *>(planes + m * plane + u * 8) = u32x2{lo, hi};
+            }
+        }
+    }
+    __builtin_amdgcn_s_waitcnt(0xC07F);                          // lgkmcnt(0): this thread's LDS writes are done
+    __builtin_amdgcn_s_barrier();                                // (not __syncthreads: that would wait for the weights too)
+    __builtin_amdgcn_sched_barrier(0);
+
+    floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+    const unsigned char *xb = planes + (j & 3) * plane + g * 8;  // column j carries term j % 4; columns 4..15 are never read back
+#pragma unroll
+    for (int t = 0; t < NT; t++) {
+        __builtin_amdgcn_sched_barrier(0);
+        const unsigned char *xp = xb + (ks + t * KS) * 256;
+#pragma unroll
+        for (int d = 0; d < 4; d++) {
+            const uint32_t w = wq[t][d];
+            const uint32_t r0 = w & 0xC0C0C0C0u, r1 = (w << 2) & 0xC0C0C0C0u, r2 = (w << 4) & 0xC0C0C0C0u, r3 = (w << 6) & 0xC0C0C0C0u;
+            const long a0 = (long)(((unsigned long)r1 << 32) | r0), a1 = (long)(((unsigned long)r3 << 32) | r2);
+            const long b0 = *reinterpret_cast<const long *>(xp + (d * 2 + 0) * 32);
+            const long b1 = *reinterpret_cast<const long *>(xp + (d * 2 + 1) * 32);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_fp8_bf8(a0, b0, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_fp8_bf8(a1, b1, acc, 0, 0, 0);
+        }
+    }
+    // D[n = 4 g + r][column j]: add the four term columns 0..3 (lanes j = 0..3 of each row of 16 lanes), each with
+    // the power of two its term was scaled by
+    const float term_weight = (j & 3) == 0 ? 1.0f : (j & 3) == 1 ? 0.25f : (j & 3) == 2 ? 0.03125f : 0.00390625f;
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        float v = acc[r] * term_weight;
+        v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, false));   // quad_perm [1,0,3,2]
+        v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, false));   // quad_perm [2,3,0,1]
+        acc[r] = v;
+    }
+    if (j == 0) {
+#pragma unroll
+        for (int r = 0; r < 4; r++) red[wv * 16 + 4 * g + r] = acc[r];
+    }
+    __syncthreads();
+    if (stores) {
+        const int c = threadIdx.x >> 4, i16 = threadIdx.x & 15;
+        float v = red[(c * KS) * 16 + i16];
+#pragma unroll
+        for (int q = 1; q < KS; q++) v += red[(c * KS + q) * 16 + i16];
+        v = v * (sc * (1.0f / kWeightUnit)) + bi;
+        if (ep.residual) v += ep.y_f16 ? (float)__builtin_bit_cast(_Float16, (uint16_t)res_bits) : __builtin_bit_cast(float, res_bits);
+        if (ep.relu) v = v < 0.f ? 0.f : v;
+        if (ep.y_f16) static_cast<_Float16 *>(ep.y)[n_out] = (_Float16)v;
+        else static_cast<float *>(ep.y)[n_out] = v;
+    }
+}
+
+template <int WAVES, int CB, int NT, int ORDER>
+int launch_gemv8(const void *x, const void *native, int64_t Kb, int64_t N, const Gemv8Epilogue &ep, void *stream) {
+    const int64_t Nb = native_blocks_n(N), grid = (Nb + CB - 1) / CB;
+    if (grid > 0x7FFFFFFF) return TMQ_ERR_TOO_LARGE;
+    const size_t lds = 4 * (size_t)(Kb * kKB + 32) + (size_t)WAVES * 16 * sizeof(float);
+    auto kernel = gemv8_kernel<WAVES, CB, NT, ORDER>;
+    if (lds > 64 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return note_hip_error(e);
+    }
+    hipLaunchKernelGGL(kernel, dim3((uint32_t)grid), dim3(64 * WAVES), lds, as_stream(stream), static_cast<const _Float16 *>(x),
+                       static_cast<const u32x4 *>(native), (int)Kb, N, Nb, ep);
+    return check_launch();
+}
+
+}  // namespace
+
+// True when the 8-bit GEMV can take a dense fp16 problem with one row.
+bool gemv8_dense_ok(const void *x, int64_t M, int64_t K) {
+    return M == 1 && K % (8 * kKB) == 0 && K >= 8 * kKB && K <= 64 * kKB && aligned16(x);
+}
+
+// gemv8_dense_ok must hold. Eight wavefronts per workgroup throughout; one channel block per workgroup up to 32
+// weight blocks per channel block, two beyond (half as many workgroups prepare the activation planes, each
+// wavefront with up to 16 KiB of weights in flight).
+int launch_gemv8_dense(const void *x, int64_t K, const void *native, int64_t N, const float *scale, const float *bias,
+                       const void *residual, int relu, void *y, int y_f16, void *stream) {
+    const Gemv8Epilogue ep{scale, bias, residual, y, relu, y_f16};
+    const int64_t Kb = K / kKB;
+    switch (Kb / 8) {
+        case 1: return launch_gemv8<8, 1, 1, 0>(x, native, Kb, N, ep, stream);
+        case 2: return launch_gemv8<8, 1, 2, 0>(x, native, Kb, N, ep, stream);
+        case 3: return launch_gemv8<8, 1, 3, 1>(x, native, Kb, N, ep, stream);
+        case 4: return launch_gemv8<8, 1, 4, 1>(x, native, Kb, N, ep, stream);
+        case 5: return launch_gemv8<8, 2, 10, 2>(x, native, Kb, N, ep, stream);
+        case 6: return launch_gemv8<8, 2, 12, 2>(x, native, Kb, N, ep, stream);
+        case 7: return launch_gemv8<8, 2, 14, 2>(x, native, Kb, N, ep, stream);
+        case 8: return launch_gemv8<8, 2, 16, 2>(x, native, Kb, N, ep, stream);
+        default: return TMQ_ERR_UNSUPPORTED;
+    }
+}
+
+}  // namespace tmq

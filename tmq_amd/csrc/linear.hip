@@ -28,6 +28,10 @@ int launch_stream_dense(const void *x, int64_t M, int64_t K, const void *native,
                         const float *bias, const void *residual, int relu, void *y, int y_f16, void *stream);
 int launch_mid_dense(const void *x, int64_t M, int64_t K, const void *native, int64_t N, const float *scale,
                      const float *bias, const void *residual, int relu, void *y, int y_f16, void *stream);
+// gemv8.hip: one fp16 row on the 8-bit matrix instructions
+bool gemv8_dense_ok(const void *x, int64_t M, int64_t K);
+int launch_gemv8_dense(const void *x, int64_t K, const void *native, int64_t N, const float *scale, const float *bias,
+                       const void *residual, int relu, void *y, int y_f16, void *stream);
 
 namespace {
 
@@ -1122,6 +1126,10 @@ int tmq_ternary_linear(const void *x, int x_dtype, int64_t M, int64_t K, const v
     if (epilogue) ep = *epilogue;
     if (ep.y_dtype != TMQ_F16 && ep.y_dtype != TMQ_F32) return TMQ_ERR_UNSUPPORTED;
     const bool x32 = x_dtype == TMQ_F32;
+    // One fp16 row, K a multiple of 2048 up to 16384: weights and activations as 8-bit MFMA operands (gemv8.hip),
+    // half the decode work per weight of the kernels below (4096^2: 3.75 -> 3.0 us, 16384^2: 17.7 -> 15.6 us).
+    if (!x32 && gemv8_dense_ok(x, M, K))
+        return launch_gemv8_dense(x, K, native, N, ep.scale, ep.bias, ep.residual, ep.relu, y, ep.y_dtype == TMQ_F16, stream);
     // At most 16 fp16 rows against eight or more weight blocks per channel: the weight-stream kernel (mid.hip).
     // Against the kernels below: M = 16 at 16384^2 67 -> 20 us, M = 8 at 8192 x 28672 34 -> 17 us, M = 1 at
     // 11008 x 4096 7.2 -> 6.2 us, even at 4096^2.
