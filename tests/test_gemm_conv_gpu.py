@@ -20,7 +20,12 @@ def _rel_err(got, want):
 GEMM_SHAPES = [(65, 64, 16), (128, 512, 64), (256, 4096, 256), (300, 147, 64), (1000, 576, 128), (513, 1000, 130),
                (4096, 512, 512), (777, 2304, 256), (3136, 256, 102), (2048, 64, 64),
                # few rows over a long reduction: the weight-stream kernel with every epilogue
-               (4, 2048, 520), (16, 2304, 1000), (1, 4096, 96)]
+               (4, 2048, 520), (16, 2304, 1000), (1, 4096, 96),
+               # 192 .. 1023 tiles of 64 x 256 over a long reduction: the kernel that issues its loads and weight
+               # expansion between the MFMAs (three-pass ring, counted waits); K = 256 b + 64 r exercises the
+               # partial last weight block with r = 1, 2, 3 tiles, ragged M and N the clamped rows / channels
+               (1024, 4096, 4096), (800, 1088, 4000), (777, 1152, 3900), (1500, 1216, 2100), (3072, 1024, 1024),
+               (13000, 1280, 130)]
 
 
 @pytest.mark.parametrize("M,K,N", GEMM_SHAPES)

@@ -21,6 +21,7 @@
 #include "mfma.h"
 #include "tile_epilogue.h"
 #include <type_traits>
+#include <utility>
 
 namespace tmq {
 
@@ -120,6 +121,40 @@ struct DenseDirect {
     }
     template <int CH, int T>
     __device__ __forceinline__ void advance(State<CH, T> &) const {}
+};
+
+// The same rows fetched through a buffer resource over x (fewer than 2^32 - 32 bytes): a chunk is a 32-bit
+// byte offset, and the loads are buffer instructions. The compiler keeps exact wait counts next to those; one
+// pending global-to-LDS load makes it wait for every outstanding load and LDS read at each use (it treats that
+// instruction like a flat access that may touch both memories). k-tiles past K deliver zeros.
+struct DenseBuffer {
+    [[maybe_unused]] static constexpr bool kDirect = true;
+    [[maybe_unused]] static constexpr bool kConv = false;
+    [[maybe_unused]] static constexpr bool kBuffer = true;
+    const _Float16 *x;
+    int64_t M, K;
+
+    template <int CH, int T>
+    struct State {
+        uint32_t row[CH];   // byte offset of the row + this thread's chunk
+        uint32_t k2;        // uniform: byte offset of the current k-tile inside a row
+    };
+    template <int CH, int T>
+    __device__ __forceinline__ void init(State<CH, T> &st, int64_t m0, int tid, int chunk) const {
+        st.k2 = 0;
+#pragma unroll
+        for (int i = 0; i < CH; i++) {
+            const int64_t m = m0 + (tid >> 3) + i * (T / 8);
+            st.row[i] = (uint32_t)((m < M ? m : M - 1) * K * 2) + chunk * 16;
+        }
+    }
+    template <int CH, int T>
+    __device__ __forceinline__ uint32_t offset(const State<CH, T> &st, int i) const {
+        return st.k2 < (uint32_t)(K * 2) ? st.row[i] + st.k2 : kPastTheEnd;
+    }
+    __device__ __forceinline__ uint32_t bytes() const { return (uint32_t)(M * K * 2); }
+    template <int CH, int T>
+    __device__ __forceinline__ void advance(State<CH, T> &st) const { st.k2 += kBK * 2; }
 };
 
 // im2col view of an NHWC fp16 tensor: row m = (b, oh, ow), k = (i * kx + j) * C + c.
@@ -619,6 +654,243 @@ __global__ __launch_bounds__(64 * WGM * WGN, 2) void tile_dma_kernel(Loader ld, 
                        nw0, M, N, ep);
 }
 
+// ---- one workgroup per CU: everything a wavefront does besides MFMAs goes between its MFMAs -----------------
+// With a single wavefront per SIMD nothing covers what the wavefront itself does not overlap. Measured with
+// the cycle counter on a 128 x 256 tile (per 64-wide k-tile and wavefront: 64 MFMAs = 1 024 cycles): the
+// expansion of the weight words costs 217 cycles when it sits in front of the MFMAs, issuing the tile's loads
+// 155 (a wavefront-wide 16-byte load occupies the issue slot for ~30 cycles, in a burst or not), a barrier
+// with its waits ~250. So here:
+//   * the operands of a k-tile's second 32-wide step are expanded between the MFMA groups of its first step,
+//     and the next tile's first-step operands between the groups of the second (VALU work issues while the
+//     matrix pipe is busy): the MFMA order is step-major, all row fragments of step 0, then all of step 1;
+//   * the loads -- the tile chunks of the pass two ahead and, once per weight block, the next block's
+//     words -- are issued one at a time between MFMA groups;
+//   * a pass is two k-tiles (one barrier per 128 reduction indices) and the ring holds three passes: what pass
+//     p requests has all of pass p + 1 to land in. The wait at the start of a pass leaves exactly the previous
+//     pass's loads outstanding (s_waitcnt vmcnt(n), n from the issue order: loads return in order).
+// Registers: up to 512 per lane at this occupancy (the accumulators may live in AGPRs). Needs a buffer loader
+// (exact wait counts, see DenseBuffer).
+template <class F, int... I>
+__device__ __forceinline__ void static_for_impl(F &&f, std::integer_sequence<int, I...>) {
+    (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N_, class F>
+__device__ __forceinline__ void static_for(F &&f) {   // f(integral_constant<int, 0>) ... f(integral_constant<int, N_ - 1>)
+    static_for_impl(f, std::make_integer_sequence<int, N_>{});
+}
+
+template <int N_>
+__device__ __forceinline__ void wait_vmcnt() {   // s_waitcnt vmcnt(N_), the other counters left alone
+    static_assert(N_ >= 0 && N_ < 64, "vmcnt is a 6-bit counter");
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (N_ & 15) | ((N_ >> 4) << 14));
+}
+
+template <int WM, int WN, int WGM, int WGN, int P, class Loader>
+__global__ __launch_bounds__(64 * WGM * WGN, 1) void tile_solo_kernel(Loader ld, const uint32_t *__restrict__ native,
+                                                                   int64_t M, int64_t K, int64_t N, int64_t Kb,
+                                                                   int64_t Nb, Epilogue ep, int tiles_m, int tiles_n) {
+    constexpr int WG = WGM * WGN, T = 64 * WG, BM = 16 * WM * WGM, BN = 16 * WN * WGN, CH = BM * 8 / T;
+    constexpr int kTileBytes = BM * kPitch * 2, kRing = 3;                 // passes in the ring, P tiles each
+    static_assert(BM * 8 % T == 0 && WM >= WN && (P == 1 || P == 2) && Loader::kBuffer, "geometry");
+    extern __shared__ __attribute__((aligned(16))) unsigned char ring_bytes[];
+
+    int id = blockIdx.x;
+    const int G = tiles_m * tiles_n;
+    if ((G & 7) == 0) id = (id & 7) * (G >> 3) + (id >> 3);
+    const int tm = id / tiles_n, tn = id % tiles_n;
+    const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
+
+    const int tid = threadIdx.x, lane = tid & 63, wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wv / WGN, wn = wv % WGN;
+    const int r16 = lane & 15, g = lane >> 4;
+
+    typename Loader::template State<CH, T> st;
+    ld.template init<CH, T>(st, m0, tid, (tid & 7) ^ ((tid >> 3) & 7));
+
+    floatx4 acc[WM][WN];
+#pragma unroll
+    for (int i = 0; i < WM; i++)
+#pragma unroll
+        for (int j = 0; j < WN; j++) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+    const uint32_t *wptr[WN];
+#pragma unroll
+    for (int j = 0; j < WN; j++) {
+        int64_t nb = n0 / 16 + wn * WN + j;
+        if (nb >= Nb) nb = Nb - 1;
+        wptr[j] = native + (nb * Kb) * 256 + lane * 4;
+    }
+    const int KT = (int)((K + kBK - 1) / kBK), KB = (KT + 3) >> 2, KBfull = KT >> 2;
+    u32x4 wblk[WN], wnext[WN];
+
+    unsigned char *const lds0 = ring_bytes + wv * 1024;
+    const BufferResource rsrc = make_buffer_resource(ld.x, ld.bytes());
+    auto chunk = [&](int tslot, int i) {   // chunk i of the loader's current tile -> tile slot of the ring
+        buffer_to_lds(rsrc, ld.template offset<CH, T>(st, i), lds0 + tslot * kTileBytes + i * (T * 16));
+    };
+
+    // the first two passes and the first weight block, before anything waits on memory
+#pragma unroll
+    for (int t = 0; t < (kRing - 1) * P; t++) {
+#pragma unroll
+        for (int i = 0; i < CH; i++) chunk(t, i);
+        ld.template advance<CH, T>(st);
+    }
+#pragma unroll
+    for (int j = 0; j < WN; j++) wblk[j] = *reinterpret_cast<const u32x4 *>(wptr[j]);
+    const int64_t nw0 = n0 + (int64_t)wn * WN * 16;
+    ColumnConstants cc;
+    load_scale_bias<WN>(ep, lane, nw0, N, cc);
+    __builtin_amdgcn_sched_barrier(0);
+
+    const int arow = (wm * WM * 16 + r16) * kPitch;
+    auto swz = [&](int i, int s) { return i * 16 * kPitch + (((4 * s + g) ^ (r16 & 7)) * 8); };
+    constexpr int NQ = 2 * WM, kAhead = 4;
+    half8 b0[2][WN], b1[WN];        // expanded operands: step 0 of the tiles of even / odd parity, step 1
+
+    // One k-tile out of tile slot `tslot`, MFMA group p = step p / WM, row fragment p % WM. Its step-0 operands
+    // are in b0[PAR]; its step-1 operands are expanded from `w` during step 0, the next tile's step-0 operands
+    // from `wn` during step 1, and after group p `between(p)` may issue one load.
+    auto multiply = [&](int tslot, auto par, const uint32_t (&w)[WN], const uint32_t (&wn_)[WN], auto between) {
+        constexpr int PAR = decltype(par)::value;
+        const _Float16 *abase = reinterpret_cast<const _Float16 *>(ring_bytes) + tslot * (BM * kPitch) + arow;
+        half8 a[NQ];
+#pragma unroll
+        for (int q = 0; q < kAhead; q++) a[q] = *reinterpret_cast<const half8 *>(abase + swz(q % WM, q / WM));
+        __builtin_amdgcn_sched_barrier(0);
+        static_for<NQ>([&](auto qc) {
+                constexpr int Q = decltype(qc)::value, fi = Q % WM, fs = Q / WM;
+#pragma unroll
+                for (int j = 0; j < WN; j++) acc[fi][j] = mfma16(a[Q], fs == 0 ? b0[PAR][j] : b1[j], acc[fi][j]);
+                if constexpr (Q + kAhead < NQ)
+                    a[Q + kAhead] = *reinterpret_cast<const half8 *>(abase + swz((Q + kAhead) % WM, (Q + kAhead) / WM));
+                if constexpr (fs == 0 && fi < WN) b1[fi] = decode_step(w[fi], 1);
+                if constexpr (fs == 1 && fi < WN) b0[PAR ^ 1][fi] = decode_step(wn_[fi], 0);
+                between(std::integral_constant<int, Q>{});
+                // issue order inside the group: two VALU operations behind every MFMA (they issue while the
+                // matrix pipe is busy; in one block behind the MFMAs they would delay the next group)
+#pragma unroll
+                for (int j = 0; j < WN; j++) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);       // MFMA
+                    __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);       // VALU
+                }
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);           // DS read
+                __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);           // VMEM read
+                __builtin_amdgcn_sched_barrier(0);
+        });
+    };
+
+    // everything the prologue asked for has landed: the counted waits start from nothing outstanding
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+#pragma unroll
+    for (int j = 0; j < WN; j++) b0[0][j] = decode_step(wblk[j][0], 0);
+    int cur = 0;                                     // ring slot of the pass being multiplied
+    // Pass H of weight block kb: tiles 4 kb + H P .. + P - 1. It requests the tiles of the pass two ahead (ring
+    // slot cur + 2) and, when H == 0, the next weight block.
+    auto pass = [&](int kb, auto hc) {
+        constexpr int H = decltype(hc)::value;
+        // this thread's chunks of the pass are in LDS: all it has asked for except what the last pass issued
+        wait_vmcnt<P * CH + ((H + 4 / P - 1) % (4 / P) == 0 ? WN : 0)>();
+        __builtin_amdgcn_s_waitcnt(0xC07F);           // (lgkmcnt(0): and its operand reads of the last pass are done)
+        __builtin_amdgcn_s_barrier();                 // ... and everybody's; the slot multiplied last is free
+        __builtin_amdgcn_sched_barrier(0);
+        const int ahead = cur == 0 ? kRing - 1 : cur - 1;     // = (cur + kRing - 1) % kRing
+        static_for<P>([&](auto ec) {
+                constexpr int E = decltype(ec)::value;
+                constexpr int q = P * H + E;          // position of the tile in its weight block
+                constexpr int kItems = CH + ((H == 0 && E == 0) ? WN : 0);
+                uint32_t w[WN], wn_[WN];
+#pragma unroll
+                for (int j = 0; j < WN; j++) {
+                    w[j] = wblk[j][q];
+                    wn_[j] = q < 3 ? wblk[j][q < 3 ? q + 1 : 0] : wnext[j][0];
+                }
+                multiply(cur * P + E, std::integral_constant<int, q & 1>{}, w, wn_, [&](auto gc) {
+                    constexpr int grp = decltype(gc)::value;
+#pragma unroll
+                    for (int t = 0; t < kItems; t++)      // item t goes out after group t NQ / kItems
+                        if (t * NQ / kItems == grp) {
+                            if (t < CH) chunk(ahead * P + E, t);
+                            else {
+                                int nb = kb + 1;
+                                if (nb >= KB) nb = KB - 1;
+                                wnext[t - CH] = *reinterpret_cast<const u32x4 *>(wptr[t - CH] + (int64_t)nb * 256);
+                            }
+                        }
+                });
+                ld.template advance<CH, T>(st);
+        });
+        cur = cur == kRing - 1 ? 0 : cur + 1;
+    };
+    for (int kb = 0; kb < KBfull; kb++) {
+        pass(kb, std::integral_constant<int, 0>{});
+        pass(kb, std::integral_constant<int, 1>{});
+        if constexpr (P == 1) {
+            pass(kb, std::integral_constant<int, 2>{});
+            pass(kb, std::integral_constant<int, 3>{});
+        }
+#pragma unroll
+        for (int j = 0; j < WN; j++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) asm volatile("v_mov_b32 %0, %1" : "=v"(wblk[j][e]) : "v"(wnext[j][e]));
+    }
+    // The last, partial weight block (1 .. 3 tiles): plain tiles, operands expanded in front of the MFMAs. The
+    // loop has requested the first (kRing - 1) P of them; a further one is fetched here, into the slot of the
+    // pass multiplied last.
+    for (int kt = KBfull * 4; kt < KT; kt++) {
+        const int e = kt & 3;
+        int ps = cur + e / P;
+        if (ps >= kRing) ps -= kRing;
+        const int tslot = ps * P + e % P;
+        if (e >= (kRing - 1) * P) {
+            __syncthreads();
+#pragma unroll
+            for (int i = 0; i < CH; i++) chunk(tslot, i);
+            ld.template advance<CH, T>(st);
+        }
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+        __syncthreads();
+        const _Float16 *abase = reinterpret_cast<const _Float16 *>(ring_bytes) + tslot * (BM * kPitch) + arow;
+        half8 bfr[2][WN];
+#pragma unroll
+        for (int j = 0; j < WN; j++) {
+            const uint32_t w = e == 0 ? wblk[j][0] : e == 1 ? wblk[j][1] : wblk[j][2];
+            bfr[0][j] = decode_step(w, 0);
+            bfr[1][j] = decode_step(w, 1);
+        }
+#pragma unroll
+        for (int q = 0; q < NQ; q++) {
+            const half8 a = *reinterpret_cast<const half8 *>(abase + swz(q >> 1, q & 1));
+#pragma unroll
+            for (int j = 0; j < WN; j++) acc[q >> 1][j] = mfma16(a, bfr[q & 1][j], acc[q >> 1][j]);
+        }
+    }
+    // drain the requests past K before the ring is reused as transpose slabs
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();
+    constexpr int kEP = 16 * WN + 4;
+    static_assert(WG * 16 * kEP * 4 <= kRing * P * kTileBytes, "epilogue slab does not fit the ring");
+    write_tile<WM, WN>(reinterpret_cast<float *>(ring_bytes) + wv * 16 * kEP, acc, cc, lane, m0 + (int64_t)wm * WM * 16,
+                       nw0, M, N, ep);
+}
+
+template <int WM, int WN, int WGM, int WGN, int P, class Loader>
+int launch_tile_solo(const Loader &ld, const void *native, int64_t M, int64_t K, int64_t N, const Epilogue &ep,
+                     void *stream) {
+    constexpr int BM = 16 * WM * WGM, BN = 16 * WN * WGN, kLds = 3 * P * BM * kPitch * 2;
+    const int64_t tm = (M + BM - 1) / BM, tn = (N + BN - 1) / BN;
+    if (tm * tn > 0x7FFFFFFF) return TMQ_ERR_TOO_LARGE;
+    auto kernel = tile_solo_kernel<WM, WN, WGM, WGN, P, Loader>;
+    if constexpr (kLds > 64 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
+        if (e != hipSuccess) return note_hip_error(e);
+    }
+    hipLaunchKernelGGL(kernel, dim3((uint32_t)(tm * tn)), dim3(64 * WGM * WGN), kLds, as_stream(stream), ld,
+                       static_cast<const uint32_t *>(native), M, K, N, native_blocks_k(K), native_blocks_n(N), ep, (int)tm,
+                       (int)tn);
+    return check_launch();
+}
+
 template <int WM, int WN, int WGM, int WGN, int P, class Loader>
 int launch_tile_dma(const Loader &ld, const void *native, int64_t M, int64_t K, int64_t N, const Epilogue &ep,
                     void *stream) {
@@ -701,6 +973,16 @@ int dispatch_tile(const Loader &ld, const void *native, int64_t M, int64_t K, in
 int launch_gemm_dense(const void *x, int64_t M, int64_t K, const void *native, int64_t N, const float *scale,
                       const float *bias, const void *residual, int relu, void *y, int y_f16, void *stream) {
     Epilogue ep{scale, bias, residual, y, relu, y_f16};
+    // A few hundred 64 x 256 tiles, i.e. one or two four-wavefront workgroups per CU and a long reduction:
+    // the kernel that puts everything between its MFMAs (K = N = 4096: M = 768 32.0 -> 29.4 us, M = 1024
+    // 36.1 -> 30.2, M = 2048 52.5 -> 51.1, M = 3072 84.8 -> 75.9; from 1024 such tiles on the 128 x 256 tiles,
+    // two workgroups per CU, win: M = 4096 99 against 105 us).
+    {
+        const int64_t t64 = ((M + 63) / 64) * ((N + 255) / 256);
+        if ((K % kBK == 0) && aligned16(x) && K >= 1024 && N > 128 && t64 >= 192 && t64 < 1024 &&
+            M * K * 2 < (int64_t)kPastTheEnd - 16)
+            return launch_tile_solo<4, 4, 1, 4, 2>(DenseBuffer{static_cast<const _Float16 *>(x), M, K}, native, M, K, N, ep, stream);
+    }
     if ((K % kBK == 0) && aligned16(x))
         return dispatch_tile(DenseDirect{static_cast<const _Float16 *>(x), M, K}, native, M, K, N, ep, stream);
     return dispatch_tile(DenseLoader{static_cast<const _Float16 *>(x), M, K}, native, M, K, N, ep, stream);
