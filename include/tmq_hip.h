@@ -252,7 +252,8 @@ typedef struct tmq_epilogue {
  * exponent range: max|x| at most 65504, and values below ~6e-5 lose precision. Tensors of any other
  * magnitude go through tmq_f32_prescale first (exact power-of-two scaling, undone in the per-channel scale of
  * the epilogue); the Python / PyTorch bindings of this library always do, because the reference multiplies
- * fp32 activations in fp32 and has no such limit.
+ * fp32 activations in fp32 and has no such limit. One case needs no prescale: a single fp32 row for which
+ * tmq_fp32_rows_self_scaled returns 1 is scaled inside the kernel and may have any magnitude.
  * Arithmetic: exact products, fp32 accumulation. One fp16 row (M == 1) with K a multiple of 2048 up to 16384
  * runs on the 8-bit matrix instructions (weights as fp8, the row as four exact bf8 terms); there the hardware adds
  * 32 products at a time aligned to the largest of them, so the result can differ from an fp32 running sum by a few
@@ -263,6 +264,11 @@ typedef struct tmq_epilogue {
  * bias passes of Linear.compact_forward (tmq/tmq.py:684-687). Any M, K, N (ragged tails masked). */
 int tmq_ternary_linear(const void *x, int x_dtype, int64_t M, int64_t K, const void *native,
                        int64_t N, const tmq_epilogue *epilogue, void *y, void *stream);
+
+/* 1 when tmq_ternary_linear(x, TMQ_F32, M, K, ...) takes fp32 activations of any magnitude as they are (one
+ * 16-byte aligned row, K a multiple of 2048 up to 8192: the kernel finds the row's largest finite |x| and scales
+ * by a power of two itself), 0 when the caller has to keep them inside fp16's range (tmq_f32_prescale). */
+int tmq_fp32_rows_self_scaled(const void *x, int64_t M, int64_t K);
 
 /* Range handling for fp32 activations (no counterpart in the reference, whose kernels multiply fp32
  * activations in fp32, tmq/tmq_cuda.cu:242-427). Scans n fp32 values and writes prescale[0] = s,

@@ -164,3 +164,48 @@ def test_agrees_with_the_fp16_kernels_on_neighbouring_shapes(cuda, oracle):
     buf[1:K + 1] = x[0]
     y3 = ops.ternary_linear(buf[1:K + 1][None], nw)                     # 2-byte aligned: not the 8-bit kernel
     assert _rel_err(y1.cpu().numpy(), y3.cpu().numpy()) <= 1e-5
+
+
+@pytest.mark.parametrize("K", [2048, 4096, 6144, 8192])
+def test_fp32_row_runs_as_two_fp16_halves(cuda, oracle, K):
+    """One fp32 row (the reference's GEMV convention) up to K = 8192: hi = fp16(x), lo = fp16(x - hi), each as four
+    bf8 terms in eight activation columns. 22 significant bits of every value reach the product."""
+    from tmq_amd import ops
+    N = 1000
+    rng = np.random.default_rng(K)
+    W, nw = _layer(cuda, oracle, rng, N, K)
+    x = rng.standard_normal((1, K)).astype(np.float32)
+    scale = (0.5 + rng.random(N)).astype(np.float32)
+    bias = rng.standard_normal(N).astype(np.float32)
+    t = lambda a: torch.from_numpy(a).to(cuda)
+    y = ops.ternary_linear(t(x), nw, t(scale), t(bias))
+    ref = (x.astype(np.float64) @ W.astype(np.float64).T) * scale + bias
+    assert y.dtype == torch.float32 and _rel_err(y.cpu().numpy(), ref) <= 1e-5
+    # far better than a single fp16 rounding of the row would be
+    y16 = ops.ternary_linear(t(x).half(), nw, t(scale), t(bias))
+    assert _rel_err(y.cpu().numpy(), ref) < 0.1 * _rel_err(y16.cpu().numpy(), ref)
+    # the reference's binding name, every rank it takes
+    words = t(oracle.pack(W).view(np.int32))
+    for shape in ((K,), (1, K), (1, 1, K)):
+        v = ops.ternary_mvm_cuda(t(x.reshape(shape)), words, N)
+        assert tuple(v.shape) == shape[:-1] + (N,)
+        assert _rel_err(v.cpu().numpy().reshape(1, N), x.astype(np.float64) @ W.astype(np.float64).T) <= 1e-5
+    # residual + ReLU, fp16 output
+    res = rng.standard_normal((1, N)).astype(np.float16)
+    y3 = ops.ternary_linear(t(x), nw, t(scale), t(bias), residual=t(res), relu=True, out_dtype=torch.float16)
+    assert _rel_err(y3.float().cpu().numpy(), np.maximum(ref + res.astype(np.float64), 0)) <= 1e-3
+
+
+def test_fp32_row_passes_22_bit_values_through_exactly(cuda, oracle):
+    """Identity weights: integers of up to 22 bits (and their power-of-two multiples, small and large) come back
+    exactly -- both halves and all eight term columns are in place."""
+    from tmq_amd import ops
+    K = N = 2048
+    nw = ops.NativeWeights(torch.from_numpy(oracle.pack(np.eye(N, dtype=np.float32)).view(np.int32)).to(cuda), N)
+    rng = np.random.default_rng(9)
+    ints = rng.integers(-(1 << 21), 1 << 21, size=(1, K)).astype(np.float32)
+    for s in (1.0, 2.0 ** -30, 2.0 ** 40, 2.0 ** -120, 2.0 ** 100):    # the kernel scales the row itself
+        x = (ints * np.float32(s)).astype(np.float32)
+        x[0, :4] = [0.0, -0.0, np.float32(s), -np.float32(s)]
+        y = ops.ternary_linear(torch.from_numpy(x).to(cuda), nw).cpu().numpy()
+        assert np.array_equal(y, x), s

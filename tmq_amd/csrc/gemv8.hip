@@ -25,10 +25,12 @@
 // wavefronts meet in LDS in wavefront order (deterministic). Measured (HIP-graph replays over rotating weight
 // buffers): K = N = 4096 3.0 us (fp16 weight-stream kernel 3.75), 8192^2 5.5 us, 16384^2 15.6 us (17.7).
 //
-// Requires fp16 activations, M == 1, K a multiple of 2048 and at most 16384, 16-byte aligned x.
+// Requires M == 1, K a multiple of 2048 and at most 16384 (fp32 activations, carried as two fp16 halves: 8192),
+// 16-byte aligned x.
 #include "common.h"
 #include "mfma.h"
 
+#include <math.h>
 #include <type_traits>
 
 namespace tmq {
@@ -70,15 +72,20 @@ struct Gemv8Epilogue {
 // no wavefront's activation loads queue behind another's weight loads (8192^2: 5.65 -> 5.3 us). 2: the
 // wavefront waits for its activation values before it asks for weights, so they do not queue behind the weight
 // requests of the whole chip either (16384^2, where 64 MiB are requested at once: 16.7 -> 15.8 us).
-template <int WAVES, int CB, int NT, int ORDER>
-__global__ __launch_bounds__(64 * WAVES) void gemv8_kernel(const _Float16 *__restrict__ x, const u32x4 *__restrict__ native,
+//
+// X32: the row is fp32, of any magnitude (the kernel scales it by a power of two itself). Each value becomes
+// hi = fp16(x) and lo = fp16(x - hi) -- 22 significant bits -- and both halves their four bf8 terms: eight
+// planes, eight of the sixteen activation columns, still one MFMA per weight operand.
+template <int WAVES, int CB, int NT, int ORDER, bool X32>
+__global__ __launch_bounds__(64 * WAVES) void gemv8_kernel(const void *__restrict__ xv, const u32x4 *__restrict__ native,
                                                            int Kb, int64_t N, int64_t Nb, Gemv8Epilogue ep) {
     constexpr int KS = WAVES / CB, kUnits = (KS * NT + 2 * WAVES - 1) / (2 * WAVES);   // units of 8 values per thread: ceil(32 Kb / threads)
+    constexpr int NP = X32 ? 8 : 4;                              // term planes
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const int K = Kb * kKB;
-    const int plane = K + 32;                                    // bytes per term plane; +32 puts the four planes on different banks
+    const int plane = K + 32;                                    // bytes per term plane; +32 puts the planes on different banks
     unsigned char *planes = smem;
-    float *red = reinterpret_cast<float *>(smem + 4 * plane);   // [WAVES][16]
+    float *red = reinterpret_cast<float *>(smem + NP * plane);  // [WAVES][16]
     const int lane = threadIdx.x & 63, wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int j = lane & 15, g = lane >> 4;
     const int cb = wv / KS, ks = wv % KS;
@@ -89,16 +96,22 @@ __global__ __launch_bounds__(64 * WAVES) void gemv8_kernel(const _Float16 *__res
     // return in issue order, so waiting for the quads leaves the weights on their way. Unit u = (kb, d, h, g')
     // covers x[256 kb + 64 d + 8 g' + 4 h + {0..3}] (quad A) and the same 32 further on (quad B): the eight
     // values whose weights lane group g' finds in one operand register pair of dword d.
-    u32x2 qa[kUnits], qb[kUnits];
+    using Quad = std::conditional_t<X32, u32x4, u32x2>;           // four activation values
+    Quad qa[kUnits], qb[kUnits];
 #pragma unroll
     for (int i = 0; i < kUnits; i++) {
         const int u = threadIdx.x + i * 64 * WAVES;
         const int gq = u & 3, h = (u >> 2) & 1, d = (u >> 3) & 3, kb = u >> 5;
         const int k0 = kKB * kb + 64 * d + 8 * gq + 4 * h;
-        qa[i] = qb[i] = u32x2{0u, 0u};
+        qa[i] = qb[i] = Quad{};
         if (u < K / 8) {
-            qa[i] = *reinterpret_cast<const u32x2 *>(x + k0);
-            qb[i] = *reinterpret_cast<const u32x2 *>(x + k0 + 32);
+            if constexpr (X32) {
+                qa[i] = *reinterpret_cast<const u32x4 *>(static_cast<const float *>(xv) + k0);
+                qb[i] = *reinterpret_cast<const u32x4 *>(static_cast<const float *>(xv) + k0 + 32);
+            } else {
+                qa[i] = *reinterpret_cast<const u32x2 *>(static_cast<const _Float16 *>(xv) + k0);
+                qb[i] = *reinterpret_cast<const u32x2 *>(static_cast<const _Float16 *>(xv) + k0 + 32);
+            }
         }
     }
     if (ORDER == 1) {
@@ -129,22 +142,72 @@ __global__ __launch_bounds__(64 * WAVES) void gemv8_kernel(const _Float16 *__res
         if (ep.residual) res_bits = ep.y_f16 ? (uint32_t)static_cast<const uint16_t *>(ep.residual)[n_out]
                                              : static_cast<const uint32_t *>(ep.residual)[n_out];
     }
+    // fp32 rows of any magnitude: the row times the power of two that brings its largest finite |x| into
+    // [1024, 2048) (exact), undone in the epilogue -- the hi / lo halves then sit well inside fp16's range. Every
+    // workgroup holds the whole row, so the maximum is one reduction through LDS.
+    float ps = 1.f, ps_inv = 1.f;
+    if constexpr (X32) {
+        float amax = 0.f;
+#pragma unroll
+        for (int i = 0; i < kUnits; i++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const float a = __builtin_fabsf(__builtin_bit_cast(float, qa[i][e])), b = __builtin_fabsf(__builtin_bit_cast(float, qb[i][e]));
+                amax = fmaxf(amax, a < INFINITY ? a : 0.f);      // NaN and Inf take no part (they propagate anyway)
+                amax = fmaxf(amax, b < INFINITY ? b : 0.f);
+            }
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
+        if (lane == 0) red[wv] = amax;
+        __builtin_amdgcn_s_waitcnt(0xC07F);                      // lgkmcnt(0)
+        __builtin_amdgcn_s_barrier();
+#pragma unroll
+        for (int q = 0; q < WAVES; q++) amax = fmaxf(amax, red[q]);
+        if (amax > 0.f) {
+            int e;
+            (void)frexpf(amax, &e);                              // amax in [2^(e-1), 2^e)
+            int p = 11 - e;
+            p = p > 126 ? 126 : (p < -126 ? -126 : p);
+            ps = ldexpf(1.f, p);
+            ps_inv = ldexpf(1.f, -p);
+        }
+        // (the partial sums below reuse red[] only after the next barrier)
+    }
+    // the planes of one unit from its two quads as packed fp16 pairs (plane offset P0: 0, or 4 for the lo halves)
+    auto write_planes = [&](int u, int p0, uint32_t a0, uint32_t a1, uint32_t b0, uint32_t b1) {
+        uint32_t ta0[4], ta1[4], tb0[4], tb1[4];
+        bf8_terms(a0, ta0);
+        bf8_terms(a1, ta1);
+        bf8_terms(b0, tb0);
+        bf8_terms(b1, tb1);
+#pragma unroll
+        for (int m = 0; m < 4; m++) {
+            // An operand register pair of dword d holds, byte by byte, the weights of (step 1, e), (step 0, e),
+            // (step 1, e + 1), (step 0, e + 1), ...: quad B and quad A interleaved, B first.
+            const uint32_t lo = __builtin_amdgcn_perm(ta0[m], tb0[m], 0x07030501u);
+            const uint32_t hi = __builtin_amdgcn_perm(ta1[m], tb1[m], 0x07030501u);
+            *reinterpret_cast<u32x2 *>(planes + (p0 + m) * plane + u * 8) = u32x2{lo, hi};
+        }
+    };
 #pragma unroll
     for (int i = 0; i < kUnits; i++) {
         const int u = threadIdx.x + i * 64 * WAVES;
         if (u < K / 8) {
-            uint32_t ta0[4], ta1[4], tb0[4], tb1[4];
-            bf8_terms(qa[i][0], ta0);
-            bf8_terms(qa[i][1], ta1);
-            bf8_terms(qb[i][0], tb0);
-            bf8_terms(qb[i][1], tb1);
+            if constexpr (X32) {
+                uint32_t hi[4], lo[4];                           // pairs (0, 1), (2, 3) of quad A, then of quad B
 #pragma unroll
-            for (int m = 0; m < 4; m++) {
-                // An operand register pair of dword d holds, byte by byte, the weights of (step 1, e), (step 0, e),
-                // (step 1, e + 1), (step 0, e + 1), ...: quad B and quad A interleaved, B first.
-                const uint32_t lo = __builtin_amdgcn_perm(ta0[m], tb0[m], 0x07030501u);
-                const uint32_t hi = __builtin_amdgcn_perm(ta1[m], tb1[m], 0x07030501u);
-                *reinterpret_cast<u32x2 *>(planes + m * plane + u * 8) = u32x2{lo, hi};
+                for (int p = 0; p < 4; p++) {
+                    const float v0 = ps * __builtin_bit_cast(float, p < 2 ? qa[i][2 * p] : qb[i][2 * p - 4]);
+                    const float v1 = ps * __builtin_bit_cast(float, p < 2 ? qa[i][2 * p + 1] : qb[i][2 * p - 3]);
+                    const _Float16 h0 = (_Float16)v0, h1 = (_Float16)v1;
+                    const _Float16 l0 = (_Float16)(v0 - (float)h0), l1 = (_Float16)(v1 - (float)h1);
+                    hi[p] = __builtin_bit_cast(uint32_t, half2_t{h0, h1});
+                    lo[p] = __builtin_bit_cast(uint32_t, half2_t{l0, l1});
+                }
+                write_planes(u, 0, hi[0], hi[1], hi[2], hi[3]);
+                write_planes(u, 4, lo[0], lo[1], lo[2], lo[3]);
+            } else {
+                write_planes(u, 0, qa[i][0], qa[i][1], qb[i][0], qb[i][1]);
             }
         }
     }
@@ -153,7 +216,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemv8_kernel(const _Float16 *__res
     __builtin_amdgcn_sched_barrier(0);
 
     floatx4 acc = {0.f, 0.f, 0.f, 0.f};
-    const unsigned char *xb = planes + (j & 3) * plane + g * 8;  // column j carries term j % 4; columns 4..15 are never read back
+    const unsigned char *xb = planes + (j & (NP - 1)) * plane + g * 8;   // column j carries plane j % NP; the other columns are never read back
 #pragma unroll
     for (int t = 0; t < NT; t++) {
         __builtin_amdgcn_sched_barrier(0);
@@ -177,6 +240,8 @@ __global__ __launch_bounds__(64 * WAVES) void gemv8_kernel(const _Float16 *__res
         float v = acc[r] * term_weight;
         v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, false));   // quad_perm [1,0,3,2]
         v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, false));   // quad_perm [2,3,0,1]
+        if constexpr (X32)                                       // + the lo half's columns 4..7
+            v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x104, 0xF, 0xF, false));   // row_shl:4
         acc[r] = v;
     }
     if (j == 0) {
@@ -189,6 +254,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemv8_kernel(const _Float16 *__res
         float v = red[(c * KS) * 16 + i16];
 #pragma unroll
         for (int q = 1; q < KS; q++) v += red[(c * KS + q) * 16 + i16];
+        if constexpr (X32) v *= ps_inv;
         v = v * (sc * (1.0f / kWeightUnit)) + bi;
         if (ep.residual) v += ep.y_f16 ? (float)__builtin_bit_cast(_Float16, (uint16_t)res_bits) : __builtin_bit_cast(float, res_bits);
         if (ep.relu) v = v < 0.f ? 0.f : v;
@@ -197,17 +263,17 @@ __global__ __launch_bounds__(64 * WAVES) void gemv8_kernel(const _Float16 *__res
     }
 }
 
-template <int WAVES, int CB, int NT, int ORDER>
+template <int WAVES, int CB, int NT, int ORDER, bool X32 = false>
 int launch_gemv8(const void *x, const void *native, int64_t Kb, int64_t N, const Gemv8Epilogue &ep, void *stream) {
     const int64_t Nb = native_blocks_n(N), grid = (Nb + CB - 1) / CB;
     if (grid > 0x7FFFFFFF) return TMQ_ERR_TOO_LARGE;
-    const size_t lds = 4 * (size_t)(Kb * kKB + 32) + (size_t)WAVES * 16 * sizeof(float);
-    auto kernel = gemv8_kernel<WAVES, CB, NT, ORDER>;
+    const size_t lds = (X32 ? 8 : 4) * (size_t)(Kb * kKB + 32) + (size_t)WAVES * 16 * sizeof(float);
+    auto kernel = gemv8_kernel<WAVES, CB, NT, ORDER, X32>;
     if (lds > 64 * 1024) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return note_hip_error(e);
     }
-    hipLaunchKernelGGL(kernel, dim3((uint32_t)grid), dim3(64 * WAVES), lds, as_stream(stream), static_cast<const _Float16 *>(x),
+    hipLaunchKernelGGL(kernel, dim3((uint32_t)grid), dim3(64 * WAVES), lds, as_stream(stream), x,
                        static_cast<const u32x4 *>(native), (int)Kb, N, Nb, ep);
     return check_launch();
 }
@@ -235,6 +301,25 @@ int launch_gemv8_dense(const void *x, int64_t K, const void *native, int64_t N, 
         case 6: return launch_gemv8<8, 2, 12, 2>(x, native, Kb, N, ep, stream);
         case 7: return launch_gemv8<8, 2, 14, 2>(x, native, Kb, N, ep, stream);
         case 8: return launch_gemv8<8, 2, 16, 2>(x, native, Kb, N, ep, stream);
+        default: return TMQ_ERR_UNSUPPORTED;
+    }
+}
+
+// One fp32 row: K a multiple of 2048 up to 8192 (eight term planes; beyond that they leave room for one workgroup
+// per CU only).
+bool gemv8_dense32_ok(const void *x, int64_t M, int64_t K) {
+    return M == 1 && K % (8 * kKB) == 0 && K >= 8 * kKB && K <= 32 * kKB && aligned16(x);
+}
+
+int launch_gemv8_dense32(const void *x, int64_t K, const void *native, int64_t N, const float *scale, const float *bias,
+                         const void *residual, int relu, void *y, int y_f16, void *stream) {
+    const Gemv8Epilogue ep{scale, bias, residual, y, relu, y_f16};
+    const int64_t Kb = K / kKB;
+    switch (Kb / 8) {
+        case 1: return launch_gemv8<8, 1, 1, 0, true>(x, native, Kb, N, ep, stream);
+        case 2: return launch_gemv8<8, 1, 2, 0, true>(x, native, Kb, N, ep, stream);
+        case 3: return launch_gemv8<8, 1, 3, 1, true>(x, native, Kb, N, ep, stream);
+        case 4: return launch_gemv8<8, 1, 4, 1, true>(x, native, Kb, N, ep, stream);
         default: return TMQ_ERR_UNSUPPORTED;
     }
 }

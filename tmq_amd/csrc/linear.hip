@@ -32,6 +32,9 @@ int launch_mid_dense(const void *x, int64_t M, int64_t K, const void *native, in
 bool gemv8_dense_ok(const void *x, int64_t M, int64_t K);
 int launch_gemv8_dense(const void *x, int64_t K, const void *native, int64_t N, const float *scale, const float *bias,
                        const void *residual, int relu, void *y, int y_f16, void *stream);
+bool gemv8_dense32_ok(const void *x, int64_t M, int64_t K);
+int launch_gemv8_dense32(const void *x, int64_t K, const void *native, int64_t N, const float *scale, const float *bias,
+                         const void *residual, int relu, void *y, int y_f16, void *stream);
 
 namespace {
 
@@ -1089,6 +1092,10 @@ int tmq_prepack_weights(const uint32_t *words, int64_t N, int64_t C, int64_t ky,
     return check_launch();
 }
 
+int tmq_fp32_rows_self_scaled(const void *x, int64_t M, int64_t K) {
+    return gemv8_dense32_ok(x, M, K) ? 1 : 0;
+}
+
 int tmq_fp32_rows_prefer_split(int64_t M, int64_t K, int64_t N) {
     // Measured: at K = N = 4096 the two fp16 passes win from about 512 rows (M = 4096: 400 -> 238 us), at
     // K = N = 1024 from about 4096; over large layers already from 9 rows (8192^2, M = 16: 34 -> 23 us) or,
@@ -1130,6 +1137,9 @@ int tmq_ternary_linear(const void *x, int x_dtype, int64_t M, int64_t K, const v
     // half the decode work per weight of the kernels below (4096^2: 3.75 -> 3.0 us, 16384^2: 17.7 -> 15.6 us).
     if (!x32 && gemv8_dense_ok(x, M, K))
         return launch_gemv8_dense(x, K, native, N, ep.scale, ep.bias, ep.residual, ep.relu, y, ep.y_dtype == TMQ_F16, stream);
+    // ... and one fp32 row (the reference's GEMV convention) up to K = 8192: the same kernel on the row's two fp16 halves
+    if (x32 && gemv8_dense32_ok(x, M, K))
+        return launch_gemv8_dense32(x, K, native, N, ep.scale, ep.bias, ep.residual, ep.relu, y, ep.y_dtype == TMQ_F16, stream);
     // At most 16 fp16 rows against eight or more weight blocks per channel: the weight-stream kernel (mid.hip).
     // Against the kernels below: M = 16 at 16384^2 67 -> 20 us, M = 8 at 8192 x 28672 34 -> 17 us, M = 1 at
     // 11008 x 4096 7.2 -> 6.2 us, even at 4096^2.

@@ -218,6 +218,10 @@ void check_mm_args(const torch::Tensor &lhs, const torch::Tensor &weights, int64
 // rows: the fp16 kernels over the two fp16 terms, y = W hi + W lo; few rows: the kernels that split on the fly.
 torch::Tensor linear_f32(const torch::Tensor &x, int64_t M, int64_t K, const torch::Tensor &native, int64_t columns,
                          torch::Tensor &y, const char *name) {
+    if (tmq_fp32_rows_self_scaled(x.data_ptr(), M, K)) {   // a single row the kernel scales itself: one launch
+        check(tmq_ternary_linear(x.data_ptr(), TMQ_F32, M, K, native.data_ptr(), columns, nullptr, y.data_ptr(), stream_of(x)), name);
+        return y;
+    }
     const bool two_pass = tmq_fp32_rows_prefer_split(M, K, columns) != 0;
     auto fopt = x.options().dtype(torch::kFloat32);
     auto prescale = torch::empty({2}, fopt), scale = torch::empty({columns}, fopt);

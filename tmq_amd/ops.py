@@ -566,7 +566,9 @@ def ternary_linear(x: torch.Tensor, nw: NativeWeights, scale=None, bias=None, re
     if x.shape[-1] != nw.K:
         raise RuntimeError(f"ternary_linear: activations have {x.shape[-1]} features, weights expect {nw.K}")
     M = x.numel() // nw.K if nw.K else 0
-    if x.dtype == torch.float32 and M > 0:
+    if x.dtype == torch.float32 and M == 1 and x.is_contiguous() and _lib().tmq_fp32_rows_self_scaled(ptr(x), M, nw.K):
+        pass            # a single row the kernel scales itself (any magnitude): one launch, no prescale pass
+    elif x.dtype == torch.float32 and M > 0:
         two_pass = (out_dtype == torch.float32 and (residual is None or residual.dtype == torch.float32)
                     and bool(_lib().tmq_fp32_rows_prefer_split(M, nw.K, nw.N)))
         ps = None
