@@ -254,7 +254,7 @@ typedef struct tmq_epilogue {
  * the epilogue); the Python / PyTorch bindings of this library always do, because the reference multiplies
  * fp32 activations in fp32 and has no such limit. One case needs no prescale: a single fp32 row for which
  * tmq_fp32_rows_self_scaled returns 1 is scaled inside the kernel and may have any magnitude.
- * Arithmetic: exact products, fp32 accumulation. One fp16 row (M == 1) with K a multiple of 2048 up to 16384
+ * Arithmetic: exact products, fp32 accumulation. One fp16 row (M == 1) with K a multiple of 256 from 2048 to 16384
  * runs on the 8-bit matrix instructions (weights as fp8, the row as four exact bf8 terms); there the hardware adds
  * 32 products at a time aligned to the largest of them, so the result can differ from an fp32 running sum by a few
  * 1e-6 of the largest output (about 1e-4 when values near 65504 sit next to values of order one) -- inside the
@@ -266,7 +266,7 @@ int tmq_ternary_linear(const void *x, int x_dtype, int64_t M, int64_t K, const v
                        int64_t N, const tmq_epilogue *epilogue, void *y, void *stream);
 
 /* 1 when tmq_ternary_linear(x, TMQ_F32, M, K, ...) takes fp32 activations of any magnitude as they are (one
- * 16-byte aligned row, K a multiple of 2048 up to 8192: the kernel finds the row's largest finite |x| and scales
+ * 16-byte aligned row, K a multiple of 256 from 2048 to 8192: the kernel finds the row's largest finite |x| and scales
  * by a power of two itself), 0 when the caller has to keep them inside fp16's range (tmq_f32_prescale). */
 int tmq_fp32_rows_self_scaled(const void *x, int64_t M, int64_t K);
 

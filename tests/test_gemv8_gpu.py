@@ -1,4 +1,4 @@
-"""One fp16 activation row with K a multiple of 2048 (up to 16384) runs on the 8-bit matrix instructions:
+"""One fp16 activation row with K a multiple of 256 (2048 .. 16384) runs on the 8-bit matrix instructions:
 weights as fp8 +-2, the activation vector as four exact bf8 terms. Checked against an fp64 product of the
 expanded weights (not the library), through every epilogue, ragged N, every K the kernel takes, and on the
 inputs where its one numerical difference from an fp32 sum (the instruction's internal alignment window over
@@ -30,7 +30,9 @@ def _layer(cuda, oracle, rng, N, K, p0=0.5):
     return W, ops.NativeWeights(torch.from_numpy(words.view(np.int32)).to(cuda), N)
 
 
-@pytest.mark.parametrize("K", [2048 * i for i in range(1, 9)])
+# every multiple of 2048, and block counts that do not deal out evenly over the wavefronts of a channel block
+# (9, 20, 27, 33, 43, 54 and 63 blocks of 256: a wavefront without a block in the last round multiplies by zero)
+@pytest.mark.parametrize("K", [2048 * i for i in range(1, 9)] + [2304, 5120, 6912, 8448, 11008, 13824, 16128])
 @pytest.mark.parametrize("N", [16, 1000, 4100])
 def test_every_reduction_length_and_ragged_channels(cuda, oracle, K, N):
     from tmq_amd import ops
@@ -166,7 +168,7 @@ def test_agrees_with_the_fp16_kernels_on_neighbouring_shapes(cuda, oracle):
     assert _rel_err(y1.cpu().numpy(), y3.cpu().numpy()) <= 1e-5
 
 
-@pytest.mark.parametrize("K", [2048, 4096, 6144, 8192])
+@pytest.mark.parametrize("K", [2048, 4096, 6144, 8192, 2304, 5120, 6912])
 def test_fp32_row_runs_as_two_fp16_halves(cuda, oracle, K):
     """One fp32 row (the reference's GEMV convention) up to K = 8192: hi = fp16(x), lo = fp16(x - hi), each as four
     bf8 terms in eight activation columns. 22 significant bits of every value reach the product."""

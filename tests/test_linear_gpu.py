@@ -45,9 +45,9 @@ def test_linear_fp16_matches_oracle(cuda, oracle, M, K, N):
     want = oracle.gemm(x.astype(np.float32), words, N, scale, bias)
     assert y.shape == (M, N) and y.dtype == torch.float32
     assert _rel_err(y.cpu().numpy(), want) <= RTOL
-    # what fp32 accumulation actually delivers; a single row with K a multiple of 2048 runs on the 8-bit matrix
+    # what fp32 accumulation actually delivers; a single row with K a multiple of 256 from 2048 on runs on the 8-bit matrix
     # instructions, whose 32-product adder rounds a little more coarsely
-    tight = 1e-5 if (M == 1 and K % 2048 == 0) else 2e-6
+    tight = 1e-5 if (M == 1 and K % 256 == 0 and K >= 2048) else 2e-6
     assert _rel_err(y.cpu().numpy(), want) <= tight
     y0 = ops.ternary_linear(tx, nw)                          # no scale / bias
     assert _rel_err(y0.cpu().numpy(), oracle.gemm(x.astype(np.float32), words, N)) <= tight

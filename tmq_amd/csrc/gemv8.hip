@@ -25,7 +25,7 @@
 // wavefronts meet in LDS in wavefront order (deterministic). Measured (HIP-graph replays over rotating weight
 // buffers): K = N = 4096 3.0 us (fp16 weight-stream kernel 3.75), 8192^2 5.5 us, 16384^2 15.6 us (17.7).
 //
-// Requires M == 1, K a multiple of 2048 and at most 16384 (fp32 activations, carried as two fp16 halves: 8192),
+// Requires M == 1, K a multiple of 256 from 2048 to 16384 (fp32 activations, carried as two fp16 halves: to 8192),
 // 16-byte aligned x.
 #include "common.h"
 #include "mfma.h"
@@ -124,11 +124,14 @@ __global__ __launch_bounds__(64 * WAVES) void gemv8_kernel(const void *__restric
         __builtin_amdgcn_s_waitcnt(0x0F70);                      // vmcnt(0)
         __builtin_amdgcn_sched_barrier(0);
     }
-    const u32x4 *wp = native + (nb * Kb + ks) * 64 + lane;
+    // wavefront ks takes blocks ks, ks + KS, ...; when Kb is no multiple of KS the last round is short: a
+    // wavefront without a block there re-reads block Kb - 1 (weights and activations) and multiplies it by zero
+    const u32x4 *wp = native + nb * Kb * 64 + lane;
     u32x4 wq[NT];
 #pragma unroll
     for (int t = 0; t < NT; t++) {
-        wq[t] = __builtin_nontemporal_load(wp + (int64_t)t * KS * 64);
+        const int kblk = ks + t * KS < Kb ? ks + t * KS : Kb - 1;
+        wq[t] = __builtin_nontemporal_load(wp + (int64_t)kblk * 64);
         __builtin_amdgcn_sched_barrier(0);                       // issue order = use order: the waits below count on it
     }
     // per-channel constants of the threads that will store, asked for now
@@ -220,11 +223,13 @@ __global__ __launch_bounds__(64 * WAVES) void gemv8_kernel(const void *__restric
 #pragma unroll
     for (int t = 0; t < NT; t++) {
         __builtin_amdgcn_sched_barrier(0);
-        const unsigned char *xp = xb + (ks + t * KS) * 256;
+        const bool live = ks + t * KS < Kb;                      // uniform
+        const unsigned char *xp = xb + (live ? ks + t * KS : Kb - 1) * 256;
+        const uint32_t mask = live ? 0xC0C0C0C0u : 0u;
 #pragma unroll
         for (int d = 0; d < 4; d++) {
             const uint32_t w = wq[t][d];
-            const uint32_t r0 = w & 0xC0C0C0C0u, r1 = (w << 2) & 0xC0C0C0C0u, r2 = (w << 4) & 0xC0C0C0C0u, r3 = (w << 6) & 0xC0C0C0C0u;
+            const uint32_t r0 = w & mask, r1 = (w << 2) & mask, r2 = (w << 4) & mask, r3 = (w << 6) & mask;
             const long a0 = (long)(((unsigned long)r1 << 32) | r0), a1 = (long)(((unsigned long)r3 << 32) | r2);
             const long b0 = *reinterpret_cast<const long *>(xp + (d * 2 + 0) * 32);
             const long b1 = *reinterpret_cast<const long *>(xp + (d * 2 + 1) * 32);
@@ -282,40 +287,56 @@ int launch_gemv8(const void *x, const void *native, int64_t Kb, int64_t N, const
 
 // True when the 8-bit GEMV can take a dense fp16 problem with one row.
 bool gemv8_dense_ok(const void *x, int64_t M, int64_t K) {
-    return M == 1 && K % (8 * kKB) == 0 && K >= 8 * kKB && K <= 64 * kKB && aligned16(x);
+    return M == 1 && K % kKB == 0 && K >= 8 * kKB && K <= 64 * kKB && aligned16(x);
 }
 
 // gemv8_dense_ok must hold. Eight wavefronts per workgroup throughout; one channel block per workgroup up to 32
-// weight blocks per channel block, two beyond (half as many workgroups prepare the activation planes, each
-// wavefront with up to 16 KiB of weights in flight).
+// weight blocks per channel block, two beyond when that still leaves two workgroups per CU (half as many
+// workgroups prepare the activation planes, each wavefront with up to 16 KiB of weights in flight).
 int launch_gemv8_dense(const void *x, int64_t K, const void *native, int64_t N, const float *scale, const float *bias,
                        const void *residual, int relu, void *y, int y_f16, void *stream) {
     const Gemv8Epilogue ep{scale, bias, residual, y, relu, y_f16};
     const int64_t Kb = K / kKB;
-    switch (Kb / 8) {
-        case 1: return launch_gemv8<8, 1, 1, 0>(x, native, Kb, N, ep, stream);
-        case 2: return launch_gemv8<8, 1, 2, 0>(x, native, Kb, N, ep, stream);
-        case 3: return launch_gemv8<8, 1, 3, 1>(x, native, Kb, N, ep, stream);
-        case 4: return launch_gemv8<8, 1, 4, 1>(x, native, Kb, N, ep, stream);
-        case 5: return launch_gemv8<8, 2, 10, 2>(x, native, Kb, N, ep, stream);
-        case 6: return launch_gemv8<8, 2, 12, 2>(x, native, Kb, N, ep, stream);
-        case 7: return launch_gemv8<8, 2, 14, 2>(x, native, Kb, N, ep, stream);
-        case 8: return launch_gemv8<8, 2, 16, 2>(x, native, Kb, N, ep, stream);
+    if (Kb <= 32) {
+        switch ((Kb + 7) / 8) {                                  // blocks per wavefront, 8 wavefronts per channel block
+            case 1: return launch_gemv8<8, 1, 1, 0>(x, native, Kb, N, ep, stream);
+            case 2: return launch_gemv8<8, 1, 2, 0>(x, native, Kb, N, ep, stream);
+            case 3: return launch_gemv8<8, 1, 3, 1>(x, native, Kb, N, ep, stream);
+            default: return launch_gemv8<8, 1, 4, 1>(x, native, Kb, N, ep, stream);
+        }
+    }
+    if (native_blocks_n(N) < 512) {                              // two channel blocks per workgroup would leave CUs idle
+        switch ((Kb + 7) / 8) {
+            case 5: return launch_gemv8<8, 1, 5, 2>(x, native, Kb, N, ep, stream);
+            case 6: return launch_gemv8<8, 1, 6, 2>(x, native, Kb, N, ep, stream);
+            case 7: return launch_gemv8<8, 1, 7, 2>(x, native, Kb, N, ep, stream);
+            default: return launch_gemv8<8, 1, 8, 2>(x, native, Kb, N, ep, stream);
+        }
+    }
+    switch ((Kb + 3) / 4) {                                      // 4 wavefronts per channel block
+        case 9: return launch_gemv8<8, 2, 9, 2>(x, native, Kb, N, ep, stream);
+        case 10: return launch_gemv8<8, 2, 10, 2>(x, native, Kb, N, ep, stream);
+        case 11: return launch_gemv8<8, 2, 11, 2>(x, native, Kb, N, ep, stream);
+        case 12: return launch_gemv8<8, 2, 12, 2>(x, native, Kb, N, ep, stream);
+        case 13: return launch_gemv8<8, 2, 13, 2>(x, native, Kb, N, ep, stream);
+        case 14: return launch_gemv8<8, 2, 14, 2>(x, native, Kb, N, ep, stream);
+        case 15: return launch_gemv8<8, 2, 15, 2>(x, native, Kb, N, ep, stream);
+        case 16: return launch_gemv8<8, 2, 16, 2>(x, native, Kb, N, ep, stream);
         default: return TMQ_ERR_UNSUPPORTED;
     }
 }
 
-// One fp32 row: K a multiple of 2048 up to 8192 (eight term planes; beyond that they leave room for one workgroup
+// One fp32 row: K a multiple of 256 from 2048 to 8192 (eight term planes; beyond that they leave room for one workgroup
 // per CU only).
 bool gemv8_dense32_ok(const void *x, int64_t M, int64_t K) {
-    return M == 1 && K % (8 * kKB) == 0 && K >= 8 * kKB && K <= 32 * kKB && aligned16(x);
+    return M == 1 && K % kKB == 0 && K >= 8 * kKB && K <= 32 * kKB && aligned16(x);
 }
 
 int launch_gemv8_dense32(const void *x, int64_t K, const void *native, int64_t N, const float *scale, const float *bias,
                          const void *residual, int relu, void *y, int y_f16, void *stream) {
     const Gemv8Epilogue ep{scale, bias, residual, y, relu, y_f16};
     const int64_t Kb = K / kKB;
-    switch (Kb / 8) {
+    switch ((Kb + 7) / 8) {
         case 1: return launch_gemv8<8, 1, 1, 0, true>(x, native, Kb, N, ep, stream);
         case 2: return launch_gemv8<8, 1, 2, 0, true>(x, native, Kb, N, ep, stream);
         case 3: return launch_gemv8<8, 1, 3, 1, true>(x, native, Kb, N, ep, stream);
