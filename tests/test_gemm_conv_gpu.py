@@ -57,6 +57,35 @@ def test_large_m_linear(cuda, oracle, M, K, N):
     assert _rel_err(y3.float().cpu().numpy(), want3) <= 1e-3
 
 
+def test_mid_size_kernel_is_deterministic_and_replays_in_a_graph(cuda, oracle):
+    """M = 1024, K = N = 2048 (256 tiles of 64 x 256: the kernel with hand-counted waits): the same bits on every
+    run, eager and as replays of a HIP graph with eager work in between."""
+    from tmq_amd import ops
+    rng = np.random.default_rng(21)
+    M, K, N = 1024, 2048, 2048
+    W = _ternary(rng, (N, K))
+    nw = ops.NativeWeights(torch.from_numpy(oracle.pack(W).view(np.int32)).to(cuda), N)
+    x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float16)).to(cuda)
+    eager = ops.ternary_linear(x, nw).clone()
+    ref = x.cpu().numpy().astype(np.float64) @ W.astype(np.float64).T
+    assert _rel_err(eager.cpu().numpy(), ref) <= 3e-6
+    for _ in range(3):
+        assert torch.equal(ops.ternary_linear(x, nw), eager)
+    graph, side = torch.cuda.CUDAGraph(), torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        y = torch.empty(M, N, device=cuda)
+        with torch.cuda.graph(graph, stream=side):
+            y.copy_(ops.ternary_linear(x, nw))
+    for rep in range(3):
+        y.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y, eager), rep
+        ops.ternary_linear(torch.randn_like(x), nw)
+        torch.cuda.synchronize()
+
+
 def test_skinny_and_tile_kernels_agree(cuda, oracle):
     """M = 64 (skinny kernel) and M = 65 (tile kernel) must give the same rows for integer data."""
     from tmq_amd import ops

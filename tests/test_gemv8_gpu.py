@@ -211,3 +211,30 @@ def test_fp32_row_passes_22_bit_values_through_exactly(cuda, oracle):
         x[0, :4] = [0.0, -0.0, np.float32(s), -np.float32(s)]
         y = ops.ternary_linear(torch.from_numpy(x).to(cuda), nw).cpu().numpy()
         assert np.array_equal(y, x), s
+
+
+def test_hip_graph_replays_match_eager(cuda, oracle):
+    """The GEMV captured into a HIP graph (K = 16384: the launch that opts in to more than 64 KiB of LDS; an fp32
+    row: the kernel that scales inside) gives the eager result on every replay, with eager work and
+    synchronisations between the replays."""
+    from tmq_amd import ops
+    rng = np.random.default_rng(11)
+    for K, N, dt in ((16384, 520, torch.float16), (4096, 1000, torch.float32), (11008, 300, torch.float16)):
+        W, nw = _layer(cuda, oracle, rng, N, K)
+        x = torch.from_numpy(rng.standard_normal((1, K)).astype(np.float32)).to(cuda).to(dt)
+        eager = ops.ternary_linear(x, nw).clone()
+        torch.cuda.synchronize()
+        graph, side = torch.cuda.CUDAGraph(), torch.cuda.Stream()
+        with torch.cuda.stream(side):
+            y = torch.empty(1, N, device=cuda)
+            with torch.cuda.graph(graph, stream=side):
+                y.copy_(ops.ternary_linear(x, nw))
+        for rep in range(3):
+            y.fill_(float("nan"))
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(y, eager), (K, rep)
+            x2 = torch.randn_like(x)                               # eager work on the same weights in between
+            ops.ternary_linear(x2, nw)
+            torch.cuda.synchronize()
