@@ -86,6 +86,30 @@ def test_mid_size_kernel_is_deterministic_and_replays_in_a_graph(cuda, oracle):
         torch.cuda.synchronize()
 
 
+@pytest.mark.parametrize("M,K,N", [(4100, 2048, 4096), (4096, 2112, 4608)])
+def test_full_chip_of_wide_tiles_against_fp64_on_the_gpu(cuda, oracle, M, K, N):
+    """At least 256 tiles of 128 x 512 over a long reduction: eight-wavefront workgroups. Too large for a CPU
+    reference in a unit test: checked against the GPU's fp64 matrix product of the expanded weights (a library
+    routine that shares nothing with these kernels), with ragged rows and every epilogue."""
+    from tmq_amd import ops
+    g = torch.Generator(device="cpu").manual_seed(M + K)
+    W = torch.randint(-1, 2, (N, K), generator=g, dtype=torch.int8)
+    nw = ops.NativeWeights(torch.from_numpy(oracle.pack(W.numpy().astype(np.float32)).view(np.int32)).to(cuda), N)
+    x = torch.randn(M, K, generator=g).half().to(cuda)
+    scale = (0.5 + torch.rand(N, generator=g)).to(cuda)
+    bias = torch.randn(N, generator=g).to(cuda)
+    ref = (x.double() @ W.to(cuda).double().t()) * scale.double() + bias.double()
+    y = ops.ternary_linear(x, nw, scale, bias)
+    assert ((y.double() - ref).abs().max() / ref.abs().max()).item() <= 3e-6
+    res = torch.randn(M, N, generator=g).half().to(cuda)
+    y2 = ops.ternary_linear(x, nw, scale, bias, residual=res, relu=True, out_dtype=torch.float16)
+    want = (ref + res.double()).clamp_min(0)
+    assert ((y2.double() - want).abs().max() / want.abs().max()).item() <= 1e-3
+    xi = torch.randint(-4, 5, (M, K), generator=g).half().to(cuda)
+    yi = ops.ternary_linear(xi, nw)
+    assert torch.equal(yi.double(), xi.double() @ W.to(cuda).double().t())        # integers: exact
+
+
 def test_skinny_and_tile_kernels_agree(cuda, oracle):
     """M = 64 (skinny kernel) and M = 65 (tile kernel) must give the same rows for integer data."""
     from tmq_amd import ops

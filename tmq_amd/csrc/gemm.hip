@@ -521,7 +521,7 @@ __device__ __forceinline__ void load_to_lds(const void *src, unsigned char *dst)
 }
 
 template <int WM, int WN, int WGM, int WGN, int P, class Loader>
-__global__ __launch_bounds__(64 * WGM * WGN, 2) void tile_dma_kernel(Loader ld, const uint32_t *__restrict__ native,
+__global__ __launch_bounds__(64 * WGM * WGN, WGM * WGN > 4 ? 1 : 2) void tile_dma_kernel(Loader ld, const uint32_t *__restrict__ native,
                                                                   int64_t M, int64_t K, int64_t N, int64_t Kb,
                                                                   int64_t Nb, Epilogue ep, int tiles_m, int tiles_n) {
     constexpr int T = 64 * WGM * WGN, BM = 16 * WM * WGM, BN = 16 * WN * WGN, CH = BM * 8 / T, S = 2 * P;
@@ -943,6 +943,11 @@ int dispatch_tile(const Loader &ld, const void *native, int64_t M, int64_t K, in
         // (measured at K = 4096: M = 4096 100 -> 93.5 us, M = 1024 52.5 -> 46.6, but M = 2048, two
         // 128 x 128 tiles per CU, 59 -> 64; every 64 x 64 case loses).
         const bool two = K >= 2048;
+        // A chip full of 128 x 512 tiles, eight wavefronts of 128 rows x 64 channels (one workgroup per CU): every
+        // activation row is read N / 512 times instead of N / 256 (M = K = N = 4096: 98.9 -> 93.8 us, M = 8192
+        // 196 -> 188, 8192^3 709 -> 693; with ragged tiles, N = 11008, it loses 1 %)
+        if (!Loader::kConv && two && N % 512 == 0 && wgs(128, 512) >= 256)
+            return launch_tile_dma<8, 4, 1, 8, 2>(ld, native, M, K, N, ep, stream);
         if (N > 128 && wgs(128, 256) >= 384)
             return two ? launch_tile_dma<8, 4, 1, 4, 2>(ld, native, M, K, N, ep, stream)
                        : launch_tile_dma<8, 4, 1, 4, 1>(ld, native, M, K, N, ep, stream);
