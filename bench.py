@@ -227,7 +227,7 @@ def bench_linear(args, torch):
         o = out["4096"]
         res["roofline"] = {"bound": "mfma", "achieved": o["tflops"], "peak": MFMA_FP16_PEAK_TFLOPS, "unit": "TFLOP/s",
                            "frac": o["frac_mfma_fp16"], "traffic": None, "algorithmic_flops": 2.0 * 4096 * N * K,
-                           "kernel": "tile_dma_kernel<128 x 512> (M = 4096)", "avg_launch_us": o["us"]}
+                           "kernel": "tile_solo_kernel<128 x 512> (M = 4096)", "avg_launch_us": o["us"]}
     if "1" in out:
         o = out["1"]
         res["roofline_gemv"] = {"bound": "hbm", "achieved": o["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",

@@ -86,7 +86,9 @@ def test_mid_size_kernel_is_deterministic_and_replays_in_a_graph(cuda, oracle):
         torch.cuda.synchronize()
 
 
-@pytest.mark.parametrize("M,K,N", [(4100, 2048, 4096), (4096, 2112, 4608)])
+# 128 x 512 tiles, one k-tile per pass: whole weight blocks, then a last block of 1 and of 3 tiles (the third is fetched
+# in the tail); 64 x 512 tiles (2000 x 4096: 256 of them)
+@pytest.mark.parametrize("M,K,N", [(4100, 2048, 4096), (4096, 2112, 4608), (4096, 2240, 4096), (2000, 1280, 4096)])
 def test_full_chip_of_wide_tiles_against_fp64_on_the_gpu(cuda, oracle, M, K, N):
     """At least 256 tiles of 128 x 512 over a long reduction: eight-wavefront workgroups. Too large for a CPU
     reference in a unit test: checked against the GPU's fp64 matrix product of the expanded weights (a library

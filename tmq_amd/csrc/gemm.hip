@@ -978,15 +978,24 @@ int dispatch_tile(const Loader &ld, const void *native, int64_t M, int64_t K, in
 int launch_gemm_dense(const void *x, int64_t M, int64_t K, const void *native, int64_t N, const float *scale,
                       const float *bias, const void *residual, int relu, void *y, int y_f16, void *stream) {
     Epilogue ep{scale, bias, residual, y, relu, y_f16};
-    // A few hundred 64 x 256 tiles, i.e. one or two four-wavefront workgroups per CU and a long reduction:
-    // the kernel that puts everything between its MFMAs (K = N = 4096: M = 768 32.0 -> 29.4 us, M = 1024
-    // 36.1 -> 30.2, M = 2048 52.5 -> 51.1, M = 3072 84.8 -> 75.9; from 1024 such tiles on the 128 x 256 tiles,
-    // two workgroups per CU, win: M = 4096 99 against 105 us).
-    {
+    // Dense rows through a buffer resource: the kernel that puts its expansion and loads between the MFMAs.
+    //  * A chip full of 128 x 512 tiles (N a multiple of 512), eight wavefronts of 128 rows x 64 channels, one k-tile
+    //    per pass: every activation row is read N / 512 times from L2. Against 128 x 256 tiles with two workgroups
+    //    per CU: M = K = N = 4096 98.9 -> 93.0 us, M = 8192 196 -> 186, M = 6144 171 -> 163.5, 4096 x 8192 x 8192
+    //    349 -> 340 (the same tiles in tile_dma_kernel: 93.8, 188, 171, 349).
+    //  * 192 .. 256 tiles of 64 x 512, eight wavefronts: M = 2048 53.0 -> 50.7 us, M = 1536 47.1 -> 43.9.
+    //  * A few hundred 64 x 256 tiles, four wavefronts, one or two workgroups per CU: M = 768 32.0 -> 29.4 us,
+    //    M = 1024 36.1 -> 30.2, M = 3072 84.8 -> 75.9; from 1024 such tiles on the 128 x 256 tiles of
+    //    tile_dma_kernel, two workgroups per CU, win (N = 11008 at M = 4096).
+    if ((K % kBK == 0) && aligned16(x) && K >= 1024 && N > 128 && M * K * 2 < (int64_t)kPastTheEnd - 16) {
+        const DenseBuffer ld{static_cast<const _Float16 *>(x), M, K};
+        if (N % 512 == 0) {
+            const int64_t t128 = ((M + 127) / 128) * (N / 512), t64 = ((M + 63) / 64) * (N / 512);
+            if (K >= 2048 && t128 >= 256) return launch_tile_solo<8, 4, 1, 8, 1>(ld, native, M, K, N, ep, stream);
+            if (t64 >= 192 && t64 <= 256) return launch_tile_solo<4, 4, 1, 8, 2>(ld, native, M, K, N, ep, stream);
+        }
         const int64_t t64 = ((M + 63) / 64) * ((N + 255) / 256);
-        if ((K % kBK == 0) && aligned16(x) && K >= 1024 && N > 128 && t64 >= 192 && t64 < 1024 &&
-            M * K * 2 < (int64_t)kPastTheEnd - 16)
-            return launch_tile_solo<4, 4, 1, 4, 2>(DenseBuffer{static_cast<const _Float16 *>(x), M, K}, native, M, K, N, ep, stream);
+        if (t64 >= 192 && t64 < 1024) return launch_tile_solo<4, 4, 1, 4, 2>(ld, native, M, K, N, ep, stream);
     }
     if ((K % kBK == 0) && aligned16(x))
         return dispatch_tile(DenseDirect{static_cast<const _Float16 *>(x), M, K}, native, M, K, N, ep, stream);
