@@ -142,6 +142,9 @@ CONV_CASES = [  # B, C, H, W, N, k, stride, pad, dil
     (5, 16, 7, 7, 64, (5, 3), (2, 1), (4, 3), (1, 2)), (2, 32, 6, 13, 24, 3, (1, 2), (3, 0), 1),
     # ... and on the split-reduction kernel (many channels, few output tiles)
     (1, 256, 5, 5, 128, 3, 1, 3, 1), (2, 512, 4, 6, 256, 3, 2, 2, 2),
+    # 129 .. 256 output channels over at least 8192 output positions: 64 x 256 tiles, eight wavefronts, loads between
+    # the MFMAs (18 k-tiles + none / 2 k-tiles only / ragged channels, stride 2 and a ragged last row tile)
+    (8, 128, 32, 32, 256, 3, 1, 1, 1), (8, 128, 32, 32, 256, 1, 1, 0, 1), (9, 64, 61, 63, 200, 3, 2, 1, 1),
 ]
 
 
