@@ -116,8 +116,8 @@ class FusedTernaryResNet18:
         B, C, H, W = x.shape
         nhwc4 = self.ops.nchw_to_nhwc4(x)
         xs = nhwc4.view(B, H, W // 2, 8).permute(0, 3, 1, 2)      # [B, 8, H, W / 2], channels_last memory
-        y = self._run(xs, self.stem, relu=True)
-        y = self.ops.maxpool2d_nhwc(y, 3, 2, 1)
+        nw, scale, bias, stride, pad = self.stem
+        y = self.ops.ternary_conv2d_relu_maxpool(xs, nw, stride, pad, 1, scale, bias)      # conv1 + bn1 + relu + maxpool
         for c1, c2, ds in self.blocks:
             idt = y if ds is None else self._run(y, ds, relu=False)
             h = self._run(y, c1, relu=True)

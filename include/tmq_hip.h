@@ -369,6 +369,17 @@ int tmq_ternary_dwconvtrans_cols(const float *x, int64_t B, int64_t P, int32_t t
 int tmq_maxpool2d_nhwc(const void *x, int32_t B, int32_t C, int32_t H, int32_t W, int32_t ky, int32_t kx,
                        int32_t sy, int32_t sx, int32_t py, int32_t px, void *y, void *stream);
 
+/* The opening of a ResNet in one launch: tmq_ternary_conv2d with a ReLU epilogue and fp16 output,
+ * followed by tmq_maxpool2d_nhwc(3, 3, 2, 2, 1, 1), without the convolution's output ever reaching
+ * memory. x, shape, native, scale and bias as for tmq_ternary_conv2d (no residual); y fp16
+ * [B][Po][Pwo][N] with Po = (Ho - 1) / 2 + 1 for the convolution's Ho, likewise Pwo. The result equals the
+ * two separate calls bit for bit (finite inputs; a NaN loses against any number in the maximum, as in
+ * tmq_maxpool2d_nhwc). For few-channel inputs with a short reduction only: C of 8, 16 or 32,
+ * C * ky * kx <= 256, N <= 64 in whole groups of 8, and an input window per 15 x 17 outputs of under 64 KiB;
+ * anything else returns TMQ_ERR_UNSUPPORTED and the caller makes the two calls.                   */
+int tmq_ternary_conv2d_relu_maxpool(const void *x, const tmq_conv_shape *shape, const void *native,
+                                    const float *scale, const float *bias, void *y, void *stream);
+
 /* Global average pool: x [B][HW][C] fp16 -> y [B][C] (TMQ_F16 or TMQ_F32), fp32 accumulation.    */
 int tmq_avgpool_global_nhwc(const void *x, int64_t B, int64_t HW, int64_t C, void *y, int y_dtype,
                             void *stream);

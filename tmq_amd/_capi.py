@@ -88,6 +88,7 @@ SIGNATURES = {
     "tmq_conv2d_out_hw": (_int, [ctypes.POINTER(ConvShape), ctypes.POINTER(ctypes.c_int32),
                                  ctypes.POINTER(ctypes.c_int32)]),
     "tmq_ternary_conv2d": (_int, [_vp, ctypes.POINTER(ConvShape), _vp, _vp, _vp, _vp]),
+    "tmq_ternary_conv2d_relu_maxpool": (_int, [_vp, ctypes.POINTER(ConvShape), _vp, _vp, _vp, _vp, _vp]),
     "tmq_ternary_dwconv2d": (_int, [_vp, ctypes.POINTER(ConvShape), _vp, _vp, _vp, _vp]),
     "tmq_ternary_dwconv_patches": (_int, [_vp, _int, _i64, ctypes.c_int32, _i64, _vp, _vp, _vp]),
     "tmq_maxpool2d_nhwc": (_int, [_vp] + [ctypes.c_int32] * 10 + [_vp, _vp]),
@@ -120,6 +121,9 @@ def load():
             fn.argtypes = args
         _lib = lib
     return _lib
+
+
+ERR_UNSUPPORTED = -2     # TMQ_ERR_UNSUPPORTED
 
 
 def check(status, what):

@@ -625,6 +625,46 @@ def ternary_conv2d(x: torch.Tensor, nw: NativeWeights, stride=1, padding=0, dila
     return y
 
 
+def ternary_conv2d_relu_maxpool(x: torch.Tensor, nw: NativeWeights, stride=1, padding=0, dilation=1, scale=None,
+                                bias=None) -> torch.Tensor:
+    """max_pool2d(relu(ternary_conv2d(x) * scale + bias), 3, 2, 1), the opening of a ResNet. Arguments as
+    ternary_conv2d; the result is fp16 [B, N, Po, Pwo] in channels_last memory. Few-channel inputs with a short
+    reduction (8, 16 or 32 channels, C * ky * kx <= 256, at most 64 output channels in groups of 8) take one
+    kernel that never writes the convolution's output; everything else makes the two calls. Both give the same
+    bits."""
+    pair = lambda v: tuple(v) if isinstance(v, (tuple, list)) else (v, v)
+    (sy, sx), (py, px), (dy, dx) = pair(stride), pair(padding), pair(dilation)
+    (py, py_end), (px, px_end) = pair(py), pair(px)
+    if not x.is_cuda or x.dim() != 4:
+        raise RuntimeError("ternary_conv2d_relu_maxpool: expected a 4-D GPU tensor")
+    if x.shape[1] != nw.C:
+        raise RuntimeError(f"ternary_conv2d_relu_maxpool: input has {x.shape[1]} channels, weights expect {nw.C}")
+    if x.dtype == torch.float32:
+        x, scale = f32_to_f16_prescaled(x, scale, nw.N)
+    if x.dtype != torch.float16 or not x.is_contiguous(memory_format=torch.channels_last):
+        x = x.to(dtype=torch.float16, memory_format=torch.channels_last)
+    B, C, H, W = x.shape
+    shp = _capi.ConvShape(B, C, H, W, nw.N, nw.ky, nw.kx, sy, sx, py, px, dy, dx, py_end, px_end)
+    ho, wo = ctypes.c_int32(0), ctypes.c_int32(0)
+    lib = _lib()
+    check(lib.tmq_conv2d_out_hw(ctypes.byref(shp), ctypes.byref(ho), ctypes.byref(wo)), "conv2d_out_hw")
+    if ho.value <= 0 or wo.value <= 0:
+        raise RuntimeError("ternary_conv2d_relu_maxpool: empty output")
+    y = torch.empty((B, nw.N, (ho.value - 1) // 2 + 1, (wo.value - 1) // 2 + 1), dtype=torch.float16, device=x.device,
+                    memory_format=torch.channels_last)
+    ep = _epilogue(nw, scale, bias, None, True, torch.float16, y)     # validates scale and bias
+    if B == 0:
+        return y
+    with torch.cuda.device(x.device):
+        status = lib.tmq_ternary_conv2d_relu_maxpool(ptr(x), ctypes.byref(shp), ptr(nw.buf), ep.scale, ep.bias, ptr(y),
+                                                     stream_of(x))
+    if status == _capi.ERR_UNSUPPORTED:
+        full = ternary_conv2d(x, nw, stride, padding, dilation, scale, bias, relu=True, out_dtype=torch.float16)
+        return maxpool2d_nhwc(full, 3, 2, 1)
+    check(status, "ternary_conv2d_relu_maxpool")
+    return y
+
+
 class _Channels:
     """What _epilogue needs to know about a depthwise layer: its channel count."""
     def __init__(self, n):
