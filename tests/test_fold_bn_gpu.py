@@ -88,6 +88,7 @@ def test_fold_resnet_and_explicit_pairs(cuda):
             gm, sites = t.fuse_epilogues(model)
             assert sites == 17
             assert not any(n.op == "call_function" and n.target in (torch.relu, torch.add) for n in gm.graph.nodes)
+            assert "maxpool" not in [n.target for n in gm.graph.nodes if n.op == "call_module"]     # taken into the stem's call
             got16f = gm(x)
         finally:
             t.set_compact_output_dtype(prev)
@@ -163,3 +164,52 @@ def test_fuse_epilogues_patterns(cuda, dtype):
     assert {"e", "f", "g", "bn"} <= set(calls) and not {"a", "b", "c", "d", "head", "act"} & set(calls)
     tol = 2e-3 if dtype == torch.float16 else 1e-5
     assert got.dtype == want.dtype and torch.allclose(got.float(), want.float(), rtol=tol, atol=tol * want.abs().max().item())
+
+
+class _Opening(torch.nn.Module):
+    def __init__(self, pool):
+        super().__init__()
+        nn = torch.nn
+        self.conv1 = nn.Conv2d(3, 64, 7, 2, 3, bias=False)
+        self.bn1 = nn.BatchNorm2d(64)
+        self.relu = nn.ReLU(inplace=True)
+        self.maxpool = pool
+        self.conv2 = nn.Conv2d(64, 16, 1, bias=True)
+
+    def forward(self, x):
+        return self.conv2(self.maxpool(self.relu(self.bn1(self.conv1(x)))))
+
+
+@pytest.mark.parametrize("native_pooling", [False, True])
+def test_fuse_epilogues_takes_the_opening_maxpool(cuda, native_pooling):
+    """maxpool(relu(conv(x))) with a 3 x 3 / 2 / 1 pool becomes one call: the same bits as the separate modules in
+    fp16, PyTorch's pooling as before in fp32; any other pool stays a module of its own."""
+    import tmq_amd as t
+    nn = torch.nn
+    for pool, taken in ((nn.MaxPool2d(3, 2, 1), True), (nn.MaxPool2d(2, 2), False), (nn.MaxPool2d(3, 2, 1, ceil_mode=True), False)):
+        torch.manual_seed(4)
+        net = _Opening(pool)
+        ctrl = t.QuantizationControl(post_scale=True)
+        t.quantize_model(net, ctrl)
+        _randomize_bn(net, torch.Generator().manual_seed(4))
+        net.to(cuda).eval()
+        ctrl.quantize()
+        t.compressed_state_dict(net, strong=False)
+        x = torch.randn(3, 3, 64, 72, device=cuda)
+        with torch.no_grad():
+            t.fold_batchnorm(net)
+            if native_pooling:
+                t.use_native_pooling(net)
+            want32 = net(x)
+            prev = t.set_compact_output_dtype(torch.float16)
+            try:
+                want16 = net(x)
+                gm, sites = t.fuse_epilogues(net)
+                got16 = gm(x)
+            finally:
+                t.set_compact_output_dtype(prev)
+            got32 = gm(x)
+        calls = [n.target for n in gm.graph.nodes if n.op == "call_module"]
+        assert sites == 1 and ("maxpool" in calls) == (not taken)
+        assert got16.dtype == torch.float16 and torch.equal(got16, want16)
+        assert got32.dtype == torch.float32 and torch.allclose(got32, want32, rtol=1e-5, atol=1e-5 * want32.abs().max().item())

@@ -774,14 +774,18 @@ class Conv2d(nn.Module, TMQLayer):
         return self._conv(x, w, self.bias)
 
     @torch.no_grad()
-    def compact_forward(self, x, residual=None, relu=False):
+    def compact_forward(self, x, residual=None, relu=False, pool=False):
         """Implicit-GEMM convolution from the packed weights (replaces the unfold / GEMM / fold
         sequence of tmq/tmq.py:822-871). Output extents follow PyTorch's formula. Returns fp32
         [B, N, Ho, Wo] (channels_last memory); a 3-D input gives a 3-D output.
-        residual / relu: added / applied in the kernel's epilogue (fuse_epilogues)."""
+        residual / relu: added / applied in the kernel's epilogue (fuse_epilogues). pool: a 3 x 3 / stride 2 /
+        pad 1 max-pool follows the ReLU (fp16 output, no residual, groups == 1): one call, and for a network's
+        first layer one kernel."""
         assert not self.training, "Compact inference is not supported in training mode"
         assert self.weight.data.dtype == torch.int32, "Compact inference requires 32-bit integer words"
         self._update_scale()
+        if pool and not (relu and residual is None and self.groups == 1 and x.dim() == 4 and _compact_out == torch.float16):
+            raise RuntimeError("compact_forward(pool=True) needs relu, no residual, groups == 1, a 4-D input and fp16 outputs")
         if x.dim() == 3:
             r3 = residual.unsqueeze(0) if residual is not None else None
             return self.compact_forward(x.unsqueeze(0), r3, relu).squeeze(0)
@@ -812,9 +816,14 @@ class Conv2d(nn.Module, TMQLayer):
                 x, scale = ops.f32_to_f16_prescaled(x, scale, int(self.original_shape[0]))
             xs = ops.nchw_to_nhwc4(x).view(B, H, W // 2, 8).permute(0, 3, 1, 2)
             (sy, _), (py, _) = _pair(self.stride), _pair(self.padding)
+            if pool:
+                return ops.ternary_conv2d_relu_maxpool(xs, nw, (sy, 1), ((py, py), (pl, pr)), 1, scale=scale, bias=bias)
             return ops.ternary_conv2d(xs, nw, (sy, 1), ((py, py), (pl, pr)), 1, scale=scale, bias=bias,
                                       residual=residual, relu=relu, out_dtype=_compact_out)
         nw = self._native_weights(conv_kernel=(ky, kx))
+        if pool:
+            return ops.ternary_conv2d_relu_maxpool(x, nw, _pair(self.stride), _pair(self.padding), _pair(self.dilation),
+                                                   scale=scale, bias=bias)
         return ops.ternary_conv2d(x, nw, _pair(self.stride), _pair(self.padding), _pair(self.dilation), scale=scale,
                                   bias=bias, residual=residual, relu=relu, out_dtype=_compact_out)
 
@@ -1183,15 +1192,22 @@ def fold_batchnorm(module: nn.Module, pairs=None):
 
 
 class _FusedEpilogue(nn.Module):
-    """A compact layer called with its residual input and / or a ReLU in the kernel's epilogue."""
+    """A compact layer called with its residual input and / or a ReLU in the kernel's epilogue; `pool`: the
+    3 x 3 / stride 2 / pad 1 max-pool module that followed the ReLU, taken into the same call when the layer
+    hands on fp16 (set_compact_output_dtype) and applied as it was otherwise."""
 
-    def __init__(self, layer, relu):
+    def __init__(self, layer, relu, pool=None):
         super().__init__()
         self.layer = layer
         self.relu = bool(relu)
+        self.pool = pool
 
     def forward(self, x, residual=None):
-        return self.layer.compact_forward(x, residual, self.relu)
+        if self.pool is None:
+            return self.layer.compact_forward(x, residual, self.relu)
+        if _compact_out == torch.float16 and x.is_cuda and x.dim() == 4:
+            return self.layer.compact_forward(x, None, True, pool=True)
+        return self.pool(self.layer.compact_forward(x, None, True))
 
 
 def fuse_epilogues(model: nn.Module):
@@ -1200,10 +1216,11 @@ def fuse_epilogues(model: nn.Module):
     README.md:150-155). The model is traced with torch.fx (TMQ layers are leaves); recognised are, with any
     number of nn.Identity modules (what fold_batchnorm leaves behind) in between,
 
-        relu(layer(x))      layer(x) + r      relu(layer(x) + r)
+        relu(layer(x))      layer(x) + r      relu(layer(x) + r)      maxpool(relu(conv(x)))
 
     where `relu` is torch.relu / F.relu / x.relu() / an nn.ReLU module, `+` is +, += or torch.add, the
-    layer is a compact Conv2d or Linear without a BatchNorm of its own, and the intermediate values have no
+    layer is a compact Conv2d or Linear without a BatchNorm of its own, `maxpool` is an nn.MaxPool2d(3, 2, 1)
+    module (a ResNet's opening; one kernel once the layers hand on fp16), and the intermediate values have no
     other use. Everything else stays as traced. For inference, after the layers went compact and after
     fold_batchnorm. Returns (GraphModule sharing the model's parameters, number of fused sites)."""
     import operator
@@ -1264,12 +1281,23 @@ def fuse_epilogues(model: nn.Module):
             end, relu = nxt, True
         if end is None:
             continue
+        # relu(conv(x)) handed only to a 3 x 3 / stride 2 / pad 1 max-pool (a ResNet's opening): the pool joins the call
+        pool = None
+        if relu and residual is None and isinstance(layer, Conv2d) and layer.groups == 1:
+            after = only_user(end)
+            if after is not None and after.op == "call_module" and len(after.args) == 1 and after.args[0] is end and not after.kwargs:
+                m = mods.get(after.target)
+                inner = m.inner if isinstance(m, _MaxPool2dNHWC) else m
+                if (isinstance(inner, nn.MaxPool2d) and _pair(inner.kernel_size) == (3, 3) and _pair(inner.stride) == (2, 2)
+                        and _pair(inner.padding) == (1, 1) and _pair(inner.dilation) == (1, 1) and not inner.ceil_mode
+                        and not inner.return_indices):
+                    pool, end = m, after
         name = "_fused_" + node.target.replace(".", "_")
         k = 0
         while hasattr(gm, name + (str(k) if k else "")):
             k += 1
         name += str(k) if k else ""
-        gm.add_submodule(name, _FusedEpilogue(layer, relu))
+        gm.add_submodule(name, _FusedEpilogue(layer, relu, pool))
         with graph.inserting_before(end):
             args = (node.args[0],) if residual is None else (node.args[0], residual)
             new = graph.call_module(name, args)
