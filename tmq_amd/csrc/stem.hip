@@ -41,6 +41,7 @@ struct StemShape {
     int chunks;                  // 16-byte pieces in the window
     int zero_off;                // LDS byte offset of a zeroed copy of the window's extent (behind the window), or 0 if not needed
     int tab_off;                 // LDS byte offset of the table of piece displacements (behind both)
+    int const_off;               // LDS byte offset of scale[64], bias[64] (behind the tile as well)
     int kchunks;                 // 16-byte pieces (8 reduction indices) per output: K / 8
     FastDiv by_tw, by_th, by_kx, by_row;   // patches per image row / column, kernel width, 16-byte pieces per window row
 };
@@ -48,7 +49,7 @@ struct StemShape {
 template <int WM, int WN>
 __global__ __launch_bounds__(kThreads, 3) void stem_pool_kernel(StemShape p, const uint32_t *__restrict__ native, int N,
                                                                 const float *__restrict__ scale, const float *__restrict__ bias,
-                                                                _Float16 *__restrict__ y, int tiles, int vec) {
+                                                                _Float16 *__restrict__ y, int tiles) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     const int tid = threadIdx.x, lane = tid & 63, wv = __builtin_amdgcn_readfirstlane(tid >> 6);
     constexpr int WGN = 4 / WN, D = WM / 2;          // wavefronts side by side; how many row fragments ahead the operand reads run
@@ -104,6 +105,13 @@ __global__ __launch_bounds__(kThreads, 3) void stem_pool_kernel(StemShape p, con
         const int d = ((((i * p.dy) * p.PC + j * p.dx) << (p.cshift - 3)) + (tid & sub_mask)) * 16;
         *reinterpret_cast<int *>(lds + p.tab_off + tid * 4) = tid < p.kchunks ? d : p.zero_off;
     }
+    // Per-channel scale (the weight unit folded in) and bias go through a table behind everything else in LDS: the
+    // trip to memory ends while the window is on its way, where a load in the epilogue would make every wavefront wait.
+    float *const constants = reinterpret_cast<float *>(lds + p.const_off);
+    if (tid < 64) {
+        constants[tid] = (tid < N && scale ? scale[tid] : 1.f) * (1.0f / kWeightUnit);
+        constants[64 + tid] = tid < N && bias ? bias[tid] : 0.f;
+    }
     const int S = (p.kchunks + 3) >> 2;
 
     floatx4 acc[WM][WN];
@@ -141,28 +149,14 @@ __global__ __launch_bounds__(kThreads, 3) void stem_pool_kernel(StemShape p, con
             disp = disp_next;
         }
     }
-    // Scale (the weight unit folded in) and bias of the lane's channels: with the weights as the first MFMA operand an
-    // accumulator holds channels 4 g .. 4 g + 3 of its 16-channel block at position r16 of its row fragment, four
-    // neighbours of a tile row.
+    // Scale and bias of the lane's channels, out of the table: with the weights as the first MFMA operand an accumulator
+    // holds channels 4 g .. 4 g + 3 of its 16-channel block at position r16 of its row fragment, four neighbours of a
+    // tile row.
     floatx4 sc[WN], bi[WN];
 #pragma unroll
     for (int j = 0; j < WN; j++) {
-        const int n = (wn * WN + j) * 16 + g * 4;
-        sc[j] = floatx4{1.f, 1.f, 1.f, 1.f};
-        bi[j] = floatx4{0.f, 0.f, 0.f, 0.f};
-        if (n < N) {                                 // N is a multiple of 8: all four or none
-            if (vec) {
-                if (scale) sc[j] = *reinterpret_cast<const floatx4 *>(scale + n);
-                if (bias) bi[j] = *reinterpret_cast<const floatx4 *>(bias + n);
-            } else {
-#pragma unroll
-                for (int r = 0; r < 4; r++) {
-                    if (scale) sc[j][r] = scale[n + r];
-                    if (bias) bi[j][r] = bias[n + r];
-                }
-            }
-        }
-        sc[j] *= 1.0f / kWeightUnit;
+        sc[j] = *reinterpret_cast<const floatx4 *>(constants + (wn * WN + j) * 16 + g * 4);
+        bi[j] = *reinterpret_cast<const floatx4 *>(constants + 64 + (wn * WN + j) * 16 + g * 4);
     }
     __syncthreads();                                // everybody is done with the window: the tile goes over it
 
@@ -245,7 +239,7 @@ int tmq_ternary_conv2d_relu_maxpool(const void *x, const tmq_conv_shape *s, cons
     const int64_t chunks = PR * PC * (s->C / 8), padded = (chunks + kThreads - 1) / kThreads * kThreads;
     const bool ragged = (K / 8) % 4 != 0;                 // the last MFMA step reaches past K
     const int64_t lds_window = padded * 16 + (ragged ? chunks * 16 : 0) + 32 * 4;   // window, zeros, displacement table
-    if (lds_window > kMaxLds) return TMQ_ERR_UNSUPPORTED;
+    if (lds_window + 128 * 4 > kMaxLds) return TMQ_ERR_UNSUPPORTED;
     p.PC = (int)PC;
     p.chunks = (int)chunks;
     p.zero_off = ragged ? (int)(padded * 16) : 0;
@@ -259,10 +253,10 @@ int tmq_ternary_conv2d_relu_maxpool(const void *x, const tmq_conv_shape *s, cons
     const int64_t tiles = (int64_t)s->B * th * tw;
     if (tiles > (int64_t)0x7FFFFFFF) return TMQ_ERR_TOO_LARGE;
     if (tiles == 0) return TMQ_OK;
-    const size_t lds = (size_t)(lds_window > kTileBytes ? lds_window : kTileBytes);
+    p.const_off = (int)(lds_window > kTileBytes ? lds_window : kTileBytes);
+    const size_t lds = (size_t)p.const_off + 128 * 4;
     hipLaunchKernelGGL((stem_pool_kernel<4, 4>), dim3((uint32_t)tiles), dim3(kThreads), lds, as_stream(stream), p,
-                       static_cast<const uint32_t *>(native), (int)s->N, scale, bias, static_cast<_Float16 *>(y), (int)tiles,
-                       (int)(aligned16(scale) && aligned16(bias)));
+                       static_cast<const uint32_t *>(native), (int)s->N, scale, bias, static_cast<_Float16 *>(y), (int)tiles);
     return check_launch();
 }
 
