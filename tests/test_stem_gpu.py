@@ -1,6 +1,7 @@
 """The fused network opening (ternary convolution -> scale / bias -> ReLU -> 3 x 3 / 2 max-pool in one kernel)
 through the C ABI. The bar is bit equality with the two separate entry points, which the convolution and
-pooling tests tie to the oracle and to PyTorch; on small integers also with PyTorch's own fp32 ops."""
+pooling tests tie to the oracle and to PyTorch; on small integers also with PyTorch's own fp32 ops, and directly
+against the oracle's convolution followed by a window maximum in numpy."""
 import pytest
 import torch
 import torch.nn.functional as F
@@ -52,6 +53,39 @@ def test_optional_scale_and_bias(cuda, with_scale, with_bias):
     ops, x, nw, scale, bias, _ = _case(cuda, 2, 8, 40, 26, 64, (7, 4), (2, 1), ((3, 3), (2, 1)), (1, 1), 5, with_scale, with_bias)
     want = ops.maxpool2d_nhwc(ops.ternary_conv2d(x, nw, (2, 1), ((3, 3), (2, 1)), 1, scale, bias, relu=True, out_dtype=torch.float16), 3, 2, 1)
     assert torch.equal(ops.ternary_conv2d_relu_maxpool(x, nw, (2, 1), ((3, 3), (2, 1)), 1, scale, bias), want)
+
+
+@pytest.mark.parametrize("B,C,H,W,N,k,stride,pad", [(2, 8, 37, 26, 64, (7, 4), (2, 1), ((3, 3), (2, 1))), (3, 16, 19, 23, 24, (3, 3), (1, 1), (1, 1))])
+def test_fused_opening_against_the_oracle(cuda, oracle, B, C, H, W, N, k, stride, pad):
+    """Against the CPU restatement: the oracle's convolution (fp32 accumulation over the reference's compact words),
+    then ReLU and a window maximum in numpy. The fused kernel rounds the convolution's value to fp16 before the
+    maximum, hence the fp16 tolerance; the maximum itself is exact."""
+    import numpy as np
+    from tmq_amd import ops
+    rng = np.random.default_rng(B + C + H + N)
+    Wt = rng.integers(-1, 2, (N, C, k[0], k[1])).astype(np.float32)
+    words = oracle.pack(Wt.reshape(N, -1))
+    x = rng.standard_normal((B, C, H, W)).astype(np.float16)
+    scale = ((0.5 + rng.random(N)) * 0.1).astype(np.float32)
+    bias = rng.standard_normal(N).astype(np.float32)
+    if isinstance(pad[0], tuple):
+        # the oracle pads symmetrically: hand it the explicitly padded image
+        xp = np.pad(x, ((0, 0), (0, 0), pad[0], pad[1]))
+        conv = oracle.conv2d(xp.astype(np.float32), words, N, k, stride, (0, 0), (1, 1), scale, bias)
+    else:
+        conv = oracle.conv2d(x.astype(np.float32), words, N, k, stride, pad, (1, 1), scale, bias)
+    act = np.maximum(conv, 0)
+    Ho, Wo = act.shape[2:]
+    padded = np.full((B, N, Ho + 2, Wo + 2), -np.inf, dtype=np.float32)
+    padded[:, :, 1:-1, 1:-1] = act
+    Po, Pwo = (Ho - 1) // 2 + 1, (Wo - 1) // 2 + 1
+    want = np.stack([padded[:, :, i:i + 2 * Po:2, j:j + 2 * Pwo:2] for i in range(3) for j in range(3)]).max(axis=0)
+    nw = ops.NativeWeights(ops.compactify_ternary(torch.from_numpy(Wt).to(cuda)), N, conv_kernel=k)
+    got = ops.ternary_conv2d_relu_maxpool(torch.from_numpy(x).to(cuda), nw, stride, pad, 1, torch.from_numpy(scale).to(cuda),
+                                          torch.from_numpy(bias).to(cuda))
+    assert tuple(got.shape) == want.shape
+    err = np.abs(got.float().cpu().numpy() - want).max() / np.abs(want).max()
+    assert err <= 1e-3, err
 
 
 def test_small_integers_against_torch(cuda):
