@@ -965,6 +965,16 @@ int dispatch(const Rows &rows, const void *native, int64_t M, int64_t K, int64_t
     // one over 64 x 64 tiles with eight wavefronts; both run one workgroup per CU. They win when they
     // save a whole pass: M = 512 at K = N = 4096 27.5 -> 23.9 us, the 512-channel 7 x 7 convolutions
     // of ResNet-18 33 -> 29.6 us; with a single pass of 64 x 64 tiles (M = 256) they lose.
+    // Convolutions with a long reduction over one to two 64 x 64 tiles per CU: four wavefronts per tile, single pairs,
+    // so that two workgroups share a CU (eight wavefronts with their double buffers fill its LDS alone) -- all tiles
+    // are resident at once and a CU's second workgroup fills the gaps that the im2col address arithmetic leaves in the
+    // first: the 512-channel 7 x 7 convolutions of ResNet-18 at batch 64 29.3 -> 26.6 us against the 64 x 128 tiles
+    // below, 256 -> 512 channels at stride 2 18.5 -> 16.7, 1024 -> 512 channels 47.8 -> 43.8 (whole weight blocks per
+    // wavefront lose here: 61 us). Dense problems of these sizes stay as they are (M = 512 at K = N = 4096: 24.0 us on
+    // 64 x 128 tiles, 27.6 this way), and so do convolutions with fewer tiles (98 tiles: 27 us on smaller tiles, 56 so).
+    constexpr bool kConv = Rows::kBuffer;
+    if (kConv && npairs >= 16 && ((M + 63) / 64) * tn >= 256 && ((M + 63) / 64) * tn <= 512)
+        return launch<4, 4, 4, Rows>(rows, native, M, K, N, ep, stream);
     {
         const int64_t tm = (M + 63) / 64, passes64 = (tm * tn + 255) / 256, passes128 = (tm * ((N + 127) / 128) + 255) / 256;
         if (npairs >= 16 && passes64 >= 2 && 17 * passes128 < 10 * passes64)
