@@ -145,6 +145,8 @@ CONV_CASES = [  # B, C, H, W, N, k, stride, pad, dil
     # 129 .. 256 output channels over at least 8192 output positions: 64 x 256 tiles, eight wavefronts, loads between
     # the MFMAs (18 k-tiles + none / 2 k-tiles only / ragged channels, stride 2 and a ragged last row tile)
     (8, 128, 32, 32, 256, 3, 1, 1, 1), (8, 128, 32, 32, 256, 1, 1, 0, 1), (9, 64, 61, 63, 200, 3, 2, 1, 1),
+    # split reduction over 256 .. 512 tiles of 64 x 64 with K >= 1024: four wavefronts per tile, two workgroups per CU
+    (16, 128, 32, 32, 64, 3, 1, 1, 1), (15, 192, 23, 25, 100, 3, 1, 1, 1),
 ]
 
 
