@@ -412,7 +412,8 @@ def bench_resnet_infer(args, torch):
                            ("drop_in_bn_folded", lambda: model(x), max(3, args.steps // 4)),
                            ("drop_in_bn_folded_fp16", lambda: model(x), max(3, args.steps // 4)),
                            ("drop_in_bn_folded_fp16_pooling", lambda: model(x), max(3, args.steps // 4)),
-                           ("drop_in_fused_graph", lambda: graph[0](x), max(3, args.steps // 4))):
+                           ("drop_in_fused_graph", lambda: graph[0](x), max(3, args.steps // 4)),
+                           ("drop_in_fused_graph_replayed", lambda: graph[1](x), args.steps)):
         if name == "drop_in_bn_folded":
             t.fold_batchnorm(model)                           # BatchNorm into the convolutions' epilogues
         if name == "drop_in_bn_folded_fp16":
@@ -421,6 +422,8 @@ def bench_resnet_infer(args, torch):
             t.use_native_pooling(model)                       # the library's fp16 NHWC max-pool / average pool
         if name == "drop_in_fused_graph":
             graph[0] = t.fuse_epilogues(model)[0]             # ReLU / residual add into the kernels' epilogues (torch.fx)
+        if name == "drop_in_fused_graph_replayed":
+            graph.append(t.GraphedForward(graph[0]))          # ... and the whole forward recorded as one HIP graph
         with torch.no_grad():
             for _ in range(max(2, args.warmup // 4)):
                 fn()

@@ -213,3 +213,38 @@ def test_fuse_epilogues_takes_the_opening_maxpool(cuda, native_pooling):
         assert sites == 1 and ("maxpool" in calls) == (not taken)
         assert got16.dtype == torch.float16 and torch.equal(got16, want16)
         assert got32.dtype == torch.float32 and torch.allclose(got32, want32, rtol=1e-5, atol=1e-5 * want32.abs().max().item())
+
+
+def test_graphed_forward_replays_equal_eager(cuda):
+    """The fused inference graph of a small network recorded as a HIP graph: every replay, with eager work and
+    synchronisations in between and with new inputs, gives the eager result; a second input shape records its own
+    graph."""
+    import tmq_amd as t
+    torch.manual_seed(6)
+    net = _Opening(torch.nn.MaxPool2d(3, 2, 1))
+    ctrl = t.QuantizationControl(post_scale=True)
+    t.quantize_model(net, ctrl)
+    _randomize_bn(net, torch.Generator().manual_seed(6))
+    net.to(cuda).eval()
+    ctrl.quantize()
+    t.compressed_state_dict(net, strong=False)
+    prev = t.set_compact_output_dtype(torch.float16)
+    try:
+        with torch.no_grad():
+            t.fold_batchnorm(net)
+            t.use_native_pooling(net)
+            gm, _ = t.fuse_epilogues(net)
+            graphed = t.GraphedForward(gm)
+            for rep in range(4):
+                x = torch.randn(3, 3, 64, 72, device=cuda).half()
+                want = gm(x)
+                torch.cuda.synchronize()
+                got = graphed(x)
+                assert torch.equal(got, want), rep
+                _ = gm(torch.randn(2, 3, 32, 40, device=cuda).half())        # eager work between the replays
+            x2 = torch.randn(1, 3, 48, 48, device=cuda).half()
+            assert torch.equal(graphed(x2), gm(x2)) and len(graphed._graphs) == 2
+            with pytest.raises(RuntimeError):
+                graphed(x2.cpu())
+    finally:
+        t.set_compact_output_dtype(prev)

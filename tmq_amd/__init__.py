@@ -5,5 +5,5 @@
 from .tmq import *  # noqa: F401,F403
 from .tmq import (QuantMode, TensorType, QuantizationScheduleBuilder, QuantizationControl, SoftStep,  # noqa: F401
                   SoftStepDerivative, TMQLayer, Linear, Conv2d, ConvTranspose2d, quantize_weights, quantize_model,
-                  compressed_state_dict, prepare_compressed_load, load_compressed_state_dict, expand_compact_layers, fold_batchnorm, set_compact_output_dtype, use_native_pooling, fuse_epilogues,
+                  compressed_state_dict, prepare_compressed_load, load_compressed_state_dict, expand_compact_layers, fold_batchnorm, set_compact_output_dtype, use_native_pooling, fuse_epilogues, GraphedForward,
                   CUDA_EXT_AVAILABLE, NATIVE_EXT_AVAILABLE)
