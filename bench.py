@@ -60,17 +60,18 @@ def timed_cpu(torch, fn, threads, budget_s, min_reps=3, max_reps=15):
 BYTES_PER_ELEM = 20                                        # load w, g; store y, dw, clamp(w)
 
 
-def measured_traffic(path, n, default_n=1 << 26):
-    """HBM bytes per launch of the dominant kernel as measured with rocprofv3 --pmc FETCH_SIZE /
-    WRITE_SIZE (scaled by a copy of known size); the figure lives in the committed profile summary.
-    Only valid for the workload size it was measured at."""
+def measured_traffic(path, n=1 << 26, default_n=1 << 26, key="traffic_bytes"):
+    """HBM bytes per launch of a kernel as measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs,
+    each scaled by what the same counter reads for a plain copy of known size). Counters cannot be read from
+    inside a timed run, so the figure comes from the committed profile summary of the same workload (a line
+    `<key>: <bytes>`), and is only handed out for the workload size it was measured at."""
     try:
         if n != default_n:
             return None
         for line in open(os.path.join(ROOT, "profiles", path)):
-            if line.startswith("traffic_bytes:"):
-                return int(line.split(":")[1])
-    except OSError:
+            if line.startswith(key + ":"):
+                return int(line.split(":")[1].split()[0])
+    except (OSError, ValueError):
         pass
     return None
 
@@ -226,19 +227,24 @@ def bench_linear(args, torch):
     if "4096" in out:
         o = out["4096"]
         res["roofline"] = {"bound": "mfma", "achieved": o["tflops"], "peak": MFMA_FP16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                           "frac": o["frac_mfma_fp16"], "traffic": None, "algorithmic_flops": 2.0 * 4096 * N * K,
+                           "frac": o["frac_mfma_fp16"],
+                           "traffic": measured_traffic("ternary_linear_k4096_n4096.md", key="traffic_bytes_m4096"),
+                           "algorithmic_bytes": int(K * N / 4 + 2 * 4096 * K + 4 * 4096 * N + 4 * N),
+                           "algorithmic_flops": 2.0 * 4096 * N * K,
                            "kernel": "tile_solo_kernel<128 x 512> (M = 4096)", "avg_launch_us": o["us"]}
     if "1" in out:
         o = out["1"]
         res["roofline_gemv"] = {"bound": "hbm", "achieved": o["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                                "frac": o["frac_hbm"], "traffic": None,
+                                "frac": o["frac_hbm"],
+                                "traffic": measured_traffic("ternary_linear_k4096_n4096.md", key="traffic_bytes_gemv_4096"),
                                 "algorithmic_bytes": int(K * N / 4 + 2 * K + 8 * N),
                                 "kernel": "gemv8_kernel (M = 1, fp8 x bf8 MFMA), %d rotating weight buffers" % nrot,
                                 "avg_launch_us": o["us"]}
     if "gemv_16384" in extra:
         o = extra["gemv_16384"]
         res["roofline_gemv_16384"] = {"bound": "hbm", "achieved": o["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                                      "frac": o["frac_hbm"], "traffic": None,
+                                      "frac": o["frac_hbm"],
+                                      "traffic": measured_traffic("ternary_linear_k4096_n4096.md", key="traffic_bytes_gemv_16384"),
                                       "algorithmic_bytes": int(16384 * 16384 / 4 + 2 * 16384 + 8 * 16384),
                                       "kernel": "gemv8_kernel (M = 1, K = N = 16384, fp8 x bf8 MFMA), 6 rotating weight buffers",
                                       "avg_launch_us": o["us"]}
@@ -386,69 +392,134 @@ def bench_pack(args, torch):
         res[name] = {"us": round(us, 3), "gbs": round(byts / us / 1e3, 1)}
         res["roofline" if name == "pack" else "roofline_unpack"] = {
             "bound": "hbm", "achieved": round(byts / us / 1e3, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": round(byts / us / 1e3 / HBM_PEAK_GBS, 4), "traffic": None, "algorithmic_bytes": int(byts),
+            "frac": round(byts / us / 1e3 / HBM_PEAK_GBS, 4),
+            "traffic": measured_traffic("pack_4096.md", key="traffic_bytes_" + name), "algorithmic_bytes": int(byts),
             "kernel": ("pack_wide_kernel<float, 4>" if name == "pack" else "unpack_wide_kernel<8>"), "avg_launch_us": round(us, 3)}
     res["value"] = res["pack"]["gbs"]
+    if not args.no_cpu:
+        res["cpu_baseline"] = cpu_baseline_pack(torch, N, K)
     return res
 
 
-def bench_resnet_infer(args, torch):
-    """BASELINE configs[3]: ResNet-18 (102 classes) ternary inference, batch 64 of 3x224x224 fp16."""
+def cpu_baseline_pack(torch, N, K):
+    """The reference's packer on the host: compactify_ternary of tmq/tmq_native.cpp:418-425 (a scalar double
+    loop, matrixTo2BitTernary 152-171) from the reference's own file compiled under oracle/_ref when that
+    library is in the tree ("reference"), else the C restatement of the same loop in oracle/ ("port"). One
+    host thread (the loop has no parallel form), the whole 4096 x 4096 matrix, GB/s on the same 4.25 B/weight."""
+    import importlib.util
+    gen = torch.Generator(device="cpu").manual_seed(10)
+    W = torch.randint(-1, 2, (N, K), generator=gen).float()
+    so = os.path.join(ROOT, "oracle", "_ref", "tmq_native.so")
+    kind, fn = "port", None
+    if os.path.exists(so):
+        try:
+            spec = importlib.util.spec_from_file_location("tmq_native", so)
+            mod = importlib.util.module_from_spec(spec)
+            spec.loader.exec_module(mod)
+            kind, fn = "reference", (lambda: mod.compactify_ternary(W))
+        except (ImportError, OSError):
+            fn = None
+    if fn is None:
+        from tests import oracle_lib
+        Wn = W.numpy()
+        fn = lambda: oracle_lib.pack(Wn)
+    t, reps = timed_cpu(torch, fn, 1, 6.0)
+    return {"value": round(N * K * 4.25 / t / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": kind, "cpu": cpu_model(),
+            "ms": round(t * 1e3, 2),
+            "sample": f"compactify_ternary of the whole {N} x {K} fp32 matrix, one thread, {reps} reps, median"}
+
+
+def _resnet_for_inference(torch, dev, calibrated):
+    """ResNet-18 / 102 classes with i.i.d. ternary weights (P(0) = .5), every layer switched to compact weights.
+    calibrated=False: BatchNorm exactly as BASELINE configs[3] words it (running_mean ~ N(0, 0.1), running_var ~
+    U(0.5, 2), gamma 1, beta 0). calibrated=True: BatchNorm statistics taken from the batch, so that the
+    activations are finite and of order one in every layer (bench_models.calibrate_batchnorm_)."""
     import tmq_amd as t
-    from bench_models import ResNet18, randomize_ternary_, FusedTernaryResNet18
-    dev = torch.device("cuda:0")
+    from bench_models import ResNet18, randomize_ternary_, calibrate_batchnorm_
     torch.manual_seed(20)
     model = ResNet18(102)
-    ctrl = t.QuantizationControl()
-    t.quantize_model(model, ctrl)
+    t.quantize_model(model, t.QuantizationControl())
     randomize_ternary_(model, torch.Generator().manual_seed(20))
-    model.to(dev).eval()
+    model.to(dev)
+    if calibrated:
+        xc = torch.randn(8, 3, 224, 224, generator=torch.Generator().manual_seed(20)).half().to(dev)
+        calibrate_batchnorm_(model, xc, torch.Generator().manual_seed(21))
+    model.eval()
     t.compressed_state_dict(model, strong=False)              # switches every layer to compact weights
+    return model
+
+
+def bench_resnet_infer(args, torch):
+    """BASELINE configs[3]: ResNet-18 (102 classes) ternary inference, batch 64 of 3x224x224 fp16.
+
+    Two networks are timed. `value` / `modes` are the configuration as BASELINE words it. With unscaled ternary
+    weights and running_var ~ U(0.5, 2) every 3 x 3 convolution multiplies the activation scale by ~17, so from
+    the end of layer1 on its fp16 activations are Inf / NaN (`output_finite` false): the kernels do all the work,
+    but on degenerate data. `calibrated` is the same network with BatchNorm statistics taken from the batch
+    (finite activations of order one in every layer, `output_finite` true); it is the figure to compare kernels by."""
+    import tmq_amd as t
+    dev = torch.device("cuda:0")
     B = args.batch or 64
     x = torch.randn(B, 3, 224, 224, generator=torch.Generator().manual_seed(20)).half().to(dev)
-    fused = FusedTernaryResNet18(model)
-    out, graph = {}, [None]
-    for name, fn, reps in (("fused", lambda: fused(x), args.steps), ("drop_in", lambda: model(x), max(3, args.steps // 4)),
-                           ("drop_in_bn_folded", lambda: model(x), max(3, args.steps // 4)),
-                           ("drop_in_bn_folded_fp16", lambda: model(x), max(3, args.steps // 4)),
-                           ("drop_in_bn_folded_fp16_pooling", lambda: model(x), max(3, args.steps // 4)),
-                           ("drop_in_fused_graph", lambda: graph[0](x), max(3, args.steps // 4)),
-                           ("drop_in_fused_graph_replayed", lambda: graph[1](x), args.steps)):
-        if name == "drop_in_bn_folded":
-            t.fold_batchnorm(model)                           # BatchNorm into the convolutions' epilogues
-        if name == "drop_in_bn_folded_fp16":
-            t.set_compact_output_dtype(torch.float16)         # fp16 channels_last between the layers
-        if name == "drop_in_bn_folded_fp16_pooling":
-            t.use_native_pooling(model)                       # the library's fp16 NHWC max-pool / average pool
-        if name == "drop_in_fused_graph":
-            graph[0] = t.fuse_epilogues(model)[0]             # ReLU / residual add into the kernels' epilogues (torch.fx)
-        if name == "drop_in_fused_graph_replayed":
-            graph.append(t.GraphedForward(graph[0]))          # ... and the whole forward recorded as one HIP graph
+
+    def timed(fn, reps):
         with torch.no_grad():
             for _ in range(max(2, args.warmup // 4)):
-                fn()
+                out = fn()
             torch.cuda.synchronize()
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             t0 = time.perf_counter()
             e0.record()
             for _ in range(reps):
-                fn()
+                out = fn()
             e1.record()
             torch.cuda.synchronize()
         dt = (time.perf_counter() - t0) / reps
-        out[name] = {"ms": round(dt * 1e3, 4), "gpu_ms": round(e0.elapsed_time(e1) / reps, 4), "img_s": round(B / dt, 1),
-                     "tflops": round(3.627e9 * B / dt / 1e12, 2)}
-    t.set_compact_output_dtype(torch.float32)
+        finite = bool(torch.isfinite(out.float()).all().item())     # after the timed loop, not inside it
+        return {"ms": round(dt * 1e3, 4), "gpu_ms": round(e0.elapsed_time(e1) / reps, 4), "img_s": round(B / dt, 1),
+                "tflops": round(3.627e9 * B / dt / 1e12, 2), "output_finite": finite}
+
+    few = max(3, args.steps // 4)
+    # ---- the configuration as worded
+    model = _resnet_for_inference(torch, dev, calibrated=False)
+    runner = t.ResNetRunner(model)
+    out = {"fused": timed(lambda: runner(x), args.steps)}
+    out["drop_in"] = timed(lambda: model(x), few)
+    t.fold_batchnorm(model)                                   # BatchNorm into the convolutions' epilogues
+    out["drop_in_bn_folded"] = timed(lambda: model(x), few)
+    prev = t.set_compact_output_dtype(torch.float16)          # fp16 channels_last between the layers
+    try:
+        out["drop_in_bn_folded_fp16"] = timed(lambda: model(x), few)
+        t.use_native_pooling(model)                           # the library's fp16 NHWC max-pool / average pool
+        out["drop_in_bn_folded_fp16_pooling"] = timed(lambda: model(x), few)
+        gm = t.fuse_epilogues(model)[0]                       # ReLU / residual add into the kernels' epilogues (torch.fx)
+        out["drop_in_fused_graph"] = timed(lambda: gm(x), few)
+        replay = t.GraphedForward(gm)                         # ... and the whole forward recorded as one HIP graph
+        out["drop_in_fused_graph_replayed"] = timed(lambda: replay(x), args.steps)
+    finally:
+        t.set_compact_output_dtype(prev)
+    del model, gm, replay
+    # ---- the same network with finite activations
+    model = _resnet_for_inference(torch, dev, calibrated=True)
+    runner = t.ResNetRunner(model)
+    cal = {"fused": timed(lambda: runner(x), args.steps)}
+    session = t.optimize_for_inference(model)                 # fold + fp16 + pooling + fx fusion + HIP graph in one call
+    cal["optimize_for_inference"] = timed(lambda: session(x), args.steps)
     best = max(out, key=lambda k: out[k]["img_s"])
+    f = cal["fused"]
     res = {"metric": "ResNet-18 img/s", "value": out["fused"]["img_s"], "unit": "img/s", "n_gpus": 1, "dtype": "f16",
            "data": "synthetic", "config": {"workload": "configs[3]: ResNet-18/102 ternary inference", "batch": B},
-           "modes": out,
-           "roofline": {"bound": "mfma", "achieved": out["fused"]["tflops"], "peak": MFMA_FP16_PEAK_TFLOPS,
-                        "unit": "TFLOP/s", "frac": round(out["fused"]["tflops"] / MFMA_FP16_PEAK_TFLOPS, 4), "traffic": None,
+           "output_finite": out["fused"]["output_finite"],
+           "note": "value: BatchNorm statistics as BASELINE words them -- fp16 activations overflow after layer1, so most "
+                   "convolutions multiply Inf / NaN; `calibrated`: the same network with BatchNorm statistics from the "
+                   "batch, finite activations in every layer",
+           "modes": out, "calibrated": cal, "value_calibrated": f["img_s"],
+           "roofline": {"bound": "mfma", "achieved": f["tflops"], "peak": MFMA_FP16_PEAK_TFLOPS,
+                        "unit": "TFLOP/s", "frac": round(f["tflops"] / MFMA_FP16_PEAK_TFLOPS, 4), "traffic": None,
                         "algorithmic_flops": 3.627e9 * B,
-                        "kernel": "whole forward of the fused runner: 20 ternary implicit-GEMM convolutions, fc, pooling, "
-                                  "input repack (22 launches)",
-                        "avg_launch_us": round(out["fused"]["gpu_ms"] * 1e3, 2)},
+                        "kernel": "whole forward of tmq_amd.ResNetRunner on the calibrated network (finite activations): 20 "
+                                  "ternary implicit-GEMM convolutions, fc, pooling, input repack (22 launches)",
+                        "avg_launch_us": round(f["gpu_ms"] * 1e3, 2)},
            "fastest_mode": best}
     if not args.no_cpu:
         res["cpu_baseline"] = cpu_baseline_resnet(torch)
@@ -611,7 +682,8 @@ def main():
         res = bench_softstep(args, torch)
         torch.cuda.empty_cache()
         res["also"] = {}
-        for name, leg in (("linear", bench_linear), ("resnet_infer", bench_resnet_infer), ("resnet_qat", bench_resnet_qat)):
+        for name, leg in (("linear", bench_linear), ("pack", bench_pack), ("resnet_infer", bench_resnet_infer),
+                          ("resnet_qat", bench_resnet_qat)):
             res["also"][name] = leg(args, torch)
             torch.cuda.empty_cache()
     elif args.workload == "softstep":

@@ -85,7 +85,7 @@ def _faithful_reference(model, x):
 
 def _calibrated_resnet(cuda, batch):
     import tmq_amd as t
-    from bench_models import ResNet18, randomize_ternary_
+    from bench_models import ResNet18, randomize_ternary_, calibrate_batchnorm_
     torch.manual_seed(20)
     model = ResNet18(102)
     ctrl = t.QuantizationControl()
@@ -95,18 +95,7 @@ def _calibrated_resnet(cuda, batch):
     x = torch.randn(batch, 3, 224, 224, generator=torch.Generator().manual_seed(20)).half().to(cuda)
     # Unscaled ternary weights multiply the activation scale by ~sqrt(fan_in / 2) per layer: set the BatchNorm
     # statistics from the batch so that activations stay O(1) in fp16, and give the affine part some life.
-    for m in model.modules():
-        if isinstance(m, nn.BatchNorm2d):
-            m.momentum = 1.0
-    model.train()
-    with torch.no_grad():
-        model(x[:8].float())
-        g = torch.Generator().manual_seed(21)
-        for m in model.modules():
-            if isinstance(m, nn.BatchNorm2d):
-                m.weight.copy_((0.75 + 0.5 * torch.rand(m.num_features, generator=g)).to(cuda))
-                m.bias.copy_((0.2 * torch.randn(m.num_features, generator=g)).to(cuda))
-        model.fc.bias.copy_((0.1 * torch.randn(102, generator=g)).to(cuda))
+    calibrate_batchnorm_(model, x[:8], torch.Generator().manual_seed(21))
     model.eval()
     return t, model, x
 

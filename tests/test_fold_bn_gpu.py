@@ -248,3 +248,91 @@ def test_graphed_forward_replays_equal_eager(cuda):
                 graphed(x2.cpu())
     finally:
         t.set_compact_output_dtype(prev)
+
+
+def test_graphed_forward_follows_changed_weights(cuda):
+    """A recorded graph replays raw addresses of the layers' native weight buffers: after the weights of a layer
+    were replaced (load_state_dict and its like rebuild those buffers) the next call must record anew and give the
+    eager result of the new weights; reset() does the same on request; so does a changed output dtype."""
+    import tmq_amd as t
+    torch.manual_seed(7)
+
+    def make(seed):
+        torch.manual_seed(seed)
+        net = _Opening(torch.nn.MaxPool2d(3, 2, 1))
+        ctrl = t.QuantizationControl(post_scale=True)
+        t.quantize_model(net, ctrl)
+        _randomize_bn(net, torch.Generator().manual_seed(6))
+        net.to(cuda).eval()
+        ctrl.quantize()
+        return net
+
+    net, other = make(7), make(8)
+    sd_other = t.compressed_state_dict(other, strong=False)
+    t.compressed_state_dict(net, strong=False)
+    x = torch.randn(2, 3, 64, 72, device=cuda).half()
+    prev = t.set_compact_output_dtype(torch.float16)
+    try:
+        with torch.no_grad():
+            graphed = t.GraphedForward(net)
+            first = graphed(x).clone()
+            assert torch.equal(first, net(x))
+            # new weights into the same modules: the compact tensors (and with them the native buffers) are replaced
+            t.load_compressed_state_dict(net, sd_other)
+            junk = [torch.full((1 << 18,), 7, dtype=torch.int32, device=cuda) for _ in range(8)]   # reuse freed memory
+            want = net(x)
+            assert not torch.equal(want, first)
+            got = graphed(x)
+            assert torch.equal(got, want)
+            del junk
+            # a switch the recording depends on
+            t.set_compact_output_dtype(torch.float32)
+            want32 = net(x)
+            got32 = graphed(x)
+            assert got32.dtype == want32.dtype and torch.equal(got32, want32)
+            graphed.reset()
+            assert graphed._graphs == {} and torch.equal(graphed(x), want32)
+    finally:
+        t.set_compact_output_dtype(prev)
+
+
+def test_optimize_for_inference_one_call(cuda):
+    """optimize_for_inference = fold_batchnorm + fp16 hand-over + native pooling + fuse_epilogues + GraphedForward:
+    same values as those steps applied by hand, the global output dtype left as it was, misuse refused."""
+    import tmq_amd as t
+    torch.manual_seed(9)
+
+    def make():
+        torch.manual_seed(9)
+        net = _Opening(torch.nn.MaxPool2d(3, 2, 1))
+        ctrl = t.QuantizationControl(post_scale=True)
+        t.quantize_model(net, ctrl)
+        _randomize_bn(net, torch.Generator().manual_seed(9))
+        net.to(cuda).eval()
+        ctrl.quantize()
+        return net
+
+    net = make()
+    with pytest.raises(RuntimeError):
+        t.optimize_for_inference(net)                            # layers not compact yet
+    t.compressed_state_dict(net, strong=False)
+    by_hand = make()
+    t.compressed_state_dict(by_hand, strong=False)
+    x = torch.randn(3, 3, 64, 72, device=cuda).half()
+    prev = t.set_compact_output_dtype(torch.float16)
+    try:
+        with torch.no_grad():
+            t.fold_batchnorm(by_hand)
+            t.use_native_pooling(by_hand)
+            want = t.fuse_epilogues(by_hand)[0](x)
+    finally:
+        t.set_compact_output_dtype(prev)
+    assert prev == torch.float32
+    session = t.optimize_for_inference(net)
+    assert session.fused_sites >= 1 and len(session.folded) >= 1
+    for _ in range(3):
+        got = session(x)
+        assert torch.equal(got, want)
+    assert t.set_compact_output_dtype(torch.float32) == torch.float32        # untouched outside the call
+    eager = t.optimize_for_inference(net, graph=False)            # idempotent on an already optimised model
+    assert torch.equal(eager(x), want)

@@ -165,3 +165,33 @@ def test_native_weight_cache_follows_the_parameter_version(cuda):
     lin.weight.data.copy_(ops.compactify_ternary(torch.zeros(32, 256, device=cuda)))   # unseen by any counter
     lin.invalidate_native()
     assert torch.equal(lin(x), torch.zeros_like(y1))
+
+
+def test_empty_fp32_batches_give_empty_outputs(cuda):
+    """An fp32 batch without entries returns an empty tensor (as the fp16 path does) instead of failing in the
+    range prescale, for the convolution, the fused opening, the depthwise kernels and the transposed convolution."""
+    import tmq_amd as t
+    from tmq_amd import ops
+    g = torch.Generator().manual_seed(8)
+    for cin, cout, k, stride, groups in ((16, 32, 3, 1, 1), (3, 16, 7, 2, 1), (32, 32, 3, 1, 32)):
+        W = torch.randint(-1, 2, (cout, cin // groups, k, k), generator=g).float()
+        layer = t.Conv2d(cin, cout, k, stride=stride, padding=k // 2, groups=groups, bias=False)
+        layer.weight = torch.nn.Parameter(W.clone())
+        layer.original_shape = W.shape
+        layer.to(cuda).eval()
+        t.compressed_state_dict(torch.nn.Sequential(layer), strong=False)
+        for dtype in (torch.float32, torch.float16):
+            y = layer(torch.empty(0, cin, 16, 16, device=cuda, dtype=dtype))
+            assert y.shape[0] == 0 and y.shape[1] == cout and y.numel() == 0
+    W = torch.randint(-1, 2, (16, 8, 3, 3), generator=g).float()
+    nw = ops.NativeWeights(ops.compactify_ternary(W.to(cuda)), 16, conv_kernel=(3, 3))
+    y = ops.ternary_conv2d_relu_maxpool(torch.empty(0, 8, 16, 16, device=cuda), nw, 1, 1)
+    assert y.shape == (0, 16, 8, 8)
+    net = torch.nn.Sequential(torch.nn.ConvTranspose2d(8, 4, 3, 2, 1, bias=False))
+    ctrl = t.QuantizationControl()
+    t.quantize_model(net, ctrl)
+    net.to(cuda).eval()
+    ctrl.quantize()
+    t.compressed_state_dict(net, strong=False)
+    y = net(torch.empty(0, 8, 6, 6, device=cuda))
+    assert y.shape[0] == 0 and y.shape[1] == 4 and y.numel() == 0

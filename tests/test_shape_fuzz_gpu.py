@@ -1,0 +1,127 @@
+"""Seeded walks over the shapes that decide which kernel family a ternary product takes: single rows and
+few rows (8-bit GEMV, weight stream, short reductions, skinny), mid-size dense products (split reduction,
+tile kernels), convolutions (three loaders, two tile families, the split-reduction form) and the fused
+opening (one kernel or two). Every case is checked against an fp64 product of the same operands
+(a11 / a12: tmq/tmq_cuda.cu:478-549, tmq/tmq.py:662-688, 822-871 compute the same sums in fp32), the fused
+opening bit for bit against the two separate kernels. Each walk stops at its first failure and prints the
+case before it runs it, so that a fault names its shape. About 100 cases per walk, well under a minute in all.
+"""
+import random
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+pytestmark = pytest.mark.gpu
+
+TOL = 2e-5          # observed: <= 3e-6; the contract is 1e-3 relative
+
+
+def _linear_case(ops, dev, i, M, K, N, dt):
+    print("fuzz linear", i, (M, K, N, str(dt)), flush=True)
+    g = torch.Generator(device=dev).manual_seed(1000 + i)
+    W = torch.randint(-1, 2, (N, K), device=dev, generator=g, dtype=torch.int8)
+    nw = ops.NativeWeights(ops.compactify_ternary(W), N)
+    x = torch.randn((M, K), device=dev, generator=g).to(dt)
+    scale = 0.5 + torch.rand(N, device=dev, generator=g)
+    bias = torch.randn(N, device=dev, generator=g)
+    relu = bool(i & 1)
+    y = ops.ternary_linear(x, nw, scale, bias, relu=relu)
+    ref = (x.double() @ W.double().t()) * scale.double() + bias.double()
+    if relu:
+        ref = ref.clamp_min(0)
+    err = ((y.double() - ref).abs().max() / ref.abs().max().clamp_min(1e-30)).item()
+    assert y.shape == ref.shape and err <= TOL, ((M, K, N, dt), err)
+
+
+def test_walk_single_and_few_rows(cuda):
+    from tmq_amd import ops
+    rnd = random.Random(1)
+    for i in range(110):
+        K = rnd.choice([256 * rnd.randint(1, 70), 64 * rnd.randint(1, 300), rnd.randint(1, 20000)])
+        N = rnd.choice([rnd.randint(1, 300), 16 * rnd.randint(1, 700), rnd.randint(1, 12000)])
+        M = 1 if i % 3 else rnd.randint(2, 20)
+        _linear_case(ops, cuda, i, M, K, N, rnd.choice([torch.float16, torch.float32]))
+
+
+def test_walk_mid_size_dense(cuda):
+    from tmq_amd import ops
+    rnd = random.Random(2)
+    for i in range(70):
+        M = rnd.choice([rnd.randint(17, 600), rnd.randint(600, 3300)])
+        K = rnd.choice([64 * rnd.randint(8, 80), 256 * rnd.randint(2, 20), rnd.randint(100, 3000)])
+        N = rnd.choice([128, 130, 256, 1000, 4096, 16 * rnd.randint(8, 300), rnd.randint(129, 5000)])
+        _linear_case(ops, cuda, 500 + i, M, K, N, torch.float16)
+
+
+def test_walk_convolutions(cuda):
+    from tmq_amd import ops
+    rnd = random.Random(3)
+    done = 0
+    for i in range(140):
+        C = rnd.choice([64, 64, 128, 192, 256, 512, 8, 16, 3, 40])
+        k = rnd.choice([1, 3, 3, 3, 5])
+        s = rnd.choice([1, 1, 2])
+        p = rnd.randint(0, k // 2 + 1)
+        N = rnd.choice([16, 64, 100, 128, 200, 256, 384, 512])
+        B = rnd.randint(1, 24)
+        H, W = rnd.randint(k, 40), rnd.randint(k, 40)
+        if B * H * W * C * N * k * k > 3e11:
+            continue
+        desc = (B, C, H, W, N, k, s, p)
+        print("fuzz conv", i, desc, flush=True)
+        g = torch.Generator(device=cuda).manual_seed(2000 + i)
+        Wt = torch.randint(-1, 2, (N, C, k, k), device=cuda, generator=g).float()
+        x = torch.randn((B, C, H, W), device=cuda, generator=g).half()
+        scale = (torch.rand(N, device=cuda, generator=g) + 0.5) * 0.05
+        bias = torch.randn(N, device=cuda, generator=g)
+        nw = ops.NativeWeights(ops.compactify_ternary(Wt), N, conv_kernel=(k, k))
+        res = None
+        if i % 4 == 0:
+            ho, wo = (H + 2 * p - k) // s + 1, (W + 2 * p - k) // s + 1
+            res = torch.randn((B, N, ho, wo), device=cuda, generator=g).contiguous(memory_format=torch.channels_last)
+        y = ops.ternary_conv2d(x, nw, s, p, 1, scale, bias, residual=res, relu=bool(i & 1))
+        ref = F.conv2d(x.double(), Wt.double(), None, s, p) * scale.double().view(1, -1, 1, 1) + bias.double().view(1, -1, 1, 1)
+        if res is not None:
+            ref = ref + res.double()
+        if i & 1:
+            ref = ref.clamp_min(0)
+        err = ((y.double() - ref).abs().max() / ref.abs().max().clamp_min(1e-30)).item()
+        assert y.shape == ref.shape and err <= TOL, (desc, err)
+        done += 1
+    assert done >= 100
+
+
+def test_walk_fused_opening(cuda):
+    from tmq_amd import ops
+    rnd = random.Random(4)
+    for i in range(100):
+        C = rnd.choice([8, 8, 8, 16, 32])
+        while True:
+            ky, kx = rnd.randint(1, 7), rnd.randint(1, 7)
+            if C * ky * kx <= 256 or rnd.random() < 0.05:
+                break
+        sy, sx = rnd.randint(1, 3), rnd.randint(1, 3)
+        dy, dx = rnd.randint(1, 2), rnd.randint(1, 2)
+        pad = ((rnd.randint(0, 3), rnd.randint(0, 3)), (rnd.randint(0, 3), rnd.randint(0, 3)))
+        N = rnd.choice([8, 16, 24, 32, 40, 48, 56, 64])
+        B = rnd.randint(1, 3)
+        H, W = rnd.randint((ky - 1) * dy + 1, 70), rnd.randint((kx - 1) * dx + 1, 70)
+        desc = (B, C, H, W, N, (ky, kx), (sy, sx), pad, (dy, dx))
+        print("fuzz opening", i, desc, flush=True)
+        g = torch.Generator(device=cuda).manual_seed(3000 + i)
+        Wt = torch.randint(-1, 2, (N, C, ky, kx), device=cuda, generator=g).float()
+        x = torch.randn((B, C, H, W), device=cuda, generator=g).half().contiguous(memory_format=torch.channels_last)
+        scale = (torch.rand(N, device=cuda, generator=g) - 0.3) * 0.2
+        bias = torch.randn(N, device=cuda, generator=g)
+        nw = ops.NativeWeights(ops.compactify_ternary(Wt), N, conv_kernel=(ky, kx))
+        full = ops.ternary_conv2d(x, nw, (sy, sx), pad, (dy, dx), scale, bias, relu=True, out_dtype=torch.float16)
+        want = ops.maxpool2d_nhwc(full, 3, 2, 1)
+        got = ops.ternary_conv2d_relu_maxpool(x, nw, (sy, sx), pad, (dy, dx), scale, bias)
+        assert got.shape == want.shape and torch.equal(got, want), desc
+        if i % 10 == 0:
+            ref = F.conv2d(x.double(), Wt.double(), None, (sy, sx), 0, (dy, dx)) if pad == ((0, 0), (0, 0)) else None
+            if ref is not None:
+                ref = (ref * scale.double().view(1, -1, 1, 1) + bias.double().view(1, -1, 1, 1)).clamp_min(0)
+                err = ((full.double() - ref).abs().max() / ref.abs().max().clamp_min(1e-30)).item()
+                assert err <= 2e-3, (desc, err)          # fp16 outputs

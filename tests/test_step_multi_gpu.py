@@ -311,3 +311,66 @@ def test_changed_hardness_or_weights_start_a_new_pass(cuda, oracle):
     with torch.no_grad():
         c = net(x)                                                # inference mode: raw weights, no staircase
     assert torch.isfinite(c).all()
+
+
+class _TwoHeads(nn.Module):
+    """A trunk and two heads of which a forward uses one."""
+
+    def __init__(self):
+        super().__init__()
+        self.trunk = nn.Linear(32, 48)
+        self.head_a = nn.Linear(48, 8)
+        self.head_b = nn.Linear(48, 8)
+
+    def forward(self, x, which):
+        h = torch.relu(self.trunk(x))
+        return self.head_a(h) if which == "a" else self.head_b(h)
+
+
+def test_branches_used_in_alternate_steps_backward_each_step(cuda, oracle):
+    """A registered layer that the previous forward skipped must not be handed that pass's result once its
+    autograd node has run backward (no quantization loss in the step, so only the soft-step node exists)."""
+    import tmq_amd as t
+    torch.manual_seed(11)
+    net = _TwoHeads()
+    ctrl = t.QuantizationControl(epoch_knots=t.QuantizationScheduleBuilder.default_schedule(150))
+    t.quantize_model(net, ctrl)
+    net.to(cuda).train()
+    x = torch.randn(4, 32, device=cuda)
+    for step, which in enumerate("abab"):
+        for p in net.parameters():
+            p.grad = None
+        net(x, which).square().mean().backward()                 # raised "backward through the graph a second time"
+        used, idle = (net.head_a, net.head_b) if which == "a" else (net.head_b, net.head_a)
+        assert used.weight.grad is not None and idle.weight.grad is None, step
+        assert torch.isfinite(net.trunk.weight.grad).all()
+    # two forwards, then one backward through both: the second head still joins the first pass's node
+    for p in net.parameters():
+        p.grad = None
+    (net(x, "a").square().mean() + net(x, "b").square().mean()).backward()
+    assert net.head_a.weight.grad is not None and net.head_b.weight.grad is not None
+
+
+def test_layer_the_controller_cannot_serve_does_not_relaunch_the_others(cuda, oracle):
+    """A registered layer whose weights the multi-tensor launch cannot take (here: a compact layer) goes its own
+    way without restarting the pass of the layers that are served."""
+    import tmq_amd as t
+    from tmq_amd import tmq as tmq_mod
+    torch.manual_seed(12)
+    net = nn.Sequential(nn.Linear(16, 16), nn.ReLU(), nn.Linear(16, 16), nn.ReLU(), nn.Linear(16, 4))
+    ctrl = t.QuantizationControl()
+    t.quantize_model(net, ctrl)
+    net.to(cuda).train()
+    calls = []
+    orig = tmq_mod._StepState.run.__func__
+    tmq_mod._StepState.run = classmethod(lambda cls, c: (calls.append(1), orig(cls, c))[1])
+    try:
+        st = tmq_mod._StepState.run(ctrl)
+        ctrl._step = st
+        calls.clear()
+        st.unserved.add(id(net[2]))                              # as run() marks a layer it leaves out
+        assert ctrl._soft_weight_of(net[2]) is None and calls == []
+        y0 = ctrl._soft_weight_of(net[0])
+        assert y0 is st.ys[0] and calls == []
+    finally:
+        tmq_mod._StepState.run = classmethod(orig)

@@ -7,3 +7,4 @@ from .tmq import (QuantMode, TensorType, QuantizationScheduleBuilder, Quantizati
                   SoftStepDerivative, TMQLayer, Linear, Conv2d, ConvTranspose2d, quantize_weights, quantize_model,
                   compressed_state_dict, prepare_compressed_load, load_compressed_state_dict, expand_compact_layers, fold_batchnorm, set_compact_output_dtype, use_native_pooling, fuse_epilogues, GraphedForward,
                   CUDA_EXT_AVAILABLE, NATIVE_EXT_AVAILABLE)
+from .inference import FoldedConv, FoldedStem, ResNetRunner, InferenceSession, optimize_for_inference  # noqa: F401,E402

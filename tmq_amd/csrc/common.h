@@ -16,6 +16,12 @@ inline int check_launch() {
     return e == hipSuccess ? TMQ_OK : note_hip_error(e);
 }
 
+// A kernel that wants more than 64 KiB of dynamic LDS has to opt in once per device
+// (hipFuncAttributeMaxDynamicSharedMemorySize). Remembers the largest size granted per kernel and device, so
+// the runtime call is made the first time only (and again if a later launch asks for more); callable from
+// any thread, with the launch's device current. TMQ_OK or TMQ_ERR_LAUNCH.
+int allow_dynamic_lds(const void *kernel, size_t bytes);
+
 inline hipStream_t as_stream(void *s) { return reinterpret_cast<hipStream_t>(s); }
 
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }

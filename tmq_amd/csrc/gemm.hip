@@ -882,8 +882,7 @@ int launch_tile_solo(const Loader &ld, const void *native, int64_t M, int64_t K,
     if (tm * tn > 0x7FFFFFFF) return TMQ_ERR_TOO_LARGE;
     auto kernel = tile_solo_kernel<WM, WN, WGM, WGN, P, Loader>;
     if constexpr (kLds > 64 * 1024) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
-        if (e != hipSuccess) return note_hip_error(e);
+        if (int st = allow_dynamic_lds(reinterpret_cast<const void *>(kernel), kLds)) return st;
     }
     hipLaunchKernelGGL(kernel, dim3((uint32_t)(tm * tn)), dim3(64 * WGM * WGN), kLds, as_stream(stream), ld,
                        static_cast<const uint32_t *>(native), M, K, N, native_blocks_k(K), native_blocks_n(N), ep, (int)tm,

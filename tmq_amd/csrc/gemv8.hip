@@ -274,10 +274,7 @@ int launch_gemv8(const void *x, const void *native, int64_t Kb, int64_t N, const
     if (grid > 0x7FFFFFFF) return TMQ_ERR_TOO_LARGE;
     const size_t lds = (X32 ? 8 : 4) * (size_t)(Kb * kKB + 32) + (size_t)WAVES * 16 * sizeof(float);
     auto kernel = gemv8_kernel<WAVES, CB, NT, ORDER, X32>;
-    if (lds > 64 * 1024) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return note_hip_error(e);
-    }
+    if (int st = allow_dynamic_lds(reinterpret_cast<const void *>(kernel), lds)) return st;
     hipLaunchKernelGGL(kernel, dim3((uint32_t)grid), dim3(64 * WAVES), lds, as_stream(stream), x,
                        static_cast<const u32x4 *>(native), (int)Kb, N, Nb, ep);
     return check_launch();

@@ -520,10 +520,7 @@ template <int MT, bool X32, bool XLDS>
 int launch_skinny_as(dim3 grid, dim3 block, size_t lds, void *stream, const SkinnyArgs &a) {
     auto kernel = skinny_kernel<MT, X32, XLDS>;
     if (lds > 64 * 1024) {
-        // opt in to the large LDS (per device; the attribute is sticky, setting it again is cheap)
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)kSkinnyLdsMax);
-        if (e != hipSuccess) return note_hip_error(e);
+        if (int st = allow_dynamic_lds(reinterpret_cast<const void *>(kernel), kSkinnyLdsMax)) return st;
     }
     const tmq_epilogue &ep = *a.ep;
     const float *scale = ep.scale, *bias = ep.bias;
@@ -561,9 +558,7 @@ int launch_skinny(const void *x, int64_t M, int64_t K, const void *native, int64
             const size_t lds = (size_t)waves * 64 * sizeof(floatx4) + (size_t)waves * per_wave * M * kShortRowPitch;
             if (Kb <= 2 * waves && lds <= kSkinnyLdsMax) {
                 if (lds > 64 * 1024) {
-                    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(short_rows_kernel),
-                                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)kSkinnyLdsMax);
-                    if (e != hipSuccess) return note_hip_error(e);
+                    if (int st = allow_dynamic_lds(reinterpret_cast<const void *>(short_rows_kernel), kSkinnyLdsMax)) return st;
                 }
                 hipLaunchKernelGGL(short_rows_kernel, dim3((uint32_t)Nb), dim3(64 * waves), lds, as_stream(stream),
                                    static_cast<const _Float16 *>(x), (int)M, K, static_cast<const u32x4 *>(native), (int)Kb, N,
@@ -794,11 +789,7 @@ int launch_mid(const void *x, int64_t M, int64_t K, const void *native, int64_t 
     const void *residual = ep.residual;
     const int relu = ep.relu, y_f16 = ep.y_dtype == TMQ_F16;
     auto go = [&](auto kernel) -> int {
-        if (lds > 64 * 1024) {
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-            if (e != hipSuccess) return note_hip_error(e);
-        }
+        if (int st = allow_dynamic_lds(reinterpret_cast<const void *>(kernel), lds)) return st;
         hipLaunchKernelGGL(kernel, dim3((uint32_t)(tm * tn)), dim3(64 * WAVES), lds, as_stream(stream), x, M, K,
                            static_cast<const u32x4 *>(native), (int)Kb, N, native_blocks_n(N), (int)tn, scale, bias,
                            residual, relu, y, y_f16);
@@ -1015,11 +1006,7 @@ int launch_mid_lds(const void *x, int64_t M, int64_t K, const void *native, int6
     constexpr size_t lds = win > redb ? win : redb;
     static_assert(lds <= kSkinnyLdsMax, "mid kernel LDS");
     auto kernel = mid_lds_kernel<WM, WN, WAVES, X32>;
-    if (lds > 64 * 1024) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return note_hip_error(e);
-    }
+    if (int st = allow_dynamic_lds(reinterpret_cast<const void *>(kernel), lds)) return st;
     const float *scale = ep.scale, *bias = ep.bias;
     const void *residual = ep.residual;
     const int relu = ep.relu, y_f16 = ep.y_dtype == TMQ_F16;

@@ -512,12 +512,7 @@ int launch(const Rows &rows, const void *native, int64_t M, int64_t K, int64_t N
     constexpr size_t lds = win > redb ? win : redb;
     static_assert(lds <= 152 * 1024, "LDS budget");
     auto kernel = mid_kernel<WM, WN, WAVES, BLK, Rows, RING>;
-    if (lds > 64 * 1024) {
-        // opt in to the large LDS (per device; the attribute is sticky, setting it again is cheap)
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return note_hip_error(e);
-    }
+    if (int st = allow_dynamic_lds(reinterpret_cast<const void *>(kernel), lds)) return st;
     hipLaunchKernelGGL(kernel, dim3((uint32_t)(tm * tn)), dim3(64 * WAVES), lds, as_stream(stream), rows,
                        static_cast<const u32x4 *>(native), M, (int)Kb, (int)((K + 63) / 64), N, native_blocks_n(N),
                        (int)tn, (2 * M * 4 > N) ? 1 : 0 /* bytes of x (2 M K) against bytes of weights (N K / 4) */, ep);
@@ -827,11 +822,7 @@ int launch_stream(const void *x, const void *native, int64_t M, int64_t K, int64
         if (Kb / WAVES < 2 * D && Kb / WAVES >= D) return launch_stream<WN, WAVES, R, 2>(x, native, M, K, N, ep, stream);
     }
     auto kernel = R != 16 && Kb / WAVES >= 2 * D ? stream_kernel<WN, WAVES, R, D, true> : stream_kernel<WN, WAVES, R, D, false>;
-    if (lds > 64 * 1024) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return note_hip_error(e);
-    }
+    if (int st = allow_dynamic_lds(reinterpret_cast<const void *>(kernel), lds)) return st;
     hipLaunchKernelGGL(kernel, dim3((uint32_t)tn), dim3(64 * WAVES), lds, as_stream(stream),
                        static_cast<const _Float16 *>(x), static_cast<const u32x4 *>(native), M, K, (int)Kb, N,
                        native_blocks_n(N), ep);

@@ -290,7 +290,7 @@ int tmq_unpack_ternary(const uint32_t *words, int64_t N, int64_t K, float *w, vo
     if (!w || !words) return TMQ_ERR_INVALID_ARG;
     const int64_t Q = (N + 15) / 16;
     const int64_t gx = (K + kTileK - 1) / kTileK, gy = (Q + kTileQ - 1) / kTileQ;
-    if (gx > 0x7FFFFFFF || gy > 65535) return TMQ_ERR_TOO_LARGE;
+    if (gx > 0x7FFFFFFF || gy > 65535 || (Q + kUnpackWaves - 1) / kUnpackWaves > 65535) return TMQ_ERR_TOO_LARGE;
     if (vec4_ok<float>(w, K) && K >= kWideK) {
         hipLaunchKernelGGL(unpack_wide_kernel<kUnpackWaves>,
                            dim3((uint32_t)((K + kWideK - 1) / kWideK), (uint32_t)((Q + kUnpackWaves - 1) / kUnpackWaves)),

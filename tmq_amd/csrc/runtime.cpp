@@ -1,5 +1,9 @@
-// Status reporting of libtmq_hip.
+// Status reporting and per-device kernel set-up of libtmq_hip.
 #include "common.h"
+
+#include <map>
+#include <mutex>
+#include <utility>
 
 namespace tmq {
 static thread_local int g_last_hip_error = 0;
@@ -7,6 +11,22 @@ static thread_local int g_last_hip_error = 0;
 int note_hip_error(hipError_t e) {
     g_last_hip_error = (int)e;
     return TMQ_ERR_LAUNCH;
+}
+
+int allow_dynamic_lds(const void *kernel, size_t bytes) {
+    if (bytes <= 64 * 1024) return TMQ_OK;
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return note_hip_error(e);
+    static std::mutex guard;
+    static std::map<std::pair<const void *, int>, size_t> granted;   // (kernel, device) -> largest size opted in to
+    std::lock_guard<std::mutex> lock(guard);
+    size_t &have = granted[std::make_pair(kernel, dev)];
+    if (have >= bytes) return TMQ_OK;
+    e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    if (e != hipSuccess) return note_hip_error(e);
+    have = bytes;
+    return TMQ_OK;
 }
 }  // namespace tmq
 

@@ -549,7 +549,7 @@ def f32_to_f16_prescaled(x: torch.Tensor, scale, channels: int):
     """One fp16 term of an fp32 activation tensor for the convolution kernels: (fp16 tensor of x's shape and
     memory format holding s x, scale / s) with the range prescale s, or (x.half(), scale) when the prescale
     is switched off."""
-    if not _fp32_prescale:
+    if not _fp32_prescale or x.numel() == 0:      # nothing to scale in an empty batch
         return x.to(torch.float16), scale
     if not (x.is_contiguous() or x.is_contiguous(memory_format=torch.channels_last)):
         x = x.contiguous()
@@ -619,6 +619,8 @@ def ternary_conv2d(x: torch.Tensor, nw: NativeWeights, stride=1, padding=0, dila
     y = torch.empty((B, nw.N, ho.value, wo.value), dtype=out_dtype, device=x.device,
                     memory_format=torch.channels_last)
     ep = _epilogue(nw, scale, bias, residual, relu, out_dtype, y)
+    if B == 0:
+        return y
     with torch.cuda.device(x.device):
         check(lib.tmq_ternary_conv2d(ptr(x), ctypes.byref(shp), ptr(nw.buf), ctypes.byref(ep), ptr(y), stream_of(x)),
               "ternary_conv2d")
@@ -699,6 +701,8 @@ def ternary_dwconv2d(x: torch.Tensor, words: torch.Tensor, kernel, stride=1, pad
         raise RuntimeError("ternary_dwconv2d: empty output")
     y = torch.empty((B, C, ho.value, wo.value), dtype=out_dtype, device=x.device, memory_format=torch.channels_last)
     ep = _epilogue(_Channels(C), scale, bias, residual, relu, out_dtype, y)
+    if B == 0:
+        return y
     with torch.cuda.device(x.device):
         check(lib.tmq_ternary_dwconv2d(ptr(x), ctypes.byref(shp), ptr(words), ctypes.byref(ep), ptr(y), stream_of(x)),
               "ternary_dwconv2d")
@@ -755,6 +759,8 @@ def ternary_dwconvtrans2d(x: torch.Tensor, words: torch.Tensor, kernel, stride=1
           "convtranspose2d_out_hw")
     y = torch.empty((B, C, ho.value, wo.value), dtype=out_dtype, device=x.device, memory_format=torch.channels_last)
     ep = _epilogue(_Channels(C), scale, bias, residual, relu, out_dtype, y)
+    if B == 0:
+        return y
     with torch.cuda.device(x.device):
         check(lib.tmq_ternary_dwconvtrans2d(ptr(x), ctypes.byref(shp), oy, ox, ptr(words), ctypes.byref(ep), ptr(y),
                                             stream_of(x)), "ternary_dwconvtrans2d")
@@ -804,6 +810,8 @@ def maxpool2d_nhwc(x: torch.Tensor, kernel, stride=None, padding=0) -> torch.Ten
         raise RuntimeError("maxpool2d_nhwc: pad should be at most half of the kernel size and the window must fit")
     ho, wo = (H + 2 * py - ky) // sy + 1, (W + 2 * px - kx) // sx + 1
     y = torch.empty((B, C, ho, wo), dtype=torch.float16, device=x.device, memory_format=torch.channels_last)
+    if y.numel() == 0:
+        return y
     with torch.cuda.device(x.device):
         check(_lib().tmq_maxpool2d_nhwc(ptr(x), B, C, H, W, ky, kx, sy, sx, py, px, ptr(y), stream_of(x)), "maxpool2d_nhwc")
     return y
@@ -817,6 +825,8 @@ def avgpool_global_nhwc(x: torch.Tensor, out_dtype=torch.float16) -> torch.Tenso
         x = x.to(dtype=torch.float16, memory_format=torch.channels_last)
     B, C, H, W = x.shape
     y = torch.empty((B, C), dtype=out_dtype, device=x.device)
+    if y.numel() == 0:
+        return y
     with torch.cuda.device(x.device):
         check(_lib().tmq_avgpool_global_nhwc(ptr(x), B, H * W, C, ptr(y), _capi.dtype_code(y), stream_of(x)),
               "avgpool_global_nhwc")
@@ -833,6 +843,8 @@ def nchw_to_nhwc4(x: torch.Tensor) -> torch.Tensor:
     if C > 4 or W % 4:
         raise RuntimeError("nchw_to_nhwc4: at most 4 channels, width a multiple of 4")
     y = torch.empty((B, H, W, 4), dtype=torch.float16, device=x.device)
+    if y.numel() == 0:
+        return y
     with torch.cuda.device(x.device):
         check(_lib().tmq_nchw_to_nhwc4(ptr(x), _capi.dtype_code(x), B, C, H, W, ptr(y), stream_of(x)), "nchw_to_nhwc4")
     return y

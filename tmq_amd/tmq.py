@@ -270,7 +270,7 @@ class QuantizationControl:
         p = float(penalty if penalty is not None else self.qpenalty)
         self._loss_wanted = True
         st = self._step
-        if (st is not None and st.loss is not None and st.strength == p and st.sharpness == float(self.qpenalty_sharpness)
+        if (st is not None and st.loss is not None and not st.spent[0] and st.strength == p and st.sharpness == float(self.qpenalty_sharpness)
                 and st.grad_mode == torch.is_grad_enabled() and st.covers(self._registry.values())):
             return st.loss
         return _QuantizationLossAll.apply(self, p, float(self.qpenalty_sharpness), *self._weights())
@@ -283,9 +283,11 @@ class QuantizationControl:
         once per pass, and a changed weight tensor, hardness or autograd mode starts a new pass.
         Returns None for a layer this controller cannot serve (then SoftStep.apply does it)."""
         st = self._step
+        if st is not None and not st.spent[0] and id(node) in st.unserved:
+            return None                    # no relaunch for the served layers on account of this one
         i = st.index.get(id(node)) if st is not None else None
         w = node.weight
-        if (i is None or st.used[i] or st.versions[i] != w._version or st.ptrs[i] != w.data_ptr()
+        if (i is None or st.spent[0] or st.used[i] or st.versions[i] != w._version or st.ptrs[i] != w.data_ptr()
                 or st.digamma != self.digamma or st.grad_mode != torch.is_grad_enabled()):
             st = self._step = _StepState.run(self)
             i = st.index.get(id(node)) if st is not None else None
@@ -298,14 +300,16 @@ class QuantizationControl:
 class _StepState:
     """Outputs of one multi-tensor soft-step forward launch and what they were computed from."""
 
-    __slots__ = ("index", "nodes", "ptrs", "versions", "used", "ys", "loss", "digamma", "sharpness", "strength", "grad_mode")
+    __slots__ = ("index", "nodes", "ptrs", "versions", "used", "ys", "loss", "digamma", "sharpness", "strength", "grad_mode",
+                 "unserved", "spent")
 
     @classmethod
     def run(cls, ctrl):
-        nodes, dev = [], None
+        nodes, unserved, dev = [], set(), None
         for node in ctrl._registry.values():
             w = getattr(node, "weight", None)
             if w is None or node.compact or not w.is_cuda or w.dtype != torch.float32 or (dev is not None and w.device != dev):
+                unserved.add(id(node))     # these go through SoftStep.apply on their own
                 continue
             dev = w.device
             nodes.append(node)
@@ -313,6 +317,12 @@ class _StepState:
             return None
         st = cls()
         st.nodes = nodes
+        st.unserved = unserved
+        # spent[0] is set by the autograd node's backward: the graph behind `ys` is freed then, so a layer that
+        # did not take its result in that pass (a branch the forward skipped) must not be handed it in a later
+        # one. A one-element list, so that the node holds the flag and not the state (no reference cycle
+        # through `ys`, whose buffers are released by reference count).
+        st.spent = [False]
         st.index = {id(n): i for i, n in enumerate(nodes)}
         weights = [n.weight for n in nodes]
         st.ptrs = [w.data_ptr() for w in weights]
@@ -321,7 +331,7 @@ class _StepState:
         st.digamma, st.sharpness, st.strength = ctrl.digamma, float(ctrl.qpenalty_sharpness), float(ctrl.qpenalty)
         st.grad_mode = torch.is_grad_enabled()
         want_loss = ctrl._loss_wanted
-        outs = _SoftStepAll.apply(st.digamma, want_loss, st.sharpness, st.strength, *weights)
+        outs = _SoftStepAll.apply(st.spent, st.digamma, want_loss, st.sharpness, st.strength, *weights)
         st.ys = outs[:len(nodes)]
         st.loss = outs[len(nodes)] if want_loss else None
         return st
@@ -346,8 +356,9 @@ class _SoftStepAll(Function):
     add (tmq/tmq.py:422-438, 475-493)."""
 
     @staticmethod
-    def forward(ctx, digamma, want_loss, sharpness, strength, *weights):
+    def forward(ctx, spent, digamma, want_loss, sharpness, strength, *weights):
         ctx.args = (digamma, want_loss, sharpness, strength)
+        ctx.spent = spent
         ctx.save_for_backward(*weights)
         ctx.set_materialize_grads(False)
         ys, loss = _b.softstep_fwd_all([w.data for w in weights], digamma, want_loss, sharpness, strength)
@@ -356,10 +367,11 @@ class _SoftStepAll(Function):
     @staticmethod
     def backward(ctx, *grads):
         digamma, want_loss, sharpness, strength = ctx.args
+        ctx.spent[0] = True
         weights = ctx.saved_tensors
         L = len(weights)
         upstream = grads[L] if want_loss else None
-        need = ctx.needs_input_grad[4:]
+        need = ctx.needs_input_grad[5:]
         live = [i for i in range(L) if need[i] and (grads[i] is not None or upstream is not None)]
         out = [None] * L
         if live:
@@ -367,7 +379,7 @@ class _SoftStepAll(Function):
                                       sharpness, strength)
             for i, dw in zip(live, dws):
                 out[i] = dw
-        return (None, None, None, None) + tuple(out)
+        return (None, None, None, None, None) + tuple(out)
 
 
 class _QuantizationLossAll(Function):
@@ -1348,6 +1360,8 @@ def use_native_pooling(module: nn.Module):
     module otherwise. For inference. Returns the qualified names of the replaced modules."""
     done = []
     for pname, parent in list(module.named_modules()):
+        if isinstance(parent, (_MaxPool2dNHWC, _GlobalAvgPoolNHWC)):
+            continue                                     # already wrapped by an earlier call
         for cname, child in list(parent.named_children()):
             name = (pname + "." if pname else "") + cname
             if (isinstance(child, nn.MaxPool2d) and child.dilation in (1, (1, 1)) and not child.ceil_mode
@@ -1366,12 +1380,49 @@ class GraphedForward:
     long on the launches as the GPU on the work (ResNet-18 after fuse_epilogues, batch 64: 0.46 ms per forward from
     Python, 0.43 replayed). The graph holds its own input and output tensors: a call copies the input in and returns the
     output tensor, which the next call overwrites (clone it to keep it). A new input shape or dtype records a new graph.
-    For inference only (recorded under torch.no_grad())."""
+    For inference only (recorded under torch.no_grad()).
+
+    A recorded graph replays raw device addresses: the layers' kernel-native weight buffers, folded scale / bias
+    vectors, the dtype the layers hand on. Every call therefore compares a stamp of the model -- each TMQ layer's
+    weight tensor (address, shape, version counter), its native-weight cache, folded BatchNorm and post-scale, and the
+    global output-dtype and fp32-prescale switches -- with the one the graphs were recorded under, and records anew
+    when it moved (load_state_dict, invalidate_native(), expand_compact_layers, fold_batchnorm,
+    set_compact_output_dtype after the recording). What the stamp cannot see -- weights overwritten in place through
+    `.data`, submodules swapped, other modules' parameters changed -- needs reset()."""
 
     def __init__(self, model, warmup: int = 2):
         self.model = model
         self.warmup = int(warmup)
         self._graphs = {}
+        self._stamp = None
+        self._layers = None
+
+    def reset(self):
+        """Forget every recorded graph (and the list of the model's TMQ layers); the next call records again."""
+        self._graphs.clear()
+        self._stamp = None
+        self._layers = None
+
+    def _model_stamp(self):
+        if self._layers is None:
+            self._layers = [m for m in self.model.modules() if isinstance(m, TMQLayer)]
+        # addresses, not object identities: a buffer rebuilt at the address the graph already reads is as good
+        def where(t):
+            return t.data_ptr() if isinstance(t, torch.Tensor) else 0
+
+        def native(entry):
+            held = entry[1] if entry is not None else None
+            if isinstance(held, ops.NativeWeights):
+                return held.buf.data_ptr()
+            if isinstance(held, dict):          # ConvTranspose2d: one sub-kernel per phase of the output grid
+                return tuple(v[0].buf.data_ptr() if isinstance(v[0], ops.NativeWeights) else 0 for v in held.values())
+            return 0
+
+        return (_compact_out, ops._fp32_prescale) + tuple(
+            (m._weight_key(), native(m._native),
+             (where(m._fold[0]), where(m._fold[1])) if m._fold is not None else 0,
+             where(m._scale_vec[1]) if m._scale_vec is not None else 0, where(getattr(m, "bias", None)),
+             m.post_scale_imm, m.compact) for m in self._layers)
 
     def _record(self, x):
         static_in = x.clone()
@@ -1393,9 +1444,13 @@ class GraphedForward:
         if not (isinstance(x, torch.Tensor) and x.is_cuda):
             raise RuntimeError("GraphedForward: expected one GPU tensor")
         key = (tuple(x.shape), x.dtype, x.device, x.stride())
+        stamp = self._model_stamp()
+        if stamp != self._stamp:
+            self._graphs.clear()                         # recorded against buffers that may be gone
         entry = self._graphs.get(key)
         if entry is None:
             entry = self._graphs[key] = self._record(x)
+            self._stamp = self._model_stamp()            # the warm-up built the native-weight caches
         graph, static_in, static_out = entry
         static_in.copy_(x)
         graph.replay()
