@@ -121,9 +121,13 @@ def bench_softstep(args, torch):
     loss = torch.empty(1, dtype=torch.float64, device=dev)
     ws = torch.empty(lib.tmq_softstep_fused_workspace_bytes(n), dtype=torch.uint8, device=dev)
     out = (y, dw, wc, loss, ws)
+    in_launch = not args.two_launch_loss
 
     def step(i):
-        ops.softstep_fused(tw, tg, HARDNESS[i % len(HARDNESS)], SHARPNESS, STRENGTH, gl, -1.0, 1.0, out=out)
+        # the loss sum is finished by the pass itself (one launch per step); --two-launch-loss: block partial sums
+        # to a workspace and a finalisation launch behind every pass
+        ops.softstep_fused(tw, tg, HARDNESS[i % len(HARDNESS)], SHARPNESS, STRENGTH, gl, -1.0, 1.0, out=out,
+                           in_launch=in_launch)
 
     if args.copy_calibration:
         # A plain copy of known size (n*4 B read + n*4 B written) for scaling rocprofv3's
@@ -163,7 +167,8 @@ def bench_softstep(args, torch):
                      "frac": round(achieved / HBM_PEAK_GBS, 4),
                      "traffic": measured_traffic("softstep_fused_2p26.md", n),
                      "algorithmic_bytes": bytes_per_launch,
-                     "kernel": "stream_kernel<FusedOp<15>> (+ 1-block loss finalisation in the same call)",
+                     "kernel": "stream_kernel<FusedOp<15>, Single, InLaunch> (the loss sum finished inside the launch)"
+                               if in_launch else "stream_kernel<FusedOp<15>> (+ 1-block loss finalisation in the same call)",
                      "avg_launch_us": round(avg_ms * 1e3, 3)},
     }
     if not args.no_cpu:
@@ -660,6 +665,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--settle-ms", type=float, default=60.0)
     ap.add_argument("--copy-calibration", action="store_true")
+    ap.add_argument("--two-launch-loss", action="store_true", help="soft-step: finalise the loss in a second launch")
     ap.add_argument("--workload", default="all")
     ap.add_argument("--elements", type=int, default=1 << 26)
     ap.add_argument("--cpu-sample", type=int, default=1 << 22)

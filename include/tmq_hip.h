@@ -192,6 +192,38 @@ int tmq_softstep_bwd_multi(const tmq_step_tensor *tensors_host, int ntensors, do
                            double sharpness, double strength, const float *loss_upstream,
                            void *stream);
 
+/* The loss reductions above finished inside the launch that computes them: no finalisation launch, no
+ * workspace. Every block adds its partial sum to a 64-bit cell as a fixed-point integer (integer addition is
+ * associative, so the result does not depend on the order in which blocks arrive; the unit, 2^-28 .. 2^-10, is
+ * chosen per tensor from its size) with one returning device-scope atomic that also counts the block; a large
+ * tensor's blocks are spread over 64 cells; the block that completes a cell passes its total on (cell ->
+ * tensor -> launch), and the block that completes the launch writes the total; every cell is zero again by
+ * then. Deterministic and within 1e-6 relative of the fp64 finalisation of the two-launch forms; NaN / Inf
+ * weights give NaN as there. *total is the sum of the per-tensor means accumulated as integers (the two-launch
+ * form adds them in fp32 in table order; the two agree to fp32 rounding).
+ *   state: tmq_loss_state_bytes() bytes of device memory, 8-byte aligned, ZERO before the first call that uses
+ *   it; every call leaves it zero, so one memset at allocation serves all later calls (and HIP-graph replays).
+ *   Calls that share a state must not overlap in time (one state per stream).
+ * TMQ_ERR_UNSUPPORTED (use the two-launch form): more than 64 tensors, a tensor beyond 2^18 blocks of 2048
+ * elements (tmq_qloss_multi_inlaunch: a launch beyond 2^18 blocks), nothing to sum.
+ * tmq_softstep_fused_inlaunch: tmq_softstep_fused with loss_sum required (tmq/tmq.py:417-419, 434-438,
+ * 469-473 + 699, 488-493, 696). tmq_qloss_multi_inlaunch: tmq_qloss_multi (tmq/tmq.py:298-310).
+ * tmq_softstep_fwd_multi_inlaunch: tmq_softstep_fwd_multi with a loss output (tmq/tmq.py:404-419 for every
+ * layer + 298-310).                                                                                      */
+size_t tmq_loss_state_bytes(void);
+int tmq_softstep_fused_inlaunch(const float *w, const float *g, float *y, float *dw, float *wc,
+                                double *loss_sum, void *state, size_t n, double digamma,
+                                double sharpness, double strength, float gl, double lo, double hi,
+                                void *stream);
+int tmq_qloss_multi_inlaunch(const tmq_segment *segs_dev, int nseg, uint32_t total_blocks,
+                             double sharpness, double strength, float *per_tensor, float *total,
+                             void *state, void *stream);
+int tmq_softstep_fwd_multi_inlaunch(const tmq_step_tensor *tensors_host, int ntensors,
+                                    double digamma, double sharpness, double strength,
+                                    float *loss_per_tensor, float *loss_total, void *state,
+                                    void *stream);
+
+
 /* w_l <- clamp(w_l, lo, hi) for every segment, one launch. */
 int tmq_clamp_multi(const tmq_segment *segs_dev, int nseg, uint32_t total_blocks, double lo,
                     double hi, void *stream);

@@ -63,6 +63,9 @@ SIGNATURES = {
     "tmq_softstep_fused": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _dbl, _dbl, _dbl, _flt, _dbl, _dbl, _vp]),
     "tmq_softstep_fused_noalloc_max_elements": (_sz, []),
     "tmq_softstep_fused_noalloc": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _sz, _dbl, _dbl, _dbl, _flt, _dbl, _dbl, _vp]),
+    "tmq_loss_state_bytes": (_sz, []),
+    "tmq_softstep_fused_inlaunch": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _dbl, _dbl, _dbl, _flt, _dbl, _dbl, _vp]),
+    "tmq_qloss_multi_inlaunch": (_int, [_vp, _int, _u32, _dbl, _dbl, _vp, _vp, _vp, _vp]),
     "tmq_selfcheck_division": (_int, [_dbl, _vp, _vp]),
     "tmq_probe_stream_read": (_int, [_vp, ctypes.c_size_t, _vp, _vp]),
     "tmq_split_f32": (_int, [_vp, _vp, _vp, _i64, _vp]),
@@ -79,6 +82,7 @@ SIGNATURES = {
     "tmq_clamp_multi": (_int, [_vp, _int, _u32, _dbl, _dbl, _vp]),
     "tmq_softstep_multi_workspace_bytes": (_sz, [ctypes.POINTER(StepTensor), _int]),
     "tmq_softstep_fwd_multi": (_int, [ctypes.POINTER(StepTensor), _int, _dbl, _dbl, _dbl, _vp, _vp, _vp, _vp]),
+    "tmq_softstep_fwd_multi_inlaunch": (_int, [ctypes.POINTER(StepTensor), _int, _dbl, _dbl, _dbl, _vp, _vp, _vp, _vp]),
     "tmq_softstep_bwd_multi": (_int, [ctypes.POINTER(StepTensor), _int, _dbl, _dbl, _dbl, _vp, _vp]),
     "tmq_pack_ternary": (_int, [_vp, _int, _i64, _i64, _vp, _vp]),
     "tmq_unpack_ternary": (_int, [_vp, _i64, _i64, _vp, _vp]),

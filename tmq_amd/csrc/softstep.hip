@@ -250,6 +250,7 @@ struct View {
     uint32_t block;  // block index inside this tensor
     float scalar;
     bool vec;        // all pointers 16-byte aligned
+    int seg;         // which tensor of the launch
 };
 
 struct Single {
@@ -259,8 +260,11 @@ struct Single {
     uint64_t n;
     bool vec;
     __device__ __forceinline__ View locate(uint32_t b) const {
-        return View{in0, in1, out0, out1, out2, n, b, 0.f, vec};
+        return View{in0, in1, out0, out1, out2, n, b, 0.f, vec, 0};
     }
+    __device__ __forceinline__ int groups() const { return 1; }
+    __device__ __forceinline__ uint32_t group_blocks(int) const { return gridDim.x; }
+    __device__ __forceinline__ uint64_t group_elems(int) const { return n; }
 };
 
 // Multi-tensor: binary search of the block range table (wave-uniform, scalar loads).
@@ -281,8 +285,13 @@ struct Multi {
         float *a = static_cast<float *>(s.aux);
         bool vec = ((reinterpret_cast<uintptr_t>(p) | reinterpret_cast<uintptr_t>(a)) & 15u) == 0;
         const float sc = upstream ? upstream[0] / (float)s.n : s.scalar;
-        return View{p, nullptr, inplace ? p : nullptr, a, nullptr, s.n, b - s.block_begin, sc, vec};
+        return View{p, nullptr, inplace ? p : nullptr, a, nullptr, s.n, b - s.block_begin, sc, vec, lo};
     }
+    __device__ __forceinline__ int groups() const { return nseg; }
+    __device__ __forceinline__ uint32_t group_blocks(int l) const {
+        return (l + 1 < nseg ? segs[l + 1].block_begin : gridDim.x) - segs[l].block_begin;
+    }
+    __device__ __forceinline__ uint64_t group_elems(int l) const { return segs[l].n; }
 };
 
 // Multi-tensor with the table inside the kernel's arguments (nothing to upload: the pointers of a
@@ -312,13 +321,137 @@ struct MultiArg {
         const uint64_t n = t.n[lo];
         bool vec = ((reinterpret_cast<uintptr_t>(w) | reinterpret_cast<uintptr_t>(g) | reinterpret_cast<uintptr_t>(o)) & 15u) == 0;
         const float sc = upstream ? upstream[0] / (float)n : 0.f;
-        return View{w, g, o, o, nullptr, n, b - t.begin[lo], sc, vec};
+        return View{w, g, o, o, nullptr, n, b - t.begin[lo], sc, vec, lo};
+    }
+    __device__ __forceinline__ int groups() const { return t.ntensors; }
+    __device__ __forceinline__ uint32_t group_blocks(int l) const { return t.begin[l + 1] - t.begin[l]; }
+    __device__ __forceinline__ uint64_t group_elems(int l) const { return t.n[l]; }
+};
+
+// ---- where a block's loss partial sum goes -----------------------------------------------------
+// Partials: one float per block into the workspace; an ordered fp64 finalisation kernel follows.
+struct Partials {
+    static constexpr int kLanes = 1;
+    float *partials;
+    template <class Loc>
+    __device__ __forceinline__ void commit(float s, const View &, const Loc &) const { partials[blockIdx.x] = s; }
+};
+
+// InLaunch: the sum is finished by the launch itself, without a second kernel and without a single
+// floating-point addition whose order depends on timing. Thread 0 of a block adds its partial sum as a
+// FIXED-POINT INTEGER (integer addition is associative, so a total is the same bits whatever the order of
+// arrival) to a 64-bit cell with one returning device-scope atomic, which counts the block in the cell's top
+// bits at the same time. The block whose add completes a cell knows the cell's total from the returned value,
+// clears the cell and passes the total on to the next level the same way:
+//   blocks of a tensor of B > 64 blocks -> its 64 sub cells (block b uses cell b mod 64, so that blocks
+//   which run at the same time hit different addresses: atomics on ONE address complete at ~22 per
+//   microsecond on this GPU, and a 1152-block layer on a single cell cost 50 us) -> the tensor's top cell;
+//   blocks of a smaller tensor -> its top cell directly;
+//   the block that completes a top cell turns the total into the tensor's mean (written to per_tensor) and
+//   adds the mean / factor, again as an integer, to the launch cell; the block that completes the launch cell
+//   writes the total. A launch over one tensor ends at the top cell (sum_out).
+// All communication between blocks goes through atomic read-modify-writes, which are coherent whatever cache
+// a block's CU sits behind, and a block issues its next atomic only after the previous one has returned, so
+// every contribution is in place before the completion that follows it. No fences, no cache write-backs, no
+// spinning (nobody waits for anybody); a block that completes nothing pays one atomic, the last block of a
+// launch a chain of two or three (~1.5 us each under a streaming load).
+//   state (device, 8-byte aligned, tmq_loss_state_bytes()): zero before the first launch that uses it; every
+//   launch leaves it zero. Launches that share a state must not overlap.
+//   A partial sum that is not a finite number in [0, 2049] (NaN / Inf weights) is counted in the cell's
+//   poison field instead, and the result is NaN, as a float sum would be.
+// Cell layouts (count | poisoned | sum): sub 15 | 15 | 34 bits, top and launch 7 | 7 | 50 bits. Block sums
+// are in units of 2^-F with F = 28 - ceil(log2 B) per tensor (a block contributes less than 2^12: a sub
+// cell's B / 64 blocks stay below 2^34, a tensor below 2^40). A float block sum s >= 2^(24 - F) is a
+// multiple of the unit, i.e. its conversion is exact (ResNet-18's largest layer, 1152 blocks: F = 17, exact
+// from s = 128 on); otherwise the error is at most 2^-(F + 1) per block (B = 2^20: 2^-9 on block sums of
+// ~600, 3e-6 -- the 1e-6 bar holds up to 2^18 blocks = 2^29 elements per tensor, which is the limit).
+// Means travel as mean / factor in [0, 1] in units of 2^-43. Limits: 64 tensors per launch.
+constexpr int kSubs = 64;
+constexpr uint32_t kMaxGroupBlocks = 1u << 18;
+struct LossState {
+    unsigned long long sub[kArgTensors][kSubs];
+    unsigned long long top[kArgTensors];
+    unsigned long long launch;
+    unsigned long long pad;
+};
+
+// (count | poisoned | sum) fields of a cell with CB count bits and as many poison bits
+template <int CB>
+struct Cell {
+    static constexpr int kSumBits = 64 - 2 * CB;
+    static constexpr unsigned long long kOne = 1ull << (64 - CB), kPoison = 1ull << kSumBits, kSumMask = kPoison - 1;
+    static __device__ __forceinline__ unsigned long long pack(bool ok, unsigned long long units) {
+        return kOne | (ok ? units : kPoison);
+    }
+    static __device__ __forceinline__ uint32_t count(unsigned long long c) { return (uint32_t)(c >> (64 - CB)); }
+    static __device__ __forceinline__ bool poisoned(unsigned long long c) { return ((c >> kSumBits) & ((1ull << CB) - 1)) != 0; }
+    static __device__ __forceinline__ unsigned long long sum(unsigned long long c) { return c & kSumMask; }
+};
+
+struct InLaunch {
+    static constexpr int kLanes = 1;
+    LossState *st;
+    double factor;          // strength * sharpness / c
+    float *per_tensor;      // optional, [tensors] (multi-tensor launches)
+    float *total;           // optional: the sum of the per-tensor means
+    double *sum_out;        // single-tensor launches: fp64 sum * factor instead of a mean
+
+    // Called by thread 0 of a block with the block's partial sum.
+    template <class Loc>
+    __device__ __forceinline__ void commit(float s, const View &v, const Loc &loc) const {
+        typedef Cell<15> Sub;
+        typedef Cell<7> Top;
+        const int grp = v.seg;
+        const uint32_t B = loc.group_blocks(grp);
+        const int f = 28 - (B <= 1u ? 0 : 32 - __builtin_clz(B - 1u));
+        const double unit = __builtin_bit_cast(double, (unsigned long long)(1023 + f) << 52);
+        const double inv_unit = __builtin_bit_cast(double, (unsigned long long)(1023 - f) << 52);
+        bool ok = s >= 0.f && s <= 2049.f;                             // false for NaN
+        unsigned long long units = ok ? (unsigned long long)((double)s * unit + 0.5) : 0ull;
+        uint32_t expect = B;                                           // arrivals at the tensor's top cell
+        if (B > (uint32_t)kSubs) {
+            const uint32_t sub = v.block % (uint32_t)kSubs;
+            const unsigned long long add = Sub::pack(ok, units);
+            const unsigned long long now = atomicAdd(&st->sub[grp][sub], add) + add;
+            if (Sub::count(now) != (B - sub + (uint32_t)kSubs - 1) / (uint32_t)kSubs) return;
+            (void)atomicExch(&st->sub[grp][sub], 0ull);
+            ok = !Sub::poisoned(now);
+            units = Sub::sum(now);
+            expect = (uint32_t)kSubs;
+        }
+        const unsigned long long add = Top::pack(ok, units);
+        const unsigned long long now = atomicAdd(&st->top[grp], add) + add;
+        if (Top::count(now) != expect) return;
+        (void)atomicExch(&st->top[grp], 0ull);
+        // this block completed its tensor
+        const double avg_unscaled = (double)Top::sum(now) * inv_unit;  // sum of dsig over the tensor
+        const bool bad = Top::poisoned(now);
+        if (sum_out) {
+            sum_out[0] = bad ? __builtin_nan("") : avg_unscaled * factor;
+            return;
+        }
+        const double avg = avg_unscaled / (double)loc.group_elems(grp);   // in [0, 1]
+        if (per_tensor) per_tensor[grp] = bad ? __builtin_nanf("") : (float)(avg * factor);
+        const int ngrp = loc.groups();
+        int live = 0;                                                  // tensors that have blocks at all
+        for (int g = 0; g < ngrp; g++) live += loc.group_blocks(g) != 0u;
+        const unsigned long long addl = Top::pack(!bad, (unsigned long long)(avg * 8796093022208.0 + 0.5));   // 2^43
+        const unsigned long long all = atomicAdd(&st->launch, addl) + addl;
+        if (Top::count(all) != (uint32_t)live) return;
+        (void)atomicExch(&st->launch, 0ull);
+        // this block completed the launch; an empty tensor's mean is NaN (torch.mean of nothing), and so is the total then
+        if (live != ngrp && per_tensor)
+            for (int g = 0; g < ngrp; g++)
+                if (loc.group_blocks(g) == 0u) per_tensor[g] = __builtin_nanf("");
+        if (total)
+            *total = (Top::poisoned(all) || live != ngrp) ? __builtin_nanf("")
+                                                          : (float)((double)Top::sum(all) * (1.0 / 8796093022208.0) * factor);
     }
 };
 
 // ---- the streaming kernel ---------------------------------------------------------------------
-template <class Op, class Loc>
-__global__ __launch_bounds__(kThreads) void stream_kernel(Loc loc, Op op, float *partials) {
+template <class Op, class Loc, class Fin = Partials>
+__global__ __launch_bounds__(kThreads) void stream_kernel(Loc loc, Op op, Fin fin) {
     __shared__ float lds[16];
     const View v = loc.locate(blockIdx.x);
     const uint64_t base = (uint64_t)v.block * kChunk;
@@ -381,7 +514,7 @@ __global__ __launch_bounds__(kThreads) void stream_kernel(Loc loc, Op op, float 
     }
     if constexpr (Op::kLoss) {
         float s = block_sum(acc, lds);
-        if (tid == 0) partials[blockIdx.x] = s;
+        if (tid < Fin::kLanes) fin.commit(s, v, loc);
     }
 }
 
@@ -560,27 +693,39 @@ int scratch_address(void **out) {
     return TMQ_OK;
 }
 
-template <class Op>
-int launch_single(const Op &op, const float *in0, const float *in1, float *o0, float *o1, float *o2, size_t n,
-                  float *partials, void *stream) {
+template <class Op, class Fin>
+int launch_single_fin(const Op &op, const float *in0, const float *in1, float *o0, float *o1, float *o2, size_t n,
+                      const Fin &fin, void *stream) {
     if (n == 0) return TMQ_OK;
     if (n > kMaxElems) return TMQ_ERR_TOO_LARGE;
     Single loc{in0, in1, o0, o1, o2, (uint64_t)n,
                aligned16(in0) && aligned16(in1) && aligned16(o0) && aligned16(o1) && aligned16(o2)};
-    hipLaunchKernelGGL((stream_kernel<Op, Single>), dim3(blocks_for(n)), dim3(kThreads), 0, as_stream(stream), loc, op,
-                       partials);
+    hipLaunchKernelGGL((stream_kernel<Op, Single, Fin>), dim3(blocks_for(n)), dim3(kThreads), 0, as_stream(stream), loc, op,
+                       fin);
+    return check_launch();
+}
+
+template <class Op>
+int launch_single(const Op &op, const float *in0, const float *in1, float *o0, float *o1, float *o2, size_t n,
+                  float *partials, void *stream) {
+    return launch_single_fin(op, in0, in1, o0, o1, o2, n, Partials{partials}, stream);
+}
+
+template <class Op, class Fin>
+int launch_multi_fin(const Op &op, const tmq_segment *segs, int nseg, uint32_t total_blocks, int inplace, const Fin &fin,
+                     void *stream, const float *upstream = nullptr) {
+    if (nseg < 0 || (nseg > 0 && !segs)) return TMQ_ERR_INVALID_ARG;
+    if (nseg == 0 || total_blocks == 0) return TMQ_OK;
+    Multi loc{segs, nseg, inplace, upstream};
+    hipLaunchKernelGGL((stream_kernel<Op, Multi, Fin>), dim3(total_blocks), dim3(kThreads), 0, as_stream(stream), loc, op,
+                       fin);
     return check_launch();
 }
 
 template <class Op>
 int launch_multi(const Op &op, const tmq_segment *segs, int nseg, uint32_t total_blocks, int inplace, float *partials,
                  void *stream, const float *upstream = nullptr) {
-    if (nseg < 0 || (nseg > 0 && !segs)) return TMQ_ERR_INVALID_ARG;
-    if (nseg == 0 || total_blocks == 0) return TMQ_OK;
-    Multi loc{segs, nseg, inplace, upstream};
-    hipLaunchKernelGGL((stream_kernel<Op, Multi>), dim3(total_blocks), dim3(kThreads), 0, as_stream(stream), loc, op,
-                       partials);
-    return check_launch();
+    return launch_multi_fin(op, segs, nseg, total_blocks, inplace, Partials{partials}, stream, upstream);
 }
 
 bool bad_hardness(double d) { return !(d > 0.0) || !(d <= 1.0e6); }
@@ -608,11 +753,16 @@ int64_t fill_table(ArgTable &t, const tmq_step_tensor *ts, int first, int count,
     return (int64_t)b;
 }
 
+template <class Op, class Fin>
+int launch_args_fin(const Op &op, const ArgTable &t, uint32_t blocks, const float *upstream, const Fin &fin, void *stream) {
+    MultiArg loc{t, upstream};
+    hipLaunchKernelGGL((stream_kernel<Op, MultiArg, Fin>), dim3(blocks), dim3(kThreads), 0, as_stream(stream), loc, op, fin);
+    return check_launch();
+}
+
 template <class Op>
 int launch_args(const Op &op, const ArgTable &t, uint32_t blocks, const float *upstream, float *partials, void *stream) {
-    MultiArg loc{t, upstream};
-    hipLaunchKernelGGL((stream_kernel<Op, MultiArg>), dim3(blocks), dim3(kThreads), 0, as_stream(stream), loc, op, partials);
-    return check_launch();
+    return launch_args_fin(op, t, blocks, upstream, Partials{partials}, stream);
 }
 
 }  // namespace
@@ -722,6 +872,31 @@ int tmq_softstep_fused(const float *w, const float *g, float *y, float *dw, floa
     return rc;
 }
 
+size_t tmq_loss_state_bytes(void) { return sizeof(LossState); }
+
+int tmq_softstep_fused_inlaunch(const float *w, const float *g, float *y, float *dw, float *wc, double *loss_sum,
+                                void *state, size_t n, double digamma, double sharpness, double strength, float gl,
+                                double lo, double hi, void *stream) {
+    if (!loss_sum || !state || (reinterpret_cast<uintptr_t>(state) & 7u)) return TMQ_ERR_INVALID_ARG;
+    if (n == 0 || !w || (dw && !g)) return TMQ_ERR_INVALID_ARG;   // a sum over nothing: no block would write it
+    if (bad_hardness(digamma) || bad_hardness(sharpness) || !(lo <= hi)) return TMQ_ERR_INVALID_ARG;
+    if (n > kMaxElems) return TMQ_ERR_TOO_LARGE;
+    if (blocks_for(n) > kMaxGroupBlocks) return TMQ_ERR_UNSUPPORTED;
+    const int mask = (y ? 1 : 0) | (dw ? 2 : 0) | (wc ? 4 : 0) | 8;
+    const StepK s = make_step(digamma, 0.0), q = make_step(sharpness, strength);
+    const InLaunch fin{static_cast<LossState *>(state), (double)q.k1 / (double)q.c, nullptr, nullptr, loss_sum};
+    switch (mask) {
+#define TMQ_CASE(M)                                                                               \
+    case M: {                                                                                     \
+        FusedOp<M> op{s, q, gl, (float)lo, (float)hi};                                            \
+        return launch_single_fin(op, w, g, y, dw, wc, n, fin, stream);                            \
+    }
+        TMQ_CASE(8) TMQ_CASE(9) TMQ_CASE(10) TMQ_CASE(11) TMQ_CASE(12) TMQ_CASE(13) TMQ_CASE(14) TMQ_CASE(15)
+#undef TMQ_CASE
+    }
+    return TMQ_ERR_INVALID_ARG;
+}
+
 int tmq_softstep_fused_noalloc(const float *w, const float *g, float *y, float *dw, float *wc, double *loss_sum,
                                size_t n, double digamma, double sharpness, double strength, float gl, double lo,
                                double hi, void *stream) {
@@ -779,6 +954,17 @@ int tmq_qloss_multi(const tmq_segment *segs, int nseg, uint32_t total_blocks, do
     return check_launch();
 }
 
+int tmq_qloss_multi_inlaunch(const tmq_segment *segs, int nseg, uint32_t total_blocks, double sharpness, double strength,
+                             float *per_tensor, float *total, void *state, void *stream) {
+    if (nseg <= 0 || !segs || !state || (reinterpret_cast<uintptr_t>(state) & 7u) || total_blocks == 0) return TMQ_ERR_INVALID_ARG;
+    if (bad_hardness(sharpness)) return TMQ_ERR_INVALID_ARG;
+    // the table lives on the device: bound every tensor's block count by the launch's
+    if (nseg > kArgTensors || total_blocks > kMaxGroupBlocks) return TMQ_ERR_UNSUPPORTED;
+    QLossOp op{make_step(sharpness, strength)};
+    const InLaunch fin{static_cast<LossState *>(state), (double)op.q.k1 / (double)op.q.c, per_tensor, total, nullptr};
+    return launch_multi_fin(op, segs, nseg, total_blocks, 0, fin, stream);
+}
+
 int tmq_qloss_bwd_multi(const tmq_segment *segs, int nseg, uint32_t total_blocks, double sharpness, double strength,
                         const float *upstream, int accumulate, void *stream) {
     if (bad_hardness(sharpness)) return TMQ_ERR_INVALID_ARG;
@@ -831,6 +1017,27 @@ int tmq_softstep_fwd_multi(const tmq_step_tensor *ts, int ntensors, double digam
         }
     }
     return TMQ_OK;
+}
+
+int tmq_softstep_fwd_multi_inlaunch(const tmq_step_tensor *ts, int ntensors, double digamma, double sharpness,
+                                    double strength, float *loss_per_tensor, float *loss_total, void *state, void *stream) {
+    if (ntensors <= 0 || !ts || !state || (reinterpret_cast<uintptr_t>(state) & 7u)) return TMQ_ERR_INVALID_ARG;
+    if (!loss_per_tensor && !loss_total) return TMQ_ERR_INVALID_ARG;
+    if (bad_hardness(digamma) || bad_hardness(sharpness)) return TMQ_ERR_INVALID_ARG;
+    if (ntensors > kArgTensors) return TMQ_ERR_UNSUPPORTED;
+    uint64_t elems = 0;
+    for (int i = 0; i < ntensors; i++) {
+        if (ts[i].n && (!ts[i].w || !ts[i].out)) return TMQ_ERR_INVALID_ARG;
+        if ((ts[i].n + kChunk - 1) / kChunk > kMaxGroupBlocks) return TMQ_ERR_UNSUPPORTED;
+        elems += ts[i].n;
+    }
+    if (elems == 0) return TMQ_ERR_UNSUPPORTED;                   // no block would finish the sum
+    const StepK s = make_step(digamma, 0.0), q = make_step(sharpness, strength);
+    ArgTable t;
+    const int64_t blocks = fill_table(t, ts, 0, ntensors, [](const tmq_step_tensor &) { return true; });
+    if (blocks < 0) return (int)blocks;
+    const InLaunch fin{static_cast<LossState *>(state), (double)q.k1 / (double)q.c, loss_per_tensor, loss_total, nullptr};
+    return launch_args_fin(FusedOp<9>{s, q, 0.f, 0.f, 0.f}, t, (uint32_t)blocks, nullptr, fin, stream);
 }
 
 int tmq_softstep_bwd_multi(const tmq_step_tensor *ts, int ntensors, double digamma, double sharpness, double strength,

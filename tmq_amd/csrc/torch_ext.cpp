@@ -11,8 +11,10 @@
 #include <c10/core/DeviceGuard.h>
 
 #include <list>
+#include <map>
 #include <mutex>
 #include <stdexcept>
+#include <utility>
 #include <vector>
 
 #include "tmq_hip.h"
@@ -108,6 +110,19 @@ std::vector<torch::Tensor> step_weights(const std::vector<torch::Tensor> &weight
     return ws;
 }
 
+// The accumulator cells of the loss reductions that finish inside their launch: one zero-filled buffer per device
+// and stream, made on first use; every launch leaves it zero.
+torch::Tensor loss_state(const torch::Tensor &like) {
+    static std::mutex guard;
+    static std::map<std::pair<int, void *>, torch::Tensor> states;
+    const auto key = std::make_pair((int)like.device().index(), stream_of(like));
+    std::lock_guard<std::mutex> lock(guard);
+    auto it = states.find(key);
+    if (it == states.end())
+        it = states.emplace(key, torch::zeros({(int64_t)tmq_loss_state_bytes()}, like.options().dtype(torch::kUInt8))).first;
+    return it->second;
+}
+
 std::tuple<std::vector<torch::Tensor>, c10::optional<torch::Tensor>> softstep_fwd_all(
         std::vector<torch::Tensor> weights, double digamma, bool want_loss, double sharpness, double strength) {
     auto ws = step_weights(weights, "softstep_fwd_all");
@@ -120,6 +135,14 @@ std::tuple<std::vector<torch::Tensor>, c10::optional<torch::Tensor>> softstep_fw
     torch::Tensor workspace;
     if (want_loss) {
         loss = torch::empty({}, ws[0].options());
+        // finished inside the launch where the shape allows (up to 64 tensors of up to 2^18 blocks each)
+        auto state = loss_state(ws[0]);
+        const int status = tmq_softstep_fwd_multi_inlaunch(table.data(), (int)table.size(), digamma, sharpness, strength,
+                                                           nullptr, loss->data_ptr<float>(), state.data_ptr(), stream_of(ws[0]));
+        if (status != TMQ_ERR_UNSUPPORTED) {
+            check(status, "softstep_fwd_all");
+            return {ys.parts, loss};
+        }
         workspace = torch::empty({(int64_t)tmq_softstep_multi_workspace_bytes(table.data(), (int)table.size())},
                                  ws[0].options().dtype(torch::kUInt8));
     }

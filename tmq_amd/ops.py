@@ -103,13 +103,30 @@ def ternarize_(weights: torch.Tensor, digamma: float = 0.0) -> torch.Tensor:
     return weights
 
 
+_loss_states = {}
+
+
+def loss_state(device):
+    """The accumulator cells of the loss reductions that finish inside their launch (tmq_*_inlaunch): one small
+    zero-filled buffer per device and stream, made on first use. Every launch leaves it zero, so it is never
+    cleared again; launches on one stream are ordered, so they can share it."""
+    device = torch.device(device)
+    key = (device.index if device.index is not None else torch.cuda.current_device(),
+           torch.cuda.current_stream(device).cuda_stream)
+    st = _loss_states.get(key)
+    if st is None:
+        st = _loss_states[key] = torch.zeros(_lib().tmq_loss_state_bytes(), dtype=torch.uint8, device=device)
+    return st
+
+
 def softstep_fused(weights, grad, digamma, sharpness, strength, gl, lo, hi, *, want_y=True, want_dw=True,
-                   want_clamp=True, want_loss=True, clamp_inplace=False, out=None):
+                   want_clamp=True, want_loss=True, clamp_inplace=False, out=None, in_launch=False):
     """One pass: y = S(w), dw = g*S'(w) + gl*Q'(w), wc = clamp(w), loss_sum = sum q(w).
 
     Returns (y, dw, wc, loss_sum) with None for outputs not requested; loss_sum is a 1-element
     fp64 tensor. `out` may carry preallocated (y, dw, wc, loss_sum, workspace) to keep
-    allocations out of a timed loop."""
+    allocations out of a timed loop. in_launch: the loss sum is finished by the pass itself (fixed-point
+    atomics, no finalisation launch, no workspace)."""
     _capi.require_gpu(weights, "weights")
     w = weights
     n = w.numel()
@@ -122,11 +139,21 @@ def softstep_fused(weights, grad, digamma, sharpness, strength, gl, lo, hi, *, w
         wc = (w if clamp_inplace else torch.empty_like(w)) if want_clamp else None
         loss = torch.empty(1, dtype=torch.float64, device=w.device) if want_loss else None
         ws = torch.empty(lib.tmq_softstep_fused_workspace_bytes(n), dtype=torch.uint8, device=w.device) \
-            if want_loss else None
+            if want_loss and not in_launch else None
     if dw is not None:
         _capi.require_gpu(grad, "grad")
         if grad.numel() != n or grad.dtype != torch.float32:
             raise RuntimeError("softstep_fused: gradient must match the weights")
+    if in_launch and loss is not None and n:
+        with torch.cuda.device(w.device):
+            status = lib.tmq_softstep_fused_inlaunch(ptr(w), ptr(grad) if dw is not None else None, ptr(y), ptr(dw), ptr(wc),
+                                                     ptr(loss), ptr(loss_state(w.device)), n, float(digamma), float(sharpness),
+                                                     float(strength), ctypes.c_float(gl), float(lo), float(hi), stream_of(w))
+        if status != _capi.ERR_UNSUPPORTED:
+            check(status, "softstep_fused_inlaunch")
+            return y, dw, wc, loss
+        if ws is None:
+            ws = torch.empty(lib.tmq_softstep_fused_workspace_bytes(n), dtype=torch.uint8, device=w.device)
     with torch.cuda.device(w.device):
         check(lib.tmq_softstep_fused(ptr(w), ptr(grad) if dw is not None else None, ptr(y), ptr(dw), ptr(wc),
                                      ptr(loss), ptr(ws), n, float(digamma), float(sharpness), float(strength),
@@ -177,6 +204,13 @@ def qloss_multi(table: SegmentTable, sharpness: float, strength: float):
     per = torch.empty(table.nseg, dtype=torch.float32, device=table.device)
     tot = torch.empty(1, dtype=torch.float32, device=table.device)
     with torch.cuda.device(table.device):
+        # finished inside the launch where the shape allows (up to 64 tensors, 2^18 blocks), else two launches
+        status = _lib().tmq_qloss_multi_inlaunch(ptr(table.table), table.nseg, table.total_blocks, float(sharpness),
+                                                 float(strength), ptr(per), ptr(tot), ptr(loss_state(table.device)),
+                                                 stream_of(table.table)) if table.total_blocks else _capi.ERR_UNSUPPORTED
+        if status != _capi.ERR_UNSUPPORTED:
+            check(status, "qloss_multi_inlaunch")
+            return per, tot
         check(_lib().tmq_qloss_multi(ptr(table.table), table.nseg, table.total_blocks, float(sharpness),
                                      float(strength), ptr(per), ptr(tot), ptr(table.workspace),
                                      stream_of(table.table)), "qloss_multi")
@@ -242,6 +276,13 @@ def softstep_fwd_all(weights, digamma: float, want_loss: bool = False, sharpness
     loss = wsp = None
     if want_loss:
         loss = torch.empty((), dtype=torch.float32, device=dev)
+        # the loss finished inside the launch where the shape allows (up to 64 tensors of up to 2^18 blocks)
+        with torch.cuda.device(dev):
+            status = lib.tmq_softstep_fwd_multi_inlaunch(arr, len(ws), float(digamma), float(sharpness), float(strength), None,
+                                                         ptr(loss), ptr(loss_state(dev)), stream_of(flat))
+        if status != _capi.ERR_UNSUPPORTED:
+            check(status, "softstep_fwd_all")
+            return ys, loss
         wsp = torch.empty(lib.tmq_softstep_multi_workspace_bytes(arr, len(ws)), dtype=torch.uint8, device=dev)
     with torch.cuda.device(dev):
         check(lib.tmq_softstep_fwd_multi(arr, len(ws), float(digamma), float(sharpness), float(strength), None, ptr(loss),
