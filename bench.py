@@ -346,6 +346,26 @@ def _gemv_floor_and_large(args, torch, natives):
     floor = _graph_time_us(torch, run, max(2, args.steps // 12), args.settle_ms)
     res["gemv_16384"] = {"us": round(us, 3), "gbs": round(byts / us / 1e3, 1), "frac_hbm": round(byts / us / 1e3 / HBM_PEAK_GBS, 4),
                          "read_floor_us": round(floor, 3), "read_floor_gbs": round(K * N / 4 / floor / 1e3, 1)}
+    # the same GEMV on activation planes made beforehand (tmq_gemv8_prepare, NOT in the timed region): what a vector
+    # multiplied with several layers, or emitted in this form by its producer, costs per layer; and with the
+    # preparation launch in front of every GEMV
+    planes = ops.gemv8_prepare(x)
+
+    def gemv_planes():
+        for nw in big:
+            ops.ternary_linear_planes(planes, nw, scale)
+        return len(big)
+
+    def gemv_prepare_and_planes():
+        for nw in big:
+            ops.ternary_linear_planes(ops.gemv8_prepare(x), nw, scale)
+        return len(big)
+    gemv_planes()
+    us_p = _graph_time_us(torch, gemv_planes, max(2, args.steps // 12), args.settle_ms)
+    us_pp = _graph_time_us(torch, gemv_prepare_and_planes, max(2, args.steps // 12), args.settle_ms)
+    res["gemv_16384"]["planes_prepared_beforehand_us"] = round(us_p, 3)
+    res["gemv_16384"]["planes_prepared_beforehand_frac_hbm"] = round(byts / us_p / 1e3 / HBM_PEAK_GBS, 4)
+    res["gemv_16384"]["prepare_launch_plus_gemv_us"] = round(us_pp, 3)
     # the same layer against 4 and 16 rows (batched decoding): the weights are still read once
     for rows in (4, 16):
         xr = torch.randn(rows, K, device=dev).half()

@@ -297,6 +297,21 @@ typedef struct tmq_epilogue {
 int tmq_ternary_linear(const void *x, int x_dtype, int64_t M, int64_t K, const void *native,
                        int64_t N, const tmq_epilogue *epilogue, void *y, void *stream);
 
+/* One to four fp16 rows with the activations already in the operand form of the 8-bit matrix instructions.
+ * The GEMV for a few rows (the reference's ternaryMVFP32, tmq/tmq_cuda.cu:242-286, 563-603; its row-batched
+ * caller tmq/tmq.py:680-683) multiplies fp8 weight operands with the rows carried exactly as four bf8 terms per
+ * value ("planes"); tmq_ternary_linear derives the planes inside every workgroup, these two calls do it once:
+ *   tmq_gemv8_prepare          x: fp16 [M][K], 16-byte aligned -> planes (tmq_gemv8_planes_bytes(M, K) bytes,
+ *                              16-byte aligned; an opaque image, valid for this M and K)
+ *   tmq_ternary_linear_planes  y = epilogue(x W^T) from the planes; same results as tmq_ternary_linear on x
+ * so that a vector multiplied with several layers (q / k / v, gate / up) or produced once and consumed later is
+ * converted once. M <= 4, K a multiple of 256 from 2048 to 16384 and M' K <= 16384 with M' = M padded to 1, 2 or
+ * 4 (else TMQ_ERR_UNSUPPORTED, and tmq_gemv8_planes_bytes returns 0).                                      */
+size_t tmq_gemv8_planes_bytes(int64_t M, int64_t K);
+int tmq_gemv8_prepare(const void *x, int64_t M, int64_t K, void *planes, void *stream);
+int tmq_ternary_linear_planes(const void *planes, int64_t M, int64_t K, const void *native, int64_t N,
+                              const tmq_epilogue *epilogue, void *y, void *stream);
+
 /* 1 when tmq_ternary_linear(x, TMQ_F32, M, K, ...) takes fp32 activations of any magnitude as they are (one
  * 16-byte aligned row, K a multiple of 256 from 2048 to 8192: the kernel finds the row's largest finite |x| and scales
  * by a power of two itself), 0 when the caller has to keep them inside fp16's range (tmq_f32_prescale). */

@@ -151,7 +151,7 @@ def test_wide_dynamic_range_within_the_stated_tolerance(cuda, oracle):
 
 
 def test_agrees_with_the_fp16_kernels_on_neighbouring_shapes(cuda, oracle):
-    """M = 2 (fp16 weight-stream kernel) on two copies of the row, and an unaligned view of the row (skinny
+    """M = 5 (fp16 weight-stream kernel) on copies of the row, and an unaligned view of the row (skinny
     kernel), give the same numbers to fp32 rounding."""
     from tmq_amd import ops
     K, N = 8192, 1024
@@ -160,8 +160,8 @@ def test_agrees_with_the_fp16_kernels_on_neighbouring_shapes(cuda, oracle):
     buf = torch.from_numpy(rng.standard_normal(K + 8).astype(np.float16)).to(cuda)
     x = buf[:K].clone()[None]
     y1 = ops.ternary_linear(x, nw)
-    y2 = ops.ternary_linear(torch.cat([x, x]), nw)
-    assert torch.equal(y2[0], y2[1])
+    y2 = ops.ternary_linear(torch.cat([x] * 5), nw)
+    assert torch.equal(y2[0], y2[4])
     assert _rel_err(y1.cpu().numpy(), y2[:1].cpu().numpy()) <= 1e-5
     buf[1:K + 1] = x[0]
     y3 = ops.ternary_linear(buf[1:K + 1][None], nw)                     # 2-byte aligned: not the 8-bit kernel
@@ -238,3 +238,108 @@ def test_hip_graph_replays_match_eager(cuda, oracle):
             x2 = torch.randn_like(x)                               # eager work on the same weights in between
             ops.ternary_linear(x2, nw)
             torch.cuda.synchronize()
+
+
+# ---- two to four rows: row m's four term planes ride in activation columns 4 m .. 4 m + 3 -----------------------
+@pytest.mark.parametrize("M,K", [(2, 2048), (2, 4096), (2, 2304), (3, 2048), (4, 2048), (2, 8192), (4, 4096)])
+@pytest.mark.parametrize("N", [16, 1000, 4100])
+def test_few_rows_on_the_8bit_instruction(cuda, oracle, M, K, N):
+    from tmq_amd import ops
+    rng = np.random.default_rng(100 * M + K + N)
+    W, nw = _layer(cuda, oracle, rng, N, K)
+    x = rng.standard_normal((M, K)).astype(np.float16)
+    x[M - 1] *= np.float16(37.0)                                  # rows of different magnitude must not mix
+    t = lambda a: torch.from_numpy(a).to(cuda)
+    y = ops.ternary_linear(t(x), nw)
+    ref = x.astype(np.float64) @ W.astype(np.float64).T
+    assert y.shape == (M, N)
+    for m in range(M):
+        assert _rel_err(y[m].cpu().numpy(), ref[m]) <= 1e-5, m
+    # on the 8-bit kernel (up to 8192 values in all rows; beyond that the fp16 weight stream takes the rows) every
+    # row equals the single-row launch of that row, bit for bit: same instruction, same order
+    if K * (M if M < 3 else 4) <= 8192:
+        for m in range(M):
+            assert torch.equal(ops.ternary_linear(t(x[m:m + 1]), nw)[0], y[m]), m
+    scale = (0.01 + 0.02 * rng.random(N)).astype(np.float32)
+    bias = rng.standard_normal(N).astype(np.float32)
+    res = rng.standard_normal((M, N)).astype(np.float16)
+    y2 = ops.ternary_linear(t(x), nw, t(scale), t(bias), residual=t(res), relu=True, out_dtype=torch.float16)
+    assert _rel_err(y2.float().cpu().numpy(), np.maximum(ref * scale + bias + res.astype(np.float64), 0)) <= 1e-3
+
+
+def test_few_rows_pass_every_finite_fp16_value_through(cuda, oracle):
+    """Identity weights, up to four rows at once: every finite fp16 value comes back exactly in its own row, from the
+    kernel that splits the rows itself (K = 2048) and from prepared planes (K = 4096)."""
+    from tmq_amd import ops
+    vals = np.arange(65536, dtype=np.uint32).astype(np.uint16).view(np.float16).copy()
+    vals[~np.isfinite(vals)] = 0
+    vals = vals[np.random.default_rng(8).permutation(65536)]
+    for K, prepared in ((2048, False), (4096, True)):
+        nw = ops.NativeWeights(torch.from_numpy(oracle.pack(np.eye(K, dtype=np.float32)).view(np.int32)).to(cuda), K)
+        for M in (2, 3, 4):
+            for c in range(0, 65536 // K - M + 1, M):
+                x = vals[c * K:(c + M) * K].reshape(M, K)
+                tx = torch.from_numpy(x).to(cuda)
+                y = ops.ternary_linear_planes(ops.gemv8_prepare(tx), nw) if prepared else ops.ternary_linear(tx, nw)
+                assert np.array_equal(y.cpu().numpy(), x.astype(np.float32)), (K, M, c)
+    # exact on integers whatever the order of summation
+    rng = np.random.default_rng(12)
+    W, nw2 = _layer(cuda, oracle, rng, 520, 4096)
+    xi = rng.integers(-8, 9, size=(4, 4096)).astype(np.float16)
+    y = ops.ternary_linear(torch.from_numpy(xi).to(cuda), nw2).cpu().numpy()
+    assert np.array_equal(y.astype(np.float64), xi.astype(np.float64) @ W.astype(np.float64).T)
+
+
+# ---- the term planes made once (tmq_gemv8_prepare) and multiplied with several layers ---------------------------
+@pytest.mark.parametrize("M,K", [(1, 2048), (1, 4096), (1, 11008), (1, 16384), (2, 8192), (2, 6912), (3, 4096), (4, 4096),
+                                 (4, 2304)])
+def test_prepared_planes_give_the_plain_call_s_values(cuda, oracle, M, K):
+    from tmq_amd import ops
+    rng = np.random.default_rng(M * 1000 + K)
+    N = 1000
+    W, nw = _layer(cuda, oracle, rng, N, K)
+    W2, nw2 = _layer(cuda, oracle, rng, 272, K)
+    x = rng.standard_normal((M, K)).astype(np.float16)
+    t = lambda a: torch.from_numpy(a).to(cuda)
+    assert ops.gemv8_planes_supported(M, K)
+    planes = ops.gemv8_prepare(t(x))
+    ref = x.astype(np.float64) @ W.astype(np.float64).T
+    y = ops.ternary_linear_planes(planes, nw)
+    assert y.shape == (M, N) and _rel_err(y.cpu().numpy(), ref) <= 1e-5
+    for m in range(M):                                             # same bits as the single-row kernel that splits in place
+        assert torch.equal(ops.ternary_linear(t(x[m:m + 1]), nw)[0], y[m]), m
+    y2 = ops.ternary_linear_planes(planes, nw2)                     # the same planes against another layer
+    assert _rel_err(y2.cpu().numpy(), x.astype(np.float64) @ W2.astype(np.float64).T) <= 1e-5
+    scale = (0.01 + 0.02 * rng.random(N)).astype(np.float32)
+    bias = rng.standard_normal(N).astype(np.float32)
+    res = rng.standard_normal((M, N)).astype(np.float32)
+    y3 = ops.ternary_linear_planes(planes, nw, t(scale), t(bias), residual=t(res), relu=True)
+    assert _rel_err(y3.cpu().numpy(), np.maximum(ref * scale + bias + res, 0)) <= 1e-5
+
+
+def test_prepared_planes_limits_and_graph_replay(cuda, oracle):
+    from tmq_amd import ops
+    assert not ops.gemv8_planes_supported(5, 4096) and not ops.gemv8_planes_supported(4, 8192)
+    assert not ops.gemv8_planes_supported(2, 16384)
+    assert not ops.gemv8_planes_supported(1, 1024) and not ops.gemv8_planes_supported(1, 4100)
+    with pytest.raises(RuntimeError):
+        ops.gemv8_prepare(torch.zeros(5, 4096, dtype=torch.float16, device=cuda))
+    rng = np.random.default_rng(13)
+    K, N = 16384, 520
+    W, nw = _layer(cuda, oracle, rng, N, K)
+    x = torch.from_numpy(rng.standard_normal((1, K)).astype(np.float16)).to(cuda)
+    eager = ops.ternary_linear_planes(ops.gemv8_prepare(x), nw).clone()
+    torch.cuda.synchronize()
+    graph, side = torch.cuda.CUDAGraph(), torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        y = torch.empty(1, N, device=cuda)
+        with torch.cuda.graph(graph, stream=side):
+            y.copy_(ops.ternary_linear_planes(ops.gemv8_prepare(x), nw))
+    for rep in range(3):
+        y.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y, eager), rep
+        ops.ternary_linear(torch.randn_like(x), nw)
+        torch.cuda.synchronize()

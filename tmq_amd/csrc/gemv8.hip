@@ -27,6 +27,16 @@
 //
 // Requires M == 1, K a multiple of 256 from 2048 to 16384 (fp32 activations, carried as two fp16 halves: to 8192),
 // 16-byte aligned x.
+//
+// Two to four rows (MR = 2, 4; three rows run as four with one of zeros) take the same kernel: row m's four
+// term planes ride in activation columns 4 m .. 4 m + 3, so four rows fill exactly the sixteen columns of the
+// instruction the single row already issues -- no extra MFMA, no extra weight expansion; only the planes (and
+// the work of preparing them) grow with the rows, which is what limits the rows: see gemv8_dense_ok.
+//
+// The planes can also come ready-made from memory (PRE): tmq_gemv8_prepare writes them once per activation
+// vector (or a producing kernel could), and the workgroup then copies its image global -> LDS with buffer loads
+// that bypass the registers -- no conversion arithmetic and no LDS writes in the GEMV, which is what every
+// workgroup otherwise repeats for the whole row. Up to 16384 / MR reduction indices (64 KiB of planes).
 #include "common.h"
 #include "mfma.h"
 
@@ -66,7 +76,11 @@ struct Gemv8Epilogue {
     const void *residual;
     void *y;
     int relu, y_f16;
+    int rows;               // rows of x that exist (<= MR; the others are zero planes and are not stored)
 };
+
+// vmcnt(n), nothing else waited for
+constexpr int vmcnt_only(int n) { return (n & 15) | ((n >> 4) << 14) | 0x0F70; }
 
 // ORDER: what separates the activation loads from the weight loads. 0: nothing. 1: a workgroup barrier, so that
 // no wavefront's activation loads queue behind another's weight loads (8192^2: 5.65 -> 5.3 us). 2: the
@@ -76,16 +90,18 @@ struct Gemv8Epilogue {
 // X32: the row is fp32, of any magnitude (the kernel scales it by a power of two itself). Each value becomes
 // hi = fp16(x) and lo = fp16(x - hi) -- 22 significant bits -- and both halves their four bf8 terms: eight
 // planes, eight of the sixteen activation columns, still one MFMA per weight operand.
-template <int WAVES, int CB, int NT, int ORDER, bool X32>
+template <int WAVES, int CB, int NT, int ORDER, bool X32, int MR, bool PRE>
 __global__ __launch_bounds__(64 * WAVES) void gemv8_kernel(const void *__restrict__ xv, const u32x4 *__restrict__ native,
                                                            int Kb, int64_t N, int64_t Nb, Gemv8Epilogue ep) {
-    constexpr int KS = WAVES / CB, kUnits = (KS * NT + 2 * WAVES - 1) / (2 * WAVES);   // units of 8 values per thread: ceil(32 Kb / threads)
-    constexpr int NP = X32 ? 8 : 4;                              // term planes
+    static_assert(!X32 || (MR == 1 && !PRE), "fp32 rows: one row, split in the kernel");
+    constexpr int KS = WAVES / CB, kUnits = (KS * NT + 2 * WAVES - 1) / (2 * WAVES);   // units of 8 values per thread and row: ceil(32 Kb / threads)
+    constexpr int NP = X32 ? 8 : 4 * MR;                         // term planes
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const int K = Kb * kKB;
     const int plane = K + 32;                                    // bytes per term plane; +32 puts the planes on different banks
     unsigned char *planes = smem;
-    float *red = reinterpret_cast<float *>(smem + NP * plane);  // [WAVES][16]
+    const int image = PRE ? ((NP * plane + 1023) & ~1023) : NP * plane;   // the copy from memory moves whole KiB
+    float *red = reinterpret_cast<float *>(smem + image);       // [WAVES][MR][16]
     const int lane = threadIdx.x & 63, wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int j = lane & 15, g = lane >> 4;
     const int cb = wv / KS, ks = wv % KS;
@@ -97,22 +113,31 @@ __global__ __launch_bounds__(64 * WAVES) void gemv8_kernel(const void *__restric
     // covers x[256 kb + 64 d + 8 g' + 4 h + {0..3}] (quad A) and the same 32 further on (quad B): the eight
     // values whose weights lane group g' finds in one operand register pair of dword d.
     using Quad = std::conditional_t<X32, u32x4, u32x2>;           // four activation values
-    Quad qa[kUnits], qb[kUnits];
+    Quad qa[MR][kUnits], qb[MR][kUnits];
+    if constexpr (PRE) {
+        // the planes as tmq_gemv8_prepare left them: NP x (K + 32) bytes, copied 1 KiB per instruction
+        const BufferResource img = make_buffer_resource(xv, (uint32_t)(NP * plane));
+        for (int c = wv * 1024; c < image; c += WAVES * 1024) buffer_to_lds(img, (uint32_t)(c + lane * 16), planes + c);
+    } else {
 #pragma unroll
-    for (int i = 0; i < kUnits; i++) {
-        const int u = threadIdx.x + i * 64 * WAVES;
-        const int gq = u & 3, h = (u >> 2) & 1, d = (u >> 3) & 3, kb = u >> 5;
-        const int k0 = kKB * kb + 64 * d + 8 * gq + 4 * h;
-        qa[i] = qb[i] = Quad{};
-        if (u < K / 8) {
-            if constexpr (X32) {
-                qa[i] = *reinterpret_cast<const u32x4 *>(static_cast<const float *>(xv) + k0);
-                qb[i] = *reinterpret_cast<const u32x4 *>(static_cast<const float *>(xv) + k0 + 32);
-            } else {
-                qa[i] = *reinterpret_cast<const u32x2 *>(static_cast<const _Float16 *>(xv) + k0);
-                qb[i] = *reinterpret_cast<const u32x2 *>(static_cast<const _Float16 *>(xv) + k0 + 32);
+        for (int m = 0; m < MR; m++)
+#pragma unroll
+            for (int i = 0; i < kUnits; i++) {
+                const int u = threadIdx.x + i * 64 * WAVES;
+                const int gq = u & 3, h = (u >> 2) & 1, d = (u >> 3) & 3, kb = u >> 5;
+                const int k0 = kKB * kb + 64 * d + 8 * gq + 4 * h;
+                qa[m][i] = qb[m][i] = Quad{};
+                if (u < K / 8 && m < ep.rows) {
+                    if constexpr (X32) {
+                        qa[m][i] = *reinterpret_cast<const u32x4 *>(static_cast<const float *>(xv) + k0);
+                        qb[m][i] = *reinterpret_cast<const u32x4 *>(static_cast<const float *>(xv) + k0 + 32);
+                    } else {
+                        const _Float16 *row = static_cast<const _Float16 *>(xv) + (size_t)m * K;
+                        qa[m][i] = *reinterpret_cast<const u32x2 *>(row + k0);
+                        qb[m][i] = *reinterpret_cast<const u32x2 *>(row + k0 + 32);
+                    }
+                }
             }
-        }
     }
     if (ORDER == 1) {
         __builtin_amdgcn_sched_barrier(0);
@@ -134,16 +159,24 @@ __global__ __launch_bounds__(64 * WAVES) void gemv8_kernel(const void *__restric
         wq[t] = __builtin_nontemporal_load(wp + (int64_t)kblk * 64);
         __builtin_amdgcn_sched_barrier(0);                       // issue order = use order: the waits below count on it
     }
+    if constexpr (PRE) {
+        // the copies were issued before the NT weight loads and retire first: wait for them alone
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_waitcnt(vmcnt_only(NT));
+        __builtin_amdgcn_sched_barrier(0);
+    }
     // per-channel constants of the threads that will store, asked for now
     float sc = 1.f, bi = 0.f;
     uint32_t res_bits = 0;                                       // converted where it is used: no wait for it here
-    const int64_t n_out = ((int64_t)blockIdx.x * CB + (threadIdx.x >> 4)) * 16 + (threadIdx.x & 15);
-    const bool stores = threadIdx.x < 16 * CB && n_out < N;
+    const int st_m = (threadIdx.x >> 4) / CB, st_c = (threadIdx.x >> 4) % CB;     // row and channel block this thread stores
+    const int64_t n_out = ((int64_t)blockIdx.x * CB + st_c) * 16 + (threadIdx.x & 15);
+    const bool stores = threadIdx.x < 16 * CB * MR && st_m < ep.rows && n_out < N;
+    const int64_t y_at = (int64_t)st_m * N + n_out;
     if (stores) {
         if (ep.scale) sc = ep.scale[n_out];
         if (ep.bias) bi = ep.bias[n_out];
-        if (ep.residual) res_bits = ep.y_f16 ? (uint32_t)static_cast<const uint16_t *>(ep.residual)[n_out]
-                                             : static_cast<const uint32_t *>(ep.residual)[n_out];
+        if (ep.residual) res_bits = ep.y_f16 ? (uint32_t)static_cast<const uint16_t *>(ep.residual)[y_at]
+                                             : static_cast<const uint32_t *>(ep.residual)[y_at];
     }
     // fp32 rows of any magnitude: the row times the power of two that brings its largest finite |x| into
     // [1024, 2048) (exact), undone in the epilogue -- the hi / lo halves then sit well inside fp16's range. Every
@@ -155,7 +188,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemv8_kernel(const void *__restric
         for (int i = 0; i < kUnits; i++)
 #pragma unroll
             for (int e = 0; e < 4; e++) {
-                const float a = __builtin_fabsf(__builtin_bit_cast(float, qa[i][e])), b = __builtin_fabsf(__builtin_bit_cast(float, qb[i][e]));
+                const float a = __builtin_fabsf(__builtin_bit_cast(float, qa[0][i][e])), b = __builtin_fabsf(__builtin_bit_cast(float, qb[0][i][e]));
                 amax = fmaxf(amax, a < INFINITY ? a : 0.f);      // NaN and Inf take no part (they propagate anyway)
                 amax = fmaxf(amax, b < INFINITY ? b : 0.f);
             }
@@ -192,27 +225,31 @@ __global__ __launch_bounds__(64 * WAVES) void gemv8_kernel(const void *__restric
             *reinterpret_cast<u32x2 *>(planes + (p0 + m) * plane + u * 8) = u32x2{lo, hi};
         }
     };
+    if constexpr (!PRE) {
 #pragma unroll
-    for (int i = 0; i < kUnits; i++) {
-        const int u = threadIdx.x + i * 64 * WAVES;
-        if (u < K / 8) {
-            if constexpr (X32) {
-                uint32_t hi[4], lo[4];                           // pairs (0, 1), (2, 3) of quad A, then of quad B
+        for (int m = 0; m < MR; m++)
 #pragma unroll
-                for (int p = 0; p < 4; p++) {
-                    const float v0 = ps * __builtin_bit_cast(float, p < 2 ? qa[i][2 * p] : qb[i][2 * p - 4]);
-                    const float v1 = ps * __builtin_bit_cast(float, p < 2 ? qa[i][2 * p + 1] : qb[i][2 * p - 3]);
-                    const _Float16 h0 = (_Float16)v0, h1 = (_Float16)v1;
-                    const _Float16 l0 = (_Float16)(v0 - (float)h0), l1 = (_Float16)(v1 - (float)h1);
-                    hi[p] = __builtin_bit_cast(uint32_t, half2_t{h0, h1});
-                    lo[p] = __builtin_bit_cast(uint32_t, half2_t{l0, l1});
+            for (int i = 0; i < kUnits; i++) {
+                const int u = threadIdx.x + i * 64 * WAVES;
+                if (u < K / 8) {
+                    if constexpr (X32) {
+                        uint32_t hi[4], lo[4];                   // pairs (0, 1), (2, 3) of quad A, then of quad B
+#pragma unroll
+                        for (int p = 0; p < 4; p++) {
+                            const float v0 = ps * __builtin_bit_cast(float, p < 2 ? qa[0][i][2 * p] : qb[0][i][2 * p - 4]);
+                            const float v1 = ps * __builtin_bit_cast(float, p < 2 ? qa[0][i][2 * p + 1] : qb[0][i][2 * p - 3]);
+                            const _Float16 h0 = (_Float16)v0, h1 = (_Float16)v1;
+                            const _Float16 l0 = (_Float16)(v0 - (float)h0), l1 = (_Float16)(v1 - (float)h1);
+                            hi[p] = __builtin_bit_cast(uint32_t, half2_t{h0, h1});
+                            lo[p] = __builtin_bit_cast(uint32_t, half2_t{l0, l1});
+                        }
+                        write_planes(u, 0, hi[0], hi[1], hi[2], hi[3]);
+                        write_planes(u, 4, lo[0], lo[1], lo[2], lo[3]);
+                    } else {
+                        write_planes(u, 4 * m, qa[m][i][0], qa[m][i][1], qb[m][i][0], qb[m][i][1]);
+                    }
                 }
-                write_planes(u, 0, hi[0], hi[1], hi[2], hi[3]);
-                write_planes(u, 4, lo[0], lo[1], lo[2], lo[3]);
-            } else {
-                write_planes(u, 0, qa[i][0], qa[i][1], qb[i][0], qb[i][1]);
             }
-        }
     }
     __builtin_amdgcn_s_waitcnt(0xC07F);                          // lgkmcnt(0): this thread's LDS writes are done
     __builtin_amdgcn_s_barrier();                                // (not __syncthreads: that would wait for the weights too)
@@ -249,78 +286,129 @@ __global__ __launch_bounds__(64 * WAVES) void gemv8_kernel(const void *__restric
             v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x104, 0xF, 0xF, false));   // row_shl:4
         acc[r] = v;
     }
-    if (j == 0) {
+    // lanes j = 4 m now hold row m's sums (X32: lane 0 the one row's)
+    if ((j & 3) == 0 && (j >> 2) < MR) {
 #pragma unroll
-        for (int r = 0; r < 4; r++) red[wv * 16 + 4 * g + r] = acc[r];
+        for (int r = 0; r < 4; r++) red[(wv * MR + (j >> 2)) * 16 + 4 * g + r] = acc[r];
     }
     __syncthreads();
     if (stores) {
-        const int c = threadIdx.x >> 4, i16 = threadIdx.x & 15;
-        float v = red[(c * KS) * 16 + i16];
+        const int i16 = threadIdx.x & 15;
+        float v = red[((st_c * KS) * MR + st_m) * 16 + i16];
 #pragma unroll
-        for (int q = 1; q < KS; q++) v += red[(c * KS + q) * 16 + i16];
+        for (int q = 1; q < KS; q++) v += red[((st_c * KS + q) * MR + st_m) * 16 + i16];
         if constexpr (X32) v *= ps_inv;
         v = v * (sc * (1.0f / kWeightUnit)) + bi;
         if (ep.residual) v += ep.y_f16 ? (float)__builtin_bit_cast(_Float16, (uint16_t)res_bits) : __builtin_bit_cast(float, res_bits);
         if (ep.relu) v = v < 0.f ? 0.f : v;
-        if (ep.y_f16) static_cast<_Float16 *>(ep.y)[n_out] = (_Float16)v;
-        else static_cast<float *>(ep.y)[n_out] = v;
+        if (ep.y_f16) static_cast<_Float16 *>(ep.y)[y_at] = (_Float16)v;
+        else static_cast<float *>(ep.y)[y_at] = v;
     }
 }
 
-template <int WAVES, int CB, int NT, int ORDER, bool X32 = false>
+// The four bf8 term planes of M fp16 rows in the order gemv8_kernel reads them, written to memory once:
+// planes[(4 m + t) (K + 32) + 8 u .. + 7] for unit u of row m (rows beyond M: zeros).
+__global__ __launch_bounds__(256) void gemv8_prepare_kernel(const _Float16 *__restrict__ x, int M, int K,
+                                                            unsigned char *__restrict__ planes) {
+    const int plane = K + 32;
+    const int u = blockIdx.x * 256 + threadIdx.x, m = blockIdx.y;
+    if (u >= K / 8) return;
+    const int gq = u & 3, h = (u >> 2) & 1, d = (u >> 3) & 3, kb = u >> 5;
+    const int k0 = kKB * kb + 64 * d + 8 * gq + 4 * h;
+    u32x2 a = {0u, 0u}, b = {0u, 0u};
+    if (m < M) {
+        a = *reinterpret_cast<const u32x2 *>(x + (size_t)m * K + k0);
+        b = *reinterpret_cast<const u32x2 *>(x + (size_t)m * K + k0 + 32);
+    }
+    uint32_t ta0[4], ta1[4], tb0[4], tb1[4];
+    bf8_terms(a[0], ta0);
+    bf8_terms(a[1], ta1);
+    bf8_terms(b[0], tb0);
+    bf8_terms(b[1], tb1);
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+        const uint32_t lo = __builtin_amdgcn_perm(ta0[t], tb0[t], 0x07030501u);
+        const uint32_t hi = __builtin_amdgcn_perm(ta1[t], tb1[t], 0x07030501u);
+        *reinterpret_cast<u32x2 *>(planes + (size_t)(4 * m + t) * plane + u * 8) = u32x2{lo, hi};
+    }
+}
+
+constexpr size_t kGemv8LdsMax = 152 * 1024;
+
+template <int WAVES, int CB, int NT, int ORDER, bool X32 = false, int MR = 1, bool PRE = false>
 int launch_gemv8(const void *x, const void *native, int64_t Kb, int64_t N, const Gemv8Epilogue &ep, void *stream) {
     const int64_t Nb = native_blocks_n(N), grid = (Nb + CB - 1) / CB;
     if (grid > 0x7FFFFFFF) return TMQ_ERR_TOO_LARGE;
-    const size_t lds = (X32 ? 8 : 4) * (size_t)(Kb * kKB + 32) + (size_t)WAVES * 16 * sizeof(float);
-    auto kernel = gemv8_kernel<WAVES, CB, NT, ORDER, X32>;
+    size_t image = (X32 ? 8 : 4 * MR) * (size_t)(Kb * kKB + 32);
+    if (PRE) image = (image + 1023) & ~(size_t)1023;
+    const size_t lds = image + (size_t)WAVES * MR * 16 * sizeof(float);
+    if (lds > kGemv8LdsMax) return TMQ_ERR_UNSUPPORTED;
+    auto kernel = gemv8_kernel<WAVES, CB, NT, ORDER, X32, MR, PRE>;
     if (int st = allow_dynamic_lds(reinterpret_cast<const void *>(kernel), lds)) return st;
     hipLaunchKernelGGL(kernel, dim3((uint32_t)grid), dim3(64 * WAVES), lds, as_stream(stream), x,
                        static_cast<const u32x4 *>(native), (int)Kb, N, Nb, ep);
     return check_launch();
 }
 
-}  // namespace
-
-// True when the 8-bit GEMV can take a dense fp16 problem with one row.
-bool gemv8_dense_ok(const void *x, int64_t M, int64_t K) {
-    return M == 1 && K % kKB == 0 && K >= 8 * kKB && K <= 64 * kKB && aligned16(x);
-}
-
-// gemv8_dense_ok must hold. Eight wavefronts per workgroup throughout; one channel block per workgroup up to 32
-// weight blocks per channel block, two beyond when that still leaves two workgroups per CU (half as many
-// workgroups prepare the activation planes, each wavefront with up to 16 KiB of weights in flight).
-int launch_gemv8_dense(const void *x, int64_t K, const void *native, int64_t N, const float *scale, const float *bias,
-                       const void *residual, int relu, void *y, int y_f16, void *stream) {
-    const Gemv8Epilogue ep{scale, bias, residual, y, relu, y_f16};
-    const int64_t Kb = K / kKB;
+// Geometry by the number of weight blocks per channel block: eight wavefronts per workgroup throughout; one
+// channel block per workgroup up to 32 weight blocks, two beyond when that still leaves two workgroups per CU
+// (half as many workgroups prepare or copy the activation planes, each wavefront with up to 16 KiB of weights
+// in flight).
+template <bool X32, int MR, bool PRE>
+int launch_gemv8_by_blocks(const void *x, int64_t Kb, const void *native, int64_t N, const Gemv8Epilogue &ep, void *stream) {
     if (Kb <= 32) {
         switch ((Kb + 7) / 8) {                                  // blocks per wavefront, 8 wavefronts per channel block
-            case 1: return launch_gemv8<8, 1, 1, 0>(x, native, Kb, N, ep, stream);
-            case 2: return launch_gemv8<8, 1, 2, 0>(x, native, Kb, N, ep, stream);
-            case 3: return launch_gemv8<8, 1, 3, 1>(x, native, Kb, N, ep, stream);
-            default: return launch_gemv8<8, 1, 4, 1>(x, native, Kb, N, ep, stream);
+            case 1: return launch_gemv8<8, 1, 1, 0, X32, MR, PRE>(x, native, Kb, N, ep, stream);
+            case 2: return launch_gemv8<8, 1, 2, 0, X32, MR, PRE>(x, native, Kb, N, ep, stream);
+            case 3: return launch_gemv8<8, 1, 3, 1, X32, MR, PRE>(x, native, Kb, N, ep, stream);
+            default: return launch_gemv8<8, 1, 4, 1, X32, MR, PRE>(x, native, Kb, N, ep, stream);
         }
     }
-    if (native_blocks_n(N) < 512) {                              // two channel blocks per workgroup would leave CUs idle
-        switch ((Kb + 7) / 8) {
-            case 5: return launch_gemv8<8, 1, 5, 2>(x, native, Kb, N, ep, stream);
-            case 6: return launch_gemv8<8, 1, 6, 2>(x, native, Kb, N, ep, stream);
-            case 7: return launch_gemv8<8, 1, 7, 2>(x, native, Kb, N, ep, stream);
-            default: return launch_gemv8<8, 1, 8, 2>(x, native, Kb, N, ep, stream);
+    if constexpr (X32 || (MR > 1 && !PRE)) {
+        return TMQ_ERR_UNSUPPORTED;                              // the planes of such rows stop at 8192 indices
+    } else {
+        // two channel blocks per workgroup would leave CUs idle on narrow layers, and need two workgroups' LDS per CU
+        if (native_blocks_n(N) < 512) {
+            switch ((Kb + 7) / 8) {
+                case 5: return launch_gemv8<8, 1, 5, 2, false, MR, PRE>(x, native, Kb, N, ep, stream);
+                case 6: return launch_gemv8<8, 1, 6, 2, false, MR, PRE>(x, native, Kb, N, ep, stream);
+                case 7: return launch_gemv8<8, 1, 7, 2, false, MR, PRE>(x, native, Kb, N, ep, stream);
+                default: return launch_gemv8<8, 1, 8, 2, false, MR, PRE>(x, native, Kb, N, ep, stream);
+            }
+        }
+        switch ((Kb + 3) / 4) {                                  // 4 wavefronts per channel block
+            case 9: return launch_gemv8<8, 2, 9, 2, false, MR, PRE>(x, native, Kb, N, ep, stream);
+            case 10: return launch_gemv8<8, 2, 10, 2, false, MR, PRE>(x, native, Kb, N, ep, stream);
+            case 11: return launch_gemv8<8, 2, 11, 2, false, MR, PRE>(x, native, Kb, N, ep, stream);
+            case 12: return launch_gemv8<8, 2, 12, 2, false, MR, PRE>(x, native, Kb, N, ep, stream);
+            case 13: return launch_gemv8<8, 2, 13, 2, false, MR, PRE>(x, native, Kb, N, ep, stream);
+            case 14: return launch_gemv8<8, 2, 14, 2, false, MR, PRE>(x, native, Kb, N, ep, stream);
+            case 15: return launch_gemv8<8, 2, 15, 2, false, MR, PRE>(x, native, Kb, N, ep, stream);
+            case 16: return launch_gemv8<8, 2, 16, 2, false, MR, PRE>(x, native, Kb, N, ep, stream);
+            default: return TMQ_ERR_UNSUPPORTED;
         }
     }
-    switch ((Kb + 3) / 4) {                                      // 4 wavefronts per channel block
-        case 9: return launch_gemv8<8, 2, 9, 2>(x, native, Kb, N, ep, stream);
-        case 10: return launch_gemv8<8, 2, 10, 2>(x, native, Kb, N, ep, stream);
-        case 11: return launch_gemv8<8, 2, 11, 2>(x, native, Kb, N, ep, stream);
-        case 12: return launch_gemv8<8, 2, 12, 2>(x, native, Kb, N, ep, stream);
-        case 13: return launch_gemv8<8, 2, 13, 2>(x, native, Kb, N, ep, stream);
-        case 14: return launch_gemv8<8, 2, 14, 2>(x, native, Kb, N, ep, stream);
-        case 15: return launch_gemv8<8, 2, 15, 2>(x, native, Kb, N, ep, stream);
-        case 16: return launch_gemv8<8, 2, 16, 2>(x, native, Kb, N, ep, stream);
-        default: return TMQ_ERR_UNSUPPORTED;
-    }
+}
+
+}  // namespace
+
+// True when the 8-bit GEMV can take a dense fp16 problem: one row up to K = 16384; two rows up to 4096 and three
+// or four at 2048 -- every workgroup prepares the planes of all rows, and beyond 8192 values that preparation costs
+// more than the weight-stream kernel's fp16 expansion (measured: two rows at 4096^2 3.9 -> 3.6 us, four rows
+// 4.0 -> 4.9 us; two rows at 8192^2 6.2 -> 7.0 us).
+bool gemv8_dense_ok(const void *x, int64_t M, int64_t K) {
+    if (M < 1 || M > 4 || K % kKB != 0 || K < 8 * kKB || !aligned16(x)) return false;
+    return M == 1 ? K <= 64 * kKB : K * (M == 3 ? 4 : M) <= 32 * kKB;
+}
+
+// gemv8_dense_ok must hold.
+int launch_gemv8_dense(const void *x, int64_t M, int64_t K, const void *native, int64_t N, const float *scale,
+                       const float *bias, const void *residual, int relu, void *y, int y_f16, void *stream) {
+    const Gemv8Epilogue ep{scale, bias, residual, y, relu, y_f16, (int)M};
+    const int64_t Kb = K / kKB;
+    if (M == 1) return launch_gemv8_by_blocks<false, 1, false>(x, Kb, native, N, ep, stream);
+    if (M == 2) return launch_gemv8_by_blocks<false, 2, false>(x, Kb, native, N, ep, stream);
+    return launch_gemv8_by_blocks<false, 4, false>(x, Kb, native, N, ep, stream);
 }
 
 // One fp32 row: K a multiple of 256 from 2048 to 8192 (eight term planes; beyond that they leave room for one workgroup
@@ -331,15 +419,36 @@ bool gemv8_dense32_ok(const void *x, int64_t M, int64_t K) {
 
 int launch_gemv8_dense32(const void *x, int64_t K, const void *native, int64_t N, const float *scale, const float *bias,
                          const void *residual, int relu, void *y, int y_f16, void *stream) {
-    const Gemv8Epilogue ep{scale, bias, residual, y, relu, y_f16};
+    const Gemv8Epilogue ep{scale, bias, residual, y, relu, y_f16, 1};
+    return launch_gemv8_by_blocks<true, 1, false>(x, K / kKB, native, N, ep, stream);
+}
+
+// Ready-made term planes (tmq_gemv8_prepare): rows padded to 1, 2 or 4; up to 64 KiB of planes per workgroup, so
+// that two workgroups share a CU (with 128 KiB and one workgroup per CU: two rows at 16384^2 23 us against 18 for
+// the weight-stream kernel, four rows at 8192^2 9.4 against 6.4).
+int64_t gemv8_padded_rows(int64_t M) { return M <= 1 ? 1 : (M == 2 ? 2 : 4); }
+
+bool gemv8_planes_ok(int64_t M, int64_t K) {
+    return M >= 1 && M <= 4 && K % kKB == 0 && K >= 8 * kKB && gemv8_padded_rows(M) * K <= 64 * kKB;
+}
+
+int launch_gemv8_planes(const void *planes, int64_t M, int64_t K, const void *native, int64_t N, const float *scale,
+                        const float *bias, const void *residual, int relu, void *y, int y_f16, void *stream) {
+    const Gemv8Epilogue ep{scale, bias, residual, y, relu, y_f16, (int)M};
     const int64_t Kb = K / kKB;
-    switch ((Kb + 7) / 8) {
-        case 1: return launch_gemv8<8, 1, 1, 0, true>(x, native, Kb, N, ep, stream);
-        case 2: return launch_gemv8<8, 1, 2, 0, true>(x, native, Kb, N, ep, stream);
-        case 3: return launch_gemv8<8, 1, 3, 1, true>(x, native, Kb, N, ep, stream);
-        case 4: return launch_gemv8<8, 1, 4, 1, true>(x, native, Kb, N, ep, stream);
-        default: return TMQ_ERR_UNSUPPORTED;
+    switch (gemv8_padded_rows(M)) {
+        case 1: return launch_gemv8_by_blocks<false, 1, true>(planes, Kb, native, N, ep, stream);
+        case 2: return launch_gemv8_by_blocks<false, 2, true>(planes, Kb, native, N, ep, stream);
+        default: return launch_gemv8_by_blocks<false, 4, true>(planes, Kb, native, N, ep, stream);
     }
+}
+
+int launch_gemv8_prepare(const void *x, int64_t M, int64_t K, void *planes, void *stream) {
+    const int64_t mr = gemv8_padded_rows(M);
+    const dim3 grid((uint32_t)((K / 8 + 255) / 256), (uint32_t)mr);
+    hipLaunchKernelGGL(gemv8_prepare_kernel, grid, dim3(256), 0, as_stream(stream), static_cast<const _Float16 *>(x), (int)M,
+                       (int)K, static_cast<unsigned char *>(planes));
+    return check_launch();
 }
 
 }  // namespace tmq

@@ -30,8 +30,13 @@ int launch_mid_dense(const void *x, int64_t M, int64_t K, const void *native, in
                      const float *bias, const void *residual, int relu, void *y, int y_f16, void *stream);
 // gemv8.hip: one fp16 row on the 8-bit matrix instructions
 bool gemv8_dense_ok(const void *x, int64_t M, int64_t K);
-int launch_gemv8_dense(const void *x, int64_t K, const void *native, int64_t N, const float *scale, const float *bias,
+int launch_gemv8_dense(const void *x, int64_t M, int64_t K, const void *native, int64_t N, const float *scale, const float *bias,
                        const void *residual, int relu, void *y, int y_f16, void *stream);
+bool gemv8_planes_ok(int64_t M, int64_t K);
+int64_t gemv8_padded_rows(int64_t M);
+int launch_gemv8_planes(const void *planes, int64_t M, int64_t K, const void *native, int64_t N, const float *scale,
+                        const float *bias, const void *residual, int relu, void *y, int y_f16, void *stream);
+int launch_gemv8_prepare(const void *x, int64_t M, int64_t K, void *planes, void *stream);
 bool gemv8_dense32_ok(const void *x, int64_t M, int64_t K);
 int launch_gemv8_dense32(const void *x, int64_t K, const void *native, int64_t N, const float *scale, const float *bias,
                          const void *residual, int relu, void *y, int y_f16, void *stream);
@@ -1110,6 +1115,28 @@ int tmq_probe_stream_read(const void *src, size_t bytes, uint32_t *sink, void *s
     return check_launch();
 }
 
+size_t tmq_gemv8_planes_bytes(int64_t M, int64_t K) {
+    if (!gemv8_planes_ok(M, K)) return 0;
+    return (size_t)(gemv8_padded_rows(M) * 4 * (K + 32));
+}
+
+int tmq_gemv8_prepare(const void *x, int64_t M, int64_t K, void *planes, void *stream) {
+    if (!x || !planes || !aligned16(x) || !aligned16(planes)) return TMQ_ERR_INVALID_ARG;
+    if (!gemv8_planes_ok(M, K)) return TMQ_ERR_UNSUPPORTED;
+    return launch_gemv8_prepare(x, M, K, planes, stream);
+}
+
+int tmq_ternary_linear_planes(const void *planes, int64_t M, int64_t K, const void *native, int64_t N,
+                              const tmq_epilogue *epilogue, void *y, void *stream) {
+    if (K <= 0 || N <= 0) return TMQ_ERR_INVALID_ARG;
+    if (!planes || !native || !y || !aligned16(native) || !aligned16(planes)) return TMQ_ERR_INVALID_ARG;
+    if (!gemv8_planes_ok(M, K)) return TMQ_ERR_UNSUPPORTED;
+    tmq_epilogue ep = {nullptr, nullptr, nullptr, 0, TMQ_F32};
+    if (epilogue) ep = *epilogue;
+    if (ep.y_dtype != TMQ_F16 && ep.y_dtype != TMQ_F32) return TMQ_ERR_UNSUPPORTED;
+    return launch_gemv8_planes(planes, M, K, native, N, ep.scale, ep.bias, ep.residual, ep.relu, y, ep.y_dtype == TMQ_F16, stream);
+}
+
 int tmq_ternary_linear(const void *x, int x_dtype, int64_t M, int64_t K, const void *native, int64_t N,
                        const tmq_epilogue *epilogue, void *y, void *stream) {
     if (M < 0 || K <= 0 || N <= 0) return TMQ_ERR_INVALID_ARG;
@@ -1120,10 +1147,11 @@ int tmq_ternary_linear(const void *x, int x_dtype, int64_t M, int64_t K, const v
     if (epilogue) ep = *epilogue;
     if (ep.y_dtype != TMQ_F16 && ep.y_dtype != TMQ_F32) return TMQ_ERR_UNSUPPORTED;
     const bool x32 = x_dtype == TMQ_F32;
-    // One fp16 row, K a multiple of 256 from 2048 to 16384: weights and activations as 8-bit MFMA operands (gemv8.hip),
-    // half the decode work per weight of the kernels below (4096^2: 3.75 -> 3.0 us, 16384^2: 17.7 -> 15.6 us).
+    // One fp16 row, K a multiple of 256 from 2048 to 16384 (two rows to 8192, three or four to 4096): weights and
+    // activations as 8-bit MFMA operands (gemv8.hip), half the decode work per weight of the kernels below (4096^2:
+    // 3.75 -> 3.0 us, 16384^2: 17.7 -> 15.6 us).
     if (!x32 && gemv8_dense_ok(x, M, K))
-        return launch_gemv8_dense(x, K, native, N, ep.scale, ep.bias, ep.residual, ep.relu, y, ep.y_dtype == TMQ_F16, stream);
+        return launch_gemv8_dense(x, M, K, native, N, ep.scale, ep.bias, ep.residual, ep.relu, y, ep.y_dtype == TMQ_F16, stream);
     // ... and one fp32 row (the reference's GEMV convention) up to K = 8192: the same kernel on the row's two fp16 halves
     if (x32 && gemv8_dense32_ok(x, M, K))
         return launch_gemv8_dense32(x, K, native, N, ep.scale, ep.bias, ep.residual, ep.relu, y, ep.y_dtype == TMQ_F16, stream);

@@ -633,6 +633,51 @@ def ternary_linear(x: torch.Tensor, nw: NativeWeights, scale=None, bias=None, re
     return y
 
 
+class ActivationPlanes:
+    """One to four fp16 activation rows in the operand form of the 8-bit GEMV (each value as four bf8 terms), made
+    once by gemv8_prepare and multiplied with any number of layers by ternary_linear_planes."""
+
+    def __init__(self, buf, rows, K, lead):
+        self.buf, self.rows, self.K, self.lead = buf, rows, K, lead
+
+
+def gemv8_planes_supported(rows: int, K: int) -> bool:
+    """Whether gemv8_prepare / ternary_linear_planes take `rows` rows of K values (at most 4 rows, K a multiple of
+    256 from 2048 to 16384, rows padded to 1 / 2 / 4 times K at most 16384)."""
+    return _lib().tmq_gemv8_planes_bytes(int(rows), int(K)) > 0
+
+
+def gemv8_prepare(x: torch.Tensor) -> ActivationPlanes:
+    """The bf8 term planes of x (fp16 [..., K], at most four rows in all): one small launch; see ActivationPlanes."""
+    _capi.require_gpu(x, "activations")
+    if x.dtype != torch.float16:
+        raise RuntimeError("gemv8_prepare: activations must be fp16")
+    K = int(x.shape[-1])
+    M = x.numel() // K if K else 0
+    lib = _lib()
+    nbytes = lib.tmq_gemv8_planes_bytes(M, K)
+    if nbytes == 0:
+        raise RuntimeError("gemv8_prepare: at most 4 rows of K = 2048 .. 16384 (a multiple of 256), rows x K <= 16384")
+    buf = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
+    with torch.cuda.device(x.device):
+        check(lib.tmq_gemv8_prepare(ptr(x), M, K, ptr(buf), stream_of(x)), "gemv8_prepare")
+    return ActivationPlanes(buf, M, K, tuple(x.shape[:-1]))
+
+
+def ternary_linear_planes(planes: ActivationPlanes, nw: NativeWeights, scale=None, bias=None, residual=None, relu=False,
+                          out_dtype=torch.float32) -> torch.Tensor:
+    """ternary_linear on rows prepared by gemv8_prepare: same values, without the conversion every workgroup of the
+    plain call repeats."""
+    if planes.K != nw.K:
+        raise RuntimeError(f"ternary_linear_planes: activations have {planes.K} features, weights expect {nw.K}")
+    y = torch.empty(planes.lead + (nw.N,), dtype=out_dtype, device=planes.buf.device)
+    ep = _epilogue(nw, scale, bias, residual, relu, out_dtype, y)
+    with torch.cuda.device(y.device):
+        check(_lib().tmq_ternary_linear_planes(ptr(planes.buf), planes.rows, nw.K, ptr(nw.buf), nw.N, ctypes.byref(ep), ptr(y),
+                                               stream_of(y)), "ternary_linear_planes")
+    return y
+
+
 def ternary_conv2d(x: torch.Tensor, nw: NativeWeights, stride=1, padding=0, dilation=1, scale=None, bias=None,
                    residual=None, relu=False, out_dtype=torch.float32) -> torch.Tensor:
     """Implicit-GEMM ternary convolution. x: fp16 [B, C, H, W] in channels_last memory (any other
