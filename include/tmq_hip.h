@@ -297,6 +297,18 @@ typedef struct tmq_epilogue {
 int tmq_ternary_linear(const void *x, int x_dtype, int64_t M, int64_t K, const void *native,
                        int64_t N, const tmq_epilogue *epilogue, void *y, void *stream);
 
+/* tmq_ternary_linear for callers that bring a workspace (the reference's hosts allocate what they need
+ * themselves, tmq/tmq_cuda.cu:478-549; this ABI never allocates): a product whose reduction pays to be cut across
+ * workgroups -- today 17 .. 32 fp16 rows over 2^28 weights or more -- runs as slices of whole 256-index weight
+ * blocks with fp32 partial sums in the workspace, added in slice order by a second launch (deterministic, no
+ * atomics). tmq_ternary_linear_workspace_bytes returns what a shape can use (0: the single-launch kernels are at
+ * least as fast); with a NULL or smaller workspace tmq_ternary_linear_ws is tmq_ternary_linear. Same results to
+ * fp32 rounding (the summation order differs).                                                            */
+size_t tmq_ternary_linear_workspace_bytes(int x_dtype, int64_t M, int64_t K, int64_t N);
+int tmq_ternary_linear_ws(const void *x, int x_dtype, int64_t M, int64_t K, const void *native, int64_t N,
+                          const tmq_epilogue *epilogue, void *y, void *workspace, size_t workspace_bytes,
+                          void *stream);
+
 /* One to four fp16 rows with the activations already in the operand form of the 8-bit matrix instructions.
  * The GEMV for a few rows (the reference's ternaryMVFP32, tmq/tmq_cuda.cu:242-286, 563-603; its row-batched
  * caller tmq/tmq.py:680-683) multiplies fp8 weight operands with the rows carried exactly as four bf8 terms per

@@ -97,6 +97,8 @@ SIGNATURES = {
     "tmq_ternary_dwconv_patches": (_int, [_vp, _int, _i64, ctypes.c_int32, _i64, _vp, _vp, _vp]),
     "tmq_maxpool2d_nhwc": (_int, [_vp] + [ctypes.c_int32] * 10 + [_vp, _vp]),
     "tmq_avgpool_global_nhwc": (_int, [_vp, _i64, _i64, _i64, _vp, _int, _vp]),
+    "tmq_ternary_linear_workspace_bytes": (_sz, [_int, _i64, _i64, _i64]),
+    "tmq_ternary_linear_ws": (_int, [_vp, _int, _i64, _i64, _vp, _i64, _vp, _vp, _vp, _sz, _vp]),
     "tmq_gemv8_planes_bytes": (_sz, [_i64, _i64]),
     "tmq_gemv8_prepare": (_int, [_vp, _i64, _i64, _vp, _vp]),
     "tmq_ternary_linear_planes": (_int, [_vp, _i64, _i64, _vp, _i64, _vp, _vp, _vp]),

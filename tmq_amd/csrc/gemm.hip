@@ -1001,11 +1001,98 @@ int launch_gemm_dense(const void *x, int64_t M, int64_t K, const void *native, i
     return dispatch_tile(DenseLoader{static_cast<const _Float16 *>(x), M, K}, native, M, K, N, ep, stream);
 }
 
+// Adds the slices of a reduction that was cut across workgroups in slice order (deterministic) and applies the
+// epilogue. partial holds `slices` fp32 matrices [M][N] with the weight unit already divided out.
+namespace {
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *__restrict__ partial, int slices, int64_t M, int64_t N,
+                                                            Epilogue ep) {
+    const int64_t MN = M * N;
+    const bool vec = (N % 4 == 0) && ((reinterpret_cast<uintptr_t>(ep.y) | reinterpret_cast<uintptr_t>(ep.residual) |
+                                       reinterpret_cast<uintptr_t>(ep.scale) | reinterpret_cast<uintptr_t>(ep.bias)) & 15u) == 0;
+    const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i >= MN) return;
+    if (vec) {
+        floatx4 v = __builtin_nontemporal_load(reinterpret_cast<const floatx4 *>(partial + i));
+        for (int s = 1; s < slices; s++) v += __builtin_nontemporal_load(reinterpret_cast<const floatx4 *>(partial + s * MN + i));
+        const int64_t n = i % N;
+        if (ep.scale) v *= *reinterpret_cast<const floatx4 *>(ep.scale + n);
+        if (ep.bias) v += *reinterpret_cast<const floatx4 *>(ep.bias + n);
+        if (ep.residual) {
+            if (ep.y_f16) {
+                const half4 r = *reinterpret_cast<const half4 *>(static_cast<const _Float16 *>(ep.residual) + i);
+#pragma unroll
+                for (int e = 0; e < 4; e++) v[e] += (float)r[e];
+            } else {
+                v += *reinterpret_cast<const floatx4 *>(static_cast<const float *>(ep.residual) + i);
+            }
+        }
+        if (ep.relu) {
+#pragma unroll
+            for (int e = 0; e < 4; e++) v[e] = v[e] < 0.f ? 0.f : v[e];
+        }
+        if (ep.y_f16) {
+            half4 h;
+#pragma unroll
+            for (int e = 0; e < 4; e++) h[e] = (_Float16)v[e];
+            *reinterpret_cast<half4 *>(static_cast<_Float16 *>(ep.y) + i) = h;
+        } else {
+            *reinterpret_cast<floatx4 *>(static_cast<float *>(ep.y) + i) = v;
+        }
+        return;
+    }
+    for (int e = 0; e < 4 && i + e < MN; e++) {
+        const int64_t o = i + e, n = o % N;
+        float f = partial[o];
+        for (int s = 1; s < slices; s++) f += partial[s * MN + o];
+        if (ep.scale) f *= ep.scale[n];
+        if (ep.bias) f += ep.bias[n];
+        if (ep.residual) f += ep.y_f16 ? (float)static_cast<const _Float16 *>(ep.residual)[o] : static_cast<const float *>(ep.residual)[o];
+        if (ep.relu) f = f < 0.f ? 0.f : f;
+        if (ep.y_f16) static_cast<_Float16 *>(ep.y)[o] = (_Float16)f;
+        else static_cast<float *>(ep.y)[o] = f;
+    }
+}
+}  // namespace
+
+int launch_splitk_reduce(const float *partial, int slices, int64_t M, int64_t N, const Epilogue &ep, void *stream) {
+    const int64_t groups = (M * N + 1023) / 1024;
+    if (groups > 0x7FFFFFFF) return TMQ_ERR_TOO_LARGE;
+    hipLaunchKernelGGL(splitk_reduce_kernel, dim3((uint32_t)groups), dim3(256), 0, as_stream(stream), partial, slices, M, N, ep);
+    return check_launch();
+}
+
+// rows.hip: 17 .. 32 rows over a very large layer, the reduction cut across workgroups
+int rows_split_slices(const void *x, int64_t M, int64_t K, int64_t N);
+int launch_rows_split(const void *x, int64_t M, int64_t K, const void *native, int64_t N, const Epilogue &ep, float *partial,
+                      int slices, void *stream);
+
 }  // namespace tmq
 
 using namespace tmq;
 
 extern "C" {
+
+size_t tmq_ternary_linear_workspace_bytes(int x_dtype, int64_t M, int64_t K, int64_t N) {
+    if (x_dtype != TMQ_F16 || M <= 0 || K <= 0 || N <= 0) return 0;
+    static const _Float16 *const aligned = nullptr;              // the plan assumes 16-byte aligned rows; _ws checks the real pointer
+    const int slices = rows_split_slices(aligned, M, K, N);
+    return slices ? (size_t)slices * (size_t)M * (size_t)N * sizeof(float) : 0;
+}
+
+int tmq_ternary_linear_ws(const void *x, int x_dtype, int64_t M, int64_t K, const void *native, int64_t N,
+                          const tmq_epilogue *epilogue, void *y, void *workspace, size_t workspace_bytes, void *stream) {
+    if (x && native && y && x_dtype == TMQ_F16 && M > 0 && K > 0 && N > 0 && workspace && aligned16(workspace) && aligned16(native)) {
+        const int slices = rows_split_slices(x, M, K, N);
+        if (slices && workspace_bytes >= (size_t)slices * (size_t)M * (size_t)N * sizeof(float)) {
+            tmq_epilogue e = {nullptr, nullptr, nullptr, 0, TMQ_F32};
+            if (epilogue) e = *epilogue;
+            if (e.y_dtype != TMQ_F16 && e.y_dtype != TMQ_F32) return TMQ_ERR_UNSUPPORTED;
+            const Epilogue ep{e.scale, e.bias, e.residual, y, e.relu, e.y_dtype == TMQ_F16 ? 1 : 0};
+            return launch_rows_split(x, M, K, native, N, ep, static_cast<float *>(workspace), slices, stream);
+        }
+    }
+    return tmq_ternary_linear(x, x_dtype, M, K, native, N, epilogue, y, stream);
+}
 
 int64_t tmq_selfcheck_fastdiv(uint32_t divisor, const uint32_t *n, int64_t count) {
     if (divisor == 0 || divisor >= 0x80000000u || !n || count < 0) return -1;

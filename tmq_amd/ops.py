@@ -627,9 +627,17 @@ def ternary_linear(x: torch.Tensor, nw: NativeWeights, scale=None, bias=None, re
             return ternary_linear(lo, nw, scale, None, t, relu, torch.float32)
     y = torch.empty(x.shape[:-1] + (nw.N,), dtype=out_dtype, device=x.device)
     ep = _epilogue(nw, scale, bias, residual, relu, out_dtype, y)
+    lib = _lib()
+    # shapes whose reduction pays to be cut across workgroups get a workspace for the partial sums
+    wsb = lib.tmq_ternary_linear_workspace_bytes(_capi.dtype_code(x), M, nw.K, nw.N) if 16 < M <= 32 else 0
     with torch.cuda.device(x.device):
-        check(_lib().tmq_ternary_linear(ptr(x), _capi.dtype_code(x), M, nw.K, ptr(nw.buf), nw.N, ctypes.byref(ep),
-                                        ptr(y), stream_of(x)), "ternary_linear")
+        if wsb:
+            ws = torch.empty(wsb, dtype=torch.uint8, device=x.device)
+            check(lib.tmq_ternary_linear_ws(ptr(x), _capi.dtype_code(x), M, nw.K, ptr(nw.buf), nw.N, ctypes.byref(ep), ptr(y),
+                                            ptr(ws), wsb, stream_of(x)), "ternary_linear")
+        else:
+            check(lib.tmq_ternary_linear(ptr(x), _capi.dtype_code(x), M, nw.K, ptr(nw.buf), nw.N, ctypes.byref(ep),
+                                         ptr(y), stream_of(x)), "ternary_linear")
     return y
 
 
