@@ -191,6 +191,10 @@ def bench_linear(args, torch):
     scale = (0.5 + torch.rand(N, generator=gen(11))).to(dev)
     nrot = 72 if args.rotate else 1
     natives = [ops.NativeWeights(packed.clone(), N) for _ in range(nrot)]
+    if args.copy_calibration:
+        # a plain copy of known size (64 MiB read + 64 MiB written) for scaling rocprofv3's FETCH_SIZE / WRITE_SIZE
+        cal = torch.empty(1 << 24, dtype=torch.float32, device=dev)
+        torch.empty_like(cal).copy_(cal)
     out = {}
     for M in [int(m) for m in args.m_list.split(",")]:
         x = torch.randn(M, K, generator=gen(12)).half().to(dev)
@@ -505,6 +509,12 @@ def bench_resnet_infer(args, torch):
                 "tflops": round(3.627e9 * B / dt / 1e12, 2), "output_finite": finite}
 
     few = max(3, args.steps // 4)
+    if args.resnet_variant == "calibrated_fused":      # for profiling: the runner on finite activations and nothing else
+        runner = t.ResNetRunner(_resnet_for_inference(torch, dev, calibrated=True))
+        f = timed(lambda: runner(x), args.steps)
+        return {"metric": "ResNet-18 img/s", "value": f["img_s"], "unit": "img/s", "n_gpus": 1, "dtype": "f16",
+                "data": "synthetic", "config": {"workload": "configs[3]: ResNet-18/102 ternary inference, calibrated BatchNorm, "
+                                                              "tmq_amd.ResNetRunner only", "batch": B}, "calibrated": {"fused": f}}
     # ---- the configuration as worded
     model = _resnet_for_inference(torch, dev, calibrated=False)
     runner = t.ResNetRunner(model)
@@ -694,6 +704,7 @@ def main():
     ap.add_argument("--rotate", type=int, default=1)
     ap.add_argument("--gemv-floor", type=int, default=1, help="linear workload: also time the read floor and a 16384^2 GEMV")
     ap.add_argument("--batch", type=int, default=0)
+    ap.add_argument("--resnet-variant", default="all", help="resnet_infer: all | calibrated_fused (that runner only, for profiling)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build targets one GPU; --gpus N with N > 1 is not supported (the path has no "
