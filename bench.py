@@ -662,8 +662,8 @@ def bench_resnet_qat(args, torch):
            "roofline": {"bound": "hbm", "achieved": round(nbytes / tmq_ms / 1e6, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                         "frac": round(nbytes / tmq_ms / 1e6 / HBM_PEAK_GBS, 4), "traffic": None,
                         "algorithmic_bytes": nbytes,
-                        "kernel": "the step's TMQ launches: multi-tensor soft-step forward + loss (8 B/weight), loss "
-                                  "finalisation, multi-tensor backward (12 B/weight), multi-tensor clamp (8 B/weight)",
+                        "kernel": "the step's TMQ launches: multi-tensor soft-step forward + loss (8 B/weight; the sum "
+                                  "finished inside the launch), multi-tensor backward (12 B/weight), multi-tensor clamp (8 B/weight)",
                         "avg_launch_us": round(tmq_ms * 1e3, 2)}}
     if not args.no_cpu:
         res["cpu_baseline"] = cpu_baseline_qat(torch, [w.cpu() for w in ws], d, sharp, p)

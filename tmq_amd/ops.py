@@ -200,7 +200,8 @@ class SegmentTable:
 
 
 def qloss_multi(table: SegmentTable, sharpness: float, strength: float):
-    """(per_tensor_means [nseg] fp32, total [1] fp32) in one launch + an ordered finalisation."""
+    """(per_tensor_means [nseg] fp32, total [1] fp32): one launch that finishes its own sums, or one launch + an ordered
+    finalisation launch beyond that form's limits."""
     per = torch.empty(table.nseg, dtype=torch.float32, device=table.device)
     tot = torch.empty(1, dtype=torch.float32, device=table.device)
     with torch.cuda.device(table.device):
