@@ -382,6 +382,25 @@ int tmq_conv2d_out_hw(const tmq_conv_shape *s, int32_t *ho, int32_t *wo);
 int tmq_ternary_conv2d(const void *x, const tmq_conv_shape *shape, const void *native,
                        const tmq_epilogue *epilogue, void *y, void *stream);
 
+/* tmq_ternary_conv2d whose output positions go into a strided NHWC destination instead of a dense
+ * [B][Ho][Wo][N] tensor. Of the computed grid (Ho x Wo per image, tmq_conv2d_out_hw) the positions
+ * h0 <= oh < h0 + h_cnt, w0 <= ow < w0 + w_cnt are kept, the others are computed and dropped; position
+ * (b, oh, ow) is written to the N contiguous channels at
+ *   y + (b * stride_b + (oh - h0) * stride_h + (ow - w0) * stride_w) * N      (strides in pixels),
+ * and epilogue->residual, when given, is read at the same offsets. view == NULL is tmq_ternary_conv2d.
+ * This is how a transposed convolution with groups == 1 is written in one pass: each phase of its output
+ * grid is a stride-1 convolution with the taps that reach it, and its view is the phase's share of the
+ * interleaved output (stride_w = sx, stride_h = sy * Wout, stride_b = Hout * Wout, y at the phase's first
+ * position) -- no dense temporary and no strided copy, where ConvTranspose2d.compact_forward
+ * (tmq/tmq.py:1007-1042) plans a GEMM into columns followed by F.fold.                               */
+typedef struct tmq_output_view {
+    int32_t h0, w0;          /* first kept row / column of the computed grid */
+    int32_t h_cnt, w_cnt;    /* kept rows / columns */
+    int64_t stride_b, stride_h, stride_w;   /* destination strides in pixels of N elements */
+} tmq_output_view;
+int tmq_ternary_conv2d_view(const void *x, const tmq_conv_shape *shape, const void *native,
+                            const tmq_epilogue *epilogue, void *y, const tmq_output_view *view, void *stream);
+
 /* Depthwise ternary convolution (groups == channels; shape->N must equal shape->C). x: fp16 NHWC;
  * words: the reference packing of a [C][1][ky][kx] weight tensor, words[ky*kx][ceil(C/16)]
  * (tmq_pack_ternary with N = C, K = ky*kx) -- read directly, no re-tiling; y: NHWC in

@@ -37,6 +37,12 @@ class ConvShape(ctypes.Structure):
                 ("B", "C", "H", "W", "N", "ky", "kx", "sy", "sx", "py", "px", "dy", "dx", "py_end", "px_end")]
 
 
+class OutputView(ctypes.Structure):
+    """tmq_output_view of include/tmq_hip.h."""
+    _fields_ = [("h0", ctypes.c_int32), ("w0", ctypes.c_int32), ("h_cnt", ctypes.c_int32), ("w_cnt", ctypes.c_int32),
+                ("stride_b", ctypes.c_int64), ("stride_h", ctypes.c_int64), ("stride_w", ctypes.c_int64)]
+
+
 class Epilogue(ctypes.Structure):
     """tmq_epilogue of include/tmq_hip.h."""
     _fields_ = [("scale", ctypes.c_void_p), ("bias", ctypes.c_void_p), ("residual", ctypes.c_void_p),
@@ -92,6 +98,7 @@ SIGNATURES = {
     "tmq_conv2d_out_hw": (_int, [ctypes.POINTER(ConvShape), ctypes.POINTER(ctypes.c_int32),
                                  ctypes.POINTER(ctypes.c_int32)]),
     "tmq_ternary_conv2d": (_int, [_vp, ctypes.POINTER(ConvShape), _vp, _vp, _vp, _vp]),
+    "tmq_ternary_conv2d_view": (_int, [_vp, ctypes.POINTER(ConvShape), _vp, _vp, _vp, ctypes.POINTER(OutputView), _vp]),
     "tmq_ternary_conv2d_relu_maxpool": (_int, [_vp, ctypes.POINTER(ConvShape), _vp, _vp, _vp, _vp, _vp]),
     "tmq_ternary_dwconv2d": (_int, [_vp, ctypes.POINTER(ConvShape), _vp, _vp, _vp, _vp]),
     "tmq_ternary_dwconv_patches": (_int, [_vp, _int, _i64, ctypes.c_int32, _i64, _vp, _vp, _vp]),

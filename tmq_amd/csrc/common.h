@@ -94,6 +94,34 @@ struct FastDiv {
 #endif
 };
 
+// Where the rows of an implicit-GEMM convolution go when they are not consecutive in y. Row m is position
+// (b, oh, ow) of the computed output grid; the kept positions (h0 <= oh < h0 + h_cnt, the same along w) go to pixel
+// b sb + (oh - h0) sh + (ow - w0) sw of the destination (a pixel is the N contiguous channels of one position),
+// the others are dropped. A phase of a transposed convolution writes its share of the interleaved output this way.
+struct NoMap {                          // rows are consecutive: row m is pixel m (an empty member of the epilogue structs)
+    static constexpr bool kDrops = false;   // pixel() never returns -1
+#if defined(__HIPCC__)
+    __device__ __forceinline__ int64_t pixel(int64_t m) const { return m; }
+#endif
+};
+
+struct RowMap {
+    static constexpr bool kDrops = true;
+    FastDiv hw, w;                     // computed positions per image / per image row
+    int32_t h0 = 0, w0 = 0, h_cnt = 0, w_cnt = 0;
+    int64_t sb = 0, sh = 0, sw = 0;    // in pixels
+#if defined(__HIPCC__)
+    __device__ __forceinline__ int64_t pixel(int64_t m) const {      // -1: dropped
+        int rem, ow;
+        const uint32_t b = hw.divmod((uint32_t)m, rem);
+        const int oh = (int)w.divmod((uint32_t)rem, ow) - h0;
+        ow -= w0;
+        if ((uint32_t)oh >= (uint32_t)h_cnt || (uint32_t)ow >= (uint32_t)w_cnt) return -1;
+        return (int64_t)b * sb + (int64_t)oh * sh + (int64_t)ow * sw;
+    }
+#endif
+};
+
 #if defined(__HIPCC__)
 // a / b and a % b for 0 <= a, 0 < b. The GPU has no integer divider: a 64-bit division expands to
 // ~100 instructions, a 32-bit one to ~20, and index arithmetic (pixel -> batch, row, column) sits in

@@ -28,7 +28,7 @@ namespace tmq {
 // mid.hip: split-reduction kernel for outputs of a few hundred 64 x 64 tiles
 bool mid_conv_ok(const void *x, const tmq_conv_shape *s);
 int launch_mid_conv(const void *x, const tmq_conv_shape *s, int ho, int wo, const void *native, const float *scale,
-                    const float *bias, const void *residual, int relu, void *y, int y_f16, void *stream);
+                    const float *bias, const void *residual, int relu, void *y, int y_f16, const RowMap *map, void *stream);
 
 namespace {
 
@@ -361,10 +361,10 @@ struct ConvLoaderFewC {
 };
 
 // ---- the tile kernel ---------------------------------------------------------------------------------
-template <int WM, int WN, int WGM, int WGN, int D, class Loader>
+template <int WM, int WN, int WGM, int WGN, int D, class Loader, class Ep>
 __global__ __launch_bounds__(64 * WGM * WGN, 2) void tile_kernel(Loader ld, const uint32_t *__restrict__ native,
                                                               int64_t M, int64_t K, int64_t N, int64_t Kb, int64_t Nb,
-                                                              Epilogue ep, int tiles_m, int tiles_n) {
+                                                              Ep ep, int tiles_m, int tiles_n) {
     constexpr int T = 64 * WGM * WGN, BM = 16 * WM * WGM, BN = 16 * WN * WGN, CH = BM * 8 / T;
     static_assert(BM * 8 % T == 0, "chunks must divide evenly");
     // two stages: the next k-tile is written while the current one is multiplied (one barrier per tile)
@@ -520,10 +520,10 @@ __device__ __forceinline__ void load_to_lds(const void *src, unsigned char *dst)
 #endif
 }
 
-template <int WM, int WN, int WGM, int WGN, int P, class Loader>
+template <int WM, int WN, int WGM, int WGN, int P, class Loader, class Ep>
 __global__ __launch_bounds__(64 * WGM * WGN, WGM * WGN > 4 ? 1 : 2) void tile_dma_kernel(Loader ld, const uint32_t *__restrict__ native,
                                                                   int64_t M, int64_t K, int64_t N, int64_t Kb,
-                                                                  int64_t Nb, Epilogue ep, int tiles_m, int tiles_n) {
+                                                                  int64_t Nb, Ep ep, int tiles_m, int tiles_n) {
     constexpr int T = 64 * WGM * WGN, BM = 16 * WM * WGM, BN = 16 * WN * WGN, CH = BM * 8 / T, S = 2 * P;
     constexpr int kTileBytes = BM * kPitch * 2;
     static_assert(BM * 8 % T == 0 && P >= 1 && P <= 2, "geometry");
@@ -685,10 +685,10 @@ __device__ __forceinline__ void wait_vmcnt() {   // s_waitcnt vmcnt(N_), the oth
     __builtin_amdgcn_s_waitcnt(0x0F70 | (N_ & 15) | ((N_ >> 4) << 14));
 }
 
-template <int WM, int WN, int WGM, int WGN, int P, class Loader>
+template <int WM, int WN, int WGM, int WGN, int P, class Loader, class Ep>
 __global__ __launch_bounds__(64 * WGM * WGN, 1) void tile_solo_kernel(Loader ld, const uint32_t *__restrict__ native,
                                                                    int64_t M, int64_t K, int64_t N, int64_t Kb,
-                                                                   int64_t Nb, Epilogue ep, int tiles_m, int tiles_n) {
+                                                                   int64_t Nb, Ep ep, int tiles_m, int tiles_n) {
     constexpr int WG = WGM * WGN, T = 64 * WG, BM = 16 * WM * WGM, BN = 16 * WN * WGN, CH = BM * 8 / T;
     constexpr int kTileBytes = BM * kPitch * 2, kRing = 3;                 // passes in the ring, P tiles each
     static_assert(BM * 8 % T == 0 && WM >= WN && (P == 1 || P == 2) && Loader::kBuffer, "geometry");
@@ -874,13 +874,13 @@ __global__ __launch_bounds__(64 * WGM * WGN, 1) void tile_solo_kernel(Loader ld,
                        nw0, M, N, ep);
 }
 
-template <int WM, int WN, int WGM, int WGN, int P, class Loader>
-int launch_tile_solo(const Loader &ld, const void *native, int64_t M, int64_t K, int64_t N, const Epilogue &ep,
+template <int WM, int WN, int WGM, int WGN, int P, class Loader, class Ep>
+int launch_tile_solo(const Loader &ld, const void *native, int64_t M, int64_t K, int64_t N, const Ep &ep,
                      void *stream) {
     constexpr int BM = 16 * WM * WGM, BN = 16 * WN * WGN, kLds = 3 * P * BM * kPitch * 2;
     const int64_t tm = (M + BM - 1) / BM, tn = (N + BN - 1) / BN;
     if (tm * tn > 0x7FFFFFFF) return TMQ_ERR_TOO_LARGE;
-    auto kernel = tile_solo_kernel<WM, WN, WGM, WGN, P, Loader>;
+    auto kernel = tile_solo_kernel<WM, WN, WGM, WGN, P, Loader, Ep>;
     if constexpr (kLds > 64 * 1024) {
         if (int st = allow_dynamic_lds(reinterpret_cast<const void *>(kernel), kLds)) return st;
     }
@@ -890,25 +890,25 @@ int launch_tile_solo(const Loader &ld, const void *native, int64_t M, int64_t K,
     return check_launch();
 }
 
-template <int WM, int WN, int WGM, int WGN, int P, class Loader>
-int launch_tile_dma(const Loader &ld, const void *native, int64_t M, int64_t K, int64_t N, const Epilogue &ep,
+template <int WM, int WN, int WGM, int WGN, int P, class Loader, class Ep>
+int launch_tile_dma(const Loader &ld, const void *native, int64_t M, int64_t K, int64_t N, const Ep &ep,
                     void *stream) {
     constexpr int BM = 16 * WM * WGM, BN = 16 * WN * WGN;
     const int64_t tm = (M + BM - 1) / BM, tn = (N + BN - 1) / BN;
     if (tm * tn > 0x7FFFFFFF) return TMQ_ERR_TOO_LARGE;
-    hipLaunchKernelGGL((tile_dma_kernel<WM, WN, WGM, WGN, P, Loader>), dim3((uint32_t)(tm * tn)), dim3(64 * WGM * WGN), 0,
+    hipLaunchKernelGGL((tile_dma_kernel<WM, WN, WGM, WGN, P, Loader, Ep>), dim3((uint32_t)(tm * tn)), dim3(64 * WGM * WGN), 0,
                        as_stream(stream), ld, static_cast<const uint32_t *>(native), M, K, N, native_blocks_k(K),
                        native_blocks_n(N), ep, (int)tm, (int)tn);
     return check_launch();
 }
 
-template <int WM, int WN, int WGM, int WGN, int D, class Loader>
-int launch_tile(const Loader &ld, const void *native, int64_t M, int64_t K, int64_t N, const Epilogue &ep,
+template <int WM, int WN, int WGM, int WGN, int D, class Loader, class Ep>
+int launch_tile(const Loader &ld, const void *native, int64_t M, int64_t K, int64_t N, const Ep &ep,
                 void *stream) {
     constexpr int BM = 16 * WM * WGM, BN = 16 * WN * WGN;
     const int64_t tm = (M + BM - 1) / BM, tn = (N + BN - 1) / BN;
     if (tm * tn > 0x7FFFFFFF) return TMQ_ERR_TOO_LARGE;
-    hipLaunchKernelGGL((tile_kernel<WM, WN, WGM, WGN, D, Loader>), dim3((uint32_t)(tm * tn)), dim3(64 * WGM * WGN), 0,
+    hipLaunchKernelGGL((tile_kernel<WM, WN, WGM, WGN, D, Loader, Ep>), dim3((uint32_t)(tm * tn)), dim3(64 * WGM * WGN), 0,
                        as_stream(stream), ld, static_cast<const uint32_t *>(native), M, K, N, native_blocks_k(K),
                        native_blocks_n(N), ep, (int)tm, (int)tn);
     return check_launch();
@@ -931,8 +931,8 @@ Loader with_divisors(Loader ld) {
     return ld;
 }
 
-template <class Loader>
-int dispatch_tile(const Loader &ld, const void *native, int64_t M, int64_t K, int64_t N, const Epilogue &ep,
+template <class Loader, class Ep>
+int dispatch_tile(const Loader &ld, const void *native, int64_t M, int64_t K, int64_t N, const Ep &ep,
                   void *stream) {
     auto wgs = [&](int bm, int bn) { return ((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
     if constexpr (Loader::kDirect) {
@@ -1068,6 +1068,40 @@ int launch_rows_split(const void *x, int64_t M, int64_t K, const void *native, i
 
 }  // namespace tmq
 
+namespace tmq {
+namespace {
+
+// The tile kernels behind tmq_ternary_conv2d for an epilogue with consecutive rows (Epilogue) or rows scattered into a
+// strided destination (ViewEpilogue).
+template <class Ep>
+int conv_tiles(const void *x, const tmq_conv_shape *s, int ho, int wo, const void *native, const Ep &ep, void *stream) {
+    const int64_t M = (int64_t)s->B * ho * wo, K = (int64_t)s->C * s->ky * s->kx;
+    const _Float16 *xp = static_cast<const _Float16 *>(x);
+    const bool small = (int64_t)s->B * s->H * s->W * s->C < (int64_t)0x7FFFFFF0 && M < (int64_t)0x7FFFFFFF;   // 32-bit offsets and rows
+    // 129 .. 256 output channels over at least 128 tiles of 64 rows: one 64 x 256 tile per workgroup, eight
+    // wavefronts of 64 rows x 32 channels -- an im2col tile is then fetched once instead of once per 64 channels
+    // (the four such 3 x 3 convolutions of ResNet-18 at batch 64: 18.9 / 25.8 / 23.3 / 23.2 -> 14.4 / 21.4 / 21.3 / 22.0 us;
+    // the 1 x 1 downsample beside them, two k-tiles, is faster on the small tiles: 5.4 against 7.9 us)
+    if ((s->C % kBK == 0) && aligned16(x) && small && s->N > 128 && s->N <= 256 && M >= 128 * 64 && K >= 8 * kBK)
+        return launch_tile_solo<4, 2, 1, 8, 1>(with_divisors(ConvLoader64{xp, M, K, s->B, s->C, s->H, s->W, ho, wo, s->ky, s->kx,
+                                                                          s->sy, s->sx, s->py, s->px, s->dy, s->dx, {}, {}}),
+                                               native, M, K, s->N, ep, stream);
+    if ((s->C % kBK == 0) && aligned16(x) && small)
+        return dispatch_tile(with_divisors(ConvLoader64{xp, M, K, s->B, s->C, s->H, s->W, ho, wo, s->ky, s->kx, s->sy,
+                                                        s->sx, s->py, s->px, s->dy, s->dx, {}, {}}), native, M, K, s->N, ep, stream);
+    if ((s->C == 8 || s->C == 16 || s->C == 32) && aligned16(x) && small)
+        return dispatch_tile(with_divisors(ConvLoaderFewC{xp, M, K, s->B, s->C, s->H, s->W, ho, wo, s->ky, s->kx, s->sy,
+                                                          s->sx, s->py, s->px, s->dy, s->dx, {}, {}}), native, M, K, s->N, ep, stream);
+    if ((s->C % 8 == 0) && aligned16(x))
+        return dispatch_tile(ConvLoader<true>{xp, M, K, s->B, s->C, s->H, s->W, ho, wo, s->ky, s->kx, s->sy, s->sx,
+                                              s->py, s->px, s->dy, s->dx}, native, M, K, s->N, ep, stream);
+    return dispatch_tile(ConvLoader<false>{xp, M, K, s->B, s->C, s->H, s->W, ho, wo, s->ky, s->kx, s->sy, s->sx, s->py,
+                                           s->px, s->dy, s->dx}, native, M, K, s->N, ep, stream);
+}
+
+}  // namespace
+}  // namespace tmq
+
 using namespace tmq;
 
 extern "C" {
@@ -1118,6 +1152,11 @@ int tmq_conv2d_out_hw(const tmq_conv_shape *s, int32_t *ho, int32_t *wo) {
 
 int tmq_ternary_conv2d(const void *x, const tmq_conv_shape *s, const void *native, const tmq_epilogue *epilogue,
                        void *y, void *stream) {
+    return tmq_ternary_conv2d_view(x, s, native, epilogue, y, nullptr, stream);
+}
+
+int tmq_ternary_conv2d_view(const void *x, const tmq_conv_shape *s, const void *native, const tmq_epilogue *epilogue,
+                            void *y, const tmq_output_view *view, void *stream) {
     if (!s || !x || !native || !y || !aligned16(native)) return TMQ_ERR_INVALID_ARG;
     tmq_epilogue e = {nullptr, nullptr, nullptr, 0, TMQ_F32};
     if (epilogue) e = *epilogue;
@@ -1132,31 +1171,25 @@ int tmq_ternary_conv2d(const void *x, const tmq_conv_shape *s, const void *nativ
     if (ho <= 0 || wo <= 0) return TMQ_ERR_INVALID_ARG;
     const int64_t M = (int64_t)s->B * ho * wo, K = (int64_t)s->C * s->ky * s->kx;
     if (M == 0) return TMQ_OK;
-    Epilogue ep{scale, bias, residual, y, relu, y_dtype == TMQ_F16 ? 1 : 0};
-    const _Float16 *xp = static_cast<const _Float16 *>(x);
+    RowMap map;
+    if (view) {
+        // the kept part of the computed grid must lie inside it; rows are decomposed with 32-bit arithmetic
+        if (view->h0 < 0 || view->w0 < 0 || view->h_cnt < 0 || view->w_cnt < 0 || view->h0 + (int64_t)view->h_cnt > ho ||
+            view->w0 + (int64_t)view->w_cnt > wo || view->stride_b < 0 || view->stride_h < 0 || view->stride_w < 0)
+            return TMQ_ERR_INVALID_ARG;
+        if (M >= (int64_t)0x7FFFFFFF) return TMQ_ERR_TOO_LARGE;
+        if (view->h_cnt == 0 || view->w_cnt == 0) return TMQ_OK;
+        map.hw = FastDiv((uint32_t)ho * (uint32_t)wo);
+        map.w = FastDiv((uint32_t)wo);
+        map.h0 = view->h0; map.w0 = view->w0; map.h_cnt = view->h_cnt; map.w_cnt = view->w_cnt;
+        map.sb = view->stride_b; map.sh = view->stride_h; map.sw = view->stride_w;
+    }
+    const int y_f16 = y_dtype == TMQ_F16 ? 1 : 0;
     // few output tiles: split the reduction inside the workgroup (mid.hip)
     if (mid_conv_ok(x, s) && split_reduction_pays(M, K, s->N))
-        return launch_mid_conv(x, s, ho, wo, native, scale, bias, residual, relu, y, y_dtype == TMQ_F16 ? 1 : 0, stream);
-    const bool small = (int64_t)s->B * s->H * s->W * s->C < (int64_t)0x7FFFFFF0 && M < (int64_t)0x7FFFFFFF;   // 32-bit offsets and rows
-    // 129 .. 256 output channels over at least 128 tiles of 64 rows: one 64 x 256 tile per workgroup, eight
-    // wavefronts of 64 rows x 32 channels -- an im2col tile is then fetched once instead of once per 64 channels
-    // (the four such 3 x 3 convolutions of ResNet-18 at batch 64: 18.9 / 25.8 / 23.3 / 23.2 -> 14.4 / 21.4 / 21.3 / 22.0 us;
-    // the 1 x 1 downsample beside them, two k-tiles, is faster on the small tiles: 5.4 against 7.9 us)
-    if ((s->C % kBK == 0) && aligned16(x) && small && s->N > 128 && s->N <= 256 && M >= 128 * 64 && K >= 8 * kBK)
-        return launch_tile_solo<4, 2, 1, 8, 1>(with_divisors(ConvLoader64{xp, M, K, s->B, s->C, s->H, s->W, ho, wo, s->ky, s->kx,
-                                                                          s->sy, s->sx, s->py, s->px, s->dy, s->dx, {}, {}}),
-                                               native, M, K, s->N, ep, stream);
-    if ((s->C % kBK == 0) && aligned16(x) && small)
-        return dispatch_tile(with_divisors(ConvLoader64{xp, M, K, s->B, s->C, s->H, s->W, ho, wo, s->ky, s->kx, s->sy,
-                                                        s->sx, s->py, s->px, s->dy, s->dx, {}, {}}), native, M, K, s->N, ep, stream);
-    if ((s->C == 8 || s->C == 16 || s->C == 32) && aligned16(x) && small)
-        return dispatch_tile(with_divisors(ConvLoaderFewC{xp, M, K, s->B, s->C, s->H, s->W, ho, wo, s->ky, s->kx, s->sy,
-                                                          s->sx, s->py, s->px, s->dy, s->dx, {}, {}}), native, M, K, s->N, ep, stream);
-    if ((s->C % 8 == 0) && aligned16(x))
-        return dispatch_tile(ConvLoader<true>{xp, M, K, s->B, s->C, s->H, s->W, ho, wo, s->ky, s->kx, s->sy, s->sx,
-                                              s->py, s->px, s->dy, s->dx}, native, M, K, s->N, ep, stream);
-    return dispatch_tile(ConvLoader<false>{xp, M, K, s->B, s->C, s->H, s->W, ho, wo, s->ky, s->kx, s->sy, s->sx, s->py,
-                                           s->px, s->dy, s->dx}, native, M, K, s->N, ep, stream);
+        return launch_mid_conv(x, s, ho, wo, native, scale, bias, residual, relu, y, y_f16, view ? &map : nullptr, stream);
+    if (view) return conv_tiles(x, s, ho, wo, native, ViewEpilogue{scale, bias, residual, y, relu, y_f16, map}, stream);
+    return conv_tiles(x, s, ho, wo, native, Epilogue{scale, bias, residual, y, relu, y_f16, {}}, stream);
 }
 
 }  // extern "C"

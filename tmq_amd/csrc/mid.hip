@@ -34,12 +34,16 @@ namespace {
 
 __device__ const u32x4 kZeroChunk[8] = {};   // 128 zero bytes: the source of padding taps / the K tail
 
-struct MidEpilogue {
+template <class Map>
+struct MidEpilogueT {
     const float *scale, *bias;
     const void *residual;
     void *y;
     int relu, y_f16;
+    [[no_unique_address]] Map map;   // where row m goes: pixel m (NoMap, no bytes) or a strided destination (RowMap)
 };
+using MidEpilogue = MidEpilogueT<NoMap>;
+static_assert(sizeof(MidEpilogue) == 40, "the dense epilogue carries no map");
 
 // Row providers. `prepare` fixes what a lane needs for its 2 WM row pieces (load c of fragment mi
 // covers rows 8 c .. 8 c + 7; the lane's row is R = 8 c + lane / 8); `source` returns the address
@@ -143,13 +147,14 @@ struct ThreadColumns {
     floatx4 sc, bi;
 };
 
-__device__ __forceinline__ bool epilogue_vectorised(int64_t N, const MidEpilogue &ep) {
+template <class Ep>
+__device__ __forceinline__ bool epilogue_vectorised(int64_t N, const Ep &ep) {
     return (N % 4 == 0) && ((reinterpret_cast<uintptr_t>(ep.y) | reinterpret_cast<uintptr_t>(ep.residual) |
                              reinterpret_cast<uintptr_t>(ep.scale) | reinterpret_cast<uintptr_t>(ep.bias)) & 15u) == 0;
 }
 
-template <int WN>
-__device__ __forceinline__ ThreadColumns load_column_constants(int64_t n0, int64_t N, const MidEpilogue &ep) {
+template <int WN, class Ep>
+__device__ __forceinline__ ThreadColumns load_column_constants(int64_t n0, int64_t N, const Ep &ep) {
     const int64_t n = n0 + (int)(threadIdx.x % (4 * WN)) * 4;
     ThreadColumns c{{1.f, 1.f, 1.f, 1.f}, {0.f, 0.f, 0.f, 0.f}};
     if (n < N) {
@@ -177,9 +182,9 @@ __device__ __forceinline__ ThreadColumns load_column_constants(int64_t n0, int64
 // A thread keeps its columns for all its rows. Its residual values are asked for before the fragments go
 // to LDS, so that they arrive while the workgroup synchronises (and before any store of this thread: the
 // residual may be the output buffer).
-template <int WM, int WN, int WAVES>
+template <int WM, int WN, int WAVES, class Ep>
 __device__ __forceinline__ void reduce_and_store(unsigned char *smem, const floatx4 (&acc)[WM][WN], int kg, int lane,
-                                                 int64_t m0, int64_t n0, int64_t M, int64_t N, const MidEpilogue &ep,
+                                                 int64_t m0, int64_t n0, int64_t M, int64_t N, const Ep &ep,
                                                  const ThreadColumns &cc) {
     constexpr int NF = WM * WN;
     const int j = lane & 15, g = lane >> 4;
@@ -199,8 +204,10 @@ __device__ __forceinline__ void reduce_and_store(unsigned char *smem, const floa
             const int row = row0 + it * kSweep;
             const int64_t m = m0 + row;
             if (row < 16 * WM && m < M) {
-                if (ep.y_f16) res16[it] = *reinterpret_cast<const half4 *>(static_cast<const _Float16 *>(ep.residual) + m * N + n);
-                else res32[it] = *reinterpret_cast<const floatx4 *>(static_cast<const float *>(ep.residual) + m * N + n);
+                const int64_t px = ep.map.pixel(m);
+                if (decltype(ep.map)::kDrops && px < 0) continue;
+                if (ep.y_f16) res16[it] = *reinterpret_cast<const half4 *>(static_cast<const _Float16 *>(ep.residual) + px * N + n);
+                else res32[it] = *reinterpret_cast<const floatx4 *>(static_cast<const float *>(ep.residual) + px * N + n);
             }
         }
     }
@@ -230,8 +237,10 @@ __device__ __forceinline__ void reduce_and_store(unsigned char *smem, const floa
             const int row = row0 + it * kSweep;
             const int64_t m = m0 + row;
             if (row >= 16 * WM || m >= M) break;
+            const int64_t px = ep.map.pixel(m);
+            if (decltype(ep.map)::kDrops && px < 0) continue;
             floatx4 v = partial_sums(row);
-            const int64_t o = m * N + n;
+            const int64_t o = px * N + n;
             if (ep.y_f16) {
                 if (ep.residual) {
 #pragma unroll
@@ -255,8 +264,10 @@ __device__ __forceinline__ void reduce_and_store(unsigned char *smem, const floa
     for (int row = row0; row < 16 * WM; row += kSweep) {
         const int64_t m = m0 + row;
         if (m >= M) break;
+        const int64_t px = ep.map.pixel(m);
+        if (decltype(ep.map)::kDrops && px < 0) continue;
         const floatx4 v = partial_sums(row);
-        const int64_t o = m * N + n;
+        const int64_t o = px * N + n;
 #pragma unroll
         for (int r = 0; r < 4; r++) {
             if (n + r >= N) break;
@@ -272,10 +283,10 @@ __device__ __forceinline__ void reduce_and_store(unsigned char *smem, const floa
     }
 }
 
-template <int WM, int WN, int WAVES, bool BLK, class Rows, int RING = 2>
+template <int WM, int WN, int WAVES, bool BLK, class Rows, int RING, class Ep>
 __global__ __launch_bounds__(64 * WAVES) void mid_kernel(Rows rows, const u32x4 *__restrict__ native, int64_t M, int Kb,
                                                          int npairs, int64_t N, int64_t Nb, int tiles_n, int by_rows,
-                                                         MidEpilogue ep) {
+                                                         Ep ep) {
     constexpr int kFrag = 16 * 128, kSlot = WM * kFrag, kWave = RING * kSlot;   // bytes: 16 rows x 128 B per fragment
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const int lane = threadIdx.x & 63, kg = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -502,8 +513,8 @@ __global__ __launch_bounds__(64 * WAVES) void mid_kernel(Rows rows, const u32x4 
     reduce_and_store<WM, WN, WAVES>(smem, acc, kg, lane, m0, n0, M, N, ep, cc);
 }
 
-template <int WM, int WN, int WAVES, class Rows, bool BLK = false, int RING = 2>
-int launch(const Rows &rows, const void *native, int64_t M, int64_t K, int64_t N, const MidEpilogue &ep, void *stream) {
+template <int WM, int WN, int WAVES, class Rows, bool BLK = false, int RING = 2, class Ep>
+int launch(const Rows &rows, const void *native, int64_t M, int64_t K, int64_t N, const Ep &ep, void *stream) {
     constexpr int BM = 16 * WM, BN = 16 * WN;
     const int64_t tm = (M + BM - 1) / BM, tn = (N + BN - 1) / BN, Kb = native_blocks_k(K);
     if (tm * tn > 0x7FFFFFFF || Kb > (1 << 20)) return TMQ_ERR_TOO_LARGE;
@@ -511,7 +522,7 @@ int launch(const Rows &rows, const void *native, int64_t M, int64_t K, int64_t N
     constexpr size_t redb = (size_t)WAVES * WM * WN * (1024 + 64);
     constexpr size_t lds = win > redb ? win : redb;
     static_assert(lds <= 152 * 1024, "LDS budget");
-    auto kernel = mid_kernel<WM, WN, WAVES, BLK, Rows, RING>;
+    auto kernel = mid_kernel<WM, WN, WAVES, BLK, Rows, RING, Ep>;
     if (int st = allow_dynamic_lds(reinterpret_cast<const void *>(kernel), lds)) return st;
     hipLaunchKernelGGL(kernel, dim3((uint32_t)(tm * tn)), dim3(64 * WAVES), lds, as_stream(stream), rows,
                        static_cast<const u32x4 *>(native), M, (int)Kb, (int)((K + 63) / 64), N, native_blocks_n(N),
@@ -941,8 +952,8 @@ int launch_stream32(const void *x, const void *native, int64_t M, int64_t K, int
 // Geometry: 64 x 128 tiles where they save a pass over the CUs (below); else the largest smaller tile
 // that keeps most CUs busy; then as many wavefronts per tile as it takes to put about ten on every CU,
 // each with at least two pairs to multiply.
-template <class Rows>
-int dispatch(const Rows &rows, const void *native, int64_t M, int64_t K, int64_t N, const MidEpilogue &ep,
+template <class Rows, class Ep>
+int dispatch(const Rows &rows, const void *native, int64_t M, int64_t K, int64_t N, const Ep &ep,
              void *stream) {
     const int64_t npairs = (K + 63) / 64, tn = (N + 63) / 64;
     // Whole weight blocks per wavefront (one 16-byte load per lane and block instead of four dword loads) when the
@@ -1077,12 +1088,12 @@ bool mid_conv_ok(const void *x, const tmq_conv_shape *s) {
 }
 
 int launch_mid_conv(const void *x, const tmq_conv_shape *s, int ho, int wo, const void *native, const float *scale,
-                    const float *bias, const void *residual, int relu, void *y, int y_f16, void *stream) {
+                    const float *bias, const void *residual, int relu, void *y, int y_f16, const RowMap *map, void *stream) {
     const int64_t M = (int64_t)s->B * ho * wo, K = (int64_t)s->C * s->ky * s->kx;
-    MidEpilogue ep{scale, bias, residual, y, relu, y_f16};
-    return dispatch(ConvRows{static_cast<const _Float16 *>(x), M, K, s->B, s->C, s->H, s->W, ho, wo, s->ky, s->kx, s->sy,
-                             s->sx, s->py, s->px, s->dy, s->dx, FastDiv((uint32_t)wo), FastDiv((uint32_t)ho)},
-                    native, M, K, s->N, ep, stream);
+    const ConvRows rows{static_cast<const _Float16 *>(x), M, K, s->B, s->C, s->H, s->W, ho, wo, s->ky, s->kx, s->sy,
+                        s->sx, s->py, s->px, s->dy, s->dx, FastDiv((uint32_t)wo), FastDiv((uint32_t)ho)};
+    if (map) return dispatch(rows, native, M, K, s->N, MidEpilogueT<RowMap>{scale, bias, residual, y, relu, y_f16, *map}, stream);
+    return dispatch(rows, native, M, K, s->N, MidEpilogue{scale, bias, residual, y, relu, y_f16, {}}, stream);
 }
 
 }  // namespace tmq

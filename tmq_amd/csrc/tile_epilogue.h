@@ -2,24 +2,31 @@
 // optional residual and ReLU, fp32 or fp16 output, written row-wise through an LDS transpose.
 #pragma once
 
+#include "common.h"
 #include "mfma.h"
 
 namespace tmq {
 
-struct Epilogue {
+template <class Map>
+struct EpilogueT {
     const float *scale;      // [N] or null
     const float *bias;       // [N] or null
     const void *residual;    // same shape/dtype as y, or null
     void *y;
     int relu;
     int y_f16;
+    [[no_unique_address]] Map map;   // where row m goes: pixel m (NoMap, no bytes) or a strided destination (RowMap)
 };
+using Epilogue = EpilogueT<NoMap>;
+using ViewEpilogue = EpilogueT<RowMap>;
+static_assert(sizeof(Epilogue) == 40, "the dense epilogue carries no map");
 
 #if defined(__HIPCC__)
 
 // fp16 results whose rows are whole 16-byte pieces are written 8 columns (16 bytes) per lane, everything
 // else 4 columns per lane: a store instruction costs the CU's address unit the same 16 cycles either way.
-__device__ __forceinline__ bool wide_rows(const Epilogue &ep, int64_t N) {
+template <class Ep>
+__device__ __forceinline__ bool wide_rows(const Ep &ep, int64_t N) {
     return ep.y_f16 && (N % 8 == 0) &&
            ((reinterpret_cast<uintptr_t>(ep.y) | reinterpret_cast<uintptr_t>(ep.residual)) & 15u) == 0;
 }
@@ -31,8 +38,8 @@ struct ColumnConstants {
     floatx4 sc[2], bi[2];
 };
 
-template <int WN>
-__device__ __forceinline__ void load_scale_bias(const Epilogue &ep, int lane, int64_t nw0, int64_t N, ColumnConstants &cc) {
+template <int WN, class Ep>
+__device__ __forceinline__ void load_scale_bias(const Ep &ep, int lane, int64_t nw0, int64_t N, ColumnConstants &cc) {
     const bool wide = wide_rows(ep, N);
     const int64_t n = wide ? nw0 + (lane % (2 * WN)) * 8 : nw0 + (lane % (4 * WN)) * 4;
     const bool vec = (N % 4 == 0) && ((reinterpret_cast<uintptr_t>(ep.scale) | reinterpret_cast<uintptr_t>(ep.bias)) & 15u) == 0;
@@ -64,9 +71,9 @@ __device__ __forceinline__ void load_scale_bias(const Epilogue &ep, int lane, in
 // transposes one 16-row slab (16 x 16 WN values) at a time through its own slice of LDS (`slab`, the
 // idle activation buffer) and writes whole rows, 16 bytes per lane: 4 fp32 or, for wide rows, 8 fp16
 // values. cc: scale and bias of the lane's columns (load_scale_bias).
-template <int WM, int WN>
+template <int WM, int WN, class Ep>
 __device__ __forceinline__ void write_tile(float *slab, const floatx4 (&acc)[WM][WN], const ColumnConstants &cc, int lane,
-                                           int64_t mw0, int64_t nw0, int64_t M, int64_t N, const Epilogue &ep) {
+                                           int64_t mw0, int64_t nw0, int64_t M, int64_t N, const Ep &ep) {
     constexpr int kEP = 16 * WN + 4;                       // slab row pitch in floats (+4: conflict-free)
     const int r16 = lane & 15, g = lane >> 4;
     const bool vec = (N % 4 == 0) && ((reinterpret_cast<uintptr_t>(ep.y) | reinterpret_cast<uintptr_t>(ep.residual)) & 15u) == 0;
@@ -88,7 +95,9 @@ __device__ __forceinline__ void write_tile(float *slab, const floatx4 (&acc)[WM]
                 floatx4 v0 = *reinterpret_cast<const floatx4 *>(&slab[row * kEP + c8 * 8]) * cc.sc[0] + cc.bi[0];
                 floatx4 v1 = *reinterpret_cast<const floatx4 *>(&slab[row * kEP + c8 * 8 + 4]) * cc.sc[1] + cc.bi[1];
                 if (m >= M || n >= N) continue;
-                const int64_t o = m * N + n;
+                const int64_t px = ep.map.pixel(m);
+                if (decltype(ep.map)::kDrops && px < 0) continue;
+                const int64_t o = px * N + n;
                 if (ep.residual) {
                     const half8 rs = *reinterpret_cast<const half8 *>(static_cast<const _Float16 *>(ep.residual) + o);
 #pragma unroll
@@ -111,7 +120,9 @@ __device__ __forceinline__ void write_tile(float *slab, const floatx4 (&acc)[WM]
             const int64_t m = mrow0 + row, n = nw0 + c4 * 4;
             floatx4 v = *reinterpret_cast<const floatx4 *>(&slab[row * kEP + c4 * 4]) * cc.sc[0] + cc.bi[0];
             if (m >= M || n >= N) continue;
-            const int64_t o = m * N + n;
+            const int64_t px = ep.map.pixel(m);
+            if (decltype(ep.map)::kDrops && px < 0) continue;
+            const int64_t o = px * N + n;
             if (vec) {
                 if (ep.y_f16) {
                     if (ep.residual) {

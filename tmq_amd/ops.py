@@ -722,6 +722,39 @@ def ternary_conv2d(x: torch.Tensor, nw: NativeWeights, stride=1, padding=0, dila
     return y
 
 
+def ternary_conv2d_into(out: torch.Tensor, x: torch.Tensor, nw: NativeWeights, stride=1, padding=0, dilation=1, scale=None,
+                        bias=None, residual=None, relu=False, first=(0, 0)) -> torch.Tensor:
+    """ternary_conv2d written straight into `out`, a strided view [B, N, h, w] of a channels_last tensor (fp16 or
+    fp32, e.g. big[:, :, 1::2, 0::2]): output position (first[0] + i, first[1] + j) of the convolution goes to
+    out[:, :, i, j]; positions of the convolution outside that h x w window are dropped. `residual`, when given, is a
+    view with out's shape and strides. One launch, no temporary. x must already be fp16."""
+    pair = lambda v: tuple(v) if isinstance(v, (tuple, list)) else (v, v)
+    (sy, sx), (py, px), (dy, dx) = pair(stride), pair(padding), pair(dilation)
+    (py, py_end), (px, px_end) = pair(py), pair(px)
+    if not x.is_cuda or x.dim() != 4 or out.dim() != 4 or out.device != x.device:
+        raise RuntimeError("ternary_conv2d_into: expected 4-D GPU tensors on one device")
+    if x.dtype != torch.float16:
+        raise RuntimeError("ternary_conv2d_into: activations must be fp16")
+    if x.shape[1] != nw.C:
+        raise RuntimeError(f"ternary_conv2d_into: input has {x.shape[1]} channels, weights expect {nw.C}")
+    if not x.is_contiguous(memory_format=torch.channels_last):
+        x = x.contiguous(memory_format=torch.channels_last)
+    B, C, H, W = x.shape
+    N = nw.N
+    sb_, sc_, sh_, sw_ = out.stride()
+    if out.shape[0] != B or out.shape[1] != N or (N > 1 and sc_ != 1) or any(v % N for v in (sb_, sh_, sw_)):
+        raise RuntimeError("ternary_conv2d_into: out must be a [B, N, h, w] view of a channels_last tensor with N channels")
+    shp = _capi.ConvShape(B, C, H, W, N, nw.ky, nw.kx, sy, sx, py, px, dy, dx, py_end, px_end)
+    ep = _epilogue(nw, scale, bias, residual, relu, out.dtype, out)
+    view = _capi.OutputView(int(first[0]), int(first[1]), int(out.shape[2]), int(out.shape[3]), sb_ // N, sh_ // N, sw_ // N)
+    if out.numel() == 0:
+        return out
+    with torch.cuda.device(x.device):
+        check(_lib().tmq_ternary_conv2d_view(ptr(x), ctypes.byref(shp), ptr(nw.buf), ctypes.byref(ep), ptr(out),
+                                             ctypes.byref(view), stream_of(x)), "ternary_conv2d_view")
+    return out
+
+
 def ternary_conv2d_relu_maxpool(x: torch.Tensor, nw: NativeWeights, stride=1, padding=0, dilation=1, scale=None,
                                 bias=None) -> torch.Tensor:
     """max_pool2d(relu(ternary_conv2d(x) * scale + bias), 3, 2, 1), the opening of a ResNet. Arguments as

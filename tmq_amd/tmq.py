@@ -969,6 +969,8 @@ class ConvTranspose2d(Conv2d):
         bias = self.bias.data.float() if self.bias is not None else None
         if x.dtype == torch.float32:
             x, scale = ops.f32_to_f16_prescaled(x, scale, cout)     # once for all phases
+        if x.dtype != torch.float16 or not x.is_contiguous(memory_format=torch.channels_last):
+            x = x.to(dtype=torch.float16, memory_format=torch.channels_last)
         y = torch.empty((B, cout, h_out, w_out), dtype=_compact_out, device=x.device, memory_format=torch.channels_last)
         for (rh, rw), (nw, geo_h, geo_w) in phases.items():
             rows, cols = _phase_extent(rh, sy, py, h_out, H, geo_h), _phase_extent(rw, sx, px, w_out, W, geo_w)
@@ -981,9 +983,9 @@ class ConvTranspose2d(Conv2d):
                 if bias is not None:
                     target += bias.to(y.dtype).view(1, -1, 1, 1)
                 continue
-            part = ops.ternary_conv2d(x, nw, (1, 1), ((pt, pb), (pl, pr)), (geo_h[2], geo_w[2]), scale=scale, bias=bias,
-                                      out_dtype=_compact_out)
-            target.copy_(part[:, :, skip_h:skip_h + cnt_h, skip_w:skip_w + cnt_w])
+            # one launch per phase, written in place: the kernel's epilogue scatters its rows into the phase's pixels
+            ops.ternary_conv2d_into(target, x, nw, (1, 1), ((pt, pb), (pl, pr)), (geo_h[2], geo_w[2]), scale=scale, bias=bias,
+                                    first=(skip_h, skip_w))
         return y
 
     def _phase_weights(self, cin, cout, ky, kx, sy, sx, dy, dx):
