@@ -248,46 +248,52 @@ struct ConvLoader64 {
     int B, C, H, W, Ho, Wo, ky, kx, sy, sx, py, px, dy, dx;
     FastDiv by_wo, by_ho;      // set by with_divisors(); M < 2^31
 
+    // A row's window is tested against the image once: bit i of `taps` says that tap row i lies inside it, bit
+    // 16 + j the same for tap column j (ky, kx <= 15, checked by the host). A k-tile's test is then one AND and one
+    // compare against the tile's two bits instead of two additions, two compares and the scalar mask logic between them.
     template <int CH, int T>
     struct State {
-        int32_t off0[CH];          // element offset of (b, ih0, iw0, channel kc); may be negative
-        int32_t ih0[CH], iw0[CH];  // top-left input coordinate of the row's window (rows past M: far outside)
+        uint32_t off0[CH];         // byte offset of (b, ih0, iw0, channel kc); wraps below zero for padding
+        uint32_t taps[CH];         // valid tap rows / columns of the row's window (rows past M: none)
         int i, j, c0;              // uniform: tap and first channel of the current k-tile
-        int32_t delta;             // uniform: element offset of (tap, c0) relative to off0
+        uint32_t delta;            // uniform: byte offset of (tap, c0) relative to off0
+        uint32_t want;             // uniform: the current tap's two bits; bit 15 (never set in taps) past the last tap
     };
     template <int CH, int T>
     __device__ __forceinline__ void init(State<CH, T> &st, int64_t m0, int tid, int chunk) const {
         st.i = st.j = st.c0 = 0;
         st.delta = 0;
+        st.want = 1u | (1u << 16);
         const int kc = chunk * 8;
 #pragma unroll
         for (int q = 0; q < CH; q++) {
             const int64_t m = m0 + (tid >> 3) + q * (T / 8);
             st.off0[q] = 0;
-            st.ih0[q] = st.iw0[q] = INT32_MIN / 2;
+            st.taps[q] = 0;
             if (m < M) {
                 int ow, oh;
                 const uint32_t t = by_wo.divmod((uint32_t)m, ow);
                 const int b = (int)by_ho.divmod(t, oh);
-                st.ih0[q] = oh * sy - py;
-                st.iw0[q] = ow * sx - px;
-                st.off0[q] = ((b * H + st.ih0[q]) * W + st.iw0[q]) * C + kc;
+                const int ih0 = oh * sy - py, iw0 = ow * sx - px;
+                st.off0[q] = (uint32_t)(((b * H + ih0) * W + iw0) * C + kc) * 2u;
+                uint32_t bits = 0;
+                for (int i = 0; i < ky; i++) bits |= ((unsigned)(ih0 + i * dy) < (unsigned)H) ? (1u << i) : 0u;
+                for (int j = 0; j < kx; j++) bits |= ((unsigned)(iw0 + j * dx) < (unsigned)W) ? (0x10000u << j) : 0u;
+                st.taps[q] = bits;
             }
         }
     }
     template <int CH, int T>
     __device__ __forceinline__ const void *addr(const State<CH, T> &st, int64_t, int q) const {
-        const bool in = (st.i < ky) & ((unsigned)(st.ih0[q] + st.i * dy) < (unsigned)H) &
-                        ((unsigned)(st.iw0[q] + st.j * dx) < (unsigned)W);
-        return in ? static_cast<const void *>(x + (st.off0[q] + st.delta)) : static_cast<const void *>(&kZeroChunk);
+        const bool in = (st.taps[q] & st.want) == st.want;
+        return in ? static_cast<const void *>(reinterpret_cast<const unsigned char *>(x) + (st.off0[q] + st.delta))
+                  : static_cast<const void *>(&kZeroChunk);
     }
     // The same chunk as a byte offset into a buffer resource over x; padding taps and the K tail get an
     // offset past its end, for which the load delivers zeros.
     template <int CH, int T>
     __device__ __forceinline__ uint32_t offset(const State<CH, T> &st, int q) const {
-        const bool in = (st.i < ky) & ((unsigned)(st.ih0[q] + st.i * dy) < (unsigned)H) &
-                        ((unsigned)(st.iw0[q] + st.j * dx) < (unsigned)W);
-        return in ? (uint32_t)(st.off0[q] + st.delta) * 2u : kPastTheEnd;
+        return (st.taps[q] & st.want) == st.want ? st.off0[q] + st.delta : kPastTheEnd;
     }
     __device__ __forceinline__ uint32_t bytes() const { return (uint32_t)((int64_t)B * H * W * C * 2); }
     template <int CH, int T>
@@ -297,7 +303,8 @@ struct ConvLoader64 {
             st.c0 = 0;
             if (++st.j == kx) { st.j = 0; ++st.i; }   // past the last tap only in the zero-padded K tail: i >= ky
         }
-        st.delta = (st.i * dy * W + st.j * dx) * C + st.c0;
+        st.delta = (uint32_t)((st.i * dy * W + st.j * dx) * C + st.c0) * 2u;
+        st.want = st.i < ky ? (1u << st.i) | (0x10000u << st.j) : 0x8000u;
     }
 };
 
@@ -1082,11 +1089,11 @@ int conv_tiles(const void *x, const tmq_conv_shape *s, int ho, int wo, const voi
     // wavefronts of 64 rows x 32 channels -- an im2col tile is then fetched once instead of once per 64 channels
     // (the four such 3 x 3 convolutions of ResNet-18 at batch 64: 18.9 / 25.8 / 23.3 / 23.2 -> 14.4 / 21.4 / 21.3 / 22.0 us;
     // the 1 x 1 downsample beside them, two k-tiles, is faster on the small tiles: 5.4 against 7.9 us)
-    if ((s->C % kBK == 0) && aligned16(x) && small && s->N > 128 && s->N <= 256 && M >= 128 * 64 && K >= 8 * kBK)
+    if ((s->C % kBK == 0) && s->ky <= 15 && s->kx <= 15 && aligned16(x) && small && s->N > 128 && s->N <= 256 && M >= 128 * 64 && K >= 8 * kBK)
         return launch_tile_solo<4, 2, 1, 8, 1>(with_divisors(ConvLoader64{xp, M, K, s->B, s->C, s->H, s->W, ho, wo, s->ky, s->kx,
                                                                           s->sy, s->sx, s->py, s->px, s->dy, s->dx, {}, {}}),
                                                native, M, K, s->N, ep, stream);
-    if ((s->C % kBK == 0) && aligned16(x) && small)
+    if ((s->C % kBK == 0) && s->ky <= 15 && s->kx <= 15 && aligned16(x) && small)
         return dispatch_tile(with_divisors(ConvLoader64{xp, M, K, s->B, s->C, s->H, s->W, ho, wo, s->ky, s->kx, s->sy,
                                                         s->sx, s->py, s->px, s->dy, s->dx, {}, {}}), native, M, K, s->N, ep, stream);
     if ((s->C == 8 || s->C == 16 || s->C == 32) && aligned16(x) && small)

@@ -66,6 +66,97 @@ __device__ __forceinline__ void load_scale_bias(const Ep &ep, int lane, int64_t 
     }
 }
 
+// v + (float)h for the low / high half of a packed pair: one v_fma_mix_f32 (conversion and addition in one
+// instruction, rounded once -- the same value as a conversion followed by an addition).
+__device__ __forceinline__ float add_half_lo(uint32_t pair, float v) {
+    float r;
+    asm("v_fma_mix_f32 %0, %1, 1.0, %2 op_sel_hi:[1,0,0]" : "=v"(r) : "v"(pair), "v"(v));
+    return r;
+}
+__device__ __forceinline__ float add_half_hi(uint32_t pair, float v) {
+    float r;
+    asm("v_fma_mix_f32 %0, %1, 1.0, %2 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "=v"(r) : "v"(pair), "v"(v));
+    return r;
+}
+
+// write_tile for fp16 results in whole 16-byte row pieces (wide_rows): 8 columns per lane. The residual pieces of
+// up to kAhead slabs are requested before the slabs are transposed, so that their trip to memory overlaps with
+// the LDS traffic instead of standing between a slab's arithmetic and its stores; a piece's offset is computed
+// once, for the request, and kept for the store. Conversions are packed (v_cvt_pk_f16_f32), the residual is
+// added with v_fma_mix_f32.
+template <int WM, int WN, class Ep>
+__device__ __forceinline__ void write_tile_wide(float *slab, const floatx4 (&acc)[WM][WN], const ColumnConstants &cc, int lane,
+                                                int64_t mw0, int64_t nw0, int64_t M, int64_t N, const Ep &ep) {
+    typedef float float2v __attribute__((ext_vector_type(2)));
+    constexpr int kEP = 16 * WN + 4, kPieces = (WN + 1) / 2;       // pieces of 8 columns per lane and slab
+    constexpr int kAhead = WM * kPieces <= 8 ? WM : (8 / kPieces > 0 ? 8 / kPieces : 1);
+    const int r16 = lane & 15, g = lane >> 4;
+    const _Float16 *res = static_cast<const _Float16 *>(ep.residual);
+    int64_t off[kAhead][kPieces];                                  // element offset of the lane's piece, -1: none
+    u32x4 rs[kAhead][kPieces];
+    auto request = [&](int i, int slot) {
+#pragma unroll
+        for (int t = 0; t < kPieces; t++) {
+            const int idx = t * 64 + lane, row = idx / (2 * WN), c8 = idx % (2 * WN);
+            const int64_t m = mw0 + (int64_t)i * 16 + row, n = nw0 + c8 * 8;
+            int64_t o = -1;
+            if (idx < 32 * WN && m < M && n < N) {
+                const int64_t px = ep.map.pixel(m);
+                if (!decltype(ep.map)::kDrops || px >= 0) o = px * N + n;
+            }
+            off[slot][t] = o;
+            if (res && o >= 0) rs[slot][t] = *reinterpret_cast<const u32x4 *>(res + o);
+        }
+    };
+#pragma unroll
+    for (int i = 0; i < kAhead; i++) request(i, i);
+#pragma unroll
+    for (int i = 0; i < WM; i++) {
+#pragma unroll
+        for (int j = 0; j < WN; j++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) slab[(g * 4 + r) * kEP + j * 16 + r16] = acc[i][j][r];
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int t = 0; t < kPieces; t++) {
+            const int idx = t * 64 + lane, row = idx / (2 * WN), c8 = idx % (2 * WN);
+            if (idx >= 32 * WN) continue;
+            floatx4 v0 = *reinterpret_cast<const floatx4 *>(&slab[row * kEP + c8 * 8]) * cc.sc[0] + cc.bi[0];
+            floatx4 v1 = *reinterpret_cast<const floatx4 *>(&slab[row * kEP + c8 * 8 + 4]) * cc.sc[1] + cc.bi[1];
+            const int64_t o = off[i % kAhead][t];
+            if (o < 0) continue;
+            if (res) {
+                const u32x4 q = rs[i % kAhead][t];
+#pragma unroll
+                for (int e = 0; e < 2; e++) {
+                    v0[2 * e] = add_half_lo(q[e], v0[2 * e]);
+                    v0[2 * e + 1] = add_half_hi(q[e], v0[2 * e + 1]);
+                    v1[2 * e] = add_half_lo(q[2 + e], v1[2 * e]);
+                    v1[2 * e + 1] = add_half_hi(q[2 + e], v1[2 * e + 1]);
+                }
+            }
+            if (ep.relu) {
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    v0[e] = v0[e] < 0.f ? 0.f : v0[e];
+                    v1[e] = v1[e] < 0.f ? 0.f : v1[e];
+                }
+            }
+            half8 h;
+#pragma unroll
+            for (int e = 0; e < 2; e++) {
+                const half2v lo = __builtin_convertvector(float2v{v0[2 * e], v0[2 * e + 1]}, half2v);
+                const half2v hi = __builtin_convertvector(float2v{v1[2 * e], v1[2 * e + 1]}, half2v);
+                h[2 * e] = lo[0]; h[2 * e + 1] = lo[1];
+                h[4 + 2 * e] = hi[0]; h[4 + 2 * e + 1] = hi[1];
+            }
+            *reinterpret_cast<half8 *>(static_cast<_Float16 *>(ep.y) + o) = h;
+        }
+        __builtin_amdgcn_wave_barrier();
+        if (i + kAhead < WM) request(i + kAhead, i % kAhead);
+    }
+}
+
 // Epilogue of one wavefront's (16 WM) x (16 WN) accumulator block. A lane holds rows 4g + r, column
 // r16 of each 16 x 16 accumulator -- 64-byte row pieces if stored directly. Instead the wavefront
 // transposes one 16-row slab (16 x 16 WN values) at a time through its own slice of LDS (`slab`, the
@@ -77,7 +168,7 @@ __device__ __forceinline__ void write_tile(float *slab, const floatx4 (&acc)[WM]
     constexpr int kEP = 16 * WN + 4;                       // slab row pitch in floats (+4: conflict-free)
     const int r16 = lane & 15, g = lane >> 4;
     const bool vec = (N % 4 == 0) && ((reinterpret_cast<uintptr_t>(ep.y) | reinterpret_cast<uintptr_t>(ep.residual)) & 15u) == 0;
-    const bool wide = wide_rows(ep, N);
+    if (wide_rows(ep, N)) return write_tile_wide<WM, WN>(slab, acc, cc, lane, mw0, nw0, M, N, ep);
 #pragma unroll
     for (int i = 0; i < WM; i++) {
 #pragma unroll
@@ -86,34 +177,6 @@ __device__ __forceinline__ void write_tile(float *slab, const floatx4 (&acc)[WM]
             for (int r = 0; r < 4; r++) slab[(g * 4 + r) * kEP + j * 16 + r16] = acc[i][j][r];
         __builtin_amdgcn_wave_barrier();
         const int64_t mrow0 = mw0 + (int64_t)i * 16;
-        if (wide) {
-#pragma unroll
-            for (int t = 0; t < (WN + 1) / 2; t++) {           // 16 rows x 2 WN pieces of 8 columns per slab
-                const int idx = t * 64 + lane, row = idx / (2 * WN), c8 = idx % (2 * WN);
-                if (idx >= 32 * WN) continue;
-                const int64_t m = mrow0 + row, n = nw0 + c8 * 8;
-                floatx4 v0 = *reinterpret_cast<const floatx4 *>(&slab[row * kEP + c8 * 8]) * cc.sc[0] + cc.bi[0];
-                floatx4 v1 = *reinterpret_cast<const floatx4 *>(&slab[row * kEP + c8 * 8 + 4]) * cc.sc[1] + cc.bi[1];
-                if (m >= M || n >= N) continue;
-                const int64_t px = ep.map.pixel(m);
-                if (decltype(ep.map)::kDrops && px < 0) continue;
-                const int64_t o = px * N + n;
-                if (ep.residual) {
-                    const half8 rs = *reinterpret_cast<const half8 *>(static_cast<const _Float16 *>(ep.residual) + o);
-#pragma unroll
-                    for (int e = 0; e < 4; e++) { v0[e] += (float)rs[e]; v1[e] += (float)rs[4 + e]; }
-                }
-                half8 h;
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    h[e] = (_Float16)((ep.relu && v0[e] < 0.f) ? 0.f : v0[e]);
-                    h[4 + e] = (_Float16)((ep.relu && v1[e] < 0.f) ? 0.f : v1[e]);
-                }
-                *reinterpret_cast<half8 *>(static_cast<_Float16 *>(ep.y) + o) = h;
-            }
-            __builtin_amdgcn_wave_barrier();
-            continue;
-        }
 #pragma unroll
         for (int t = 0; t < WN; t++) {                     // 16 rows x (16 WN / 4) float4 = 64 WN float4 per slab
             const int idx = t * 64 + lane, row = idx / (4 * WN), c4 = idx % (4 * WN);
