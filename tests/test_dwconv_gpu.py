@@ -39,6 +39,13 @@ def test_patches_form_matches_oracle(cuda, oracle, P, T, C):
     # square 5 x 5 and 7 x 7 windows on the several-positions-per-thread kernel: strides 1 and 2, ragged widths
     (2, 24, 13, 11, 5, 1, 2, 1), (1, 16, 14, 15, 5, 2, 2, 1), (2, 8, 9, 10, 7, 1, 3, 1), (1, 40, 15, 13, 7, 2, 3, 1),
     (1, 8, 3, 3, 7, 1, 3, 1), (1, 16, 20, 17, 5, (1, 2), (2, 0), 1),
+    # rectangular and dilated windows on the same kernel: 1 .. 5 or 7 columns, any number of rows, horizontal stride and
+    # dilation of 1 or 2, any vertical ones
+    (2, 16, 12, 13, (1, 7), 1, (0, 3), 1), (1, 24, 11, 12, (5, 2), (1, 2), (2, 1), 1), (2, 8, 10, 10, 4, 2, 1, 1),
+    (1, 32, 16, 15, 3, 2, 2, 2), (1, 16, 17, 16, (3, 5), 1, (3, 4), (3, 2)), (2, 8, 9, 9, (7, 1), 1, (3, 0), 1),
+    (1, 8, 18, 19, (2, 7), 1, (1, 6), (1, 2)), (1, 16, 21, 22, (9, 4), (3, 2), (4, 3), (1, 2)), (2, 8, 8, 30, (1, 5), (1, 2), (0, 4), (1, 2)),
+    # what stays on the one-position-per-thread kernel: 6 columns, horizontal dilation 3, horizontal stride 3
+    (1, 8, 9, 12, (2, 6), 1, (0, 2), 1), (1, 8, 10, 14, 3, 1, 3, 3), (1, 16, 9, 13, 3, 3, 1, 1),
 ])
 def test_image_form_exact_on_integers(cuda, B, C, H, W, k, stride, pad, dil):
     """Small-integer activations: every product and sum is exact, so the result must equal torch's

@@ -23,6 +23,8 @@
 //   * columns: y[b][c T + t][p] = x[b][p][c] * T[c][t], the calling convention of the reference's
 //     ternary_dwconvtrans_cuda (tmq/tmq_cuda.cu:118-162, host 645-686; caller tmq/tmq.py:1026-1029),
 //     whose result the caller scatters with F.fold. Pure data movement: 4 B in, 4 T B out per element.
+#include <type_traits>
+
 #include "common.h"
 #include "mfma.h"
 
@@ -170,18 +172,21 @@ __global__ __launch_bounds__(256) void dwconv_image_kernel(const _Float16 *__res
     else store8(ep, p * C + c0, c0, C, acc, vec);
 }
 
-// The common cases -- KS x KS taps (3, 5 or 7), no dilation, whole groups of 8 channels, fewer than 2^31 threads. A
+// The common cases -- windows of ky rows x KS columns (KS of 1 .. 5 or 7, any ky), horizontal stride 1 or 2 and
+// dilation DX of 1 or 2, any vertical stride and dilation, whole groups of 8 channels, fewer than 2^31 threads. A
 // thread owns 8 channels of PX horizontally adjacent output positions: the columns their windows share are loaded once
 // (for stride 1, PX + KS - 1 columns per row instead of KS PX), the 8 weights of a tap are expanded to floats once
 // for all PX positions, and the index arithmetic is multiply-high (FastDiv). All loads of a row are in
 // flight together; taps outside the image read the clamped pixel and are replaced by zero. Per output the
 // taps are accumulated in the same order as in dwconv_image_kernel (fp32, every product exact).
-template <int KS, int PX, int SX>
+// KY: the window's rows when they equal KS and neither direction is dilated (the square windows of the common
+// depthwise layers keep a compile-time row count), 0: ky and dy from the arguments.
+template <int KS, int PX, int SX, int DX = 1, int KY = 0>
 __global__ __launch_bounds__(256) void dwconv_square_image_kernel(const _Float16 *__restrict__ x, const uint32_t *__restrict__ words,
                                                               uint32_t total, int C, int H, int W, int Wo, FastDiv by_g,
-                                                              FastDiv by_wg, FastDiv by_ho, int sy, int py, int px,
-                                                              DwEpilogue ep) {
-    constexpr int NC = (PX - 1) * SX + KS;                         // input columns the PX windows cover
+                                                              FastDiv by_wg, FastDiv by_ho, int ky, int sy, int py, int px,
+                                                              int dy, DwEpilogue ep) {
+    constexpr int NC = (PX - 1) * SX + (KS - 1) * DX + 1;          // input columns the PX windows cover
     const uint32_t id = blockIdx.x * 256u + threadIdx.x;
     if (id >= total) return;
     int cg, wg, oh;
@@ -198,20 +203,30 @@ __global__ __launch_bounds__(256) void dwconv_square_image_kernel(const _Float16
 #pragma unroll
         for (int e = 0; e < 8; e++) acc[q][e] = 0.f;
 
+    const int rows = KY ? KY : ky, step = KY ? 1 : dy;
 #pragma unroll 1
-    for (int i = 0; i < KS; i++) {                                 // one row at a time: its NC loads in flight, few registers
-        const int ih = oh * sy - py + i;
+    for (int i = 0; i < rows; i++) {                               // one row at a time: its NC loads in flight, few registers
+        const int ih = oh * sy - py + i * step;
         const bool row_in = (unsigned)ih < (unsigned)H;
         const int ihc = ih < 0 ? 0 : (ih >= H ? H - 1 : ih);
         const _Float16 *row = img + (int64_t)ihc * W * C;
+        // a column is needed when some window reads it: c = q SX + j DX (with stride and dilation both 2, every other one)
+        constexpr auto used = [](int c) {
+            for (int q = 0; q < PX; q++)
+                for (int j = 0; j < KS; j++)
+                    if (q * SX + j * DX == c) return true;
+            return false;
+        };
         half8 v[NC];
 #pragma unroll
         for (int c = 0; c < NC; c++) {
+            if (!used(c)) continue;
             const int iw = iw0 + c, iwc = iw < 0 ? 0 : (iw >= W ? W - 1 : iw);
             v[c] = *reinterpret_cast<const half8 *>(row + (int64_t)iwc * C);
         }
 #pragma unroll
         for (int c = 0; c < NC; c++) {
+            if (!used(c)) continue;
             const int iw = iw0 + c;
             if (!(row_in && (unsigned)iw < (unsigned)W)) v[c] = half8{0, 0, 0, 0, 0, 0, 0, 0};
         }
@@ -227,7 +242,7 @@ __global__ __launch_bounds__(256) void dwconv_square_image_kernel(const _Float16
 #pragma unroll
             for (int q = 0; q < PX; q++)
 #pragma unroll
-                for (int e = 0; e < 8; e++) acc[q][e] = __builtin_fmaf((float)v[q * SX + j][e], w[e], acc[q][e]);
+                for (int e = 0; e < 8; e++) acc[q][e] = __builtin_fmaf((float)v[q * SX + j * DX][e], w[e], acc[q][e]);
         }
     }
     // epilogue: the 8 channels' scale and bias once for all PX positions, 16-byte accesses throughout
@@ -369,24 +384,44 @@ int tmq_ternary_dwconv2d(const void *x, const tmq_conv_shape *s, const uint32_t 
     int vec = (s->C % 8 == 0) && aligned_for(x, 16) && aligned_for(y, ya) && (!e.residual || aligned_for(e.residual, ya));
     if (vec && aligned_for(e.scale, 16) && aligned_for(e.bias, 16)) vec |= 2;       // the 16-byte epilogue as well
     DwEpilogue ep{e.scale, e.bias, e.residual, y, e.relu, y_f16};
-    const bool square = s->ky == s->kx && (s->ky == 3 || s->ky == 5 || s->ky == 7);
-    if ((vec & 2) && square && s->dy == 1 && s->dx == 1 && (s->sx == 1 || s->sx == 2) && total < (int64_t)0x7FFFFFFF &&
+    const bool columns = (s->kx >= 1 && s->kx <= 5) || s->kx == 7;
+    if ((vec & 2) && columns && (s->dx == 1 || s->dx == 2) && (s->sx == 1 || s->sx == 2) && total < (int64_t)0x7FFFFFFF &&
         (int64_t)s->B * ho * wo < (int64_t)0x7FFFFFFF) {
-        // output positions per thread, measured: 4 except at stride 2 with 3 x 3 or 5 x 5 windows (the windows then
-        // share few columns, and 4 positions would hold 9 or 11 columns of a row in registers)
-        const int px_per_thread = (s->sx == 1 || s->ky == 7) ? 4 : 2;
+        // output positions per thread, measured on square windows: 4 except at stride 2 with fewer than 7 columns (the
+        // windows then share few columns, and 4 positions would hold 9 or 11 columns of a row in registers); dilated
+        // windows: 4 while that keeps at most 11 columns of a row in registers
+        const int px_per_thread = s->dx == 1 ? ((s->sx == 1 || s->kx == 7) ? 4 : 2) : (s->kx <= (s->sx == 1 ? 4 : 3) ? 4 : 2);
         const int64_t wgroups = (wo + px_per_thread - 1) / px_per_thread, G = s->C / 8;
         const int64_t threads = (int64_t)s->B * ho * wgroups * G, nblocks = (threads + 255) / 256;
         const FastDiv by_g((uint32_t)G), by_wg((uint32_t)wgroups), by_ho((uint32_t)ho);
         auto go = [&](auto kernel) {
             hipLaunchKernelGGL(kernel, dim3((uint32_t)nblocks), dim3(256), 0, as_stream(stream),
                                static_cast<const _Float16 *>(x), words, (uint32_t)threads, s->C, s->H, s->W, wo, by_g, by_wg,
-                               by_ho, s->sy, s->py, s->px, ep);
+                               by_ho, s->ky, s->sy, s->py, s->px, s->dy, ep);
             return check_launch();
         };
-        if (s->ky == 3) return s->sx == 1 ? go(dwconv_square_image_kernel<3, 4, 1>) : go(dwconv_square_image_kernel<3, 2, 2>);
-        if (s->ky == 5) return s->sx == 1 ? go(dwconv_square_image_kernel<5, 4, 1>) : go(dwconv_square_image_kernel<5, 2, 2>);
-        return s->sx == 1 ? go(dwconv_square_image_kernel<7, 4, 1>) : go(dwconv_square_image_kernel<7, 4, 2>);
+        auto by_positions = [&](auto ks, auto sx, auto dx) {
+            constexpr int KS = decltype(ks)::value, SX = decltype(sx)::value, DX = decltype(dx)::value;
+            if constexpr (DX == 1 && (KS == 3 || KS == 5 || KS == 7)) {
+                if (s->ky == KS && s->dy == 1)
+                    return px_per_thread == 4 ? go(dwconv_square_image_kernel<KS, 4, SX, 1, KS>) : go(dwconv_square_image_kernel<KS, 2, SX, 1, KS>);
+            }
+            return px_per_thread == 4 ? go(dwconv_square_image_kernel<KS, 4, SX, DX>) : go(dwconv_square_image_kernel<KS, 2, SX, DX>);
+        };
+        auto by_step = [&](auto ks) {
+            using one = std::integral_constant<int, 1>;
+            using two = std::integral_constant<int, 2>;
+            if (s->sx == 1) return s->dx == 1 ? by_positions(ks, one{}, one{}) : by_positions(ks, one{}, two{});
+            return s->dx == 1 ? by_positions(ks, two{}, one{}) : by_positions(ks, two{}, two{});
+        };
+        switch (s->kx) {
+            case 1: return by_step(std::integral_constant<int, 1>{});
+            case 2: return by_step(std::integral_constant<int, 2>{});
+            case 3: return by_step(std::integral_constant<int, 3>{});
+            case 4: return by_step(std::integral_constant<int, 4>{});
+            case 5: return by_step(std::integral_constant<int, 5>{});
+            default: return by_step(std::integral_constant<int, 7>{});
+        }
     }
     hipLaunchKernelGGL(dwconv_image_kernel, dim3((uint32_t)blocks), dim3(256), 0, as_stream(stream),
                        static_cast<const _Float16 *>(x), words, s->B, s->C, s->H, s->W, ho, wo, s->ky, s->kx, s->sy, s->sx,
