@@ -225,3 +225,26 @@ def test_resnet_layer_shapes_against_torch(cuda):
         ref = torch.nn.functional.conv2d(x.to(cuda).float(), Wt.to(cuda), None, s, p)
         err = (y - ref).abs().max().item() / ref.abs().max().item()
         assert err <= 1e-5, (C, HW, N, k, err)
+
+
+@pytest.mark.parametrize("B,C,HW,N,k,s,p", [(64, 128, 28, 128, 3, 1, 1), (64, 64, 54, 128, 3, 2, 1), (59, 64, 27, 128, 3, 1, 1)])
+def test_conv_on_112_row_tiles(cuda, B, C, HW, N, k, s, p):
+    """Between one and two 128 x 128 tiles per CU: the convolution runs on 112-row tiles that are loaded as 128 rows
+    (whole, ragged in the last tile, and with rows that do not divide by 112). Against torch's fp64 convolution
+    (a12: tmq/tmq.py:822-871), with residual, ReLU and fp16 output as the networks use it."""
+    from tmq_amd import ops
+    g = torch.Generator(device=cuda).manual_seed(B + HW)
+    Wt = torch.randint(-1, 2, (N, C, k, k), device=cuda, generator=g).float()
+    x = torch.randn((B, C, HW, HW), device=cuda, generator=g).half().contiguous(memory_format=torch.channels_last)
+    nw = ops.NativeWeights(ops.compactify_ternary(Wt), N, conv_kernel=(k, k))
+    scale = (torch.rand(N, device=cuda, generator=g) + 0.5) * 0.03
+    bias = torch.randn(N, device=cuda, generator=g)
+    ref = torch.nn.functional.conv2d(x.double(), Wt.double(), None, s, p) * scale.double().view(1, -1, 1, 1) + bias.double().view(1, -1, 1, 1)
+    M = ref.shape[0] * ref.shape[2] * ref.shape[3]
+    assert (M + 127) // 128 > 256 and (M + 111) // 112 <= 512           # the shape the rule is for
+    y = ops.ternary_conv2d(x, nw, s, p, 1, scale, bias)
+    assert ((y.double() - ref).abs().max() / ref.abs().max()).item() <= 2e-5
+    res = torch.randn(ref.shape, device=cuda, generator=g).half().contiguous(memory_format=torch.channels_last)
+    y16 = ops.ternary_conv2d(x, nw, s, p, 1, scale, bias, residual=res, relu=True, out_dtype=torch.float16)
+    want = torch.relu(ref + res.double())
+    assert ((y16.double() - want).abs().max() / want.abs().max()).item() <= 1e-3

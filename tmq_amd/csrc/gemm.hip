@@ -531,10 +531,13 @@ template <int WM, int WN, int WGM, int WGN, int P, class Loader, class Ep>
 __global__ __launch_bounds__(64 * WGM * WGN, WGM * WGN > 4 ? 1 : 2) void tile_dma_kernel(Loader ld, const uint32_t *__restrict__ native,
                                                                   int64_t M, int64_t K, int64_t N, int64_t Kb,
                                                                   int64_t Nb, Ep ep, int tiles_m, int tiles_n) {
-    constexpr int T = 64 * WGM * WGN, BM = 16 * WM * WGM, BN = 16 * WN * WGN, CH = BM * 8 / T, S = 2 * P;
-    constexpr int kTileBytes = BM * kPitch * 2;
-    static_assert(BM * 8 % T == 0 && P >= 1 && P <= 2, "geometry");
-    __shared__ __attribute__((aligned(16))) _Float16 As[S][BM * kPitch];
+    // BL: rows per tile as loaded -- BM rounded up to whole chunk rounds of the workgroup (a 112-row tile of four
+    // wavefronts is loaded as 128 rows: the 16 extra rows are the next tile's, fetched and never read)
+    constexpr int T = 64 * WGM * WGN, BM = 16 * WM * WGM, BN = 16 * WN * WGN, BL = (BM * 8 + T - 1) / T * T / 8;
+    constexpr int CH = BL * 8 / T, S = 2 * P;
+    constexpr int kTileBytes = BL * kPitch * 2;
+    static_assert(P >= 1 && P <= 2, "geometry");
+    __shared__ __attribute__((aligned(16))) _Float16 As[S][BL * kPitch];
 
     int id = blockIdx.x;
     const int G = tiles_m * tiles_n;
@@ -601,7 +604,7 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGM * WGN > 4 ? 1 : 2) void tile_dm
     auto swz = [&](int i, int s) { return i * 16 * kPitch + (((4 * s + g) ^ (r16 & 7)) * 8); };
     // one k-tile out of ring buffer `slot`: operand reads four ahead of the MFMAs that use them
     auto multiply = [&](int slot, const uint32_t (&w)[WN]) {
-        const _Float16 *abase = &As[0][0] + slot * (BM * kPitch) + arow;
+        const _Float16 *abase = &As[0][0] + slot * (BL * kPitch) + arow;
         constexpr int NQ = 2 * WM, kAhead = NQ < 4 ? NQ : 4;
         half8 a[NQ];
         half8 bfr[2][WN];
@@ -957,6 +960,14 @@ int dispatch_tile(const Loader &ld, const void *native, int64_t M, int64_t K, in
         if (N > 128 && wgs(128, 256) >= 384)
             return two ? launch_tile_dma<8, 4, 1, 4, 2>(ld, native, M, K, N, ep, stream)
                        : launch_tile_dma<8, 4, 1, 4, 1>(ld, native, M, K, N, ep, stream);
+        // Convolutions whose 128 x 128 tiles come to between one and two per CU (all resident at once, two workgroups
+        // per CU): 112-row tiles, while those are all resident too, leave every workgroup an eighth less to do for the
+        // same number of rounds -- 128 -> 128 channels on 28 x 28 at batch 64 (392 tiles -> 448) 24.2 -> 22.7 us, the
+        // strided 64 -> 128 before it 16.9 -> 16.5; 96-row tiles (523) would need a third round.
+        if constexpr (std::is_same<Loader, ConvLoader64>::value) {
+            if (N % 128 == 0 && wgs(128, 128) > 256 && wgs(112, 128) <= 512)
+                return launch_tile_dma<7, 2, 1, 4, 1>(ld, native, M, K, N, ep, stream);
+        }
         if (N > 64 && wgs(128, 128) >= 256) {
             const bool one = wgs(128, 128) <= 256;      // at most one workgroup per CU
             if (Loader::kConv || one)
