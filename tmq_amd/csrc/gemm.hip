@@ -239,6 +239,18 @@ struct ConvLoader {
 // 64 consecutive channels of ONE filter tap, so tap and channel offset are the same for the whole
 // workgroup and live in scalar registers. Per row the loader keeps one 32-bit element offset and the
 // window's top-left coordinate; a fetch is two unsigned compares, one add and the load.
+// Bit t set when 0 <= x0 + t d < limit, for the taps t = 0 .. n - 1 (n <= 15) of one axis of a window that starts at x0.
+// Without dilation the taps inside are a run lo .. hi, built from two shifts; dilated windows test tap by tap.
+__device__ __forceinline__ uint32_t taps_inside(int x0, int n, int d, int limit) {
+    if (d == 1) {
+        const int lo = x0 < 0 ? -x0 : 0, hi = (limit - x0 < n ? limit - x0 : n) - 1;      // first and last tap inside
+        return hi >= lo ? ((2u << hi) - 1u) & ~((1u << lo) - 1u) : 0u;
+    }
+    uint32_t bits = 0;
+    for (int t = 0; t < n; t++) bits |= ((unsigned)(x0 + t * d) < (unsigned)limit) ? (1u << t) : 0u;
+    return bits;
+}
+
 struct ConvLoader64 {
     static constexpr bool kDirect = true;
     [[maybe_unused]] static constexpr bool kConv = true;
@@ -276,10 +288,7 @@ struct ConvLoader64 {
                 const int b = (int)by_ho.divmod(t, oh);
                 const int ih0 = oh * sy - py, iw0 = ow * sx - px;
                 st.off0[q] = (uint32_t)(((b * H + ih0) * W + iw0) * C + kc) * 2u;
-                uint32_t bits = 0;
-                for (int i = 0; i < ky; i++) bits |= ((unsigned)(ih0 + i * dy) < (unsigned)H) ? (1u << i) : 0u;
-                for (int j = 0; j < kx; j++) bits |= ((unsigned)(iw0 + j * dx) < (unsigned)W) ? (0x10000u << j) : 0u;
-                st.taps[q] = bits;
+                st.taps[q] = taps_inside(ih0, ky, dy, H) | (taps_inside(iw0, kx, dx, W) << 16);
             }
         }
     }
