@@ -114,7 +114,7 @@ class ResNetRunner:
     conv1 / bn1 / conv2 / bn2 [/ conv3 / bn3] and an optional downsample = (conv, bn)), avgpool (global), fc.
     Every convolution is one ternary implicit-GEMM launch with BatchNorm, ReLU and the residual add in its epilogue,
     activations are fp16 channels_last between the layers, the opening is one kernel (FoldedStem). ResNet-18 at
-    batch 64 is 22 launches. Takes an fp16 (or fp32) NCHW batch, returns fp32 logits."""
+    batch 64 is 23 launches. Takes an fp16 (or fp32) NCHW batch, returns fp32 logits."""
 
     def __init__(self, model):
         self.stem = FoldedStem(model.conv1, model.bn1)
