@@ -1,10 +1,11 @@
 """Seeded walks over the shapes that decide which kernel family a ternary product takes: single rows and
 few rows (8-bit GEMV, weight stream, short reductions, skinny), mid-size dense products (split reduction,
 tile kernels), convolutions (three loaders, two tile families, the split-reduction form) and the fused
-opening (one kernel or two). Every case is checked against an fp64 product of the same operands
+opening (one kernel or two), convolutions written into strided views, transposed convolutions and depthwise windows.
+Every case is checked against an fp64 product of the same operands
 (a11 / a12: tmq/tmq_cuda.cu:478-549, tmq/tmq.py:662-688, 822-871 compute the same sums in fp32), the fused
 opening bit for bit against the two separate kernels. Each walk stops at its first failure and prints the
-case before it runs it, so that a fault names its shape. About 100 cases per walk, well under a minute in all.
+case before it runs it, so that a fault names its shape. About 100 cases per walk, about a minute in all.
 """
 import random
 
@@ -125,3 +126,95 @@ def test_walk_fused_opening(cuda):
                 ref = (ref * scale.double().view(1, -1, 1, 1) + bias.double().view(1, -1, 1, 1)).clamp_min(0)
                 err = ((full.double() - ref).abs().max() / ref.abs().max().clamp_min(1e-30)).item()
                 assert err <= 2e-3, (desc, err)          # fp16 outputs
+
+
+def test_walk_convolutions_into_views(cuda):
+    """tmq_ternary_conv2d_view over all loaders and tile families: a random window of the computed grid, written into a
+    strided destination, must equal the dense call followed by a copy bit for bit, and touch nothing else."""
+    from tmq_amd import ops
+    rnd = random.Random(5)
+    done = 0
+    for i in range(110):
+        C = rnd.choice([64, 128, 8, 16, 32, 24, 5, 192])
+        k = (rnd.randint(1, 4), rnd.randint(1, 4))
+        N = rnd.choice([8, 16, 40, 64, 128, 192, 256, 7])
+        B = rnd.randint(1, 6)
+        H, W = rnd.randint(k[0], 30), rnd.randint(k[1], 30)
+        pad = ((rnd.randint(0, 2), rnd.randint(0, 2)), (rnd.randint(0, 2), rnd.randint(0, 2)))
+        dil = (rnd.randint(1, 2), rnd.randint(1, 2))
+        if (k[0] - 1) * dil[0] + 1 > H + sum(pad[0]) or (k[1] - 1) * dil[1] + 1 > W + sum(pad[1]):
+            continue
+        dtype = rnd.choice([torch.float16, torch.float32])
+        desc = (B, C, H, W, N, k, pad, dil, str(dtype))
+        print("fuzz view", i, desc, flush=True)
+        g = torch.Generator(device=cuda).manual_seed(5000 + i)
+        Wt = torch.randint(-1, 2, (N, C) + k, device=cuda, generator=g).float()
+        nw = ops.NativeWeights(ops.compactify_ternary(Wt), N, conv_kernel=k)
+        x = torch.randn((B, C, H, W), device=cuda, generator=g).half().contiguous(memory_format=torch.channels_last)
+        scale = torch.rand(N, device=cuda, generator=g) * 0.1
+        bias = torch.randn(N, device=cuda, generator=g)
+        dense = ops.ternary_conv2d(x, nw, 1, pad, dil, scale, bias, out_dtype=dtype)
+        ho, wo = dense.shape[2:]
+        h0, w0 = rnd.randint(0, ho - 1), rnd.randint(0, wo - 1)
+        hc, wc = rnd.randint(1, ho - h0), rnd.randint(1, wo - w0)
+        sy, sx, oy, ox = rnd.randint(1, 3), rnd.randint(1, 3), rnd.randint(0, 2), rnd.randint(0, 2)
+        big = torch.full((B, N, oy + sy * hc + 1, ox + sx * wc + 1), 3.0, dtype=dtype, device=cuda).contiguous(memory_format=torch.channels_last)
+        want = big.clone()
+        want[:, :, oy:oy + sy * hc:sy, ox:ox + sx * wc:sx] = dense[:, :, h0:h0 + hc, w0:w0 + wc]
+        ops.ternary_conv2d_into(big[:, :, oy:oy + sy * hc:sy, ox:ox + sx * wc:sx], x, nw, 1, pad, dil, scale, bias, first=(h0, w0))
+        assert torch.equal(big, want), desc
+        done += 1
+    assert done >= 80
+
+
+def test_walk_transposed_and_depthwise(cuda):
+    """Transposed convolutions (one stride-1 convolution per output phase, written in place; a14 / f4:
+    tmq/tmq.py:1007-1042) and depthwise windows of every shape (tmq/tmq_cuda.cu:166-238) on small integers, where every
+    product and sum is exact: equal to torch's own operators on the ternarised weights bit for bit."""
+    import tmq_amd as t
+    from tmq_amd import ops
+    rnd = random.Random(6)
+    for i in range(45):
+        cin, cout = rnd.choice([4, 8, 16, 64, 24]), rnd.choice([4, 8, 16, 64, 40])
+        k = (rnd.randint(1, 5), rnd.randint(1, 5))
+        s = (rnd.randint(1, 3), rnd.randint(1, 3))
+        d = (rnd.randint(1, 2), rnd.randint(1, 2))
+        p = (rnd.randint(0, 2), rnd.randint(0, 2))
+        op = (rnd.randint(0, max(s[0], d[0]) - 1), rnd.randint(0, max(s[1], d[1]) - 1))
+        H, W, B = rnd.randint(1, 9), rnd.randint(1, 9), rnd.randint(1, 3)
+        ho = (H - 1) * s[0] - 2 * p[0] + d[0] * (k[0] - 1) + 1 + op[0]
+        wo = (W - 1) * s[1] - 2 * p[1] + d[1] * (k[1] - 1) + 1 + op[1]
+        if ho <= 0 or wo <= 0:
+            continue
+        desc = (cin, cout, k, s, p, op, d, (B, H, W))
+        print("fuzz transposed", i, desc, flush=True)
+        torch.manual_seed(6000 + i)
+        net = torch.nn.Sequential(torch.nn.ConvTranspose2d(cin, cout, k, s, p, output_padding=op, bias=True, dilation=d))
+        ctrl = t.QuantizationControl()
+        t.quantize_model(net, ctrl)
+        net.to(cuda).eval()
+        with torch.no_grad():
+            net[0].bias.copy_(torch.randint(-4, 5, (cout,)).float())
+        x = torch.randint(-3, 4, (B, cin, H, W), device=cuda).float()
+        ctrl.quantize()
+        want = net(x)
+        t.compressed_state_dict(net, strong=False)
+        got = net(x)
+        assert got.shape == want.shape and torch.equal(got, want), desc
+    for i in range(110):
+        C = rnd.choice([8, 16, 24, 40, 5, 96])
+        k = (rnd.randint(1, 9), rnd.randint(1, 8))
+        s = (rnd.randint(1, 3), rnd.randint(1, 3))
+        d = (rnd.randint(1, 3), rnd.randint(1, 3))
+        p = (rnd.randint(0, 4), rnd.randint(0, 4))
+        B, H, W = rnd.randint(1, 3), rnd.randint(1, 24), rnd.randint(1, 24)
+        if (k[0] - 1) * d[0] + 1 > H + 2 * p[0] or (k[1] - 1) * d[1] + 1 > W + 2 * p[1]:
+            continue
+        desc = (B, C, H, W, k, s, p, d)
+        print("fuzz depthwise", i, desc, flush=True)
+        g = torch.Generator(device=cuda).manual_seed(7000 + i)
+        Wt = torch.randint(-1, 2, (C, 1) + k, device=cuda, generator=g).float()
+        x = torch.randint(-4, 5, (B, C, H, W), device=cuda, generator=g).float()
+        y = ops.ternary_dwconv2d(x.half(), ops.compactify_ternary(Wt), k, s, p, d)
+        ref = F.conv2d(x, Wt, None, s, p, d, groups=C)
+        assert y.shape == ref.shape and torch.equal(y.float(), ref), desc
