@@ -462,6 +462,15 @@ int tmq_ternary_conv2d_relu_maxpool(const void *x, const tmq_conv_shape *shape, 
 int tmq_avgpool_global_nhwc(const void *x, int64_t B, int64_t HW, int64_t C, void *y, int y_dtype,
                             void *stream);
 
+/* A classifier head in one launch: tmq_avgpool_global_nhwc into fp16 means followed by tmq_ternary_linear of those
+ * means (native: tmq_prepack_weights(words, N, C, 1, 1); epilogue: scale, bias, ReLU, output type; no residual),
+ * y [B][N]. The means are computed and rounded as tmq_avgpool_global_nhwc does; the product's fp32 sums may differ from
+ * the two-call form in the last bits (another order of accumulation). C <= 512 in whole groups of 8 and 16-byte
+ * aligned x; anything else returns TMQ_ERR_UNSUPPORTED and the caller makes the two calls. No counterpart in the
+ * reference (its sample leaves the head to PyTorch: samples/resnet_test.py:91-118).                             */
+int tmq_avgpool_linear(const void *x, int64_t B, int64_t HW, int64_t C, const void *native, int64_t N,
+                       const tmq_epilogue *epilogue, void *y, void *stream);
+
 /* Network input repack: x [B][C][H][W] (TMQ_F16 or TMQ_F32, C <= 4, W % 4 == 0) -> y [B][H][W][4]
  * fp16, channels C..3 zero (the layout the few-channel convolution loader wants).               */
 int tmq_nchw_to_nhwc4(const void *x, int x_dtype, int64_t B, int32_t C, int64_t H, int64_t W, void *y,

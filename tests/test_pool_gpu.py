@@ -55,3 +55,39 @@ def test_input_repack(cuda, B, C, H, W, dtype):
         ops.nchw_to_nhwc4(torch.zeros((1, 5, 4, 4), device=cuda))
     with pytest.raises(RuntimeError):
         ops.nchw_to_nhwc4(torch.zeros((1, 3, 4, 6), device=cuda))
+
+
+@pytest.mark.parametrize("B,C,H,W,N", [(64, 512, 7, 7, 102), (3, 512, 7, 7, 1000), (5, 256, 4, 5, 10), (2, 8, 3, 3, 17), (1, 264, 1, 1, 33),
+                                       (2, 1024, 2, 2, 10), (2, 20, 3, 3, 5)])
+def test_head_pool_and_classifier_in_one_launch(cuda, B, C, H, W, N):
+    """tmq_avgpool_linear: the classifier applied to the global average pool. The means are the pooling kernel's
+    (bit for bit: small integers make the product exact as well); on random data the product matches the two-call form
+    to fp32 rounding and an fp64 product of the fp16 means to 1e-5. More than 512 channels, or channels not in
+    groups of 8, take the two calls."""
+    from tmq_amd import ops
+    g = torch.Generator(device=cuda).manual_seed(B + C + N)
+    Wt = torch.randint(-1, 2, (N, C), device=cuda, generator=g).float()
+    nw = ops.NativeWeights(ops.compactify_ternary(Wt), N)
+    scale = torch.rand(N, device=cuda, generator=g) + 0.5
+    bias = torch.randn(N, device=cuda, generator=g)
+    # exact case: integer activations whose sums divide evenly (H W copies of one value per channel)
+    v = torch.randint(-8, 9, (B, C, 1, 1), device=cuda, generator=g).half()
+    xi = v.expand(B, C, H, W).contiguous(memory_format=torch.channels_last)
+    two = ops.ternary_linear(ops.avgpool_global_nhwc(xi), nw)
+    one = ops.avgpool_linear(xi, nw)
+    if (H * W) & (H * W - 1) == 0:                              # 1 / (H W) exact: the means are the integers themselves
+        assert torch.equal(two, v.view(B, C).float() @ Wt.t())
+    assert torch.equal(one, two)
+    x = torch.randn((B, C, H, W), device=cuda, generator=g).half().contiguous(memory_format=torch.channels_last)
+    means = ops.avgpool_global_nhwc(x)
+    if C <= 512:                                                # an identity classifier hands the means through: every bit equal
+        eye = ops.NativeWeights(ops.compactify_ternary(torch.eye(C, device=cuda)), C)
+        assert torch.equal(ops.avgpool_linear(x, eye), means.float())
+    ref = (means.double() @ Wt.double().t()) * scale.double() + bias.double()
+    for relu, dt in ((False, torch.float32), (True, torch.float16)):
+        want = torch.relu(ref) if relu else ref
+        got = ops.avgpool_linear(x, nw, scale, bias, relu=relu, out_dtype=dt)
+        two = ops.ternary_linear(means, nw, scale, bias, relu=relu, out_dtype=dt)
+        tol = 1e-5 if dt == torch.float32 else 2e-3
+        assert got.dtype == dt and ((got.double() - want).abs().max() / want.abs().max().clamp_min(1e-30)).item() <= tol
+        assert ((got.double() - two.double()).abs().max() / want.abs().max().clamp_min(1e-30)).item() <= tol

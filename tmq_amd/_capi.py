@@ -97,6 +97,7 @@ SIGNATURES = {
     "tmq_ternary_linear": (_int, [_vp, _int, _i64, _i64, _vp, _i64, _vp, _vp, _vp]),
     "tmq_conv2d_out_hw": (_int, [ctypes.POINTER(ConvShape), ctypes.POINTER(ctypes.c_int32),
                                  ctypes.POINTER(ctypes.c_int32)]),
+    "tmq_avgpool_linear": (_int, [_vp, _i64, _i64, _i64, _vp, _i64, _vp, _vp, _vp]),
     "tmq_ternary_conv2d": (_int, [_vp, ctypes.POINTER(ConvShape), _vp, _vp, _vp, _vp]),
     "tmq_ternary_conv2d_view": (_int, [_vp, ctypes.POINTER(ConvShape), _vp, _vp, _vp, ctypes.POINTER(OutputView), _vp]),
     "tmq_ternary_conv2d_relu_maxpool": (_int, [_vp, ctypes.POINTER(ConvShape), _vp, _vp, _vp, _vp, _vp]),

@@ -136,6 +136,79 @@ __global__ __launch_bounds__(256) void avgpool_global_nhwc_kernel(const _Float16
     }
 }
 
+// A network's head in one launch: the global average pool of an image (avgpool_global_nhwc_kernel's arithmetic, the
+// means rounded to fp16 as that kernel stores them) followed by the classifier's ternary product on those means.
+// One workgroup per image (C <= 512: 64 groups of 8 channels); the means stay in LDS, the four wavefronts share the
+// classifier's 16-channel blocks, and the row of means is row 0 of the MFMA's activation operand (the other 15 rows
+// are zero: at one row per image the instruction's idle rows cost nothing that matters next to a saved launch).
+__global__ __launch_bounds__(256) void avgpool_linear_kernel(const _Float16 *__restrict__ x, int64_t HW, int64_t C,
+                                                             const u32x4 *__restrict__ native, int64_t N, int Nb, int Kb,
+                                                             const float *__restrict__ scale, const float *__restrict__ bias,
+                                                             int relu, void *__restrict__ y, int y_f16) {
+    __shared__ float part[4][64][9];
+    __shared__ __attribute__((aligned(16))) _Float16 means[512];
+    const int64_t b = blockIdx.x, G = C / 8;
+    const int lane = threadIdx.x & 63, slice = threadIdx.x >> 6;
+    const int64_t c0 = (int64_t)lane * 8;
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    if (lane < G) {
+        const _Float16 *src = x + b * HW * C + c0;
+        int64_t p = slice;
+        for (; p + 12 < HW; p += 16) {             // four loads in flight
+            half8 v[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) v[u] = *reinterpret_cast<const half8 *>(src + (p + 4 * u) * C);
+#pragma unroll
+            for (int u = 0; u < 4; u++)
+#pragma unroll
+                for (int e = 0; e < 8; e++) acc[e] += (float)v[u][e];
+        }
+        for (; p < HW; p += 4) {
+            const half8 v = *reinterpret_cast<const half8 *>(src + p * C);
+#pragma unroll
+            for (int e = 0; e < 8; e++) acc[e] += (float)v[e];
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < 8; e++) part[slice][lane][e] = acc[e];
+    __syncthreads();
+    if (slice == 0) {
+        const float inv = 1.0f / (float)HW;
+        half8 m;
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            // the mean is rounded to fp32 and then to fp16, as the pooling kernel stores it; without the empty asm the
+            // compiler folds product and conversion into v_fma_mixlo_f16, which rounds once and differs on fp16 ties
+            float mean = (((part[0][lane][e] + part[1][lane][e]) + part[2][lane][e]) + part[3][lane][e]) * inv;
+            asm volatile("" : "+v"(mean));
+            m[e] = lane < G ? (_Float16)mean : (_Float16)0;
+        }
+        *reinterpret_cast<half8 *>(&means[lane * 8]) = m;      // channels past C: zero (the weights there are zero too)
+    }
+    __syncthreads();
+    const int j = lane & 15, g = lane >> 4;
+    for (int nb = slice; nb < Nb; nb += 4) {
+        floatx4 d = {0.f, 0.f, 0.f, 0.f};
+        for (int kb = 0; kb < Kb; kb++) {
+            const u32x4 w = native[((int64_t)nb * Kb + kb) * 64 + lane];
+#pragma unroll
+            for (int ks = 0; ks < 8; ks++) {
+                half8 a = {0, 0, 0, 0, 0, 0, 0, 0};
+                if (j == 0) a = *reinterpret_cast<const half8 *>(&means[kb * 256 + ks * 32 + g * 8]);
+                d = mfma16(a, decode_step(w[ks >> 1], ks & 1), d);
+            }
+        }
+        // row 0 of the result: element 0 of the lanes with g == 0, column j
+        const int64_t n = (int64_t)nb * 16 + j;
+        if (g == 0 && n < N) {
+            float v = d[0] * ((scale ? scale[n] : 1.0f) * (1.0f / kWeightUnit)) + (bias ? bias[n] : 0.0f);
+            if (relu && v < 0.f) v = 0.f;
+            if (y_f16) static_cast<_Float16 *>(y)[b * N + n] = (_Float16)v;
+            else static_cast<float *>(y)[b * N + n] = v;
+        }
+    }
+}
+
 // NCHW (fp16 or fp32, C <= 4) -> NHWC fp16 with 4 channels, the missing ones zero.
 // Thread = 4 neighbouring pixels of one row (W % 4 == 0): reads along W, writes 32 contiguous bytes.
 template <typename T>
@@ -207,6 +280,22 @@ int tmq_avgpool_global_nhwc(const void *x, int64_t B, int64_t HW, int64_t C, voi
     const int vec = (C % 8 == 0) && aligned16(x);
     hipLaunchKernelGGL(avgpool_global_nhwc_kernel, dim3((uint32_t)blocks), dim3(256), 0, as_stream(stream),
                        static_cast<const _Float16 *>(x), B, HW, C, vec, y, y_dtype == TMQ_F16 ? 1 : 0);
+    return check_launch();
+}
+
+int tmq_avgpool_linear(const void *x, int64_t B, int64_t HW, int64_t C, const void *native, int64_t N,
+                       const tmq_epilogue *epilogue, void *y, void *stream) {
+    if (B < 0 || HW <= 0 || C <= 0 || N <= 0) return TMQ_ERR_INVALID_ARG;
+    tmq_epilogue e = {nullptr, nullptr, nullptr, 0, TMQ_F32};
+    if (epilogue) e = *epilogue;
+    if (e.y_dtype != TMQ_F16 && e.y_dtype != TMQ_F32) return TMQ_ERR_UNSUPPORTED;
+    // one workgroup per image holds all channel means: at most 512 channels in whole groups of 8, no residual
+    if (C > 512 || C % 8 != 0 || e.residual || !aligned16(x) || B > 0x7FFFFFFF || native_blocks_n(N) > 0x7FFFFFFF) return TMQ_ERR_UNSUPPORTED;
+    if (B == 0) return TMQ_OK;
+    if (!x || !native || !y || !aligned16(native)) return TMQ_ERR_INVALID_ARG;
+    hipLaunchKernelGGL(avgpool_linear_kernel, dim3((uint32_t)B), dim3(256), 0, as_stream(stream),
+                       static_cast<const _Float16 *>(x), HW, C, static_cast<const u32x4 *>(native), N, (int)native_blocks_n(N),
+                       (int)native_blocks_k(C), e.scale, e.bias, e.relu, y, e.y_dtype == TMQ_F16 ? 1 : 0);
     return check_launch();
 }
 

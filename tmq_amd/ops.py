@@ -961,6 +961,28 @@ def avgpool_global_nhwc(x: torch.Tensor, out_dtype=torch.float16) -> torch.Tenso
     return y
 
 
+def avgpool_linear(x: torch.Tensor, nw: NativeWeights, scale=None, bias=None, relu=False, out_dtype=torch.float32) -> torch.Tensor:
+    """ternary_linear(avgpool_global_nhwc(x), nw, ...), a network's head: one launch when the feature map has at most 512
+    channels in whole groups of 8, else the two calls. x: fp16 [B, C, H, W] in channels_last memory."""
+    if not x.is_cuda or x.dim() != 4:
+        raise RuntimeError("avgpool_linear: expected a 4-D GPU tensor")
+    if x.dtype != torch.float16 or not x.is_contiguous(memory_format=torch.channels_last):
+        x = x.to(dtype=torch.float16, memory_format=torch.channels_last)
+    B, C, H, W = x.shape
+    if C != nw.K:
+        raise RuntimeError(f"avgpool_linear: feature map has {C} channels, weights expect {nw.K}")
+    y = torch.empty((B, nw.N), dtype=out_dtype, device=x.device)
+    ep = _epilogue(nw, scale, bias, None, relu, out_dtype, y)
+    if y.numel() == 0:
+        return y
+    with torch.cuda.device(x.device):
+        status = _lib().tmq_avgpool_linear(ptr(x), B, H * W, C, ptr(nw.buf), nw.N, ctypes.byref(ep), ptr(y), stream_of(x))
+    if status == _capi.ERR_UNSUPPORTED:
+        return ternary_linear(avgpool_global_nhwc(x), nw, scale=scale, bias=bias, relu=relu, out_dtype=out_dtype)
+    check(status, "avgpool_linear")
+    return y
+
+
 def nchw_to_nhwc4(x: torch.Tensor) -> torch.Tensor:
     """Contiguous NCHW network input (fp16 or fp32, at most 4 channels, W a multiple of 4) -> fp16
     [B, H, W, 4] with the missing channels zero."""
