@@ -383,6 +383,33 @@ def _gemv_floor_and_large(args, torch, natives):
         byts = K * N / 4 + 2 * rows * K + 4 * N + 4 * rows * N
         res["rows%d_16384" % rows] = {"us": round(us, 3), "gbs": round(byts / us / 1e3, 1),
                                       "frac_hbm": round(byts / us / 1e3 / HBM_PEAK_GBS, 4)}
+    # 17 and 32 rows: ops.ternary_linear brings a workspace, so the product runs with its reduction cut across
+    # workgroups (tmq_ternary_linear_ws: partial sums + an ordered second launch, both inside the timed call); the same
+    # rows through the entry point without a workspace beside it
+    for rows in (17, 32):
+        xr = torch.randn(rows, K, device=dev).half()
+        ys = torch.empty((rows, N), dtype=torch.float32, device=dev)
+        ep = _capi.Epilogue(scale.data_ptr(), None, None, 0, _capi.F32)
+
+        def with_ws(xr=xr):
+            for nw in big:
+                ops.ternary_linear(xr, nw, scale)
+            return len(big)
+
+        def without_ws(xr=xr):
+            s = _capi.stream_of(xr)
+            for nw in big:
+                _capi.check(lib.tmq_ternary_linear(_capi.ptr(xr), _capi.F16, rows, K, _capi.ptr(nw.buf), N, ctypes.byref(ep),
+                                                   _capi.ptr(ys), s), "ternary_linear")
+            return len(big)
+        with_ws()
+        without_ws()
+        us = _graph_time_us(torch, with_ws, max(2, args.steps // 12), args.settle_ms)
+        us0 = _graph_time_us(torch, without_ws, max(2, args.steps // 12), args.settle_ms)
+        byts = K * N / 4 + 2 * rows * K + 4 * N + 4 * rows * N
+        res["rows%d_16384" % rows] = {"us": round(us, 3), "without_workspace_us": round(us0, 3), "gbs": round(byts / us / 1e3, 1),
+                                      "frac_hbm": round(byts / us / 1e3 / HBM_PEAK_GBS, 4),
+                                      "kernel": "rows_split_kernel + splitk_reduce_kernel (tmq_ternary_linear_ws)"}
     return res
 
 
