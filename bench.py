@@ -413,6 +413,60 @@ def _gemv_floor_and_large(args, torch, natives):
     return res
 
 
+def bench_layers(args, torch):
+    """The layer types beside Linear / Conv2d (groups == 1): depthwise convolutions (tmq/tmq_cuda.cu:166-238) and
+    transposed convolutions (tmq/tmq.py:978-1087) from 2-bit weights, fp16 NHWC. Memory-bound (one multiply-add per loaded
+    element for the depthwise ones): reported as bytes of input + output per second against the HBM peak. Rotating
+    inputs, HIP-graph replays."""
+    import tmq_amd as t
+    from tmq_amd import ops
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev).manual_seed(7)
+    res = {"metric": "depthwise / transposed ternary layers", "unit": "us", "n_gpus": 1, "dtype": "f16", "data": "synthetic",
+           "config": {"workload": "batch 64, 128 channels, 56 x 56 depthwise windows; ConvTranspose2d 128 -> 64, 4 x 4 / 2, 56 x 56, batch 32"}}
+    B, C, H, W = 64, 128, 56, 56
+    xs = [torch.randn((B, C, H, W), device=dev, generator=g).half().contiguous(memory_format=torch.channels_last) for _ in range(4)]
+    for name, k, pad, dil in (("dw3x3", (3, 3), 1, 1), ("dw3x5", (3, 5), (1, 2), 1), ("dw3x3_dilated2", (3, 3), 2, 2), ("dw5x5", (5, 5), 2, 1)):
+        Wt = torch.randint(-1, 2, (C, 1) + k, device=dev, generator=g).float()
+        words = ops.compactify_ternary(Wt)
+
+        def run(words=words, k=k, pad=pad, dil=dil):
+            for x in xs:
+                ops.ternary_dwconv2d(x, words, k, 1, pad, dil, out_dtype=torch.float16)
+            return len(xs)
+        run()
+        us = _graph_time_us(torch, run, max(2, args.steps // 4), args.settle_ms)
+        byts = 2 * xs[0].numel() * 2
+        res[name] = {"us": round(us, 3), "gbs": round(byts / us / 1e3, 1), "frac_hbm": round(byts / us / 1e3 / HBM_PEAK_GBS, 4)}
+    net = torch.nn.Sequential(torch.nn.ConvTranspose2d(128, 64, 4, 2, 1, bias=True))
+    ctrl = t.QuantizationControl()
+    t.quantize_model(net, ctrl)
+    net.to(dev).eval()
+    ctrl.quantize()
+    t.compressed_state_dict(net, strong=False)
+    prev = t.set_compact_output_dtype(torch.float16)
+    try:
+        xt = [torch.randn((32, 128, 56, 56), device=dev, generator=g).half().contiguous(memory_format=torch.channels_last) for _ in range(4)]
+        with torch.no_grad():
+            y = net(xt[0])
+
+            def run_t():
+                for x in xt:
+                    net(x)
+                return len(xt)
+            us = _graph_time_us(torch, run_t, max(2, args.steps // 4), args.settle_ms)
+    finally:
+        t.set_compact_output_dtype(prev)
+    byts = (xt[0].numel() + y.numel()) * 2
+    res["convtranspose_128_64_k4s2"] = {"us": round(us, 3), "launches": 4, "out_MB": round(y.numel() * 2 / 1e6, 1), "gbs": round(byts / us / 1e3, 1),
+                                        "note": "one stride-1 implicit-GEMM convolution per output phase, written in place (tmq_ternary_conv2d_view)"}
+    res["value"] = res["dw3x3"]["us"]
+    res["roofline"] = {"bound": "hbm", "achieved": res["dw3x3"]["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": res["dw3x3"]["frac_hbm"],
+                       "traffic": None, "algorithmic_bytes": 2 * xs[0].numel() * 2, "kernel": "dwconv_square_image_kernel<3, 4, 1, 1, 3>",
+                       "avg_launch_us": res["dw3x3"]["us"]}
+    return res
+
+
 def bench_pack(args, torch):
     """2-bit pack / unpack of a 4096 x 4096 fp32 weight matrix (the layer of BASELINE configs[2]): 4.25 B per
     weight (4 on the fp32 side, 1/4 on the packed side). Rotates over distinct fp32 buffers (> 256 MB in total)
@@ -747,7 +801,7 @@ def main():
         torch.cuda.empty_cache()
         res["also"] = {}
         for name, leg in (("linear", bench_linear), ("pack", bench_pack), ("resnet_infer", bench_resnet_infer),
-                          ("resnet_qat", bench_resnet_qat)):
+                          ("resnet_qat", bench_resnet_qat), ("layers", bench_layers)):
             res["also"][name] = leg(args, torch)
             torch.cuda.empty_cache()
     elif args.workload == "softstep":
@@ -756,6 +810,8 @@ def main():
         res = bench_linear(args, torch)
     elif args.workload == "pack":
         res = bench_pack(args, torch)
+    elif args.workload == "layers":
+        res = bench_layers(args, torch)
     elif args.workload == "resnet_infer":
         res = bench_resnet_infer(args, torch)
     elif args.workload == "resnet_qat":
