@@ -634,7 +634,7 @@ def bench_resnet_infer(args, torch):
                         "unit": "TFLOP/s", "frac": round(f["tflops"] / MFMA_FP16_PEAK_TFLOPS, 4), "traffic": None,
                         "algorithmic_flops": 3.627e9 * B,
                         "kernel": "whole forward of tmq_amd.ResNetRunner on the calibrated network (finite activations): 20 "
-                                  "ternary implicit-GEMM convolutions, fc, pooling, input repack (22 launches)",
+                                  "ternary implicit-GEMM convolutions, fc, pooling, the input read from its NCHW planes by the opening kernel (21 launches)",
                         "avg_launch_us": round(f["gpu_ms"] * 1e3, 2)},
            "fastest_mode": best}
     if not args.no_cpu:

@@ -458,6 +458,14 @@ int tmq_maxpool2d_nhwc(const void *x, int32_t B, int32_t C, int32_t H, int32_t W
 int tmq_ternary_conv2d_relu_maxpool(const void *x, const tmq_conv_shape *shape, const void *native,
                                     const float *scale, const float *bias, void *y, void *stream);
 
+/* The same opening straight from the network's own input: x is NCHW fp16 [B][planes][H][2 W] with 1 .. 4 planes,
+ * read as shape->C == 8 channel "super-pixels" of two neighbouring pixels x 4 channels (missing planes zero), i.e.
+ * exactly the tensor tmq_nchw_to_nhwc4 would have written and shape describes ([B][H][W][8]) -- without that tensor ever
+ * existing in memory. Same result bit for bit as tmq_nchw_to_nhwc4 followed by tmq_ternary_conv2d_relu_maxpool.
+ * planes == 0 is tmq_ternary_conv2d_relu_maxpool (x NHWC). x 4-byte aligned. No counterpart in the reference.        */
+int tmq_ternary_conv2d_relu_maxpool_planar(const void *x, int32_t planes, const tmq_conv_shape *shape, const void *native,
+                                           const float *scale, const float *bias, void *y, void *stream);
+
 /* Global average pool: x [B][HW][C] fp16 -> y [B][C] (TMQ_F16 or TMQ_F32), fp32 accumulation.    */
 int tmq_avgpool_global_nhwc(const void *x, int64_t B, int64_t HW, int64_t C, void *y, int y_dtype,
                             void *stream);

@@ -159,3 +159,35 @@ def test_replays_in_a_graph(cuda):
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(out, eager)
+
+
+@pytest.mark.parametrize("B,C,H,W,N,k,pad", [(4, 3, 224, 224, 64, 7, 3), (2, 3, 33, 48, 64, 7, 3), (3, 1, 20, 24, 16, 5, 2), (2, 4, 17, 20, 40, 3, 1),
+                                             (1, 2, 9, 12, 8, 7, 3), (2, 3, 64, 60, 32, 3, 0)])
+def test_opening_from_nchw_planes_equals_the_repacked_form(cuda, B, C, H, W, N, k, pad):
+    """tmq_ternary_conv2d_relu_maxpool_planar gathers the pixel pairs from the NCHW planes itself: bit for bit the result of
+    repacking the input to 4-channel NHWC first (tmq_nchw_to_nhwc4) and running the opening on that."""
+    import tmq_amd as t
+    from tmq_amd import ops
+    torch.manual_seed(B + C + H)
+    net = torch.nn.Sequential(torch.nn.Conv2d(C, N, k, 2, pad, bias=False))
+    ctrl = t.QuantizationControl()
+    t.quantize_model(net, ctrl)
+    net.to(cuda).eval()
+    ctrl.quantize()
+    t.compressed_state_dict(net, strong=False)
+    conv = net[0]
+    x = torch.randn((B, C, H, W), device=cuda).half()
+    sp = conv._superpixel_plan(x)
+    assert sp is not None
+    nw, kxs, pl, pr = sp
+    scale = torch.rand(N, device=cuda) - 0.3
+    bias = torch.randn(N, device=cuda)
+    xs = ops.nchw_to_nhwc4(x).view(B, H, W // 2, 8).permute(0, 3, 1, 2)
+    want = ops.ternary_conv2d_relu_maxpool(xs, nw, (2, 1), ((pad, pad), (pl, pr)), 1, scale, bias)
+    got = ops.ternary_conv2d_relu_maxpool_planar(x, nw, (2, 1), ((pad, pad), (pl, pr)), 1, scale, bias)
+    assert got.shape == want.shape and torch.equal(got, want)
+    # a view that is not contiguous, and fp32 input (repacked first), give the same
+    wide = torch.randn((B, C, H, W + 4), device=cuda).half()
+    wide[..., 2:W + 2] = x
+    assert torch.equal(ops.ternary_conv2d_relu_maxpool_planar(wide[..., 2:W + 2], nw, (2, 1), ((pad, pad), (pl, pr)), 1, scale, bias), want)
+    assert torch.equal(ops.ternary_conv2d_relu_maxpool_planar(x.float(), nw, (2, 1), ((pad, pad), (pl, pr)), 1, scale, bias), want)

@@ -101,6 +101,7 @@ SIGNATURES = {
     "tmq_ternary_conv2d": (_int, [_vp, ctypes.POINTER(ConvShape), _vp, _vp, _vp, _vp]),
     "tmq_ternary_conv2d_view": (_int, [_vp, ctypes.POINTER(ConvShape), _vp, _vp, _vp, ctypes.POINTER(OutputView), _vp]),
     "tmq_ternary_conv2d_relu_maxpool": (_int, [_vp, ctypes.POINTER(ConvShape), _vp, _vp, _vp, _vp, _vp]),
+    "tmq_ternary_conv2d_relu_maxpool_planar": (_int, [_vp, ctypes.c_int32, ctypes.POINTER(ConvShape), _vp, _vp, _vp, _vp, _vp]),
     "tmq_ternary_dwconv2d": (_int, [_vp, ctypes.POINTER(ConvShape), _vp, _vp, _vp, _vp]),
     "tmq_ternary_dwconv_patches": (_int, [_vp, _int, _i64, ctypes.c_int32, _i64, _vp, _vp, _vp]),
     "tmq_maxpool2d_nhwc": (_int, [_vp] + [ctypes.c_int32] * 10 + [_vp, _vp]),

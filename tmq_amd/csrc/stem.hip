@@ -44,6 +44,8 @@ struct StemShape {
     int const_off;               // LDS byte offset of scale[64], bias[64] (behind the tile as well)
     int kchunks;                 // 16-byte pieces (8 reduction indices) per output: K / 8
     FastDiv by_tw, by_th, by_kx, by_row;   // patches per image row / column, kernel width, 16-byte pieces per window row
+    int planes;                  // 0: x is NHWC; 1 .. 4: x is the network's own NCHW fp16 input with that many channels, read as
+                                 // 8-channel "super-pixels" of two neighbouring pixels x 4 channels (cshift == 3, W = width / 2)
 };
 
 template <int WM, int WN>
@@ -67,6 +69,30 @@ __global__ __launch_bounds__(kThreads, 3) void stem_pool_kernel(StemShape p, con
     // ---- the input window -> LDS, 16 bytes per lane; pixels outside the image (padding) arrive as zeros ----
     const BufferResource rsrc = make_buffer_resource(p.x, p.x_bytes);
     const int sub_mask = (1 << (p.cshift - 3)) - 1;
+    if (p.planes) {
+        // Planar input: a piece of the window is two neighbouring pixels of up to four planes. One 4-byte load per plane
+        // (the pixel pair), interleaved in registers to (c0 c1 c2 c3 | c0 c1 c2 c3) and written to the place the
+        // 16-byte copy of the NHWC path would have filled: no repacked copy of the input ever exists in memory.
+        const int64_t plane = (int64_t)p.H * p.W;                       // pixel pairs per plane
+        const uint32_t *img = reinterpret_cast<const uint32_t *>(p.x) + (int64_t)b * p.planes * plane;
+        for (int c0 = 0; c0 < p.chunks; c0 += kThreads) {
+            const int c = c0 + tid;
+            int rc;
+            const int prow = (int)p.by_row.divmod((uint32_t)c, rc);
+            const int ih = ih_base + prow, iw = iw_base + rc;
+            const bool in = (c < p.chunks) & ((unsigned)ih < (unsigned)p.H) & ((unsigned)iw < (unsigned)p.W);
+            uint32_t v[4] = {0u, 0u, 0u, 0u};
+            if (in) {
+                const uint32_t *src = img + (int64_t)ih * p.W + iw;
+#pragma unroll
+                for (int q = 0; q < 4; q++)
+                    if (q < p.planes) v[q] = src[q * plane];
+            }
+            if (c < p.chunks)
+                *reinterpret_cast<u32x4 *>(lds + c * 16) = u32x4{(v[0] & 0xFFFFu) | (v[1] << 16), (v[2] & 0xFFFFu) | (v[3] << 16),
+                                                                (v[0] >> 16) | (v[1] & 0xFFFF0000u), (v[2] >> 16) | (v[3] & 0xFFFF0000u)};
+        }
+    } else
     for (int c0 = 0; c0 < p.chunks; c0 += kThreads) {
         const int c = c0 + tid;
         int rc;
@@ -215,17 +241,24 @@ extern "C" {
 
 int tmq_ternary_conv2d_relu_maxpool(const void *x, const tmq_conv_shape *s, const void *native, const float *scale,
                                     const float *bias, void *y, void *stream) {
-    if (!s || !x || !native || !y || !aligned16(native)) return TMQ_ERR_INVALID_ARG;
+    return tmq_ternary_conv2d_relu_maxpool_planar(x, 0, s, native, scale, bias, y, stream);
+}
+
+int tmq_ternary_conv2d_relu_maxpool_planar(const void *x, int32_t planes, const tmq_conv_shape *s, const void *native,
+                                           const float *scale, const float *bias, void *y, void *stream) {
+    if (!s || !x || !native || !y || !aligned16(native) || planes < 0 || planes > 4) return TMQ_ERR_INVALID_ARG;
+    if (planes && (s->C != 8 || (reinterpret_cast<uintptr_t>(x) & 3u))) return TMQ_ERR_UNSUPPORTED;
     int32_t ho, wo;
     const int rc = tmq_conv2d_out_hw(s, &ho, &wo);
     if (rc != TMQ_OK) return rc;
     if (s->B < 0 || s->C <= 0 || s->H <= 0 || s->W <= 0 || s->N <= 0 || s->py < 0 || s->px < 0) return TMQ_ERR_INVALID_ARG;
     if (ho <= 0 || wo <= 0) return TMQ_ERR_INVALID_ARG;
     const int64_t K = (int64_t)s->C * s->ky * s->kx, x_bytes = (int64_t)s->B * s->H * s->W * s->C * 2;
-    if (!(s->C == 8 || s->C == 16 || s->C == 32) || K > kKB || s->N > 64 || s->N % 8 != 0 || !aligned16(x) || !aligned16(y) ||
+    if (!(s->C == 8 || s->C == 16 || s->C == 32) || K > kKB || s->N > 64 || s->N % 8 != 0 || (!planes && !aligned16(x)) || !aligned16(y) ||
         x_bytes >= (int64_t)kPastTheEnd - 16)
         return TMQ_ERR_UNSUPPORTED;
     StemShape p{};
+    p.planes = planes;
     p.x = static_cast<const _Float16 *>(x);
     p.x_bytes = (uint32_t)x_bytes;
     p.cshift = s->C == 8 ? 3 : (s->C == 16 ? 4 : 5);

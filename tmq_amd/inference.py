@@ -68,8 +68,8 @@ class FoldedConv:
 
 class FoldedStem:
     """A network's opening, max_pool(relu(bn(conv(x))), 3, 2, 1), on an NCHW image of at most 4 channels: the
-    image is repacked to 4-channel NHWC, the convolution (horizontal stride 2) runs over pairs of pixels read as one
-    pixel of 8 channels (Conv2d._superpixel_plan: a 7 x 7 / 2 stem reduces over 7 x 4 x 8 = 224 indices), and
+    convolution (horizontal stride 2) runs over pairs of pixels read as one pixel of 8 channels, which the kernel gathers
+    from the NCHW planes itself (Conv2d._superpixel_plan: a 7 x 7 / 2 stem reduces over 7 x 4 x 8 = 224 indices), and
     convolution, BatchNorm, ReLU and pooling are one kernel that never writes the convolution's output. A layer the
     rewrite does not apply to runs as FoldedConv + the pooling kernel (same bits)."""
 
@@ -103,9 +103,8 @@ class FoldedStem:
                 self.plain.scale, self.plain.bias = self.scale, self.bias
             return ops.maxpool2d_nhwc(self.plain(x, relu=True), 3, 2, 1)
         nw, stride, pad = plan
-        b, c, h, w = x.shape
-        xs = ops.nchw_to_nhwc4(x).view(b, h, w // 2, 8).permute(0, 3, 1, 2)      # [B, 8, H, W / 2], channels_last memory
-        return ops.ternary_conv2d_relu_maxpool(xs, nw, stride, pad, 1, self.scale, self.bias)
+        # the kernel reads the NCHW planes itself, as pairs of pixels: no repacked copy of the input
+        return ops.ternary_conv2d_relu_maxpool_planar(x, nw, stride, pad, 1, self.scale, self.bias)
 
 
 class ResNetRunner:
@@ -114,7 +113,7 @@ class ResNetRunner:
     conv1 / bn1 / conv2 / bn2 [/ conv3 / bn3] and an optional downsample = (conv, bn)), avgpool (global), fc.
     Every convolution is one ternary implicit-GEMM launch with BatchNorm, ReLU and the residual add in its epilogue,
     activations are fp16 channels_last between the layers, the opening is one kernel (FoldedStem). ResNet-18 at
-    batch 64 is 22 launches. Takes an fp16 (or fp32) NCHW batch, returns fp32 logits."""
+    batch 64 is 21 launches. Takes an fp16 (or fp32) NCHW batch, returns fp32 logits."""
 
     def __init__(self, model):
         self.stem = FoldedStem(model.conv1, model.bn1)

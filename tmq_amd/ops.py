@@ -795,6 +795,47 @@ def ternary_conv2d_relu_maxpool(x: torch.Tensor, nw: NativeWeights, stride=1, pa
     return y
 
 
+def ternary_conv2d_relu_maxpool_planar(x: torch.Tensor, nw: NativeWeights, stride=1, padding=0, dilation=1, scale=None,
+                                       bias=None) -> torch.Tensor:
+    """ternary_conv2d_relu_maxpool on the network's own input: x is NCHW fp16 [B, C <= 4, H, W] (W even), nw the weights of
+    the convolution over 8-channel "super-pixels" (two neighbouring pixels x 4 channels) that stride, padding and dilation
+    describe -- what nchw_to_nhwc4(x).view(B, H, W / 2, 8) would feed the other call, without that copy of the input.
+    Same bits as the two-step form, which it falls back to where the one-kernel opening does not apply."""
+    pair = lambda v: tuple(v) if isinstance(v, (tuple, list)) else (v, v)
+    (sy, sx), (py, px), (dy, dx) = pair(stride), pair(padding), pair(dilation)
+    (py, py_end), (px, px_end) = pair(py), pair(px)
+    if not x.is_cuda or x.dim() != 4 or x.shape[1] > 4 or x.shape[3] % 2 or nw.C != 8:
+        raise RuntimeError("ternary_conv2d_relu_maxpool_planar: expected an NCHW GPU tensor of at most 4 channels and even "
+                           "width, and weights over 8-channel super-pixels")
+
+    def two_step():
+        B, C, H, W = x.shape
+        xs = nchw_to_nhwc4(x).view(B, H, W // 2, 8).permute(0, 3, 1, 2)      # [B, 8, H, W / 2], channels_last memory
+        return ternary_conv2d_relu_maxpool(xs, nw, stride, padding, dilation, scale, bias)
+    if x.dtype != torch.float16:
+        return two_step()
+    x = x.contiguous()
+    B, C, H, W = x.shape
+    shp = _capi.ConvShape(B, 8, H, W // 2, nw.N, nw.ky, nw.kx, sy, sx, py, px, dy, dx, py_end, px_end)
+    ho, wo = ctypes.c_int32(0), ctypes.c_int32(0)
+    lib = _lib()
+    check(lib.tmq_conv2d_out_hw(ctypes.byref(shp), ctypes.byref(ho), ctypes.byref(wo)), "conv2d_out_hw")
+    if ho.value <= 0 or wo.value <= 0:
+        raise RuntimeError("ternary_conv2d_relu_maxpool_planar: empty output")
+    y = torch.empty((B, nw.N, (ho.value - 1) // 2 + 1, (wo.value - 1) // 2 + 1), dtype=torch.float16, device=x.device,
+                    memory_format=torch.channels_last)
+    ep = _epilogue(nw, scale, bias, None, True, torch.float16, y)     # validates scale and bias
+    if B == 0:
+        return y
+    with torch.cuda.device(x.device):
+        status = lib.tmq_ternary_conv2d_relu_maxpool_planar(ptr(x), C, ctypes.byref(shp), ptr(nw.buf), ep.scale, ep.bias, ptr(y),
+                                                            stream_of(x))
+    if status == _capi.ERR_UNSUPPORTED:
+        return two_step()
+    check(status, "ternary_conv2d_relu_maxpool_planar")
+    return y
+
+
 class _Channels:
     """What _epilogue needs to know about a depthwise layer: its channel count."""
     def __init__(self, n):

@@ -826,10 +826,10 @@ class Conv2d(nn.Module, TMQLayer):
             B, C, H, W = x.shape
             if x.dtype == torch.float32:
                 x, scale = ops.f32_to_f16_prescaled(x, scale, int(self.original_shape[0]))
-            xs = ops.nchw_to_nhwc4(x).view(B, H, W // 2, 8).permute(0, 3, 1, 2)
             (sy, _), (py, _) = _pair(self.stride), _pair(self.padding)
-            if pool:
-                return ops.ternary_conv2d_relu_maxpool(xs, nw, (sy, 1), ((py, py), (pl, pr)), 1, scale=scale, bias=bias)
+            if pool:      # the one-kernel opening gathers the pixel pairs from the NCHW planes itself
+                return ops.ternary_conv2d_relu_maxpool_planar(x, nw, (sy, 1), ((py, py), (pl, pr)), 1, scale=scale, bias=bias)
+            xs = ops.nchw_to_nhwc4(x).view(B, H, W // 2, 8).permute(0, 3, 1, 2)
             return ops.ternary_conv2d(xs, nw, (sy, 1), ((py, py), (pl, pr)), 1, scale=scale, bias=bias,
                                       residual=residual, relu=relu, out_dtype=_compact_out)
         nw = self._native_weights(conv_kernel=(ky, kx))
