@@ -79,6 +79,10 @@ struct Gemv8Epilogue {
     int rows;               // rows of x that exist (<= MR; the others are zero planes and are not stored)
 };
 
+// weight blocks (1 KiB per wavefront each) a wavefront has asked for ahead of the one it multiplies: 3 and 4 measured
+// level at 16384^2 and 12288 x 16384, 2 and 6 about 3 % slower, 8 7 % and all 16 at once 25 %
+constexpr int kGemv8Ahead = 4;
+
 // vmcnt(n), nothing else waited for
 constexpr int vmcnt_only(int n) { return (n & 15) | ((n >> 4) << 14) | 0x0F70; }
 
@@ -108,8 +112,8 @@ __global__ __launch_bounds__(64 * WAVES) void gemv8_kernel(const void *__restric
     int64_t nb = (int64_t)blockIdx.x * CB + cb;
     if (nb >= Nb) nb = Nb - 1;                                   // finite bits, never stored
 
-    // The activation quads of this thread's units first, then the weight blocks, all in flight at once; loads
-    // return in issue order, so waiting for the quads leaves the weights on their way. Unit u = (kb, d, h, g')
+    // The activation quads of this thread's units first, then the first weight blocks; loads return in issue
+    // order, so waiting for the quads leaves the weights on their way. Unit u = (kb, d, h, g')
     // covers x[256 kb + 64 d + 8 g' + 4 h + {0..3}] (quad A) and the same 32 further on (quad B): the eight
     // values whose weights lane group g' finds in one operand register pair of dword d.
     using Quad = std::conditional_t<X32, u32x4, u32x2>;           // four activation values
@@ -151,18 +155,28 @@ __global__ __launch_bounds__(64 * WAVES) void gemv8_kernel(const void *__restric
     }
     // wavefront ks takes blocks ks, ks + KS, ...; when Kb is no multiple of KS the last round is short: a
     // wavefront without a block there re-reads block Kb - 1 (weights and activations) and multiplies it by zero
+    //
+    // Only the first D weight blocks are asked for here, the others one at a time as the blocks in front of them
+    // are multiplied. A wavefront cannot issue a load while the CU's memory pipeline is full, and with every
+    // wavefront of the chip asking for all of its 16 KiB at once it is full for microseconds: the wavefront then
+    // sits at a load instruction instead of preparing its share of the planes, its workgroup's barrier waits for
+    // it, and the arithmetic of wavefronts whose weights have long arrived starts when most of the matrix has
+    // been read (16384^2: the barrier passed 3.3 .. 10.3 us after the first wavefront started, the kernel ended
+    // at 14.2; with four blocks ahead 2.2 .. 6.6 and 12.2 -- by wall-clock stamps of every wavefront).
+    constexpr int D = NT < kGemv8Ahead ? NT : kGemv8Ahead;
     const u32x4 *wp = native + nb * Kb * 64 + lane;
     u32x4 wq[NT];
-#pragma unroll
-    for (int t = 0; t < NT; t++) {
+    auto ask = [&](int t) {
         const int kblk = ks + t * KS < Kb ? ks + t * KS : Kb - 1;
         wq[t] = __builtin_nontemporal_load(wp + (int64_t)kblk * 64);
-        __builtin_amdgcn_sched_barrier(0);                       // issue order = use order: the waits below count on it
-    }
+        __builtin_amdgcn_sched_barrier(0);                       // issue order = use order
+    };
+#pragma unroll
+    for (int t = 0; t < D; t++) ask(t);
     if constexpr (PRE) {
-        // the copies were issued before the NT weight loads and retire first: wait for them alone
+        // the copies were issued before the D weight loads and retire first: wait for them alone
         __builtin_amdgcn_sched_barrier(0);
-        __builtin_amdgcn_s_waitcnt(vmcnt_only(NT));
+        __builtin_amdgcn_s_waitcnt(vmcnt_only(D));
         __builtin_amdgcn_sched_barrier(0);
     }
     // per-channel constants of the threads that will store, asked for now
@@ -260,6 +274,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemv8_kernel(const void *__restric
 #pragma unroll
     for (int t = 0; t < NT; t++) {
         __builtin_amdgcn_sched_barrier(0);
+        if (t + D < NT) ask(t + D);
         const bool live = ks + t * KS < Kb;                      // uniform
         const unsigned char *xp = xb + (live ? ks + t * KS : Kb - 1) * 256;
         const uint32_t mask = live ? 0xC0C0C0C0u : 0u;
