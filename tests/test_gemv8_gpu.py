@@ -168,10 +168,11 @@ def test_agrees_with_the_fp16_kernels_on_neighbouring_shapes(cuda, oracle):
     assert _rel_err(y1.cpu().numpy(), y3.cpu().numpy()) <= 1e-5
 
 
-@pytest.mark.parametrize("K", [2048, 4096, 6144, 8192, 2304, 5120, 6912])
+@pytest.mark.parametrize("K", [2048, 4096, 6144, 8192, 2304, 5120, 6912, 8448, 11008, 12288, 13824, 16128, 16384])
 def test_fp32_row_runs_as_two_fp16_halves(cuda, oracle, K):
-    """One fp32 row (the reference's GEMV convention) up to K = 8192: hi = fp16(x), lo = fp16(x - hi), each as four
-    bf8 terms in eight activation columns. 22 significant bits of every value reach the product."""
+    """One fp32 row (the reference's GEMV convention) up to K = 16384: hi = fp16(x), lo = fp16(x - hi), each as four
+    bf8 terms in eight activation columns (beyond 8192 in workgroups of sixteen wavefronts). 22 significant bits of
+    every value reach the product."""
     from tmq_amd import ops
     N = 1000
     rng = np.random.default_rng(K)
@@ -198,11 +199,35 @@ def test_fp32_row_runs_as_two_fp16_halves(cuda, oracle, K):
     assert _rel_err(y3.float().cpu().numpy(), np.maximum(ref + res.astype(np.float64), 0)) <= 1e-3
 
 
-def test_fp32_row_passes_22_bit_values_through_exactly(cuda, oracle):
+@pytest.mark.parametrize("K", [2048, 2816, 4096, 6912, 8192, 8448, 11008, 16384])
+def test_wide_layers(cuda, oracle, K):
+    """1025 channel blocks (ragged): several channel blocks per workgroup, for an fp16 row and for an fp32 row."""
+    from tmq_amd import ops
+    N = 16400
+    rng = np.random.default_rng(K)
+    W = torch.from_numpy(rng.integers(-1, 2, size=(N, K), dtype=np.int8))
+    words = torch.from_numpy(oracle.pack(W.numpy().astype(np.float32)).view(np.int32)).to(cuda)
+    nw = ops.NativeWeights(words, N)
+    Wd = W.to(cuda).double()
+    for dt, tol in ((np.float16, 1e-5), (np.float32, 1e-5)):
+        x = torch.from_numpy(rng.standard_normal((1, K)).astype(dt)).to(cuda)
+        scale = torch.from_numpy((0.5 + rng.random(N)).astype(np.float32)).to(cuda)
+        bias = torch.from_numpy(rng.standard_normal(N).astype(np.float32)).to(cuda)
+        y = ops.ternary_linear(x, nw, scale, bias)
+        ref = (x.double() @ Wd.t()) * scale.double() + bias.double()
+        err = ((y.double() - ref).abs().max() / ref.abs().max()).item()
+        assert err <= tol, (K, dt, err)
+        assert torch.equal(ops.ternary_linear(x, nw, scale, bias), y)
+        if dt == np.float16:                # planes prepared beforehand: the same geometry, the same values
+            assert torch.equal(ops.ternary_linear_planes(ops.gemv8_prepare(x), nw, scale, bias), y)
+
+
+@pytest.mark.parametrize("K", [2048, 16384])
+def test_fp32_row_passes_22_bit_values_through_exactly(cuda, oracle, K):
     """Identity weights: integers of up to 22 bits (and their power-of-two multiples, small and large) come back
     exactly -- both halves and all eight term columns are in place."""
     from tmq_amd import ops
-    K = N = 2048
+    N = K
     nw = ops.NativeWeights(torch.from_numpy(oracle.pack(np.eye(N, dtype=np.float32)).view(np.int32)).to(cuda), N)
     rng = np.random.default_rng(9)
     ints = rng.integers(-(1 << 21), 1 << 21, size=(1, K)).astype(np.float32)

@@ -365,12 +365,40 @@ int launch_gemv8(const void *x, const void *native, int64_t Kb, int64_t N, const
     return check_launch();
 }
 
-// Geometry by the number of weight blocks per channel block: eight wavefronts per workgroup throughout; one
-// channel block per workgroup up to 32 weight blocks, two beyond when that still leaves two workgroups per CU
-// (half as many workgroups prepare or copy the activation planes, each wavefront with up to 16 KiB of weights
-// in flight).
+// Geometry by the number of weight blocks per channel block: eight wavefronts per workgroup (sixteen for the eight
+// planes of an fp32 row beyond 8192 indices or over wide layers); one channel block per workgroup up to 32 weight
+// blocks unless the layer is wide, two beyond when that still leaves two workgroups per CU (half as many workgroups
+// prepare or copy the activation planes).
 template <bool X32, int MR, bool PRE>
 int launch_gemv8_by_blocks(const void *x, int64_t Kb, const void *native, int64_t N, const Gemv8Epilogue &ep, void *stream) {
+    if constexpr (X32) {
+        // wide layers: four channel blocks per workgroup of sixteen wavefronts keep all workgroups resident at once
+        // (8192 x 28672: 1792 workgroups in 3.5 rounds -> 448 in one)
+        if (Kb > 16 && Kb <= 32 && native_blocks_n(N) >= 1024) {
+            switch ((Kb + 3) / 4) {
+                case 5: return launch_gemv8<16, 4, 5, 2, true, 1, false>(x, native, Kb, N, ep, stream);
+                case 6: return launch_gemv8<16, 4, 6, 2, true, 1, false>(x, native, Kb, N, ep, stream);
+                case 7: return launch_gemv8<16, 4, 7, 2, true, 1, false>(x, native, Kb, N, ep, stream);
+                default: return launch_gemv8<16, 4, 8, 2, true, 1, false>(x, native, Kb, N, ep, stream);
+            }
+        }
+    }
+    if constexpr (!X32 && MR == 1) {
+        // 1024 channel blocks or more: two per workgroup, so that all workgroups are resident at once (four fit a CU)
+        // and half as many prepare the planes -- 4096 x 28672 8.0 -> 7.3 us, 3072 x 24576 6.7 -> 5.5, 8192 x 28672
+        // 13.0 -> 12.0, 8192 x 16384 8.7 -> 8.15
+        if (Kb >= 8 && Kb <= 32 && native_blocks_n(N) >= 1024) {
+            switch ((Kb + 3) / 4) {
+                case 2: return launch_gemv8<8, 2, 2, 0, false, 1, PRE>(x, native, Kb, N, ep, stream);
+                case 3: return launch_gemv8<8, 2, 3, 1, false, 1, PRE>(x, native, Kb, N, ep, stream);
+                case 4: return launch_gemv8<8, 2, 4, 1, false, 1, PRE>(x, native, Kb, N, ep, stream);
+                case 5: return launch_gemv8<8, 2, 5, 2, false, 1, PRE>(x, native, Kb, N, ep, stream);
+                case 6: return launch_gemv8<8, 2, 6, 2, false, 1, PRE>(x, native, Kb, N, ep, stream);
+                case 7: return launch_gemv8<8, 2, 7, 2, false, 1, PRE>(x, native, Kb, N, ep, stream);
+                default: return launch_gemv8<8, 2, 8, 2, false, 1, PRE>(x, native, Kb, N, ep, stream);
+            }
+        }
+    }
     if (Kb <= 32) {
         switch ((Kb + 7) / 8) {                                  // blocks per wavefront, 8 wavefronts per channel block
             case 1: return launch_gemv8<8, 1, 1, 0, X32, MR, PRE>(x, native, Kb, N, ep, stream);
@@ -379,7 +407,29 @@ int launch_gemv8_by_blocks(const void *x, int64_t Kb, const void *native, int64_
             default: return launch_gemv8<8, 1, 4, 1, X32, MR, PRE>(x, native, Kb, N, ep, stream);
         }
     }
-    if constexpr (X32 || (MR > 1 && !PRE)) {
+    if constexpr (X32) {
+        // Eight planes of up to 16 KiB each: one workgroup per CU, so sixteen wavefronts in it, four per channel
+        // block where the layer is wide enough for that to cover the CUs, else eight
+        if (Kb > 64) return TMQ_ERR_UNSUPPORTED;
+        if (native_blocks_n(N) >= 1024) {
+            switch ((Kb + 3) / 4) {
+                case 9: return launch_gemv8<16, 4, 9, 2, true, 1, false>(x, native, Kb, N, ep, stream);
+                case 10: return launch_gemv8<16, 4, 10, 2, true, 1, false>(x, native, Kb, N, ep, stream);
+                case 11: return launch_gemv8<16, 4, 11, 2, true, 1, false>(x, native, Kb, N, ep, stream);
+                case 12: return launch_gemv8<16, 4, 12, 2, true, 1, false>(x, native, Kb, N, ep, stream);
+                case 13: return launch_gemv8<16, 4, 13, 2, true, 1, false>(x, native, Kb, N, ep, stream);
+                case 14: return launch_gemv8<16, 4, 14, 2, true, 1, false>(x, native, Kb, N, ep, stream);
+                case 15: return launch_gemv8<16, 4, 15, 2, true, 1, false>(x, native, Kb, N, ep, stream);
+                default: return launch_gemv8<16, 4, 16, 2, true, 1, false>(x, native, Kb, N, ep, stream);
+            }
+        }
+        switch ((Kb + 7) / 8) {
+            case 5: return launch_gemv8<16, 2, 5, 2, true, 1, false>(x, native, Kb, N, ep, stream);
+            case 6: return launch_gemv8<16, 2, 6, 2, true, 1, false>(x, native, Kb, N, ep, stream);
+            case 7: return launch_gemv8<16, 2, 7, 2, true, 1, false>(x, native, Kb, N, ep, stream);
+            default: return launch_gemv8<16, 2, 8, 2, true, 1, false>(x, native, Kb, N, ep, stream);
+        }
+    } else if constexpr (MR > 1 && !PRE) {
         return TMQ_ERR_UNSUPPORTED;                              // the planes of such rows stop at 8192 indices
     } else {
         // two channel blocks per workgroup would leave CUs idle on narrow layers, and need two workgroups' LDS per CU
@@ -426,10 +476,10 @@ int launch_gemv8_dense(const void *x, int64_t M, int64_t K, const void *native, 
     return launch_gemv8_by_blocks<false, 4, false>(x, Kb, native, N, ep, stream);
 }
 
-// One fp32 row: K a multiple of 256 from 2048 to 8192 (eight term planes; beyond that they leave room for one workgroup
-// per CU only).
+// One fp32 row: K a multiple of 256 from 2048 to 16384 (eight term planes; beyond 8192 they leave room for one
+// workgroup per CU only, which then has sixteen wavefronts).
 bool gemv8_dense32_ok(const void *x, int64_t M, int64_t K) {
-    return M == 1 && K % kKB == 0 && K >= 8 * kKB && K <= 32 * kKB && aligned16(x);
+    return M == 1 && K % kKB == 0 && K >= 8 * kKB && K <= 64 * kKB && aligned16(x);
 }
 
 int launch_gemv8_dense32(const void *x, int64_t K, const void *native, int64_t N, const float *scale, const float *bias,
