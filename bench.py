@@ -383,6 +383,21 @@ def _gemv_floor_and_large(args, torch, natives):
         byts = K * N / 4 + 2 * rows * K + 4 * N + 4 * rows * N
         res["rows%d_16384" % rows] = {"us": round(us, 3), "gbs": round(byts / us / 1e3, 1),
                                       "frac_hbm": round(byts / us / 1e3 / HBM_PEAK_GBS, 4)}
+    # fp32 rows, the reference's own convention (tmq/tmq_cuda.cu:242-286 takes an fp32 vector): one row is scaled and
+    # split into its two fp16 terms inside the GEMV; four rows are split once into fp16 row pairs (a launch of its
+    # own, inside the timed call) and take one pass of the fp16 weight stream
+    for rows in (1, 4):
+        xr = torch.randn(rows, K, device=dev)
+
+        def few32(xr=xr):
+            for nw in big:
+                ops.ternary_linear(xr, nw, scale)
+            return len(big)
+        few32()
+        us = _graph_time_us(torch, few32, max(2, args.steps // 12), args.settle_ms)
+        byts = K * N / 4 + 4 * rows * K + 4 * N + 4 * rows * N
+        res["rows%d_16384_fp32" % rows] = {"us": round(us, 3), "gbs": round(byts / us / 1e3, 1),
+                                           "frac_hbm": round(byts / us / 1e3 / HBM_PEAK_GBS, 4)}
     # 17 and 32 rows: ops.ternary_linear brings a workspace, so the product runs with its reduction cut across
     # workgroups (tmq_ternary_linear_ws: partial sums + an ordered second launch, both inside the timed call); the same
     # rows through the entry point without a workspace beside it

@@ -182,10 +182,23 @@ __device__ __forceinline__ ThreadColumns load_column_constants(int64_t n0, int64
 // A thread keeps its columns for all its rows. Its residual values are asked for before the fragments go
 // to LDS, so that they arrive while the workgroup synchronises (and before any store of this thread: the
 // residual may be the output buffer).
-template <int WM, int WN, int WAVES, class Ep>
+//
+// Pairs: fp32 rows carried as two fp16 rows each (hi = fp16(s x), lo = fp16(s x - hi), row m and row m + pair of the
+// tile, s the row's own power of two). With RowPairs the two rows' sums are added -- hi's partial sums in wavefront
+// order, then lo's -- and multiplied by row_scale[m] = 1 / s before the per-channel scale; M counts output rows.
+struct NoPairs {
+    static constexpr bool kOn = false;
+};
+struct RowPairs {
+    static constexpr bool kOn = true;
+    int pair;
+    const float *row_scale;
+};
+
+template <int WM, int WN, int WAVES, class Ep, class Pairs = NoPairs>
 __device__ __forceinline__ void reduce_and_store(unsigned char *smem, const floatx4 (&acc)[WM][WN], int kg, int lane,
                                                  int64_t m0, int64_t n0, int64_t M, int64_t N, const Ep &ep,
-                                                 const ThreadColumns &cc) {
+                                                 const ThreadColumns &cc, const Pairs &pairs = Pairs{}) {
     constexpr int NF = WM * WN;
     const int j = lane & 15, g = lane >> 4;
     constexpr int kFragPitch = 1024 + 64;                       // bytes; +64 spreads the nj over the banks
@@ -224,11 +237,16 @@ __device__ __forceinline__ void reduce_and_store(unsigned char *smem, const floa
 
     if (n >= N) return;
     const floatx4 sc = cc.sc, bi = cc.bi;
-    auto partial_sums = [&](int row) {
+    auto row_sums = [&](int row) {
         const unsigned char *src = smem + (size_t)((row >> 4) * WN + (c4 >> 2)) * kFragPitch + ((row & 15) * 4 + ((c4 & 3) ^ ((row >> 2) & 3))) * 16;
         floatx4 v = *reinterpret_cast<const floatx4 *>(src);
 #pragma unroll
         for (int q = 1; q < WAVES; q++) v += *reinterpret_cast<const floatx4 *>(src + (size_t)q * NF * kFragPitch);
+        return v;
+    };
+    auto partial_sums = [&](int row) {
+        floatx4 v = row_sums(row);
+        if constexpr (Pairs::kOn) v = (v + row_sums(row + pairs.pair)) * pairs.row_scale[m0 + row];
         return v * sc + bi;
     };
     if (vec) {
@@ -588,10 +606,10 @@ constexpr int stream_waves_per_simd(int WN, int WAVES, int R, int D) {
     return w < 1 ? 1 : (w > 4 ? 4 : w);
 }
 
-template <int WN, int WAVES, int R, int D, bool LONG>
+template <int WN, int WAVES, int R, int D, bool LONG, class Pairs>
 __global__ __launch_bounds__(64 * WAVES, stream_waves_per_simd(WN, WAVES, R, D)) void stream_kernel(const _Float16 *__restrict__ x, const u32x4 *__restrict__ native,
                                                             int64_t M, int64_t K, int Kb, int64_t N, int64_t Nb,
-                                                            MidEpilogue ep) {
+                                                            MidEpilogue ep, Pairs pairs) {
     using Rows = StreamRows<R>;
     constexpr int kLoads = Rows::kLoads, kSlot = Rows::kSlot, kWave = D * kSlot, kPerBlock = WN + kLoads;
     static_assert((D - 1) * kPerBlock < 64, "vmcnt is a 6-bit counter");
@@ -817,11 +835,15 @@ __global__ __launch_bounds__(64 * WAVES, stream_waves_per_simd(WN, WAVES, R, D))
             if constexpr (D > 3) if (t + 2 < nt) step(t + 2, std::integral_constant<int, 2>{}, std::false_type{});
         }
     }
-    reduce_and_store<1, WN, WAVES>(smem, acc, kg, lane, 0, n0, M, N, ep, load_column_constants<WN>(n0, N, ep));
+    int64_t rows_out = M;
+    if constexpr (Pairs::kOn) rows_out = pairs.pair;
+    reduce_and_store<1, WN, WAVES>(smem, acc, kg, lane, 0, n0, rows_out, N, ep, load_column_constants<WN>(n0, N, ep), pairs);
 }
 
+// pairs: null, or the fp16 rows are M / 2 fp32 rows' hi terms followed by their lo terms
 template <int WN, int WAVES, int R, int D>
-int launch_stream(const void *x, const void *native, int64_t M, int64_t K, int64_t N, const MidEpilogue &ep, void *stream) {
+int launch_stream(const void *x, const void *native, int64_t M, int64_t K, int64_t N, const MidEpilogue &ep, void *stream,
+                  const RowPairs *pairs = nullptr) {
     const int64_t tn = (N + 16 * WN - 1) / (16 * WN), Kb = native_blocks_k(K);
     if (tn > 0x7FFFFFFF || Kb > (1 << 20)) return TMQ_ERR_TOO_LARGE;
     constexpr size_t win = (size_t)WAVES * D * R * 512, redb = (size_t)WAVES * WN * (1024 + 64);
@@ -830,14 +852,22 @@ int launch_stream(const void *x, const void *native, int64_t M, int64_t K, int64
     // the variant with a steady-state loop needs 2 D blocks in every wavefront; with fewer, half the depth
     // and a steady state beats the full depth without one
     if constexpr (D == 4) {
-        if (Kb / WAVES < 2 * D && Kb / WAVES >= D) return launch_stream<WN, WAVES, R, 2>(x, native, M, K, N, ep, stream);
+        if (Kb / WAVES < 2 * D && Kb / WAVES >= D) return launch_stream<WN, WAVES, R, 2>(x, native, M, K, N, ep, stream, pairs);
     }
-    auto kernel = R != 16 && Kb / WAVES >= 2 * D ? stream_kernel<WN, WAVES, R, D, true> : stream_kernel<WN, WAVES, R, D, false>;
-    if (int st = allow_dynamic_lds(reinterpret_cast<const void *>(kernel), lds)) return st;
-    hipLaunchKernelGGL(kernel, dim3((uint32_t)tn), dim3(64 * WAVES), lds, as_stream(stream),
-                       static_cast<const _Float16 *>(x), static_cast<const u32x4 *>(native), M, K, (int)Kb, N,
-                       native_blocks_n(N), ep);
-    return check_launch();
+    auto go = [&](auto kernel, auto pairs_arg) {
+        if (int st = allow_dynamic_lds(reinterpret_cast<const void *>(kernel), lds)) return st;
+        hipLaunchKernelGGL(kernel, dim3((uint32_t)tn), dim3(64 * WAVES), lds, as_stream(stream),
+                           static_cast<const _Float16 *>(x), static_cast<const u32x4 *>(native), M, K, (int)Kb, N,
+                           native_blocks_n(N), ep, pairs_arg);
+        return check_launch();
+    };
+    const bool steady = R != 16 && Kb / WAVES >= 2 * D;
+    if constexpr (R >= 4) {
+        if (pairs)
+            return steady ? go(stream_kernel<WN, WAVES, R, D, true, RowPairs>, *pairs) : go(stream_kernel<WN, WAVES, R, D, false, RowPairs>, *pairs);
+    }
+    if (pairs) return TMQ_ERR_UNSUPPORTED;
+    return steady ? go(stream_kernel<WN, WAVES, R, D, true, NoPairs>, NoPairs{}) : go(stream_kernel<WN, WAVES, R, D, false, NoPairs>, NoPairs{});
 }
 
 // ---- weight stream, fp32 activations, at most 16 rows -------------------------------------------------
@@ -1063,24 +1093,37 @@ int launch_stream32_dense(const void *x, int64_t M, int64_t K, const void *nativ
 // 2 at R = 4 and at R = 8 with two blocks in flight, 1 at R = 16 (2 with four wavefronts). So: the
 // narrowest tile whose workgroups fit in one pass (narrow tiles mean more wavefronts streaming), measured
 // on 4096 x {4096, 5120, 11008, 13824}, 8192 x {6144, 8192, 16384, 28672} and 16384^2.
-int launch_stream_dense(const void *x, int64_t M, int64_t K, const void *native, int64_t N, const float *scale,
-                        const float *bias, const void *residual, int relu, void *y, int y_f16, void *stream) {
-    MidEpilogue ep{scale, bias, residual, y, relu, y_f16};
+static int stream_by_shape(const void *x, int64_t M, int64_t K, const void *native, int64_t N, const MidEpilogue &ep,
+                           void *stream, const RowPairs *pairs) {
     const int64_t Nb = native_blocks_n(N);
-    if (M <= 2) return launch_stream<1, 8, 2, 4>(x, native, M, K, N, ep, stream);
+    if (M <= 2) return launch_stream<1, 8, 2, 4>(x, native, M, K, N, ep, stream, pairs);
     if (M <= 4) {
-        if (Nb >= 512) return launch_stream<2, 8, 4, 4>(x, native, M, K, N, ep, stream);
-        return launch_stream<1, 8, 4, 4>(x, native, M, K, N, ep, stream);
+        if (Nb >= 512) return launch_stream<2, 8, 4, 4>(x, native, M, K, N, ep, stream, pairs);
+        return launch_stream<1, 8, 4, 4>(x, native, M, K, N, ep, stream, pairs);
     }
     if (M <= 8) {
-        if (Nb <= 256) return launch_stream<1, 8, 8, 4>(x, native, M, K, N, ep, stream);
-        if (Nb <= 1024) return launch_stream<2, 8, 8, 2>(x, native, M, K, N, ep, stream);
-        return launch_stream<4, 8, 8, 2>(x, native, M, K, N, ep, stream);
+        if (Nb <= 256) return launch_stream<1, 8, 8, 4>(x, native, M, K, N, ep, stream, pairs);
+        if (Nb <= 1024) return launch_stream<2, 8, 8, 2>(x, native, M, K, N, ep, stream, pairs);
+        return launch_stream<4, 8, 8, 2>(x, native, M, K, N, ep, stream, pairs);
     }
-    if (Nb <= 256) return launch_stream<1, 8, 16, 2>(x, native, M, K, N, ep, stream);
-    if (Nb <= 512) return launch_stream<2, 8, 16, 2>(x, native, M, K, N, ep, stream);
-    if (Nb <= 1024) return launch_stream<4, 8, 16, 2>(x, native, M, K, N, ep, stream);
-    return launch_stream<4, 4, 16, 2>(x, native, M, K, N, ep, stream);
+    if (Nb <= 256) return launch_stream<1, 8, 16, 2>(x, native, M, K, N, ep, stream, pairs);
+    if (Nb <= 512) return launch_stream<2, 8, 16, 2>(x, native, M, K, N, ep, stream, pairs);
+    if (Nb <= 1024) return launch_stream<4, 8, 16, 2>(x, native, M, K, N, ep, stream, pairs);
+    return launch_stream<4, 4, 16, 2>(x, native, M, K, N, ep, stream, pairs);
+}
+
+int launch_stream_dense(const void *x, int64_t M, int64_t K, const void *native, int64_t N, const float *scale,
+                        const float *bias, const void *residual, int relu, void *y, int y_f16, void *stream) {
+    return stream_by_shape(x, M, K, native, N, MidEpilogue{scale, bias, residual, y, relu, y_f16}, stream, nullptr);
+}
+
+// M fp32 rows as 2 M fp16 rows (x16: the M hi terms, then the M lo terms; row_scale[m] undoes row m's power of two):
+// one pass of the weight-stream kernel, the two sums of a row added in its epilogue. 2 <= 2 M <= 16.
+int launch_stream_pairs(const void *x16, int64_t M, int64_t K, const void *native, int64_t N, const float *row_scale,
+                        const float *scale, const float *bias, const void *residual, int relu, void *y, int y_f16,
+                        void *stream) {
+    const RowPairs pairs{(int)M, row_scale};
+    return stream_by_shape(x16, 2 * M, K, native, N, MidEpilogue{scale, bias, residual, y, relu, y_f16}, stream, &pairs);
 }
 
 bool mid_conv_ok(const void *x, const tmq_conv_shape *s) {

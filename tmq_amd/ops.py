@@ -608,8 +608,14 @@ def ternary_linear(x: torch.Tensor, nw: NativeWeights, scale=None, bias=None, re
     if x.shape[-1] != nw.K:
         raise RuntimeError(f"ternary_linear: activations have {x.shape[-1]} features, weights expect {nw.K}")
     M = x.numel() // nw.K if nw.K else 0
+    pairs = 0
     if x.dtype == torch.float32 and M == 1 and x.is_contiguous() and _lib().tmq_fp32_rows_self_scaled(ptr(x), M, nw.K):
         pass            # a single row the kernel scales itself (any magnitude): one launch, no prescale pass
+    elif (x.dtype == torch.float32 and 2 <= M <= 8 and x.is_contiguous() and x.data_ptr() % 16 == 0
+          and _lib().tmq_ternary_linear_workspace_bytes(_capi.F32, M, nw.K, nw.N)):
+        # a few rows: split once into fp16 row pairs (each row scaled by its own power of two, any magnitude) in the
+        # workspace, then one pass of the fp16 weight stream
+        pairs = _lib().tmq_ternary_linear_workspace_bytes(_capi.F32, M, nw.K, nw.N)
     elif x.dtype == torch.float32 and M > 0:
         two_pass = (out_dtype == torch.float32 and (residual is None or residual.dtype == torch.float32)
                     and bool(_lib().tmq_fp32_rows_prefer_split(M, nw.K, nw.N)))
@@ -630,7 +636,7 @@ def ternary_linear(x: torch.Tensor, nw: NativeWeights, scale=None, bias=None, re
     ep = _epilogue(nw, scale, bias, residual, relu, out_dtype, y)
     lib = _lib()
     # shapes whose reduction pays to be cut across workgroups get a workspace for the partial sums
-    wsb = lib.tmq_ternary_linear_workspace_bytes(_capi.dtype_code(x), M, nw.K, nw.N) if 16 < M <= 32 else 0
+    wsb = pairs or (lib.tmq_ternary_linear_workspace_bytes(_capi.dtype_code(x), M, nw.K, nw.N) if 16 < M <= 32 else 0)
     with torch.cuda.device(x.device):
         if wsb:
             ws = torch.empty(wsb, dtype=torch.uint8, device=x.device)
