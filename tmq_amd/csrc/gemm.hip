@@ -1093,15 +1093,16 @@ int rows_split_slices(const void *x, int64_t M, int64_t K, int64_t N);
 int launch_rows_split(const void *x, int64_t M, int64_t K, const void *native, int64_t N, const Epilogue &ep, float *partial,
                       int slices, void *stream);
 
-// Two to eight fp32 rows over whole weight blocks: split once into fp16 row pairs (prescale.hip), then one pass of the
-// fp16 weight-stream kernel over twice the rows (mid.hip) -- against the kernel that splits every block's
-// activations on the fly in each workgroup: 8192^2, 4 rows 17.7 -> 9.5 us, 8 rows 25.7 -> 10 us.
-int launch_split_rows(const float *x, int64_t M, int64_t K, void *x16, float *row_scale, void *stream);
+// Two to sixteen fp32 rows over whole weight blocks: split once into fp16 row pairs (prescale.hip), then one pass of
+// the fp16 weight-stream kernel over twice the rows (mid.hip; two passes of about half the rows each from nine rows)
+// -- against the kernel that splits every block's activations on the fly in each workgroup: 8192^2, 4 rows
+// 17.4 -> 10.8 us, 8 rows 25.5 -> 11.7 us.
+int launch_split_rows(const float *x, int64_t M, int64_t K, int64_t group, void *x16, float *row_scale, void *stream);
 int launch_stream_pairs(const void *x16, int64_t M, int64_t K, const void *native, int64_t N, const float *row_scale,
                         const float *scale, const float *bias, const void *residual, int relu, void *y, int y_f16,
                         void *stream);
 inline bool row_pairs_ok(const void *x, int64_t M, int64_t K) {
-    return M >= 2 && M <= 8 && K % kKB == 0 && K >= 8 * kKB && aligned16(x) && 2 * M * K < (int64_t)0x7FFFFFFF;
+    return M >= 2 && M <= 16 && K % kKB == 0 && K >= 8 * kKB && aligned16(x) && 2 * M * K < (int64_t)0x7FFFFFFF;
 }
 inline size_t row_pairs_bytes(int64_t M, int64_t K) { return 256 + (size_t)(2 * M * K) * sizeof(_Float16); }
 
@@ -1164,9 +1165,20 @@ int tmq_ternary_linear_ws(const void *x, int x_dtype, int64_t M, int64_t K, cons
         // the rows' 1 / s first (256 bytes), then the 2 M fp16 rows
         float *row_scale = static_cast<float *>(workspace);
         void *x16 = static_cast<unsigned char *>(workspace) + 256;
-        if (int st = launch_split_rows(static_cast<const float *>(x), M, K, x16, row_scale, stream)) return st;
-        return launch_stream_pairs(x16, M, K, native, N, row_scale, e.scale, e.bias, e.residual, e.relu, y,
-                                   e.y_dtype == TMQ_F16 ? 1 : 0, stream);
+        // up to eight rows make one pass of sixteen fp16 rows; nine to sixteen go as two groups of about equal size
+        const int64_t group = M <= 8 ? M : (M + 1) / 2;
+        if (int st = launch_split_rows(static_cast<const float *>(x), M, K, group, x16, row_scale, stream)) return st;
+        const size_t out_elt = e.y_dtype == TMQ_F16 ? 2 : 4;
+        for (int64_t m0 = 0; m0 < M; m0 += group) {
+            const int64_t rows = M - m0 < group ? M - m0 : group;
+            const unsigned char *res = static_cast<const unsigned char *>(e.residual);
+            const int st = launch_stream_pairs(static_cast<const _Float16 *>(x16) + 2 * m0 * K, rows, K, native, N, row_scale + m0,
+                                               e.scale, e.bias, res ? res + (size_t)(m0 * N) * out_elt : nullptr, e.relu,
+                                               static_cast<unsigned char *>(y) + (size_t)(m0 * N) * out_elt,
+                                               e.y_dtype == TMQ_F16 ? 1 : 0, stream);
+            if (st) return st;
+        }
+        return TMQ_OK;
     }
     if (x && native && y && x_dtype == TMQ_F16 && M > 0 && K > 0 && N > 0 && workspace && aligned16(workspace) && aligned16(native)) {
         const int slices = rows_split_slices(x, M, K, N);

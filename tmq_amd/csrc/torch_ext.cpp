@@ -238,7 +238,7 @@ void check_mm_args(const torch::Tensor &lhs, const torch::Tensor &weights, int64
 // fp32 activations (the reference's convention). The kernels carry them as fp16 terms, so the tensor is first
 // scaled by the power of two that brings its largest value into fp16's range (tmq_f32_prescale; exact, undone
 // in the epilogue's per-channel scale): any magnitude works, as with the reference's fp32 arithmetic. Many
-// rows: the fp16 kernels over the two fp16 terms, y = W hi + W lo; two to eight rows over whole weight blocks: the
+// rows: the fp16 kernels over the two fp16 terms, y = W hi + W lo; two to sixteen rows over whole weight blocks: the
 // two terms as row pairs of one fp16 pass; otherwise the kernels that split on the fly.
 torch::Tensor linear_f32(const torch::Tensor &x, int64_t M, int64_t K, const torch::Tensor &native, int64_t columns,
                          torch::Tensor &y, const char *name) {
