@@ -230,6 +230,22 @@ def bench_linear(args, torch):
     extra = {}
     if args.gemv_floor:
         extra = _gemv_floor_and_large(args, torch, natives)
+        # fp32 activations, the reference's own calling convention (tmq/tmq.py:680-683 hands fp32 rows to its kernels):
+        # ops.ternary_linear splits them into fp16 row pairs in a workspace (one launch, inside the timed call) and
+        # runs the fp16 kernels once over twice the rows -- 22 significant bits per value
+        f32 = {}
+        for M in (256, 4096):
+            x = torch.randn(M, K, generator=gen(13)).to(dev)
+            per_graph = 24 if M < 4096 else 4
+
+            def run32(x=x, per_graph=per_graph):
+                for i in range(per_graph):
+                    ops.ternary_linear(x, natives[i % nrot], scale)
+                return per_graph
+            run32()
+            us = _graph_time_us(torch, run32, max(2, args.steps // 8), args.settle_ms)
+            f32[str(M)] = {"us": round(us, 3), "tflops": round(2.0 * M * N * K / us / 1e6, 3)}
+        extra["by_M_fp32_rows"] = f32
     res = {"metric": "ternary-GEMM eff. TFLOP/s (K=N=4096)", "unit": "TFLOP/s", "n_gpus": 1, "dtype": "f16",
            "data": "synthetic", "config": {"workload": "configs[2]: ternary linear K=N=4096", "rotate_buffers": nrot},
            "value": out.get("4096", {}).get("tflops"), "by_M": out, **extra}

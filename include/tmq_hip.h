@@ -305,7 +305,10 @@ int tmq_ternary_linear(const void *x, int x_dtype, int64_t M, int64_t K, const v
  * tmq/tmq_cuda.cu:242-427) use the workspace differently: a first launch splits every row into two fp16 rows
  * (hi = fp16(s x), lo = fp16(s x - hi), s the row's own power of two: any magnitude, 22 significant bits), the fp16
  * weight-stream kernel then runs once over twice the rows (from nine rows: twice, over about half of them each)
- * and adds each pair in its epilogue (256 + 4 M K bytes).
+ * and adds each pair in its epilogue (256 + 4 M K bytes). Seventeen fp32 rows or more with K a multiple of 64 from
+ * 256 are split in groups of eight rows, each group under a power of two of its own, laid out so that a row's two
+ * terms share a 16-row MFMA fragment; the fp16 GEMM kernels then run once over 16 ceil(M / 8) rows and add the pairs
+ * where they write the tile (ceil(M / 8) floats rounded up to 256 bytes + 32 ceil(M / 8) K bytes).
  * tmq_ternary_linear_workspace_bytes returns what a shape can use (0: the single-launch kernels are at
  * least as fast); with a NULL or smaller workspace tmq_ternary_linear_ws is tmq_ternary_linear. Same results to
  * fp32 rounding (the summation order differs). The workspace must be 16-byte aligned.                     */

@@ -3,6 +3,9 @@ tmq/tmq_cuda.cu:242-427, tmq/tmq.py:680-683): tmq_ternary_linear_ws splits them 
 fp16(s x), lo = fp16(s x - hi), s the row's own power of two -- and runs the fp16 weight stream once over twice the
 rows, adding each pair in the epilogue (nine to sixteen rows: two such passes over about half the rows each).
 
+Seventeen rows or more take groups of eight rows, each group with a power of two of its own, laid out so that a row's
+two terms sit in one 16-row MFMA fragment of whatever fp16 kernel the shape reaches; the epilogues add them.
+
 Bar: 1e-5 of each row's largest output against an fp64 product of the expanded weights (22 significant bits per
 value; a single fp16 rounding of the row is ~100 times worse), rows of any magnitude side by side, 22-bit integers
 through identity weights exactly, every epilogue, and the plain entry point when the workspace is missing.
@@ -94,7 +97,7 @@ def test_c_abi_workspace_rules_and_graph_replay(cuda, oracle):
     from tmq_amd import ops, _capi
     lib = _capi.load()
     K, N, M = 4096, 520, 12
-    for m, k in ((1, 4096), (17, 4096), (4, 4096 + 128), (4, 1024)):
+    for m, k in ((1, 4096), (4, 4096 + 128), (4, 1024)):
         assert lib.tmq_ternary_linear_workspace_bytes(_capi.F32, m, k, N) == 0
     rng = np.random.default_rng(3)
     W, nw = _layer(cuda, oracle, rng, N, K)
@@ -122,5 +125,104 @@ def test_c_abi_workspace_rules_and_graph_replay(cuda, oracle):
     for _ in range(3):
         out.zero_()
         g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager)
+
+
+# ---- seventeen rows or more: groups of eight rows, pairs inside one 16-row MFMA fragment -------------------------------
+# (M, K, N): which fp16 kernel the 16 ceil(M / 8) rows reach
+MANY = [
+    (17, 4096, 4096),      # split reduction, 32 x 32 tiles
+    (23, 1024, 1000),      # ragged N (a multiple of 4 and 8), M not a multiple of 8
+    (64, 256, 72),         # the shortest reduction the path takes
+    (100, 2304, 4100),     # N a multiple of 4 only
+    (128, 576, 67),        # scalar stores (N odd)
+    (256, 4096, 4096),     # split reduction, 64 x 64 tiles, eight wavefronts
+    (300, 8192, 520),      # long reduction, narrow layer
+    (1000, 1024, 1024),    # direct-to-LDS tiles
+    (1024, 4096, 4096),    # 64 x 512 tiles, eight wavefronts
+    (2048, 4096, 2048),    # 128 x 512 tiles
+    (4096, 1024, 11008),   # 128 x 256 tiles, two workgroups per CU
+]
+
+
+@pytest.mark.parametrize("M,K,N", MANY)
+def test_many_rows_against_fp64(cuda, oracle, M, K, N):
+    from tmq_amd import ops, _capi
+    print("fp32 row groups", M, K, N, flush=True)
+    g = torch.Generator(device=cuda).manual_seed(M + K + N)
+    W = torch.randint(-1, 2, (N, K), device=cuda, generator=g).to(torch.int8)
+    words = torch.from_numpy(oracle.pack(W.float().cpu().numpy()).view(np.int32)).to(cuda)
+    nw = ops.NativeWeights(words, N)
+    groups = (M + 7) // 8
+    assert _capi.load().tmq_ternary_linear_workspace_bytes(_capi.F32, M, K, N) == (4 * groups + 255) // 256 * 256 + 32 * groups * K
+    x = torch.randn((M, K), device=cuda, generator=g)
+    # every group of eight rows its own magnitude: the groups are scaled separately
+    x *= (2.0 ** torch.randint(-40, 40, (groups, 1), device=cuda, generator=g).float()).repeat_interleave(8, 0)[:M]
+    Wd = W.double()
+    ref = x.double() @ Wd.t()
+    rows = lambda got, want: float(((got.double() - want).abs().amax(1) / want.abs().amax(1).clamp_min(1e-300)).max())
+    y = ops.ternary_linear(x, nw)
+    assert y.shape == (M, N) and y.dtype == torch.float32
+    err = rows(y, ref)
+    assert err <= 1e-5, err
+    assert torch.equal(ops.ternary_linear(x, nw), y)
+    scale = torch.rand(N, device=cuda, generator=g) + 0.5
+    bias = torch.randn(N, device=cuda, generator=g)
+    res = torch.randn((M, N), device=cuda, generator=g) * ref.abs().amax(1, keepdim=True).float()
+    full = ref * scale.double() + bias.double()
+    y2 = ops.ternary_linear(x, nw, scale, bias, residual=res, relu=True)
+    assert rows(y2, torch.relu(full + res.double())) <= 1e-5
+    # fp16 output (the wide-row epilogue where N is a multiple of 8): rows of order one
+    x1 = torch.randn((M, K), device=cuda, generator=g)
+    ref1 = (x1.double() @ Wd.t()) * (scale.double() / K ** 0.5) + bias.double()
+    res16 = torch.randn((M, N), device=cuda, generator=g).half()
+    y3 = ops.ternary_linear(x1, nw, scale / K ** 0.5, bias, residual=res16, out_dtype=torch.float16)
+    assert y3.dtype == torch.float16 and rows(y3, ref1 + res16.double()) <= 1e-3
+
+
+def test_many_rows_22_bit_values_pass_through_exactly(cuda, oracle):
+    from tmq_amd import ops
+    K = N = 1024
+    nw = ops.NativeWeights(torch.from_numpy(oracle.pack(np.eye(N, dtype=np.float32)).view(np.int32)).to(cuda), N)
+    rng = np.random.default_rng(21)
+    M = 77
+    x = rng.integers(-(1 << 21), 1 << 21, size=(M, K)).astype(np.float32)
+    x[:, :4] = [0.0, -0.0, 1.0, -1.0]
+    x *= np.repeat((2.0 ** rng.integers(-60, 60, size=((M + 7) // 8, 1))).astype(np.float32), 8, axis=0)[:M]
+    y = ops.ternary_linear(torch.from_numpy(x).to(cuda), nw).cpu().numpy()
+    assert np.array_equal(y, x)
+
+
+def test_many_rows_workspace_rules_and_graph_replay(cuda, oracle):
+    from tmq_amd import ops, _capi
+    lib = _capi.load()
+    M, K, N = 200, 1024, 520
+    for m, k in ((200, 1024 + 32), (200, 128)):                   # K not a multiple of 64, K below 256: the older paths
+        assert lib.tmq_ternary_linear_workspace_bytes(_capi.F32, m, k, N) == 0
+    g = torch.Generator(device=cuda).manual_seed(8)
+    W = torch.randint(-1, 2, (N, K), device=cuda, generator=g).to(torch.int8)
+    nw = ops.NativeWeights(ops.compactify_ternary(W), N)
+    x = torch.randn((M, K), device=cuda, generator=g)
+    ref = x.double() @ W.double().t()
+    ep = _capi.Epilogue(None, None, None, 0, _capi.F32)
+    need = lib.tmq_ternary_linear_workspace_bytes(_capi.F32, M, K, N)
+    ws = torch.empty(need, dtype=torch.uint8, device=cuda)
+    for wptr, wbytes in ((ops.ptr(ws), need), (None, 0), (ops.ptr(ws), need - 1)):
+        y = torch.empty((M, N), dtype=torch.float32, device=cuda)
+        assert lib.tmq_ternary_linear_ws(ops.ptr(x), _capi.F32, M, K, ops.ptr(nw.buf), N, ctypes.byref(ep), ops.ptr(y),
+                                         wptr, wbytes, None) == 0
+        torch.cuda.synchronize()
+        assert ((y.double() - ref).abs().max() / ref.abs().max()).item() <= 1e-5
+    eager = ops.ternary_linear(x, nw)
+    s = torch.cuda.Stream()
+    with torch.cuda.stream(s):
+        ops.ternary_linear(x, nw)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=s):
+            out = ops.ternary_linear(x, nw)
+    for _ in range(3):
+        out.zero_()
+        graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(out, eager)

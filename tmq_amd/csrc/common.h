@@ -100,6 +100,7 @@ struct FastDiv {
 // the others are dropped. A phase of a transposed convolution writes its share of the interleaved output this way.
 struct NoMap {                          // rows are consecutive: row m is pixel m (an empty member of the epilogue structs)
     static constexpr bool kDrops = false;   // pixel() never returns -1
+    static constexpr bool kPairs = false;   // rows r and r ^ 8 of a 16-row fragment are not added
 #if defined(__HIPCC__)
     __device__ __forceinline__ int64_t pixel(int64_t m) const { return m; }
 #endif
@@ -107,6 +108,7 @@ struct NoMap {                          // rows are consecutive: row m is pixel 
 
 struct RowMap {
     static constexpr bool kDrops = true;
+    static constexpr bool kPairs = false;
     FastDiv hw, w;                     // computed positions per image / per image row
     int32_t h0 = 0, w0 = 0, h_cnt = 0, w_cnt = 0;
     int64_t sb = 0, sh = 0, sw = 0;    // in pixels
@@ -118,6 +120,29 @@ struct RowMap {
         ow -= w0;
         if ((uint32_t)oh >= (uint32_t)h_cnt || (uint32_t)ow >= (uint32_t)w_cnt) return -1;
         return (int64_t)b * sb + (int64_t)oh * sh + (int64_t)ow * sw;
+    }
+#endif
+};
+
+// fp32 rows carried as two fp16 rows each (hi = fp16(s x), lo = fp16(s x - hi)), eight rows at a time: rows
+// 16 q .. 16 q + 7 of the fp16 matrix are the hi terms of output rows 8 q .. 8 q + 7, rows 16 q + 8 .. 16 q + 15 their
+// lo terms -- a pair always sits in one 16-row MFMA fragment, whatever the tile. Every group of eight rows has a power
+// of two s of its own. The epilogues add rows r and r ^ 8 of a fragment where they read it back from LDS (kPairs) and
+// multiply by the group's 1 / s (group_scale[m / 16]) before the per-channel scale; the lo rows are dropped and row m
+// goes to output row 8 (m / 16) + m % 8.
+struct PairMap {
+    static constexpr bool kDrops = true;
+    static constexpr bool kPairs = true;
+    int64_t rows_out = 0;
+    const float *group_scale = nullptr;     // ceil(rows_out / 8) floats
+#if defined(__HIPCC__)
+    __device__ __forceinline__ int64_t pixel(int64_t m) const {
+        const int64_t o = ((m >> 4) << 3) + (m & 7);
+        return (m & 8) || o >= rows_out ? -1 : o;
+    }
+    // 1 / s of the fragment that starts at row m16 (a multiple of 16); fragments past the last group: 0
+    __device__ __forceinline__ float fragment_scale(int64_t m16) const {
+        return (m16 >> 1) < rows_out ? group_scale[m16 >> 4] : 0.f;
     }
 #endif
 };

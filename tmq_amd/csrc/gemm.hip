@@ -1001,9 +1001,8 @@ int dispatch_tile(const Loader &ld, const void *native, int64_t M, int64_t K, in
 
 }  // namespace
 
-int launch_gemm_dense(const void *x, int64_t M, int64_t K, const void *native, int64_t N, const float *scale,
-                      const float *bias, const void *residual, int relu, void *y, int y_f16, void *stream) {
-    Epilogue ep{scale, bias, residual, y, relu, y_f16};
+template <class Ep>
+static int gemm_dense(const void *x, int64_t M, int64_t K, const void *native, int64_t N, const Ep &ep, void *stream) {
     // Dense rows through a buffer resource: the kernel that puts its expansion and loads between the MFMAs.
     //  * A chip full of 128 x 512 tiles (N a multiple of 512), eight wavefronts of 128 rows x 64 channels, one k-tile
     //    per pass: every activation row is read N / 512 times from L2. Against 128 x 256 tiles with two workgroups
@@ -1025,7 +1024,20 @@ int launch_gemm_dense(const void *x, int64_t M, int64_t K, const void *native, i
     }
     if ((K % kBK == 0) && aligned16(x))
         return dispatch_tile(DenseDirect{static_cast<const _Float16 *>(x), M, K}, native, M, K, N, ep, stream);
-    return dispatch_tile(DenseLoader{static_cast<const _Float16 *>(x), M, K}, native, M, K, N, ep, stream);
+    if constexpr (decltype(ep.map)::kPairs) return TMQ_ERR_UNSUPPORTED;      // row pairs are made aligned
+    else return dispatch_tile(DenseLoader{static_cast<const _Float16 *>(x), M, K}, native, M, K, N, ep, stream);
+}
+
+int launch_gemm_dense(const void *x, int64_t M, int64_t K, const void *native, int64_t N, const float *scale,
+                      const float *bias, const void *residual, int relu, void *y, int y_f16, void *stream) {
+    return gemm_dense(x, M, K, native, N, Epilogue{scale, bias, residual, y, relu, y_f16}, stream);
+}
+
+// The same on M16 fp16 rows that are the hi / lo terms of rows_out fp32 rows in groups of eight (PairMap).
+int launch_gemm_dense_pairs(const void *x16, int64_t M16, int64_t K, const void *native, int64_t N, const float *scale,
+                            const float *bias, const void *residual, int relu, void *y, int y_f16, int64_t rows_out,
+                            const float *group_scale, void *stream) {
+    return gemm_dense(x16, M16, K, native, N, PairEpilogue{scale, bias, residual, y, relu, y_f16, PairMap{rows_out, group_scale}}, stream);
 }
 
 // Adds the slices of a reduction that was cut across workgroups in slice order (deterministic) and applies the
@@ -1106,6 +1118,24 @@ inline bool row_pairs_ok(const void *x, int64_t M, int64_t K) {
 }
 inline size_t row_pairs_bytes(int64_t M, int64_t K) { return 256 + (size_t)(2 * M * K) * sizeof(_Float16); }
 
+// Seventeen fp32 rows or more over K a multiple of 64: one launch splits them into fp16 row pairs in groups of eight,
+// every group scaled by a power of two of its own (PairMap); the fp16 kernels then run once over 16 ceil(M / 8) rows
+// and their epilogues add each pair and undo the group's scale. Against the kernels that split on the fly, or two
+// fp16 passes chained through the residual.
+int launch_split_groups(const float *x, int64_t M, int64_t K, void *x16, float *group_scale, void *stream);
+int launch_mid_dense_pairs(const void *x16, int64_t M16, int64_t K, const void *native, int64_t N, const float *scale,
+                           const float *bias, const void *residual, int relu, void *y, int y_f16, int64_t rows_out,
+                           const float *group_scale, void *stream);
+inline int64_t pair_rows16(int64_t M) { return (M + 7) / 8 * 16; }
+inline bool pair_rows_ok(const void *x, int64_t M, int64_t K, int64_t N) {
+    return M >= 17 && K % 64 == 0 && K >= 256 && aligned16(x) && pair_rows16(M) * K < (int64_t)0x7FFFFFFF;
+}
+// the workspace: the groups' 1 / s (padded to 256 bytes), then the fp16 rows
+inline size_t pair_scale_bytes(int64_t M) { return ((size_t)((M + 7) / 8) * sizeof(float) + 255) & ~(size_t)255; }
+inline size_t pair_rows_bytes(int64_t M, int64_t K, int64_t N) {
+    return pair_scale_bytes(M) + (size_t)(pair_rows16(M) * K) * sizeof(_Float16);
+}
+
 }  // namespace tmq
 
 namespace tmq {
@@ -1148,7 +1178,8 @@ extern "C" {
 
 size_t tmq_ternary_linear_workspace_bytes(int x_dtype, int64_t M, int64_t K, int64_t N) {
     if (M <= 0 || K <= 0 || N <= 0) return 0;
-    if (x_dtype == TMQ_F32) return row_pairs_ok(nullptr, M, K) ? row_pairs_bytes(M, K) : 0;
+    if (x_dtype == TMQ_F32)
+        return row_pairs_ok(nullptr, M, K) ? row_pairs_bytes(M, K) : pair_rows_ok(nullptr, M, K, N) ? pair_rows_bytes(M, K, N) : 0;
     if (x_dtype != TMQ_F16) return 0;
     static const _Float16 *const aligned = nullptr;              // the plan assumes 16-byte aligned rows; _ws checks the real pointer
     const int slices = rows_split_slices(aligned, M, K, N);
@@ -1179,6 +1210,20 @@ int tmq_ternary_linear_ws(const void *x, int x_dtype, int64_t M, int64_t K, cons
             if (st) return st;
         }
         return TMQ_OK;
+    }
+    if (x && native && y && x_dtype == TMQ_F32 && N > 0 && workspace && aligned16(workspace) && aligned16(native) &&
+        !row_pairs_ok(x, M, K) && pair_rows_ok(x, M, K, N) && workspace_bytes >= pair_rows_bytes(M, K, N)) {
+        tmq_epilogue e = {nullptr, nullptr, nullptr, 0, TMQ_F32};
+        if (epilogue) e = *epilogue;
+        if (e.y_dtype != TMQ_F16 && e.y_dtype != TMQ_F32) return TMQ_ERR_UNSUPPORTED;
+        float *group_scale = static_cast<float *>(workspace);
+        void *x16 = static_cast<unsigned char *>(workspace) + pair_scale_bytes(M);
+        if (int st = launch_split_groups(static_cast<const float *>(x), M, K, x16, group_scale, stream)) return st;
+        const int64_t M16 = pair_rows16(M);
+        const int y_f16 = e.y_dtype == TMQ_F16 ? 1 : 0;
+        if (split_reduction_pays(M16, K, N))
+            return launch_mid_dense_pairs(x16, M16, K, native, N, e.scale, e.bias, e.residual, e.relu, y, y_f16, M, group_scale, stream);
+        return launch_gemm_dense_pairs(x16, M16, K, native, N, e.scale, e.bias, e.residual, e.relu, y, y_f16, M, group_scale, stream);
     }
     if (x && native && y && x_dtype == TMQ_F16 && M > 0 && K > 0 && N > 0 && workspace && aligned16(workspace) && aligned16(native)) {
         const int slices = rows_split_slices(x, M, K, N);

@@ -247,6 +247,8 @@ __device__ __forceinline__ void reduce_and_store(unsigned char *smem, const floa
     auto partial_sums = [&](int row) {
         floatx4 v = row_sums(row);
         if constexpr (Pairs::kOn) v = (v + row_sums(row + pairs.pair)) * pairs.row_scale[m0 + row];
+        if constexpr (decltype(ep.map)::kPairs)                                  // the hi row's sums, then its lo row's, / s
+            v = (v + row_sums(row ^ 8)) * ep.map.fragment_scale((m0 + row) & ~(int64_t)15);
         return v * sc + bi;
     };
     if (vec) {
@@ -1062,6 +1064,14 @@ int launch_mid_dense(const void *x, int64_t M, int64_t K, const void *native, in
                      const float *bias, const void *residual, int relu, void *y, int y_f16, void *stream) {
     MidEpilogue ep{scale, bias, residual, y, relu, y_f16};
     return dispatch(DenseRows{static_cast<const _Float16 *>(x), M, K}, native, M, K, N, ep, stream);
+}
+
+// The same on M16 fp16 rows that are the hi / lo terms of rows_out fp32 rows in groups of eight (PairMap).
+int launch_mid_dense_pairs(const void *x16, int64_t M16, int64_t K, const void *native, int64_t N, const float *scale,
+                           const float *bias, const void *residual, int relu, void *y, int y_f16, int64_t rows_out,
+                           const float *group_scale, void *stream) {
+    MidEpilogueT<PairMap> ep{scale, bias, residual, y, relu, y_f16, PairMap{rows_out, group_scale}};
+    return dispatch(DenseRows{static_cast<const _Float16 *>(x16), M16, K}, native, M16, K, N, ep, stream);
 }
 
 // True when the weight-stream kernel can take a dense fp16 problem of at most 16 rows.

@@ -205,7 +205,83 @@ __global__ __launch_bounds__(1024) void split_rows_kernel(const float *__restric
     }
 }
 
+// Many fp32 rows as fp16 row pairs in groups of eight, every group under a power of two s of its own: a workgroup
+// of 1024 takes the group's 8 K values -- float4 number 1024 i + t to thread t, up to NQ of them in
+// registers and all asked for at once (a single trip to memory; longer rows are read a second time) -- finds the
+// largest finite |x|, and writes hi = fp16(s x) of row m to x16 row 16 (m / 8) + m % 8, lo = fp16(s x - hi) eight rows
+// further on (rows past M of the last group: zeros) and 1 / s to group_scale[m / 8]. K a multiple of 4.
+template <int NQ>
+__global__ __launch_bounds__(1024) void split_groups_kernel(const float *__restrict__ x, int64_t M, int64_t K,
+                                                            _Float16 *__restrict__ x16, float *__restrict__ group_scale) {
+    __shared__ float lds[17];
+    const int64_t g = blockIdx.x, q_row = K / 4, quads = 8 * q_row;              // float4s per row / per group
+    const float *src = x + g * 8 * K;
+    int64_t live = (M - g * 8) * q_row;                                            // float4s that exist
+    if (live > quads) live = quads;
+    const bool held = quads <= (int64_t)NQ * 1024;
+    floatx4 q[NQ];
+    float amax = 0.f;
+    if (held) {
+#pragma unroll
+        for (int i = 0; i < NQ; i++) {
+            const int64_t at = (int64_t)i * 1024 + threadIdx.x;
+            q[i] = at < live ? __builtin_nontemporal_load(reinterpret_cast<const floatx4 *>(src) + at) : floatx4{0.f, 0.f, 0.f, 0.f};
+        }
+#pragma unroll
+        for (int i = 0; i < NQ; i++)
+            amax = fmaxf(fmaxf(amax, fmaxf(finite_abs(q[i][0]), finite_abs(q[i][1]))), fmaxf(finite_abs(q[i][2]), finite_abs(q[i][3])));
+    } else {
+        for (int64_t at = threadIdx.x; at < live; at += 1024) {
+            const floatx4 v = *(reinterpret_cast<const floatx4 *>(src) + at);
+            amax = fmaxf(fmaxf(amax, fmaxf(finite_abs(v[0]), finite_abs(v[1]))), fmaxf(finite_abs(v[2]), finite_abs(v[3])));
+        }
+    }
+    amax = block_max(amax, lds);
+    float s, inv;
+    make_prescale(amax, s, inv);
+    if (threadIdx.x == 0 && blockIdx.y == 0) group_scale[g] = inv;
+    // gridDim.y workgroups (a power of two) share a group: each takes the whole group for the maximum -- one CU pulls
+    // ~40 GB/s, and the idle CUs are free -- and converts every gridDim.y-th run of 1024 float4s
+    const int share = gridDim.y - 1, mine = blockIdx.y;
+    _Float16 *dst = x16 + g * 16 * K;                                              // the group's hi rows, then its lo rows
+    auto emit = [&](int64_t at, floatx4 v) {
+        v *= s;
+        half4 h, l;
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            h[e] = (_Float16)v[e];
+            l[e] = (_Float16)(v[e] - (float)h[e]);
+        }
+        *reinterpret_cast<half4 *>(dst + 4 * at) = h;                              // row at / q_row of the group, same position
+        *reinterpret_cast<half4 *>(dst + 8 * K + 4 * at) = l;
+    };
+    if (held) {
+#pragma unroll
+        for (int i = 0; i < NQ; i++) {
+            const int64_t at = (int64_t)i * 1024 + threadIdx.x;
+            if ((i & share) == mine && at < quads) emit(at, q[i]);
+        }
+    } else {
+        for (int64_t at = (int64_t)mine * 1024 + threadIdx.x; at < quads; at += (int64_t)(share + 1) * 1024)
+            emit(at, at < live ? *(reinterpret_cast<const floatx4 *>(src) + at) : floatx4{0.f, 0.f, 0.f, 0.f});
+    }
+}
+
 }  // namespace
+
+// x16: 16 ceil(M / 8) rows of K fp16 values; group_scale: ceil(M / 8) floats. K % 4 == 0, x and x16 16-byte aligned.
+int launch_split_groups(const float *x, int64_t M, int64_t K, void *x16, float *group_scale, void *stream) {
+    const int64_t groups = (M + 7) / 8, quads = 8 * (K / 4);
+    if (groups > 0x7FFFFFFF) return TMQ_ERR_TOO_LARGE;
+    auto kernel = quads <= 2 * 1024 ? split_groups_kernel<2> : quads <= 4 * 1024 ? split_groups_kernel<4>
+                : quads <= 8 * 1024 ? split_groups_kernel<8> : split_groups_kernel<16>;
+    // up to 64 groups share a group among up to four workgroups (M = 32 at K = 4096: 14.5 -> 13.4 us in all, M = 512
+    // 42.4 -> 40.8; M = 1024, where the CUs are busy anyway, 62.0 -> 63.1)
+    const uint32_t share = groups > 64 || quads <= 1024 ? 1 : quads <= 2048 ? 2 : 4;
+    hipLaunchKernelGGL(kernel, dim3((uint32_t)groups, share), dim3(1024), 0, as_stream(stream), x, M, K,
+                       static_cast<_Float16 *>(x16), group_scale);
+    return check_launch();
+}
 
 // x16: 2 M rows of K fp16 values, row_scale: M floats; K % 8 == 0, x and x16 16-byte aligned.
 int launch_split_rows(const float *x, int64_t M, int64_t K, int64_t group, void *x16, float *row_scale, void *stream) {

@@ -19,6 +19,7 @@ struct EpilogueT {
 };
 using Epilogue = EpilogueT<NoMap>;
 using ViewEpilogue = EpilogueT<RowMap>;
+using PairEpilogue = EpilogueT<PairMap>;
 static_assert(sizeof(Epilogue) == 40, "the dense epilogue carries no map");
 
 #if defined(__HIPCC__)
@@ -94,6 +95,11 @@ __device__ __forceinline__ void write_tile_wide(float *slab, const floatx4 (&acc
     const _Float16 *res = static_cast<const _Float16 *>(ep.residual);
     int64_t off[kAhead][kPieces];                                  // element offset of the lane's piece, -1: none
     u32x4 rs[kAhead][kPieces];
+    float gs[WM];                                                  // row pairs: 1 / s of each fragment's group
+    if constexpr (decltype(ep.map)::kPairs) {
+#pragma unroll
+        for (int i = 0; i < WM; i++) gs[i] = ep.map.fragment_scale(mw0 + (int64_t)i * 16);
+    }
     auto request = [&](int i, int slot) {
 #pragma unroll
         for (int t = 0; t < kPieces; t++) {
@@ -121,8 +127,14 @@ __device__ __forceinline__ void write_tile_wide(float *slab, const floatx4 (&acc
         for (int t = 0; t < kPieces; t++) {
             const int idx = t * 64 + lane, row = idx / (2 * WN), c8 = idx % (2 * WN);
             if (idx >= 32 * WN) continue;
-            floatx4 v0 = *reinterpret_cast<const floatx4 *>(&slab[row * kEP + c8 * 8]) * cc.sc[0] + cc.bi[0];
-            floatx4 v1 = *reinterpret_cast<const floatx4 *>(&slab[row * kEP + c8 * 8 + 4]) * cc.sc[1] + cc.bi[1];
+            floatx4 v0 = *reinterpret_cast<const floatx4 *>(&slab[row * kEP + c8 * 8]);
+            floatx4 v1 = *reinterpret_cast<const floatx4 *>(&slab[row * kEP + c8 * 8 + 4]);
+            if constexpr (decltype(ep.map)::kPairs) {              // (hi row + its lo row) / s
+                v0 = (v0 + *reinterpret_cast<const floatx4 *>(&slab[(row ^ 8) * kEP + c8 * 8])) * gs[i];
+                v1 = (v1 + *reinterpret_cast<const floatx4 *>(&slab[(row ^ 8) * kEP + c8 * 8 + 4])) * gs[i];
+            }
+            v0 = v0 * cc.sc[0] + cc.bi[0];
+            v1 = v1 * cc.sc[1] + cc.bi[1];
             const int64_t o = off[i % kAhead][t];
             if (o < 0) continue;
             if (res) {
@@ -169,6 +181,11 @@ __device__ __forceinline__ void write_tile(float *slab, const floatx4 (&acc)[WM]
     const int r16 = lane & 15, g = lane >> 4;
     const bool vec = (N % 4 == 0) && ((reinterpret_cast<uintptr_t>(ep.y) | reinterpret_cast<uintptr_t>(ep.residual)) & 15u) == 0;
     if (wide_rows(ep, N)) return write_tile_wide<WM, WN>(slab, acc, cc, lane, mw0, nw0, M, N, ep);
+    float gs[WM];                                          // row pairs: 1 / s of each fragment's group
+    if constexpr (decltype(ep.map)::kPairs) {
+#pragma unroll
+        for (int i = 0; i < WM; i++) gs[i] = ep.map.fragment_scale(mw0 + (int64_t)i * 16);
+    }
 #pragma unroll
     for (int i = 0; i < WM; i++) {
 #pragma unroll
@@ -181,7 +198,9 @@ __device__ __forceinline__ void write_tile(float *slab, const floatx4 (&acc)[WM]
         for (int t = 0; t < WN; t++) {                     // 16 rows x (16 WN / 4) float4 = 64 WN float4 per slab
             const int idx = t * 64 + lane, row = idx / (4 * WN), c4 = idx % (4 * WN);
             const int64_t m = mrow0 + row, n = nw0 + c4 * 4;
-            floatx4 v = *reinterpret_cast<const floatx4 *>(&slab[row * kEP + c4 * 4]) * cc.sc[0] + cc.bi[0];
+            floatx4 v = *reinterpret_cast<const floatx4 *>(&slab[row * kEP + c4 * 4]);
+            if constexpr (decltype(ep.map)::kPairs) v = (v + *reinterpret_cast<const floatx4 *>(&slab[(row ^ 8) * kEP + c4 * 4])) * gs[i];
+            v = v * cc.sc[0] + cc.bi[0];
             if (m >= M || n >= N) continue;
             const int64_t px = ep.map.pixel(m);
             if (decltype(ep.map)::kDrops && px < 0) continue;

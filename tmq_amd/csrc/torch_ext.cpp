@@ -238,15 +238,16 @@ void check_mm_args(const torch::Tensor &lhs, const torch::Tensor &weights, int64
 // fp32 activations (the reference's convention). The kernels carry them as fp16 terms, so the tensor is first
 // scaled by the power of two that brings its largest value into fp16's range (tmq_f32_prescale; exact, undone
 // in the epilogue's per-channel scale): any magnitude works, as with the reference's fp32 arithmetic. Many
-// rows: the fp16 kernels over the two fp16 terms, y = W hi + W lo; two to sixteen rows over whole weight blocks: the
-// two terms as row pairs of one fp16 pass; otherwise the kernels that split on the fly.
+// The two terms travel as row pairs of one fp16 pass wherever tmq_ternary_linear_ws takes the shape; otherwise many
+// rows run the fp16 kernels over the two fp16 terms, y = W hi + W lo, and few rows the kernels that split on the fly.
 torch::Tensor linear_f32(const torch::Tensor &x, int64_t M, int64_t K, const torch::Tensor &native, int64_t columns,
                          torch::Tensor &y, const char *name) {
     if (tmq_fp32_rows_self_scaled(x.data_ptr(), M, K)) {   // a single row the kernel scales itself: one launch
         check(tmq_ternary_linear(x.data_ptr(), TMQ_F32, M, K, native.data_ptr(), columns, nullptr, y.data_ptr(), stream_of(x)), name);
         return y;
     }
-    // a few rows: fp16 row pairs made once in a workspace, one pass of the fp16 weight stream (tmq_ternary_linear_ws)
+    // fp16 row pairs made once in a workspace, one pass of the fp16 kernels with the pairs added in the epilogue
+    // (tmq_ternary_linear_ws: two or more rows over whole 64-index tiles)
     if (const size_t pairs = tmq_ternary_linear_workspace_bytes(TMQ_F32, M, K, columns);
         pairs && reinterpret_cast<uintptr_t>(x.data_ptr()) % 16 == 0) {
         auto ws = torch::empty({(int64_t)pairs}, x.options().dtype(torch::kUInt8));

@@ -611,10 +611,10 @@ def ternary_linear(x: torch.Tensor, nw: NativeWeights, scale=None, bias=None, re
     pairs = 0
     if x.dtype == torch.float32 and M == 1 and x.is_contiguous() and _lib().tmq_fp32_rows_self_scaled(ptr(x), M, nw.K):
         pass            # a single row the kernel scales itself (any magnitude): one launch, no prescale pass
-    elif (x.dtype == torch.float32 and 2 <= M <= 16 and x.is_contiguous() and x.data_ptr() % 16 == 0
+    elif (x.dtype == torch.float32 and M >= 2 and x.is_contiguous() and x.data_ptr() % 16 == 0
           and _lib().tmq_ternary_linear_workspace_bytes(_capi.F32, M, nw.K, nw.N)):
-        # a few rows: split once into fp16 row pairs (each row scaled by its own power of two, any magnitude) in the
-        # workspace, then one pass of the fp16 weight stream
+        # split once into fp16 row pairs in the workspace (a few rows: each scaled by its own power of two; from
+        # seventeen: the whole tensor by one), then one pass of the fp16 kernels with the pairs added in the epilogue
         pairs = _lib().tmq_ternary_linear_workspace_bytes(_capi.F32, M, nw.K, nw.N)
     elif x.dtype == torch.float32 and M > 0:
         two_pass = (out_dtype == torch.float32 and (residual is None or residual.dtype == torch.float32)
