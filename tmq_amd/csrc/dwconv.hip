@@ -175,10 +175,12 @@ __global__ __launch_bounds__(256) void dwconv_image_kernel(const _Float16 *__res
 // The common cases -- windows of ky rows x KS columns (KS of 1 .. 5 or 7, any ky), horizontal stride 1 or 2 and
 // dilation DX of 1 or 2, any vertical stride and dilation, whole groups of 8 channels, fewer than 2^31 threads. A
 // thread owns 8 channels of PX horizontally adjacent output positions: the columns their windows share are loaded once
-// (for stride 1, PX + KS - 1 columns per row instead of KS PX), the 8 weights of a tap are expanded to floats once
-// for all PX positions, and the index arithmetic is multiply-high (FastDiv). All loads of a row are in
+// (for stride 1, PX + KS - 1 columns per row instead of KS PX), the 8 weights of a tap are expanded to fp16 operands
+// once for all PX positions, and the index arithmetic is multiply-high (FastDiv). All loads of a row are in
 // flight together; taps outside the image read the clamped pixel and are replaced by zero. Per output the
-// taps are accumulated in the same order as in dwconv_image_kernel (fp32, every product exact).
+// taps are accumulated in the same order as in dwconv_image_kernel (fp32, every product exact). Workgroups are taken
+// in an order that keeps one XCD on neighbouring pieces of the image (the input rows that vertically adjacent
+// outputs share then come from that XCD's L2: batch 64, 128 channels, 56 x 56, 3 x 3: 32.8 -> 28.4 us).
 // KY: the window's rows when they equal KS and neither direction is dilated (the square windows of the common
 // depthwise layers keep a compile-time row count), 0: ky and dy from the arguments.
 template <int KS, int PX, int SX, int DX = 1, int KY = 0>
@@ -187,7 +189,9 @@ __global__ __launch_bounds__(256) void dwconv_square_image_kernel(const _Float16
                                                               FastDiv by_wg, FastDiv by_ho, int ky, int sy, int py, int px,
                                                               int dy, DwEpilogue ep) {
     constexpr int NC = (PX - 1) * SX + (KS - 1) * DX + 1;          // input columns the PX windows cover
-    const uint32_t id = blockIdx.x * 256u + threadIdx.x;
+    // workgroups of one XCD take neighbouring pieces of the image: the rows that vertically adjacent outputs share
+    // are then found in that XCD's L2
+    const uint32_t id = (uint32_t)xcd_contiguous((int)blockIdx.x, (int)gridDim.x) * 256u + threadIdx.x;
     if (id >= total) return;
     int cg, wg, oh;
     const uint32_t p = by_g.divmod(id, cg);                         // channel group fastest: neighbours share a pixel
@@ -232,17 +236,23 @@ __global__ __launch_bounds__(256) void dwconv_square_image_kernel(const _Float16
         }
 #pragma unroll
         for (int j = 0; j < KS; j++) {
-            const uint32_t codes = codes8(words, Q, i * KS + j, c0);
-            float w[8];
+            // The 8 codes as fp16 operands, two per register: 01 / 10 / 11 become 01 / 11 / 10 (an fp16's 2.0 bit and
+            // sign: +2, -2, -0), channels 4 .. 7 move 8 bits down, and (t << 2 e) & 0xC000C000 is channel e's weight in
+            // the high half and channel e + 4's in the low half -- 15 operations per tap instead of 32, and every
+            // product one v_fma_mix_f32 on two fp16 sources. The sums run at exactly twice their value.
+            uint32_t codes = codes8(words, Q, i * KS + j, c0);
+            codes ^= (codes >> 1) & 0x55555555u;
+            const uint32_t t = (codes & 0xFF000000u) | ((codes >> 8) & 0x0000FF00u);
+            half2v w[4];
 #pragma unroll
-            for (int e = 0; e < 8; e++) {
-                const uint32_t cd = (codes >> (30 - 2 * e)) & 3u;   // 01 -> +1, 10 -> -1, 00 / 11 -> 0
-                w[e] = (float)((int)(cd & 1u) - (int)(cd >> 1));
-            }
+            for (int e = 0; e < 4; e++) w[e] = __builtin_bit_cast(half2v, (t << (2 * e)) & 0xC000C000u);
 #pragma unroll
             for (int q = 0; q < PX; q++)
 #pragma unroll
-                for (int e = 0; e < 8; e++) acc[q][e] = __builtin_fmaf((float)v[q * SX + j * DX][e], w[e], acc[q][e]);
+                for (int e = 0; e < 4; e++) {
+                    acc[q][e] = __builtin_fmaf((float)v[q * SX + j * DX][e], (float)w[e][1], acc[q][e]);
+                    acc[q][4 + e] = __builtin_fmaf((float)v[q * SX + j * DX][4 + e], (float)w[e][0], acc[q][4 + e]);
+                }
         }
     }
     // epilogue: the 8 channels' scale and bias once for all PX positions, 16-byte accesses throughout
@@ -250,6 +260,8 @@ __global__ __launch_bounds__(256) void dwconv_square_image_kernel(const _Float16
 #pragma unroll
     for (int q = 0; q < PX; q++) {
         if (ow0 + q >= Wo) break;
+#pragma unroll
+        for (int e = 0; e < 8; e++) acc[q][e] *= 0.5f;             // exact: the weights were +-2
         store8_vec(ep, cc, ((int64_t)(r * (uint32_t)Wo) + ow0 + q) * C + c0, acc[q]);
     }
 }
