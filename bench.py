@@ -493,7 +493,8 @@ def bench_layers(args, torch):
                                         "note": "one stride-1 implicit-GEMM convolution per output phase, written in place (tmq_ternary_conv2d_view)"}
     res["value"] = res["dw3x3"]["us"]
     res["roofline"] = {"bound": "hbm", "achieved": res["dw3x3"]["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": res["dw3x3"]["frac_hbm"],
-                       "traffic": None, "algorithmic_bytes": 2 * xs[0].numel() * 2, "kernel": "dwconv_square_image_kernel<3, 4, 1, 1, 3>",
+                       "traffic": measured_traffic("depthwise_layers_batch64.md", key="traffic_bytes_dw3x3"),
+                       "algorithmic_bytes": 2 * xs[0].numel() * 2, "kernel": "dwconv_square_image_kernel<3, 4, 1, 1, 3>",
                        "avg_launch_us": res["dw3x3"]["us"]}
     return res
 
