@@ -469,6 +469,19 @@ def bench_layers(args, torch):
         us = _graph_time_us(torch, run, max(2, args.steps // 4), args.settle_ms)
         byts = 2 * xs[0].numel() * 2
         res[name] = {"us": round(us, 3), "gbs": round(byts / us / 1e3, 1), "frac_hbm": round(byts / us / 1e3 / HBM_PEAK_GBS, 4)}
+    # depthwise transposed convolution (tmq/tmq_cuda.cu:118-162), 128 channels, 28 x 28 -> 56 x 56, 4 x 4 / 2, gathered
+    # per output position
+    xh = [torch.randn((B, C, 28, 28), device=dev, generator=g).half().contiguous(memory_format=torch.channels_last) for _ in range(4)]
+    words_t = ops.compactify_ternary(torch.randint(-1, 2, (C, 1, 4, 4), device=dev, generator=g).float())
+
+    def run_dwt():
+        for x in xh:
+            ops.ternary_dwconvtrans2d(x, words_t, 4, 2, 1, 0, 1, out_dtype=torch.float16)
+        return len(xh)
+    run_dwt()
+    us = _graph_time_us(torch, run_dwt, max(2, args.steps // 4), args.settle_ms)
+    byts = 5 * xh[0].numel() * 2
+    res["dwconvtrans4x4s2"] = {"us": round(us, 3), "gbs": round(byts / us / 1e3, 1), "frac_hbm": round(byts / us / 1e3 / HBM_PEAK_GBS, 4)}
     net = torch.nn.Sequential(torch.nn.ConvTranspose2d(128, 64, 4, 2, 1, bias=True))
     ctrl = t.QuantizationControl()
     t.quantize_model(net, ctrl)

@@ -158,15 +158,27 @@ __global__ __launch_bounds__(256) void dwconv_image_kernel(const _Float16 *__res
             const _Float16 *src = x + (((int64_t)b * H + ih) * W + iw) * C + c0;
             uint32_t codes = codes8(words, Q, i * kx + j, c0);
             if (vec) {
+                // the codes as fp16 +-2.0 operands, two per register (see dwconv_square_image_kernel): the sums run at
+                // twice their value and are halved below
                 const half8 v = *reinterpret_cast<const half8 *>(src);
+                codes ^= (codes >> 1) & 0x55555555u;
+                const uint32_t t = (codes & 0xFF000000u) | ((codes >> 8) & 0x0000FF00u);
 #pragma unroll
-                for (int e = 0; e < 8; e++) acc[e] += apply_code((float)v[e], codes << (2 * e));
+                for (int e = 0; e < 4; e++) {
+                    const half2v w = __builtin_bit_cast(half2v, (t << (2 * e)) & 0xC000C000u);
+                    acc[e] = __builtin_fmaf((float)v[e], (float)w[1], acc[e]);
+                    acc[4 + e] = __builtin_fmaf((float)v[4 + e], (float)w[0], acc[4 + e]);
+                }
             } else {
 #pragma unroll
                 for (int e = 0; e < 8; e++)
                     if (c0 + e < C) acc[e] += apply_code((float)src[e], codes << (2 * e));
             }
         }
+    }
+    if (vec) {
+#pragma unroll
+        for (int e = 0; e < 8; e++) acc[e] *= 0.5f;                 // exact: the weights were +-2
     }
     if (vec & 2) store8_vec(ep, load_channel_constants(ep, c0), p * C + c0, acc);
     else store8(ep, p * C + c0, c0, C, acc, vec);
@@ -314,30 +326,56 @@ __global__ __launch_bounds__(256) void dwconvtrans_image_kernel(const _Float16 *
     const int64_t r = div_rem(p, Wo, ow);
     const int b = (int)div_rem(r, Ho, oh);
     float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    for (int i = 0; i < ky; i++) {
-        const int ny = oh + py - i * dy;
-        if (ny < 0 || ny % sy) continue;
-        const int ih = ny / sy;
-        if (ih >= H) continue;
-        for (int j = 0; j < kx; j++) {
-            const int nx = ow + px - j * dx;
-            if (nx < 0 || nx % sx) continue;
-            const int iw = nx / sx;
-            if (iw >= W) continue;
-            const _Float16 *src = x + (((int64_t)b * H + ih) * W + iw) * C + c0;
-            const uint32_t codes = codes8(words, Q, i * kx + j, c0);
-            if (vec) {
-                const half8 v = *reinterpret_cast<const half8 *>(src);
+    auto tap = [&](int i, int j, int ih, int iw) {
+        const _Float16 *src = x + (((int64_t)b * H + ih) * W + iw) * C + c0;
+        const uint32_t codes = codes8(words, Q, i * kx + j, c0);
+        if (vec) {
+            // the codes as fp16 +-2.0 operands, two per register (see dwconv_square_image_kernel): the sums run at twice
+            // their value and are halved below
+            const half8 v = *reinterpret_cast<const half8 *>(src);
+            const uint32_t fixed = codes ^ ((codes >> 1) & 0x55555555u);
+            const uint32_t t = (fixed & 0xFF000000u) | ((fixed >> 8) & 0x0000FF00u);
 #pragma unroll
-                for (int e = 0; e < 8; e++) acc[e] += apply_code((float)v[e], codes << (2 * e));
-            } else {
+            for (int e = 0; e < 4; e++) {
+                const half2v w = __builtin_bit_cast(half2v, (t << (2 * e)) & 0xC000C000u);
+                acc[e] = __builtin_fmaf((float)v[e], (float)w[1], acc[e]);
+                acc[4 + e] = __builtin_fmaf((float)v[4 + e], (float)w[0], acc[4 + e]);
+            }
+        } else {
 #pragma unroll
-                for (int e = 0; e < 8; e++)
-                    if (c0 + e < C) acc[e] += apply_code((float)src[e], codes << (2 * e));
+            for (int e = 0; e < 8; e++)
+                if (c0 + e < C) acc[e] += apply_code((float)src[e], codes << (2 * e));
+        }
+    };
+    if (dy == 1 && dx == 1) {
+        // undilated: the taps that reach this position are i = (oh + py) % sy, + sy, ... (source row (oh + py - i) / sy,
+        // one lower per step), and the same along x -- no divisibility test per tap, ceil(ky / sy) ceil(kx / sx) visits
+        const int ty = oh + py, tx = ow + px, j0 = tx % sx;
+        for (int i = ty % sy, ih = ty / sy; i < ky && ih >= 0; i += sy, ih--) {
+            if (ih >= H) continue;
+            for (int j = j0, iw = tx / sx; j < kx && iw >= 0; j += sx, iw--)
+                if (iw < W) tap(i, j, ih, iw);
+        }
+    } else {
+        for (int i = 0; i < ky; i++) {
+            const int ny = oh + py - i * dy;
+            if (ny < 0 || ny % sy) continue;
+            const int ih = ny / sy;
+            if (ih >= H) continue;
+            for (int j = 0; j < kx; j++) {
+                const int nx = ow + px - j * dx;
+                if (nx < 0 || nx % sx) continue;
+                const int iw = nx / sx;
+                if (iw < W) tap(i, j, ih, iw);
             }
         }
     }
-    store8(ep, p * C + c0, c0, C, acc, vec);
+    if (vec) {
+#pragma unroll
+        for (int e = 0; e < 8; e++) acc[e] *= 0.5f;                 // exact: the weights were +-2
+    }
+    if (vec & 2) store8_vec(ep, load_channel_constants(ep, c0), p * C + c0, acc);
+    else store8(ep, p * C + c0, c0, C, acc, vec);
 }
 
 // Column form. A workgroup transposes a 64-patch x 64-channel tile of one batch entry through LDS:
@@ -487,7 +525,8 @@ int tmq_ternary_dwconvtrans2d(const void *x, const tmq_conv_shape *s, int32_t ou
     if (total == 0) return TMQ_OK;
     if (blocks > 0x7FFFFFFF) return TMQ_ERR_TOO_LARGE;
     const int y_f16 = e.y_dtype == TMQ_F16;
-    const int vec = (s->C % 8 == 0) && aligned_for(x, 16) && aligned_for(y, 16) && (!e.residual || aligned_for(e.residual, 16));
+    int vec = (s->C % 8 == 0) && aligned_for(x, 16) && aligned_for(y, 16) && (!e.residual || aligned_for(e.residual, 16));
+    if (vec && aligned_for(e.scale, 16) && aligned_for(e.bias, 16)) vec |= 2;       // the 16-byte epilogue as well
     DwEpilogue ep{e.scale, e.bias, e.residual, y, e.relu, y_f16};
     hipLaunchKernelGGL(dwconvtrans_image_kernel, dim3((uint32_t)blocks), dim3(256), 0, as_stream(stream),
                        static_cast<const _Float16 *>(x), words, s->B, s->C, s->H, s->W, ho, wo, s->ky, s->kx, s->sy, s->sx,
