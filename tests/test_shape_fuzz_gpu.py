@@ -1,6 +1,6 @@
 """Seeded walks over the shapes that decide which kernel family a ternary product takes: single rows and
 few rows (8-bit GEMV, weight stream, short reductions, skinny), mid-size dense products (split reduction,
-tile kernels), convolutions (three loaders, two tile families, the split-reduction form) and the fused
+tile kernels; fp32 rows as fp16 row pairs), convolutions (three loaders, two tile families, the split-reduction form) and the fused
 opening (one kernel or two), convolutions written into strided views, transposed convolutions and depthwise windows.
 Every case is checked against an fp64 product of the same operands
 (a11 / a12: tmq/tmq_cuda.cu:478-549, tmq/tmq.py:662-688, 822-871 compute the same sums in fp32), the fused
@@ -53,6 +53,18 @@ def test_walk_mid_size_dense(cuda):
         K = rnd.choice([64 * rnd.randint(8, 80), 256 * rnd.randint(2, 20), rnd.randint(100, 3000)])
         N = rnd.choice([128, 130, 256, 1000, 4096, 16 * rnd.randint(8, 300), rnd.randint(129, 5000)])
         _linear_case(ops, cuda, 500 + i, M, K, N, torch.float16)
+
+
+def test_walk_mid_size_fp32_rows(cuda):
+    """fp32 activations (the reference's convention): row pairs through the fp16 kernels where K is a multiple of 64,
+    the kernels that split on the fly elsewhere."""
+    from tmq_amd import ops
+    rnd = random.Random(7)
+    for i in range(60):
+        M = rnd.choice([rnd.randint(2, 40), rnd.randint(17, 600), rnd.randint(600, 2500)])
+        K = rnd.choice([64 * rnd.randint(4, 80), 256 * rnd.randint(2, 40), rnd.randint(100, 3000)])
+        N = rnd.choice([64, 130, 256, 1000, 4096, 16 * rnd.randint(8, 300), rnd.randint(1, 5000)])
+        _linear_case(ops, cuda, 900 + i, M, K, N, torch.float32)
 
 
 def test_walk_convolutions(cuda):
