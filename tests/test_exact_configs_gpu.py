@@ -121,7 +121,7 @@ def test_config4_resnet18_fused_paths_against_fp16_faithful_reference(cuda, batc
             t.fold_batchnorm(model)
             t.use_native_pooling(model)
             gm, sites = t.fuse_epilogues(model)
-            assert sites == 17
+            assert sites == 18
             got_fx = gm(x).float()
     finally:
         t.set_compact_output_dtype(prev)

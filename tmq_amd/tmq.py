@@ -1224,6 +1224,28 @@ class _FusedEpilogue(nn.Module):
         return self.pool(self.layer.compact_forward(x, None, True))
 
 
+class _FusedHead(nn.Module):
+    """linear(flatten(global_average_pool(x), 1)) as one launch when x is an fp16 channels_last feature map of up to
+    512 channels (the means stay in LDS and are the product's only activation row per image); the three modules as
+    they were otherwise."""
+
+    def __init__(self, pool, layer):
+        super().__init__()
+        self.pool = pool
+        self.layer = layer
+
+    @torch.no_grad()
+    def forward(self, x):
+        layer = self.layer
+        if (x.is_cuda and x.dim() == 4 and x.dtype == torch.float16 and x.is_contiguous(memory_format=torch.channels_last)
+                and not layer.training and layer.compact and layer.bn is None):
+            layer._update_scale()
+            nw = layer._native_weights()
+            scale, bias = layer._epilogue(nw.N, x.device)
+            return ops.avgpool_linear(x, nw, scale=scale, bias=bias, out_dtype=_compact_out)
+        return layer(torch.flatten(self.pool(x), 1))
+
+
 def fuse_epilogues(model: nn.Module):
     """Move the ReLU and the residual addition that follow a compact Conv2d / Linear in the model's forward
     into that layer's kernel epilogue (the reference's README lists this fusion as future work,
@@ -1231,10 +1253,12 @@ def fuse_epilogues(model: nn.Module):
     number of nn.Identity modules (what fold_batchnorm leaves behind) in between,
 
         relu(layer(x))      layer(x) + r      relu(layer(x) + r)      maxpool(relu(conv(x)))
+        linear(flatten(avgpool(x), 1))
 
     where `relu` is torch.relu / F.relu / x.relu() / an nn.ReLU module, `+` is +, += or torch.add, the
     layer is a compact Conv2d or Linear without a BatchNorm of its own, `maxpool` is an nn.MaxPool2d(3, 2, 1)
-    module (a ResNet's opening; one kernel once the layers hand on fp16), and the intermediate values have no
+    module (a ResNet's opening; one kernel once the layers hand on fp16), `avgpool` an nn.AdaptiveAvgPool2d(1) module
+    (a network's head: pooling and classifier in one launch on fp16 feature maps), and the intermediate values have no
     other use. Everything else stays as traced. For inference, after the layers went compact and after
     fold_batchnorm. Returns (GraphModule sharing the model's parameters, number of fused sites)."""
     import operator
@@ -1322,6 +1346,37 @@ def fuse_epilogues(model: nn.Module):
             cur = cur.args[0] if (cur.args[0] is not residual or not is_add(cur)) else cur.args[1]
             chain.append(cur)
         for n in chain:
+            graph.erase_node(n)
+        fused += 1
+    # a network's head: linear(flatten(avgpool(x), 1)) with a global average pool becomes one call
+    for node in list(graph.nodes):
+        if node.op != "call_module":
+            continue
+        layer = mods.get(node.target)
+        if not (isinstance(layer, Linear) and layer.compact and getattr(layer, "bn", None) is None and len(node.args) == 1
+                and not node.kwargs and isinstance(node.args[0], fx.Node)):
+            continue
+        fl = node.args[0]
+        flat = ((fl.op == "call_function" and fl.target is torch.flatten) or (fl.op == "call_method" and fl.target == "flatten"))
+        if not (flat and len(fl.users) == 1 and len(fl.args) >= 1 and isinstance(fl.args[0], fx.Node)
+                and (tuple(fl.args[1:]) == (1,) or (len(fl.args) == 1 and dict(fl.kwargs) == {"start_dim": 1}))):
+            continue
+        pl = fl.args[0]
+        pm = mods.get(pl.target) if pl.op == "call_module" else None
+        inner = pm.inner if isinstance(pm, _GlobalAvgPoolNHWC) else pm
+        if not (isinstance(inner, nn.AdaptiveAvgPool2d) and inner.output_size in (1, (1, 1)) and len(pl.users) == 1
+                and len(pl.args) == 1 and not pl.kwargs):
+            continue
+        name = "_fused_" + node.target.replace(".", "_")
+        k = 0
+        while hasattr(gm, name + (str(k) if k else "")):
+            k += 1
+        name += str(k) if k else ""
+        gm.add_submodule(name, _FusedHead(pm, layer))
+        with graph.inserting_before(node):
+            new = graph.call_module(name, (pl.args[0],))
+        node.replace_all_uses_with(new)
+        for n in (node, fl, pl):
             graph.erase_node(n)
         fused += 1
     graph.lint()
