@@ -4,6 +4,7 @@ torch is used only to own device memory and to name the current stream; every co
 through the shared library. There is no CPU or PyTorch fallback: if the library is missing or a
 call fails, an exception is raised.
 """
+import contextlib
 import ctypes
 import os
 
@@ -157,8 +158,24 @@ def ptr(t):
     return None if t is None else ctypes.c_void_p(t.data_ptr())
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_current_device = getattr(torch._C, "_cuda_getDevice", None)
+_STAY = contextlib.nullcontext()
+
+
+def on_device(device):
+    """Context in which `device` (a tensor's .device) is the current one: nothing to do, and nothing to pay, when it
+    already is -- the usual case."""
+    if _current_device is not None and device.index == _current_device():
+        return _STAY
+    return torch.cuda.device(device)
+
+
 def stream_of(t):
-    """The current HIP stream of the tensor's device, as the void* the ABI expects."""
+    """The current HIP stream of the tensor's device, as the void* the ABI expects. (The raw handle where this
+    PyTorch has the accessor: building a torch.cuda.Stream object per call costs ~4 us, more than a small kernel.)"""
+    if _raw_stream is not None:
+        return ctypes.c_void_p(_raw_stream(t.device.index))
     return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
 
 

@@ -34,7 +34,7 @@ def fwd_softstep(weights: torch.Tensor, digamma: float) -> torch.Tensor:
     """Forward mapping for the soft-step function (tmq/tmq_cuda.cu:740-764)."""
     w = _f32_cuda(weights, "fwd_softstep")
     out = torch.empty_like(w)
-    with torch.cuda.device(w.device):
+    with _capi.on_device(w.device):
         check(_lib().tmq_softstep_fwd(ptr(w), ptr(out), w.numel(), float(digamma), stream_of(w)), "fwd_softstep")
     return out.view(weights.shape)
 
@@ -48,7 +48,7 @@ def bwd_softstep(weights: torch.Tensor, digamma: float, scale: float, grad: torc
         raise RuntimeError("bwd_softstep: gradient must match the weights in dtype and size")
     g = grad if grad.is_contiguous() else grad.contiguous()
     out = torch.empty_like(w)
-    with torch.cuda.device(w.device):
+    with _capi.on_device(w.device):
         check(_lib().tmq_softstep_bwd(ptr(w), ptr(g), ptr(out), w.numel(), float(digamma), float(scale),
                                       stream_of(w)), "bwd_softstep")
     return out.view(weights.shape)
@@ -58,7 +58,7 @@ def fwd_softstep_derivative(weights: torch.Tensor, digamma: float, strength: flo
     """Forward mapping for the derivative of the soft-step function (tmq/tmq_cuda.cu:690-709)."""
     w = _f32_cuda(weights, "fwd_softstep_derivative")
     out = torch.empty_like(w)
-    with torch.cuda.device(w.device):
+    with _capi.on_device(w.device):
         check(_lib().tmq_softstep_deriv_fwd(ptr(w), ptr(out), w.numel(), float(digamma), float(strength),
                                             stream_of(w)), "fwd_softstep_derivative")
     return out.view(weights.shape)
@@ -73,7 +73,7 @@ def bwd_softstep_derivative(weights: torch.Tensor, digamma: float, scale: float,
         raise RuntimeError("bwd_softstep_derivative: gradient must match the weights in dtype and size")
     g = grad if grad.is_contiguous() else grad.contiguous()
     out = torch.empty_like(w)
-    with torch.cuda.device(w.device):
+    with _capi.on_device(w.device):
         check(_lib().tmq_softstep_deriv_bwd(ptr(w), ptr(g), ptr(out), w.numel(), float(digamma), float(scale),
                                             stream_of(w)), "bwd_softstep_derivative")
     return out.view(weights.shape)
@@ -85,7 +85,7 @@ def clamp_(weights: torch.Tensor, lo: float, hi: float) -> torch.Tensor:
     _capi.require_gpu(weights, "weights")
     if weights.dtype != torch.float32:
         raise ValueError("clamp_: fp32 only")
-    with torch.cuda.device(weights.device):
+    with _capi.on_device(weights.device):
         check(_lib().tmq_clamp_inplace(ptr(weights), weights.numel(), float(lo), float(hi), stream_of(weights)),
               "clamp_")
     return weights
@@ -97,7 +97,7 @@ def ternarize_(weights: torch.Tensor, digamma: float = 0.0) -> torch.Tensor:
     _capi.require_gpu(weights, "weights")
     if weights.dtype != torch.float32:
         raise ValueError("ternarize_: fp32 only")
-    with torch.cuda.device(weights.device):
+    with _capi.on_device(weights.device):
         check(_lib().tmq_ternarize_inplace(ptr(weights), weights.numel(), float(digamma), stream_of(weights)),
               "ternarize_")
     return weights
@@ -145,7 +145,7 @@ def softstep_fused(weights, grad, digamma, sharpness, strength, gl, lo, hi, *, w
         if grad.numel() != n or grad.dtype != torch.float32:
             raise RuntimeError("softstep_fused: gradient must match the weights")
     if in_launch and loss is not None and n:
-        with torch.cuda.device(w.device):
+        with _capi.on_device(w.device):
             status = lib.tmq_softstep_fused_inlaunch(ptr(w), ptr(grad) if dw is not None else None, ptr(y), ptr(dw), ptr(wc),
                                                      ptr(loss), ptr(loss_state(w.device)), n, float(digamma), float(sharpness),
                                                      float(strength), ctypes.c_float(gl), float(lo), float(hi), stream_of(w))
@@ -154,7 +154,7 @@ def softstep_fused(weights, grad, digamma, sharpness, strength, gl, lo, hi, *, w
             return y, dw, wc, loss
         if ws is None:
             ws = torch.empty(lib.tmq_softstep_fused_workspace_bytes(n), dtype=torch.uint8, device=w.device)
-    with torch.cuda.device(w.device):
+    with _capi.on_device(w.device):
         check(lib.tmq_softstep_fused(ptr(w), ptr(grad) if dw is not None else None, ptr(y), ptr(dw), ptr(wc),
                                      ptr(loss), ptr(ws), n, float(digamma), float(sharpness), float(strength),
                                      ctypes.c_float(gl), float(lo), float(hi), stream_of(w)), "softstep_fused")
@@ -204,7 +204,7 @@ def qloss_multi(table: SegmentTable, sharpness: float, strength: float):
     finalisation launch beyond that form's limits."""
     per = torch.empty(table.nseg, dtype=torch.float32, device=table.device)
     tot = torch.empty(1, dtype=torch.float32, device=table.device)
-    with torch.cuda.device(table.device):
+    with _capi.on_device(table.device):
         # finished inside the launch where the shape allows (up to 64 tensors, 2^18 blocks), else two launches
         status = _lib().tmq_qloss_multi_inlaunch(ptr(table.table), table.nseg, table.total_blocks, float(sharpness),
                                                  float(strength), ptr(per), ptr(tot), ptr(loss_state(table.device)),
@@ -225,7 +225,7 @@ def qloss_bwd_multi(table: SegmentTable, sharpness: float, strength: float, accu
         _capi.require_gpu(upstream, "upstream")
         if upstream.dtype != torch.float32 or upstream.numel() != 1:
             raise RuntimeError("qloss_bwd_multi: upstream must be one fp32 value")
-    with torch.cuda.device(table.device):
+    with _capi.on_device(table.device):
         check(_lib().tmq_qloss_bwd_multi(ptr(table.table), table.nseg, table.total_blocks, float(sharpness),
                                          float(strength), ptr(upstream), int(bool(accumulate)),
                                          stream_of(table.table)), "qloss_bwd_multi")
@@ -278,14 +278,14 @@ def softstep_fwd_all(weights, digamma: float, want_loss: bool = False, sharpness
     if want_loss:
         loss = torch.empty((), dtype=torch.float32, device=dev)
         # the loss finished inside the launch where the shape allows (up to 64 tensors of up to 2^18 blocks)
-        with torch.cuda.device(dev):
+        with _capi.on_device(dev):
             status = lib.tmq_softstep_fwd_multi_inlaunch(arr, len(ws), float(digamma), float(sharpness), float(strength), None,
                                                          ptr(loss), ptr(loss_state(dev)), stream_of(flat))
         if status != _capi.ERR_UNSUPPORTED:
             check(status, "softstep_fwd_all")
             return ys, loss
         wsp = torch.empty(lib.tmq_softstep_multi_workspace_bytes(arr, len(ws)), dtype=torch.uint8, device=dev)
-    with torch.cuda.device(dev):
+    with _capi.on_device(dev):
         check(lib.tmq_softstep_fwd_multi(arr, len(ws), float(digamma), float(sharpness), float(strength), None, ptr(loss),
                                          ptr(wsp), stream_of(flat)), "softstep_fwd_all")
     return ys, loss
@@ -325,7 +325,7 @@ def softstep_bwd_all(weights, grads, loss_upstream, digamma: float, sharpness: f
         arr[k].w, arr[k].g, arr[k].out, arr[k].n = ws[i].data_ptr(), (g.data_ptr() if g is not None else None), \
             dws[k].data_ptr(), ws[i].numel()
         out[i] = dws[k]
-    with torch.cuda.device(dev):
+    with _capi.on_device(dev):
         check(_lib().tmq_softstep_bwd_multi(arr, len(live), float(digamma), float(sharpness), float(strength),
                                             ptr(loss_upstream), stream_of(flat)), "softstep_bwd_all")
     return out
@@ -335,7 +335,7 @@ def softstep_map(weights: torch.Tensor, digamma: float, derivative: bool = False
     """SoftStep.map / SoftStep.dmap (tmq/tmq.py:328-350) on an fp32 GPU tensor."""
     w = _f32_cuda(weights, "softstep_map")
     out = torch.empty_like(w)
-    with torch.cuda.device(w.device):
+    with _capi.on_device(w.device):
         check(_lib().tmq_softstep_map(ptr(w), ptr(out), w.numel(), float(digamma), int(bool(derivative)),
                                       stream_of(w)), "softstep_map")
     return out.view(weights.shape)
@@ -345,14 +345,14 @@ def sigmoid_piece(x: torch.Tensor, order: int) -> torch.Tensor:
     """SoftStep.sigmoid (order 0), dsigmoid (1), d2sigmoid (2) of an fp32 GPU tensor (tmq/tmq.py:353-381)."""
     v = _f32_cuda(x, "sigmoid_piece")
     out = torch.empty_like(v)
-    with torch.cuda.device(v.device):
+    with _capi.on_device(v.device):
         check(_lib().tmq_sigmoid_piece(ptr(v), ptr(out), v.numel(), int(order), stream_of(v)), "sigmoid_piece")
     return out.view(x.shape)
 
 
 def clamp_multi_(table: SegmentTable, lo: float, hi: float):
     """In-place clamp of every segment's weight tensor, one launch."""
-    with torch.cuda.device(table.device):
+    with _capi.on_device(table.device):
         check(_lib().tmq_clamp_multi(ptr(table.table), table.nseg, table.total_blocks, float(lo), float(hi),
                                      stream_of(table.table)), "clamp_multi_")
 
@@ -385,7 +385,7 @@ def compactify_ternary(input: torch.Tensor) -> torch.Tensor:
     Q = (N + 15) // 16
     shape = (src.shape[1], Q) if src.dim() == 2 else (src.shape[1], src.shape[2], src.shape[3], Q)
     out = torch.empty(shape, dtype=torch.int32, device=src.device)
-    with torch.cuda.device(src.device):
+    with _capi.on_device(src.device):
         check(_lib().tmq_pack_ternary(ptr(src), _capi.dtype_code(src), N, K, ptr(out), stream_of(src)),
               "compactify_ternary")
     return out.cpu() if on_cpu else out
@@ -411,7 +411,7 @@ def expand_ternary(input: torch.Tensor, orig_shape, entropy_decode: bool = False
     if src.numel() != K * ((N + 15) // 16):
         raise RuntimeError("expand_ternary: packed tensor does not match the original shape")
     out = torch.empty(orig_shape, dtype=torch.float32, device=src.device)
-    with torch.cuda.device(src.device):
+    with _capi.on_device(src.device):
         check(_lib().tmq_unpack_ternary(ptr(src), N, K, ptr(out), stream_of(src)), "expand_ternary")
     return out.cpu() if on_cpu else out
 
@@ -485,7 +485,7 @@ class NativeWeights:
         self.C, self.ky, self.kx = C, ky, kx
         lib = _lib()
         self.buf = torch.empty(lib.tmq_native_weight_bytes(self.N, self.K), dtype=torch.uint8, device=words.device)
-        with torch.cuda.device(words.device):
+        with _capi.on_device(words.device):
             check(lib.tmq_prepack_weights(ptr(w2), self.N, C, ky, kx, ptr(self.buf), stream_of(w2)), "prepack_weights")
         self.key = (words.data_ptr(), tuple(words.shape), words._version)
 
@@ -568,7 +568,7 @@ def f32_prescale(x: torch.Tensor, scale=None, channels: int = 0, want_copy: bool
         raise RuntimeError("scale must be fp32 with one entry per output channel")
     wsb = lib.tmq_f32_prescale_workspace_bytes(n)
     ws = torch.empty(wsb, dtype=torch.uint8, device=x.device) if wsb else None
-    with torch.cuda.device(x.device):
+    with _capi.on_device(x.device):
         check(lib.tmq_f32_prescale(ptr(x), n, ptr(ps), ptr(xs), ptr(scale), ptr(adj), channels, ptr(ws), stream_of(x)),
               "f32_prescale")
     return ps, xs, adj
@@ -582,7 +582,7 @@ def split_f32(x: torch.Tensor, prescale=None, want_lo: bool = True):
         raise RuntimeError("split_f32: expected fp32")
     hi = torch.empty_like(x, dtype=torch.float16)
     lo = torch.empty_like(x, dtype=torch.float16) if want_lo else None
-    with torch.cuda.device(x.device):
+    with _capi.on_device(x.device):
         check(_lib().tmq_split_f32_scaled(ptr(x), ptr(prescale), ptr(hi), ptr(lo), x.numel(), stream_of(x)), "split_f32")
     return hi, lo
 
@@ -637,7 +637,7 @@ def ternary_linear(x: torch.Tensor, nw: NativeWeights, scale=None, bias=None, re
     lib = _lib()
     # shapes whose reduction pays to be cut across workgroups get a workspace for the partial sums
     wsb = pairs or (lib.tmq_ternary_linear_workspace_bytes(_capi.dtype_code(x), M, nw.K, nw.N) if 16 < M <= 32 else 0)
-    with torch.cuda.device(x.device):
+    with _capi.on_device(x.device):
         if wsb:
             ws = torch.empty(wsb, dtype=torch.uint8, device=x.device)
             check(lib.tmq_ternary_linear_ws(ptr(x), _capi.dtype_code(x), M, nw.K, ptr(nw.buf), nw.N, ctypes.byref(ep), ptr(y),
@@ -674,7 +674,7 @@ def gemv8_prepare(x: torch.Tensor) -> ActivationPlanes:
     if nbytes == 0:
         raise RuntimeError("gemv8_prepare: at most 4 rows of K = 2048 .. 16384 (a multiple of 256), rows x K <= 16384")
     buf = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
-    with torch.cuda.device(x.device):
+    with _capi.on_device(x.device):
         check(lib.tmq_gemv8_prepare(ptr(x), M, K, ptr(buf), stream_of(x)), "gemv8_prepare")
     return ActivationPlanes(buf, M, K, tuple(x.shape[:-1]))
 
@@ -687,7 +687,7 @@ def ternary_linear_planes(planes: ActivationPlanes, nw: NativeWeights, scale=Non
         raise RuntimeError(f"ternary_linear_planes: activations have {planes.K} features, weights expect {nw.K}")
     y = torch.empty(planes.lead + (nw.N,), dtype=out_dtype, device=planes.buf.device)
     ep = _epilogue(nw, scale, bias, residual, relu, out_dtype, y)
-    with torch.cuda.device(y.device):
+    with _capi.on_device(y.device):
         check(_lib().tmq_ternary_linear_planes(ptr(planes.buf), planes.rows, nw.K, ptr(nw.buf), nw.N, ctypes.byref(ep), ptr(y),
                                                stream_of(y)), "ternary_linear_planes")
     return y
@@ -722,7 +722,7 @@ def ternary_conv2d(x: torch.Tensor, nw: NativeWeights, stride=1, padding=0, dila
     ep = _epilogue(nw, scale, bias, residual, relu, out_dtype, y)
     if B == 0:
         return y
-    with torch.cuda.device(x.device):
+    with _capi.on_device(x.device):
         check(lib.tmq_ternary_conv2d(ptr(x), ctypes.byref(shp), ptr(nw.buf), ctypes.byref(ep), ptr(y), stream_of(x)),
               "ternary_conv2d")
     return y
@@ -755,7 +755,7 @@ def ternary_conv2d_into(out: torch.Tensor, x: torch.Tensor, nw: NativeWeights, s
     view = _capi.OutputView(int(first[0]), int(first[1]), int(out.shape[2]), int(out.shape[3]), sb_ // N, sh_ // N, sw_ // N)
     if out.numel() == 0:
         return out
-    with torch.cuda.device(x.device):
+    with _capi.on_device(x.device):
         check(_lib().tmq_ternary_conv2d_view(ptr(x), ctypes.byref(shp), ptr(nw.buf), ctypes.byref(ep), ptr(out),
                                              ctypes.byref(view), stream_of(x)), "ternary_conv2d_view")
     return out
@@ -791,7 +791,7 @@ def ternary_conv2d_relu_maxpool(x: torch.Tensor, nw: NativeWeights, stride=1, pa
     ep = _epilogue(nw, scale, bias, None, True, torch.float16, y)     # validates scale and bias
     if B == 0:
         return y
-    with torch.cuda.device(x.device):
+    with _capi.on_device(x.device):
         status = lib.tmq_ternary_conv2d_relu_maxpool(ptr(x), ctypes.byref(shp), ptr(nw.buf), ep.scale, ep.bias, ptr(y),
                                                      stream_of(x))
     if status == _capi.ERR_UNSUPPORTED:
@@ -833,7 +833,7 @@ def ternary_conv2d_relu_maxpool_planar(x: torch.Tensor, nw: NativeWeights, strid
     ep = _epilogue(nw, scale, bias, None, True, torch.float16, y)     # validates scale and bias
     if B == 0:
         return y
-    with torch.cuda.device(x.device):
+    with _capi.on_device(x.device):
         status = lib.tmq_ternary_conv2d_relu_maxpool_planar(ptr(x), C, ctypes.byref(shp), ptr(nw.buf), ep.scale, ep.bias, ptr(y),
                                                             stream_of(x))
     if status == _capi.ERR_UNSUPPORTED:
@@ -878,7 +878,7 @@ def ternary_dwconv2d(x: torch.Tensor, words: torch.Tensor, kernel, stride=1, pad
     ep = _epilogue(_Channels(C), scale, bias, residual, relu, out_dtype, y)
     if B == 0:
         return y
-    with torch.cuda.device(x.device):
+    with _capi.on_device(x.device):
         check(lib.tmq_ternary_dwconv2d(ptr(x), ctypes.byref(shp), ptr(words), ctypes.byref(ep), ptr(y), stream_of(x)),
               "ternary_dwconv2d")
     return y
@@ -901,7 +901,7 @@ def ternary_dwconv_cuda(input: torch.Tensor, weights: torch.Tensor, kx: int, ky:
     x = input.contiguous()
     P = x.numel() // (taps * channels)
     y = torch.empty(tuple(input.shape[:-1]) + (channels,), dtype=torch.float32, device=x.device)
-    with torch.cuda.device(x.device):
+    with _capi.on_device(x.device):
         check(_lib().tmq_ternary_dwconv_patches(ptr(x), _capi.dtype_code(x), P, taps, channels, ptr(weights.contiguous()),
                                                 ptr(y), stream_of(x)), "ternary_dwconv_cuda")
     return y
@@ -936,7 +936,7 @@ def ternary_dwconvtrans2d(x: torch.Tensor, words: torch.Tensor, kernel, stride=1
     ep = _epilogue(_Channels(C), scale, bias, residual, relu, out_dtype, y)
     if B == 0:
         return y
-    with torch.cuda.device(x.device):
+    with _capi.on_device(x.device):
         check(lib.tmq_ternary_dwconvtrans2d(ptr(x), ctypes.byref(shp), oy, ox, ptr(words), ctypes.byref(ep), ptr(y),
                                             stream_of(x)), "ternary_dwconvtrans2d")
     return y
@@ -964,7 +964,7 @@ def ternary_dwconvtrans_cuda(input: torch.Tensor, weights: torch.Tensor, kx: int
     x = input.contiguous()
     y = torch.empty(tuple(input.shape[:-2]) + (C * taps, P), dtype=torch.float32, device=x.device)
     if y.numel():
-        with torch.cuda.device(x.device):
+        with _capi.on_device(x.device):
             check(_lib().tmq_ternary_dwconvtrans_cols(ptr(x), B, P, taps, C, ptr(weights.contiguous()), ptr(y), stream_of(x)),
                   "ternary_dwconvtrans_cuda")
     return y
@@ -987,7 +987,7 @@ def maxpool2d_nhwc(x: torch.Tensor, kernel, stride=None, padding=0) -> torch.Ten
     y = torch.empty((B, C, ho, wo), dtype=torch.float16, device=x.device, memory_format=torch.channels_last)
     if y.numel() == 0:
         return y
-    with torch.cuda.device(x.device):
+    with _capi.on_device(x.device):
         check(_lib().tmq_maxpool2d_nhwc(ptr(x), B, C, H, W, ky, kx, sy, sx, py, px, ptr(y), stream_of(x)), "maxpool2d_nhwc")
     return y
 
@@ -1002,7 +1002,7 @@ def avgpool_global_nhwc(x: torch.Tensor, out_dtype=torch.float16) -> torch.Tenso
     y = torch.empty((B, C), dtype=out_dtype, device=x.device)
     if y.numel() == 0:
         return y
-    with torch.cuda.device(x.device):
+    with _capi.on_device(x.device):
         check(_lib().tmq_avgpool_global_nhwc(ptr(x), B, H * W, C, ptr(y), _capi.dtype_code(y), stream_of(x)),
               "avgpool_global_nhwc")
     return y
@@ -1022,7 +1022,7 @@ def avgpool_linear(x: torch.Tensor, nw: NativeWeights, scale=None, bias=None, re
     ep = _epilogue(nw, scale, bias, None, relu, out_dtype, y)
     if y.numel() == 0:
         return y
-    with torch.cuda.device(x.device):
+    with _capi.on_device(x.device):
         status = _lib().tmq_avgpool_linear(ptr(x), B, H * W, C, ptr(nw.buf), nw.N, ctypes.byref(ep), ptr(y), stream_of(x))
     if status == _capi.ERR_UNSUPPORTED:
         return ternary_linear(avgpool_global_nhwc(x), nw, scale=scale, bias=bias, relu=relu, out_dtype=out_dtype)
@@ -1042,7 +1042,7 @@ def nchw_to_nhwc4(x: torch.Tensor) -> torch.Tensor:
     y = torch.empty((B, H, W, 4), dtype=torch.float16, device=x.device)
     if y.numel() == 0:
         return y
-    with torch.cuda.device(x.device):
+    with _capi.on_device(x.device):
         check(_lib().tmq_nchw_to_nhwc4(ptr(x), _capi.dtype_code(x), B, C, H, W, ptr(y), stream_of(x)), "nchw_to_nhwc4")
     return y
 
