@@ -362,6 +362,15 @@ int tmq_f32_prescale(const float *x, int64_t n, float *prescale, float *xs, cons
 int tmq_split_f32_scaled(const float *x, const float *prescale, void *hi, void *lo, int64_t n, void *stream);
 int tmq_split_f32(const float *x, void *hi, void *lo, int64_t n, void *stream);
 
+/* tmq_f32_prescale followed by tmq_split_f32_scaled(..., lo = NULL) in two launches whatever the size: the largest
+ * finite |x| (partial maxima in `workspace`, tmq_f32_to_f16_prescaled_workspace_bytes(n) bytes), then hi[i] = fp16(s x[i])
+ * with prescale[0] = s, prescale[1] = 1 / s and, when scale_out is given, scale_out[c] = (scale_in ? scale_in[c] : 1) / s.
+ * What a convolution on fp32 activations needs in front of it (the reference's convolutions take fp32,
+ * tmq/tmq.py:822-871); same values as the two separate calls.                                            */
+size_t tmq_f32_to_f16_prescaled_workspace_bytes(int64_t n);
+int tmq_f32_to_f16_prescaled(const float *x, int64_t n, float *prescale, void *hi, const float *scale_in, float *scale_out,
+                             int64_t channels, void *workspace, void *stream);
+
 /* 1 if M fp32 rows against a K x N layer are faster as two fp16 passes over tmq_split_f32's terms than
  * as one tmq_ternary_linear call with x_dtype TMQ_F32 (many rows, or a few rows over a large
  * layer), else 0. Host-only arithmetic on the shape; no counterpart in the reference.               */

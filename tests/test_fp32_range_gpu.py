@@ -195,3 +195,26 @@ def test_empty_fp32_batches_give_empty_outputs(cuda):
     t.compressed_state_dict(net, strong=False)
     y = net(torch.empty(0, 8, 6, 6, device=cuda))
     assert y.shape[0] == 0 and y.shape[1] == 4 and y.numel() == 0
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape", [(7,), (3, 5, 9, 11), (2, 64, 56, 56), (4, 3, 224, 224), (1, 1, 1, 4099)])
+def test_one_call_conversion_equals_prescale_then_split(cuda, shape):
+    """tmq_f32_to_f16_prescaled (what a convolution on fp32 activations runs in front of it): the same prescale, the
+    same fp16 term and the same adjusted scale as tmq_f32_prescale + tmq_split_f32_scaled, in two launches."""
+    from tmq_amd import ops
+    g = torch.Generator(device=cuda).manual_seed(sum(shape))
+    for mag in (1.0, 3e-20, 7e25):
+        x = torch.randn(shape, device=cuda, generator=g) * mag
+        if len(shape) == 4:
+            x = x.contiguous(memory_format=torch.channels_last)
+        x[(0,) * len(shape)] = float("inf") if mag == 1.0 else 0.0     # non-finite values take no part in the maximum
+        scale = torch.rand(24, device=cuda, generator=g) + 0.5
+        ps, _, adj = ops.f32_prescale(x, scale, 24)
+        want = ops.split_f32(x, ps, want_lo=False)[0]
+        hi, adj2 = ops.f32_to_f16_prescaled(x, scale, 24)
+        assert hi.dtype == torch.float16 and hi.shape == x.shape and hi.stride() == x.stride()
+        assert torch.equal(hi.view(torch.int16), want.view(torch.int16))
+        assert torch.equal(adj2, adj)
+        hi3, adj3 = ops.f32_to_f16_prescaled(x, None, 24)
+        assert torch.equal(hi3.view(torch.int16), want.view(torch.int16)) and torch.equal(adj3, ops.f32_prescale(x, None, 24)[2])

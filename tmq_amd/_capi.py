@@ -78,6 +78,8 @@ SIGNATURES = {
     "tmq_split_f32": (_int, [_vp, _vp, _vp, _i64, _vp]),
     "tmq_split_f32_scaled": (_int, [_vp, _vp, _vp, _vp, _i64, _vp]),
     "tmq_f32_prescale_workspace_bytes": (_sz, [_i64]),
+    "tmq_f32_to_f16_prescaled_workspace_bytes": (_sz, [_i64]),
+    "tmq_f32_to_f16_prescaled": (_int, [_vp, _i64, _vp, _vp, _vp, _vp, _i64, _vp, _vp]),
     "tmq_f32_prescale": (_int, [_vp, _i64, _vp, _vp, _vp, _vp, _i64, _vp, _vp]),
     "tmq_selfcheck_fastdiv": (_i64, [_u32, _vp, _i64]),
     "tmq_fp32_rows_prefer_split": (_int, [_i64, _i64, _i64]),

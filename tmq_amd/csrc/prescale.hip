@@ -205,6 +205,73 @@ __global__ __launch_bounds__(1024) void split_rows_kernel(const float *__restric
     }
 }
 
+// Largest finite |x| of 4096 values per workgroup and round (four 16-byte loads per thread in flight), one partial
+// per workgroup. x 16-byte aligned; the n % 4 values at the end go to workgroup 0.
+__global__ __launch_bounds__(256) void absmax_wide_kernel(const float *__restrict__ x, int64_t n, float *partials) {
+    __shared__ float lds[17];
+    const int64_t n4 = n / 4;
+    float m = 0.f;
+    for (int64_t base = (int64_t)blockIdx.x * 1024; base < n4; base += (int64_t)gridDim.x * 1024) {
+        floatx4 v[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int64_t at = base + i * 256 + threadIdx.x;
+            v[i] = at < n4 ? __builtin_nontemporal_load(reinterpret_cast<const floatx4 *>(x) + at) : floatx4{0.f, 0.f, 0.f, 0.f};
+        }
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            m = fmaxf(fmaxf(m, fmaxf(finite_abs(v[i][0]), finite_abs(v[i][1]))), fmaxf(finite_abs(v[i][2]), finite_abs(v[i][3])));
+    }
+    if (blockIdx.x == 0 && threadIdx.x < (n & 3)) m = fmaxf(m, finite_abs(x[4 * n4 + threadIdx.x]));
+    m = block_max(m, lds);
+    if (threadIdx.x == 0) partials[blockIdx.x] = m;
+}
+
+// hi = fp16(s x) for the whole tensor in the launch after absmax_wide_kernel: every workgroup asks for its 8192 values
+// first, reduces the partial maxima itself while they are on their way (at most 1024 floats), derives s, converts, and
+// writes its slice of the per-channel scale divided by s; workgroup 0 also writes the prescale.
+__global__ __launch_bounds__(256) void convert_prescaled_kernel(const float *__restrict__ x, int64_t n,
+                                                                const float *__restrict__ partials, int count,
+                                                                _Float16 *__restrict__ hi, float *prescale,
+                                                                const float *scale_in, float *scale_out, int64_t channels,
+                                                                int vec) {
+    __shared__ float lds[17];
+    constexpr int kQuads = 8;                                      // float4s per thread
+    const int64_t n4 = n / 4, base = (int64_t)blockIdx.x * (256 * kQuads);
+    floatx4 v[kQuads];
+    if (vec) {
+#pragma unroll
+        for (int i = 0; i < kQuads; i++) {
+            const int64_t at = base + i * 256 + threadIdx.x;
+            v[i] = at < n4 ? __builtin_nontemporal_load(reinterpret_cast<const floatx4 *>(x) + at) : floatx4{0.f, 0.f, 0.f, 0.f};
+        }
+    }
+    float pm = 0.f;
+    for (int i = threadIdx.x; i < count; i += 256) pm = fmaxf(pm, partials[i]);
+    const float amax = block_max(pm, lds);
+    float s, inv;
+    make_prescale(amax, s, inv);
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+        prescale[0] = s;
+        prescale[1] = inv;
+    }
+    if (scale_out)
+        for (int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x; c < channels; c += (int64_t)gridDim.x * 256)
+            scale_out[c] = (scale_in ? scale_in[c] : 1.f) * inv;
+    if (vec) {
+#pragma unroll
+        for (int i = 0; i < kQuads; i++) {
+            const int64_t at = base + i * 256 + threadIdx.x;
+            if (at >= n4) continue;
+            const floatx4 a = v[i] * s;
+            *reinterpret_cast<half4 *>(hi + 4 * at) = half4{(_Float16)a[0], (_Float16)a[1], (_Float16)a[2], (_Float16)a[3]};
+        }
+        if (blockIdx.x == 0 && threadIdx.x < (n & 3)) hi[4 * n4 + threadIdx.x] = (_Float16)(x[4 * n4 + threadIdx.x] * s);
+    } else {
+        for (int64_t i = base * 4 + threadIdx.x; i < n && i < (base + 256 * kQuads) * 4; i += 256) hi[i] = (_Float16)(x[i] * s);
+    }
+}
+
 // Many fp32 rows as fp16 row pairs in groups of eight, every group under a power of two s of its own: a workgroup
 // of 1024 takes the group's 8 K values -- float4 number 1024 i + t to thread t, up to NQ of them in
 // registers and all asked for at once (a single trip to memory; longer rows are read a second time) -- finds the
@@ -335,6 +402,30 @@ int tmq_split_f32_scaled(const float *x, const float *prescale, void *hi, void *
                      : (prescale ? split_terms_kernel<false, true> : split_terms_kernel<false, false>);
     hipLaunchKernelGGL(kernel, dim3((uint32_t)blocks), dim3(256), 0, as_stream(stream), x, prescale,
                        static_cast<_Float16 *>(hi), static_cast<_Float16 *>(lo), n, vec);
+    return check_launch();
+}
+
+size_t tmq_f32_to_f16_prescaled_workspace_bytes(int64_t n) { return n > 0 ? kPartials * sizeof(float) : 0; }
+
+int tmq_f32_to_f16_prescaled(const float *x, int64_t n, float *prescale, void *hi, const float *scale_in, float *scale_out,
+                             int64_t channels, void *workspace, void *stream) {
+    if (n <= 0 || !x || !prescale || !hi || !workspace || channels < 0 || (scale_out && channels == 0)) return TMQ_ERR_INVALID_ARG;
+    float *partials = static_cast<float *>(workspace);
+    const int vec = aligned16(x) && (reinterpret_cast<uintptr_t>(hi) & 7u) == 0;
+    int64_t blocks = (n + 4095) / 4096;                    // 16 values per thread and round
+    if (blocks > kPartials) blocks = kPartials;
+    if (vec) {
+        hipLaunchKernelGGL(absmax_wide_kernel, dim3((uint32_t)blocks), dim3(256), 0, as_stream(stream), x, n, partials);
+    } else {
+        blocks = (n + 8191) / 8192;
+        if (blocks > kPartials) blocks = kPartials;
+        hipLaunchKernelGGL(absmax_partial_kernel, dim3((uint32_t)blocks), dim3(256), 0, as_stream(stream), x, n, partials, 0);
+    }
+    if (int rc = check_launch()) return rc;
+    const int64_t groups = (n + 8191) / 8192;
+    if (groups > 0x7FFFFFFF) return TMQ_ERR_TOO_LARGE;
+    hipLaunchKernelGGL(convert_prescaled_kernel, dim3((uint32_t)groups), dim3(256), 0, as_stream(stream), x, n, partials, (int)blocks,
+                       static_cast<_Float16 *>(hi), prescale, scale_in, scale_out, channels, vec);
     return check_launch();
 }
 

@@ -595,8 +595,19 @@ def f32_to_f16_prescaled(x: torch.Tensor, scale, channels: int):
         return x.to(torch.float16), scale
     if not (x.is_contiguous() or x.is_contiguous(memory_format=torch.channels_last)):
         x = x.contiguous()
-    ps, _, adj = f32_prescale(x, scale, channels)
-    return split_f32(x, ps, want_lo=False)[0], adj
+    _capi.require_gpu_dense(x, "activations")
+    if scale is not None and (scale.dtype != torch.float32 or scale.numel() != channels or not scale.is_cuda):
+        raise RuntimeError("scale must be fp32 with one entry per output channel")
+    lib = _lib()
+    n = x.numel()
+    ps = torch.empty(2, dtype=torch.float32, device=x.device)
+    hi = torch.empty_like(x, dtype=torch.float16)
+    adj = torch.empty(channels, dtype=torch.float32, device=x.device) if channels else None
+    ws = torch.empty(lib.tmq_f32_to_f16_prescaled_workspace_bytes(n), dtype=torch.uint8, device=x.device)
+    with _capi.on_device(x.device):
+        check(lib.tmq_f32_to_f16_prescaled(ptr(x), n, ptr(ps), ptr(hi), ptr(scale), ptr(adj), channels, ptr(ws), stream_of(x)),
+              "f32_to_f16_prescaled")
+    return hi, (adj if channels else scale)
 
 
 def ternary_linear(x: torch.Tensor, nw: NativeWeights, scale=None, bias=None, residual=None, relu=False,
