@@ -222,6 +222,46 @@ def test_wide_layers(cuda, oracle, K):
             assert torch.equal(ops.ternary_linear_planes(ops.gemv8_prepare(x), nw, scale, bias), y)
 
 
+@pytest.mark.parametrize("K", [8448, 11008, 12288, 16384])
+def test_two_long_rows_against_wide_layers(cuda, oracle, K):
+    """Two fp16 rows of more than 8192 indices against 16384 channels or more: eight planes on the sixteen-wavefront
+    workgroups. Rows of different magnitude stay apart, every row equals its own single-row launch bit for bit, every
+    finite fp16 value passes an identity layer, and a narrower layer (the weight-stream kernel) agrees."""
+    from tmq_amd import ops
+    N = 16400
+    rng = np.random.default_rng(K + 2)
+    W = torch.from_numpy(rng.integers(-1, 2, size=(N, K), dtype=np.int8))
+    nw = ops.NativeWeights(torch.from_numpy(oracle.pack(W.numpy().astype(np.float32)).view(np.int32)).to(cuda), N)
+    Wd = W.to(cuda).double()
+    x = rng.standard_normal((2, K)).astype(np.float16)
+    x[1] *= np.float16(37.0)
+    x = torch.from_numpy(x).to(cuda)
+    scale = torch.from_numpy((0.5 + rng.random(N)).astype(np.float32)).to(cuda)
+    bias = torch.from_numpy(rng.standard_normal(N).astype(np.float32)).to(cuda)
+    y = ops.ternary_linear(x, nw, scale, bias)
+    ref = (x.double() @ Wd.t()) * scale.double() + bias.double()
+    for m in range(2):
+        err = ((y[m].double() - ref[m]).abs().max() / ref[m].abs().max()).item()
+        assert err <= 1e-5, (K, m, err)
+        assert torch.equal(ops.ternary_linear(x[m:m + 1], nw, scale, bias)[0], y[m]), (K, m)
+    res = torch.from_numpy(rng.standard_normal((2, N)).astype(np.float16)).to(cuda)
+    y2 = ops.ternary_linear(x, nw, scale, bias, residual=res, relu=True, out_dtype=torch.float16)
+    ref2 = torch.clamp_min(ref + res.double(), 0)
+    assert ((y2.double() - ref2).abs().max() / ref2.abs().max()).item() <= 1e-3
+    narrow = ops.NativeWeights(torch.from_numpy(oracle.pack(W[:4100].numpy().astype(np.float32)).view(np.int32)).to(cuda), 4100)
+    yn = ops.ternary_linear(x, narrow, scale[:4100], bias[:4100])
+    assert ((yn.double() - y[:, :4100].double()).abs().max() / ref.abs().max()).item() <= 1e-5
+    if K == 16384:
+        vals = np.arange(65536, dtype=np.uint32).astype(np.uint16).view(np.float16).copy()
+        vals[~np.isfinite(vals)] = 0
+        vals = vals[np.random.default_rng(8).permutation(65536)]
+        eye = ops.NativeWeights(torch.from_numpy(oracle.pack(np.eye(K, dtype=np.float32)).view(np.int32)).to(cuda), K)
+        for c in (0, 2):
+            xv = vals[c * K:(c + 2) * K].reshape(2, K)
+            yv = ops.ternary_linear(torch.from_numpy(xv).to(cuda), eye)
+            assert np.array_equal(yv.cpu().numpy(), xv.astype(np.float32)), c
+
+
 @pytest.mark.parametrize("K", [2048, 16384])
 def test_fp32_row_passes_22_bit_values_through_exactly(cuda, oracle, K):
     """Identity weights: integers of up to 22 bits (and their power-of-two multiples, small and large) come back

@@ -429,6 +429,19 @@ int launch_gemv8_by_blocks(const void *x, int64_t Kb, const void *native, int64_
             case 7: return launch_gemv8<16, 2, 7, 2, true, 1, false>(x, native, Kb, N, ep, stream);
             default: return launch_gemv8<16, 2, 8, 2, true, 1, false>(x, native, Kb, N, ep, stream);
         }
+    } else if constexpr (MR == 2 && !PRE) {
+        // Two fp16 rows of 8193 .. 16384 indices: eight planes, the shape of an fp32 row's
+        if (Kb > 64 || native_blocks_n(N) < 1024) return TMQ_ERR_UNSUPPORTED;
+        switch ((Kb + 3) / 4) {
+            case 9: return launch_gemv8<16, 4, 9, 2, false, 2, false>(x, native, Kb, N, ep, stream);
+            case 10: return launch_gemv8<16, 4, 10, 2, false, 2, false>(x, native, Kb, N, ep, stream);
+            case 11: return launch_gemv8<16, 4, 11, 2, false, 2, false>(x, native, Kb, N, ep, stream);
+            case 12: return launch_gemv8<16, 4, 12, 2, false, 2, false>(x, native, Kb, N, ep, stream);
+            case 13: return launch_gemv8<16, 4, 13, 2, false, 2, false>(x, native, Kb, N, ep, stream);
+            case 14: return launch_gemv8<16, 4, 14, 2, false, 2, false>(x, native, Kb, N, ep, stream);
+            case 15: return launch_gemv8<16, 4, 15, 2, false, 2, false>(x, native, Kb, N, ep, stream);
+            default: return launch_gemv8<16, 4, 16, 2, false, 2, false>(x, native, Kb, N, ep, stream);
+        }
     } else if constexpr (MR > 1 && !PRE) {
         return TMQ_ERR_UNSUPPORTED;                              // the planes of such rows stop at 8192 indices
     } else {
@@ -460,9 +473,13 @@ int launch_gemv8_by_blocks(const void *x, int64_t Kb, const void *native, int64_
 // True when the 8-bit GEMV can take a dense fp16 problem: one row up to K = 16384; two rows up to 4096 and three
 // or four at 2048 -- every workgroup prepares the planes of all rows, and beyond 8192 values that preparation costs
 // more than the weight-stream kernel's fp16 expansion (measured: two rows at 4096^2 3.9 -> 3.6 us, four rows
-// 4.0 -> 4.9 us; two rows at 8192^2 6.2 -> 7.0 us).
-bool gemv8_dense_ok(const void *x, int64_t M, int64_t K) {
+// 4.0 -> 4.9 us; two rows at 8192^2 6.9 -> 7.1 us, at 8192 x 28672 15.5 -> 17.7 us). Two rows of more than 8192
+// indices against 16384 or more channels are the exception: their eight planes fill the LDS like one fp32 row's, the
+// sixteen-wavefront workgroups of that row take them, and the weight-stream kernel is the slower one there
+// (16384^2: 17.9 -> 15.5 us, 12288 x 16384: 13.8 -> 11.9 us; 11008 x 4096, on eight wavefronts: 6.2 -> 7.6 us, refused).
+bool gemv8_dense_ok(const void *x, int64_t M, int64_t K, int64_t N) {
     if (M < 1 || M > 4 || K % kKB != 0 || K < 8 * kKB || !aligned16(x)) return false;
+    if (M == 2 && K > 32 * kKB) return K <= 64 * kKB && native_blocks_n(N) >= 1024;
     return M == 1 ? K <= 64 * kKB : K * (M == 3 ? 4 : M) <= 32 * kKB;
 }
 

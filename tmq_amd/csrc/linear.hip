@@ -29,7 +29,7 @@ int launch_stream_dense(const void *x, int64_t M, int64_t K, const void *native,
 int launch_mid_dense(const void *x, int64_t M, int64_t K, const void *native, int64_t N, const float *scale,
                      const float *bias, const void *residual, int relu, void *y, int y_f16, void *stream);
 // gemv8.hip: one fp16 row on the 8-bit matrix instructions
-bool gemv8_dense_ok(const void *x, int64_t M, int64_t K);
+bool gemv8_dense_ok(const void *x, int64_t M, int64_t K, int64_t N);
 int launch_gemv8_dense(const void *x, int64_t M, int64_t K, const void *native, int64_t N, const float *scale, const float *bias,
                        const void *residual, int relu, void *y, int y_f16, void *stream);
 bool gemv8_planes_ok(int64_t M, int64_t K);
@@ -1147,10 +1147,11 @@ int tmq_ternary_linear(const void *x, int x_dtype, int64_t M, int64_t K, const v
     if (epilogue) ep = *epilogue;
     if (ep.y_dtype != TMQ_F16 && ep.y_dtype != TMQ_F32) return TMQ_ERR_UNSUPPORTED;
     const bool x32 = x_dtype == TMQ_F32;
-    // One fp16 row, K a multiple of 256 from 2048 to 16384 (two rows to 8192, three or four to 4096): weights and
+    // One fp16 row, K a multiple of 256 from 2048 to 16384 (two rows to 4096, or beyond 8192 against 16384 channels
+    // or more; three or four rows to 2048): weights and
     // activations as 8-bit MFMA operands (gemv8.hip), half the decode work per weight of the kernels below (4096^2:
     // 3.75 -> 3.0 us, 16384^2: 17.7 -> 15.6 us).
-    if (!x32 && gemv8_dense_ok(x, M, K))
+    if (!x32 && gemv8_dense_ok(x, M, K, N))
         return launch_gemv8_dense(x, M, K, native, N, ep.scale, ep.bias, ep.residual, ep.relu, y, ep.y_dtype == TMQ_F16, stream);
     // ... and one fp32 row (the reference's GEMV convention) up to K = 8192: the same kernel on the row's two fp16 halves
     if (x32 && gemv8_dense32_ok(x, M, K))
