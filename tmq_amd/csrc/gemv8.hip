@@ -25,7 +25,7 @@
 // wavefronts meet in LDS in wavefront order (deterministic). Measured (HIP-graph replays over rotating weight
 // buffers): K = N = 4096 3.0 us (fp16 weight-stream kernel 3.75), 8192^2 5.5 us, 16384^2 15.6 us (17.7).
 //
-// Requires M == 1, K a multiple of 256 from 2048 to 16384 (fp32 activations, carried as two fp16 halves: to 8192),
+// Requires M == 1, K a multiple of 256 from 2048 to 16384 (fp32 activations, carried as two fp16 halves, too),
 // 16-byte aligned x.
 //
 // Two to four rows (MR = 2, 4; three rows run as four with one of zeros) take the same kernel: row m's four

@@ -1153,7 +1153,7 @@ int tmq_ternary_linear(const void *x, int x_dtype, int64_t M, int64_t K, const v
     // 3.75 -> 3.0 us, 16384^2: 17.7 -> 15.6 us).
     if (!x32 && gemv8_dense_ok(x, M, K, N))
         return launch_gemv8_dense(x, M, K, native, N, ep.scale, ep.bias, ep.residual, ep.relu, y, ep.y_dtype == TMQ_F16, stream);
-    // ... and one fp32 row (the reference's GEMV convention) up to K = 8192: the same kernel on the row's two fp16 halves
+    // ... and one fp32 row (the reference's GEMV convention) up to K = 16384: the same kernel on the row's two fp16 halves
     if (x32 && gemv8_dense32_ok(x, M, K))
         return launch_gemv8_dense32(x, K, native, N, ep.scale, ep.bias, ep.residual, ep.relu, y, ep.y_dtype == TMQ_F16, stream);
     // At most 16 fp16 rows against eight or more weight blocks per channel: the weight-stream kernel (mid.hip).
