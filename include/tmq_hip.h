@@ -284,8 +284,9 @@ typedef struct tmq_epilogue {
  * exponent range: max|x| at most 65504, and values below ~6e-5 lose precision. Tensors of any other
  * magnitude go through tmq_f32_prescale first (exact power-of-two scaling, undone in the per-channel scale of
  * the epilogue); the Python / PyTorch bindings of this library always do, because the reference multiplies
- * fp32 activations in fp32 and has no such limit. One case needs no prescale: a single fp32 row for which
- * tmq_fp32_rows_self_scaled returns 1 is scaled inside the kernel and may have any magnitude.
+ * fp32 activations in fp32 and has no such limit. One case needs no prescale: fp32 rows for which
+ * tmq_fp32_rows_self_scaled_for returns 1 (one row, or two over a small layer) are scaled inside the kernel, each by
+ * its own power of two, and may have any magnitude.
  * Arithmetic: exact products, fp32 accumulation. One fp16 row (M == 1) with K a multiple of 256 from 2048 to 16384
  * runs on the 8-bit matrix instructions (weights as fp8, the row as four exact bf8 terms); there the hardware adds
  * 32 products at a time aligned to the largest of them, so the result can differ from an fp32 running sum by a few
@@ -302,7 +303,8 @@ int tmq_ternary_linear(const void *x, int x_dtype, int64_t M, int64_t K, const v
  * workgroups -- today 17 .. 32 fp16 rows over 2^28 weights or more -- runs as slices of whole 256-index weight
  * blocks with fp32 partial sums in the workspace, added in slice order by a second launch (deterministic, no
  * atomics). Two to sixteen fp32 rows with K a multiple of 256 from 2048 (the reference's kernels take fp32 activations,
- * tmq/tmq_cuda.cu:242-427) use the workspace differently: a first launch splits every row into two fp16 rows
+ * tmq/tmq_cuda.cu:242-427; two rows with K, N <= 6144 excepted: tmq_ternary_linear takes them in one launch) use the
+ * workspace differently: a first launch splits every row into two fp16 rows
  * (hi = fp16(s x), lo = fp16(s x - hi), s the row's own power of two: any magnitude, 22 significant bits), the fp16
  * weight-stream kernel then runs once over twice the rows (from nine rows: twice, over about half of them each)
  * and adds each pair in its epilogue (256 + 4 M K bytes). Seventeen fp32 rows or more with K a multiple of 64 from
@@ -336,6 +338,9 @@ int tmq_ternary_linear_planes(const void *planes, int64_t M, int64_t K, const vo
  * 16-byte aligned row, K a multiple of 256 from 2048 to 16384: the kernel finds the row's largest finite |x| and scales
  * by a power of two itself), 0 when the caller has to keep them inside fp16's range (tmq_f32_prescale). */
 int tmq_fp32_rows_self_scaled(const void *x, int64_t M, int64_t K);
+/* The same question for a layer of N channels: also 1 for two 16-byte aligned rows with K a multiple of 256 from
+ * 2048 to 6144 and N <= 6144 (each row scaled by its own power of two inside the one launch). */
+int tmq_fp32_rows_self_scaled_for(const void *x, int64_t M, int64_t K, int64_t N);
 
 /* Range handling for fp32 activations (no counterpart in the reference, whose kernels multiply fp32
  * activations in fp32, tmq/tmq_cuda.cu:242-427). Scans n fp32 values and writes prescale[0] = s,

@@ -37,7 +37,8 @@ def test_rows_against_fp64(cuda, oracle, M, K, N):
     print("fp32 row pairs", M, K, N, flush=True)
     rng = np.random.default_rng(M * 100000 + K + N)
     W, nw = _layer(cuda, oracle, rng, N, K)
-    assert _capi.load().tmq_ternary_linear_workspace_bytes(_capi.F32, M, K, N) == 256 + 4 * M * K
+    one_launch = M == 2 and K <= 6144 and N <= 6144              # two rows over a small layer: the 8-bit GEMV splits them itself
+    assert _capi.load().tmq_ternary_linear_workspace_bytes(_capi.F32, M, K, N) == (0 if one_launch else 256 + 4 * M * K)
     x = rng.standard_normal((M, K)).astype(np.float32)
     ref = x.astype(np.float64) @ W.astype(np.float64).T
     t = lambda a: torch.from_numpy(a).to(cuda)
@@ -76,6 +77,44 @@ def test_rows_of_any_magnitude_side_by_side(cuda, oracle):
     assert np.all(np.isfinite(y))
     assert _row_err(y[:5], ref[:5]) <= 1e-5
     assert np.array_equal(y[5], np.zeros(N, np.float32))
+
+
+@pytest.mark.parametrize("K", [2048, 2304, 4096, 5120, 6144])
+def test_two_rows_over_small_layers_in_one_launch(cuda, oracle, K):
+    """Two fp32 rows, K <= 6144, N <= 6144: sixteen term planes in the 8-bit GEMV, each row scaled by its own power of
+    two inside the launch. Rows 60 orders of magnitude apart, a row of zeros, the C ABI without any workspace, and the
+    neighbouring shape (N = 6160: fp16 row pairs) agree."""
+    from tmq_amd import ops, _capi
+    lib = _capi.load()
+    rng = np.random.default_rng(K)
+    for N in (16, 1000, 4100, 6144):
+        W, nw = _layer(cuda, oracle, rng, N, K)
+        x = rng.standard_normal((2, K)).astype(np.float32)
+        x[0] *= np.float32(1e-30)
+        x[1] *= np.float32(1e30)
+        tx = torch.from_numpy(x).to(cuda)
+        assert lib.tmq_fp32_rows_self_scaled_for(ops.ptr(tx), 2, K, N) == 1
+        assert lib.tmq_fp32_rows_self_scaled(ops.ptr(tx), 2, K) == 0
+        ref = x.astype(np.float64) @ W.astype(np.float64).T
+        y = ops.ternary_linear(tx, nw)
+        assert np.all(np.isfinite(y.cpu().numpy()))
+        assert _row_err(y.cpu().numpy(), ref) <= 1e-5, (K, N)
+        for m in range(2):                                       # each row is the single-row launch of that row
+            assert torch.equal(ops.ternary_linear(tx[m:m + 1], nw)[0], y[m]), (K, N, m)
+        ep = _capi.Epilogue(None, None, None, 0, _capi.F32)
+        y2 = torch.empty_like(y)
+        assert lib.tmq_ternary_linear(ops.ptr(tx), _capi.F32, 2, K, ops.ptr(nw.buf), N, ctypes.byref(ep), ops.ptr(y2), None) == 0
+        torch.cuda.synchronize()
+        assert torch.equal(y2, y)
+        x[0] = 0.0
+        y0 = ops.ternary_linear(torch.from_numpy(x).to(cuda), nw).cpu().numpy()
+        assert np.array_equal(y0[0], np.zeros(N, np.float32)) and np.array_equal(y0[1], y[1].cpu().numpy())
+    W, nw = _layer(cuda, oracle, rng, 6160, K)
+    x = torch.from_numpy(rng.standard_normal((2, K)).astype(np.float32)).to(cuda)
+    assert lib.tmq_fp32_rows_self_scaled_for(ops.ptr(x), 2, K, 6160) == 0
+    small = ops.NativeWeights(torch.from_numpy(oracle.pack(W[:6144]).view(np.int32)).to(cuda), 6144)
+    ya, yb = ops.ternary_linear(x, nw)[:, :6144], ops.ternary_linear(x, small)
+    assert ((ya - yb).abs().max() / ya.abs().max()).item() <= 1e-5
 
 
 @pytest.mark.parametrize("M", [2, 5, 8, 13])

@@ -84,6 +84,7 @@ SIGNATURES = {
     "tmq_selfcheck_fastdiv": (_i64, [_u32, _vp, _i64]),
     "tmq_fp32_rows_prefer_split": (_int, [_i64, _i64, _i64]),
     "tmq_fp32_rows_self_scaled": (_int, [_vp, _i64, _i64]),
+    "tmq_fp32_rows_self_scaled_for": (_int, [_vp, _i64, _i64, _i64]),
     "tmq_multi_plan": (_int, [ctypes.POINTER(Segment), _int, ctypes.POINTER(_u32)]),
     "tmq_qloss_multi_workspace_bytes": (_sz, [_u32]),
     "tmq_qloss_multi": (_int, [_vp, _int, _u32, _dbl, _dbl, _vp, _vp, _vp, _vp]),

@@ -1113,7 +1113,9 @@ int launch_split_rows(const float *x, int64_t M, int64_t K, int64_t group, void 
 int launch_stream_pairs(const void *x16, int64_t M, int64_t K, const void *native, int64_t N, const float *row_scale,
                         const float *scale, const float *bias, const void *residual, int relu, void *y, int y_f16,
                         void *stream);
-inline bool row_pairs_ok(const void *x, int64_t M, int64_t K) {
+bool gemv8_dense32_ok(const void *x, int64_t M, int64_t K, int64_t N);
+inline bool row_pairs_ok(const void *x, int64_t M, int64_t K, int64_t N) {
+    if (gemv8_dense32_ok(x, M, K, N)) return false;               // two rows over a small layer: one launch (gemv8.hip)
     return M >= 2 && M <= 16 && K % kKB == 0 && K >= 8 * kKB && aligned16(x) && 2 * M * K < (int64_t)0x7FFFFFFF;
 }
 inline size_t row_pairs_bytes(int64_t M, int64_t K) { return 256 + (size_t)(2 * M * K) * sizeof(_Float16); }
@@ -1179,7 +1181,7 @@ extern "C" {
 size_t tmq_ternary_linear_workspace_bytes(int x_dtype, int64_t M, int64_t K, int64_t N) {
     if (M <= 0 || K <= 0 || N <= 0) return 0;
     if (x_dtype == TMQ_F32)
-        return row_pairs_ok(nullptr, M, K) ? row_pairs_bytes(M, K) : pair_rows_ok(nullptr, M, K, N) ? pair_rows_bytes(M, K, N) : 0;
+        return row_pairs_ok(nullptr, M, K, N) ? row_pairs_bytes(M, K) : pair_rows_ok(nullptr, M, K, N) ? pair_rows_bytes(M, K, N) : 0;
     if (x_dtype != TMQ_F16) return 0;
     static const _Float16 *const aligned = nullptr;              // the plan assumes 16-byte aligned rows; _ws checks the real pointer
     const int slices = rows_split_slices(aligned, M, K, N);
@@ -1189,7 +1191,7 @@ size_t tmq_ternary_linear_workspace_bytes(int x_dtype, int64_t M, int64_t K, int
 int tmq_ternary_linear_ws(const void *x, int x_dtype, int64_t M, int64_t K, const void *native, int64_t N,
                           const tmq_epilogue *epilogue, void *y, void *workspace, size_t workspace_bytes, void *stream) {
     if (x && native && y && x_dtype == TMQ_F32 && N > 0 && workspace && aligned16(workspace) && aligned16(native) &&
-        row_pairs_ok(x, M, K) && workspace_bytes >= row_pairs_bytes(M, K)) {
+        row_pairs_ok(x, M, K, N) && workspace_bytes >= row_pairs_bytes(M, K)) {
         tmq_epilogue e = {nullptr, nullptr, nullptr, 0, TMQ_F32};
         if (epilogue) e = *epilogue;
         if (e.y_dtype != TMQ_F16 && e.y_dtype != TMQ_F32) return TMQ_ERR_UNSUPPORTED;
@@ -1212,7 +1214,7 @@ int tmq_ternary_linear_ws(const void *x, int x_dtype, int64_t M, int64_t K, cons
         return TMQ_OK;
     }
     if (x && native && y && x_dtype == TMQ_F32 && N > 0 && workspace && aligned16(workspace) && aligned16(native) &&
-        !row_pairs_ok(x, M, K) && pair_rows_ok(x, M, K, N) && workspace_bytes >= pair_rows_bytes(M, K, N)) {
+        !row_pairs_ok(x, M, K, N) && pair_rows_ok(x, M, K, N) && workspace_bytes >= pair_rows_bytes(M, K, N)) {
         tmq_epilogue e = {nullptr, nullptr, nullptr, 0, TMQ_F32};
         if (epilogue) e = *epilogue;
         if (e.y_dtype != TMQ_F16 && e.y_dtype != TMQ_F32) return TMQ_ERR_UNSUPPORTED;

@@ -97,9 +97,9 @@ constexpr int vmcnt_only(int n) { return (n & 15) | ((n >> 4) << 14) | 0x0F70; }
 template <int WAVES, int CB, int NT, int ORDER, bool X32, int MR, bool PRE>
 __global__ __launch_bounds__(64 * WAVES) void gemv8_kernel(const void *__restrict__ xv, const u32x4 *__restrict__ native,
                                                            int Kb, int64_t N, int64_t Nb, Gemv8Epilogue ep) {
-    static_assert(!X32 || (MR == 1 && !PRE), "fp32 rows: one row, split in the kernel");
+    static_assert(!X32 || (MR <= 2 && !PRE), "fp32 rows: one or two, split in the kernel");
     constexpr int KS = WAVES / CB, kUnits = (KS * NT + 2 * WAVES - 1) / (2 * WAVES);   // units of 8 values per thread and row: ceil(32 Kb / threads)
-    constexpr int NP = X32 ? 8 : 4 * MR;                         // term planes
+    constexpr int NP = (X32 ? 8 : 4) * MR;                       // term planes
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const int K = Kb * kKB;
     const int plane = K + 32;                                    // bytes per term plane; +32 puts the planes on different banks
@@ -133,8 +133,9 @@ __global__ __launch_bounds__(64 * WAVES) void gemv8_kernel(const void *__restric
                 qa[m][i] = qb[m][i] = Quad{};
                 if (u < K / 8 && m < ep.rows) {
                     if constexpr (X32) {
-                        qa[m][i] = *reinterpret_cast<const u32x4 *>(static_cast<const float *>(xv) + k0);
-                        qb[m][i] = *reinterpret_cast<const u32x4 *>(static_cast<const float *>(xv) + k0 + 32);
+                        const float *row = static_cast<const float *>(xv) + (size_t)m * K;
+                        qa[m][i] = *reinterpret_cast<const u32x4 *>(row + k0);
+                        qb[m][i] = *reinterpret_cast<const u32x4 *>(row + k0 + 32);
                     } else {
                         const _Float16 *row = static_cast<const _Float16 *>(xv) + (size_t)m * K;
                         qa[m][i] = *reinterpret_cast<const u32x2 *>(row + k0);
@@ -195,31 +196,40 @@ __global__ __launch_bounds__(64 * WAVES) void gemv8_kernel(const void *__restric
     // fp32 rows of any magnitude: the row times the power of two that brings its largest finite |x| into
     // [1024, 2048) (exact), undone in the epilogue -- the hi / lo halves then sit well inside fp16's range. Every
     // workgroup holds the whole row, so the maximum is one reduction through LDS.
-    float ps = 1.f, ps_inv = 1.f;
+    float ps[MR], ps_inv[MR];
+#pragma unroll
+    for (int m = 0; m < MR; m++) ps[m] = ps_inv[m] = 1.f;
     if constexpr (X32) {
-        float amax = 0.f;
+        float amax[MR];
 #pragma unroll
-        for (int i = 0; i < kUnits; i++)
+        for (int m = 0; m < MR; m++) {
+            amax[m] = 0.f;
 #pragma unroll
-            for (int e = 0; e < 4; e++) {
-                const float a = __builtin_fabsf(__builtin_bit_cast(float, qa[0][i][e])), b = __builtin_fabsf(__builtin_bit_cast(float, qb[0][i][e]));
-                amax = fmaxf(amax, a < INFINITY ? a : 0.f);      // NaN and Inf take no part (they propagate anyway)
-                amax = fmaxf(amax, b < INFINITY ? b : 0.f);
-            }
+            for (int i = 0; i < kUnits; i++)
 #pragma unroll
-        for (int off = 32; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
-        if (lane == 0) red[wv] = amax;
+                for (int e = 0; e < 4; e++) {
+                    const float a = __builtin_fabsf(__builtin_bit_cast(float, qa[m][i][e])), b = __builtin_fabsf(__builtin_bit_cast(float, qb[m][i][e]));
+                    amax[m] = fmaxf(amax[m], a < INFINITY ? a : 0.f);   // NaN and Inf take no part (they propagate anyway)
+                    amax[m] = fmaxf(amax[m], b < INFINITY ? b : 0.f);
+                }
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) amax[m] = fmaxf(amax[m], __shfl_xor(amax[m], off, 64));
+            if (lane == 0) red[wv * MR + m] = amax[m];
+        }
         __builtin_amdgcn_s_waitcnt(0xC07F);                      // lgkmcnt(0)
         __builtin_amdgcn_s_barrier();
 #pragma unroll
-        for (int q = 0; q < WAVES; q++) amax = fmaxf(amax, red[q]);
-        if (amax > 0.f) {
-            int e;
-            (void)frexpf(amax, &e);                              // amax in [2^(e-1), 2^e)
-            int p = 11 - e;
-            p = p > 126 ? 126 : (p < -126 ? -126 : p);
-            ps = ldexpf(1.f, p);
-            ps_inv = ldexpf(1.f, -p);
+        for (int m = 0; m < MR; m++) {
+#pragma unroll
+            for (int q = 0; q < WAVES; q++) amax[m] = fmaxf(amax[m], red[q * MR + m]);
+            if (amax[m] > 0.f) {                                 // every row its own power of two
+                int e;
+                (void)frexpf(amax[m], &e);                       // amax in [2^(e-1), 2^e)
+                int p = 11 - e;
+                p = p > 126 ? 126 : (p < -126 ? -126 : p);
+                ps[m] = ldexpf(1.f, p);
+                ps_inv[m] = ldexpf(1.f, -p);
+            }
         }
         // (the partial sums below reuse red[] only after the next barrier)
     }
@@ -250,15 +260,15 @@ __global__ __launch_bounds__(64 * WAVES) void gemv8_kernel(const void *__restric
                         uint32_t hi[4], lo[4];                   // pairs (0, 1), (2, 3) of quad A, then of quad B
 #pragma unroll
                         for (int p = 0; p < 4; p++) {
-                            const float v0 = ps * __builtin_bit_cast(float, p < 2 ? qa[0][i][2 * p] : qb[0][i][2 * p - 4]);
-                            const float v1 = ps * __builtin_bit_cast(float, p < 2 ? qa[0][i][2 * p + 1] : qb[0][i][2 * p - 3]);
+                            const float v0 = ps[m] * __builtin_bit_cast(float, p < 2 ? qa[m][i][2 * p] : qb[m][i][2 * p - 4]);
+                            const float v1 = ps[m] * __builtin_bit_cast(float, p < 2 ? qa[m][i][2 * p + 1] : qb[m][i][2 * p - 3]);
                             const _Float16 h0 = (_Float16)v0, h1 = (_Float16)v1;
                             const _Float16 l0 = (_Float16)(v0 - (float)h0), l1 = (_Float16)(v1 - (float)h1);
                             hi[p] = __builtin_bit_cast(uint32_t, half2_t{h0, h1});
                             lo[p] = __builtin_bit_cast(uint32_t, half2_t{l0, l1});
                         }
-                        write_planes(u, 0, hi[0], hi[1], hi[2], hi[3]);
-                        write_planes(u, 4, lo[0], lo[1], lo[2], lo[3]);
+                        write_planes(u, 8 * m, hi[0], hi[1], hi[2], hi[3]);
+                        write_planes(u, 8 * m + 4, lo[0], lo[1], lo[2], lo[3]);
                     } else {
                         write_planes(u, 4 * m, qa[m][i][0], qa[m][i][1], qb[m][i][0], qb[m][i][1]);
                     }
@@ -301,10 +311,11 @@ __global__ __launch_bounds__(64 * WAVES) void gemv8_kernel(const void *__restric
             v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x104, 0xF, 0xF, false));   // row_shl:4
         acc[r] = v;
     }
-    // lanes j = 4 m now hold row m's sums (X32: lane 0 the one row's)
-    if ((j & 3) == 0 && (j >> 2) < MR) {
+    // lanes j = 4 m now hold row m's sums (X32: lanes j = 8 m)
+    constexpr int kCols = X32 ? 8 : 4;
+    if ((j & (kCols - 1)) == 0 && j / kCols < MR) {
 #pragma unroll
-        for (int r = 0; r < 4; r++) red[(wv * MR + (j >> 2)) * 16 + 4 * g + r] = acc[r];
+        for (int r = 0; r < 4; r++) red[(wv * MR + j / kCols) * 16 + 4 * g + r] = acc[r];
     }
     __syncthreads();
     if (stores) {
@@ -312,7 +323,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemv8_kernel(const void *__restric
         float v = red[((st_c * KS) * MR + st_m) * 16 + i16];
 #pragma unroll
         for (int q = 1; q < KS; q++) v += red[((st_c * KS + q) * MR + st_m) * 16 + i16];
-        if constexpr (X32) v *= ps_inv;
+        if constexpr (X32) v *= MR > 1 && st_m ? ps_inv[MR - 1] : ps_inv[0];
         v = v * (sc * (1.0f / kWeightUnit)) + bi;
         if (ep.residual) v += ep.y_f16 ? (float)__builtin_bit_cast(_Float16, (uint16_t)res_bits) : __builtin_bit_cast(float, res_bits);
         if (ep.relu) v = v < 0.f ? 0.f : v;
@@ -354,7 +365,7 @@ template <int WAVES, int CB, int NT, int ORDER, bool X32 = false, int MR = 1, bo
 int launch_gemv8(const void *x, const void *native, int64_t Kb, int64_t N, const Gemv8Epilogue &ep, void *stream) {
     const int64_t Nb = native_blocks_n(N), grid = (Nb + CB - 1) / CB;
     if (grid > 0x7FFFFFFF) return TMQ_ERR_TOO_LARGE;
-    size_t image = (X32 ? 8 : 4 * MR) * (size_t)(Kb * kKB + 32);
+    size_t image = (X32 ? 8 : 4) * MR * (size_t)(Kb * kKB + 32);
     if (PRE) image = (image + 1023) & ~(size_t)1023;
     const size_t lds = image + (size_t)WAVES * MR * 16 * sizeof(float);
     if (lds > kGemv8LdsMax) return TMQ_ERR_UNSUPPORTED;
@@ -371,7 +382,15 @@ int launch_gemv8(const void *x, const void *native, int64_t Kb, int64_t N, const
 // prepare or copy the activation planes).
 template <bool X32, int MR, bool PRE>
 int launch_gemv8_by_blocks(const void *x, int64_t Kb, const void *native, int64_t N, const Gemv8Epilogue &ep, void *stream) {
-    if constexpr (X32) {
+    if constexpr (X32 && MR == 2) {
+        // Two fp32 rows: sixteen planes, the LDS of one fp32 row of twice the length (gemv8_dense32_ok: K <= 6144)
+        if (Kb > 24) return TMQ_ERR_UNSUPPORTED;
+        switch ((Kb + 7) / 8) {
+            case 1: return launch_gemv8<8, 1, 1, 0, true, 2, false>(x, native, Kb, N, ep, stream);
+            case 2: return launch_gemv8<8, 1, 2, 0, true, 2, false>(x, native, Kb, N, ep, stream);
+            default: return launch_gemv8<16, 2, 3, 1, true, 2, false>(x, native, Kb, N, ep, stream);
+        }
+    } else if constexpr (X32) {
         // wide layers: four channel blocks per workgroup of sixteen wavefronts keep all workgroups resident at once
         // (8192 x 28672: 1792 workgroups in 3.5 rounds -> 448 in one)
         if (Kb > 16 && Kb <= 32 && native_blocks_n(N) >= 1024) {
@@ -494,14 +513,19 @@ int launch_gemv8_dense(const void *x, int64_t M, int64_t K, const void *native, 
 }
 
 // One fp32 row: K a multiple of 256 from 2048 to 16384 (eight term planes; beyond 8192 they leave room for one
-// workgroup per CU only, which then has sixteen wavefronts).
-bool gemv8_dense32_ok(const void *x, int64_t M, int64_t K) {
-    return M == 1 && K % kKB == 0 && K >= 8 * kKB && K <= 64 * kKB && aligned16(x);
+// workgroup per CU only, which then has sixteen wavefronts). Two fp32 rows (sixteen planes, all sixteen activation
+// columns) while the layer is small: every workgroup splits both rows, which beats a split launch in front of the
+// fp16 weight stream up to about 6144^2 (2048^2 5.96 -> 4.3 us, 4096^2 7.45 -> 6.1, 6144^2 9.9 -> 8.7) and loses on
+// wider or longer layers (4096 x 11008 9.7 -> 11.5, 8192^2 10.3 -> 11.4, 8192 x 1024 8.1 -> 9.8).
+bool gemv8_dense32_ok(const void *x, int64_t M, int64_t K, int64_t N) {
+    if (K % kKB != 0 || K < 8 * kKB || !aligned16(x)) return false;
+    return M == 1 ? K <= 64 * kKB : M == 2 && K <= 24 * kKB && N <= 6144;
 }
 
-int launch_gemv8_dense32(const void *x, int64_t K, const void *native, int64_t N, const float *scale, const float *bias,
+int launch_gemv8_dense32(const void *x, int64_t M, int64_t K, const void *native, int64_t N, const float *scale, const float *bias,
                          const void *residual, int relu, void *y, int y_f16, void *stream) {
-    const Gemv8Epilogue ep{scale, bias, residual, y, relu, y_f16, 1};
+    const Gemv8Epilogue ep{scale, bias, residual, y, relu, y_f16, (int)M};
+    if (M == 2) return launch_gemv8_by_blocks<true, 2, false>(x, K / kKB, native, N, ep, stream);
     return launch_gemv8_by_blocks<true, 1, false>(x, K / kKB, native, N, ep, stream);
 }
 

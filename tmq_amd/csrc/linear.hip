@@ -37,8 +37,8 @@ int64_t gemv8_padded_rows(int64_t M);
 int launch_gemv8_planes(const void *planes, int64_t M, int64_t K, const void *native, int64_t N, const float *scale,
                         const float *bias, const void *residual, int relu, void *y, int y_f16, void *stream);
 int launch_gemv8_prepare(const void *x, int64_t M, int64_t K, void *planes, void *stream);
-bool gemv8_dense32_ok(const void *x, int64_t M, int64_t K);
-int launch_gemv8_dense32(const void *x, int64_t K, const void *native, int64_t N, const float *scale, const float *bias,
+bool gemv8_dense32_ok(const void *x, int64_t M, int64_t K, int64_t N);
+int launch_gemv8_dense32(const void *x, int64_t M, int64_t K, const void *native, int64_t N, const float *scale, const float *bias,
                          const void *residual, int relu, void *y, int y_f16, void *stream);
 
 namespace {
@@ -1085,7 +1085,11 @@ int tmq_prepack_weights(const uint32_t *words, int64_t N, int64_t C, int64_t ky,
 }
 
 int tmq_fp32_rows_self_scaled(const void *x, int64_t M, int64_t K) {
-    return gemv8_dense32_ok(x, M, K) ? 1 : 0;
+    return M == 1 && gemv8_dense32_ok(x, M, K, 16) ? 1 : 0;
+}
+
+int tmq_fp32_rows_self_scaled_for(const void *x, int64_t M, int64_t K, int64_t N) {
+    return gemv8_dense32_ok(x, M, K, N) ? 1 : 0;
 }
 
 int tmq_fp32_rows_prefer_split(int64_t M, int64_t K, int64_t N) {
@@ -1153,9 +1157,9 @@ int tmq_ternary_linear(const void *x, int x_dtype, int64_t M, int64_t K, const v
     // 3.75 -> 3.0 us, 16384^2: 17.7 -> 15.6 us).
     if (!x32 && gemv8_dense_ok(x, M, K, N))
         return launch_gemv8_dense(x, M, K, native, N, ep.scale, ep.bias, ep.residual, ep.relu, y, ep.y_dtype == TMQ_F16, stream);
-    // ... and one fp32 row (the reference's GEMV convention) up to K = 16384: the same kernel on the row's two fp16 halves
-    if (x32 && gemv8_dense32_ok(x, M, K))
-        return launch_gemv8_dense32(x, K, native, N, ep.scale, ep.bias, ep.residual, ep.relu, y, ep.y_dtype == TMQ_F16, stream);
+    // ... and one fp32 row (the reference's GEMV convention) up to K = 16384, two over small layers: the same kernel on the rows' two fp16 halves
+    if (x32 && gemv8_dense32_ok(x, M, K, N))
+        return launch_gemv8_dense32(x, M, K, native, N, ep.scale, ep.bias, ep.residual, ep.relu, y, ep.y_dtype == TMQ_F16, stream);
     // At most 16 fp16 rows against eight or more weight blocks per channel: the weight-stream kernel (mid.hip).
     // Against the kernels below: M = 16 at 16384^2 67 -> 20 us, M = 8 at 8192 x 28672 34 -> 17 us, M = 1 at
     // 11008 x 4096 7.2 -> 6.2 us, even at 4096^2.

@@ -242,7 +242,7 @@ void check_mm_args(const torch::Tensor &lhs, const torch::Tensor &weights, int64
 // rows run the fp16 kernels over the two fp16 terms, y = W hi + W lo, and few rows the kernels that split on the fly.
 torch::Tensor linear_f32(const torch::Tensor &x, int64_t M, int64_t K, const torch::Tensor &native, int64_t columns,
                          torch::Tensor &y, const char *name) {
-    if (tmq_fp32_rows_self_scaled(x.data_ptr(), M, K)) {   // a single row the kernel scales itself: one launch
+    if (tmq_fp32_rows_self_scaled_for(x.data_ptr(), M, K, columns)) {   // one row (two over a small layer) the kernel scales itself: one launch
         check(tmq_ternary_linear(x.data_ptr(), TMQ_F32, M, K, native.data_ptr(), columns, nullptr, y.data_ptr(), stream_of(x)), name);
         return y;
     }
