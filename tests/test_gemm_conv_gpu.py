@@ -208,6 +208,24 @@ def test_conv2d_asymmetric_padding(cuda, C, H, W, N, k, stride, pad, dil):
     assert torch.equal(y, ref)
 
 
+def test_residual_with_a_dimension_of_size_one(cuda):
+    """One output channel (or one row, one column): the residual's stride along a dimension of size one says nothing
+    about its layout, so a channels_last residual is accepted whichever value torch left there."""
+    from tmq_amd import ops
+    g = torch.Generator(device=cuda).manual_seed(5)
+    for N, H, W in ((1, 9, 11), (8, 1, 12), (8, 7, 1)):
+        Wt = torch.randint(-1, 2, (N, 16, 1, 1), device=cuda, generator=g).float()
+        x = torch.randint(-4, 5, (2, 16, H, W), device=cuda, generator=g).float()
+        nw = ops.NativeWeights(ops.compactify_ternary(Wt), N, conv_kernel=(1, 1))
+        ref = torch.nn.functional.conv2d(x, Wt)
+        for res in (torch.randint(-3, 4, ref.shape, device=cuda, generator=g).float(),
+                    torch.randint(-3, 4, ref.shape, device=cuda, generator=g).float().contiguous(memory_format=torch.channels_last)):
+            if not res.is_contiguous(memory_format=torch.channels_last):
+                continue
+            y = ops.ternary_conv2d(x.half(), nw, residual=res)
+            assert torch.equal(y, ref + res), (N, H, W)
+
+
 def test_resnet_layer_shapes_against_torch(cuda):
     """Full-size ResNet-18 layer shapes (batch 8): checked against torch's fp32 convolution on the
     expanded weights, which the small cases above tie to the oracle."""
