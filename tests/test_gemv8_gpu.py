@@ -222,10 +222,10 @@ def test_wide_layers(cuda, oracle, K):
             assert torch.equal(ops.ternary_linear_planes(ops.gemv8_prepare(x), nw, scale, bias), y)
 
 
-@pytest.mark.parametrize("K", [8448, 11008, 12288, 16384])
+@pytest.mark.parametrize("K", [6144, 8448, 11008, 12288, 16384])
 def test_two_long_rows_against_wide_layers(cuda, oracle, K):
     """Two fp16 rows of more than 8192 indices against 16384 channels or more: eight planes on the sixteen-wavefront
-    workgroups. Rows of different magnitude stay apart, every row equals its own single-row launch bit for bit, every
+    workgroups (and 6144 indices, whose 24 weight blocks deal out evenly over eight wavefronts: the same kernel at any width). Rows of different magnitude stay apart, every row equals its own single-row launch bit for bit, every
     finite fp16 value passes an identity layer, and a narrower layer (the weight-stream kernel) agrees."""
     from tmq_amd import ops
     N = 16400
@@ -306,7 +306,7 @@ def test_hip_graph_replays_match_eager(cuda, oracle):
 
 
 # ---- two to four rows: row m's four term planes ride in activation columns 4 m .. 4 m + 3 -----------------------
-@pytest.mark.parametrize("M,K", [(2, 2048), (2, 4096), (2, 2304), (3, 2048), (4, 2048), (2, 8192), (4, 4096)])
+@pytest.mark.parametrize("M,K", [(2, 2048), (2, 4096), (2, 2304), (3, 2048), (4, 2048), (2, 8192), (4, 4096), (2, 6144), (2, 5120), (2, 7168)])
 @pytest.mark.parametrize("N", [16, 1000, 4100])
 def test_few_rows_on_the_8bit_instruction(cuda, oracle, M, K, N):
     from tmq_amd import ops

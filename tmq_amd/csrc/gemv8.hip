@@ -492,13 +492,17 @@ int launch_gemv8_by_blocks(const void *x, int64_t Kb, const void *native, int64_
 // True when the 8-bit GEMV can take a dense fp16 problem: one row up to K = 16384; two rows up to 4096 and three
 // or four at 2048 -- every workgroup prepares the planes of all rows, and beyond 8192 values that preparation costs
 // more than the weight-stream kernel's fp16 expansion (measured: two rows at 4096^2 3.9 -> 3.6 us, four rows
-// 4.0 -> 4.9 us; two rows at 8192^2 6.9 -> 7.1 us, at 8192 x 28672 15.5 -> 17.7 us). Two rows of more than 8192
-// indices against 16384 or more channels are the exception: their eight planes fill the LDS like one fp32 row's, the
-// sixteen-wavefront workgroups of that row take them, and the weight-stream kernel is the slower one there
+// 4.0 -> 4.9 us; two rows at 8192 x 28672 15.5 -> 17.7 us). Two longer rows where it measured faster (medians,
+// weight stream -> this kernel): up to 8192 indices against at most 4096 channels (8192 x 4096 5.1 -> 4.75 us,
+// 7168 x 4096 5.2 -> 4.6), up to 6144 indices against at most 6144 channels or when the weight blocks deal out
+// evenly over the eight wavefronts (6144 x 11008 7.7 -> 6.85, 6144 x 16384 9.65 -> 8.9; 5120 x 16384 8.3 -> 8.4 and
+// 7168 x 11008 8.2 -> 8.8 stay on the weight stream). More than 8192 indices against 16384 or more channels: the
+// eight planes fill the LDS like one fp32 row's, the sixteen-wavefront workgroups of that row take them
 // (16384^2: 17.9 -> 15.5 us, 12288 x 16384: 13.8 -> 11.9 us; 11008 x 4096, on eight wavefronts: 6.2 -> 7.6 us, refused).
 bool gemv8_dense_ok(const void *x, int64_t M, int64_t K, int64_t N) {
     if (M < 1 || M > 4 || K % kKB != 0 || K < 8 * kKB || !aligned16(x)) return false;
     if (M == 2 && K > 32 * kKB) return K <= 64 * kKB && native_blocks_n(N) >= 1024;
+    if (M == 2 && K > 16 * kKB) return N <= 4096 || (K <= 24 * kKB && (N <= 6144 || (K / kKB) % 8 == 0));
     return M == 1 ? K <= 64 * kKB : K * (M == 3 ? 4 : M) <= 32 * kKB;
 }
 
