@@ -243,7 +243,11 @@ def test_two_long_rows_against_wide_layers(cuda, oracle, K):
     for m in range(2):
         err = ((y[m].double() - ref[m]).abs().max() / ref[m].abs().max()).item()
         assert err <= 1e-5, (K, m, err)
-        assert torch.equal(ops.ternary_linear(x[m:m + 1], nw, scale, bias)[0], y[m]), (K, m)
+        single = ops.ternary_linear(x[m:m + 1], nw, scale, bias)[0]
+        if K > 8192:                         # the same geometry as the single row: the same sums in the same order
+            assert torch.equal(single, y[m]), (K, m)
+        else:                                # (a single row of 6144 indices splits its blocks over four wavefronts, two rows over eight)
+            assert ((single.double() - y[m].double()).abs().max() / ref[m].abs().max()).item() <= 2e-6, (K, m)
     res = torch.from_numpy(rng.standard_normal((2, N)).astype(np.float16)).to(cuda)
     y2 = ops.ternary_linear(x, nw, scale, bias, residual=res, relu=True, out_dtype=torch.float16)
     ref2 = torch.clamp_min(ref + res.double(), 0)
