@@ -31,7 +31,8 @@
 // Two to four rows (MR = 2, 4; three rows run as four with one of zeros) take the same kernel: row m's four
 // term planes ride in activation columns 4 m .. 4 m + 3, so four rows fill exactly the sixteen columns of the
 // instruction the single row already issues -- no extra MFMA, no extra weight expansion; only the planes (and
-// the work of preparing them) grow with the rows, which is what limits the rows: see gemv8_dense_ok.
+// the work of preparing them) grow with the rows, which is what limits the rows: two split inside the kernel
+// (gemv8_dense_ok), three and four only with the planes prepared beforehand.
 //
 // The planes can also come ready-made from memory (PRE): tmq_gemv8_prepare writes them once per activation
 // vector (or a producing kernel could), and the workgroup then copies its image global -> LDS with buffer loads
@@ -489,10 +490,11 @@ int launch_gemv8_by_blocks(const void *x, int64_t Kb, const void *native, int64_
 
 }  // namespace
 
-// True when the 8-bit GEMV can take a dense fp16 problem: one row up to K = 16384; two rows up to 4096 and three
-// or four at 2048 -- every workgroup prepares the planes of all rows, and beyond 8192 values that preparation costs
-// more than the weight-stream kernel's fp16 expansion (measured: two rows at 4096^2 3.9 -> 3.6 us, four rows
-// 4.0 -> 4.9 us; two rows at 8192 x 28672 15.5 -> 17.7 us). Two longer rows where it measured faster (medians,
+// True when the 8-bit GEMV can take a dense fp16 problem: one row up to K = 16384, two rows up to 4096 -- every
+// workgroup prepares the planes of all rows, and that preparation soon costs more than the weight-stream kernel's
+// fp16 expansion (measured: two rows at 4096^2 4.2 -> 3.6 us, at 2048^2 3.1 -> 3.0, at 8192 x 28672 15.5 -> 17.7;
+// three or four rows lose at every length -- 2048^2 3.2 -> 3.6 us, 2048 x 11008 4.7 -> 5.9, 4096^2 4.3 -> 5.2 -- and
+// reach this kernel only with planes prepared beforehand). Two longer rows where it measured faster (medians,
 // weight stream -> this kernel): up to 8192 indices against at most 4096 channels (8192 x 4096 5.1 -> 4.75 us,
 // 7168 x 4096 5.2 -> 4.6), up to 6144 indices against at most 6144 channels or when the weight blocks deal out
 // evenly over the eight wavefronts (6144 x 11008 7.7 -> 6.85, 6144 x 16384 9.65 -> 8.9; 5120 x 16384 8.3 -> 8.4 and
@@ -500,10 +502,10 @@ int launch_gemv8_by_blocks(const void *x, int64_t Kb, const void *native, int64_
 // eight planes fill the LDS like one fp32 row's, the sixteen-wavefront workgroups of that row take them
 // (16384^2: 17.9 -> 15.5 us, 12288 x 16384: 13.8 -> 11.9 us; 11008 x 4096, on eight wavefronts: 6.2 -> 7.6 us, refused).
 bool gemv8_dense_ok(const void *x, int64_t M, int64_t K, int64_t N) {
-    if (M < 1 || M > 4 || K % kKB != 0 || K < 8 * kKB || !aligned16(x)) return false;
+    if (M < 1 || M > 2 || K % kKB != 0 || K < 8 * kKB || !aligned16(x)) return false;
     if (M == 2 && K > 32 * kKB) return K <= 64 * kKB && native_blocks_n(N) >= 1024;
     if (M == 2 && K > 16 * kKB) return N <= 4096 || (K <= 24 * kKB && (N <= 6144 || (K / kKB) % 8 == 0));
-    return M == 1 ? K <= 64 * kKB : K * (M == 3 ? 4 : M) <= 32 * kKB;
+    return K <= (M == 1 ? 64 : 16) * kKB;
 }
 
 // gemv8_dense_ok must hold.
@@ -512,8 +514,7 @@ int launch_gemv8_dense(const void *x, int64_t M, int64_t K, const void *native, 
     const Gemv8Epilogue ep{scale, bias, residual, y, relu, y_f16, (int)M};
     const int64_t Kb = K / kKB;
     if (M == 1) return launch_gemv8_by_blocks<false, 1, false>(x, Kb, native, N, ep, stream);
-    if (M == 2) return launch_gemv8_by_blocks<false, 2, false>(x, Kb, native, N, ep, stream);
-    return launch_gemv8_by_blocks<false, 4, false>(x, Kb, native, N, ep, stream);
+    return launch_gemv8_by_blocks<false, 2, false>(x, Kb, native, N, ep, stream);
 }
 
 // One fp32 row: K a multiple of 256 from 2048 to 16384 (eight term planes; beyond 8192 they leave room for one

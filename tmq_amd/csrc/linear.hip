@@ -1152,7 +1152,7 @@ int tmq_ternary_linear(const void *x, int x_dtype, int64_t M, int64_t K, const v
     if (ep.y_dtype != TMQ_F16 && ep.y_dtype != TMQ_F32) return TMQ_ERR_UNSUPPORTED;
     const bool x32 = x_dtype == TMQ_F32;
     // One fp16 row, K a multiple of 256 from 2048 to 16384 (two rows to 4096 and where gemv8_dense_ok measured them
-    // faster beyond; three or four rows to 2048): weights and
+    // faster beyond): weights and
     // activations as 8-bit MFMA operands (gemv8.hip), half the decode work per weight of the kernels below (4096^2:
     // 3.75 -> 3.0 us, 16384^2: 17.7 -> 15.6 us).
     if (!x32 && gemv8_dense_ok(x, M, K, N))
