@@ -311,6 +311,9 @@ int tmq_ternary_linear(const void *x, int x_dtype, int64_t M, int64_t K, const v
  * 256 are split in groups of eight rows, each group under a power of two of its own, laid out so that a row's two
  * terms share a 16-row MFMA fragment; the fp16 GEMM kernels then run once over 16 ceil(M / 8) rows and add the pairs
  * where they write the tile (ceil(M / 8) floats rounded up to 256 bytes + 32 ceil(M / 8) K bytes).
+ * Seventeen fp16 rows or more whose K is no multiple of 64 are copied once to rows of the next multiple of 64, zeros
+ * behind (2 M ceil(K / 64) 64 bytes), and take the kernels that want whole 64-index tiles of 16-byte aligned rows
+ * instead of the one that guards every load (K = 4000, M = 1024, N = 4096: 261 -> 39 us).
  * tmq_ternary_linear_workspace_bytes returns what a shape can use (0: the single-launch kernels are at
  * least as fast); with a NULL or smaller workspace tmq_ternary_linear_ws is tmq_ternary_linear. Same results to
  * fp32 rounding (the summation order differs). The workspace must be 16-byte aligned.                     */

@@ -56,9 +56,10 @@ def test_workspace_contract(cuda):
     nw = ops.NativeWeights(ops.compactify_ternary(W), N)
     need = lib.tmq_ternary_linear_workspace_bytes(_capi.F16, M, K, N)
     assert need >= 2 * M * N * 4
-    for Mx, Kx, Nx in ((16, 16384, 16384), (33, 16384, 16384), (28, 2048, 131072), (28, 16384, 16392), (28, 16392, 16384),
-                       (28, 8192, 8192)):
+    for Mx, Kx, Nx in ((16, 16384, 16384), (33, 16384, 16384), (28, 2048, 131072), (28, 16384, 16392), (28, 8192, 8192)):
         assert lib.tmq_ternary_linear_workspace_bytes(_capi.F16, Mx, Kx, Nx) == 0, (Mx, Kx, Nx)
+    # a ragged length asks for the rows' padded copy instead (test_ragged_rows_gpu.py)
+    assert lib.tmq_ternary_linear_workspace_bytes(_capi.F16, 28, 16392, 16384) == 2 * 28 * 16448
     # fp32 rows use the workspace for their fp16 row pairs, not for partial sums (test_fp32_row_pairs_gpu.py)
     assert lib.tmq_ternary_linear_workspace_bytes(_capi.F32, M, K, N) == 256 + 32 * ((M + 7) // 8) * K
     ep = _capi.Epilogue()

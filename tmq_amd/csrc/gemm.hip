@@ -1120,6 +1120,16 @@ inline bool row_pairs_ok(const void *x, int64_t M, int64_t K, int64_t N) {
 }
 inline size_t row_pairs_bytes(int64_t M, int64_t K) { return 256 + (size_t)(2 * M * K) * sizeof(_Float16); }
 
+// Seventeen fp16 rows or more whose reduction length is no multiple of 64: the kernels with direct global -> LDS
+// loads want whole 64-index tiles of 16-byte aligned rows, and the register-staged kernel that takes everything else
+// guards every load (K = 4000 against 4096 at M = 1024, N = 4096: 261 us against 35). With a workspace the rows are
+// copied once to rows of the next multiple of 64, zeros behind (the native weights are padded with zeros to whole
+// 256-index blocks anyway), and take the aligned kernels: 261 -> 39 us, K = 784, M = 128, N = 1024 24.4 -> 6 us.
+int launch_pad_rows(const void *x, int64_t M, int64_t K, int64_t Kp, void *out, void *stream);
+inline int64_t padded_k(int64_t K) { return (K + 63) / 64 * 64; }
+inline bool pad_rows_ok(int64_t M, int64_t K) { return M >= 17 && K % 64 != 0 && M * padded_k(K) < (int64_t)0x7FFFFFFF; }
+inline size_t pad_rows_bytes(int64_t M, int64_t K) { return (size_t)(M * padded_k(K)) * sizeof(_Float16); }
+
 // Seventeen fp32 rows or more over K a multiple of 64: one launch splits them into fp16 row pairs in groups of eight,
 // every group scaled by a power of two of its own (PairMap); the fp16 kernels then run once over 16 ceil(M / 8) rows
 // and their epilogues add each pair and undo the group's scale. Against the kernels that split on the fly, or two
@@ -1185,7 +1195,8 @@ size_t tmq_ternary_linear_workspace_bytes(int x_dtype, int64_t M, int64_t K, int
     if (x_dtype != TMQ_F16) return 0;
     static const _Float16 *const aligned = nullptr;              // the plan assumes 16-byte aligned rows; _ws checks the real pointer
     const int slices = rows_split_slices(aligned, M, K, N);
-    return slices ? (size_t)slices * (size_t)M * (size_t)N * sizeof(float) : 0;
+    if (slices) return (size_t)slices * (size_t)M * (size_t)N * sizeof(float);
+    return pad_rows_ok(M, K) ? pad_rows_bytes(M, K) : 0;
 }
 
 int tmq_ternary_linear_ws(const void *x, int x_dtype, int64_t M, int64_t K, const void *native, int64_t N,
@@ -1235,6 +1246,10 @@ int tmq_ternary_linear_ws(const void *x, int x_dtype, int64_t M, int64_t K, cons
             if (e.y_dtype != TMQ_F16 && e.y_dtype != TMQ_F32) return TMQ_ERR_UNSUPPORTED;
             const Epilogue ep{e.scale, e.bias, e.residual, y, e.relu, e.y_dtype == TMQ_F16 ? 1 : 0};
             return launch_rows_split(x, M, K, native, N, ep, static_cast<float *>(workspace), slices, stream);
+        }
+        if (!slices && pad_rows_ok(M, K) && workspace_bytes >= pad_rows_bytes(M, K)) {
+            if (int st = launch_pad_rows(x, M, K, padded_k(K), workspace, stream)) return st;
+            return tmq_ternary_linear(workspace, TMQ_F16, M, padded_k(K), native, N, epilogue, y, stream);
         }
     }
     return tmq_ternary_linear(x, x_dtype, M, K, native, N, epilogue, y, stream);

@@ -350,6 +350,37 @@ int launch_split_groups(const float *x, int64_t M, int64_t K, void *x16, float *
     return check_launch();
 }
 
+// Rows of K fp16 values copied to rows of Kp >= K values (Kp a multiple of 8), zeros behind the K-th: a thread moves
+// one 16-byte piece of the destination (vec: K % 8 == 0 and x 16-byte aligned, so the piece is one load as well).
+__global__ __launch_bounds__(256) void pad_rows_kernel(const _Float16 *__restrict__ x, uint32_t pieces, int K, FastDiv by_row,
+                                                       _Float16 *__restrict__ out, int vec) {
+    const uint32_t id = blockIdx.x * 256u + threadIdx.x;
+    if (id >= pieces) return;
+    int c;
+    const uint32_t m = by_row.divmod(id, c);
+    const int k0 = c * 8;
+    const _Float16 *src = x + (int64_t)m * K + k0;
+    half8 v = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (vec) {
+        if (k0 < K) v = *reinterpret_cast<const half8 *>(src);
+    } else {
+#pragma unroll
+        for (int e = 0; e < 8; e++)
+            if (k0 + e < K) v[e] = src[e];
+    }
+    *reinterpret_cast<half8 *>(out + (int64_t)id * 8) = v;
+}
+
+// out: M rows of Kp fp16 values, 16-byte aligned; Kp % 8 == 0, M Kp < 2^31.
+int launch_pad_rows(const void *x, int64_t M, int64_t K, int64_t Kp, void *out, void *stream) {
+    const int64_t pieces = M * (Kp / 8);
+    if (pieces <= 0 || pieces > 0x7FFFFFFF) return TMQ_ERR_TOO_LARGE;
+    hipLaunchKernelGGL(pad_rows_kernel, dim3((uint32_t)((pieces + 255) / 256)), dim3(256), 0, as_stream(stream),
+                       static_cast<const _Float16 *>(x), (uint32_t)pieces, (int)K, FastDiv((uint32_t)(Kp / 8)),
+                       static_cast<_Float16 *>(out), (K % 8 == 0 && aligned16(x)) ? 1 : 0);
+    return check_launch();
+}
+
 // x16: 2 M rows of K fp16 values, row_scale: M floats; K % 8 == 0, x and x16 16-byte aligned.
 int launch_split_rows(const float *x, int64_t M, int64_t K, int64_t group, void *x16, float *row_scale, void *stream) {
     hipLaunchKernelGGL(split_rows_kernel, dim3((uint32_t)M), dim3(1024), 0, as_stream(stream), x, K, (int)M, (int)group,

@@ -296,6 +296,14 @@ torch::Tensor ternary_mmm_cuda(torch::Tensor lhs, torch::Tensor weights, int64_t
     const int64_t M = K ? x.numel() / K : 0;
     if (M == 0) return y;
     if (x.scalar_type() == torch::kFloat32) return linear_f32(x, M, K, native, columns, y, "ternary_mmm_cuda");
+    // shapes that gain from a workspace (partial sums of a reduction cut across workgroups; a padded copy of rows
+    // whose length is no multiple of 64) get one
+    if (const size_t bytes = M > 16 && (M <= 32 || K % 64) ? tmq_ternary_linear_workspace_bytes(TMQ_F16, M, K, columns) : 0) {
+        auto ws = torch::empty({(int64_t)bytes}, x.options().dtype(torch::kUInt8));
+        check(tmq_ternary_linear_ws(x.data_ptr(), TMQ_F16, M, K, native.data_ptr(), columns, nullptr, y.data_ptr(), ws.data_ptr(),
+                                    bytes, stream_of(x)), "ternary_mmm_cuda");
+        return y;
+    }
     check(tmq_ternary_linear(x.data_ptr(), TMQ_F16, M, K, native.data_ptr(), columns, nullptr, y.data_ptr(), stream_of(x)),
           "ternary_mmm_cuda");
     return y;

@@ -649,8 +649,10 @@ def ternary_linear(x: torch.Tensor, nw: NativeWeights, scale=None, bias=None, re
     y = torch.empty(x.shape[:-1] + (nw.N,), dtype=out_dtype, device=x.device)
     ep = _epilogue(nw, scale, bias, residual, relu, out_dtype, y)
     lib = _lib()
-    # shapes whose reduction pays to be cut across workgroups get a workspace for the partial sums
-    wsb = pairs or (lib.tmq_ternary_linear_workspace_bytes(_capi.dtype_code(x), M, nw.K, nw.N) if 16 < M <= 32 else 0)
+    # shapes whose reduction pays to be cut across workgroups get a workspace for the partial sums, and rows of a
+    # ragged length one for their copy padded to whole 64-index tiles
+    wsb = pairs or (lib.tmq_ternary_linear_workspace_bytes(_capi.dtype_code(x), M, nw.K, nw.N)
+                    if M > 16 and (M <= 32 or nw.K % 64) else 0)
     with _capi.on_device(x.device):
         if wsb:
             ws = torch.empty(wsb, dtype=torch.uint8, device=x.device)
