@@ -1134,18 +1134,19 @@ inline size_t pad_rows_bytes(int64_t M, int64_t K) { return (size_t)(M * padded_
 // every group scaled by a power of two of its own (PairMap); the fp16 kernels then run once over 16 ceil(M / 8) rows
 // and their epilogues add each pair and undo the group's scale. Against the kernels that split on the fly, or two
 // fp16 passes chained through the residual.
-int launch_split_groups(const float *x, int64_t M, int64_t K, void *x16, float *group_scale, void *stream);
+int launch_split_groups(const float *x, int64_t M, int64_t K, int64_t Kp, void *x16, float *group_scale, void *stream);
 int launch_mid_dense_pairs(const void *x16, int64_t M16, int64_t K, const void *native, int64_t N, const float *scale,
                            const float *bias, const void *residual, int relu, void *y, int y_f16, int64_t rows_out,
                            const float *group_scale, void *stream);
 inline int64_t pair_rows16(int64_t M) { return (M + 7) / 8 * 16; }
 inline bool pair_rows_ok(const void *x, int64_t M, int64_t K, int64_t N) {
-    return M >= 17 && K % 64 == 0 && K >= 256 && aligned16(x) && pair_rows16(M) * K < (int64_t)0x7FFFFFFF;
+    (void)x;                                                       // rows of any alignment: the splitter reads them element-wise if it must
+    return M >= 17 && K >= 256 && pair_rows16(M) * padded_k(K) < (int64_t)0x7FFFFFFF;
 }
 // the workspace: the groups' 1 / s (padded to 256 bytes), then the fp16 rows
 inline size_t pair_scale_bytes(int64_t M) { return ((size_t)((M + 7) / 8) * sizeof(float) + 255) & ~(size_t)255; }
 inline size_t pair_rows_bytes(int64_t M, int64_t K, int64_t N) {
-    return pair_scale_bytes(M) + (size_t)(pair_rows16(M) * K) * sizeof(_Float16);
+    return pair_scale_bytes(M) + (size_t)(pair_rows16(M) * padded_k(K)) * sizeof(_Float16);
 }
 
 }  // namespace tmq
@@ -1231,12 +1232,15 @@ int tmq_ternary_linear_ws(const void *x, int x_dtype, int64_t M, int64_t K, cons
         if (e.y_dtype != TMQ_F16 && e.y_dtype != TMQ_F32) return TMQ_ERR_UNSUPPORTED;
         float *group_scale = static_cast<float *>(workspace);
         void *x16 = static_cast<unsigned char *>(workspace) + pair_scale_bytes(M);
-        if (int st = launch_split_groups(static_cast<const float *>(x), M, K, x16, group_scale, stream)) return st;
+        // (a length that is no multiple of 64: rows of the next multiple, zeros behind -- the native weights are padded
+        // with zeros to whole 256-index blocks)
+        const int64_t Kp = padded_k(K);
+        if (int st = launch_split_groups(static_cast<const float *>(x), M, K, Kp, x16, group_scale, stream)) return st;
         const int64_t M16 = pair_rows16(M);
         const int y_f16 = e.y_dtype == TMQ_F16 ? 1 : 0;
-        if (split_reduction_pays(M16, K, N))
-            return launch_mid_dense_pairs(x16, M16, K, native, N, e.scale, e.bias, e.residual, e.relu, y, y_f16, M, group_scale, stream);
-        return launch_gemm_dense_pairs(x16, M16, K, native, N, e.scale, e.bias, e.residual, e.relu, y, y_f16, M, group_scale, stream);
+        if (split_reduction_pays(M16, Kp, N))
+            return launch_mid_dense_pairs(x16, M16, Kp, native, N, e.scale, e.bias, e.residual, e.relu, y, y_f16, M, group_scale, stream);
+        return launch_gemm_dense_pairs(x16, M16, Kp, native, N, e.scale, e.bias, e.residual, e.relu, y, y_f16, M, group_scale, stream);
     }
     if (x && native && y && x_dtype == TMQ_F16 && M > 0 && K > 0 && N > 0 && workspace && aligned16(workspace) && aligned16(native)) {
         const int slices = rows_split_slices(x, M, K, N);

@@ -336,10 +336,54 @@ __global__ __launch_bounds__(1024) void split_groups_kernel(const float *__restr
 
 }  // namespace
 
-// x16: 16 ceil(M / 8) rows of K fp16 values; group_scale: ceil(M / 8) floats. K % 4 == 0, x and x16 16-byte aligned.
-int launch_split_groups(const float *x, int64_t M, int64_t K, void *x16, float *group_scale, void *stream) {
+// The same split for rows of any length and alignment, written as rows of Kp >= K values (Kp a multiple of 8) with
+// zeros behind the K-th: one workgroup per group of eight rows, element-wise reads, one 16-byte piece of a hi row and
+// of its lo row per thread and step. The second pass over the group's 32 K bytes comes from L2.
+__global__ __launch_bounds__(1024) void split_groups_padded_kernel(const float *__restrict__ x, int64_t M, int K, int Kp,
+                                                                   FastDiv by_row, _Float16 *__restrict__ x16,
+                                                                   float *__restrict__ group_scale) {
+    __shared__ float lds[17];
+    const int64_t g = blockIdx.x;
+    const float *src = x + g * 8 * (int64_t)K;
+    const int rows = M - g * 8 < 8 ? (int)(M - g * 8) : 8;
+    float amax = 0.f;
+    for (int at = threadIdx.x; at < rows * K; at += 1024) amax = fmaxf(amax, finite_abs(src[at]));
+    amax = block_max(amax, lds);
+    float s, inv;
+    make_prescale(amax, s, inv);
+    if (threadIdx.x == 0) group_scale[g] = inv;
+    _Float16 *dst = x16 + g * 16 * (int64_t)Kp;                    // the group's hi rows, then its lo rows
+    const uint32_t pieces = 8u * (uint32_t)(Kp / 8);
+    for (uint32_t p = threadIdx.x; p < pieces; p += 1024) {
+        int c;
+        const int r = (int)by_row.divmod(p, c);
+        const int k0 = c * 8;
+        half8 h = {0, 0, 0, 0, 0, 0, 0, 0}, l = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (r < rows) {
+#pragma unroll
+            for (int e = 0; e < 8; e++)
+                if (k0 + e < K) {
+                    const float v = s * src[(int64_t)r * K + k0 + e];
+                    h[e] = (_Float16)v;
+                    l[e] = (_Float16)(v - (float)h[e]);
+                }
+        }
+        *reinterpret_cast<half8 *>(dst + (int64_t)r * Kp + k0) = h;
+        *reinterpret_cast<half8 *>(dst + (int64_t)(8 + r) * Kp + k0) = l;
+    }
+}
+
+// x16: 16 ceil(M / 8) rows of Kp fp16 values (Kp >= K, a multiple of 8; zeros behind the K-th), 16-byte aligned;
+// group_scale: ceil(M / 8) floats. Whole float4s of 16-byte aligned rows and Kp == K take the kernel above.
+int launch_split_groups(const float *x, int64_t M, int64_t K, int64_t Kp, void *x16, float *group_scale, void *stream) {
     const int64_t groups = (M + 7) / 8, quads = 8 * (K / 4);
     if (groups > 0x7FFFFFFF) return TMQ_ERR_TOO_LARGE;
+    if (Kp != K || K % 4 != 0 || !aligned16(x)) {
+        if (8 * Kp > 0x7FFFFFFF) return TMQ_ERR_TOO_LARGE;
+        hipLaunchKernelGGL(split_groups_padded_kernel, dim3((uint32_t)groups), dim3(1024), 0, as_stream(stream), x, M, (int)K,
+                           (int)Kp, FastDiv((uint32_t)(Kp / 8)), static_cast<_Float16 *>(x16), group_scale);
+        return check_launch();
+    }
     auto kernel = quads <= 2 * 1024 ? split_groups_kernel<2> : quads <= 4 * 1024 ? split_groups_kernel<4>
                 : quads <= 8 * 1024 ? split_groups_kernel<8> : split_groups_kernel<16>;
     // up to 64 groups share a group among up to four workgroups (M = 32 at K = 4096: 14.5 -> 13.4 us in all, M = 512
