@@ -198,29 +198,35 @@ struct ConvLoader {
             }
         }
     }
-    __device__ __forceinline__ _Float16 at(const _Float16 *img, int ih0, int iw0, int64_t k) const {
-        if (k >= K) return (_Float16)0;
-        const int c = (int)(k % C), tap = (int)(k / C), j = tap % kx, i = tap / kx;
-        const int ih = ih0 + i * dy, iw = iw0 + j * dx;
-        if (ih < 0 || ih >= H || iw < 0 || iw >= W) return (_Float16)0;
-        return img[((int64_t)ih * W + iw) * C + c];
-    }
     template <int CH, int T>
     __device__ __forceinline__ void fetch(State<CH, T> &st, int64_t k0, u32x4 (&out)[CH]) const {
         const int64_t k = k0 + (threadIdx.x & 7) * 8;
 #pragma unroll
         for (int q = 0; q < CH; q++) {
             u32x4 v = {0u, 0u, 0u, 0u};
-            if (st.img[q] && k < K) {
-                if constexpr (VEC) {
-                    const int ih = st.ih0[q] + st.i * dy, iw = st.iw0[q] + st.j * dx;
-                    if (ih >= 0 && ih < H && iw >= 0 && iw < W)
-                        v = *reinterpret_cast<const u32x4 *>(st.img[q] + ((int64_t)ih * W + iw) * C + st.c);
-                } else {
-                    half8 h;
-                    for (int e = 0; e < 8; e++) h[e] = at(st.img[q], st.ih0[q], st.iw0[q], k + e);
-                    v = __builtin_bit_cast(u32x4, h);
+            if constexpr (VEC) {
+                // one unconditional load: chunks outside the image, past K or of rows past M read 16 bytes of zeros
+                // (conditions joined without short circuit -- as branches they are an exec-mask round trip per chunk)
+                const int ih = st.ih0[q] + st.i * dy, iw = st.iw0[q] + st.j * dx;
+                const bool in = (st.img[q] != nullptr) & (k < K) & ((unsigned)ih < (unsigned)H) & ((unsigned)iw < (unsigned)W);
+                const _Float16 *src = in ? st.img[q] + ((int64_t)ih * W + iw) * C + st.c
+                                         : reinterpret_cast<const _Float16 *>(&kZeroChunk);
+                v = *reinterpret_cast<const u32x4 *>(src);
+            } else if (st.img[q] && k < K) {
+                // element by element from the chunk's tap and channel onwards (a chunk may run over into the next tap)
+                half8 h = {0, 0, 0, 0, 0, 0, 0, 0};
+                int i = st.i, j = st.j, c = st.c;
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    const int ih = st.ih0[q] + i * dy, iw = st.iw0[q] + j * dx;
+                    if (k + e < K && (unsigned)ih < (unsigned)H && (unsigned)iw < (unsigned)W)
+                        h[e] = st.img[q][((int64_t)ih * W + iw) * C + c];
+                    if (++c == C) {
+                        c = 0;
+                        if (++j == kx) { j = 0; ++i; }
+                    }
                 }
+                v = __builtin_bit_cast(u32x4, h);
             }
             out[q] = v;
         }
