@@ -49,7 +49,9 @@ constexpr int kPitch = 64;       // LDS row pitch in halfs: 128 bytes = 8 chunks
 //     tap, so a chunk is one address -- the zero chunk for padding -- and can be loaded straight into
 //     LDS. The kernel tells init() which of the row's 8 chunks the thread fetches.
 
-// Dense rows, any K / alignment.
+// Dense rows, any K / alignment. VEC: K is a multiple of 8 and x 16-byte aligned, so a chunk is 16 aligned bytes that
+// lie wholly inside or wholly outside the row: one unconditional load, of zeros for what does not exist.
+template <bool VEC>
 struct DenseLoader {
     static constexpr bool kDirect = false;
     [[maybe_unused]] static constexpr bool kConv = false;
@@ -78,13 +80,19 @@ struct DenseLoader {
         const int64_t k = k0 + st.kc;
 #pragma unroll
         for (int i = 0; i < CH; i++) {
-            half8 h = {0, 0, 0, 0, 0, 0, 0, 0};
-            if (st.live[i]) {
+            if constexpr (VEC) {
+                const bool in = st.live[i] & (k < K);
+                const _Float16 *src = in ? st.row[i] + k : reinterpret_cast<const _Float16 *>(&kZeroChunk);
+                out[i] = *reinterpret_cast<const u32x4 *>(src);
+            } else {
+                half8 h = {0, 0, 0, 0, 0, 0, 0, 0};
+                if (st.live[i]) {
 #pragma unroll
-                for (int e = 0; e < 8; e++)
-                    if (k + e < K) h[e] = st.row[i][k + e];
+                    for (int e = 0; e < 8; e++)
+                        if (k + e < K) h[e] = st.row[i][k + e];
+                }
+                out[i] = __builtin_bit_cast(u32x4, h);
             }
-            out[i] = __builtin_bit_cast(u32x4, h);
         }
     }
     template <int CH, int T>
@@ -1031,7 +1039,9 @@ static int gemm_dense(const void *x, int64_t M, int64_t K, const void *native, i
     if ((K % kBK == 0) && aligned16(x))
         return dispatch_tile(DenseDirect{static_cast<const _Float16 *>(x), M, K}, native, M, K, N, ep, stream);
     if constexpr (decltype(ep.map)::kPairs) return TMQ_ERR_UNSUPPORTED;      // row pairs are made aligned
-    else return dispatch_tile(DenseLoader{static_cast<const _Float16 *>(x), M, K}, native, M, K, N, ep, stream);
+    else if (K % 8 == 0 && aligned16(x))
+        return dispatch_tile(DenseLoader<true>{static_cast<const _Float16 *>(x), M, K}, native, M, K, N, ep, stream);
+    else return dispatch_tile(DenseLoader<false>{static_cast<const _Float16 *>(x), M, K}, native, M, K, N, ep, stream);
 }
 
 int launch_gemm_dense(const void *x, int64_t M, int64_t K, const void *native, int64_t N, const float *scale,

@@ -18,6 +18,9 @@
 
 namespace tmq {
 
+// gemm.hip: the MFMA-bound tile kernels for large M (fp16 activations)
+int launch_gemm_dense(const void *x, int64_t M, int64_t K, const void *native, int64_t N, const float *scale,
+                      const float *bias, const void *residual, int relu, void *y, int y_f16, void *stream);
 // mid.hip: staged split-reduction kernel for mid-size fp16 problems
 bool mid_dense_ok(const void *x, int64_t M, int64_t K);
 bool stream_dense_ok(const void *x, int64_t M, int64_t K);
@@ -1039,6 +1042,14 @@ int mid_rows(const void *x, int64_t M, int64_t K, const void *native, int64_t N,
             return launch_mid_dense(x, M, K, native, N, ep.scale, ep.bias, ep.residual, ep.relu, y,
                                     ep.y_dtype == TMQ_F16, stream);
     }
+    if constexpr (!X32) {
+        // more than 64 fp16 rows of a length that is no multiple of 64 (16-byte aligned, a multiple of 8): the tile
+        // kernel's register-staged loader fetches such rows in whole 16-byte chunks, the kernel below element by element
+        // (K = 784, M = 128, N = 1024: 25.0 -> 9.0 us; K = 4000, M = 1024: 225 -> 27; up to 64 rows the skinny kernels
+        // stay: K = 4000, M = 32 10.1 against 25.6)
+        if (K % 8 == 0 && aligned16(x))
+            return launch_gemm_dense(x, M, K, native, N, ep.scale, ep.bias, ep.residual, ep.relu, y, ep.y_dtype == TMQ_F16, stream);
+    }
     if (wgs(64, 32) >= 256) return launch_mid<2, 2, 2, 16, 2, X32>(x, M, K, native, N, ep, y, stream);
     return launch_mid<2, 1, 2, 16, 2, X32>(x, M, K, native, N, ep, y, stream);
 }
@@ -1055,10 +1066,6 @@ __global__ __launch_bounds__(1024) void probe_read_kernel(const u32x4 *__restric
 }
 
 }  // namespace
-
-// gemm.hip: the MFMA-bound tile kernel for large M (fp16 activations).
-int launch_gemm_dense(const void *x, int64_t M, int64_t K, const void *native, int64_t N, const float *scale,
-                      const float *bias, const void *residual, int relu, void *y, int y_f16, void *stream);
 
 }  // namespace tmq
 
