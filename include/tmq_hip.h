@@ -339,11 +339,11 @@ int tmq_ternary_linear_planes(const void *planes, int64_t M, int64_t K, const vo
                               const tmq_epilogue *epilogue, void *y, void *stream);
 
 /* 1 when tmq_ternary_linear(x, TMQ_F32, M, K, ...) takes fp32 activations of any magnitude as they are (one
- * 16-byte aligned row, K a multiple of 256 from 2048 to 16384: the kernel finds the row's largest finite |x| and scales
+ * 16-byte aligned row, K a multiple of 256 up to 16384: the kernel finds the row's largest finite |x| and scales
  * by a power of two itself), 0 when the caller has to keep them inside fp16's range (tmq_f32_prescale). */
 int tmq_fp32_rows_self_scaled(const void *x, int64_t M, int64_t K);
-/* The same question for a layer of N channels: also 1 for two 16-byte aligned rows with K a multiple of 256 from
- * 2048 to 6144 and N <= 6144 (each row scaled by its own power of two inside the one launch). */
+/* The same question for a layer of N channels: also 1 for two 16-byte aligned rows with K a multiple of 256 up to
+ * 6144 and N <= 6144 (each row scaled by its own power of two inside the one launch). */
 int tmq_fp32_rows_self_scaled_for(const void *x, int64_t M, int64_t K, int64_t N);
 
 /* Range handling for fp32 activations (no counterpart in the reference, whose kernels multiply fp32

@@ -79,7 +79,7 @@ def test_rows_of_any_magnitude_side_by_side(cuda, oracle):
     assert np.array_equal(y[5], np.zeros(N, np.float32))
 
 
-@pytest.mark.parametrize("K", [2048, 2304, 4096, 5120, 6144])
+@pytest.mark.parametrize("K", [256, 1024, 2048, 2304, 4096, 5120, 6144])
 def test_two_rows_over_small_layers_in_one_launch(cuda, oracle, K):
     """Two fp32 rows, K <= 6144, N <= 6144: sixteen term planes in the 8-bit GEMV, each row scaled by its own power of
     two inside the launch. Rows 60 orders of magnitude apart, a row of zeros, the C ABI without any workspace, and the

@@ -168,7 +168,7 @@ def test_agrees_with_the_fp16_kernels_on_neighbouring_shapes(cuda, oracle):
     assert _rel_err(y1.cpu().numpy(), y3.cpu().numpy()) <= 1e-5
 
 
-@pytest.mark.parametrize("K", [2048, 4096, 6144, 8192, 2304, 5120, 6912, 8448, 11008, 12288, 13824, 16128, 16384])
+@pytest.mark.parametrize("K", [256, 512, 1024, 1792, 2048, 4096, 6144, 8192, 2304, 5120, 6912, 8448, 11008, 12288, 13824, 16128, 16384])
 def test_fp32_row_runs_as_two_fp16_halves(cuda, oracle, K):
     """One fp32 row (the reference's GEMV convention) up to K = 16384: hi = fp16(x), lo = fp16(x - hi), each as four
     bf8 terms in eight activation columns (beyond 8192 in workgroups of sixteen wavefronts). 22 significant bits of
@@ -266,7 +266,7 @@ def test_two_long_rows_against_wide_layers(cuda, oracle, K):
             assert np.array_equal(yv.cpu().numpy(), xv.astype(np.float32)), c
 
 
-@pytest.mark.parametrize("K", [2048, 16384])
+@pytest.mark.parametrize("K", [256, 2048, 16384])
 def test_fp32_row_passes_22_bit_values_through_exactly(cuda, oracle, K):
     """Identity weights: integers of up to 22 bits (and their power-of-two multiples, small and large) come back
     exactly -- both halves and all eight term columns are in place."""

@@ -517,13 +517,14 @@ int launch_gemv8_dense(const void *x, int64_t M, int64_t K, const void *native, 
     return launch_gemv8_by_blocks<false, 2, false>(x, Kb, native, N, ep, stream);
 }
 
-// One fp32 row: K a multiple of 256 from 2048 to 16384 (eight term planes; beyond 8192 they leave room for one
-// workgroup per CU only, which then has sixteen wavefronts). Two fp32 rows (sixteen planes, all sixteen activation
+// One fp32 row: K a multiple of 256 up to 16384 (eight term planes; beyond 8192 they leave room for one workgroup per
+// CU only, which then has sixteen wavefronts). Short rows too -- wavefronts without a weight block multiply by zero --
+// because the alternative for fp32 is a prescale launch in front of another kernel (K = 1024, N = 4096: 7.1 -> 3.5 us). Two fp32 rows (sixteen planes, all sixteen activation
 // columns) while the layer is small: every workgroup splits both rows, which beats a split launch in front of the
 // fp16 weight stream up to about 6144^2 (2048^2 5.96 -> 4.3 us, 4096^2 7.45 -> 6.1, 6144^2 9.9 -> 8.7) and loses on
 // wider or longer layers (4096 x 11008 9.7 -> 11.5, 8192^2 10.3 -> 11.4, 8192 x 1024 8.1 -> 9.8).
 bool gemv8_dense32_ok(const void *x, int64_t M, int64_t K, int64_t N) {
-    if (K % kKB != 0 || K < 8 * kKB || !aligned16(x)) return false;
+    if (K % kKB != 0 || !aligned16(x)) return false;
     return M == 1 ? K <= 64 * kKB : M == 2 && K <= 24 * kKB && N <= 6144;
 }
 
