@@ -549,7 +549,8 @@ def set_fp32_prescale(flag: bool) -> bool:
     scaled by the power of two that puts its largest value into fp16's comfortable range (one extra small
     launch, exact, undone in the epilogue), so any magnitude works, as in the reference, which multiplies in
     fp32. A caller who knows its activations are of order 1 (max|x| <= 65504, nothing of interest below ~1e-4)
-    can switch that off. Returns the previous setting."""
+    can switch that off. (Rows over whole 256-index weight blocks, and seventeen rows or more, take kernels that
+    scale every row or group of rows themselves: the switch changes nothing for them.) Returns the previous setting."""
     global _fp32_prescale
     prev, _fp32_prescale = _fp32_prescale, bool(flag)
     return prev
