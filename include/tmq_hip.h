@@ -307,7 +307,7 @@ int tmq_ternary_linear(const void *x, int x_dtype, int64_t M, int64_t K, const v
  * workspace differently: a first launch splits every row into two fp16 rows
  * (hi = fp16(s x), lo = fp16(s x - hi), s the row's own power of two: any magnitude, 22 significant bits), the fp16
  * weight-stream kernel then runs once over twice the rows (from nine rows: twice, over about half of them each)
- * and adds each pair in its epilogue (256 + 4 M K bytes). Seventeen fp32 rows or more with K >= 256 are split in
+ * and adds each pair in its epilogue (256 + 4 M K bytes). Seventeen fp32 rows or more are split in
  * groups of eight rows, each group under a power of two of its own, laid out so that a row's two terms share a
  * 16-row MFMA fragment; the fp16 GEMM kernels then run once over 16 ceil(M / 8) rows and add the pairs where they
  * write the tile (ceil(M / 8) floats rounded up to 256 bytes + 32 ceil(M / 8) K' bytes, K' = K rounded up to a

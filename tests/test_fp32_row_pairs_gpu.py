@@ -237,7 +237,7 @@ def test_many_rows_workspace_rules_and_graph_replay(cuda, oracle):
     from tmq_amd import ops, _capi
     lib = _capi.load()
     M, K, N = 200, 1024, 520
-    assert lib.tmq_ternary_linear_workspace_bytes(_capi.F32, 200, 128, N) == 0       # K below 256: the older paths
+    assert lib.tmq_ternary_linear_workspace_bytes(_capi.F32, 200, 128, N) == 256 + 32 * 25 * 128   # short reductions as well
     # a length that is no multiple of 64: the pairs are written as zero-padded rows of the next multiple (test_ragged_rows_gpu.py)
     assert lib.tmq_ternary_linear_workspace_bytes(_capi.F32, 200, 1024 + 32, N) == 256 + 32 * 25 * 1088
     g = torch.Generator(device=cuda).manual_seed(8)

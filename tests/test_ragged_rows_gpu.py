@@ -2,7 +2,7 @@
 tmq/tmq_cuda.cu:289-427, host 478-549): with a workspace tmq_ternary_linear_ws copies the rows once to rows of the
 next multiple of 64, zeros behind, and runs the kernels that want whole tiles; without one the guarded kernel runs.
 
-fp32 rows of such lengths (seventeen or more, K >= 256) are split into fp16 row pairs that are written padded the same way.
+fp32 rows of such lengths (seventeen or more) are split into fp16 row pairs that are written padded the same way.
 
 Bar: both routes against an fp64 product of the expanded weights (fp16 inputs, fp32 accumulation: 2e-5 of the largest
 output), exact on small integers, every epilogue, rows that are not 16-byte aligned, and the workspace rules of the ABI.
@@ -46,7 +46,7 @@ def test_ragged_lengths_against_fp64(cuda, oracle, M, N, K):
     assert torch.equal(ops.ternary_linear(xi, nw).double(), xi.double() @ Wd.t())      # integers: exact whatever the order
 
 
-@pytest.mark.parametrize("K", [257, 520, 784, 1000, 4000, 4100])
+@pytest.mark.parametrize("K", [7, 64, 100, 257, 520, 784, 1000, 4000, 4100])
 @pytest.mark.parametrize("M,N", [(17, 1000), (128, 520), (300, 4100), (1030, 64)])
 def test_ragged_fp32_rows_against_fp64(cuda, oracle, M, N, K):
     """fp32 rows (the reference's convention) of such lengths: split into fp16 row pairs in groups of eight, written as

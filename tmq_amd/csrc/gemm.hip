@@ -1158,7 +1158,7 @@ int launch_mid_dense_pairs(const void *x16, int64_t M16, int64_t K, const void *
 inline int64_t pair_rows16(int64_t M) { return (M + 7) / 8 * 16; }
 inline bool pair_rows_ok(const void *x, int64_t M, int64_t K, int64_t N) {
     (void)x;                                                       // rows of any alignment: the splitter reads them element-wise if it must
-    return M >= 17 && K >= 256 && pair_rows16(M) * padded_k(K) < (int64_t)0x7FFFFFFF;
+    return M >= 17 && K >= 1 && pair_rows16(M) * padded_k(K) < (int64_t)0x7FFFFFFF;
 }
 // the workspace: the groups' 1 / s (padded to 256 bytes), then the fp16 rows
 inline size_t pair_scale_bytes(int64_t M) { return ((size_t)((M + 7) / 8) * sizeof(float) + 255) & ~(size_t)255; }

@@ -1177,10 +1177,11 @@ int tmq_ternary_linear(const void *x, int x_dtype, int64_t M, int64_t K, const v
     if (x32 && stream32_dense_ok(x, M, K) && K >= 8 * kKB)
         return launch_stream32_dense(x, M, K, native, N, ep.scale, ep.bias, ep.residual, ep.relu, y, ep.y_dtype == TMQ_F16, stream);
     // Otherwise up to 16 rows take the skinny kernels (activations staged in LDS). They also take 17 .. 64
-    // rows when K is ragged or the rows are unaligned; with whole 256-index blocks the split-reduction
-    // kernels are as fast at K = 4096 and two to three times faster at short K, where staging all of
-    // x in every workgroup dominates (M = 64, K = 512: 11.2 -> 4.6 us; fp32 input at K = 4096: 33 -> 14 us).
-    const bool blocks_ok = (K % kKB == 0) && aligned16(x);
+    // rows when K is ragged or the rows are unaligned; with whole 64-index tiles of aligned rows the split-reduction
+    // kernels are as fast at K = 4096 and two to five times faster elsewhere, where staging all of x in every
+    // workgroup dominates (M = 64, K = 512: 11.2 -> 4.6 us; K = 576, N = 512: 15.7 -> 3.8; K = 8256, N = 16384:
+    // 126 -> 23; fp32 input at K = 4096: 33 -> 14 us). fp32 rows need whole 256-index blocks for their kernel.
+    const bool blocks_ok = (K % (x32 ? kKB : 64) == 0) && aligned16(x);
     if (M <= 16 || (M <= 64 && !blocks_ok))
         return x32 ? skinny_rows<true>(x, M, K, native, N, ep, y, stream)
                    : skinny_rows<false>(x, M, K, native, N, ep, y, stream);
