@@ -338,7 +338,10 @@ __global__ __launch_bounds__(1024) void split_groups_kernel(const float *__restr
 
 // The same split for rows of any length and alignment, written as rows of Kp >= K values (Kp a multiple of 8) with
 // zeros behind the K-th: one workgroup per group of eight rows, element-wise reads, one 16-byte piece of a hi row and
-// of its lo row per thread and step. The second pass over the group's 32 K bytes comes from L2.
+// of its lo row per thread and step. The second pass over the group's 32 K bytes comes from L2. With few groups,
+// gridDim.y workgroups share one: each finds the group's maximum itself and writes every gridDim.y-th run of pieces.
+// VEC: K is a multiple of 4 and x 16-byte aligned -- whole float4s, two per piece (K a multiple of 8: never across the end).
+template <bool VEC>
 __global__ __launch_bounds__(1024) void split_groups_padded_kernel(const float *__restrict__ x, int64_t M, int K, int Kp,
                                                                    FastDiv by_row, _Float16 *__restrict__ x16,
                                                                    float *__restrict__ group_scale) {
@@ -347,26 +350,47 @@ __global__ __launch_bounds__(1024) void split_groups_padded_kernel(const float *
     const float *src = x + g * 8 * (int64_t)K;
     const int rows = M - g * 8 < 8 ? (int)(M - g * 8) : 8;
     float amax = 0.f;
-    for (int at = threadIdx.x; at < rows * K; at += 1024) amax = fmaxf(amax, finite_abs(src[at]));
+    if constexpr (VEC) {
+        for (int at = threadIdx.x; at < rows * (K / 4); at += 1024) {
+            const floatx4 v = *(reinterpret_cast<const floatx4 *>(src) + at);
+            amax = fmaxf(fmaxf(amax, fmaxf(finite_abs(v[0]), finite_abs(v[1]))), fmaxf(finite_abs(v[2]), finite_abs(v[3])));
+        }
+    } else {
+        for (int at = threadIdx.x; at < rows * K; at += 1024) amax = fmaxf(amax, finite_abs(src[at]));
+    }
     amax = block_max(amax, lds);
     float s, inv;
     make_prescale(amax, s, inv);
-    if (threadIdx.x == 0) group_scale[g] = inv;
+    if (threadIdx.x == 0 && blockIdx.y == 0) group_scale[g] = inv;
     _Float16 *dst = x16 + g * 16 * (int64_t)Kp;                    // the group's hi rows, then its lo rows
     const uint32_t pieces = 8u * (uint32_t)(Kp / 8);
-    for (uint32_t p = threadIdx.x; p < pieces; p += 1024) {
+    for (uint32_t p = blockIdx.y * 1024u + threadIdx.x; p < pieces; p += 1024u * gridDim.y) {
         int c;
         const int r = (int)by_row.divmod(p, c);
         const int k0 = c * 8;
         half8 h = {0, 0, 0, 0, 0, 0, 0, 0}, l = {0, 0, 0, 0, 0, 0, 0, 0};
         if (r < rows) {
+            if constexpr (VEC) {
 #pragma unroll
-            for (int e = 0; e < 8; e++)
-                if (k0 + e < K) {
-                    const float v = s * src[(int64_t)r * K + k0 + e];
-                    h[e] = (_Float16)v;
-                    l[e] = (_Float16)(v - (float)h[e]);
-                }
+                for (int q = 0; q < 2; q++)
+                    if (k0 + 4 * q < K) {
+                        const floatx4 f = *reinterpret_cast<const floatx4 *>(src + (int64_t)r * K + k0 + 4 * q);
+#pragma unroll
+                        for (int e = 0; e < 4; e++) {
+                            const float v = s * f[e];
+                            h[4 * q + e] = (_Float16)v;
+                            l[4 * q + e] = (_Float16)(v - (float)h[4 * q + e]);
+                        }
+                    }
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; e++)
+                    if (k0 + e < K) {
+                        const float v = s * src[(int64_t)r * K + k0 + e];
+                        h[e] = (_Float16)v;
+                        l[e] = (_Float16)(v - (float)h[e]);
+                    }
+            }
         }
         *reinterpret_cast<half8 *>(dst + (int64_t)r * Kp + k0) = h;
         *reinterpret_cast<half8 *>(dst + (int64_t)(8 + r) * Kp + k0) = l;
@@ -380,7 +404,11 @@ int launch_split_groups(const float *x, int64_t M, int64_t K, int64_t Kp, void *
     if (groups > 0x7FFFFFFF) return TMQ_ERR_TOO_LARGE;
     if (Kp != K || K % 4 != 0 || !aligned16(x)) {
         if (8 * Kp > 0x7FFFFFFF) return TMQ_ERR_TOO_LARGE;
-        hipLaunchKernelGGL(split_groups_padded_kernel, dim3((uint32_t)groups), dim3(1024), 0, as_stream(stream), x, M, (int)K,
+        // few groups: up to eight workgroups each (M = 17, K = 4000: 3 workgroups -> 12)
+        const int64_t runs = (Kp + 1023) / 1024;
+        const uint32_t share = groups > 64 ? 1 : (uint32_t)(runs < 1 ? 1 : runs > 8 ? 8 : runs);
+        auto padded = K % 4 == 0 && aligned16(x) ? split_groups_padded_kernel<true> : split_groups_padded_kernel<false>;
+        hipLaunchKernelGGL(padded, dim3((uint32_t)groups, share), dim3(1024), 0, as_stream(stream), x, M, (int)K,
                            (int)Kp, FastDiv((uint32_t)(Kp / 8)), static_cast<_Float16 *>(x16), group_scale);
         return check_launch();
     }
