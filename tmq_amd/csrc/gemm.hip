@@ -1126,16 +1126,18 @@ int launch_rows_split(const void *x, int64_t M, int64_t K, const void *native, i
 // -- against the kernel that splits every block's activations on the fly in each workgroup: 8192^2, 4 rows
 // 17.4 -> 10.8 us, 8 rows 25.5 -> 11.7 us; and on short reductions against a prescale launch in front of the skinny
 // kernels: K = 1024, N = 4096, 4 rows 7.9 -> 6.0 us, 8 rows 9.5 -> 6.4, 16 rows 12.3 -> 9.4.
-int launch_split_rows(const float *x, int64_t M, int64_t K, int64_t group, void *x16, float *row_scale, void *stream);
+int launch_split_rows(const float *x, int64_t M, int64_t K, int64_t Kp, int64_t group, void *x16, float *row_scale, void *stream);
+inline int64_t padded_blocks(int64_t K) { return (K + kKB - 1) / kKB * kKB; }   // the weight stream wants whole 256-index blocks
 int launch_stream_pairs(const void *x16, int64_t M, int64_t K, const void *native, int64_t N, const float *row_scale,
                         const float *scale, const float *bias, const void *residual, int relu, void *y, int y_f16,
                         void *stream);
 bool gemv8_dense32_ok(const void *x, int64_t M, int64_t K, int64_t N);
 inline bool row_pairs_ok(const void *x, int64_t M, int64_t K, int64_t N) {
     if (gemv8_dense32_ok(x, M, K, N)) return false;               // two rows over a small layer: one launch (gemv8.hip)
-    return M >= 2 && M <= 16 && K % kKB == 0 && aligned16(x) && 2 * M * K < (int64_t)0x7FFFFFFF;
+    // (a ragged length is written zero-padded to whole blocks, rows of any alignment are read element-wise)
+    return M >= 2 && M <= 16 && K >= 1 && 2 * M * padded_blocks(K) < (int64_t)0x7FFFFFFF;
 }
-inline size_t row_pairs_bytes(int64_t M, int64_t K) { return 256 + (size_t)(2 * M * K) * sizeof(_Float16); }
+inline size_t row_pairs_bytes(int64_t M, int64_t K) { return 256 + (size_t)(2 * M * padded_blocks(K)) * sizeof(_Float16); }
 
 // Seventeen fp16 rows or more whose reduction length is no multiple of 64: the kernels with direct global -> LDS
 // loads want whole 64-index tiles of 16-byte aligned rows, and the register-staged kernel that takes everything else
@@ -1229,12 +1231,13 @@ int tmq_ternary_linear_ws(const void *x, int x_dtype, int64_t M, int64_t K, cons
         void *x16 = static_cast<unsigned char *>(workspace) + 256;
         // up to eight rows make one pass of sixteen fp16 rows; nine to sixteen go as two groups of about equal size
         const int64_t group = M <= 8 ? M : (M + 1) / 2;
-        if (int st = launch_split_rows(static_cast<const float *>(x), M, K, group, x16, row_scale, stream)) return st;
+        const int64_t Kp = padded_blocks(K);
+        if (int st = launch_split_rows(static_cast<const float *>(x), M, K, Kp, group, x16, row_scale, stream)) return st;
         const size_t out_elt = e.y_dtype == TMQ_F16 ? 2 : 4;
         for (int64_t m0 = 0; m0 < M; m0 += group) {
             const int64_t rows = M - m0 < group ? M - m0 : group;
             const unsigned char *res = static_cast<const unsigned char *>(e.residual);
-            const int st = launch_stream_pairs(static_cast<const _Float16 *>(x16) + 2 * m0 * K, rows, K, native, N, row_scale + m0,
+            const int st = launch_stream_pairs(static_cast<const _Float16 *>(x16) + 2 * m0 * Kp, rows, Kp, native, N, row_scale + m0,
                                                e.scale, e.bias, res ? res + (size_t)(m0 * N) * out_elt : nullptr, e.relu,
                                                static_cast<unsigned char *>(y) + (size_t)(m0 * N) * out_elt,
                                                e.y_dtype == TMQ_F16 ? 1 : 0, stream);

@@ -176,22 +176,31 @@ __global__ __launch_bounds__(256) void split_terms_kernel(const float *__restric
 // A few fp32 rows as fp16 row pairs, each row with a prescale of its own: one workgroup per row finds the row's
 // largest finite |x|, scales by the power of two s that brings it into [1024, 2048) and writes hi = fp16(s x) and
 // lo = fp16(s x - hi) to x16, 1 / s to row_scale[m]. The rows go in groups of `group` (the last may be shorter):
-// group g occupies x16 rows 2 g group onwards, its hi rows first, then its lo rows. K a multiple of 8, rows
-// 16-byte aligned.
-__global__ __launch_bounds__(1024) void split_rows_kernel(const float *__restrict__ x, int64_t K, int rows, int group,
-                                                          _Float16 *__restrict__ x16, float *__restrict__ row_scale) {
+// group g occupies x16 rows 2 g group onwards, its hi rows first, then its lo rows. The fp16 rows have Kp >= K values
+// (a multiple of 8), zeros behind the K-th. vec: K a multiple of 4 and x 16-byte aligned (whole float4s).
+__global__ __launch_bounds__(1024) void split_rows_kernel(const float *__restrict__ x, int64_t K, int64_t Kp, int rows, int group,
+                                                          _Float16 *__restrict__ x16, float *__restrict__ row_scale, int vec) {
     __shared__ float lds[17];
     const int m = blockIdx.x;
     const int g = m / group, w = m - g * group, in_group = rows - g * group < group ? rows - g * group : group;
     const float *row = x + (int64_t)m * K;
-    const float amax = block_max(scan_abs_max(row, K, threadIdx.x, 1024, true), lds);
+    const float amax = block_max(scan_abs_max(row, K, threadIdx.x, 1024, vec != 0), lds);
     float s, inv;
     make_prescale(amax, s, inv);
     if (threadIdx.x == 0) row_scale[m] = inv;
-    _Float16 *hi = x16 + (int64_t)(2 * g * group + w) * K, *lo = hi + (int64_t)in_group * K;
-    for (int64_t i0 = (int64_t)threadIdx.x * 8; i0 < K; i0 += 8192) {
-        const floatx4 a = *reinterpret_cast<const floatx4 *>(row + i0) * s;
-        const floatx4 b = *reinterpret_cast<const floatx4 *>(row + i0 + 4) * s;
+    _Float16 *hi = x16 + (int64_t)(2 * g * group + w) * Kp, *lo = hi + (int64_t)in_group * Kp;
+    for (int64_t i0 = (int64_t)threadIdx.x * 8; i0 < Kp; i0 += 8192) {
+        floatx4 a = {0.f, 0.f, 0.f, 0.f}, b = {0.f, 0.f, 0.f, 0.f};
+        if (vec) {
+            if (i0 < K) a = *reinterpret_cast<const floatx4 *>(row + i0) * s;
+            if (i0 + 4 < K) b = *reinterpret_cast<const floatx4 *>(row + i0 + 4) * s;
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                if (i0 + e < K) a[e] = row[i0 + e] * s;
+                if (i0 + 4 + e < K) b[e] = row[i0 + 4 + e] * s;
+            }
+        }
         half8 h, l;
 #pragma unroll
         for (int e = 0; e < 4; e++) {
@@ -453,10 +462,10 @@ int launch_pad_rows(const void *x, int64_t M, int64_t K, int64_t Kp, void *out, 
     return check_launch();
 }
 
-// x16: 2 M rows of K fp16 values, row_scale: M floats; K % 8 == 0, x and x16 16-byte aligned.
-int launch_split_rows(const float *x, int64_t M, int64_t K, int64_t group, void *x16, float *row_scale, void *stream) {
-    hipLaunchKernelGGL(split_rows_kernel, dim3((uint32_t)M), dim3(1024), 0, as_stream(stream), x, K, (int)M, (int)group,
-                       static_cast<_Float16 *>(x16), row_scale);
+// x16: 2 M rows of Kp >= K fp16 values (Kp % 8 == 0, zeros behind the K-th), 16-byte aligned; row_scale: M floats.
+int launch_split_rows(const float *x, int64_t M, int64_t K, int64_t Kp, int64_t group, void *x16, float *row_scale, void *stream) {
+    hipLaunchKernelGGL(split_rows_kernel, dim3((uint32_t)M), dim3(1024), 0, as_stream(stream), x, K, Kp, (int)M, (int)group,
+                       static_cast<_Float16 *>(x16), row_scale, (K % 4 == 0 && aligned16(x)) ? 1 : 0);
     return check_launch();
 }
 
