@@ -302,7 +302,7 @@ int tmq_ternary_linear(const void *x, int x_dtype, int64_t M, int64_t K, const v
  * themselves, tmq/tmq_cuda.cu:478-549; this ABI never allocates): a product whose reduction pays to be cut across
  * workgroups -- today 17 .. 32 fp16 rows over 2^28 weights or more -- runs as slices of whole 256-index weight
  * blocks with fp32 partial sums in the workspace, added in slice order by a second launch (deterministic, no
- * atomics). Two to sixteen fp32 rows (the reference's kernels take fp32 activations,
+ * atomics). Up to sixteen fp32 rows that tmq_ternary_linear does not scale itself (the reference's kernels take fp32 activations,
  * tmq/tmq_cuda.cu:242-427; two rows with K, N <= 6144 excepted: tmq_ternary_linear takes them in one launch) use the
  * workspace differently: a first launch splits every row into two fp16 rows
  * (hi = fp16(s x), lo = fp16(s x - hi), s the row's own power of two: any magnitude, 22 significant bits), the fp16

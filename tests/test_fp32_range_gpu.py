@@ -67,11 +67,10 @@ def test_prescale_values_and_the_switch(cuda):
                 assert np.log2(s) == int(np.log2(s)) and s * inv == 1.0      # a power of two and its reciprocal
             assert torch.equal(xs[torch.isfinite(xm)], fin * s)
             assert torch.equal(adj, scale * inv)
-    # without the prescale a tensor beyond fp16's range overflows: the switch exists for callers who know (a single row
-    # of a length that is no multiple of 256: two rows or more, and whole weight blocks, take kernels that scale every
-    # row themselves, switch or not)
+    # without the prescale a tensor beyond fp16's range overflows: the switch exists for callers who know (rows that
+    # do not start on 16 bytes: aligned rows take kernels that scale every row themselves, switch or not)
     W, packed, nw = _layer(cuda, 64, 520, 3)
-    x = torch.randn(1, 520, generator=torch.Generator().manual_seed(4)).to(cuda) * 1e6
+    x = (torch.randn(3 * 520 + 1, generator=torch.Generator().manual_seed(4)).to(cuda) * 1e6)[1:].view(3, 520)
     want = x.double().cpu() @ W.double().t()
     prev = ops.set_fp32_prescale(False)
     try:

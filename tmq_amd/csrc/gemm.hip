@@ -1135,7 +1135,7 @@ bool gemv8_dense32_ok(const void *x, int64_t M, int64_t K, int64_t N);
 inline bool row_pairs_ok(const void *x, int64_t M, int64_t K, int64_t N) {
     if (gemv8_dense32_ok(x, M, K, N)) return false;               // two rows over a small layer: one launch (gemv8.hip)
     // (a ragged length is written zero-padded to whole blocks, rows of any alignment are read element-wise)
-    return M >= 2 && M <= 16 && K >= 1 && 2 * M * padded_blocks(K) < (int64_t)0x7FFFFFFF;
+    return M >= 1 && M <= 16 && K >= 1 && 2 * M * padded_blocks(K) < (int64_t)0x7FFFFFFF;
 }
 inline size_t row_pairs_bytes(int64_t M, int64_t K) { return 256 + (size_t)(2 * M * padded_blocks(K)) * sizeof(_Float16); }
 

@@ -1112,7 +1112,7 @@ int launch_stream32_dense(const void *x, int64_t M, int64_t K, const void *nativ
 static int stream_by_shape(const void *x, int64_t M, int64_t K, const void *native, int64_t N, const MidEpilogue &ep,
                            void *stream, const RowPairs *pairs) {
     const int64_t Nb = native_blocks_n(N);
-    if (M <= 2) return launch_stream<1, 8, 2, 4>(x, native, M, K, N, ep, stream, pairs);
+    if (M <= 2 && !pairs) return launch_stream<1, 8, 2, 4>(x, native, M, K, N, ep, stream, pairs);   // (a pair is added where four rows meet)
     if (M <= 4) {
         if (Nb >= 512) return launch_stream<2, 8, 4, 4>(x, native, M, K, N, ep, stream, pairs);
         return launch_stream<1, 8, 4, 4>(x, native, M, K, N, ep, stream, pairs);

@@ -626,7 +626,7 @@ def ternary_linear(x: torch.Tensor, nw: NativeWeights, scale=None, bias=None, re
     if (x.dtype == torch.float32 and 1 <= M <= 2 and x.is_contiguous()
             and _lib().tmq_fp32_rows_self_scaled_for(ptr(x), M, nw.K, nw.N)):
         pass            # one row (two over a small layer) the kernel scales itself, any magnitude: one launch
-    elif (x.dtype == torch.float32 and M >= 2 and x.is_contiguous() and x.data_ptr() % 16 == 0
+    elif (x.dtype == torch.float32 and M >= 1 and x.is_contiguous() and x.data_ptr() % 16 == 0
           and _lib().tmq_ternary_linear_workspace_bytes(_capi.F32, M, nw.K, nw.N)):
         # split once into fp16 row pairs in the workspace (a few rows: each scaled by its own power of two; from
         # seventeen: the whole tensor by one), then one pass of the fp16 kernels with the pairs added in the epilogue
