@@ -302,17 +302,16 @@ int tmq_ternary_linear(const void *x, int x_dtype, int64_t M, int64_t K, const v
  * themselves, tmq/tmq_cuda.cu:478-549; this ABI never allocates): a product whose reduction pays to be cut across
  * workgroups -- today 17 .. 32 fp16 rows over 2^28 weights or more -- runs as slices of whole 256-index weight
  * blocks with fp32 partial sums in the workspace, added in slice order by a second launch (deterministic, no
- * atomics). Up to sixteen fp32 rows that tmq_ternary_linear does not scale itself (the reference's kernels take fp32 activations,
- * tmq/tmq_cuda.cu:242-427; two rows with K, N <= 6144 excepted: tmq_ternary_linear takes them in one launch) use the
- * workspace differently: a first launch splits every row into two fp16 rows
- * (hi = fp16(s x), lo = fp16(s x - hi), s the row's own power of two: any magnitude, 22 significant bits), the fp16
- * weight-stream kernel then runs once over twice the rows (from nine rows: twice, over about half of them each)
- * and adds each pair in its epilogue (256 + 4 M K" bytes, K" = K rounded up to a multiple of 256: the pairs of a
- * ragged length are written with zeros behind). Seventeen fp32 rows or more are split in
- * groups of eight rows, each group under a power of two of its own, laid out so that a row's two terms share a
- * 16-row MFMA fragment; the fp16 GEMM kernels then run once over 16 ceil(M / 8) rows and add the pairs where they
- * write the tile (ceil(M / 8) floats rounded up to 256 bytes + 32 ceil(M / 8) K' bytes, K' = K rounded up to a
- * multiple of 64: the pairs of a ragged length are written with zeros behind).
+ * atomics). fp32 rows (the reference's kernels take fp32 activations, tmq/tmq_cuda.cu:242-427) use the workspace
+ * differently, unless tmq_ternary_linear scales them itself in one launch (tmq_fp32_rows_self_scaled_for). Up to
+ * sixteen rows: a first launch splits every row into two fp16 rows (hi = fp16(s x), lo = fp16(s x - hi), s the row's
+ * own power of two: any magnitude, 22 significant bits), the fp16 weight-stream kernel then runs once over twice the
+ * rows (from nine rows: twice, over about half of them each) and adds each pair in its epilogue (256 + 4 M K" bytes,
+ * K" = K rounded up to a multiple of 256: the pairs of a ragged length are written with zeros behind). Seventeen
+ * rows or more are split in groups of eight rows, each group under a power of two of its own, laid out so that a
+ * row's two terms share a 16-row MFMA fragment; the fp16 GEMM kernels then run once over 16 ceil(M / 8) rows and add
+ * the pairs where they write the tile (ceil(M / 8) floats rounded up to 256 bytes + 32 ceil(M / 8) K' bytes, K' = K
+ * rounded up to a multiple of 64, zeros behind the K-th value again).
  * Seventeen fp16 rows or more whose K is no multiple of 64 are copied once to rows of the next multiple of 64, zeros
  * behind (2 M ceil(K / 64) 64 bytes), and take the kernels that want whole 64-index tiles of 16-byte aligned rows
  * instead of the one that guards every load (K = 4000, M = 1024, N = 4096: 261 -> 39 us).
