@@ -219,3 +219,21 @@ def test_one_call_conversion_equals_prescale_then_split(cuda, shape):
         assert torch.equal(adj2, adj)
         hi3, adj3 = ops.f32_to_f16_prescaled(x, None, 24)
         assert torch.equal(hi3.view(torch.int16), want.view(torch.int16)) and torch.equal(adj3, ops.f32_prescale(x, None, 24)[2])
+
+
+def test_switch_sends_many_rows_against_a_narrow_layer_to_the_one_pass_kernel(cuda):
+    """With the prescale switched off (values promised to lie in fp16's range), a thousand fp32 rows or more against at
+    most 128 channels skip the row-pair route, whose split pass would move the rows three times: same values to fp32
+    rounding either way."""
+    from tmq_amd import ops
+    W, packed, nw = _layer(cuda, 16, 1024, 9)
+    x = torch.randn(2048, 1024, generator=torch.Generator().manual_seed(10)).to(cuda)
+    want = x.double() @ W.to(cuda).double().t()
+    y_pairs = ops.ternary_linear(x, nw)
+    prev = ops.set_fp32_prescale(False)
+    try:
+        y_plain = ops.ternary_linear(x, nw)
+    finally:
+        ops.set_fp32_prescale(prev)
+    for y in (y_pairs, y_plain):
+        assert ((y.double() - want).abs().max() / want.abs().max()).item() <= 1e-5

@@ -549,8 +549,10 @@ def set_fp32_prescale(flag: bool) -> bool:
     scaled by the power of two that puts its largest value into fp16's comfortable range (one extra small
     launch, exact, undone in the epilogue), so any magnitude works, as in the reference, which multiplies in
     fp32. A caller who knows its activations are of order 1 (max|x| <= 65504, nothing of interest below ~1e-4)
-    can switch that off. (Rows over whole 256-index weight blocks, and seventeen rows or more, take kernels that
-    scale every row or group of rows themselves: the switch changes nothing for them.) Returns the previous setting."""
+    can switch that off. (Most shapes take kernels that scale every row or group of rows themselves and the switch
+    changes nothing for them; a thousand rows or more against at most 128 channels are the case where it pays: the
+    kernel that splits fp32 values on the fly then reads the rows once, K = 4096, N = 16, M = 32768: 335 -> 128 us.)
+    Returns the previous setting."""
     global _fp32_prescale
     prev, _fp32_prescale = _fp32_prescale, bool(flag)
     return prev
@@ -627,6 +629,7 @@ def ternary_linear(x: torch.Tensor, nw: NativeWeights, scale=None, bias=None, re
             and _lib().tmq_fp32_rows_self_scaled_for(ptr(x), M, nw.K, nw.N)):
         pass            # one row (two over a small layer) the kernel scales itself, any magnitude: one launch
     elif (x.dtype == torch.float32 and M >= 1 and x.is_contiguous() and x.data_ptr() % 16 == 0
+          and not (not _fp32_prescale and M >= 1024 and nw.N <= 128)
           and _lib().tmq_ternary_linear_workspace_bytes(_capi.F32, M, nw.K, nw.N)):
         # split once into fp16 row pairs in the workspace (a few rows: each scaled by its own power of two; from
         # seventeen: the whole tensor by one), then one pass of the fp16 kernels with the pairs added in the epilogue
