@@ -46,6 +46,10 @@ def test_patches_form_matches_oracle(cuda, oracle, P, T, C):
     (1, 8, 18, 19, (2, 7), 1, (1, 6), (1, 2)), (1, 16, 21, 22, (9, 4), (3, 2), (4, 3), (1, 2)), (2, 8, 8, 30, (1, 5), (1, 2), (0, 4), (1, 2)),
     # what stays on the one-position-per-thread kernel: 6 columns, horizontal dilation 3, horizontal stride 3
     (1, 8, 9, 12, (2, 6), 1, (0, 2), 1), (1, 8, 10, 14, 3, 1, 3, 3), (1, 16, 9, 13, 3, 3, 1, 1),
+    # channel counts that are a multiple of 4 but not of 8: pixels start on 8 bytes, whole groups of 8 channels come as
+    # two 8-byte loads and the last, partial group reads on into the next pixel (element by element at the last pixel)
+    (2, 12, 9, 10, 3, 1, 1, 1), (1, 100, 14, 13, 5, 2, 2, 1), (3, 20, 8, 8, (3, 5), 1, (1, 2), 1), (1, 4, 6, 7, 3, 1, 1, 1),
+    (2, 36, 7, 9, 3, 2, 0, 2),
 ])
 def test_image_form_exact_on_integers(cuda, B, C, H, W, k, stride, pad, dil):
     """Small-integer activations: every product and sum is exact, so the result must equal torch's

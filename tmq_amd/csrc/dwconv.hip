@@ -51,7 +51,7 @@ __device__ __forceinline__ float apply_code(float v, uint32_t codes) {
     return c == 1u ? v : (c == 2u ? -v : 0.0f);
 }
 
-__device__ __forceinline__ void store8(const DwEpilogue &ep, int64_t o, int64_t c0, int64_t C, float (&acc)[8], bool vec) {
+__device__ __forceinline__ void store8(const DwEpilogue &ep, int64_t o, int64_t c0, int64_t C, float (&acc)[8], int vec) {
 #pragma unroll
     for (int e = 0; e < 8; e++) {
         if (c0 + e >= C) break;
@@ -63,7 +63,13 @@ __device__ __forceinline__ void store8(const DwEpilogue &ep, int64_t o, int64_t 
         if (ep.relu) v = v < 0.f ? 0.f : v;
         acc[e] = v;
     }
-    if (vec) {
+    if (vec == 2 && ep.y_f16) {                                    // a whole group whose pixel starts on 8 bytes
+        half4 lo, hi;
+#pragma unroll
+        for (int e = 0; e < 4; e++) { lo[e] = (_Float16)acc[e]; hi[e] = (_Float16)acc[4 + e]; }
+        *reinterpret_cast<half4 *>(static_cast<_Float16 *>(ep.y) + o) = lo;
+        *reinterpret_cast<half4 *>(static_cast<_Float16 *>(ep.y) + o + 4) = hi;
+    } else if (vec) {
         if (ep.y_f16) {
             half8 h;
 #pragma unroll
@@ -149,18 +155,31 @@ __global__ __launch_bounds__(256) void dwconv_image_kernel(const _Float16 *__res
     const int64_t r = div_rem(p, Wo, ow);
     const int b = (int)div_rem(r, Ho, oh);
     float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    // Groups of 8 channels in 16- or 8-byte loads. With 8-byte pixels (vec & 4) the last, partial group of a pixel
+    // reads on into the next pixel -- values that meet weight codes of zero and sums that are never stored -- except at
+    // the tensor's last pixel, which goes element by element.
+    const bool fast = (vec & 3) || (vec & 4);
+    const int64_t last_pixel = (int64_t)B * H * W - 1;
     for (int i = 0; i < ky; i++) {
         const int ih = oh * sy - py + i * dy;
         if (ih < 0 || ih >= H) continue;
         for (int j = 0; j < kx; j++) {
             const int iw = ow * sx - px + j * dx;
             if (iw < 0 || iw >= W) continue;
-            const _Float16 *src = x + (((int64_t)b * H + ih) * W + iw) * C + c0;
+            const int64_t pixel = ((int64_t)b * H + ih) * W + iw;
+            const _Float16 *src = x + pixel * C + c0;
             uint32_t codes = codes8(words, Q, i * kx + j, c0);
-            if (vec) {
+            if (fast && ((vec & 3) || c0 + 8 <= C || pixel < last_pixel)) {
                 // the codes as fp16 +-2.0 operands, two per register (see dwconv_square_image_kernel): the sums run at
-                // twice their value and are halved below
-                const half8 v = *reinterpret_cast<const half8 *>(src);
+                // twice their value and are halved below. (vec & 4: pixels start on 8 bytes only -- C a multiple of 4 --
+                // and a whole group of 8 channels comes as two 8-byte loads.)
+                half8 v;
+                if (vec & 3) {
+                    v = *reinterpret_cast<const half8 *>(src);
+                } else {
+                    const half4 lo = *reinterpret_cast<const half4 *>(src), hi = *reinterpret_cast<const half4 *>(src + 4);
+                    v = half8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                }
                 codes ^= (codes >> 1) & 0x55555555u;
                 const uint32_t t = (codes & 0xFF000000u) | ((codes >> 8) & 0x0000FF00u);
 #pragma unroll
@@ -170,18 +189,19 @@ __global__ __launch_bounds__(256) void dwconv_image_kernel(const _Float16 *__res
                     acc[4 + e] = __builtin_fmaf((float)v[4 + e], (float)w[0], acc[4 + e]);
                 }
             } else {
+                // (fast: the sums run at twice their value, so this tap counts twice as well)
 #pragma unroll
                 for (int e = 0; e < 8; e++)
-                    if (c0 + e < C) acc[e] += apply_code((float)src[e], codes << (2 * e));
+                    if (c0 + e < C) acc[e] += (fast ? 2.f : 1.f) * apply_code((float)src[e], codes << (2 * e));
             }
         }
     }
-    if (vec) {
+    if (fast) {
 #pragma unroll
         for (int e = 0; e < 8; e++) acc[e] *= 0.5f;                 // exact: the weights were +-2
     }
     if (vec & 2) store8_vec(ep, load_channel_constants(ep, c0), p * C + c0, acc);
-    else store8(ep, p * C + c0, c0, C, acc, vec);
+    else store8(ep, p * C + c0, c0, C, acc, (vec & 1) ? 1 : (((vec & 8) && c0 + 8 <= C) ? 2 : 0));
 }
 
 // The common cases -- windows of ky rows x KS columns (KS of 1 .. 5 or 7, any ky), horizontal stride 1 or 2 and
@@ -472,6 +492,10 @@ int tmq_ternary_dwconv2d(const void *x, const tmq_conv_shape *s, const uint32_t 
             case 5: return by_step(std::integral_constant<int, 5>{});
             default: return by_step(std::integral_constant<int, 7>{});
         }
+    }
+    if (!vec && s->C % 4 == 0 && aligned_for(x, 8)) {              // pixels on 8 bytes: whole channel groups as two 8-byte loads
+        vec = 4;
+        if (aligned_for(y, 16) && (!e.residual || y_f16)) vec |= 8;   // ... and stores (fp32 pixels then start on 16 bytes)
     }
     hipLaunchKernelGGL(dwconv_image_kernel, dim3((uint32_t)blocks), dim3(256), 0, as_stream(stream),
                        static_cast<const _Float16 *>(x), words, s->B, s->C, s->H, s->W, ho, wo, s->ky, s->kx, s->sy, s->sx,
