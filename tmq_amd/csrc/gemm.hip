@@ -175,6 +175,7 @@ struct ConvLoader {
     const _Float16 *x;
     int64_t M, K;
     int B, C, H, W, Ho, Wo, ky, kx, sy, sx, py, px, dy, dx;
+    int quads = 0;                 // !VEC: C is a multiple of 4 and x 8-byte aligned -- a chunk is two 8-byte loads
 
     template <int CH, int T>
     struct State {
@@ -220,6 +221,26 @@ struct ConvLoader {
                 const _Float16 *src = in ? st.img[q] + ((int64_t)ih * W + iw) * C + st.c
                                          : reinterpret_cast<const _Float16 *>(&kZeroChunk);
                 v = *reinterpret_cast<const u32x4 *>(src);
+            } else if (quads) {
+                // two halves of four channels, each inside one tap (the second may be the next tap's first four); what
+                // does not exist is read from 16 bytes of zeros
+                typedef uint32_t u32x2v __attribute__((ext_vector_type(2)));
+                int i = st.i, j = st.j, c = st.c;
+                u32x2v half[2];
+#pragma unroll
+                for (int h = 0; h < 2; h++) {
+                    const int ih = st.ih0[q] + i * dy, iw = st.iw0[q] + j * dx;
+                    const bool in = (st.img[q] != nullptr) & (k + 4 * h < K) & ((unsigned)ih < (unsigned)H) & ((unsigned)iw < (unsigned)W);
+                    const _Float16 *src = in ? st.img[q] + ((int64_t)ih * W + iw) * C + c
+                                             : reinterpret_cast<const _Float16 *>(&kZeroChunk);
+                    half[h] = *reinterpret_cast<const u32x2v *>(src);
+                    c += 4;
+                    if (c == C) {
+                        c = 0;
+                        if (++j == kx) { j = 0; ++i; }
+                    }
+                }
+                v = u32x4{half[0][0], half[0][1], half[1][0], half[1][1]};
             } else if (st.img[q] && k < K) {
                 // element by element from the chunk's tap and channel onwards (a chunk may run over into the next tap)
                 half8 h = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -1198,7 +1219,8 @@ int conv_tiles(const void *x, const tmq_conv_shape *s, int ho, int wo, const voi
         return dispatch_tile(ConvLoader<true>{xp, M, K, s->B, s->C, s->H, s->W, ho, wo, s->ky, s->kx, s->sy, s->sx,
                                               s->py, s->px, s->dy, s->dx}, native, M, K, s->N, ep, stream);
     return dispatch_tile(ConvLoader<false>{xp, M, K, s->B, s->C, s->H, s->W, ho, wo, s->ky, s->kx, s->sy, s->sx, s->py,
-                                           s->px, s->dy, s->dx}, native, M, K, s->N, ep, stream);
+                                           s->px, s->dy, s->dx, (s->C % 4 == 0 && (reinterpret_cast<uintptr_t>(x) & 7u) == 0) ? 1 : 0},
+                         native, M, K, s->N, ep, stream);
 }
 
 }  // namespace
