@@ -549,7 +549,7 @@ def bench_pack(args, torch):
             "bound": "hbm", "achieved": round(byts / us / 1e3, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
             "frac": round(byts / us / 1e3 / HBM_PEAK_GBS, 4),
             "traffic": measured_traffic("pack_4096.md", key="traffic_bytes_" + name), "algorithmic_bytes": int(byts),
-            "kernel": ("pack_wide_kernel<float, 4>" if name == "pack" else "unpack_wide_kernel<8>"), "avg_launch_us": round(us, 3)}
+            "kernel": ("pack_wide_kernel<float, 4, 1>" if name == "pack" else "unpack_wide_kernel<8>"), "avg_launch_us": round(us, 3)}
     res["value"] = res["pack"]["gbs"]
     if not args.no_cpu:
         res["cpu_baseline"] = cpu_baseline_pack(torch, N, K)

@@ -513,6 +513,7 @@ class TMQLayer:
         self._scale_dirty = True
         self._native = None          # cached kernel-native weights for compact inference
         self._scale_vec = None
+        self._pair_epilogue = None   # scale / bias repeated for the pixel-pair form of a first layer
         self._fold = None            # (scale [N], bias [N]) of a BatchNorm folded into the compact epilogue
 
     def compact_inference_mode(self):
@@ -832,12 +833,74 @@ class Conv2d(nn.Module, TMQLayer):
             xs = ops.nchw_to_nhwc4(x).view(B, H, W // 2, 8).permute(0, 3, 1, 2)
             return ops.ternary_conv2d(xs, nw, (sy, 1), ((py, py), (pl, pr)), 1, scale=scale, bias=bias,
                                       residual=residual, relu=relu, out_dtype=_compact_out)
+        pp = None if pool else self._pixelpair_plan(x)
+        if pp is not None:
+            # a first layer with at most 4 input channels and horizontal stride 1: pairs of input pixels are read as
+            # one pixel of 8 channels and pairs of output pixels come out as one pixel of 2 N channels, see _pixelpair_plan
+            nw, kxs, pl, pr, scale, bias = pp
+            B, C, H, W = x.shape
+            N = int(self.original_shape[0])
+            if x.dtype == torch.float32:
+                x, scale = ops.f32_to_f16_prescaled(x, scale, 2 * N)
+            (sy, _), (py, _) = _pair(self.stride), _pair(self.padding)
+            xs = ops.nchw_to_nhwc4(x).view(B, H, W // 2, 8).permute(0, 3, 1, 2)
+            if residual is not None:      # [B, N, Ho, Wo] in NHWC memory is [B, Ho, Wo / 2, 2 N]
+                Ho, Wo = int(residual.shape[2]), int(residual.shape[3])
+                residual = residual.permute(0, 2, 3, 1).view(B, Ho, Wo // 2, 2 * N).permute(0, 3, 1, 2)
+            ys = ops.ternary_conv2d(xs, nw, (sy, 1), ((py, py), (pl, pr)), 1, scale=scale, bias=bias, residual=residual,
+                                    relu=relu, out_dtype=_compact_out)
+            Ho, Wh = int(ys.shape[2]), int(ys.shape[3])
+            return ys.permute(0, 2, 3, 1).view(B, Ho, 2 * Wh, N).permute(0, 3, 1, 2)
         nw = self._native_weights(conv_kernel=(ky, kx))
         if pool:
             return ops.ternary_conv2d_relu_maxpool(x, nw, _pair(self.stride), _pair(self.padding), _pair(self.dilation),
                                                    scale=scale, bias=bias)
         return ops.ternary_conv2d(x, nw, _pair(self.stride), _pair(self.padding), _pair(self.dilation), scale=scale,
                                   bias=bias, residual=residual, relu=relu, out_dtype=_compact_out)
+
+    def _pixelpair_plan(self, x):
+        """For a convolution with at most 4 input channels, horizontal stride 1, no dilation and an odd window
+        width on a contiguous NCHW fp16 / fp32 input (a network's own input) of a width that is a multiple of 4:
+        the equivalent convolution whose input pixels are pairs (2u, 2u + 1) of image pixels stored NHWC with 4
+        channels (8 channels, the 16-byte loader applies) and whose output pixels are pairs (2u, 2u + 1) of
+        output pixels (2 N channels: filter v' N + n produces column 2u + v' of filter n). Output column
+        2u + v' reads image columns 2u + v' - px + j = 2 (u + t) + v, so pair tap t, channel 4 v + c of filter
+        v' N + n carries the weight of (n, c, j = 2 t + v - v' + px). In memory [B, Ho, Wo / 2, 2 N] is
+        [B, Ho, Wo, N]: the result needs no rearrangement. Returns (native weights, pair taps, pad left,
+        pad right, scale or None, bias or None -- both repeated for the 2 N filters) or None when the layer
+        does not qualify; inputs already in channels-last memory keep the generic loader."""
+        N, C, ky, kx = (int(v) for v in self.original_shape)
+        (sy, sx), (py, px), (dy, dx) = _pair(self.stride), _pair(self.padding), _pair(self.dilation)
+        W = int(x.shape[-1])
+        if C > 4 or x.shape[1] != C or sx != 1 or (dy, dx) != (1, 1) or W % 4 or kx % 2 == 0 or x.numel() == 0 or \
+                x.dtype not in (torch.float16, torch.float32) or not x.is_contiguous() or \
+                isinstance(py, (tuple, list)) or isinstance(px, (tuple, list)):
+            return None
+        t_min, t_max = (-px) // 2, (kx - px) // 2
+        kxs, pl = t_max - t_min + 1, -t_min
+        wo = W + 2 * px - kx + 1
+        pr = wo // 2 - 1 + kxs - W // 2 - pl
+        if wo < 2 or wo % 2 or pr < 0:
+            return None
+        key = self._weight_key("pixelpair")
+        if self._native is None or self._native[0] != key:
+            full = ops.expand_ternary(self.weight.data, [N, C, ky, kx])
+            wpp = torch.zeros((2 * N, 8, ky, kxs), dtype=full.dtype, device=full.device)
+            for t in range(kxs):
+                for v in range(2):
+                    for vo in range(2):
+                        j = 2 * (t + t_min) + v - vo + px
+                        if 0 <= j < kx:
+                            wpp[vo * N:(vo + 1) * N, 4 * v:4 * v + C, :, t] = full[:, :, :, j]
+            self._native = (key, ops.NativeWeights(ops.compactify_ternary(wpp), 2 * N, (ky, kxs)))
+        b = getattr(self, "bias", None)
+        ekey = (self.post_scale_imm, id(self._fold), None if b is None else (b.data_ptr(), b._version), x.device)
+        if self._pair_epilogue is None or self._pair_epilogue[0] != ekey:
+            scale, bias = self._epilogue(N, x.device)
+            # the folded pair is kept in the entry so that its id cannot be handed to a later one while the entry lives
+            self._pair_epilogue = (ekey, None if scale is None else scale.repeat(2), None if bias is None else bias.repeat(2),
+                                   self._fold)
+        return self._native[1], kxs, pl, pr, self._pair_epilogue[1], self._pair_epilogue[2]
 
     def _superpixel_plan(self, x):
         """For a convolution with at most 4 input channels, horizontal stride 2 and no dilation on an
