@@ -336,3 +336,55 @@ def test_optimize_for_inference_one_call(cuda):
     assert t.set_compact_output_dtype(torch.float32) == torch.float32        # untouched outside the call
     eager = t.optimize_for_inference(net, graph=False)            # idempotent on an already optimised model
     assert torch.equal(eager(x), want)
+
+
+class _SmallImageNet(torch.nn.Module):
+    """A CIFAR-style network: 3 x 3 / stride 1 opening on three channels, one residual block, a linear head."""
+
+    def __init__(self):
+        super().__init__()
+        nn = torch.nn
+        self.conv1 = nn.Conv2d(3, 32, 3, 1, 1, bias=False)
+        self.bn1 = nn.BatchNorm2d(32)
+        self.conv2 = nn.Conv2d(32, 32, 3, 1, 1, bias=False)
+        self.bn2 = nn.BatchNorm2d(32)
+        self.head = nn.Linear(32, 10)
+
+    def forward(self, x):
+        h = torch.relu(self.bn1(self.conv1(x)))
+        y = torch.relu(self.bn2(self.conv2(h)) + h)
+        return self.head(y.mean(dim=(2, 3)))
+
+
+@pytest.mark.parametrize("in_dtype", [torch.float16, torch.float32])
+def test_optimize_for_inference_stride_one_opening(cuda, in_dtype):
+    """The opening of a small-image network (horizontal stride 1) runs in its pixel-pair form inside the optimised
+    model, eager and as graph replays, with the folded BatchNorm and the ReLU in its epilogue: same values as the
+    generic loader gives for the same model, and the float model's within fp16 tolerance."""
+    import tmq_amd as t
+
+    def make():
+        torch.manual_seed(21)
+        net = _SmallImageNet()
+        ctrl = t.QuantizationControl(post_scale=True)
+        t.quantize_model(net, ctrl)
+        _randomize_bn(net, torch.Generator().manual_seed(21))
+        net.to(cuda).eval()
+        ctrl.quantize()
+        return net
+
+    net = make()
+    x = torch.randn(8, 3, 32, 32, device=cuda).to(in_dtype)
+    with torch.no_grad():
+        want = net(x.float())
+    t.compressed_state_dict(net, strong=False)
+    generic = make()
+    t.compressed_state_dict(generic, strong=False)
+    generic.conv1._pixelpair_plan = lambda x: None
+    assert net.conv1._pixelpair_plan(x) is not None
+    session = t.optimize_for_inference(net)
+    reference = t.optimize_for_inference(generic, graph=False)(x)
+    for _ in range(3):
+        got = session(x)
+        assert torch.allclose(got.float(), reference.float(), rtol=2e-3, atol=2e-3 * want.abs().max().item())
+        assert torch.allclose(got.float(), want, rtol=3e-2, atol=3e-2 * want.abs().max().item())
