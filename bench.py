@@ -454,7 +454,7 @@ def bench_layers(args, torch):
     dev = torch.device("cuda:0")
     g = torch.Generator(device=dev).manual_seed(7)
     res = {"metric": "depthwise / transposed ternary layers", "unit": "us", "n_gpus": 1, "dtype": "f16", "data": "synthetic",
-           "config": {"workload": "batch 64, 128 channels, 56 x 56 depthwise windows; ConvTranspose2d 128 -> 64, 4 x 4 / 2, 56 x 56, batch 32"}}
+           "config": {"workload": "batch 64, 128 channels, 56 x 56 depthwise windows; ConvTranspose2d 128 -> 64, 4 x 4 / 2, 56 x 56, batch 32; first layer 3 -> 64, 3 x 3 / 1, 32 x 32, batch 128"}}
     B, C, H, W = 64, 128, 56, 56
     xs = [torch.randn((B, C, H, W), device=dev, generator=g).half().contiguous(memory_format=torch.channels_last) for _ in range(4)]
     for name, k, pad, dil in (("dw3x3", (3, 3), 1, 1), ("dw3x5", (3, 5), (1, 2), 1), ("dw3x3_dilated2", (3, 3), 2, 2), ("dw5x5", (5, 5), 2, 1)):
@@ -504,6 +504,30 @@ def bench_layers(args, torch):
     byts = (xt[0].numel() + y.numel()) * 2
     res["convtranspose_128_64_k4s2"] = {"us": round(us, 3), "launches": 4, "out_MB": round(y.numel() * 2 / 1e6, 1), "gbs": round(byts / us / 1e3, 1),
                                         "note": "one stride-1 implicit-GEMM convolution per output phase, written in place (tmq_ternary_conv2d_view)"}
+    # a small-image network's opening (3 -> 64, 3 x 3, stride 1, 32 x 32, batch 128, NCHW fp16 in, fp16 NHWC out): the
+    # pixel-pair form of Conv2d.compact_forward (repack launch + one convolution launch; tmq/tmq.py:822-871)
+    first = torch.nn.Sequential(torch.nn.Conv2d(3, 64, 3, 1, 1, bias=True))
+    ctrl = t.QuantizationControl()
+    t.quantize_model(first, ctrl)
+    first.to(dev).eval()
+    ctrl.quantize()
+    t.compressed_state_dict(first, strong=False)
+    prev = t.set_compact_output_dtype(torch.float16)
+    try:
+        xf = [torch.randn((128, 3, 32, 32), device=dev, generator=g).half() for _ in range(4)]
+        with torch.no_grad():
+            yf = first[0].compact_forward(xf[0], relu=True)
+
+            def run_f():
+                for x in xf:
+                    first[0].compact_forward(x, relu=True)
+                return len(xf)
+            us = _graph_time_us(torch, run_f, max(2, args.steps // 4), args.settle_ms)
+    finally:
+        t.set_compact_output_dtype(prev)
+    byts = (xf[0].numel() + yf.numel()) * 2
+    res["first_layer_3_64_k3s1"] = {"us": round(us, 3), "launches": 2, "gbs": round(byts / us / 1e3, 1),
+                                    "note": "input pixel pairs as 8 channels, output pixel pairs as 128 filters (Conv2d._pixelpair_plan)"}
     res["value"] = res["dw3x3"]["us"]
     res["roofline"] = {"bound": "hbm", "achieved": res["dw3x3"]["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": res["dw3x3"]["frac_hbm"],
                        "traffic": measured_traffic("depthwise_layers_batch64.md", key="traffic_bytes_dw3x3"),
