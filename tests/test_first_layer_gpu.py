@@ -34,7 +34,7 @@ def test_first_layer_compact_equals_float(cuda, cin, cout, k, stride, pad, H, W)
 
 
 @pytest.mark.parametrize("cin,cout,k,stride,pad,H,W", [
-    (3, 64, 3, 1, 1, 32, 32), (1, 16, 5, 1, 2, 28, 28), (4, 24, 3, 1, 0, 8, 8), (2, 8, 1, 1, 0, 6, 8),
+    (3, 64, 3, 1, 1, 32, 32), (1, 16, 5, 1, 2, 28, 28), (4, 24, 3, 1, 0, 8, 8), (2, 8, 1, 1, 0, 6, 8), (4, 64, 3, 1, 1, 16, 24),
     (3, 40, (3, 5), (2, 1), (1, 0), 9, 12), (3, 32, 7, 1, 3, 16, 16), (3, 8, 3, 1, (0, 3), 8, 12), (3, 16, (3, 1), 1, (0, 1), 8, 12),
 ])
 def test_first_layer_stride_one_compact_equals_float(cuda, cin, cout, k, stride, pad, H, W):
@@ -59,10 +59,13 @@ def test_first_layer_stride_one_compact_equals_float(cuda, cin, cout, k, stride,
     res = torch.randint(-5, 6, want.shape, device=cuda).float()
     fused = net[0].compact_forward(x, residual=res, relu=True)
     assert torch.equal(fused.float(), torch.relu(want + res))
-    # the generic loader gives the same for the same image in channels-last memory, where the route does not apply
+    # the same image in channels-last memory: the generic loader for two or three channels
     xl = x.contiguous(memory_format=torch.channels_last)
-    if cin > 1:
+    if cin in (2, 3):
         assert net[0]._pixelpair_plan(xl) is None
-        assert torch.equal(net(xl), want)
+    elif cin == 4:      # four channels in channels-last memory are the pixel pairs already: the route without its repack
+        assert net[0]._pixelpair_plan(xl) is not None
+        assert torch.equal(net(xl.half()), want)
+    assert torch.equal(net(xl), want)
     # an odd width, an even window width or a dilated window keep the generic loader
     assert net[0]._pixelpair_plan(x[..., :W - 1].contiguous()) is None

@@ -843,7 +843,10 @@ class Conv2d(nn.Module, TMQLayer):
             if x.dtype == torch.float32:
                 x, scale = ops.f32_to_f16_prescaled(x, scale, 2 * N)
             (sy, _), (py, _) = _pair(self.stride), _pair(self.padding)
-            xs = ops.nchw_to_nhwc4(x).view(B, H, W // 2, 8).permute(0, 3, 1, 2)
+            if x.is_contiguous():
+                xs = ops.nchw_to_nhwc4(x).view(B, H, W // 2, 8).permute(0, 3, 1, 2)
+            else:                         # 4 channels in channels-last memory are the pixel pairs already
+                xs = x.permute(0, 2, 3, 1).view(B, H, W // 2, 8).permute(0, 3, 1, 2)
             if residual is not None:      # [B, N, Ho, Wo] in NHWC memory is [B, Ho, Wo / 2, 2 N]
                 Ho, Wo = int(residual.shape[2]), int(residual.shape[3])
                 residual = residual.permute(0, 2, 3, 1).view(B, Ho, Wo // 2, 2 * N).permute(0, 3, 1, 2)
@@ -868,12 +871,14 @@ class Conv2d(nn.Module, TMQLayer):
         v' N + n carries the weight of (n, c, j = 2 t + v - v' + px). In memory [B, Ho, Wo / 2, 2 N] is
         [B, Ho, Wo, N]: the result needs no rearrangement. Returns (native weights, pair taps, pad left,
         pad right, scale or None, bias or None -- both repeated for the 2 N filters) or None when the layer
-        does not qualify; inputs already in channels-last memory keep the generic loader."""
+        does not qualify. Four channels in channels-last memory are pixel pairs as they lie (no repack launch); fewer
+        channels in channels-last memory keep the generic loader."""
         N, C, ky, kx = (int(v) for v in self.original_shape)
         (sy, sx), (py, px), (dy, dx) = _pair(self.stride), _pair(self.padding), _pair(self.dilation)
         W = int(x.shape[-1])
         if C > 4 or x.shape[1] != C or sx != 1 or (dy, dx) != (1, 1) or W % 4 or kx % 2 == 0 or x.numel() == 0 or \
-                x.dtype not in (torch.float16, torch.float32) or not x.is_contiguous() or \
+                x.dtype not in (torch.float16, torch.float32) or \
+                not (x.is_contiguous() or (C == 4 and x.is_contiguous(memory_format=torch.channels_last))) or \
                 isinstance(py, (tuple, list)) or isinstance(px, (tuple, list)):
             return None
         t_min, t_max = (-px) // 2, (kx - px) // 2
