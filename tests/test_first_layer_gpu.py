@@ -59,6 +59,12 @@ def test_first_layer_stride_one_compact_equals_float(cuda, cin, cout, k, stride,
     res = torch.randint(-5, 6, want.shape, device=cuda).float()
     fused = net[0].compact_forward(x, residual=res, relu=True)
     assert torch.equal(fused.float(), torch.relu(want + res))
+    prev = t.set_compact_output_dtype(torch.float16)          # with the opening's max-pool behind it (fp16 outputs)
+    try:
+        pooled = net[0].compact_forward(x, relu=True, pool=True)
+    finally:
+        t.set_compact_output_dtype(prev)
+    assert torch.equal(pooled.float(), torch.nn.functional.max_pool2d(torch.relu(want), 3, 2, 1))
     # the same image in channels-last memory: the generic loader for two or three channels
     xl = x.contiguous(memory_format=torch.channels_last)
     if cin in (2, 3):

@@ -833,7 +833,7 @@ class Conv2d(nn.Module, TMQLayer):
             xs = ops.nchw_to_nhwc4(x).view(B, H, W // 2, 8).permute(0, 3, 1, 2)
             return ops.ternary_conv2d(xs, nw, (sy, 1), ((py, py), (pl, pr)), 1, scale=scale, bias=bias,
                                       residual=residual, relu=relu, out_dtype=_compact_out)
-        pp = None if pool else self._pixelpair_plan(x)
+        pp = self._pixelpair_plan(x)
         if pp is not None:
             # a first layer with at most 4 input channels and horizontal stride 1: pairs of input pixels are read as
             # one pixel of 8 channels and pairs of output pixels come out as one pixel of 2 N channels, see _pixelpair_plan
@@ -853,7 +853,8 @@ class Conv2d(nn.Module, TMQLayer):
             ys = ops.ternary_conv2d(xs, nw, (sy, 1), ((py, py), (pl, pr)), 1, scale=scale, bias=bias, residual=residual,
                                     relu=relu, out_dtype=_compact_out)
             Ho, Wh = int(ys.shape[2]), int(ys.shape[3])
-            return ys.permute(0, 2, 3, 1).view(B, Ho, 2 * Wh, N).permute(0, 3, 1, 2)
+            y = ys.permute(0, 2, 3, 1).view(B, Ho, 2 * Wh, N).permute(0, 3, 1, 2)
+            return ops.maxpool2d_nhwc(y, 3, 2, 1) if pool else y      # the one-kernel opening is for horizontal stride 2
         nw = self._native_weights(conv_kernel=(ky, kx))
         if pool:
             return ops.ternary_conv2d_relu_maxpool(x, nw, _pair(self.stride), _pair(self.padding), _pair(self.dilation),
